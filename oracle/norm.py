@@ -1,0 +1,106 @@
+"""RMSNorm / residual-block oracle.
+
+Restates R1:5165-5168 (eager block head: x_new = l1*x + l2*x0, norm(x_new)), R1:5594 (rmsnorm_fast),
+R1:6106-6159 (head_skip / tail_norm2 / final_norm eager forms), R2:8805-8825 (nf_norm_rows and its
+backward: upcast, rs = rsqrt(mean(x^2) + eps), one rounding per output; G = inv * (g - x * (g.x) * inv^2 / C)).
+The optional per-channel weight and eps are BASELINE config 1's generalisation (reference: no weight, eps 2^-23).
+
+Pinned by: torch.nn.functional.rms_norm (forward), torch.autograd on an fp64 restatement (backward),
+the invariant that J^T(g) is orthogonal to x when weight is None.
+"""
+import torch
+
+RMS_EPS = float(2.0 ** -23)
+
+
+def rmsnorm(x, weight=None, eps=RMS_EPS):
+    """(y, inv): y = dtype(x32 * rs * w32), inv = rs [rows] fp32."""
+    xf = x.float()
+    rs = torch.rsqrt(xf.square().mean(dim=-1, keepdim=True) + eps)
+    y = xf * rs
+    if weight is not None:
+        y = y * weight.float()
+    return y.to(x.dtype), rs.reshape(-1)
+
+
+def rmsnorm_backward(gy, x, inv, weight=None):
+    """(dx, dw): dx in x.dtype, dw fp32 [C] (None without weight). fp32 math, one rounding."""
+    C = x.shape[-1]
+    g = gy.float().reshape(-1, C)
+    xf = x.float().reshape(-1, C)
+    rs = inv.float().reshape(-1, 1)
+    dw = None
+    if weight is not None:
+        dw = (g * xf * rs).sum(dim=0)
+        g = g * weight.float()
+    dot = (g * xf).sum(dim=-1, keepdim=True)
+    dx = rs * (g - xf * (dot * rs * rs / C))
+    return dx.reshape(x.shape), dw
+
+
+def add_rmsnorm(x, res, weight=None, eps=RMS_EPS):
+    """tail_norm2 / final_norm: s = dtype(x + res); (s, norm(s), inv)."""
+    s = (x.float() + res.float()).to(x.dtype)
+    y, inv = rmsnorm(s, weight, eps)
+    return s, y, inv
+
+
+def add_rmsnorm_backward(gs, gy, s, inv, weight=None):
+    """Gradient wrt s (= wrt x = wrt res): gs + J^T(gy), rounded once; and dw."""
+    dx, dw = rmsnorm_backward(gy, s, inv, weight)
+    if gs is not None:
+        dx = dx + gs.float()
+    return dx.to(s.dtype), dw
+
+
+def block_head(x, x0, l1, l2, skip=None, l3=None, eps=RMS_EPS):
+    """x_new = dtype(l1*x + l2*x0 [+ l3*skip]) in fp32 from fp32 gains; x_norm = norm(x_new); inv."""
+    v = l1.float() * x.float() + l2.float() * x0.float()
+    if skip is not None:
+        v = v + l3.float() * skip.float()
+    x_new = v.to(x.dtype)
+    x_norm, inv = rmsnorm(x_new, None, eps)
+    return x_new, x_norm, inv
+
+
+def block_head_backward(g_new, g_norm, x, x0, x_new, inv, l1, l2, skip=None, l3=None):
+    """(dx, dx0, dskip, dl1, dl2, dl3) with G = g_new + J^T(g_norm); gain grads fp32 sums of G * input."""
+    jt, _ = rmsnorm_backward(g_norm, x_new, inv, None)
+    G = jt if g_new is None else jt + g_new.float()
+    dt = x.dtype
+    dx = (l1.float() * G).to(dt)
+    dx0 = (l2.float() * G).to(dt)
+    dl1 = (G * x.float()).sum()
+    dl2 = (G * x0.float()).sum()
+    if skip is None:
+        return dx, dx0, None, dl1, dl2, None
+    return dx, dx0, (l3.float() * G).to(dt), dl1, dl2, (G * skip.float()).sum()
+
+
+def relu2(x):
+    """R1:663 relu_squared: relu(x)^2 computed in fp32, one rounding."""
+    r = torch.relu(x.float())
+    return (r * r).to(x.dtype)
+
+
+def relu2_backward(x, gy):
+    """R1:597: gy * 2 * relu(x), one rounding."""
+    return (gy.float() * 2.0 * torch.relu(x.float())).to(x.dtype)
+
+
+def relu2_backward_from_h(h, dh):
+    """R1:625-631: dtype(dtype(sqrt(4 h)) * dh): the gradient from the saved output h = relu(x)^2."""
+    root = torch.sqrt(4.0 * h.float()).to(h.dtype)
+    return (root.float() * dh.float()).to(h.dtype)
+
+
+def resmix_backward(g, x, x0, a, b):
+    """K/nki_resmix.py:148-162: x_new = a*x + b*x0 backward in one pass: dx = g*a, dx0 = g*b (gains rounded to
+    the stream dtype as the eager chain does), gain grads = fp32 sums of the dtype-rounded products."""
+    dt = g.dtype
+    ad, bd = a.to(dt), b.to(dt)
+    dx = g * ad
+    dx0 = g * bd
+    da = (g * x).float().sum()
+    db = (g * x0).float().sum()
+    return dx, dx0, da, db

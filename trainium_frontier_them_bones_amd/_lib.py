@@ -1,0 +1,57 @@
+"""ctypes binding of the C-ABI library (include/tfb_kernels.h).
+
+The library is the product path: if it has not been built, or a symbol is missing, loading
+raises. There is no CPU or PyTorch fallback behind these entry points.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libtfb_hip.so")
+
+_vp = ctypes.c_void_p
+_i = ctypes.c_int
+_l = ctypes.c_long
+_f = ctypes.c_float
+
+# name -> argtypes (restype is always int status unless listed in _RESTYPE)
+SIGNATURES = {
+    "tfb_gemm_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _vp],
+    "tfb_norm_bwd_blocks": [_l],
+    "tfb_rmsnorm_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _f, _vp],
+    "tfb_rmsnorm_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _l, _i, _vp],
+    "tfb_block_head_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _f, _vp],
+    "tfb_block_head_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _vp],
+}
+
+STATUS = {0: "ok", 1: "unsupported shape", 2: "bad argument", 3: "kernel launch failed", 4: "workspace too small"}
+
+
+class TfbError(RuntimeError):
+    def __init__(self, fn, status):
+        self.status = status
+        super().__init__("%s returned %d (%s)" % (fn, status, STATUS.get(status, "?")))
+
+
+_LIB = None
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "HIP extension %s is not built; run `python -m trainium_frontier_them_bones_amd.build`" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        for name, args in SIGNATURES.items():
+            fn = getattr(L, name)  # AttributeError if the symbol is missing
+            fn.argtypes = args
+            fn.restype = _i
+        _LIB = L
+    return _LIB
+
+
+def call(name, *args):
+    st = getattr(lib(), name)(*args)
+    if st != 0:
+        raise TfbError(name, st)

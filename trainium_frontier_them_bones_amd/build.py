@@ -1,0 +1,60 @@
+"""Compile the HIP sources under csrc/ for gfx950 into one C-ABI shared library, in-tree.
+
+`python -m trainium_frontier_them_bones_amd.build` (or `build_library()`) runs hipcc on every
+`csrc/*.hip` in parallel and links `libtfb_hip.so` next to this file. hipcc cross-compiles, so
+no GPU is needed to build. The flags switch packed-fp32 code generation off for device code.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_NAME = "libtfb_hip.so"
+LIB_PATH = os.path.join(HERE, LIB_NAME)
+OBJ_DIR = os.path.join(HERE, "build")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def sources():
+    return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def _compile(src):
+    obj = os.path.join(OBJ_DIR, src[:-4] + ".o")
+    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "not a recognized feature" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed on %s:\n%s" % (src, err))
+    return obj, err
+
+
+def build_library(verbose=True, jobs=None):
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    srcs = sources()
+    jobs = jobs or min(8, len(srcs))
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        results = list(ex.map(_compile, srcs))
+    objs = [o for o, _ in results]
+    for (o, err), s in zip(results, srcs):
+        if verbose and err.strip():
+            print("[%s]\n%s" % (s, err), file=sys.stderr)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stderr)
+    if verbose:
+        print("built %s from %d sources" % (LIB_PATH, len(srcs)))
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build_library()

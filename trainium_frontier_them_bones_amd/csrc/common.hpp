@@ -1,0 +1,88 @@
+// Shared device helpers for the gfx950 (CDNA4) kernels: bf16 / fp8 conversion with the
+// rounding the reference's torch emulations use (round to nearest even, one rounding per
+// output), 128-bit vector types, wavefront (64-lane) reductions and the status codes the
+// C-ABI returns.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define TFB_OK 0
+#define TFB_ERR_SHAPE 1     // a dimension the kernels do not take (caller falls back or raises)
+#define TFB_ERR_ARG 2       // null pointer / bad enum
+#define TFB_ERR_LAUNCH 3    // hipGetLastError() after the launch was not hipSuccess
+#define TFB_ERR_WORKSPACE 4 // workspace too small
+
+#define TFB_WAVE 64
+
+typedef uint16_t bf16_t;  // raw bf16 bits; arithmetic is always done in fp32
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float bf2f(bf16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+// fp32 -> bf16, round to nearest even (torch's .to(torch.bfloat16)); NaN stays NaN.
+__device__ __forceinline__ bf16_t f2bf(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ uint32_t pack2bf(float lo, float hi) {
+  return (uint32_t)f2bf(lo) | ((uint32_t)f2bf(hi) << 16);
+}
+__device__ __forceinline__ float bflo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bfhi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// Round an fp32 value to the nearest bf16 and return it as fp32 (a rounding point of the
+// reference arithmetic that stays in registers).
+__device__ __forceinline__ float round_bf(float f) { return bf2f(f2bf(f)); }
+
+// fp32 -> OCP fp8 bytes (gfx950's v_cvt_pk_*_f32 are OCP e4m3fn / e5m2, round to nearest
+// even). Inputs are clamped to the format's finite range first, so a value beyond it
+// saturates instead of becoming NaN/Inf; inside the range the bytes are torch's
+// .to(float8_e4m3fn) / .to(float8_e5m2).
+#define TFB_E4M3_MAX 448.0f
+#define TFB_E5M2_MAX 57344.0f
+#define TFB_FMT_E4M3 0
+#define TFB_FMT_E5M2 1
+
+template <int FMT>
+__device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, float d) {
+  const float mx = FMT == TFB_FMT_E4M3 ? TFB_E4M3_MAX : TFB_E5M2_MAX;
+  a = fminf(fmaxf(a, -mx), mx);
+  b = fminf(fmaxf(b, -mx), mx);
+  c = fminf(fmaxf(c, -mx), mx);
+  d = fminf(fmaxf(d, -mx), mx);
+  int w = 0;
+  if (FMT == TFB_FMT_E4M3) {
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+  } else {
+    w = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, w, false);
+    w = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, w, true);
+  }
+  return (uint32_t)w;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+#define TFB_LAUNCH_CHECK()                                  \
+  do {                                                      \
+    if (hipGetLastError() != hipSuccess) return TFB_ERR_LAUNCH; \
+  } while (0)

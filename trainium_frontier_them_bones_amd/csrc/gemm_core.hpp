@@ -1,0 +1,255 @@
+// MFMA GEMM core for gfx950: D[p][q] = sum_k P[p][k] * Q[q][k], fp32 accumulation.
+//
+// One workgroup of WP x WQ wavefronts owns a BP x BQ output tile. Both operand tiles are
+// staged in LDS as [row][128 bytes of k] with a 16-byte row pad (conflict-free 128-bit
+// fragment reads), double-buffered, the next k-tile's global loads in flight while the
+// MFMAs of the current one run. The P tile feeds the MFMA A operand (rows), the Q tile
+// the B operand (columns), so a lane ends up holding D[p .. p+3][q] for four consecutive
+// p: callers put the dimension that is contiguous in the output on the P side and get
+// 64- or 128-bit stores from the epilogue.
+//
+// Element types: bf16 (v_mfma_f32_32x32x16_bf16, 64 k per tile) or OCP fp8
+// (v_mfma_scale_f32_32x32x64_f8f6f4 with unit scales, 128 k per tile, e4m3/e5m2 per side).
+// Operand layouts: K_CONTIG = [rows][K] (k contiguous); K_STRIDED = [K][rows] (bf16 only,
+// transposed on the way into LDS through 4k x 8row register micro-blocks), which is what
+// the weight-gradient GEMMs (contraction over tokens) read.
+#pragma once
+#include "common.hpp"
+
+#define TFB_K_CONTIG 0
+#define TFB_K_STRIDED 1
+#define TFB_LDS_ROW 144  // 128 bytes of k + 16 pad
+
+struct GemmOperand {
+  const uint8_t* base;
+  long ld;  // bytes between consecutive rows (K_CONTIG) or consecutive k (K_STRIDED)
+};
+
+struct GemmArgs {
+  GemmOperand P, Q;
+  int np, nq;   // output extent (multiples of BP / BQ)
+  int nkt;      // k-tiles (128 bytes of k each) per split
+  int ntp;      // tiles along p
+};
+
+struct LoadIdentity {
+  __device__ __forceinline__ u32x4 operator()(u32x4 v) const { return v; }
+};
+
+template <int BP_, int BQ_, int WP_, int WQ_, int ES_, int LAYP_, int LAYQ_, int FMTP_ = 0, int FMTQ_ = 0>
+struct GemmCfg {
+  static constexpr int BP = BP_, BQ = BQ_, WP = WP_, WQ = WQ_, ES = ES_;
+  static constexpr int LAYP = LAYP_, LAYQ = LAYQ_, FMTP = FMTP_, FMTQ = FMTQ_;
+  static constexpr int NT = WP * WQ * 64;
+  static constexpr int TP = BP / WP / 32, TQ = BQ / WQ / 32;
+  static constexpr int BK = 128 / ES;  // elements of k per tile
+  static constexpr int LDS_BYTES = 2 * (BP + BQ) * TFB_LDS_ROW;
+  static_assert(ES == 1 || ES == 2, "fp8 or bf16");
+  static_assert(ES == 2 || (LAYP == TFB_K_CONTIG && LAYQ == TFB_K_CONTIG), "fp8 operands are k-contiguous");
+  static_assert((BP * 8) % NT == 0 && (BQ * 8) % NT == 0, "tile rows vs threads");
+};
+
+// ---- global -> register -> LDS staging of one operand tile ---------------------------------
+template <int ROWS, int NT, int LAY>
+struct TileLoader;
+
+template <int ROWS, int NT>
+struct TileLoader<ROWS, NT, TFB_K_CONTIG> {
+  static constexpr int N = ROWS * 8 / NT;
+  u32x4 g[N];
+  __device__ __forceinline__ void load(const GemmOperand& o, long row0, long kbyte0, int tid) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      int c = tid + i * NT;
+      int row = c >> 3, cc = c & 7;
+      g[i] = *(const u32x4*)(o.base + (row0 + row) * o.ld + kbyte0 + cc * 16);
+    }
+  }
+  template <class Pre>
+  __device__ __forceinline__ void store(uint8_t* lds, int tid, const Pre& pre) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      int c = tid + i * NT;
+      int row = c >> 3, cc = c & 7;
+      *(u32x4*)(lds + row * TFB_LDS_ROW + cc * 16) = pre(g[i]);
+    }
+  }
+};
+
+template <int ROWS, int NT>
+struct TileLoader<ROWS, NT, TFB_K_STRIDED> {
+  // bf16 only: 64 k x ROWS tile, micro-blocks of 4 k x 8 rows
+  static constexpr int N = ROWS * 2 / NT;
+  static_assert((ROWS * 2) % NT == 0 && N >= 1, "K_STRIDED tile rows vs threads");
+  u32x4 g[N][4];
+  __device__ __forceinline__ void load(const GemmOperand& o, long row0, long kbyte0, int tid) {
+    const long k0 = kbyte0 >> 1;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      int mb = tid + i * NT;
+      int rg = mb % (ROWS / 8), kg = mb / (ROWS / 8);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        g[i][j] = *(const u32x4*)(o.base + (k0 + 4 * kg + j) * o.ld + (row0 + 8 * rg) * 2);
+    }
+  }
+  template <class Pre>
+  __device__ __forceinline__ void store(uint8_t* lds, int tid, const Pre& pre) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      int mb = tid + i * NT;
+      int rg = mb % (ROWS / 8), kg = mb / (ROWS / 8);
+      u32x4 v0 = pre(g[i][0]), v1 = pre(g[i][1]), v2 = pre(g[i][2]), v3 = pre(g[i][3]);
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        // rows 2w (low halves) and 2w+1 (high halves) of the micro-block
+        u32x2 lo, hi;
+        lo.x = (v0[w] & 0xffffu) | (v1[w] << 16);
+        lo.y = (v2[w] & 0xffffu) | (v3[w] << 16);
+        hi.x = (v0[w] >> 16) | (v1[w] & 0xffff0000u);
+        hi.y = (v2[w] >> 16) | (v3[w] & 0xffff0000u);
+        *(u32x2*)(lds + (8 * rg + 2 * w) * TFB_LDS_ROW + kg * 8) = lo;
+        *(u32x2*)(lds + (8 * rg + 2 * w + 1) * TFB_LDS_ROW + kg * 8) = hi;
+      }
+    }
+  }
+};
+
+// ---- MFMA fragments ------------------------------------------------------------------------
+template <int ES>
+struct Frag;
+template <>
+struct Frag<2> {
+  bf16x8 v;
+  static constexpr int KSTEPS = 4;  // 4 x 16 bf16 per 128-byte tile row
+  __device__ __forceinline__ void read(const uint8_t* lds, int row, int s, int h) {
+    v = *(const bf16x8*)(lds + row * TFB_LDS_ROW + s * 32 + h * 16);
+  }
+};
+template <>
+struct Frag<1> {
+  i32x8 v;
+  static constexpr int KSTEPS = 2;  // 2 x 64 fp8 per 128-byte tile row
+  __device__ __forceinline__ void read(const uint8_t* lds, int row, int s, int h) {
+    const i32x4* p = (const i32x4*)(lds + row * TFB_LDS_ROW + s * 64 + h * 32);
+    i32x4 a = p[0], b = p[1];
+    v = i32x8{a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+  }
+};
+
+template <int ES, int FMTP, int FMTQ>
+__device__ __forceinline__ f32x16 mfma32(const Frag<ES>& a, const Frag<ES>& b, f32x16 c) {
+  if constexpr (ES == 2) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
+  } else {
+    // formats: 0 = e4m3, 1 = e5m2; E8M0 scale byte 127 = 2^0
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a.v, b.v, c, FMTP, FMTQ, 0, 127, 0, 127);
+  }
+}
+
+// The workgroup's (tile_p, tile_q): consecutive workgroup ids are dealt round-robin to the
+// 8 XCDs (each with its own L2), so ids are re-dealt so that one XCD gets a contiguous run
+// of tiles; p runs fastest, so a run shares its Q rows through that XCD's L2.
+__device__ __forceinline__ int xcd_remap(int pid, int nb) {
+  return (nb & 7) == 0 ? (pid & 7) * (nb >> 3) + (pid >> 3) : pid;
+}
+
+// Epi: __device__ void operator()(int p, int q, f32x4 v, int split) -- v = D[p..p+3][q]
+template <class Cfg, class PreP, class PreQ, class Epi>
+__global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, PreQ preq, Epi epi) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  constexpr int BP = Cfg::BP, BQ = Cfg::BQ, NT = Cfg::NT, TP = Cfg::TP, TQ = Cfg::TQ, ES = Cfg::ES;
+  constexpr int BUF = (BP + BQ) * TFB_LDS_ROW;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int wp = wave % Cfg::WP, wq = wave / Cfg::WP;
+  const int lr = lane & 31, lh = lane >> 5;
+
+  const int lid = xcd_remap(blockIdx.x, gridDim.x);
+  const int tile_p = lid % a.ntp, tile_q = lid / a.ntp;
+  const long p0 = (long)tile_p * BP, q0 = (long)tile_q * BQ;
+  const long kt0 = (long)blockIdx.z * a.nkt;
+
+  TileLoader<BP, NT, Cfg::LAYP> lp;
+  TileLoader<BQ, NT, Cfg::LAYQ> lq;
+
+  f32x16 acc[TP][TQ];
+#pragma unroll
+  for (int i = 0; i < TP; ++i)
+#pragma unroll
+    for (int j = 0; j < TQ; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  lp.load(a.P, p0, kt0 * 128, tid);
+  lq.load(a.Q, q0, kt0 * 128, tid);
+  lp.store(smem, tid, prep);
+  lq.store(smem + BP * TFB_LDS_ROW, tid, preq);
+  __syncthreads();
+
+  for (int t = 0; t < a.nkt; ++t) {
+    const uint8_t* sp = smem + (t & 1) * BUF;
+    const uint8_t* sq = sp + BP * TFB_LDS_ROW;
+    const bool more = (t + 1 < a.nkt);
+    if (more) {
+      lp.load(a.P, p0, (kt0 + t + 1) * 128, tid);
+      lq.load(a.Q, q0, (kt0 + t + 1) * 128, tid);
+    }
+#pragma unroll
+    for (int s = 0; s < Frag<ES>::KSTEPS; ++s) {
+      Frag<ES> fa[TP], fb[TQ];
+#pragma unroll
+      for (int i = 0; i < TP; ++i) fa[i].read(sp, wp * (TP * 32) + i * 32 + lr, s, lh);
+#pragma unroll
+      for (int j = 0; j < TQ; ++j) fb[j].read(sq, wq * (TQ * 32) + j * 32 + lr, s, lh);
+#pragma unroll
+      for (int i = 0; i < TP; ++i)
+#pragma unroll
+        for (int j = 0; j < TQ; ++j) acc[i][j] = mfma32<ES, Cfg::FMTP, Cfg::FMTQ>(fa[i], fb[j], acc[i][j]);
+    }
+    if (more) {
+      uint8_t* np_ = smem + ((t + 1) & 1) * BUF;
+      lp.store(np_, tid, prep);
+      lq.store(np_ + BP * TFB_LDS_ROW, tid, preq);
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int i = 0; i < TP; ++i)
+#pragma unroll
+    for (int j = 0; j < TQ; ++j)
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        int p = (int)p0 + wp * (TP * 32) + i * 32 + jj * 8 + lh * 4;
+        int q = (int)q0 + wq * (TQ * 32) + j * 32 + lr;
+        f32x4 v = {acc[i][j][jj * 4 + 0], acc[i][j][jj * 4 + 1], acc[i][j][jj * 4 + 2], acc[i][j][jj * 4 + 3]};
+        epi(p, q, v, (int)blockIdx.z);
+      }
+}
+
+// Host-side launch: np, nq multiples of the tile; kbytes a multiple of 128 * splits.
+template <class Cfg, class PreP, class PreQ, class Epi>
+static int gemm_launch(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes, int splits, PreP prep, PreQ preq,
+                       Epi epi, hipStream_t stream) {
+  if (np <= 0 || nq <= 0 || kbytes <= 0 || splits <= 0) return TFB_ERR_SHAPE;
+  if (np % Cfg::BP || nq % Cfg::BQ || kbytes % (128L * splits)) return TFB_ERR_SHAPE;
+  GemmArgs a;
+  a.P = P;
+  a.Q = Q;
+  a.np = np;
+  a.nq = nq;
+  a.nkt = (int)(kbytes / 128 / splits);
+  a.ntp = np / Cfg::BP;
+  auto kern = gemm_kernel<Cfg, PreP, PreQ, Epi>;
+  static bool attr_set = false;  // per template instantiation
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES) != hipSuccess)
+      return TFB_ERR_LAUNCH;
+    attr_set = true;
+  }
+  dim3 grid(a.ntp * (nq / Cfg::BQ), 1, splits);
+  hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, a, prep, preq, epi);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}

@@ -1,0 +1,375 @@
+// RMSNorm family (bandwidth-bound): one wavefront per row, 128-bit coalesced loads, the row
+// kept in registers, fp32 math, one rounding per output, wavefront shuffles for the row sums.
+//
+//   rmsnorm fwd / bwd, optionally with a fused residual add in front (s = x + res, y = norm(s))
+//     and an optional per-channel weight                 round1/source/train.py:5594 (rmsnorm_fast),
+//                                                        6117 (tail_norm2), 6826 (final_norm);
+//                                                        round2/source/train.py:8805-8825 (nf_norm_rows / backward)
+//   block head: x_new = l1*x + l2*x0 (+ l3*skip), x_norm = RMSNorm(x_new)
+//                                                        round1/source/train.py:5578 (block_head), 6106 (head_skip)
+//
+// The value that is normalised is the bf16-rounded sum, as the eager chain normalises its bf16
+// tensor. Gain / weight gradients are fp32 partial sums per workgroup finished by a column sum.
+#include "common.hpp"
+
+namespace {
+
+constexpr int ROWS_PER_BLOCK = 4;  // one wavefront per row, 4 wavefronts per workgroup
+
+template <int NCH>
+struct Row {
+  float v[NCH][8];
+  __device__ __forceinline__ void load(const bf16_t* p, int C, int lane) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      int c = (lane + 64 * i) * 8;
+      if (c < C) {
+        u32x4 u = *(const u32x4*)(p + c);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          v[i][2 * k] = bflo(u[k]);
+          v[i][2 * k + 1] = bfhi(u[k]);
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[i][k] = 0.f;
+      }
+    }
+  }
+  __device__ __forceinline__ void store(bf16_t* p, int C, int lane) const {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      int c = (lane + 64 * i) * 8;
+      if (c < C) {
+        u32x4 u;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) u[k] = pack2bf(v[i][2 * k], v[i][2 * k + 1]);
+        *(u32x4*)(p + c) = u;
+      }
+    }
+  }
+  __device__ __forceinline__ void round() {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[i][k] = round_bf(v[i][k]);
+  }
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[i][k] = 0.f;
+  }
+};
+
+template <int NCH>
+__device__ __forceinline__ float row_dot(const Row<NCH>& a, const Row<NCH>& b) {
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+#pragma unroll
+    for (int k = 0; k < 8; ++k) s += a.v[i][k] * b.v[i][k];
+  return wave_sum(s);
+}
+
+// ------------------------------------------------------------------------------------------
+template <int NCH>
+__global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ res,
+                                                         const bf16_t* __restrict__ w, bf16_t* __restrict__ s_out,
+                                                         bf16_t* __restrict__ y, float* __restrict__ inv, long nrows,
+                                                         int C, float eps) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  Row<NCH> wr;
+  if (w) wr.load(w, C, lane);
+  for (long row = (long)blockIdx.x * ROWS_PER_BLOCK + wave; row < nrows; row += (long)gridDim.x * ROWS_PER_BLOCK) {
+    Row<NCH> a;
+    a.load(x + row * C, C, lane);
+    if (res) {
+      Row<NCH> r;
+      r.load(res + row * C, C, lane);
+#pragma unroll
+      for (int i = 0; i < NCH; ++i)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) a.v[i][k] = round_bf(a.v[i][k] + r.v[i][k]);
+      if (s_out) a.store(s_out + row * C, C, lane);
+    }
+    float ss = row_dot(a, a);
+    float rs = 1.0f / sqrtf(ss * (1.0f / C) + eps);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) a.v[i][k] = w ? a.v[i][k] * rs * wr.v[i][k] : a.v[i][k] * rs;
+    a.store(y + row * C, C, lane);
+    if (inv && lane == 0) inv[row] = rs;
+  }
+}
+
+// dx = gs + J^T(gy): J^T(gy) = inv * (gh - s * (gh . s) * inv^2 / C), gh = gy * w.
+// dw partial [gridDim.x][C] = sum over the workgroup's rows of gy * s * inv.
+template <int NCH>
+__global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16_t* __restrict__ gy, const bf16_t* __restrict__ gs,
+                                                         const bf16_t* __restrict__ s, const bf16_t* __restrict__ w,
+                                                         const float* __restrict__ inv, bf16_t* __restrict__ dx,
+                                                         float* __restrict__ dw_part, long nrows, int C) {
+  __shared__ float red[ROWS_PER_BLOCK][NCH * 512];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  Row<NCH> wr, dwacc;
+  if (w) wr.load(w, C, lane);
+  dwacc.zero();
+  for (long row = (long)blockIdx.x * ROWS_PER_BLOCK + wave; row < nrows; row += (long)gridDim.x * ROWS_PER_BLOCK) {
+    Row<NCH> g, a;
+    g.load(gy + row * C, C, lane);
+    a.load(s + row * C, C, lane);
+    const float rs = inv[row];
+    if (w) {
+#pragma unroll
+      for (int i = 0; i < NCH; ++i)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          dwacc.v[i][k] += g.v[i][k] * a.v[i][k] * rs;
+          g.v[i][k] *= wr.v[i][k];
+        }
+    }
+    float dot = row_dot(g, a);
+    float coef = dot * rs * rs * (1.0f / C);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) g.v[i][k] = rs * (g.v[i][k] - a.v[i][k] * coef);
+    if (gs) {
+      Row<NCH> r;
+      r.load(gs + row * C, C, lane);
+#pragma unroll
+      for (int i = 0; i < NCH; ++i)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) g.v[i][k] += r.v[i][k];
+    }
+    g.store(dx + row * C, C, lane);
+  }
+  if (w && dw_part) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) red[wave][(lane + 64 * i) * 8 + k] = dwacc.v[i][k];
+    __syncthreads();
+    for (int c = threadIdx.x; c < C; c += 256) {
+      float t = 0.f;
+#pragma unroll
+      for (int r = 0; r < ROWS_PER_BLOCK; ++r) t += red[r][c];
+      dw_part[(long)blockIdx.x * C + c] = t;
+    }
+  }
+}
+
+__global__ void colsum_kernel(const float* __restrict__ part, float* __restrict__ out, int rows, int C, int accumulate) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  float t = 0.f;
+  for (int r = 0; r < rows; ++r) t += part[(long)r * C + c];
+  out[c] = accumulate ? out[c] + t : t;
+}
+
+// ------------------------------------------------------------------------------------------ block head
+template <int NCH>
+__global__ __launch_bounds__(256) void block_head_fwd_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ x0,
+                                                            const bf16_t* __restrict__ skip,
+                                                            const float* __restrict__ gains, bf16_t* __restrict__ x_new,
+                                                            bf16_t* __restrict__ x_norm, float* __restrict__ inv,
+                                                            long nrows, int C, float eps) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float l1 = gains[0], l2 = gains[1], l3 = skip ? gains[2] : 0.f;
+  for (long row = (long)blockIdx.x * ROWS_PER_BLOCK + wave; row < nrows; row += (long)gridDim.x * ROWS_PER_BLOCK) {
+    Row<NCH> a, b;
+    a.load(x + row * C, C, lane);
+    b.load(x0 + row * C, C, lane);
+    if (skip) {
+      Row<NCH> c;
+      c.load(skip + row * C, C, lane);
+#pragma unroll
+      for (int i = 0; i < NCH; ++i)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) a.v[i][k] = round_bf(l1 * a.v[i][k] + l2 * b.v[i][k] + l3 * c.v[i][k]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < NCH; ++i)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) a.v[i][k] = round_bf(l1 * a.v[i][k] + l2 * b.v[i][k]);
+    }
+    a.store(x_new + row * C, C, lane);
+    float ss = row_dot(a, a);
+    float rs = 1.0f / sqrtf(ss * (1.0f / C) + eps);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) a.v[i][k] *= rs;
+    a.store(x_norm + row * C, C, lane);
+    if (lane == 0) inv[row] = rs;
+  }
+}
+
+// G = g_new + inv * (g_norm - x_new * (g_norm . x_new) * inv^2 / C);
+// dx = l1 G, dx0 = l2 G, dskip = l3 G; gain partials [gridDim.x][4] = sum G.x, G.x0, G.skip, 0
+template <int NCH>
+__global__ __launch_bounds__(256) void block_head_bwd_kernel(const bf16_t* __restrict__ g_new,
+                                                            const bf16_t* __restrict__ g_norm,
+                                                            const bf16_t* __restrict__ x, const bf16_t* __restrict__ x0,
+                                                            const bf16_t* __restrict__ skip,
+                                                            const bf16_t* __restrict__ x_new,
+                                                            const float* __restrict__ inv, const float* __restrict__ gains,
+                                                            bf16_t* __restrict__ dx, bf16_t* __restrict__ dx0,
+                                                            bf16_t* __restrict__ dskip, float* __restrict__ gain_part,
+                                                            long nrows, int C) {
+  __shared__ float red[ROWS_PER_BLOCK][3];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float l1 = gains[0], l2 = gains[1], l3 = skip ? gains[2] : 0.f;
+  float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  for (long row = (long)blockIdx.x * ROWS_PER_BLOCK + wave; row < nrows; row += (long)gridDim.x * ROWS_PER_BLOCK) {
+    Row<NCH> g, xn, t;
+    g.load(g_norm + row * C, C, lane);
+    xn.load(x_new + row * C, C, lane);
+    const float rs = inv[row];
+    float dot = row_dot(g, xn);
+    float coef = dot * rs * rs * (1.0f / C);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) g.v[i][k] = rs * (g.v[i][k] - xn.v[i][k] * coef);
+    if (g_new) {
+      t.load(g_new + row * C, C, lane);
+#pragma unroll
+      for (int i = 0; i < NCH; ++i)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) g.v[i][k] += t.v[i][k];
+    }
+    // g is G (fp32)
+    t.load(x + row * C, C, lane);
+    s1 += row_dot(g, t);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) t.v[i][k] = l1 * g.v[i][k];
+    t.store(dx + row * C, C, lane);
+    t.load(x0 + row * C, C, lane);
+    s2 += row_dot(g, t);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) t.v[i][k] = l2 * g.v[i][k];
+    t.store(dx0 + row * C, C, lane);
+    if (skip) {
+      t.load(skip + row * C, C, lane);
+      s3 += row_dot(g, t);
+#pragma unroll
+      for (int i = 0; i < NCH; ++i)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) t.v[i][k] = l3 * g.v[i][k];
+      t.store(dskip + row * C, C, lane);
+    }
+  }
+  if (lane == 0) {
+    red[wave][0] = s1;
+    red[wave][1] = s2;
+    red[wave][2] = s3;
+  }
+  __syncthreads();
+  if (threadIdx.x < 3) {
+    float t = 0.f;
+    for (int r = 0; r < ROWS_PER_BLOCK; ++r) t += red[r][threadIdx.x];
+    gain_part[(long)blockIdx.x * 4 + threadIdx.x] = t;
+  }
+  if (threadIdx.x == 3) gain_part[(long)blockIdx.x * 4 + 3] = 0.f;
+}
+
+inline int grid_for(long nrows, int cap) {
+  long b = (nrows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
+  return (int)(b < cap ? b : cap);
+}
+
+}  // namespace
+
+#define DISPATCH_NCH(C, CALL)            \
+  do {                                   \
+    if ((C) <= 512) { CALL(1); }         \
+    else if ((C) <= 1024) { CALL(2); }   \
+    else if ((C) <= 2048) { CALL(4); }   \
+    else { CALL(8); }                    \
+  } while (0)
+
+static bool norm_shape_ok(long nrows, int C) { return nrows > 0 && C > 0 && C % 8 == 0 && C <= 4096; }
+
+extern "C" int tfb_norm_bwd_blocks(long nrows) { return grid_for(nrows, 1024); }
+
+extern "C" int tfb_rmsnorm_fwd(const void* x, const void* res, const void* w, void* s_out, void* y, void* inv, long nrows,
+                               int C, float eps, void* stream) {
+  if (!x || !y) return TFB_ERR_ARG;
+  if (res && !s_out) return TFB_ERR_ARG;
+  if (!norm_shape_ok(nrows, C)) return TFB_ERR_SHAPE;
+  int grid = grid_for(nrows, 8192);
+#define CALL(N)                                                                                                       \
+  hipLaunchKernelGGL(rmsnorm_fwd_kernel<N>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x,          \
+                     (const bf16_t*)res, (const bf16_t*)w, (bf16_t*)s_out, (bf16_t*)y, (float*)inv, nrows, C, eps)
+  DISPATCH_NCH(C, CALL);
+#undef CALL
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// dw_part: fp32 [tfb_norm_bwd_blocks(nrows)][C] scratch (only when w != NULL); dw: fp32 [C].
+extern "C" int tfb_rmsnorm_bwd(const void* gy, const void* gs, const void* s, const void* w, const void* inv, void* dx,
+                               void* dw_part, void* dw, int dw_accumulate, long nrows, int C, void* stream) {
+  if (!gy || !s || !inv || !dx) return TFB_ERR_ARG;
+  if (w && (!dw_part || !dw)) return TFB_ERR_ARG;
+  if (!norm_shape_ok(nrows, C)) return TFB_ERR_SHAPE;
+  int grid = grid_for(nrows, 1024);
+#define CALL(N)                                                                                                        \
+  hipLaunchKernelGGL(rmsnorm_bwd_kernel<N>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)gy,          \
+                     (const bf16_t*)gs, (const bf16_t*)s, (const bf16_t*)w, (const float*)inv, (bf16_t*)dx,            \
+                     (float*)dw_part, nrows, C)
+  DISPATCH_NCH(C, CALL);
+#undef CALL
+  TFB_LAUNCH_CHECK();
+  if (w) {
+    hipLaunchKernelGGL(colsum_kernel, dim3((C + 255) / 256), dim3(256), 0, (hipStream_t)stream, (const float*)dw_part,
+                       (float*)dw, grid, C, dw_accumulate);
+    TFB_LAUNCH_CHECK();
+  }
+  return TFB_OK;
+}
+
+// gains: device fp32 [3] = l1, l2, l3 (l3 read only when skip != NULL)
+extern "C" int tfb_block_head_fwd(const void* x, const void* x0, const void* skip, const void* gains, void* x_new,
+                                  void* x_norm, void* inv, long nrows, int C, float eps, void* stream) {
+  if (!x || !x0 || !gains || !x_new || !x_norm || !inv) return TFB_ERR_ARG;
+  if (!norm_shape_ok(nrows, C)) return TFB_ERR_SHAPE;
+  int grid = grid_for(nrows, 8192);
+#define CALL(N)                                                                                                      \
+  hipLaunchKernelGGL(block_head_fwd_kernel<N>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x,      \
+                     (const bf16_t*)x0, (const bf16_t*)skip, (const float*)gains, (bf16_t*)x_new, (bf16_t*)x_norm,  \
+                     (float*)inv, nrows, C, eps)
+  DISPATCH_NCH(C, CALL);
+#undef CALL
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// gain_part: fp32 [tfb_norm_bwd_blocks(nrows)][4] scratch; dgains: fp32 [4] (sum G.x, G.x0, G.skip, 0)
+extern "C" int tfb_block_head_bwd(const void* g_new, const void* g_norm, const void* x, const void* x0, const void* skip,
+                                  const void* x_new, const void* inv, const void* gains, void* dx, void* dx0,
+                                  void* dskip, void* gain_part, void* dgains, long nrows, int C, void* stream) {
+  if (!g_norm || !x || !x0 || !x_new || !inv || !gains || !dx || !dx0 || !gain_part || !dgains) return TFB_ERR_ARG;
+  if (skip && !dskip) return TFB_ERR_ARG;
+  if (!norm_shape_ok(nrows, C)) return TFB_ERR_SHAPE;
+  int grid = grid_for(nrows, 1024);
+#define CALL(N)                                                                                                        \
+  hipLaunchKernelGGL(block_head_bwd_kernel<N>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)g_new,    \
+                     (const bf16_t*)g_norm, (const bf16_t*)x, (const bf16_t*)x0, (const bf16_t*)skip,                  \
+                     (const bf16_t*)x_new, (const float*)inv, (const float*)gains, (bf16_t*)dx, (bf16_t*)dx0,          \
+                     (bf16_t*)dskip, (float*)gain_part, nrows, C)
+  DISPATCH_NCH(C, CALL);
+#undef CALL
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(colsum_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const float*)gain_part, (float*)dgains,
+                     grid, 4, 0);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
