@@ -22,7 +22,18 @@ SIGNATURES = {
     "tfb_rmsnorm_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _l, _i, _vp],
     "tfb_block_head_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_block_head_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _vp],
+    "tfb_mlp8_scale_scratch_floats": [_i],
+    "tfb_mlp8_forward_scales": [_vp, _vp, _vp, _vp, _i, _i, _f, _f, _vp],
+    "tfb_mlp8_backward_scales": [_vp, _vp, _vp, _vp, _l, _i, _vp],
+    "tfb_amax_scale": [_vp, _l, _f, _i, _i, _vp, _vp, _vp],
+    "tfb_quant_fp8": [_vp, _vp, _f, _i, _vp, _l, _vp],
+    "tfb_mlp8_precast": [_vp, _vp, _vp, _vp, _i, _i, _vp],
+    "tfb_mlp8_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_mlp8_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_mlp_dw_proj": [_vp, _vp, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
 }
+
+_LONG_RESULT = {"tfb_mlp8_scale_scratch_floats"}
 
 STATUS = {0: "ok", 1: "unsupported shape", 2: "bad argument", 3: "kernel launch failed", 4: "workspace too small"}
 
@@ -46,7 +57,7 @@ def lib():
         for name, args in SIGNATURES.items():
             fn = getattr(L, name)  # AttributeError if the symbol is missing
             fn.argtypes = args
-            fn.restype = _i
+            fn.restype = _l if name in _LONG_RESULT else _i
         _LIB = L
     return _LIB
 

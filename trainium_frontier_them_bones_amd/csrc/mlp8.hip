@@ -1,0 +1,546 @@
+// fp8 fused MLP (up-projection -> ReLU^2 -> down-projection) for gfx950.
+//
+// Replaces _mlp8_fwd_kernel / _mlp8_bwd_kernel and their host helpers
+// (round2/source/kernels/nki_mlp_fused8.py:509, 571, 742-858) and the per-step weight pre-cast
+// (round2/source/kernels/nki_mlp_l4t.py:392, 948-970).
+//
+// MI355X design: the hidden activation of a 128-token block (128 x 3072 fp8 = 384 KB) does not
+// fit a CU's 160 KB LDS, so the two GEMMs are two launches and h lives in HBM as e4m3 bytes
+// (50 MB at 16384 x 3072: inside the 256 MB Infinity Cache between producer and consumer);
+// everything elementwise (descale, ReLU, the saved r, clamp, square, fp8 casts, the ReLU^2
+// backward) is fused into the GEMM epilogues, and weights are cast once per optimizer step into a
+// pack of four k-contiguous byte layouts so that all four activation GEMMs are NT fp8 GEMMs on
+// v_mfma_scale_f32_32x32x64_f8f6f4. Rounding points are the reference emulation's:
+//   x8 = e4m3(x * s_x); r = bf16(max(acc * dq_fc, 0)); rc = bf16(min(r * c_h, 15.375));
+//   h8 = e4m3(rc^2); y = bf16(acc * dq_proj); dy8 = e5m2(dy * s_dy);
+//   dpre = bf16((acc * dq_dh2) * r); dp8 = e5m2(dpre * s_dp); dx = bf16(acc * dq_dx).
+#include "gemm_core.hpp"
+
+// scale-row columns (nki_mlp_fused8.py:111-114)
+#define SC_S_WFC 0
+#define SC_DQ_FC 1
+#define SC_C_H 2
+#define SC_S_WPROJ 3
+#define SC_DQ_PROJ 4
+#define SC_S_DY 5
+#define SC_DQ_DH2 6
+#define SC_S_DP 7
+#define SC_DQ_DX 8
+#define SC_RHO2 9
+#define SC_KAPPA2 10
+#define SC_I_WFC 11
+#define SC_I_WPROJ 12
+#define SC_S_H 13
+#define SC_AMAX_WFC 14
+#define SC_AMAX_WPROJ 15
+#define NSC 16
+
+namespace {
+
+constexpr float H_CLAMP = 15.375f;
+
+// ------------------------------------------------------------------------------------ scale search
+// s = 2^e, largest e in [e_lo, e_hi] with v * s <= limit; comparisons and power-of-two products
+// only (nki_mlp_fused8.py:742-758), so s and 1/s are exact.
+__device__ void pow2_le(float v, float limit, int e_lo, int e_hi, float* s_out, float* inv_out) {
+  float s = ldexpf(1.0f, e_lo), inv = ldexpf(1.0f, -e_lo);
+  const float top = ldexpf(1.0f, e_hi);
+  const int span = e_hi - e_lo;
+  for (int b = 64; b >= 1; b >>= 1) {
+    if (b > span) continue;
+    float cand = s * ldexpf(1.0f, b);
+    bool ok = (v * cand <= limit) && (cand <= top);
+    if (ok) {
+      s = cand;
+      inv = inv * ldexpf(1.0f, -b);
+    }
+  }
+  *s_out = s;
+  *inv_out = inv;
+}
+
+// s = 4^e (nki_mlp_fused8.py:761-779); c = 2^e.
+__device__ void pow4_le(float v, float limit, int e_lo, int e_hi, float* s_out, float* inv_out, float* c_out) {
+  float s = ldexpf(1.0f, 2 * e_lo), inv = ldexpf(1.0f, -2 * e_lo), c = ldexpf(1.0f, e_lo);
+  const float top = ldexpf(1.0f, 2 * e_hi);
+  const int span = e_hi - e_lo;
+  for (int b = 32; b >= 1; b >>= 1) {
+    if (b > span) continue;
+    float cand = s * ldexpf(1.0f, 2 * b);
+    bool ok = (v * cand <= limit) && (cand <= top);
+    if (ok) {
+      s = cand;
+      inv = inv * ldexpf(1.0f, -2 * b);
+      c = c * ldexpf(1.0f, b);
+    }
+  }
+  *s_out = s;
+  *inv_out = inv;
+  *c_out = c;
+}
+
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float m = red[0];
+  for (int i = 1; i < (int)(blockDim.x >> 6); ++i) m = fmaxf(m, red[i]);
+  return m;
+}
+
+// ------------------------------------------------------------------------------------ statistics
+// amax over a bf16 tensor: per-workgroup partials.
+__global__ __launch_bounds__(256) void amax_partial_kernel(const bf16_t* __restrict__ x, long n, float* __restrict__ part) {
+  __shared__ float red[4];
+  float m = 0.f;
+  for (long i = ((long)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += (long)gridDim.x * 256 * 8) {
+    u32x4 u = *(const u32x4*)(x + i);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) m = fmaxf(m, fmaxf(fabsf(bflo(u[k])), fabsf(bfhi(u[k]))));
+  }
+  m = block_max(m, red);
+  if (threadIdx.x == 0) part[blockIdx.x] = m;
+}
+
+// One wavefront per row of w [rows][cols]: sum of squares per row; amax partial per workgroup.
+__global__ __launch_bounds__(256) void row_stats_kernel(const bf16_t* __restrict__ w, int rows, int cols,
+                                                       float* __restrict__ rowss, float* __restrict__ amax_part) {
+  __shared__ float red[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float m = 0.f;
+  for (int r = blockIdx.x * 4 + wave; r < rows; r += gridDim.x * 4) {
+    float ss = 0.f;
+    for (int c = lane * 8; c < cols; c += 512) {
+      u32x4 u = *(const u32x4*)(w + (long)r * cols + c);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float a = bflo(u[k]), b = bfhi(u[k]);
+        ss += a * a;
+        ss += b * b;
+        m = fmaxf(m, fmaxf(fabsf(a), fabsf(b)));
+      }
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) rowss[r] = ss;
+  }
+  m = block_max(m, red);
+  if (threadIdx.x == 0) amax_part[blockIdx.x] = m;
+}
+
+// Column sums of squares of w [rows][cols]: a workgroup owns 512 columns (64 lanes x 8), its 4
+// wavefronts take interleaved rows; amax partial per workgroup.
+__global__ __launch_bounds__(256) void col_stats_kernel(const bf16_t* __restrict__ w, int rows, int cols,
+                                                       float* __restrict__ colss, float* __restrict__ amax_part) {
+  __shared__ float red[4];
+  __shared__ float acc[4][512];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = blockIdx.x * 512 + lane * 8;
+  float ss[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  float m = 0.f;
+  if (c < cols) {
+    for (int r = wave; r < rows; r += 4) {
+      u32x4 u = *(const u32x4*)(w + (long)r * cols + c);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float a = bflo(u[k]), b = bfhi(u[k]);
+        ss[2 * k] += a * a;
+        ss[2 * k + 1] += b * b;
+        m = fmaxf(m, fmaxf(fabsf(a), fabsf(b)));
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 8; ++k) acc[wave][lane * 8 + k] = ss[k];
+  m = block_max(m, red);  // contains the barriers that publish acc
+  for (int i = threadIdx.x; i < 512; i += 256) {
+    int cc = blockIdx.x * 512 + i;
+    if (cc < cols) colss[cc] = acc[0][i] + acc[1][i] + acc[2][i] + acc[3][i];
+  }
+  if (threadIdx.x == 0) amax_part[blockIdx.x] = m;
+}
+
+__device__ float reduce_max_array(const float* a, int n, float* red) {
+  float m = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) m = fmaxf(m, a[i]);
+  return block_max(m, red);
+}
+
+// One workgroup: the forward scale row (nki_mlp_fused8.py:782-800).
+__global__ __launch_bounds__(256) void forward_scales_kernel(const float* rowss, int F, const float* amax_fc_part, int nfc,
+                                                            const float* colss, const float* amax_pj_part, int npj,
+                                                            float e4m3_limit, float h_bound, float inv_x_scale,
+                                                            float* row_out) {
+  __shared__ float red[4];
+  float rho2 = reduce_max_array(rowss, F, red);
+  float kappa2 = reduce_max_array(colss, F, red);
+  float amax_fc = reduce_max_array(amax_fc_part, nfc, red);
+  float amax_pj = reduce_max_array(amax_pj_part, npj, red);
+  if (threadIdx.x == 0) {
+    float s_wfc, i_wfc, s_wpj, i_wpj, s_h, i_h, c_h;
+    pow2_le(amax_fc, e4m3_limit, -24, 40, &s_wfc, &i_wfc);
+    pow2_le(amax_pj, e4m3_limit, -24, 40, &s_wpj, &i_wpj);
+    pow4_le(rho2 * h_bound, e4m3_limit, -16, 8, &s_h, &i_h, &c_h);
+    row_out[SC_S_WFC] = s_wfc;
+    row_out[SC_DQ_FC] = i_wfc * inv_x_scale;
+    row_out[SC_C_H] = c_h;
+    row_out[SC_S_WPROJ] = s_wpj;
+    row_out[SC_DQ_PROJ] = i_h * i_wpj;
+    row_out[SC_S_DY] = 0.f;
+    row_out[SC_DQ_DH2] = 0.f;
+    row_out[SC_S_DP] = 0.f;
+    row_out[SC_DQ_DX] = 0.f;
+    row_out[SC_RHO2] = rho2;
+    row_out[SC_KAPPA2] = kappa2;
+    row_out[SC_I_WFC] = i_wfc;
+    row_out[SC_I_WPROJ] = i_wpj;
+    row_out[SC_S_H] = s_h;
+    row_out[SC_AMAX_WFC] = amax_fc;
+    row_out[SC_AMAX_WPROJ] = amax_pj;
+  }
+}
+
+// One workgroup: the backward call's row from amax(dy) (nki_mlp_fused8.py:803-813).
+__global__ __launch_bounds__(256) void backward_scales_kernel(const float* amax_part, int npart, const float* row_in,
+                                                             float dp_factor, float* row_out) {
+  __shared__ float red[4];
+  float amax_dy = reduce_max_array(amax_part, npart, red);
+  if (threadIdx.x < NSC) row_out[threadIdx.x] = row_in[threadIdx.x];
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s_dy, i_dy, s_dp, i_dp;
+    pow2_le(amax_dy, TFB_E5M2_MAX / 2.0f, -40, 60, &s_dy, &i_dy);
+    float bound = sqrtf(row_in[SC_RHO2] * row_in[SC_KAPPA2]) * amax_dy * dp_factor;
+    pow2_le(bound, TFB_E5M2_MAX, -40, 60, &s_dp, &i_dp);
+    row_out[SC_S_DY] = s_dy;
+    row_out[SC_DQ_DH2] = i_dy * row_in[SC_I_WPROJ] * 2.0f;
+    row_out[SC_S_DP] = s_dp;
+    row_out[SC_DQ_DX] = i_dp * row_in[SC_I_WFC];
+  }
+}
+
+// One workgroup: out[0] = s = 2^e (largest with amax * s <= limit), out[1] = 1/s.
+__global__ __launch_bounds__(256) void amax_scale_kernel(const float* amax_part, int npart, float limit, int e_lo, int e_hi,
+                                                        float* out) {
+  __shared__ float red[4];
+  float amax = reduce_max_array(amax_part, npart, red);
+  if (threadIdx.x == 0) {
+    float s, inv;
+    pow2_le(amax, limit, e_lo, e_hi, &s, &inv);
+    out[0] = s;
+    out[1] = inv;
+    out[2] = amax;
+  }
+}
+
+// ------------------------------------------------------------------------------------ casts
+template <int FMT>
+__global__ __launch_bounds__(256) void quant_kernel(const bf16_t* __restrict__ x, const float* __restrict__ scale_ptr,
+                                                   float scale_imm, uint8_t* __restrict__ out, long n) {
+  const float s = scale_ptr ? *scale_ptr : scale_imm;
+  for (long i = ((long)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += (long)gridDim.x * 256 * 8) {
+    u32x4 u = *(const u32x4*)(x + i);
+    u32x2 o;
+    o.x = cvt4_fp8<FMT>(bflo(u[0]) * s, bfhi(u[0]) * s, bflo(u[1]) * s, bfhi(u[1]) * s);
+    o.y = cvt4_fp8<FMT>(bflo(u[2]) * s, bfhi(u[2]) * s, bflo(u[3]) * s, bfhi(u[3]) * s);
+    *(u32x2*)(out + i) = o;
+  }
+}
+
+// w [R][C] bf16 -> out [R][C] e4m3 and outT [C][R] e4m3, 64 x 64 tiles through LDS.
+__global__ __launch_bounds__(256) void precast_kernel(const bf16_t* __restrict__ w, const float* __restrict__ scale_ptr,
+                                                     uint8_t* __restrict__ out, uint8_t* __restrict__ outT, int R, int C) {
+  __shared__ uint8_t t[64][80];
+  const float s = *scale_ptr;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    int ch = threadIdx.x + i * 256;  // 512 chunks of 8 elements
+    int r = ch >> 3, cc = (ch & 7) * 8;
+    u32x4 u = *(const u32x4*)(w + (long)(r0 + r) * C + c0 + cc);
+    u32x2 o;
+    o.x = cvt4_fp8<TFB_FMT_E4M3>(bflo(u[0]) * s, bfhi(u[0]) * s, bflo(u[1]) * s, bfhi(u[1]) * s);
+    o.y = cvt4_fp8<TFB_FMT_E4M3>(bflo(u[2]) * s, bfhi(u[2]) * s, bflo(u[3]) * s, bfhi(u[3]) * s);
+    *(u32x2*)(out + (long)(r0 + r) * C + c0 + cc) = o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      t[cc + k][r] = (uint8_t)(o.x >> (8 * k));
+      t[cc + 4 + k][r] = (uint8_t)(o.y >> (8 * k));
+    }
+  }
+  __syncthreads();
+  {
+    int c = threadIdx.x >> 2, j = (threadIdx.x & 3) * 16;
+    u32x4 v = *(const u32x4*)(&t[c][j]);
+    *(u32x4*)(outT + (long)(c0 + c) * R + r0 + j) = v;
+  }
+}
+
+// ------------------------------------------------------------------------------------ GEMM epilogues
+// All activation GEMMs: P side = the weight pack layout whose rows are the output's contiguous
+// dimension, Q side = the token-major fp8 activation. p = output column (4 consecutive), q = token.
+
+struct EpiUp {  // pre = x8 @ wf8^T: r, h8
+  const float* sc;
+  bf16_t* r;     // [M][F]
+  uint8_t* h8;   // [M][F]
+  long F;
+  __device__ __forceinline__ void operator()(int p, int q, f32x4 v, int) const {
+    const float dq = sc[SC_DQ_FC], c = sc[SC_C_H];
+    float rr[4], hh[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      rr[i] = round_bf(fmaxf(v[i] * dq, 0.f));
+      float rc = round_bf(fminf(rr[i] * c, H_CLAMP));
+      hh[i] = rc * rc;
+    }
+    u32x2 o = {pack2bf(rr[0], rr[1]), pack2bf(rr[2], rr[3])};
+    *(u32x2*)(r + (long)q * F + p) = o;
+    *(uint32_t*)(h8 + (long)q * F + p) = cvt4_fp8<TFB_FMT_E4M3>(hh[0], hh[1], hh[2], hh[3]);
+  }
+};
+
+struct EpiScaleStore {  // out = bf16(acc * sc[col])
+  const float* sc;
+  int col;
+  bf16_t* out;
+  long ld;
+  __device__ __forceinline__ void operator()(int p, int q, f32x4 v, int) const {
+    const float dq = sc[col];
+    u32x2 o = {pack2bf(v[0] * dq, v[1] * dq), pack2bf(v[2] * dq, v[3] * dq)};
+    *(u32x2*)(out + (long)q * ld + p) = o;
+  }
+};
+
+struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*s_dp), optional h = bf16(r^2)
+  const float* sc;
+  const bf16_t* r;  // [M][F]
+  bf16_t* dpre;     // [M][F]
+  uint8_t* dp8;     // [M][F]
+  bf16_t* h;        // [M][F] or null
+  long F;
+  __device__ __forceinline__ void operator()(int p, int q, f32x4 v, int) const {
+    const float dq = sc[SC_DQ_DH2], sdp = sc[SC_S_DP];
+    const long off = (long)q * F + p;
+    u32x2 ru = *(const u32x2*)(r + off);
+    float rr[4] = {bflo(ru.x), bfhi(ru.x), bflo(ru.y), bfhi(ru.y)};
+    float dp[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dp[i] = round_bf((v[i] * dq) * rr[i]);
+    u32x2 o = {pack2bf(dp[0], dp[1]), pack2bf(dp[2], dp[3])};
+    *(u32x2*)(dpre + off) = o;
+    *(uint32_t*)(dp8 + off) = cvt4_fp8<TFB_FMT_E5M2>(dp[0] * sdp, dp[1] * sdp, dp[2] * sdp, dp[3] * sdp);
+    if (h) {
+      u32x2 ho = {pack2bf(rr[0] * rr[0], rr[1] * rr[1]), pack2bf(rr[2] * rr[2], rr[3] * rr[3])};
+      *(u32x2*)(h + off) = ho;
+    }
+  }
+};
+
+// h = bf16(r^2) applied to the 8 bf16 of a 128-bit load (the dW_proj GEMM reads r, not h).
+struct LoadSquare {
+  __device__ __forceinline__ u32x4 operator()(u32x4 v) const {
+    u32x4 o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float a = bflo(v[k]), b = bfhi(v[k]);
+      o[k] = pack2bf(a * a, b * b);
+    }
+    return o;
+  }
+};
+
+struct EpiSplitF32 {
+  float* ws;
+  long ld, slab;
+  __device__ __forceinline__ void operator()(int p, int q, f32x4 v, int split) const {
+    *(f32x4*)(ws + (long)split * slab + (long)q * ld + p) = v;
+  }
+};
+
+__global__ void reduce_store_kernel(const float* __restrict__ ws, void* out, long n, int splits, int f32, int accumulate) {
+  long i = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i >= n) return;
+  f32x4 s = *(const f32x4*)(ws + i);
+  for (int k = 1; k < splits; ++k) s += *(const f32x4*)(ws + (long)k * n + i);
+  if (f32) {
+    float* o = (float*)out + i;
+    if (accumulate) s += *(const f32x4*)o;
+    *(f32x4*)o = s;
+  } else {
+    bf16_t* o = (bf16_t*)out + i;
+    if (accumulate) {
+      u32x2 c = *(const u32x2*)o;
+      s[0] += bflo(c.x);
+      s[1] += bfhi(c.x);
+      s[2] += bflo(c.y);
+      s[3] += bfhi(c.y);
+    }
+    u32x2 r = {pack2bf(s[0], s[1]), pack2bf(s[2], s[3])};
+    *(u32x2*)o = r;
+  }
+}
+
+inline bool shapes8(long M, int d, int F) { return M > 0 && M % 128 == 0 && d > 0 && d % 256 == 0 && F > 0 && F % 256 == 0; }
+
+template <int FMT>
+int launch_quant(const void* x, const float* sp, float si, void* out, long n, hipStream_t s) {
+  if (n % 8) return TFB_ERR_SHAPE;
+  long blocks = (n / 8 + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(quant_kernel<FMT>, dim3((unsigned)blocks), dim3(256), 0, s, (const bf16_t*)x, sp, si, (uint8_t*)out, n);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+constexpr int AMAX_BLOCKS = 1024;
+
+}  // namespace
+
+// Scratch the scale kernels need (fp32 elements): partial maxima and the per-row / per-column norms.
+extern "C" long tfb_mlp8_scale_scratch_floats(int F) { return 2L * F + 4L * AMAX_BLOCKS; }
+
+// row_out: fp32 [16] device. e4m3_limit: 240 reproduces the reference's rows; 448 is the OCP maximum.
+extern "C" int tfb_mlp8_forward_scales(const void* w_fc, const void* w_proj, void* row_out, void* scratch, int F, int d,
+                                       float e4m3_limit, float x_scale, void* stream) {
+  if (!w_fc || !w_proj || !row_out || !scratch) return TFB_ERR_ARG;
+  if (F <= 0 || d <= 0 || F % 8 || d % 8) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  float* rowss = (float*)scratch;
+  float* colss = rowss + F;
+  float* pa = colss + F;
+  float* pb = pa + AMAX_BLOCKS;
+  int nfc = (F + 3) / 4;
+  if (nfc > AMAX_BLOCKS) nfc = AMAX_BLOCKS;
+  int npj = (F + 511) / 512;
+  hipLaunchKernelGGL(row_stats_kernel, dim3(nfc), dim3(256), 0, s, (const bf16_t*)w_fc, F, d, rowss, pa);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(col_stats_kernel, dim3(npj), dim3(256), 0, s, (const bf16_t*)w_proj, d, F, colss, pb);
+  TFB_LAUNCH_CHECK();
+  const float h_bound = (float)(1.3 * (double)d);
+  hipLaunchKernelGGL(forward_scales_kernel, dim3(1), dim3(256), 0, s, rowss, F, pa, nfc, colss, pb, npj, e4m3_limit, h_bound,
+                     (float)(1.0 / (double)x_scale), (float*)row_out);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+extern "C" int tfb_mlp8_backward_scales(const void* dy, const void* row_in, void* row_out, void* scratch, long M, int d,
+                                        void* stream) {
+  if (!dy || !row_in || !row_out || !scratch) return TFB_ERR_ARG;
+  long n = M * d;
+  if (n <= 0 || n % 8) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  long blocks = (n / 8 + 255) / 256;
+  if (blocks > AMAX_BLOCKS) blocks = AMAX_BLOCKS;
+  hipLaunchKernelGGL(amax_partial_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (const bf16_t*)dy, n, (float*)scratch);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(backward_scales_kernel, dim3(1), dim3(256), 0, s, (const float*)scratch, (int)blocks,
+                     (const float*)row_in, (float)(36.16 * (double)d), (float*)row_out);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// out: fp32 [3] device = {s, 1/s, amax}: per-tensor power-of-two scale from the exact amax.
+extern "C" int tfb_amax_scale(const void* x, long n, float limit, int e_lo, int e_hi, void* out, void* scratch,
+                              void* stream) {
+  if (!x || !out || !scratch) return TFB_ERR_ARG;
+  if (n <= 0 || n % 8) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  long blocks = (n / 8 + 255) / 256;
+  if (blocks > AMAX_BLOCKS) blocks = AMAX_BLOCKS;
+  hipLaunchKernelGGL(amax_partial_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (const bf16_t*)x, n, (float*)scratch);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(amax_scale_kernel, dim3(1), dim3(256), 0, s, (const float*)scratch, (int)blocks, limit, e_lo, e_hi,
+                     (float*)out);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// out8 = fp8(x * scale): scale from device memory (scale_ptr) or immediate. fmt 0 = e4m3, 1 = e5m2.
+extern "C" int tfb_quant_fp8(const void* x, const void* scale_ptr, float scale_imm, int fmt, void* out8, long n,
+                             void* stream) {
+  if (!x || !out8) return TFB_ERR_ARG;
+  if (n <= 0) return TFB_ERR_SHAPE;
+  if (fmt == TFB_FMT_E4M3) return launch_quant<TFB_FMT_E4M3>(x, (const float*)scale_ptr, scale_imm, out8, n, (hipStream_t)stream);
+  if (fmt == TFB_FMT_E5M2) return launch_quant<TFB_FMT_E5M2>(x, (const float*)scale_ptr, scale_imm, out8, n, (hipStream_t)stream);
+  return TFB_ERR_ARG;
+}
+
+// w8: uint8 [4][F*d] = wf8 [F][d], wf8T [d][F], wp8 [d][F], wp8T [F][d] (all e4m3, scaled by the row's s_w).
+extern "C" int tfb_mlp8_precast(const void* w_fc, const void* w_proj, const void* row, void* w8, int F, int d, void* stream) {
+  if (!w_fc || !w_proj || !row || !w8) return TFB_ERR_ARG;
+  if (F <= 0 || d <= 0 || F % 64 || d % 64) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  uint8_t* b = (uint8_t*)w8;
+  const long n = (long)F * d;
+  hipLaunchKernelGGL(precast_kernel, dim3(d / 64, F / 64), dim3(256), 0, s, (const bf16_t*)w_fc,
+                     (const float*)row + SC_S_WFC, b, b + n, F, d);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(precast_kernel, dim3(F / 64, d / 64), dim3(256), 0, s, (const bf16_t*)w_proj,
+                     (const float*)row + SC_S_WPROJ, b + 2 * n, b + 3 * n, d, F);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+using Cfg8 = GemmCfg<128, 128, 2, 2, 1, TFB_K_CONTIG, TFB_K_CONTIG, TFB_FMT_E4M3, TFB_FMT_E4M3>;
+using Cfg8g = GemmCfg<128, 128, 2, 2, 1, TFB_K_CONTIG, TFB_K_CONTIG, TFB_FMT_E4M3, TFB_FMT_E5M2>;
+
+// Forward: x8 [M][d] e4m3 (already cast at s_x), w8 pack, row -> y [M][d] bf16, r [M][F] bf16, h8 [M][F] e4m3 scratch.
+extern "C" int tfb_mlp8_fwd(const void* x8, const void* w8, const void* row, void* y, void* r, void* h8, long M, int d, int F,
+                            void* stream) {
+  if (!x8 || !w8 || !row || !y || !r || !h8) return TFB_ERR_ARG;
+  if (!shapes8(M, d, F)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const uint8_t* b = (const uint8_t*)w8;
+  const long n = (long)F * d;
+  GemmOperand Pw{b, (long)d}, Qx{(const uint8_t*)x8, (long)d};
+  EpiUp e1{(const float*)row, (bf16_t*)r, (uint8_t*)h8, (long)F};
+  int st = gemm_launch<Cfg8>(Pw, Qx, F, (int)M, (long)d, 1, LoadIdentity{}, LoadIdentity{}, e1, s);
+  if (st != TFB_OK) return st;
+  GemmOperand Pp{b + 2 * n, (long)F}, Qh{(const uint8_t*)h8, (long)F};
+  EpiScaleStore e2{(const float*)row, SC_DQ_PROJ, (bf16_t*)y, (long)d};
+  return gemm_launch<Cfg8>(Pp, Qh, d, (int)M, (long)F, 1, LoadIdentity{}, LoadIdentity{}, e2, s);
+}
+
+// Backward: dy8 [M][d] e5m2 (cast at the row's s_dy), r [M][F] -> dx [M][d], dpre [M][F] bf16, h [M][F] bf16 (optional,
+// may be NULL), dp8 [M][F] e5m2 scratch.
+extern "C" int tfb_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* row, void* dx, void* h, void* dpre,
+                            void* dp8, long M, int d, int F, void* stream) {
+  if (!dy8 || !r || !w8 || !row || !dx || !dpre || !dp8) return TFB_ERR_ARG;
+  if (!shapes8(M, d, F)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const uint8_t* b = (const uint8_t*)w8;
+  const long n = (long)F * d;
+  GemmOperand Pw{b + 3 * n, (long)d}, Qg{(const uint8_t*)dy8, (long)d};  // wp8T [F][d]
+  EpiDh e1{(const float*)row, (const bf16_t*)r, (bf16_t*)dpre, (uint8_t*)dp8, (bf16_t*)h, (long)F};
+  int st = gemm_launch<Cfg8g>(Pw, Qg, F, (int)M, (long)d, 1, LoadIdentity{}, LoadIdentity{}, e1, s);
+  if (st != TFB_OK) return st;
+  GemmOperand Pf{b + n, (long)F}, Qd{(const uint8_t*)dp8, (long)F};  // wf8T [d][F]
+  EpiScaleStore e2{(const float*)row, SC_DQ_DX, (bf16_t*)dx, (long)d};
+  return gemm_launch<Cfg8g>(Pf, Qd, d, (int)M, (long)F, 1, LoadIdentity{}, LoadIdentity{}, e2, s);
+}
+
+// dW_proj [d][F] (+)= dy^T @ bf16(r^2): the token-contraction GEMM with the square applied while r is staged, so h
+// is never written. out bf16 or fp32; workspace fp32 for split-K (tokens are the long dimension).
+extern "C" int tfb_mlp_dw_proj(const void* dy, const void* r, void* dw, long M, int d, int F, int out_f32, int accumulate,
+                               void* workspace, long workspace_bytes, void* stream) {
+  if (!dy || !r || !dw) return TFB_ERR_ARG;
+  if (M <= 0 || M % 64 || d % 128 || F % 128) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  using Cfg = GemmCfg<128, 128, 2, 2, 2, TFB_K_STRIDED, TFB_K_STRIDED>;
+  GemmOperand P{(const uint8_t*)r, (long)F * 2}, Q{(const uint8_t*)dy, (long)d * 2};
+  const int nkt = (int)(M / 64);
+  const long tiles = (long)(F / 128) * (d / 128);
+  int splits = (int)((768 + tiles - 1) / tiles);
+  while (splits > 1 && (nkt % splits != 0 || nkt / splits < 8)) --splits;
+  if (!workspace || (long)splits * d * F * 4 > workspace_bytes) return TFB_ERR_WORKSPACE;
+  EpiSplitF32 e{(float*)workspace, (long)F, (long)d * F};
+  int st = gemm_launch<Cfg>(P, Q, F, d, M * 2, splits, LoadSquare{}, LoadIdentity{}, e, s);
+  if (st != TFB_OK) return st;
+  long nn = (long)d * F;
+  hipLaunchKernelGGL(reduce_store_kernel, dim3((unsigned)((nn / 4 + 255) / 256)), dim3(256), 0, s, (const float*)workspace, dw,
+                     nn, splits, out_f32, accumulate);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
