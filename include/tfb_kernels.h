@@ -1,0 +1,177 @@
+/* C-ABI of libtfb_hip.so: hand-written HIP kernels for gfx950 (MI355X) that replace the NKI kernels on the
+ * training-step hot path of Danishlynx/trainium-frontier-them-bones.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the comment says "host"; bf16 tensors are raw 16-bit words,
+ *     fp8 tensors raw bytes (OCP e4m3fn / e5m2), row-major, contiguous unless strides are passed;
+ *   - `stream` is a hipStream_t; kernels are launched on it and the call returns without synchronising;
+ *   - no entry point allocates, frees or synchronises; scratch and workspaces are caller-owned;
+ *   - return value: 0 ok, 1 unsupported shape (the reference wrappers' "shapes_apply() is false": the caller runs
+ *     its own fallback or raises), 2 bad argument, 3 launch failed, 4 workspace too small.
+ *
+ * Each declaration cites the reference interface it replaces (paths relative to the reference repository).
+ */
+#ifndef TFB_KERNELS_H
+#define TFB_KERNELS_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- bf16 GEMM ------------------------------------------------------------------------------------------------
+ * C[M,N] (+)= op(A) @ op(B); A is [M,K] (trans_a=0) or [K,M]; B is [K,N] (trans_b=0) or [N,K]; fp32 accumulation;
+ * C bf16 (out_f32=0) or fp32; accumulate=1 adds into C (one rounding). M, N multiples of 128, K of 64.
+ * workspace: optional fp32 split-K scratch (used when the output has few tiles and K is long).
+ * Replaces nki_matmul(a, b, trans_a, trans_b): round1/source/train.py:1137 (kernels 926, 1052) and the in-place
+ * weight-gradient accumulate of round1/source/train.py:8463-8509. */
+int tfb_gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int trans_a, int trans_b, int out_f32,
+                  int accumulate, void* workspace, long workspace_bytes, void* stream);
+
+/* ---- RMSNorm family --------------------------------------------------------------------------------------------
+ * Number of partial-sum rows the backward kernels write for `nrows` rows (host helper, no GPU work). */
+int tfb_norm_bwd_blocks(long nrows);
+
+/* s = x (res NULL) or bf16(x + res) written to s_out; y = bf16(s * rsqrt(mean(s^2) + eps) * w) (w NULL = no weight);
+ * inv fp32 [nrows] = the rsqrt factor. C multiple of 8, <= 4096.
+ * Replaces rmsnorm_fast (round1/source/train.py:5594, kernels 5378), tail_norm2 (6117, kernel 5887), final_norm
+ * (6826) and nf_norm_rows (round2/source/train.py:8805). */
+int tfb_rmsnorm_fwd(const void* x, const void* res, const void* w, void* s_out, void* y, void* inv, long nrows, int C,
+                    float eps, void* stream);
+
+/* dx = gs + inv * (gh - s * (gh . s) * inv^2 / C), gh = gy * w; dw fp32 [C] (+)= sum_rows gy * s * inv.
+ * dw_part: fp32 [tfb_norm_bwd_blocks(nrows)][C] scratch (needed only with w).
+ * Replaces _rms_bwd_kernel / _tail_bwd (round1/source/train.py:5410, 5927) and nf_norm_backward
+ * (round2/source/train.py:8813-8825). */
+int tfb_rmsnorm_bwd(const void* gy, const void* gs, const void* s, const void* w, const void* inv, void* dx, void* dw_part,
+                    void* dw, int dw_accumulate, long nrows, int C, void* stream);
+
+/* x_new = bf16(l1 x + l2 x0 [+ l3 skip]); x_norm = RMSNorm(x_new); gains = fp32 [3] device (l1, l2, l3).
+ * Replaces block_head (round1/source/train.py:5578, kernel 5257) and head_skip (6106, kernel 5743). */
+int tfb_block_head_fwd(const void* x, const void* x0, const void* skip, const void* gains, void* x_new, void* x_norm,
+                       void* inv, long nrows, int C, float eps, void* stream);
+
+/* G = g_new + J^T(g_norm); dx = l1 G, dx0 = l2 G, dskip = l3 G; dgains fp32 [4] = (sum G.x, sum G.x0, sum G.skip, 0).
+ * gain_part: fp32 [tfb_norm_bwd_blocks(nrows)][4] scratch.
+ * Replaces _bh_bwd_kernel / _hs_bwd (round1/source/train.py:5301, 5793). */
+int tfb_block_head_bwd(const void* g_new, const void* g_norm, const void* x, const void* x0, const void* skip,
+                       const void* x_new, const void* inv, const void* gains, void* dx, void* dx0, void* dskip,
+                       void* gain_part, void* dgains, long nrows, int C, void* stream);
+
+/* ---- elementwise ------------------------------------------------------------------------------------------------
+ * mode 0: out = relu(a)^2; mode 1: out = b * 2 relu(a) (a = x, b = gy); mode 2: out = bf16(sqrt(4 a)) * b (a = h).
+ * Replaces relu_squared / relu2_backward / relu2_backward_from_h (round1/source/train.py:663, 597, 633). */
+int tfb_relu2(const void* a, const void* b, void* out, long n, int mode, void* stream);
+
+/* Half-split rotation of `nheads` heads of D columns at the start of each row (row r = token r % T); cos/sin bf16
+ * [T][D/2]; inverse=1 applies the transpose rotation (the backward). In place when out == x.
+ * Replaces the RoPE step of round1/source/train.py:4188-4193 (rope_norm 4447 without its QK-norm). */
+int tfb_rope(const void* x, const void* cos_t, const void* sin_t, void* out, long rows, int T, int nheads, int D,
+             long row_stride, long out_stride, int inverse, void* stream);
+
+int tfb_resmix_bwd_blocks(long n);
+/* dx = g bf16(a), dx0 = g bf16(b), dab fp32 [2] = (sum bf16(g x), sum bf16(g x0)); ab fp32 [2] device;
+ * part: fp32 [2 * tfb_resmix_bwd_blocks(n)] scratch.
+ * Replaces _resmix_bwd_kernel (round2/source/kernels/nki_resmix.py; emulate :148-162). */
+int tfb_resmix_bwd(const void* g, const void* x, const void* x0, const void* ab, void* dx, void* dx0, void* part, void* dab,
+                   long n, void* stream);
+
+/* out[i] = w[idx[i]] rows; idx int64 (idx64=1) or int32. Replaces embedding_fwd (round1/source/train.py:8407). */
+int tfb_embedding_fwd(const void* idx, int idx64, const void* w, void* out, long n, int C, void* stream);
+/* dw_f32[idx[i]] += dy[i] (fp32 atomics). Replaces _emb_bwd_kernel (round1/source/train.py:8303). */
+int tfb_embedding_bwd(const void* idx, int idx64, const void* dy, void* dw_f32, long n, int C, void* stream);
+
+/* One AdamW update in place on fp32 p, m, v from g (fp32 if g_f32 else bf16); optional bf16 copy of p.
+ * p *= 1 - lr wd; m = lerp(m, g, 1-b1); v = lerp(v, g^2, 1-b2); p -= lr (m / bias1) / (sqrt(v / bias2) + eps).
+ * Replaces adamw_fused_step (round1/source/train.py:1573, kernel 1410; math 9670-9677). */
+int tfb_adamw(void* p, const void* g, int g_f32, void* m, void* v, void* p_bf16, long n, float lr, float wd,
+              float one_minus_beta1, float one_minus_beta2, float eps, float bias1, float bias2, void* stream);
+
+/* p[0..n) = val with a kernel (safe inside HIP graph capture, unlike a memset node). No reference counterpart. */
+int tfb_fill_f32(void* p, float val, long n, void* stream);
+
+/* ---- fp8 fused MLP ------------------------------------------------------------------------------------------------
+ * fp32 scratch elements tfb_mlp8_forward_scales needs (host helper). */
+long tfb_mlp8_scale_scratch_floats(int F);
+
+/* row_out fp32 [16] = the layer's scale row from w_fc [F][d], w_proj [d][F] (bf16): columns s_wfc, dq_fc, c_h, s_wproj,
+ * dq_proj, s_dy, dq_dh2, s_dp, dq_dx, rho2, kappa2, i_wfc, i_wproj, s_h, amax_wfc, amax_wproj.
+ * Replaces forward_scales (round2/source/kernels/nki_mlp_fused8.py:782-800) and the statistics kernels of
+ * round2/source/kernels/nki_scstat.py. e4m3_limit 240 gives the reference's rows. */
+int tfb_mlp8_forward_scales(const void* w_fc, const void* w_proj, void* row_out, void* scratch, int F, int d,
+                            float e4m3_limit, float x_scale, void* stream);
+
+/* row_out = row_in with s_dy, dq_dh2, s_dp, dq_dx filled from amax(dy); scratch fp32 [1024].
+ * Replaces backward_scales (nki_mlp_fused8.py:803-813). */
+int tfb_mlp8_backward_scales(const void* dy, const void* row_in, void* row_out, void* scratch, long M, int d, void* stream);
+
+/* out fp32 [3] = (s, 1/s, amax): s = 2^e the largest with amax(x) s <= limit, e in [e_lo, e_hi]; scratch fp32 [1024].
+ * The reference's _pow2_le (nki_mlp_fused8.py:742) applied to a tensor's amax. */
+int tfb_amax_scale(const void* x, long n, float limit, int e_lo, int e_hi, void* out, void* scratch, void* stream);
+
+/* out8 = fp8(x * scale): scale read from scale_ptr (device fp32) when non-NULL, else scale_imm. fmt 0 e4m3, 1 e5m2.
+ * The reference's q8 (nki_mlp_fused8.py:821-825) producing bytes. */
+int tfb_quant_fp8(const void* x, const void* scale_ptr, float scale_imm, int fmt, void* out8, long n, void* stream);
+
+/* w8 uint8 [4][F*d] = e4m3(w_fc s_wfc) as [F][d] and [d][F], e4m3(w_proj s_wproj) as [d][F] and [F][d].
+ * Replaces _precast8_kernel / precast_ref (round2/source/kernels/nki_mlp_l4t.py:392, 948-970). */
+int tfb_mlp8_precast(const void* w_fc, const void* w_proj, const void* row, void* w8, int F, int d, void* stream);
+
+/* Forward from x8 = e4m3(x s_x) [M][d]: y bf16 [M][d], r bf16 [M][F] (saved for backward), h8 [M][F] byte scratch.
+ * M % 128 == 0, d % 256 == 0, F % 256 == 0 (the reference's shapes_apply8, nki_mlp_fused8.py:666).
+ * Replaces _mlp8_fwd_kernel / _mlp8_fwd_pc_kernel (nki_mlp_fused8.py:509, nki_mlp_l4t.py:434); op s2mlp8::fwd
+ * (round2/source/train.py:6858). r is token-major [M][F] (the reference returns its transpose rT [F][M]). */
+int tfb_mlp8_fwd(const void* x8, const void* w8, const void* row, void* y, void* r, void* h8, long M, int d, int F,
+                 void* stream);
+
+/* Backward from dy8 = e5m2(dy s_dy) [M][d]: dx bf16 [M][d], dpre bf16 [M][F], h = bf16(r^2) [M][F] (NULL to skip),
+ * dp8 [M][F] byte scratch. row = the backward row.
+ * Replaces _mlp8_bwd_kernel / _mlp8_bwd_pc_kernel (nki_mlp_fused8.py:571, nki_mlp_l4t.py:496); op s2mlp8::bwd
+ * (round2/source/train.py:6868), dw_mode "token" layout. */
+int tfb_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* row, void* dx, void* h, void* dpre, void* dp8,
+                 long M, int d, int F, void* stream);
+
+/* dw [d][F] (+)= dy^T @ bf16(r^2) (bf16 GEMM over the tokens, h never materialised). workspace fp32 split-K scratch.
+ * Replaces the dw_proj half of weight_grads (nki_mlp_fused8.py:706-711) / l4_weight_grads (nki_mlp_l4t.py:932). */
+int tfb_mlp_dw_proj(const void* dy, const void* r, void* dw, long M, int d, int F, int out_f32, int accumulate,
+                    void* workspace, long workspace_bytes, void* stream);
+
+/* ---- attention ----------------------------------------------------------------------------------------------------
+ * Causal flash attention, bf16. Every tensor comes with host long[3] element strides (batch, head, token); head dim
+ * contiguous; so q/k/v can be [B,H,T,D], [B,T,H,D] or thirds of a fused [B,T,3C] projection. lse fp32 [B*H][T].
+ * T % 128 == 0, D == 64.
+ * Replaces _attn_fwd_kernel behind nki_causal_attention (round1/source/train.py:7536, 8069;
+ * round2/source/kernels/nki_attn_bandpro.py:1850); op s2attn::*_fwd (round2/source/train.py:4988). */
+int tfb_attn_fwd(const void* q, const long* q_strides, const void* k, const long* k_strides, const void* v,
+                 const long* v_strides, void* o, const long* o_strides, void* lse, int B, int H, int T, int D, float scale,
+                 void* stream);
+
+/* dq, dk, dv from (q, k, v, o, do, lse); delta fp32 [B*H][T] scratch.
+ * Replaces _attn_bwd_kernel / NkiAttnFn.backward (round1/source/train.py:7591, 8036). */
+int tfb_attn_bwd(const void* q, const long* q_strides, const void* k, const long* k_strides, const void* v,
+                 const long* v_strides, const void* o, const long* o_strides, const void* d_o, const long* do_strides,
+                 void* dq, const long* dq_strides, void* dk, const long* dk_strides, void* dv, const long* dv_strides,
+                 const void* lse, void* delta, int B, int H, int T, int D, float scale, void* stream);
+
+/* ---- loss head ------------------------------------------------------------------------------------------------------
+ * loss[row] = row_w[row] * (lse - s_target), lse[row] = log sum exp(s), s = softcap tanh(x / softcap) (softcap <= 0:
+ * s = x); target < 0 = ignored row (loss 0). logits bf16 [rows][V]; targets int64 (idx64) or int32.
+ * Replaces _loss_fwd_kernel behind fused_loss (round1/source/train.py:4543, 4691) and _lh_fwd_kernel
+ * (round2/source/train.py:5238; host chunked_loss_mean 6364). */
+int tfb_loss_fwd(const void* logits, const void* targets, int idx64, const void* row_w, void* loss, void* lse, long rows,
+                 int V, float softcap, void* stream);
+
+/* dlogits = grow[row] (softmax - onehot) (1 - tanh^2), bf16; may alias logits.
+ * Replaces _loss_bwd_kernel (round1/source/train.py:4584) / _lh_bwd_kernel (round2/source/train.py:5297). */
+int tfb_loss_bwd(const void* logits, const void* targets, int idx64, const void* lse, const void* grow, void* dlogits,
+                 long rows, int V, float softcap, void* stream);
+
+/* logits = x @ W^T (x [rows][d], W [V][d]) with the row log-sum-exp reduced in the GEMM epilogue, then loss / lse as
+ * tfb_loss_fwd. part: fp32 [rows][V/64][2] scratch. rows, V multiples of 128, d of 64.
+ * Replaces the lm_head matmul + loss forward pair (round1/source/train.py:8668, 9191-9212). */
+int tfb_lmhead_fwd(const void* x, const void* W, const void* targets, int idx64, const void* row_w, void* logits, void* part,
+                   void* loss, void* lse, long rows, int d, int V, float softcap, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

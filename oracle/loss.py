@@ -1,0 +1,81 @@
+"""Loss-head oracle: softcap + log-softmax + cross-entropy on the raw LM-head output, and the composition
+final RMSNorm -> LM-head GEMM -> loss that BASELINE config 1 times.
+
+Restates R1:4481-4495 (eager loss rows: logits.float(), softcap * tanh(logits / softcap), log_softmax, one-hot
+pick), the gradient stated in the R1 loss-head docstring (R1:4466: d x = g (softmax - onehot) (1 - tanh^2)),
+R2:6364-6391 / 11688-11703 (mean over valid rows with ignore_index -1 as row weights valid / sum(valid)), and
+the LM head in front of it (R1:8668 `y = x2d @ W`, R1:9191-9212). The reference never fuses the GEMM with the
+loss; its oracle is this composition, with the logits rounded to bf16 between the two.
+
+Pinned by (tests/test_oracle_loss.py): torch.nn.functional.cross_entropy on the softcapped fp32 logits,
+torch.autograd for the gradient, loss at uniform logits = ln V, sum_v dlogits / (1 - tanh^2) = 0 per row.
+"""
+import torch
+import torch.nn.functional as F
+
+
+def softcap_logits(x, softcap):
+    xf = x.float()
+    if softcap:
+        return softcap * torch.tanh(xf / softcap)
+    return xf
+
+
+def loss_rows(logits2, targets, softcap=15.0):
+    """(rows fp32 [N], lse fp32 [N]); rows with target < 0 give 0."""
+    s = softcap_logits(logits2, softcap)
+    lse = torch.logsumexp(s, dim=-1)
+    t = targets.reshape(-1).long()
+    valid = t >= 0
+    picked = s.gather(1, t.clamp_min(0)[:, None]).squeeze(1)
+    return torch.where(valid, lse - picked, torch.zeros_like(lse)), lse
+
+
+def row_weights(targets, reduction="mean"):
+    """valid / sum(valid) for "mean", valid for "sum"."""
+    valid = (targets.reshape(-1) >= 0).float()
+    return valid / valid.sum().clamp_min(1.0) if reduction == "mean" else valid
+
+
+def fused_loss(logits, targets, reduction="mean", softcap=15.0):
+    V = logits.shape[-1]
+    rows, _ = loss_rows(logits.reshape(-1, V), targets, softcap)
+    if reduction == "none":
+        return rows.view_as(targets)
+    return (rows * row_weights(targets, reduction)).sum()
+
+
+def loss_backward(logits2, targets, lse, grow, softcap=15.0):
+    """dlogits in logits' dtype; grow [N] fp32 (upstream gradient times row weight)."""
+    xf = logits2.float()
+    t = targets.reshape(-1).long()
+    valid = (t >= 0).float()
+    onehot = F.one_hot(t.clamp_min(0), xf.shape[-1]).float()
+    if softcap:
+        th = torch.tanh(xf / softcap)
+        p = torch.exp(softcap * th - lse[:, None])
+        d = (p - onehot) * (1.0 - th * th)
+    else:
+        d = torch.exp(xf - lse[:, None]) - onehot
+    return (d * (grow * valid)[:, None]).to(logits2.dtype)
+
+
+def lmhead_loss(x, norm_w, W, targets, eps=1e-6, softcap=None):
+    """Config 1 forward: mean loss from hidden states x [N, d] (bf16), norm weight [d], head weight W [V, d]."""
+    from . import norm as _n
+    xn, inv = _n.rmsnorm(x, norm_w, eps)
+    logits = (xn.float() @ W.float().t()).to(x.dtype)
+    return fused_loss(logits, targets, "mean", softcap), (xn, inv, logits)
+
+
+def lmhead_loss_backward(x, norm_w, W, targets, saved, eps=1e-6, softcap=None, gloss=1.0):
+    """(dx bf16 [N, d], dnorm_w fp32 [d], dW bf16 [V, d]) for the mean loss."""
+    from . import norm as _n
+    xn, inv, logits = saved
+    _, lse = loss_rows(logits, targets, softcap)
+    grow = row_weights(targets, "mean") * gloss
+    dl = loss_backward(logits, targets, lse, grow, softcap)
+    dxn = (dl.float() @ W.float()).to(x.dtype)
+    dW = (dl.float().t() @ xn.float()).to(x.dtype)
+    dx, dw = _n.rmsnorm_backward(dxn, x, inv, norm_w)
+    return dx.to(x.dtype), dw, dW

@@ -13,6 +13,7 @@ _vp = ctypes.c_void_p
 _i = ctypes.c_int
 _l = ctypes.c_long
 _f = ctypes.c_float
+_lp = ctypes.POINTER(ctypes.c_long)
 
 # name -> argtypes (restype is always int status unless listed in _RESTYPE)
 SIGNATURES = {
@@ -30,6 +31,20 @@ SIGNATURES = {
     "tfb_mlp8_precast": [_vp, _vp, _vp, _vp, _i, _i, _vp],
     "tfb_mlp8_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_mlp8_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_attn_fwd": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _i, _i, _i, _i, _f, _vp],
+    "tfb_attn_bwd": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _vp, _i, _i, _i, _i,
+                     _f, _vp],
+    "tfb_relu2": [_vp, _vp, _vp, _l, _i, _vp],
+    "tfb_rope": [_vp, _vp, _vp, _vp, _l, _i, _i, _i, _l, _l, _i, _vp],
+    "tfb_resmix_bwd_blocks": [_l],
+    "tfb_resmix_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _vp],
+    "tfb_embedding_fwd": [_vp, _i, _vp, _vp, _l, _i, _vp],
+    "tfb_embedding_bwd": [_vp, _i, _vp, _vp, _l, _i, _vp],
+    "tfb_adamw": [_vp, _vp, _i, _vp, _vp, _vp, _l, _f, _f, _f, _f, _f, _f, _f, _vp],
+    "tfb_fill_f32": [_vp, _f, _l, _vp],
+    "tfb_loss_fwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
+    "tfb_loss_bwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
+    "tfb_lmhead_fwd": [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _f, _vp],
     "tfb_mlp_dw_proj": [_vp, _vp, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
 }
 

@@ -1,0 +1,292 @@
+"""torch.autograd.Function wrappers around the HIP ops: the same role the reference's `*Fn` classes play
+(round1/source/train.py NkiAttnFn 8016, FcRelu2NNFn 4062, _ProjFn 3666, the loss head's LossHeadFn, Head2Fn 6599,
+_LinearGemm / _LmHeadDwSplit 8419-8711). Weight gradients follow the reference's in-place convention
+(round1/source/train.py:8463-8472): when a weight carries a `grad_buf` tensor the gradient GEMM accumulates into it
+and autograd gets None for that weight; otherwise the gradient is returned as usual.
+"""
+import math
+
+import torch
+
+from . import ops
+
+bf16 = torch.bfloat16
+
+
+def _accumulate_into(w):
+    """(buffer, accumulate flag) for a weight with an in-place gradient buffer, else (None, False)."""
+    buf = getattr(w, "grad_buf", None)
+    if buf is None:
+        return None, False
+    fresh = getattr(w, "grad_fresh", True)
+    w.grad_fresh = False
+    return buf, not fresh
+
+
+class RMSNormFn(torch.autograd.Function):
+    """y = RMSNorm(x) * weight (weight optional)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, eps):
+        x = x.contiguous()
+        _, y, inv = ops.rmsnorm_fwd(x, weight, eps)
+        ctx.save_for_backward(x, inv, weight)
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        x, inv, weight = ctx.saved_tensors
+        buf, acc = (None, False) if weight is None else _accumulate_into(weight)
+        dx, dw = ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, None, buf, acc)
+        if weight is None or buf is not None:
+            return dx, None, None
+        return dx, dw.to(weight.dtype), None
+
+
+class AddRMSNormFn(torch.autograd.Function):
+    """(s, y) = (x + res, RMSNorm(x + res) * weight): the residual add fused in front of the norm
+    (round1/source/train.py:6117 tail_norm2, 6826 final_norm)."""
+
+    @staticmethod
+    def forward(ctx, x, res, weight, eps):
+        s, y, inv = ops.rmsnorm_fwd(x.contiguous(), weight, eps, res=res.contiguous())
+        ctx.save_for_backward(s, inv, weight)
+        return s, y
+
+    @staticmethod
+    def backward(ctx, gs, gy):
+        s, inv, weight = ctx.saved_tensors
+        buf, acc = (None, False) if weight is None else _accumulate_into(weight)
+        if gy is None:
+            return gs, gs, None, None
+        dx, dw = ops.rmsnorm_bwd(gy.contiguous(), s, inv, weight, None if gs is None else gs.contiguous(), buf, acc)
+        gw = dw.to(weight.dtype) if (weight is not None and buf is None) else None
+        return dx, dx, gw, None
+
+
+class BlockHeadFn(torch.autograd.Function):
+    """(x_new, x_norm) = (l1 x + l2 x0 [+ l3 skip], RMSNorm(x_new)); gains are (1,) fp32 tensors."""
+
+    @staticmethod
+    def forward(ctx, x, x0, l1, l2, skip, l3, eps):
+        gains = torch.cat([l1.reshape(1).float(), l2.reshape(1).float(),
+                           (l3.reshape(1).float() if skip is not None else torch.zeros_like(l1.reshape(1).float()))])
+        x, x0 = x.contiguous(), x0.contiguous()
+        skip = None if skip is None else skip.contiguous()
+        x_new, x_norm, inv = ops.block_head_fwd(x, x0, gains, skip, eps)
+        ctx.save_for_backward(x, x0, skip, x_new, inv, gains)
+        ctx.has_skip = skip is not None
+        return x_new, x_norm
+
+    @staticmethod
+    def backward(ctx, g_new, g_norm):
+        x, x0, skip, x_new, inv, gains = ctx.saved_tensors
+        if g_norm is None:
+            g_norm = torch.zeros_like(x)
+        dx, dx0, dskip, dg = ops.block_head_bwd(None if g_new is None else g_new.contiguous(), g_norm.contiguous(), x, x0, x_new,
+                                                inv, gains, skip)
+        return dx, dx0, dg[0:1], dg[1:2], dskip, (dg[2:3] if ctx.has_skip else None), None
+
+
+class LinearFn(torch.autograd.Function):
+    """y = x @ w^T with w [out, in] (nn.Linear layout); dW accumulates into w.grad_buf when present."""
+
+    @staticmethod
+    def forward(ctx, x, w):
+        x2 = x.reshape(-1, x.shape[-1]).contiguous()
+        y = ops.matmul(x2, w, trans_b=True)
+        ctx.save_for_backward(x2, w)
+        ctx.xshape = x.shape
+        return y.view(*x.shape[:-1], w.shape[0])
+
+    @staticmethod
+    def backward(ctx, gy):
+        x2, w = ctx.saved_tensors
+        g2 = gy.reshape(-1, gy.shape[-1]).contiguous()
+        dx = ops.matmul(g2, w).view(ctx.xshape)
+        buf, acc = _accumulate_into(w)
+        if buf is not None:
+            ops.matmul(g2, x2, trans_a=True, out=buf, accumulate=acc)
+            return dx, None
+        return dx, ops.matmul(g2, x2, trans_a=True)
+
+
+class CausalAttentionFn(torch.autograd.Function):
+    """nki_causal_attention(q, k, v, scale): q, k, v [B, H, T, D] -> [B, T, H, D] (round1/source/train.py:8069)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, scale):
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        o, lse = ops.attn_fwd(q, k, v, scale, "bhtd")
+        ctx.save_for_backward(q, k, v, o, lse)
+        ctx.scale = scale
+        return o
+
+    @staticmethod
+    def backward(ctx, go):
+        q, k, v, o, lse = ctx.saved_tensors
+        dq, dk, dv = ops.attn_bwd(q, k, v, o, go.contiguous(), lse, ctx.scale, "bhtd")
+        return dq, dk, dv, None
+
+
+class RopeAttentionFn(torch.autograd.Function):
+    """Attention straight from the fused projection output qkv [B, T, 3C]: RoPE on the q and k thirds (in place, the
+    buffer has no other reader), causal attention reading the thirds through strides, one dqkv [B, T, 3C] back
+    (the call shape of nki_rope_attention, round1/source/train.py:8197, without its QK-norm)."""
+
+    @staticmethod
+    def forward(ctx, qkv, cos, sin, n_head, scale):
+        B, T, C3 = qkv.shape
+        C = C3 // 3
+        D = C // n_head
+        qkv = qkv.contiguous()
+        ops.rope_(qkv.view(B * T, C3), cos, sin, T, 2 * n_head, D)
+        q, k, v = (t.view(B, T, n_head, D) for t in qkv.split(C, dim=-1))
+        o, lse = ops.attn_fwd(q, k, v, scale, "bthd")
+        ctx.save_for_backward(qkv, o, lse, cos, sin)
+        ctx.n_head, ctx.scale = n_head, scale
+        return o.view(B, T, C)
+
+    @staticmethod
+    def backward(ctx, go):
+        qkv, o, lse, cos, sin = ctx.saved_tensors
+        B, T, C3 = qkv.shape
+        C = C3 // 3
+        H = ctx.n_head
+        D = C // H
+        q, k, v = (t.view(B, T, H, D) for t in qkv.split(C, dim=-1))
+        dqkv = torch.empty_like(qkv)
+        dq, dk, dv = (t.view(B, T, H, D) for t in dqkv.split(C, dim=-1))
+        ops.attn_bwd(q, k, v, o, go.contiguous().view(B, T, H, D), lse, ctx.scale, "bthd", dq, dk, dv, "bthd")
+        ops.rope_(dqkv.view(B * T, C3), cos, sin, T, 2 * H, D, inverse=True)
+        return dqkv, None, None, None, None
+
+
+class Mlp8State:
+    """Per-layer fp8 state refreshed once per optimizer step: the scale row and the e4m3 weight pack
+    (round2/source/train.py:6617 fp8_refresh_weights, 7003 mlp8_scales_into, 7267 mlp8_precast_into)."""
+
+    def __init__(self, e4m3_limit=240.0, x_scale=4.0):
+        self.e4m3_limit, self.x_scale = e4m3_limit, x_scale
+        self.row = None
+        self.w8 = None
+
+    def refresh(self, w_fc, w_proj):
+        self.row = ops.mlp8_forward_scales(w_fc.detach(), w_proj.detach(), self.e4m3_limit, self.x_scale)
+        self.w8 = ops.mlp8_precast(w_fc.detach(), w_proj.detach(), self.row)
+
+
+class Mlp8Fn(torch.autograd.Function):
+    """y = c_proj(relu(c_fc(x))^2) with the four activation GEMMs in fp8 and bf16 weight gradients."""
+
+    @staticmethod
+    def forward(ctx, x, w_fc, w_proj, state):
+        x2 = x.reshape(-1, x.shape[-1]).contiguous()
+        y, r = ops.mlp8_fwd(x2, state.w8, state.row, w_fc.shape[0], state.x_scale)
+        ctx.save_for_backward(x2, r, w_fc, w_proj)
+        ctx.state = state
+        ctx.xshape = x.shape
+        return y.view(x.shape)
+
+    @staticmethod
+    def backward(ctx, gy):
+        x2, r, w_fc, w_proj = ctx.saved_tensors
+        st = ctx.state
+        g2 = gy.reshape(-1, gy.shape[-1]).contiguous()
+        rowb = ops.mlp8_backward_scales(g2, st.row)
+        dx, _, dpre = ops.mlp8_bwd(g2, r, st.w8, rowb, want_h=False)
+        buf, acc = _accumulate_into(w_fc)
+        if buf is not None:
+            ops.matmul(dpre, x2, trans_a=True, out=buf, accumulate=acc)
+            dw_fc = None
+        else:
+            dw_fc = ops.matmul(dpre, x2, trans_a=True)
+        buf, acc = _accumulate_into(w_proj)
+        if buf is not None:
+            ops.mlp_dw_proj(g2, r, out=buf, accumulate=acc)
+            dw_proj = None
+        else:
+            dw_proj = ops.mlp_dw_proj(g2, r)
+        return dx.view(ctx.xshape), dw_fc, dw_proj, None
+
+
+class LmHeadLossFn(torch.autograd.Function):
+    """loss = reduce(CE(softcap(x @ W^T), targets)): the LM-head GEMM with the log-sum-exp in its epilogue, then (in
+    the backward) dlogits written in place over the logits and the two gradient GEMMs."""
+
+    @staticmethod
+    def forward(ctx, x, W, targets, softcap, reduction):
+        x2 = x.reshape(-1, x.shape[-1]).contiguous()
+        tg = targets.reshape(-1)
+        valid = (tg >= 0).to(torch.float32)
+        w = valid / valid.sum().clamp_min(1.0) if reduction == "mean" else valid
+        logits, rows, lse = ops.lmhead_fwd(x2, W, tg, softcap, w)
+        ctx.save_for_backward(x2, W, tg, logits, lse, w)
+        ctx.softcap = softcap
+        ctx.xshape = x.shape
+        return rows.sum()
+
+    @staticmethod
+    def backward(ctx, g):
+        x2, W, tg, logits, lse, w = ctx.saved_tensors
+        grow = (w * g.to(torch.float32)).contiguous()
+        dl = ops.loss_bwd(logits, tg, lse, grow, ctx.softcap, inplace=True)
+        dx = ops.matmul(dl, W).view(ctx.xshape)
+        buf, acc = _accumulate_into(W)
+        if buf is not None:
+            ops.matmul(dl, x2, trans_a=True, out=buf, accumulate=acc)
+            return dx, None, None, None, None
+        return dx, ops.matmul(dl, x2, trans_a=True), None, None, None
+
+
+class FusedLossFn(torch.autograd.Function):
+    """fused_loss(logits, targets, reduction, softcap) rows on materialised logits (round1/source/train.py:4691)."""
+
+    @staticmethod
+    def forward(ctx, logits2, targets, softcap):
+        rows, lse = ops.loss_fwd(logits2, targets, softcap)
+        ctx.save_for_backward(logits2, targets, lse)
+        ctx.softcap = softcap
+        return rows
+
+    @staticmethod
+    def backward(ctx, grows):
+        logits2, targets, lse = ctx.saved_tensors
+        return ops.loss_bwd(logits2, targets, lse, grows.contiguous().float(), ctx.softcap), None, None
+
+
+class EmbeddingFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, idx, weight):
+        ctx.save_for_backward(idx, weight)
+        return ops.embedding_fwd(idx, weight)
+
+    @staticmethod
+    def backward(ctx, gy):
+        idx, weight = ctx.saved_tensors
+        buf, acc = _accumulate_into(weight)
+        if buf is not None:
+            if not acc:
+                ops.fill_f32_(buf, 0.0)
+            ops.embedding_bwd(idx, gy.contiguous(), buf)
+            return None, None
+        dw = ops.fill_f32_(torch.empty(weight.shape, dtype=torch.float32, device=weight.device), 0.0)
+        ops.embedding_bwd(idx, gy.contiguous(), dw)
+        return None, dw.to(weight.dtype)
+
+
+class Relu2Fn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        x = x.contiguous()
+        ctx.save_for_backward(x)
+        return ops.relu2(x)
+
+    @staticmethod
+    def backward(ctx, gy):
+        (x,) = ctx.saved_tensors
+        return ops.relu2_bwd(x, gy.contiguous())
+
+
+def default_scale(D):
+    return 1.0 / math.sqrt(D)

@@ -1,0 +1,311 @@
+// Bandwidth-bound elementwise kernels: ReLU^2 family, RoPE, residual-mix backward, embedding
+// gather / scatter-add, fused AdamW. All use 128-bit coalesced accesses (8 bf16 or 4 fp32 per
+// lane), fp32 math and one rounding per output.
+//
+//   relu2 fwd / bwd / bwd-from-output      round1/source/train.py:663, 597, 633 (625-631)
+//   rope (half-split rotation)             round1/source/train.py:4188-4193
+//   resmix backward                        round2/source/kernels/nki_resmix.py:148-162
+//   embedding                              round1/source/train.py:8407 (embedding_fwd), 8303 (backward as dW = onehot^T dY)
+//   adamw                                  round1/source/train.py:9670-9677, round2/source/train.py:13756-13766
+#include "common.hpp"
+
+namespace {
+
+inline int blocks_for(long nvec, int cap = 16384) {
+  long b = (nvec + 255) / 256;
+  return (int)(b < cap ? (b > 0 ? b : 1) : cap);
+}
+
+// mode 0: y = relu(x)^2 ; mode 1: dx = g * 2 relu(x) ; mode 2: dx = bf16(sqrt(4 h)) * g  (a = x or h, b = g)
+template <int MODE>
+__global__ __launch_bounds__(256) void relu2_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ b,
+                                                   bf16_t* __restrict__ out, long n) {
+  for (long i = ((long)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += (long)gridDim.x * 256 * 8) {
+    u32x4 ua = *(const u32x4*)(a + i);
+    u32x4 ub = {0, 0, 0, 0};
+    if (MODE != 0) ub = *(const u32x4*)(b + i);
+    u32x4 o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float x0 = bflo(ua[k]), x1 = bfhi(ua[k]);
+      float r0, r1;
+      if (MODE == 0) {
+        x0 = fmaxf(x0, 0.f);
+        x1 = fmaxf(x1, 0.f);
+        r0 = x0 * x0;
+        r1 = x1 * x1;
+      } else if (MODE == 1) {
+        r0 = bflo(ub[k]) * 2.0f * fmaxf(x0, 0.f);
+        r1 = bfhi(ub[k]) * 2.0f * fmaxf(x1, 0.f);
+      } else {
+        r0 = round_bf(sqrtf(4.0f * x0)) * bflo(ub[k]);
+        r1 = round_bf(sqrtf(4.0f * x1)) * bfhi(ub[k]);
+      }
+      o[k] = pack2bf(r0, r1);
+    }
+    *(u32x4*)(out + i) = o;
+  }
+}
+
+// x [rows][row_stride] holds nheads heads of D contiguous elements starting at column 0; row r is token r % T.
+// y1 = x1 c + x2 s, y2 = x2 c - x1 s  (inverse: y1 = x1 c - x2 s, y2 = x2 c + x1 s). In place when out == x.
+__global__ __launch_bounds__(256) void rope_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ cs,
+                                                  const bf16_t* __restrict__ sn, bf16_t* __restrict__ out, long rows, int T,
+                                                  int nheads, int D, long row_stride, long out_stride, int inverse) {
+  const int hc = D / 16;  // 8-element chunks per half head
+  const long per_row = (long)nheads * hc;
+  const long total = rows * per_row;
+  for (long idx = (long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (long)gridDim.x * 256) {
+    long row = idx / per_row;
+    int rem = (int)(idx % per_row);
+    int head = rem / hc, c = rem % hc;
+    int t = (int)(row % T);
+    const bf16_t* p1 = x + row * row_stride + (long)head * D + c * 8;
+    u32x4 a = *(const u32x4*)p1;
+    u32x4 b = *(const u32x4*)(p1 + D / 2);
+    u32x4 cc = *(const u32x4*)(cs + (long)t * (D / 2) + c * 8);
+    u32x4 ss = *(const u32x4*)(sn + (long)t * (D / 2) + c * 8);
+    u32x4 o1, o2;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float a0 = bflo(a[k]), a1 = bfhi(a[k]), b0 = bflo(b[k]), b1 = bfhi(b[k]);
+      float c0 = bflo(cc[k]), c1 = bfhi(cc[k]);
+      float s0 = bflo(ss[k]), s1 = bfhi(ss[k]);
+      if (inverse) {
+        s0 = -s0;
+        s1 = -s1;
+      }
+      o1[k] = pack2bf(a0 * c0 + b0 * s0, a1 * c1 + b1 * s1);
+      o2[k] = pack2bf(b0 * c0 - a0 * s0, b1 * c1 - a1 * s1);
+    }
+    bf16_t* q1 = out + row * out_stride + (long)head * D + c * 8;
+    *(u32x4*)q1 = o1;
+    *(u32x4*)(q1 + D / 2) = o2;
+  }
+}
+
+// dx = g * bf16(a), dx0 = g * bf16(b) (products rounded to bf16), partial sums of bf16(g x) and bf16(g x0) in fp32.
+__global__ __launch_bounds__(256) void resmix_bwd_kernel(const bf16_t* __restrict__ g, const bf16_t* __restrict__ x,
+                                                        const bf16_t* __restrict__ x0, const float* __restrict__ ab,
+                                                        bf16_t* __restrict__ dx, bf16_t* __restrict__ dx0,
+                                                        float* __restrict__ part, long n) {
+  __shared__ float red[2][4];
+  const float a = round_bf(ab[0]), b = round_bf(ab[1]);
+  float sa = 0.f, sb = 0.f;
+  for (long i = ((long)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += (long)gridDim.x * 256 * 8) {
+    u32x4 ug = *(const u32x4*)(g + i), ux = *(const u32x4*)(x + i), u0 = *(const u32x4*)(x0 + i);
+    u32x4 o1, o2;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float g0 = bflo(ug[k]), g1 = bfhi(ug[k]);
+      o1[k] = pack2bf(g0 * a, g1 * a);
+      o2[k] = pack2bf(g0 * b, g1 * b);
+      sa += round_bf(g0 * bflo(ux[k])) + round_bf(g1 * bfhi(ux[k]));
+      sb += round_bf(g0 * bflo(u0[k])) + round_bf(g1 * bfhi(u0[k]));
+    }
+    *(u32x4*)(dx + i) = o1;
+    *(u32x4*)(dx0 + i) = o2;
+  }
+  sa = wave_sum(sa);
+  sb = wave_sum(sb);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    red[0][wave] = sa;
+    red[1][wave] = sb;
+  }
+  __syncthreads();
+  if (threadIdx.x < 2) part[(long)blockIdx.x * 2 + threadIdx.x] = red[threadIdx.x][0] + red[threadIdx.x][1] + red[threadIdx.x][2] + red[threadIdx.x][3];
+}
+
+__global__ void sum_pairs_kernel(const float* __restrict__ part, int nblocks, float* __restrict__ out) {
+  __shared__ float red[2][4];
+  float s0 = 0.f, s1 = 0.f;
+  for (int i = threadIdx.x; i < nblocks; i += 256) {
+    s0 += part[2 * i];
+    s1 += part[2 * i + 1];
+  }
+  s0 = wave_sum(s0);
+  s1 = wave_sum(s1);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    red[0][wave] = s0;
+    red[1][wave] = s1;
+  }
+  __syncthreads();
+  if (threadIdx.x < 2) out[threadIdx.x] = red[threadIdx.x][0] + red[threadIdx.x][1] + red[threadIdx.x][2] + red[threadIdx.x][3];
+}
+
+template <typename IDX>
+__global__ __launch_bounds__(256) void embedding_fwd_kernel(const IDX* __restrict__ idx, const bf16_t* __restrict__ w,
+                                                           bf16_t* __restrict__ out, long n, int C) {
+  const int cpr = C / 8;
+  const long total = n * cpr;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    long row = i / cpr;
+    int c = (int)(i % cpr) * 8;
+    long tok = (long)idx[row];
+    *(u32x4*)(out + row * C + c) = *(const u32x4*)(w + tok * C + c);
+  }
+}
+
+// dW[idx[row]] += dY[row] in fp32 with atomics (dW fp32, zeroed or accumulated into by the caller).
+template <typename IDX>
+__global__ __launch_bounds__(256) void embedding_bwd_kernel(const IDX* __restrict__ idx, const bf16_t* __restrict__ dy,
+                                                           float* __restrict__ dw, long n, int C) {
+  const int cpr = C / 8;
+  const long total = n * cpr;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    long row = i / cpr;
+    int c = (int)(i % cpr) * 8;
+    long tok = (long)idx[row];
+    u32x4 u = *(const u32x4*)(dy + row * C + c);
+    float* d = dw + tok * C + c;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      atomicAdd(d + 2 * k, bflo(u[k]));
+      atomicAdd(d + 2 * k + 1, bfhi(u[k]));
+    }
+  }
+}
+
+struct AdamScalars {
+  float lr, wd, omb1, omb2, eps, bias1, bias2;
+};
+
+__device__ __forceinline__ float lerp_torch(float a, float b, float w) {
+  // torch.lerp: a + w (b - a) for w < 0.5, else b - (b - a)(1 - w)
+  float d = b - a;
+  return w < 0.5f ? fmaf(w, d, a) : fmaf(-d, 1.0f - w, b);  // torch's lerp contracts to one fma
+}
+
+// p (fp32 master) updated in place; optional bf16 copy written; g is fp32 (GF32) or bf16.
+template <bool GF32>
+__global__ __launch_bounds__(256) void adamw_kernel(float* __restrict__ p, const void* __restrict__ g, float* __restrict__ m,
+                                                   float* __restrict__ v, bf16_t* __restrict__ p16, long n, AdamScalars s) {
+  for (long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4; i < n; i += (long)gridDim.x * 256 * 4) {
+    f32x4 pp = *(const f32x4*)(p + i), mm = *(const f32x4*)(m + i), vv = *(const f32x4*)(v + i), gg;
+    if (GF32) {
+      gg = *(const f32x4*)((const float*)g + i);
+    } else {
+      u32x2 u = *(const u32x2*)((const bf16_t*)g + i);
+      gg = f32x4{bflo(u.x), bfhi(u.x), bflo(u.y), bfhi(u.y)};
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float pk = pp[k];
+      if (s.wd > 0.f) pk = pk * (1.0f - s.lr * s.wd);
+      float mk = lerp_torch(mm[k], gg[k], s.omb1);
+      float vk = lerp_torch(vv[k], gg[k] * gg[k], s.omb2);
+      float upd = mk / s.bias1 / (sqrtf(vk / s.bias2) + s.eps);
+      pk = pk - upd * s.lr;
+      pp[k] = pk;
+      mm[k] = mk;
+      vv[k] = vk;
+    }
+    *(f32x4*)(p + i) = pp;
+    *(f32x4*)(m + i) = mm;
+    *(f32x4*)(v + i) = vv;
+    if (p16) {
+      u32x2 o = {pack2bf(pp[0], pp[1]), pack2bf(pp[2], pp[3])};
+      *(u32x2*)(p16 + i) = o;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void fill_f32_kernel(float* __restrict__ p, float val, long n) {
+  for (long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4; i < n; i += (long)gridDim.x * 256 * 4) {
+    if (i + 3 < n) {
+      *(f32x4*)(p + i) = f32x4{val, val, val, val};
+    } else {
+      for (long j = i; j < n; ++j) p[j] = val;
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int tfb_relu2(const void* a, const void* b, void* out, long n, int mode, void* stream) {
+  if (!a || !out || (mode != 0 && !b)) return TFB_ERR_ARG;
+  if (n <= 0 || n % 8) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  int nb = blocks_for(n / 8);
+  if (mode == 0) hipLaunchKernelGGL(relu2_kernel<0>, dim3(nb), dim3(256), 0, s, (const bf16_t*)a, (const bf16_t*)b, (bf16_t*)out, n);
+  else if (mode == 1) hipLaunchKernelGGL(relu2_kernel<1>, dim3(nb), dim3(256), 0, s, (const bf16_t*)a, (const bf16_t*)b, (bf16_t*)out, n);
+  else if (mode == 2) hipLaunchKernelGGL(relu2_kernel<2>, dim3(nb), dim3(256), 0, s, (const bf16_t*)a, (const bf16_t*)b, (bf16_t*)out, n);
+  else return TFB_ERR_ARG;
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+extern "C" int tfb_rope(const void* x, const void* cos_t, const void* sin_t, void* out, long rows, int T, int nheads, int D,
+                        long row_stride, long out_stride, int inverse, void* stream) {
+  if (!x || !cos_t || !sin_t || !out) return TFB_ERR_ARG;
+  if (rows <= 0 || T <= 0 || nheads <= 0 || D <= 0 || D % 16 || row_stride % 8 || out_stride % 8) return TFB_ERR_SHAPE;
+  long total = rows * nheads * (D / 16);
+  hipLaunchKernelGGL(rope_kernel, dim3(blocks_for(total)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x,
+                     (const bf16_t*)cos_t, (const bf16_t*)sin_t, (bf16_t*)out, rows, T, nheads, D, row_stride, out_stride, inverse);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+extern "C" int tfb_resmix_bwd_blocks(long n) { return blocks_for(n / 8, 1024); }
+
+// ab: device fp32 [2] gains; part: fp32 [2 * tfb_resmix_bwd_blocks(n)] scratch; dab: fp32 [2] = (sum g x, sum g x0)
+extern "C" int tfb_resmix_bwd(const void* g, const void* x, const void* x0, const void* ab, void* dx, void* dx0, void* part,
+                              void* dab, long n, void* stream) {
+  if (!g || !x || !x0 || !ab || !dx || !dx0 || !part || !dab) return TFB_ERR_ARG;
+  if (n <= 0 || n % 8) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  int nb = blocks_for(n / 8, 1024);
+  hipLaunchKernelGGL(resmix_bwd_kernel, dim3(nb), dim3(256), 0, s, (const bf16_t*)g, (const bf16_t*)x, (const bf16_t*)x0,
+                     (const float*)ab, (bf16_t*)dx, (bf16_t*)dx0, (float*)part, n);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sum_pairs_kernel, dim3(1), dim3(256), 0, s, (const float*)part, nb, (float*)dab);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+extern "C" int tfb_embedding_fwd(const void* idx, int idx64, const void* w, void* out, long n, int C, void* stream) {
+  if (!idx || !w || !out) return TFB_ERR_ARG;
+  if (n <= 0 || C <= 0 || C % 8) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  int nb = blocks_for(n * (C / 8));
+  if (idx64) hipLaunchKernelGGL(embedding_fwd_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, (const bf16_t*)w, (bf16_t*)out, n, C);
+  else hipLaunchKernelGGL(embedding_fwd_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, (const bf16_t*)w, (bf16_t*)out, n, C);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+extern "C" int tfb_embedding_bwd(const void* idx, int idx64, const void* dy, void* dw_f32, long n, int C, void* stream) {
+  if (!idx || !dy || !dw_f32) return TFB_ERR_ARG;
+  if (n <= 0 || C <= 0 || C % 8) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  int nb = blocks_for(n * (C / 8));
+  if (idx64) hipLaunchKernelGGL(embedding_bwd_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, (const bf16_t*)dy, (float*)dw_f32, n, C);
+  else hipLaunchKernelGGL(embedding_bwd_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, (const bf16_t*)dy, (float*)dw_f32, n, C);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// One AdamW update over n elements: p fp32 master in place, m / v fp32 in place, optional bf16 copy of p.
+extern "C" int tfb_adamw(void* p, const void* g, int g_f32, void* m, void* v, void* p_bf16, long n, float lr, float wd,
+                         float one_minus_beta1, float one_minus_beta2, float eps, float bias1, float bias2, void* stream) {
+  if (!p || !g || !m || !v) return TFB_ERR_ARG;
+  if (n <= 0 || n % 4) return TFB_ERR_SHAPE;
+  AdamScalars sc{lr, wd, one_minus_beta1, one_minus_beta2, eps, bias1, bias2};
+  hipStream_t s = (hipStream_t)stream;
+  int nb = blocks_for(n / 4);
+  if (g_f32) hipLaunchKernelGGL(adamw_kernel<true>, dim3(nb), dim3(256), 0, s, (float*)p, g, (float*)m, (float*)v, (bf16_t*)p_bf16, n, sc);
+  else hipLaunchKernelGGL(adamw_kernel<false>, dim3(nb), dim3(256), 0, s, (float*)p, g, (float*)m, (float*)v, (bf16_t*)p_bf16, n, sc);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// A fill kernel in place of hipMemsetAsync (safe to record into a HIP graph).
+extern "C" int tfb_fill_f32(void* p, float val, long n, void* stream) {
+  if (!p) return TFB_ERR_ARG;
+  if (n <= 0) return TFB_ERR_SHAPE;
+  hipLaunchKernelGGL(fill_f32_kernel, dim3(blocks_for((n + 3) / 4)), dim3(256), 0, (hipStream_t)stream, (float*)p, val, n);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}

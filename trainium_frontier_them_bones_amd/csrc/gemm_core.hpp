@@ -14,6 +14,8 @@
 // transposed on the way into LDS through 4k x 8row register micro-blocks), which is what
 // the weight-gradient GEMMs (contraction over tokens) read.
 #pragma once
+#include <type_traits>
+
 #include "common.hpp"
 
 #define TFB_K_CONTIG 0
@@ -154,7 +156,13 @@ __device__ __forceinline__ int xcd_remap(int pid, int nb) {
   return (nb & 7) == 0 ? (pid & 7) * (nb >> 3) + (pid >> 3) : pid;
 }
 
-// Epi: __device__ void operator()(int p, int q, f32x4 v, int split) -- v = D[p..p+3][q]
+template <class T, class = void>
+struct has_tile_epilogue : std::false_type {};
+template <class T>
+struct has_tile_epilogue<T, std::void_t<decltype(T::kTileEpilogue)>> : std::true_type {};
+
+// Epi: either  __device__ void operator()(int p, int q, f32x4 v, int split)  with v = D[p..p+3][q],
+// or (with a static member kTileEpilogue)  __device__ void tile(acc, pw, qw, lr, lh, tile_id, split).
 template <class Cfg, class PreP, class PreQ, class Epi>
 __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, PreQ preq, Epi epi) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -215,17 +223,23 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, Pr
     __syncthreads();
   }
 
+  const int pw = (int)p0 + wp * (TP * 32), qw = (int)q0 + wq * (TQ * 32);
+  if constexpr (has_tile_epilogue<Epi>::value) {
+    // whole-accumulator epilogue: acc[i][j][4*jj + e] = D[pw + 32 i + 8 jj + 4 lh + e][qw + 32 j + lr]
+    epi.tile(acc, pw, qw, lr, lh, lid, (int)blockIdx.z);
+  } else {
 #pragma unroll
-  for (int i = 0; i < TP; ++i)
+    for (int i = 0; i < TP; ++i)
 #pragma unroll
-    for (int j = 0; j < TQ; ++j)
+      for (int j = 0; j < TQ; ++j)
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        int p = (int)p0 + wp * (TP * 32) + i * 32 + jj * 8 + lh * 4;
-        int q = (int)q0 + wq * (TQ * 32) + j * 32 + lr;
-        f32x4 v = {acc[i][j][jj * 4 + 0], acc[i][j][jj * 4 + 1], acc[i][j][jj * 4 + 2], acc[i][j][jj * 4 + 3]};
-        epi(p, q, v, (int)blockIdx.z);
-      }
+        for (int jj = 0; jj < 4; ++jj) {
+          int p = pw + i * 32 + jj * 8 + lh * 4;
+          int q = qw + j * 32 + lr;
+          f32x4 v = {acc[i][j][jj * 4 + 0], acc[i][j][jj * 4 + 1], acc[i][j][jj * 4 + 2], acc[i][j][jj * 4 + 3]};
+          epi(p, q, v, (int)blockIdx.z);
+        }
+  }
 }
 
 // Host-side launch: np, nq multiples of the tile; kbytes a multiple of 128 * splits.

@@ -1,0 +1,287 @@
+// Loss head: softcap + log-softmax + cross-entropy on bf16 logits, and the LM-head GEMM with the
+// log-sum-exp fused into its epilogue.
+//
+// Replaces _loss_fwd_kernel / _loss_bwd_kernel behind fused_loss(logits, targets, reduction, softcap)
+// (round1/source/train.py:4543, 4584, 4691; eager form 4481-4495), the row-weighted form of
+// round2/source/train.py:6364-6391 (ignore_index -1 = weight 0), and the lm_head matmul in front of
+// them (round1/source/train.py:8668, 9191-9212).
+//
+// Math per row, fp32 from the bf16-rounded logits x: s_v = c tanh(x_v / c) (or s_v = x_v without a
+// softcap), lse = log sum_v exp(s_v), loss = lse - s_target; d x_v = g (softmax_v - [v = target])
+// (1 - tanh^2). Only lse is saved; the backward recomputes tanh / exp.
+//
+// lmhead_fwd is the GEMM logits = x @ W^T (W [V, d]) whose epilogue rounds each accumulator to bf16,
+// stores it, and reduces exp(s - shift) over the 64 vocabulary columns a wavefront holds for each row
+// (in registers: a lane owns 32 of them, its partner lane the rest) into a [rows][V/64] table of
+// (max, sum) pairs; a finishing kernel merges a row's pairs, reads the target logit and writes lse and
+// the row loss. The logits make one trip to HBM (written once, read once by the backward).
+#include "gemm_core.hpp"
+
+namespace {
+
+__device__ __forceinline__ float fexp(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+
+// c * tanh(x / c) and tanh(x / c)
+__device__ __forceinline__ float tanh_fast(float y) {
+  // tanh(y) = 1 - 2 / (exp(2y) + 1); exp overflow gives 1, underflow gives -1
+  float e = __builtin_amdgcn_exp2f(y * 2.8853900817779268f);
+  return 1.0f - 2.0f / (e + 1.0f);
+}
+
+struct MS {
+  float m, s;
+};
+__device__ __forceinline__ MS ms_merge(MS a, MS b) {
+  float m = fmaxf(a.m, b.m);
+  MS r;
+  r.m = m;
+  r.s = a.s * fexp(a.m - m) + b.s * fexp(b.m - m);
+  return r;
+}
+
+// ------------------------------------------------------------------------------------ loss on logits
+// One workgroup per row. loss_row = w * (lse - s_t) with w = row_w[row] (or 1), 0 for target < 0.
+template <typename IDX>
+__global__ __launch_bounds__(256) void loss_fwd_kernel(const bf16_t* __restrict__ x, const IDX* __restrict__ tg,
+                                                      const float* __restrict__ row_w, float* __restrict__ loss,
+                                                      float* __restrict__ lse, int V, float cap) {
+  __shared__ float rm[4], rs[4];
+  const long row = blockIdx.x;
+  const bf16_t* xr = x + row * V;
+  const float icap = cap > 0.f ? 1.0f / cap : 0.f;
+  MS a{-1e30f, 0.f};
+  for (int i = threadIdx.x * 8; i < V; i += 256 * 8) {
+    u32x4 u = *(const u32x4*)(xr + i);
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      v[2 * k] = bflo(u[k]);
+      v[2 * k + 1] = bfhi(u[k]);
+    }
+    if (cap > 0.f) {
+      // fixed shift: every s is in [-cap, cap]
+#pragma unroll
+      for (int k = 0; k < 8; ++k) a.s += fexp(cap * tanh_fast(v[k] * icap) - cap);
+      a.m = cap;
+    } else {
+      float mx = a.m;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) mx = fmaxf(mx, v[k]);
+      float sc = fexp(a.m - mx), t = 0.f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) t += fexp(v[k] - mx);
+      a.s = a.s * sc + t;
+      a.m = mx;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    MS b{__shfl_xor(a.m, o, 64), __shfl_xor(a.s, o, 64)};
+    a = ms_merge(a, b);
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    rm[wave] = a.m;
+    rs[wave] = a.s;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    MS t{rm[0], rs[0]};
+    for (int i = 1; i < 4; ++i) t = ms_merge(t, MS{rm[i], rs[i]});
+    float l = t.m + logf(t.s);
+    lse[row] = l;
+    long tt = (long)tg[row];
+    float out = 0.f;
+    if (tt >= 0) {
+      float xt = bf2f(xr[tt]);
+      float st = cap > 0.f ? cap * tanh_fast(xt * icap) : xt;
+      out = (l - st) * (row_w ? row_w[row] : 1.0f);
+    }
+    loss[row] = out;
+  }
+}
+
+// d x_v = g_row (softmax_v - [v == t]) (1 - tanh^2); g_row = grow[row] (upstream grad x row weight); target < 0 -> 0.
+template <typename IDX>
+__global__ __launch_bounds__(256) void loss_bwd_kernel(const bf16_t* __restrict__ x, const IDX* __restrict__ tg,
+                                                      const float* __restrict__ lse, const float* __restrict__ grow,
+                                                      bf16_t* __restrict__ dx, int V, float cap) {
+  const long row = blockIdx.x;
+  const bf16_t* xr = x + row * V;
+  bf16_t* dr = dx + row * V;
+  const long tt = (long)tg[row];
+  const float g = tt >= 0 ? grow[row] : 0.f;
+  const float l = lse[row];
+  const float icap = cap > 0.f ? 1.0f / cap : 0.f;
+  for (int i = threadIdx.x * 8; i < V; i += 256 * 8) {
+    u32x4 u = *(const u32x4*)(xr + i);
+    float v[8], d[8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      v[2 * k] = bflo(u[k]);
+      v[2 * k + 1] = bfhi(u[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      float hot = (i + k == tt) ? 1.0f : 0.0f;
+      if (cap > 0.f) {
+        float t = tanh_fast(v[k] * icap);
+        float p = fexp(cap * t - l);
+        d[k] = g * (p - hot) * (1.0f - t * t);
+      } else {
+        d[k] = g * (fexp(v[k] - l) - hot);
+      }
+    }
+    u32x4 o = {pack2bf(d[0], d[1]), pack2bf(d[2], d[3]), pack2bf(d[4], d[5]), pack2bf(d[6], d[7])};
+    *(u32x4*)(dr + i) = o;
+  }
+}
+
+// ------------------------------------------------------------------------------------ LM head GEMM + lse partials
+struct EpiLmHead {
+  static constexpr bool kTileEpilogue = true;
+  bf16_t* logits;  // [rows][V]
+  float* part;     // [rows][V/64][2] (max, sum)
+  long V;
+  int nchunk;      // V / 64
+  float cap;
+  template <int TP, int TQ>
+  __device__ __forceinline__ void tile(const f32x16 (&acc)[TP][TQ], int pw, int qw, int lr, int lh, int, int) const {
+    static_assert(TP == 2, "a wavefront spans 64 vocabulary columns");
+    const float icap = cap > 0.f ? 1.0f / cap : 0.f;
+#pragma unroll
+    for (int j = 0; j < TQ; ++j) {
+      const long row = qw + j * 32 + lr;
+      float v[TP * 16];
+#pragma unroll
+      for (int i = 0; i < TP; ++i)
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const int p = pw + i * 32 + jj * 8 + lh * 4;
+          uint32_t w0 = pack2bf(acc[i][j][4 * jj], acc[i][j][4 * jj + 1]);
+          uint32_t w1 = pack2bf(acc[i][j][4 * jj + 2], acc[i][j][4 * jj + 3]);
+          u32x2 o = {w0, w1};
+          *(u32x2*)(logits + row * V + p) = o;
+          v[i * 16 + 4 * jj] = bflo(w0);
+          v[i * 16 + 4 * jj + 1] = bfhi(w0);
+          v[i * 16 + 4 * jj + 2] = bflo(w1);
+          v[i * 16 + 4 * jj + 3] = bfhi(w1);
+        }
+      MS a;
+      if (cap > 0.f) {
+        a.m = cap;
+        a.s = 0.f;
+#pragma unroll
+        for (int k = 0; k < TP * 16; ++k) a.s += fexp(cap * tanh_fast(v[k] * icap) - cap);
+        a.s += __shfl_xor(a.s, 32, 64);
+      } else {
+        float mx = v[0];
+#pragma unroll
+        for (int k = 1; k < TP * 16; ++k) mx = fmaxf(mx, v[k]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        float t = 0.f;
+#pragma unroll
+        for (int k = 0; k < TP * 16; ++k) t += fexp(v[k] - mx);
+        t += __shfl_xor(t, 32, 64);
+        a.m = mx;
+        a.s = t;
+      }
+      if (lh == 0) {
+        float* pp = part + (row * nchunk + (pw >> 6)) * 2;
+        pp[0] = a.m;
+        pp[1] = a.s;
+      }
+    }
+  }
+};
+
+// One wavefront per row: merge the row's partial pairs, read the target logit, write lse and the row loss.
+template <typename IDX>
+__global__ __launch_bounds__(256) void lmhead_finish_kernel(const float* __restrict__ part, const bf16_t* __restrict__ logits,
+                                                           const IDX* __restrict__ tg, const float* __restrict__ row_w,
+                                                           float* __restrict__ loss, float* __restrict__ lse, long rows, long V,
+                                                           int nchunk, float cap) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long row = (long)blockIdx.x * 4 + wave;
+  if (row >= rows) return;
+  MS a{-1e30f, 0.f};
+  for (int c = lane; c < nchunk; c += 64) {
+    const float* pp = part + (row * nchunk + c) * 2;
+    a = ms_merge(a, MS{pp[0], pp[1]});
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    MS b{__shfl_xor(a.m, o, 64), __shfl_xor(a.s, o, 64)};
+    a = ms_merge(a, b);
+  }
+  if (lane == 0) {
+    float l = a.m + logf(a.s);
+    lse[row] = l;
+    long tt = (long)tg[row];
+    float out = 0.f;
+    if (tt >= 0) {
+      float xt = bf2f(logits[row * V + tt]);
+      float st = cap > 0.f ? cap * tanh_fast(xt / cap) : xt;
+      out = (l - st) * (row_w ? row_w[row] : 1.0f);
+    }
+    loss[row] = out;
+  }
+}
+
+}  // namespace
+
+// logits bf16 [rows][V]; targets int64 (idx64) or int32, negative = ignored; row_w fp32 [rows] or NULL;
+// loss fp32 [rows] (already weighted); lse fp32 [rows]. softcap <= 0 means no softcap.
+extern "C" int tfb_loss_fwd(const void* logits, const void* targets, int idx64, const void* row_w, void* loss, void* lse,
+                            long rows, int V, float softcap, void* stream) {
+  if (!logits || !targets || !loss || !lse) return TFB_ERR_ARG;
+  if (rows <= 0 || V <= 0 || V % 8) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  if (idx64)
+    hipLaunchKernelGGL(loss_fwd_kernel<long>, dim3((unsigned)rows), dim3(256), 0, s, (const bf16_t*)logits, (const long*)targets,
+                       (const float*)row_w, (float*)loss, (float*)lse, V, softcap);
+  else
+    hipLaunchKernelGGL(loss_fwd_kernel<int>, dim3((unsigned)rows), dim3(256), 0, s, (const bf16_t*)logits, (const int*)targets,
+                       (const float*)row_w, (float*)loss, (float*)lse, V, softcap);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// dlogits may alias logits (in place). grow fp32 [rows] = upstream gradient of each row's loss times its weight.
+extern "C" int tfb_loss_bwd(const void* logits, const void* targets, int idx64, const void* lse, const void* grow, void* dlogits,
+                            long rows, int V, float softcap, void* stream) {
+  if (!logits || !targets || !lse || !grow || !dlogits) return TFB_ERR_ARG;
+  if (rows <= 0 || V <= 0 || V % 8) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  if (idx64)
+    hipLaunchKernelGGL(loss_bwd_kernel<long>, dim3((unsigned)rows), dim3(256), 0, s, (const bf16_t*)logits, (const long*)targets,
+                       (const float*)lse, (const float*)grow, (bf16_t*)dlogits, V, softcap);
+  else
+    hipLaunchKernelGGL(loss_bwd_kernel<int>, dim3((unsigned)rows), dim3(256), 0, s, (const bf16_t*)logits, (const int*)targets,
+                       (const float*)lse, (const float*)grow, (bf16_t*)dlogits, V, softcap);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// Fused LM head forward: x bf16 [rows][d], W bf16 [V][d] -> logits bf16 [rows][V], loss fp32 [rows], lse fp32 [rows].
+// part: fp32 scratch [rows][V/64][2].
+extern "C" int tfb_lmhead_fwd(const void* x, const void* W, const void* targets, int idx64, const void* row_w, void* logits,
+                              void* part, void* loss, void* lse, long rows, int d, int V, float softcap, void* stream) {
+  if (!x || !W || !targets || !logits || !part || !loss || !lse) return TFB_ERR_ARG;
+  if (rows <= 0 || rows % 128 || V <= 0 || V % 128 || d <= 0 || d % 64) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  using Cfg = GemmCfg<128, 128, 2, 2, 2, TFB_K_CONTIG, TFB_K_CONTIG>;
+  GemmOperand P{(const uint8_t*)W, (long)d * 2}, Q{(const uint8_t*)x, (long)d * 2};
+  EpiLmHead e{(bf16_t*)logits, (float*)part, (long)V, V / 64, softcap};
+  int st = gemm_launch<Cfg>(P, Q, V, (int)rows, (long)d * 2, 1, LoadIdentity{}, LoadIdentity{}, e, s);
+  if (st != TFB_OK) return st;
+  unsigned nb = (unsigned)((rows + 3) / 4);
+  if (idx64)
+    hipLaunchKernelGGL(lmhead_finish_kernel<long>, dim3(nb), dim3(256), 0, s, (const float*)part, (const bf16_t*)logits,
+                       (const long*)targets, (const float*)row_w, (float*)loss, (float*)lse, rows, (long)V, V / 64, softcap);
+  else
+    hipLaunchKernelGGL(lmhead_finish_kernel<int>, dim3(nb), dim3(256), 0, s, (const float*)part, (const bf16_t*)logits,
+                       (const int*)targets, (const float*)row_w, (float*)loss, (float*)lse, rows, (long)V, V / 64, softcap);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}

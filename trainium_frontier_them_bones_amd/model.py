@@ -1,0 +1,179 @@
+"""Decoder-only transformer training step on the HIP kernels: the caller side of the hot path.
+
+The reference's model is GPT / Block / CausalSelfAttention / MLP (round1/source/train.py:8713-9237,
+round2/source/train.py:10136-11750) driven by `loss = model(x, y); loss.backward(); optimizer.step()`
+(round1/source/train.py:10328-10367). This module is that loop for the benchmark configuration: pre-norm blocks
+(weighted RMSNorm, fused QKV projection, RoPE, causal attention, output projection, residual add fused with the
+next norm, fp8 squared-ReLU MLP), untied LM head with the fused loss, AdamW on fp32 masters with bf16 working
+weights. Every tensor op is one of the library's kernels; torch provides memory, streams and the autograd tape.
+"""
+import math
+from dataclasses import dataclass
+
+import torch
+
+from . import autograd as A
+from . import ops
+
+bf16 = torch.bfloat16
+
+
+@dataclass
+class GPTConfig:
+    n_layer: int = 12
+    d_model: int = 768
+    n_head: int = 12
+    d_ff: int = 3072
+    vocab: int = 32768
+    seq_len: int = 2048
+    rope_base: float = 10000.0
+    norm_eps: float = 1e-6
+    softcap: float = 0.0          # 0 = no logit softcap (the reference model uses 15)
+    init_std: float = 0.02
+    e4m3_limit: float = 240.0     # fp8 scale search limit (240 = the reference's rows, 448 = OCP maximum)
+    x_scale: float = 4.0          # constant activation scale of the fp8 MLP input (a unit-RMS norm output)
+
+    @property
+    def head_dim(self):
+        return self.d_model // self.n_head
+
+
+def rope_tables(T, D, base, device):
+    """cos, sin bf16 [T, D/2] (round1/source/train.py:8951-8962)."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, D, 2, dtype=torch.float32) / D))
+    ang = torch.outer(torch.arange(T, dtype=torch.float32), inv_freq)
+    return ang.cos().to(bf16).to(device), ang.sin().to(bf16).to(device)
+
+
+class FlatParams:
+    """Parameters of one AdamW group as views into flat buffers: bf16 working copy, fp32 master, fp32 moments and a
+    gradient buffer (bf16 for matrices, fp32 for the rest), so the optimizer is one launch per group."""
+
+    def __init__(self, shapes, grad_dtype, device):
+        self.names = list(shapes)
+        self.shapes = shapes
+        sizes = [int(math.prod(s)) for s in shapes.values()]
+        pad = [(-n) % 8 for n in sizes]
+        self.offsets = {}
+        off = 0
+        for name, n, p in zip(self.names, sizes, pad):
+            self.offsets[name] = (off, n)
+            off += n + p
+        self.numel = off
+        self.w = torch.zeros(off, dtype=bf16, device=device)
+        self.master = torch.zeros(off, dtype=torch.float32, device=device)
+        self.m = torch.zeros(off, dtype=torch.float32, device=device)
+        self.v = torch.zeros(off, dtype=torch.float32, device=device)
+        self.grad = torch.zeros(off, dtype=grad_dtype, device=device)
+        self.params = {}
+        for name in self.names:
+            o, n = self.offsets[name]
+            p = self.w[o:o + n].view(shapes[name]).requires_grad_(True)
+            p.grad_buf = self.grad[o:o + n].view(shapes[name])
+            p.grad_fresh = True
+            self.params[name] = p
+
+    def load(self, name, value):
+        o, n = self.offsets[name]
+        self.master[o:o + n].copy_(value.reshape(-1).float())
+        self.w[o:o + n].copy_(value.reshape(-1).to(bf16))
+
+    def mark_fresh(self):
+        for p in self.params.values():
+            p.grad_fresh = True
+
+
+class GPT:
+    def __init__(self, cfg: GPTConfig, device, seed=0):
+        self.cfg = cfg
+        self.device = device
+        d, F, V, L = cfg.d_model, cfg.d_ff, cfg.vocab, cfg.n_layer
+        mats, others = {}, {}
+        others["wte"] = (V, d)
+        for i in range(L):
+            others["norm1.%d" % i] = (d,)
+            mats["w_qkv.%d" % i] = (3 * d, d)
+            mats["w_o.%d" % i] = (d, d)
+            others["norm2.%d" % i] = (d,)
+            mats["w_fc.%d" % i] = (F, d)
+            mats["w_proj.%d" % i] = (d, F)
+        others["norm_f"] = (d,)
+        mats["lm_head"] = (V, d)
+        self.mats = FlatParams(mats, bf16, device)
+        self.others = FlatParams(others, torch.float32, device)
+        self.p = {}
+        self.p.update(self.mats.params)
+        self.p.update(self.others.params)
+        self.mlp_state = [A.Mlp8State(cfg.e4m3_limit, cfg.x_scale) for _ in range(L)]
+        self.cos, self.sin = rope_tables(cfg.seq_len, cfg.head_dim, cfg.rope_base, device)
+        self.step_count = 0
+        self.init_weights(seed)
+
+    def init_weights(self, seed):
+        """N(0, init_std) for every matrix and the embedding, ones for the norm weights; generated on the CPU so that
+        the oracle model can be given identical values."""
+        g = torch.Generator().manual_seed(seed)
+        self.init_values = {}
+        for grp in (self.mats, self.others):
+            for name in grp.names:
+                shape = grp.shapes[name]
+                if name.startswith("norm"):
+                    val = torch.ones(shape)
+                else:
+                    val = torch.randn(shape, generator=g) * self.cfg.init_std
+                val = val.to(bf16)
+                self.init_values[name] = val
+                grp.load(name, val.to(self.device))
+        self.refresh_fp8()
+
+    def refresh_fp8(self):
+        """Per-optimizer-step refresh of each layer's fp8 scale row and e4m3 weight pack."""
+        for i, st in enumerate(self.mlp_state):
+            st.refresh(self.p["w_fc.%d" % i], self.p["w_proj.%d" % i])
+
+    def forward(self, idx, targets):
+        cfg, p = self.cfg, self.p
+        B, T = idx.shape
+        scale = 1.0 / math.sqrt(cfg.head_dim)
+        x = A.EmbeddingFn.apply(idx, p["wte"])
+        h = A.RMSNormFn.apply(x, p["norm1.0"], cfg.norm_eps)
+        for i in range(cfg.n_layer):
+            qkv = A.LinearFn.apply(h, p["w_qkv.%d" % i])
+            att = A.RopeAttentionFn.apply(qkv, self.cos[:T], self.sin[:T], cfg.n_head, scale)
+            att = A.LinearFn.apply(att, p["w_o.%d" % i])
+            x, h = A.AddRMSNormFn.apply(x, att, p["norm2.%d" % i], cfg.norm_eps)
+            m = A.Mlp8Fn.apply(h, p["w_fc.%d" % i], p["w_proj.%d" % i], self.mlp_state[i])
+            nw = p["norm1.%d" % (i + 1)] if i + 1 < cfg.n_layer else p["norm_f"]
+            x, h = A.AddRMSNormFn.apply(x, m, nw, cfg.norm_eps)
+        return A.LmHeadLossFn.apply(h, p["lm_head"], targets, cfg.softcap, "mean")
+
+    def zero_grad(self):
+        self.mats.mark_fresh()
+        self.others.mark_fresh()
+
+    def optimizer_step(self, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1):
+        self.step_count += 1
+        for grp, wd in ((self.mats, weight_decay), (self.others, 0.0)):
+            ops.adamw_(grp.master, grp.grad, grp.m, grp.v, self.step_count, lr, betas[0], betas[1], eps, wd, grp.w)
+        self.refresh_fp8()
+        self.zero_grad()
+
+    def train_step(self, idx, targets, **opt):
+        """One fwd + bwd + AdamW step; returns the loss tensor (no host sync)."""
+        loss = self.forward(idx, targets)
+        loss.backward()
+        self.optimizer_step(**opt)
+        return loss
+
+    def num_params(self):
+        return sum(int(math.prod(s)) for grp in (self.mats, self.others) for s in grp.shapes.values())
+
+
+def zipf_tokens(B, T, vocab, s=1.1, seed=0):
+    """B sequences of T+1 token ids drawn Zipfian (p_r ~ r^-s) on the CPU: (inputs [B,T], next-token targets [B,T])."""
+    g = torch.Generator().manual_seed(seed)
+    ranks = torch.arange(1, vocab + 1, dtype=torch.float64)
+    prob = ranks.pow(-s)
+    prob = prob / prob.sum()
+    tok = torch.multinomial(prob.float(), B * (T + 1), replacement=True, generator=g).view(B, T + 1)
+    return tok[:, :-1].contiguous(), tok[:, 1:].contiguous()

@@ -78,8 +78,9 @@ def rmsnorm_fwd(x, weight=None, eps=2.0 ** -23, res=None):
     return s, y, inv
 
 
-def rmsnorm_bwd(gy, s, inv, weight=None, gs=None, dw=None):
-    """dx = gs + J^T(gy) for y = RMSNorm(s) * weight. Returns (dx, dw fp32 [C] or None); dw given => accumulated into."""
+def rmsnorm_bwd(gy, s, inv, weight=None, gs=None, dw=None, accumulate=False):
+    """dx = gs + J^T(gy) for y = RMSNorm(s) * weight. Returns (dx, dw fp32 [C] or None); a given dw is written, or
+    added into with accumulate=True."""
     _chk(gy), _chk(s), _chk(weight), _chk(gs), _chk(inv, torch.float32)
     C = s.shape[-1]
     rows = s.numel() // C
@@ -93,7 +94,7 @@ def rmsnorm_bwd(gy, s, inv, weight=None, gs=None, dw=None):
             dw = torch.empty(C, dtype=torch.float32, device=s.device)
         else:
             _chk(dw, torch.float32)
-            acc = 1
+            acc = int(accumulate)
     _lib.call("tfb_rmsnorm_bwd", _p(gy), _p(gs), _p(s), _p(weight), _p(inv), _p(dx), _p(part), _p(dw), acc, rows, C,
               _stream())
     return dx, dw
@@ -227,3 +228,188 @@ def mlp_dw_proj(dy2, r, out=None, accumulate=False, out_dtype=bf16):
     _lib.call("tfb_mlp_dw_proj", _p(dy2), _p(r), _p(out), M, d, F, int(out.dtype == torch.float32), int(accumulate), _p(ws),
               ws.numel() * 4, _stream())
     return out
+
+
+# ------------------------------------------------------------------------------------------ attention
+import ctypes as _ct
+
+_L3 = _ct.c_long * 3
+
+
+def _bht(t, layout):
+    """(batch, head, token) element strides of a 4-D tensor given as "bhtd" or "bthd" (head dim contiguous)."""
+    if t.stride(3) != 1:
+        raise RuntimeError("head dimension must be contiguous")
+    if layout == "bhtd":
+        return _L3(t.stride(0), t.stride(1), t.stride(2))
+    return _L3(t.stride(0), t.stride(2), t.stride(1))
+
+
+def _attn_chk(t):
+    if not t.is_cuda or t.dtype != bf16:
+        raise TypeError("attention takes bf16 device tensors")
+
+
+def attn_fwd(q, k, v, scale, layout="bhtd"):
+    """q, k, v: 4-D views [B,H,T,D] ("bhtd") or [B,T,H,D] ("bthd"), arbitrary batch/head/token strides.
+    Returns o [B,T,H,D] contiguous and lse [B,H,T] fp32."""
+    for t in (q, k, v):
+        _attn_chk(t)
+    if layout == "bhtd":
+        B, H, T, D = q.shape
+    else:
+        B, T, H, D = q.shape
+    o = torch.empty(B, T, H, D, dtype=bf16, device=q.device)
+    lse = torch.empty(B, H, T, dtype=torch.float32, device=q.device)
+    _lib.call("tfb_attn_fwd", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o), _bht(o, "bthd"),
+              _p(lse), B, H, T, D, float(scale), _stream())
+    return o, lse
+
+
+def attn_bwd(q, k, v, o, do, lse, scale, layout="bhtd", dq=None, dk=None, dv=None, out_layout="bhtd"):
+    """Gradients of attn_fwd. o, do are [B,T,H,D]. dq/dk/dv may be given as (strided) views with `out_layout`;
+    otherwise dq, dk are allocated [B,H,T,D] and dv [B,T,H,D] (returned as a [B,H,T,D] view), as the reference returns."""
+    for t in (q, k, v, o, do):
+        _attn_chk(t)
+    if layout == "bhtd":
+        B, H, T, D = q.shape
+    else:
+        B, T, H, D = q.shape
+    if dq is None:
+        dq = torch.empty(B, H, T, D, dtype=bf16, device=q.device)
+        dk = torch.empty(B, H, T, D, dtype=bf16, device=q.device)
+        dv = torch.empty(B, T, H, D, dtype=bf16, device=q.device).permute(0, 2, 1, 3)
+        out_layout = "bhtd"
+    delta = torch.empty(B, H, T, dtype=torch.float32, device=q.device)
+    _lib.call("tfb_attn_bwd", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o), _bht(o, "bthd"),
+              _p(do), _bht(do, "bthd"), _p(dq), _bht(dq, out_layout), _p(dk), _bht(dk, out_layout), _p(dv),
+              _bht(dv, out_layout), _p(lse), _p(delta), B, H, T, D, float(scale), _stream())
+    return dq, dk, dv
+
+
+# ------------------------------------------------------------------------------------------ elementwise
+def relu2(x):
+    _chk(x)
+    out = torch.empty_like(x)
+    _lib.call("tfb_relu2", _p(x), None, _p(out), x.numel(), 0, _stream())
+    return out
+
+
+def relu2_bwd(x, gy):
+    _chk(x), _chk(gy)
+    out = torch.empty_like(x)
+    _lib.call("tfb_relu2", _p(x), _p(gy), _p(out), x.numel(), 1, _stream())
+    return out
+
+
+def relu2_bwd_from_h(h, dh):
+    _chk(h), _chk(dh)
+    out = torch.empty_like(h)
+    _lib.call("tfb_relu2", _p(h), _p(dh), _p(out), h.numel(), 2, _stream())
+    return out
+
+
+def rope_(x, cos, sin, T, nheads, D, inverse=False, out=None):
+    """Rotate the first nheads*D columns of each row of x ([rows, row_stride] view, contiguous rows) in place
+    (or into `out`). cos, sin: bf16 [T, D/2]; row r is token r % T."""
+    _chk(cos), _chk(sin)
+    if not x.is_cuda or x.dtype != bf16 or x.stride(-1) != 1:
+        raise TypeError("rope_ takes a bf16 device tensor with contiguous rows")
+    x2 = x.reshape(-1, x.shape[-1]) if x.is_contiguous() else x
+    rows, stride = x2.shape[0], x2.stride(0)
+    o = x2 if out is None else out
+    _lib.call("tfb_rope", _p(x2), _p(cos), _p(sin), _p(o), rows, T, nheads, D, stride, o.stride(0), int(inverse), _stream())
+    return x if out is None else out
+
+
+def resmix_bwd(g, x, x0, ab):
+    """dx = g*a, dx0 = g*b, dab = (sum g*x, sum g*x0) for x_new = a*x + b*x0; ab: fp32 device [2]."""
+    _chk(g), _chk(x), _chk(x0), _chk(ab, torch.float32)
+    dx, dx0 = torch.empty_like(g), torch.empty_like(g)
+    nb = _lib.lib().tfb_resmix_bwd_blocks(g.numel())
+    part = torch.empty(2 * nb, dtype=torch.float32, device=g.device)
+    dab = torch.empty(2, dtype=torch.float32, device=g.device)
+    _lib.call("tfb_resmix_bwd", _p(g), _p(x), _p(x0), _p(ab), _p(dx), _p(dx0), _p(part), _p(dab), g.numel(), _stream())
+    return dx, dx0, dab
+
+
+def embedding_fwd(idx, weight):
+    _chk(weight)
+    if idx.dtype not in (torch.int64, torch.int32) or not idx.is_cuda:
+        raise TypeError("idx must be an int32/int64 device tensor")
+    idx = idx.contiguous()
+    C = weight.shape[1]
+    out = torch.empty(*idx.shape, C, dtype=bf16, device=weight.device)
+    _lib.call("tfb_embedding_fwd", _p(idx), int(idx.dtype == torch.int64), _p(weight), _p(out), idx.numel(), C, _stream())
+    return out
+
+
+def embedding_bwd(idx, dy, dw):
+    """dw (fp32 [V, C]) += scatter of dy rows by idx."""
+    _chk(dy), _chk(dw, torch.float32)
+    idx = idx.contiguous()
+    _lib.call("tfb_embedding_bwd", _p(idx), int(idx.dtype == torch.int64), _p(dy), _p(dw), idx.numel(), dy.shape[-1], _stream())
+    return dw
+
+
+def fill_f32_(t, val=0.0):
+    _chk(t, torch.float32)
+    _lib.call("tfb_fill_f32", _p(t), float(val), t.numel(), _stream())
+    return t
+
+
+def adamw_(p, g, m, v, step, lr, beta1, beta2, eps, weight_decay, p_bf16=None):
+    """One in-place AdamW update of the fp32 master p (and its optional bf16 copy) from g (fp32 or bf16)."""
+    _chk(p, torch.float32), _chk(m, torch.float32), _chk(v, torch.float32), _chk(g, g.dtype), _chk(p_bf16)
+    if g.dtype not in (torch.float32, bf16):
+        raise TypeError("grad must be fp32 or bf16")
+    bias1 = 1.0 - beta1 ** step
+    bias2 = 1.0 - beta2 ** step
+    _lib.call("tfb_adamw", _p(p), _p(g), int(g.dtype == torch.float32), _p(m), _p(v), _p(p_bf16), p.numel(), float(lr),
+              float(weight_decay), float(1.0 - beta1), float(1.0 - beta2), float(eps), float(bias1), float(bias2), _stream())
+
+
+# ------------------------------------------------------------------------------------------ loss head
+def _tg(targets):
+    if targets.dtype not in (torch.int64, torch.int32) or not targets.is_cuda:
+        raise TypeError("targets must be an int32/int64 device tensor")
+    return targets.contiguous()
+
+
+def loss_fwd(logits2, targets, softcap=15.0, row_w=None):
+    """Row losses (already multiplied by row_w) and lse, from bf16 logits [N, V]; targets < 0 are ignored."""
+    _chk(logits2), _chk(row_w, torch.float32)
+    tg = _tg(targets)
+    N, V = logits2.shape
+    loss = torch.empty(N, dtype=torch.float32, device=logits2.device)
+    lse = torch.empty(N, dtype=torch.float32, device=logits2.device)
+    _lib.call("tfb_loss_fwd", _p(logits2), _p(tg), int(tg.dtype == torch.int64), _p(row_w), _p(loss), _p(lse), N, V,
+              float(softcap or 0.0), _stream())
+    return loss, lse
+
+
+def loss_bwd(logits2, targets, lse, grow, softcap=15.0, inplace=False):
+    """dlogits bf16 [N, V]; grow fp32 [N] = d(total)/d(row loss) * row weight."""
+    _chk(logits2), _chk(lse, torch.float32), _chk(grow, torch.float32)
+    tg = _tg(targets)
+    N, V = logits2.shape
+    out = logits2 if inplace else torch.empty_like(logits2)
+    _lib.call("tfb_loss_bwd", _p(logits2), _p(tg), int(tg.dtype == torch.int64), _p(lse), _p(grow), _p(out), N, V,
+              float(softcap or 0.0), _stream())
+    return out
+
+
+def lmhead_fwd(x2, W, targets, softcap=None, row_w=None):
+    """logits = x2 @ W^T (W [V, d]) with the row log-sum-exp fused into the GEMM epilogue.
+    Returns (logits bf16 [N, V], loss rows fp32 [N], lse fp32 [N])."""
+    _chk(x2), _chk(W), _chk(row_w, torch.float32)
+    tg = _tg(targets)
+    N, d = x2.shape
+    V = W.shape[0]
+    logits = torch.empty(N, V, dtype=bf16, device=x2.device)
+    part = torch.empty(N, V // 64, 2, dtype=torch.float32, device=x2.device)
+    loss = torch.empty(N, dtype=torch.float32, device=x2.device)
+    lse = torch.empty(N, dtype=torch.float32, device=x2.device)
+    _lib.call("tfb_lmhead_fwd", _p(x2), _p(W), _p(tg), int(tg.dtype == torch.int64), _p(row_w), _p(logits), _p(part), _p(loss),
+              _p(lse), N, d, V, float(softcap or 0.0), _stream())
+    return logits, loss, lse
