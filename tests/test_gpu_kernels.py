@@ -1,0 +1,365 @@
+"""Parity of the HIP kernels (called through the C-ABI) against the CPU oracle on the same seeded inputs.
+Tolerances: bit-exact for integer / byte work (fp8 bytes, weight packs, gathers, power-of-two scales); rel-L2 <= 5e-3
+for bf16 paths and <= 2e-2 for fp8 paths; losses within 1e-3 relative."""
+import math
+
+import pytest
+import torch
+
+from helpers import fp8_table, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = 5e-3
+FP8_TOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from trainium_frontier_them_bones_amd import ops as _ops
+    return _ops
+
+
+def _g(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+# ------------------------------------------------------------------------------------------ GEMM
+@pytest.mark.parametrize("shape", [(128, 128, 64), (256, 384, 512), (1024, 768, 768), (768, 768, 8192), (128, 256, 16384)])
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+def test_gemm_layouts(ops, dev, shape, ta, tb):
+    M, N, K = shape
+    g = _g(M + N + K)
+    a = torch.randn((K, M) if ta else (M, K), generator=g).bfloat16()
+    b = torch.randn((N, K) if tb else (K, N), generator=g).bfloat16()
+    ref = (a.float().t() if ta else a.float()) @ (b.float().t() if tb else b.float())
+    c = ops.matmul(a.to(dev), b.to(dev), ta, tb)
+    assert rel_l2(c, ref.bfloat16()) < 1e-3 and rel_l2(c, ref) < BF16_TOL
+    base = torch.randn(M, N, generator=g)
+    c32 = ops.matmul(a.to(dev), b.to(dev), ta, tb, out=base.to(dev).clone(), accumulate=True)
+    assert rel_l2(c32, ref + base) < 1e-5
+    cb = ops.matmul(a.to(dev), b.to(dev), ta, tb, out=base.bfloat16().to(dev), accumulate=True)
+    assert rel_l2(cb, ref + base.bfloat16().float()) < BF16_TOL
+
+
+def test_gemm_rejects_bad_shapes(ops, dev):
+    from trainium_frontier_them_bones_amd._lib import TfbError
+    with pytest.raises(TfbError) as e:
+        ops.matmul(torch.zeros(100, 64, dtype=torch.bfloat16, device=dev), torch.zeros(64, 128, dtype=torch.bfloat16, device=dev))
+    assert e.value.status == 1
+
+
+# ------------------------------------------------------------------------------------------ norms / elementwise
+@pytest.mark.parametrize("C", [256, 768, 1024, 2048])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_rmsnorm_fwd_bwd(ops, dev, C, weighted):
+    from oracle import norm as O
+    g = _g(C)
+    N = 512 + 4
+    x, r, gy, gs = (torch.randn(N, C, generator=g).bfloat16() for _ in range(4))
+    w = (1 + 0.02 * torch.randn(C, generator=g)).bfloat16() if weighted else None
+    eps = 1e-6 if weighted else O.RMS_EPS
+    s, y, inv = ops.rmsnorm_fwd(x.to(dev), None if w is None else w.to(dev), eps, res=r.to(dev))
+    so, yo, invo = O.add_rmsnorm(x, r, w, eps)
+    assert torch.equal(s.cpu(), so)
+    assert (y.cpu() != yo).float().mean().item() < 1e-3 and rel_l2(y, yo) < 1e-3       # at most rare 1-ulp flips
+    assert rel_l2(inv, invo) < 1e-6
+    dx, dw = ops.rmsnorm_bwd(gy.to(dev), s, inv, None if w is None else w.to(dev), gs.to(dev))
+    dxo, dwo = O.add_rmsnorm_backward(gs, gy, so, invo, w)
+    assert rel_l2(dx, dxo) < 1e-3
+    if weighted:
+        assert rel_l2(dw, dwo) < 1e-4
+    _, y1, _ = ops.rmsnorm_fwd(x.to(dev), None if w is None else w.to(dev), eps)
+    assert rel_l2(y1, O.rmsnorm(x, w, eps)[0]) < 1e-3
+
+
+def test_block_head(ops, dev):
+    from oracle import norm as O
+    g = _g(11)
+    x, x0, sk, g1, g2 = (torch.randn(1024, 768, generator=g).bfloat16() for _ in range(5))
+    gains = torch.tensor([0.9, 0.25, -0.4])
+    for skip in (None, sk):
+        xn, xnorm, inv = ops.block_head_fwd(x.to(dev), x0.to(dev), gains.to(dev), None if skip is None else skip.to(dev))
+        o = O.block_head(x, x0, gains[0], gains[1], skip, gains[2])
+        assert torch.equal(xn.cpu(), o[0]) and rel_l2(xnorm, o[1]) < 1e-3
+        dx, dx0, dsk, dg = ops.block_head_bwd(g1.to(dev), g2.to(dev), x.to(dev), x0.to(dev), xn, inv, gains.to(dev),
+                                              None if skip is None else skip.to(dev))
+        ob = O.block_head_backward(g1, g2, x, x0, o[0], o[2], gains[0], gains[1], skip, gains[2])
+        assert rel_l2(dx, ob[0]) < 1e-3 and rel_l2(dx0, ob[1]) < 1e-3
+        assert abs(dg[0].item() - ob[3].item()) < 1e-3 * abs(ob[3].item()) + 0.05
+        assert abs(dg[1].item() - ob[4].item()) < 1e-3 * abs(ob[4].item()) + 0.05
+        if skip is not None:
+            assert rel_l2(dsk, ob[2]) < 1e-3 and abs(dg[2].item() - ob[5].item()) < 1e-3 * abs(ob[5].item()) + 0.05
+
+
+def test_relu2_rope_resmix_embedding_bit_exact(ops, dev):
+    from oracle import attention as OA
+    from oracle import norm as O
+    g = _g(12)
+    x, gy = (torch.randn(512, 3072, generator=g).bfloat16() for _ in range(2))
+    assert torch.equal(ops.relu2(x.to(dev)).cpu(), O.relu2(x))
+    assert torch.equal(ops.relu2_bwd(x.to(dev), gy.to(dev)).cpu(), O.relu2_backward(x, gy))
+    h = O.relu2(x)
+    assert rel_l2(ops.relu2_bwd_from_h(h.to(dev), gy.to(dev)), O.relu2_backward_from_h(h, gy)) < 1e-3
+    B, T, H, D = 2, 256, 4, 64
+    qkv = torch.randn(B, T, 3 * H * D, generator=g).bfloat16()
+    cos, sin = OA.rope_tables(T, D)
+    qd = qkv.to(dev).clone()
+    ops.rope_(qd, cos.to(dev), sin.to(dev), T, 2 * H, D)
+    ref = qkv.clone()
+    ref[..., : 2 * H * D] = OA.rope(qkv[..., : 2 * H * D].reshape(B, T, 2 * H, D), cos, sin).reshape(B, T, 2 * H * D)
+    assert torch.equal(qd.cpu(), ref)                      # the v third is untouched, q and k rotate bit-exactly
+    gback = qd.clone()
+    ops.rope_(gback, cos.to(dev), sin.to(dev), T, 2 * H, D, inverse=True)
+    want = ref.clone()
+    want[..., : 2 * H * D] = OA.rope_backward(ref[..., : 2 * H * D].reshape(B, T, 2 * H, D), cos, sin).reshape(B, T, 2 * H * D)
+    assert torch.equal(gback.cpu(), want)
+    gx, xx, x0 = (torch.randn(4096, 768, generator=g).bfloat16() for _ in range(3))
+    ab = torch.tensor([0.9, 0.3])
+    dx, dx0, dab = ops.resmix_bwd(gx.to(dev), xx.to(dev), x0.to(dev), ab.to(dev))
+    r = O.resmix_backward(gx, xx, x0, ab[0], ab[1])
+    assert torch.equal(dx.cpu(), r[0]) and torch.equal(dx0.cpu(), r[1])
+    assert abs(dab[0].item() - r[2].item()) < 1e-3 * abs(r[2].item()) + 0.05
+    idx = torch.randint(0, 1000, (4, 128), generator=g)
+    idx[0, :64] = 7                                          # heavy collisions
+    w = torch.randn(1000, 768, generator=g).bfloat16()
+    assert torch.equal(ops.embedding_fwd(idx.to(dev), w.to(dev)).cpu(), w[idx])
+    assert torch.equal(ops.embedding_fwd(idx.int().to(dev), w.to(dev)).cpu(), w[idx])
+    dy = torch.randn(4, 128, 768, generator=g).bfloat16()
+    dw = ops.fill_f32_(torch.empty(1000, 768, device=dev), 0.0)
+    ops.embedding_bwd(idx.to(dev), dy.to(dev), dw)
+    want = torch.zeros(1000, 768).index_add_(0, idx.reshape(-1), dy.float().reshape(-1, 768))
+    assert rel_l2(dw, want) < 1e-6
+
+
+def test_adamw(ops, dev):
+    from oracle import optim as O
+    g = _g(13)
+    n = 1 << 18
+    p = torch.randn(n, generator=g)
+    m, v = torch.zeros(n), torch.zeros(n)
+    pd, md, vd = p.to(dev), m.to(dev), v.to(dev)
+    p16 = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    for step in (1, 2, 3):
+        gr = torch.randn(n, generator=g).bfloat16()
+        ops.adamw_(pd, gr.to(dev), md, vd, step, 3e-4, 0.9, 0.95, 1e-8, 0.1, p16)
+        O.adamw_step(p, gr, m, v, step, 3e-4, 0.9, 0.95, 1e-8, 0.1)
+    assert (pd.cpu() - p).abs().max().item() < 5e-7 and rel_l2(md, m) < 1e-6 and rel_l2(vd, v) < 1e-6
+    assert torch.equal(p16.cpu(), pd.cpu().bfloat16())
+
+
+# ------------------------------------------------------------------------------------------ fp8 MLP
+def test_fp8_casts_exhaustive_against_format_tables(ops, dev):
+    from oracle import mlp8 as O
+    allb = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    allb = allb[torch.isfinite(allb.float())]
+    allb = torch.cat([allb, torch.zeros((-allb.numel()) % 8, dtype=torch.bfloat16)])
+    for fmt, name, lim in ((0, "e4m3fn", 448.0), (1, "e5m2", 57344.0)):
+        table = fp8_table(name)
+        for sc in (1.0, 4.0, 0.03125, 2048.0):
+            q = ops.quant_fp8(allb.to(dev), sc, fmt).cpu()
+            v = allb.float() * sc
+            ok = v.abs() <= lim
+            assert torch.equal(q[ok], O.fp8_bytes(v, fmt)[ok])             # every bf16 value: bytes equal torch's cast
+            dec = table[q.long()]
+            assert bool(((dec[ok] - v[ok].double()).abs() <= (v[ok].double().abs() * 2.0 ** -3 + 2.0 ** -10)).all())
+            sat = table[q[~ok].long()].abs()
+            assert bool((sat == lim).all())                               # beyond the range: saturates
+        s = torch.tensor([0.5], device=dev)
+        assert torch.equal(ops.quant_fp8(allb.to(dev), s, fmt).cpu(), ops.quant_fp8(allb.to(dev), 0.5, fmt).cpu())
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 512), (1024, 768, 3072), (384, 1024, 2816 - 2816 % 256)])
+@pytest.mark.parametrize("limit", [240.0, 448.0])
+def test_mlp8_scales_precast_forward_backward(ops, dev, shape, limit):
+    from oracle import mlp8 as O
+    M, d, F = shape
+    g = _g(M + d + F)
+    x = torch.randn(M, d, generator=g).bfloat16()
+    wf = (0.02 * torch.randn(F, d, generator=g)).bfloat16()
+    wp = (0.02 * torch.randn(d, F, generator=g)).bfloat16()
+    dy = torch.randn(M, d, generator=g).bfloat16()
+    row_o = O.forward_scales(wf, wp, limit)
+    xd, wfd, wpd, dyd = x.to(dev), wf.to(dev), wp.to(dev), dy.to(dev)
+    row = ops.mlp8_forward_scales(wfd, wpd, limit)
+    pow2_cols = [0, 1, 2, 3, 4, 11, 12, 13, 14, 15]
+    assert torch.equal(row.cpu()[pow2_cols], row_o[pow2_cols])              # scales and amax: exact
+    assert torch.allclose(row.cpu()[9:11], row_o[9:11], rtol=1e-5)         # norms: fp32 summation order
+    w8 = ops.mlp8_precast(wfd, wpd, row)
+    a8 = O.fp8_bytes(wf.float() * row_o[0], 0)
+    b8 = O.fp8_bytes(wp.float() * row_o[3], 0)
+    for got, want in zip(w8.cpu(), (a8, a8.t(), b8, b8.t())):
+        assert torch.equal(got, want.reshape(-1))
+    y, r = ops.mlp8_fwd(xd, w8, row, F)
+    yo, ro = O.forward(x, wf, wp, row_o)
+    assert rel_l2(r, ro) < 2e-3 and rel_l2(y, yo) < FP8_TOL
+    rowb_o = O.backward_scales(dy, row_o)
+    rowb = ops.mlp8_backward_scales(dyd, row)
+    assert torch.equal(rowb.cpu()[5:9], rowb_o[5:9])
+    dx, h, dpre = ops.mlp8_bwd(dyd, r, w8, rowb)
+    dxo, ho, dpo = O.backward(dy, r.cpu(), wf, wp, rowb_o)
+    assert torch.equal(h.cpu(), ho) and rel_l2(dpre, dpo) < 2e-3 and rel_l2(dx, dxo) < FP8_TOL
+    dwfo, dwpo = O.weight_grads(dy, x, h.cpu(), dpre.cpu())
+    assert rel_l2(ops.matmul(dpre, xd, trans_a=True), dwfo) < BF16_TOL
+    assert rel_l2(ops.mlp_dw_proj(dyd, r), dwpo) < BF16_TOL
+    acc = torch.randn(d, F, generator=g)
+    got = ops.mlp_dw_proj(dyd, r, out=acc.to(dev).clone(), accumulate=True)
+    assert rel_l2(got, (dy.float().t() @ ho.float()) + acc) < 1e-4
+    st = ops.amax_scale(dyd, 28672.0, -40, 60).cpu()
+    assert st[0].item() == rowb_o[5].item() and st[2].item() == dy.float().abs().max().item()
+
+
+def test_mlp8_full_size_properties(ops, dev):
+    """BASELINE config 3 sizes: exact equivariance under a permutation of the tokens and agreement of 512-row slices
+    with the oracle."""
+    from oracle import mlp8 as O
+    M, d, F = 16384, 768, 3072
+    g = _g(3)
+    x = torch.randn(M, d, generator=g).bfloat16()
+    wf = (0.02 * torch.randn(d, F, generator=g)).bfloat16().t().contiguous()      # W_up [768, 3072] -> [F, d]
+    wp = (0.02 * torch.randn(F, d, generator=g)).bfloat16().t().contiguous()      # W_down [3072, 768] -> [d, F]
+    dy = torch.randn(M, d, generator=g).bfloat16()
+    xd, wfd, wpd, dyd = x.to(dev), wf.to(dev), wp.to(dev), dy.to(dev)
+    row = ops.mlp8_forward_scales(wfd, wpd)
+    w8 = ops.mlp8_precast(wfd, wpd, row)
+    y, r = ops.mlp8_fwd(xd, w8, row, F)
+    row_o = O.forward_scales(wf, wp)
+    yo, ro = O.forward(x[:512], wf, wp, row_o)
+    assert rel_l2(y[:512], yo) < FP8_TOL and rel_l2(r[:512], ro) < 2e-3
+    perm = torch.randperm(M, generator=g).to(dev)
+    y2, r2 = ops.mlp8_fwd(xd[perm].contiguous(), w8, row, F)
+    assert torch.equal(r2, r[perm]) and torch.equal(y2, y[perm])                   # tokens are independent: exact equivariance
+    rowb = ops.mlp8_backward_scales(dyd, row)
+    dx, _, dpre = ops.mlp8_bwd(dyd, r, w8, rowb, want_h=False)
+    dxo, _, dpo = O.backward(dy[-512:], r[-512:].cpu(), wf, wp, O.backward_scales(dy, row_o))
+    assert rel_l2(dx[-512:], dxo) < FP8_TOL and rel_l2(dpre[-512:], dpo) < 2e-3
+    assert torch.isfinite(dx.float()).all() and torch.isfinite(y.float()).all()
+
+
+# ------------------------------------------------------------------------------------------ attention
+@pytest.mark.parametrize("shape", [(1, 2, 128, 64), (2, 3, 512, 64), (1, 1, 1024, 64), (1, 2, 256, 128), (2, 1, 512, 128)])
+def test_attention_fwd_bwd(ops, dev, shape):
+    from oracle import attention as O
+    B, H, T, D = shape
+    g = _g(T + H)
+    q, k, v = (torch.randn(B, H, T, D, generator=g).bfloat16() for _ in range(3))
+    do = torch.randn(B, T, H, D, generator=g).bfloat16()
+    scale = 1.0 / math.sqrt(D)
+    o, lse = ops.attn_fwd(q.to(dev), k.to(dev), v.to(dev), scale)
+    oo, lo = O.forward(q, k, v, scale)
+    assert rel_l2(o, oo) < BF16_TOL and rel_l2(lse, lo) < 1e-4
+    assert rel_l2(o, O.sdpa_reference(q, k, v, scale)) < BF16_TOL             # and against the library routine
+    dq, dk, dv = ops.attn_bwd(q.to(dev), k.to(dev), v.to(dev), o, do.to(dev), lse, scale)
+    dqo, dko, dvo = O.backward(q, k, v, o.cpu(), do, lse.cpu(), scale)
+    assert rel_l2(dq, dqo) < BF16_TOL and rel_l2(dk, dko) < BF16_TOL and rel_l2(dv, dvo) < BF16_TOL
+
+
+def test_attention_strided_qkv_and_rejects(ops, dev):
+    from oracle import attention as O
+    from trainium_frontier_them_bones_amd._lib import TfbError
+    B, H, T, D = 2, 4, 256, 64
+    g = _g(5)
+    qkv = torch.randn(B, T, 3 * H * D, generator=g).bfloat16()
+    do = torch.randn(B, T, H, D, generator=g).bfloat16()
+    qd = qkv.to(dev)
+    q, k, v = (t.view(B, T, H, D) for t in qd.split(H * D, dim=-1))
+    o, lse = ops.attn_fwd(q, k, v, 0.125, layout="bthd")
+    q4, k4, v4 = (t.reshape(B, T, H, D).permute(0, 2, 1, 3) for t in qkv.split(H * D, dim=-1))
+    oo, lo = O.forward(q4, k4, v4, 0.125)
+    assert rel_l2(o, oo) < BF16_TOL
+    dqkv = torch.empty_like(qd)
+    dq, dk, dv = (t.view(B, T, H, D) for t in dqkv.split(H * D, dim=-1))
+    ops.attn_bwd(q, k, v, o, do.to(dev), lse, 0.125, "bthd", dq, dk, dv, "bthd")
+    dqo, dko, dvo = O.backward(q4, k4, v4, o.cpu(), do, lse.cpu(), 0.125)
+    want = torch.cat([t.permute(0, 2, 1, 3).reshape(B, T, H * D) for t in (dqo, dko, dvo)], dim=-1)
+    assert rel_l2(dqkv, want) < BF16_TOL
+    with pytest.raises(TfbError):
+        ops.attn_fwd(q[:, :100], k[:, :100], v[:, :100], 0.125, layout="bthd")       # T % 128 != 0
+
+
+def test_attention_full_size_properties(ops, dev):
+    """BASELINE config 2 (B16 H12 T2048 D64, RoPE'd q and k): two (b, h) pairs against the oracle, causality by
+    perturbing the future, and dV with dO = 1 equal to the column sums of P."""
+    from oracle import attention as O
+    B, H, T, D = 16, 12, 2048, 64
+    g = _g(2)
+    q, k, v = (torch.randn(B, H, T, D, generator=g) for _ in range(3))
+    cos, sin = O.rope_tables(T, D, 10000.0, torch.float32)
+    q = O.rope(q.transpose(1, 2), cos, sin).transpose(1, 2).bfloat16().contiguous()
+    k = O.rope(k.transpose(1, 2), cos, sin).transpose(1, 2).bfloat16().contiguous()
+    v = v.bfloat16()
+    do = torch.randn(B, T, H, D, generator=g).bfloat16()
+    qd, kd, vd, dod = q.to(dev), k.to(dev), v.to(dev), do.to(dev)
+    o, lse = ops.attn_fwd(qd, kd, vd, 0.125)
+    dq, dk, dv = ops.attn_bwd(qd, kd, vd, o, dod, lse, 0.125)
+    for (b, h) in ((0, 0), (15, 11)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        oo, lo = O.forward(q[sl], k[sl], v[sl], 0.125)
+        assert rel_l2(o[b:b + 1, :, h:h + 1], oo) < BF16_TOL
+        dqo, dko, dvo = O.backward(q[sl], k[sl], v[sl], o[b:b + 1, :, h:h + 1].cpu(), do[b:b + 1, :, h:h + 1], lse[sl].cpu(), 0.125)
+        assert rel_l2(dq[sl], dqo) < BF16_TOL and rel_l2(dk[sl], dko) < BF16_TOL and rel_l2(dv[sl], dvo) < BF16_TOL
+    k2, v2 = kd.clone(), vd.clone()
+    k2[:, :, 1500:] += 1.0
+    v2[:, :, 1500:] -= 1.0
+    o2, _ = ops.attn_fwd(qd, k2, v2, 0.125)
+    assert torch.equal(o2[:, :1500], o[:, :1500])
+    ones = torch.ones_like(dod)
+    _, _, dv1 = ops.attn_bwd(qd, kd, vd, o, ones, lse, 0.125)
+    p = torch.exp((q[3, 5].float() @ k[3, 5].float().t()) * 0.125 - lse[3, 5].cpu()[:, None]).bfloat16().float() * O.mask(T)
+    assert rel_l2(dv1[3, 5, :, 0], p.sum(0)) < BF16_TOL
+
+
+# ------------------------------------------------------------------------------------------ loss head
+@pytest.mark.parametrize("cap", [15.0, None])
+def test_loss_fwd_bwd(ops, dev, cap):
+    from oracle import loss as O
+    g = _g(21)
+    N, V = 512, 8192
+    x = (3 * torch.randn(N, V, generator=g)).bfloat16()
+    t = torch.randint(0, V, (N,), generator=g)
+    t[5] = -1
+    w = O.row_weights(t, "mean")
+    rows, lse = ops.loss_fwd(x.to(dev), t.to(dev), cap, w.to(dev))
+    ro, lo = O.loss_rows(x, t, cap)
+    assert rel_l2(rows, ro * w) < 1e-5 and rel_l2(lse, lo) < 1e-6
+    assert abs(rows.sum().item() - O.fused_loss(x, t, "mean", cap).item()) < 1e-3 * O.fused_loss(x, t, "mean", cap).item()
+    rows32, _ = ops.loss_fwd(x.to(dev), t.int().to(dev), cap, w.to(dev))
+    assert torch.equal(rows32, rows)
+    grow = torch.rand(N, generator=g) / N
+    d = ops.loss_bwd(x.to(dev), t.to(dev), lse, grow.to(dev), cap)
+    assert rel_l2(d, O.loss_backward(x, t, lo, grow, cap)) < BF16_TOL
+    assert float(d[5].float().abs().max()) == 0.0                              # the ignored row gets no gradient
+
+
+def test_lmhead_config1(ops, dev):
+    """BASELINE config 1 at full size through the autograd layer: RMSNorm -> LM-head GEMM (+lse) -> CE, fwd + bwd."""
+    from oracle import loss as O
+    from trainium_frontier_them_bones_amd import autograd as A
+    g = _g(20261)
+    N, d, V = 8192, 768, 32768
+    x = torch.randn(N, d, generator=g).bfloat16()
+    nw = (1 + 0.02 * torch.randn(d, generator=g)).bfloat16()
+    W = (0.02 * torch.randn(V, d, generator=g)).bfloat16()
+    t = torch.randint(0, V, (N,), generator=g)
+    xd = x.to(dev).requires_grad_(True)
+    nd = nw.to(dev).requires_grad_(True)
+    Wd = W.to(dev).requires_grad_(True)
+    loss = A.LmHeadLossFn.apply(A.RMSNormFn.apply(xd, nd, 1e-6), Wd, t.to(dev), 0.0, "mean")
+    loss.backward()
+    lo, saved = O.lmhead_loss(x, nw, W, t, 1e-6, None)
+    assert abs(loss.item() - lo.item()) < 1e-3 * lo.item()
+    dx, dnw, dW = O.lmhead_loss_backward(x, nw, W, t, saved, 1e-6, None)
+    assert rel_l2(xd.grad, dx) < BF16_TOL and rel_l2(Wd.grad, dW) < BF16_TOL and rel_l2(nd.grad, dnw) < BF16_TOL
+
+
+def test_lmhead_softcap_matches_materialised_path(ops, dev):
+    g = _g(22)
+    N, d, V = 1024, 768, 32768
+    x = torch.randn(N, d, generator=g).bfloat16().to(dev)
+    W = (0.05 * torch.randn(V, d, generator=g)).bfloat16().to(dev)
+    t = torch.randint(0, V, (N,), generator=g).to(dev)
+    logits, rows, lse = ops.lmhead_fwd(x, W, t, 15.0)
+    assert torch.equal(logits, ops.matmul(x, W, trans_b=True))
+    rows2, lse2 = ops.loss_fwd(logits, t, 15.0)
+    assert rel_l2(rows, rows2) < 1e-5 and rel_l2(lse, lse2) < 1e-6

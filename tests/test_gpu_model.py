@@ -1,0 +1,60 @@
+"""The full training step on the HIP kernels against the oracle model (same seeded weights and tokens)."""
+import pytest
+import torch
+
+from helpers import rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def test_small_model_losses_and_gradients_track_oracle(dev):
+    from oracle.model import OracleGPT
+    from trainium_frontier_them_bones_amd.model import GPT, GPTConfig, zipf_tokens
+    cfg = GPTConfig(n_layer=2, d_model=256, n_head=4, d_ff=1024, vocab=1024, seq_len=256)
+    m = GPT(cfg, dev, seed=1)
+    o = OracleGPT(cfg, m.init_values)
+    idx, tg = zipf_tokens(2, 256, cfg.vocab, seed=3)
+    loss = m.forward(idx.to(dev), tg.to(dev))
+    loss.backward()
+    lo = o.forward(idx, tg)
+    lo.backward()
+    assert abs(loss.item() - lo.item()) < 1e-3 * lo.item()
+    # end-to-end gradients compound bf16 / fp8 rounding differences through the layers; the per-kernel tests hold the
+    # tight tolerances, here the last layers must agree closely and the first ones within a few percent
+    assert rel_l2(m.p["lm_head"].grad_buf, o.p["lm_head"].grad) < 2e-2
+    assert rel_l2(m.p["norm_f"].grad_buf, o.p["norm_f"].grad) < 2e-2
+    for name in ("w_qkv.0", "w_fc.0", "wte"):
+        assert rel_l2(m.p[name].grad_buf, o.p[name].grad) < 8e-2, name
+    m2, o2 = GPT(cfg, dev, seed=1), OracleGPT(cfg, m.init_values)
+    for _ in range(4):
+        a = m2.train_step(idx.to(dev), tg.to(dev)).item()
+        b = o2.train_step(idx, tg).item()
+        assert abs(a - b) < 1e-3 * b
+    assert a < 6.5                                                  # it learns
+
+
+def test_gradient_accumulation_in_place(dev):
+    from trainium_frontier_them_bones_amd.model import GPT, GPTConfig, zipf_tokens
+    cfg = GPTConfig(n_layer=1, d_model=256, n_head=4, d_ff=512, vocab=512, seq_len=128)
+    m = GPT(cfg, dev, seed=2)
+    idx, tg = zipf_tokens(4, 128, cfg.vocab, seed=4)
+    idx, tg = idx.to(dev), tg.to(dev)
+    m.zero_grad()
+    m.forward(idx, tg).backward()
+    once = {k: p.grad_buf.clone() for k, p in m.p.items()}
+    m.forward(idx, tg).backward()                                   # second micro-step adds into the same buffers
+    for k, p in m.p.items():
+        assert rel_l2(p.grad_buf, 2 * once[k].float()) < 1e-2, k
+
+
+def test_full_size_step_runs_and_loss_is_sane(dev):
+    from trainium_frontier_them_bones_amd.model import GPT, GPTConfig, zipf_tokens
+    import math
+    cfg = GPTConfig()
+    m = GPT(cfg, dev, seed=0)
+    idx, tg = zipf_tokens(16, cfg.seq_len, cfg.vocab, seed=0)
+    l0 = m.train_step(idx.to(dev), tg.to(dev)).item()
+    assert abs(l0 - math.log(cfg.vocab)) < 0.5                     # random init: loss ~ ln V + var(logits) / 2
+    for _ in range(3):
+        l = m.train_step(idx.to(dev), tg.to(dev)).item()
+    assert l < l0 and math.isfinite(l)

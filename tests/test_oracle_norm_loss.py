@@ -1,0 +1,141 @@
+"""Pins oracle/norm.py, oracle/loss.py, oracle/optim.py against library routines, autograd and closed forms."""
+import math
+
+import torch
+import torch.nn.functional as F
+
+from oracle import loss as OL
+from oracle import norm as ON
+from oracle import optim as OO
+from helpers import rel_l2
+
+
+def test_rmsnorm_matches_library():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(64, 768, generator=g).bfloat16()
+    w = (1 + 0.02 * torch.randn(768, generator=g)).bfloat16()
+    y, inv = ON.rmsnorm(x, w, 1e-6)
+    ref = F.rms_norm(x.float(), (768,), w.float(), 1e-6)
+    assert rel_l2(y, ref) < 4e-3
+    y0, _ = ON.rmsnorm(x, None, ON.RMS_EPS)
+    assert torch.equal(y0, F.rms_norm(x, (768,), None, ON.RMS_EPS))
+    assert torch.allclose(inv, torch.rsqrt(x.float().pow(2).mean(-1) + 1e-6))
+
+
+def test_rmsnorm_backward_is_autograd_and_orthogonal():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(32, 256, generator=g).bfloat16()
+    w = (1 + 0.1 * torch.randn(256, generator=g)).bfloat16()
+    gy = torch.randn(32, 256, generator=g).bfloat16()
+    _, inv = ON.rmsnorm(x, w, 1e-6)
+    dx, dw = ON.rmsnorm_backward(gy, x, inv, w)
+    xd, wd = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    (xd * torch.rsqrt(xd.pow(2).mean(-1, keepdim=True) + 1e-6) * wd).backward(gy.double())
+    assert rel_l2(dx, xd.grad) < 1e-5 and rel_l2(dw, wd.grad) < 1e-5
+    _, inv0 = ON.rmsnorm(x, None, 0.0)
+    dx0, _ = ON.rmsnorm_backward(gy, x, inv0, None)
+    assert float((dx0 * x.float()).sum(-1).abs().max()) < 1e-3    # J^T g is orthogonal to x when eps = 0
+
+
+def test_block_head_and_tail_match_eager_autograd():
+    g = torch.Generator().manual_seed(2)
+    x, x0, sk = (torch.randn(16, 128, generator=g).bfloat16() for _ in range(3))
+    l1, l2, l3 = torch.tensor(0.9), torch.tensor(0.25), torch.tensor(-0.4)
+    x_new, x_norm, inv = ON.block_head(x, x0, l1, l2, sk, l3)
+    assert rel_l2(x_new, 0.9 * x.float() + 0.25 * x0.float() - 0.4 * sk.float()) < 4e-3
+    assert torch.equal(x_norm, F.rms_norm(x_new, (128,), None, ON.RMS_EPS))
+    gn, gm = torch.randn(16, 128, generator=g).bfloat16(), torch.randn(16, 128, generator=g).bfloat16()
+    dx, dx0, dsk, d1, d2, d3 = ON.block_head_backward(gn, gm, x, x0, x_new, inv, l1, l2, sk, l3)
+    xs = [t.double().requires_grad_(True) for t in (x, x0, sk)]
+    ls = [t.double().requires_grad_(True) for t in (l1, l2, l3)]
+    v = ls[0] * xs[0] + ls[1] * xs[1] + ls[2] * xs[2]
+    n = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + ON.RMS_EPS)
+    (v * gn.double()).sum().backward(retain_graph=True)
+    (n * gm.double()).sum().backward()
+    assert rel_l2(dx, xs[0].grad) < 1e-2 and rel_l2(dx0, xs[1].grad) < 1e-2 and rel_l2(dsk, xs[2].grad) < 1e-2
+    assert abs(d1.item() - ls[0].grad.item()) < 2e-2 * abs(ls[0].grad.item()) + 1e-2
+    assert abs(d3.item() - ls[2].grad.item()) < 2e-2 * abs(ls[2].grad.item()) + 1e-2
+    s, y, inv = ON.add_rmsnorm(x, x0)
+    assert torch.equal(s, x + x0) and torch.equal(y, F.rms_norm(s, (128,), None, ON.RMS_EPS))
+
+
+def test_relu2_family():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(8, 256, generator=g).bfloat16()
+    gy = torch.randn(8, 256, generator=g).bfloat16()
+    assert torch.equal(ON.relu2(x), F.relu(x).square())
+    xr = x.float().requires_grad_(True)
+    F.relu(xr).square().backward(gy.float())
+    assert rel_l2(ON.relu2_backward(x, gy), xr.grad) < 4e-3
+    assert rel_l2(ON.relu2_backward_from_h(ON.relu2(x), gy), xr.grad) < 1e-2
+
+
+def test_loss_matches_cross_entropy_and_autograd():
+    g = torch.Generator().manual_seed(4)
+    N, V = 64, 512
+    x = (3 * torch.randn(N, V, generator=g)).bfloat16()
+    t = torch.randint(0, V, (N,), generator=g)
+    t[3] = -1
+    for cap in (15.0, None):
+        s = (cap * torch.tanh(x.float() / cap)) if cap else x.float()
+        rows, lse = OL.loss_rows(x, t, cap)
+        ref = F.cross_entropy(s, t, ignore_index=-1, reduction="none")
+        assert torch.allclose(rows, ref, atol=1e-5)
+        assert abs(OL.fused_loss(x, t, "mean", cap).item() - F.cross_entropy(s, t, ignore_index=-1).item()) < 1e-5
+        xr = x.float().requires_grad_(True)
+        sr = (cap * torch.tanh(xr / cap)) if cap else xr
+        F.cross_entropy(sr, t, ignore_index=-1).backward()
+        d = OL.loss_backward(x.float(), t, lse, OL.row_weights(t, "mean"), cap)
+        assert rel_l2(d, xr.grad) < 1e-5
+        if cap:
+            th = torch.tanh(x.float() / cap)
+            assert float((d / (1 - th * th)).sum(-1).abs().max()) < 1e-6     # sum_v dlogits / (1 - t^2) = 0
+
+
+def test_loss_uniform_logits_is_log_vocab():
+    t = torch.randint(0, 1000, (16,))
+    assert abs(OL.fused_loss(torch.zeros(16, 1000), t, "mean", 15.0).item() - math.log(1000)) < 1e-5
+
+
+def test_lmhead_composition_matches_autograd():
+    g = torch.Generator().manual_seed(5)
+    N, d, V = 128, 64, 256
+    x = torch.randn(N, d, generator=g).bfloat16()
+    nw = (1 + 0.02 * torch.randn(d, generator=g)).bfloat16()
+    W = (0.05 * torch.randn(V, d, generator=g)).bfloat16()
+    t = torch.randint(0, V, (N,), generator=g)
+    loss, saved = OL.lmhead_loss(x, nw, W, t)
+    dx, dnw, dW = OL.lmhead_loss_backward(x, nw, W, t, saved)
+    xd, nd, Wd = (a.double().requires_grad_(True) for a in (x, nw, W))
+    h = xd * torch.rsqrt(xd.pow(2).mean(-1, keepdim=True) + 1e-6) * nd
+    ref = F.cross_entropy(h @ Wd.t(), t)
+    ref.backward()
+    assert abs(loss.item() - ref.item()) < 1e-3 * ref.item()
+    assert rel_l2(dx, xd.grad) < 2e-2 and rel_l2(dW, Wd.grad) < 2e-2 and rel_l2(dnw, nd.grad) < 2e-2
+
+
+def test_adamw_against_torch_and_first_step_closed_form():
+    g = torch.Generator().manual_seed(6)
+    p0 = torch.randn(1000, generator=g)
+    p = p0.clone()
+    m, v = torch.zeros(1000), torch.zeros(1000)
+    ref = torch.nn.Parameter(p0.clone())
+    opt = torch.optim.AdamW([ref], lr=1e-2, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    for step in range(1, 6):
+        gr = torch.randn(1000, generator=g)
+        if step == 1:
+            want = p0 * (1 - 1e-2 * 0.1) - 1e-2 * gr / (gr.abs() + 1e-8)
+        OO.adamw_step(p, gr, m, v, step, 1e-2, 0.9, 0.95, 1e-8, 0.1)
+        if step == 1:
+            assert torch.allclose(p, want, atol=1e-6)
+        ref.grad = gr.clone()
+        opt.step()
+        assert torch.allclose(p, ref.detach(), atol=2e-6)
+
+
+def test_resmix_backward_sums():
+    g = torch.Generator().manual_seed(7)
+    gg, x, x0 = (torch.randn(64, 128, generator=g).bfloat16() for _ in range(3))
+    dx, dx0, da, db = ON.resmix_backward(gg, x, x0, torch.tensor(0.9), torch.tensor(0.3))
+    assert rel_l2(dx, 0.9 * gg.float()) < 4e-3 and rel_l2(dx0, 0.3 * gg.float()) < 4e-3
+    assert abs(da.item() - (gg.float() * x.float()).sum().item()) < 0.5

@@ -77,7 +77,21 @@ def lib():
     return _LIB
 
 
+# name -> list: when an entry point is listed here every call is bracketed by events on torch's current stream
+# (the stream the kernels are launched on) and the (start, end) pair appended; used by the benchmark only.
+TIMED = {}
+
+
 def call(name, *args):
-    st = getattr(lib(), name)(*args)
+    rec = TIMED.get(name) if TIMED else None
+    if rec is None:
+        st = getattr(lib(), name)(*args)
+    else:
+        import torch
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        st = getattr(lib(), name)(*args)
+        e.record()
+        rec.append((s, e))
     if st != 0:
         raise TfbError(name, st)

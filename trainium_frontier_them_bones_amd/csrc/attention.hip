@@ -162,32 +162,33 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnT q, AttnT k, AttnT v
       }
       const bool diag = k0 + 63 > qw0;
       const int kbase = k0 + lh * 4 - myq;  // key - q for element (kt, e) is kbase + kt*32 + (e>>2)*8 + (e&3)
-      float mx = m;
+      float mx = m;                         // running maximum of the raw scores
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          float tv = st[kt][e] * sl2;
-          if (diag && (kbase + kt * 32 + (e >> 2) * 8 + (e & 3) > 0)) tv = -INFINITY;
-          st[kt][e] = tv;
-          mx = fmaxf(mx, tv);
+          if (diag && (kbase + kt * 32 + (e >> 2) * 8 + (e & 3) > 0)) st[kt][e] = -INFINITY;
+          mx = fmaxf(mx, st[kt][e]);
         }
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float alpha = fast_exp2(m - mx);
+      if (__builtin_amdgcn_ballot_w64(mx > m) != 0) {  // some row's maximum moved: rescale (wavefront-uniform branch)
+        const float alpha = fast_exp2((m - mx) * sl2);
+        l *= alpha;
+#pragma unroll
+        for (int i = 0; i < DT; ++i)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) oacc[i][e] *= alpha;
+      }
       m = mx;
-      l *= alpha;
-#pragma unroll
-      for (int i = 0; i < DT; ++i)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) oacc[i][e] *= alpha;
+      const float negm = -mx * sl2;
       uint32_t pk[2][8];
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int e = 0; e < 16; e += 2) {
-          float p0 = fast_exp2(st[kt][e] - m), p1 = fast_exp2(st[kt][e + 1] - m);
+          float p0 = fast_exp2(fmaf(st[kt][e], sl2, negm)), p1 = fast_exp2(fmaf(st[kt][e + 1], sl2, negm));
           uint32_t w = pack2bf(p0, p1);
-          l += bflo(w) + bfhi(w);
+          l = sum2bf(w, l);  // the row sum runs over the rounded values
           pk[kt][e >> 1] = w;
         }
       const uint8_t* vt = cur + KBYTES;
@@ -217,7 +218,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnT q, AttnT k, AttnT v
                  pack2bf(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv)};
       *(u32x2*)(op + (long)myq * o.st + d) = w;
     }
-  if (lh == 0) lse[(long)bh * T + myq] = (m + log2f(l)) * LN2;
+  if (lh == 0) lse[(long)bh * T + myq] = (m * sl2 + log2f(l)) * LN2;  // m is the raw-score maximum
 }
 
 // =========================================================================================== delta
@@ -293,7 +294,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnT q, AttnT k, At
       int m = t2 + i * 128;
       mb[i].load(src, st_, r0 + 4 * (m & 15), 8 * (m >> 4));
     }
-    if (tid < 64) stat = lsep[r0 + tid] * LOG2E;
+    if (tid < 64) stat = -lsep[r0 + tid] * LOG2E;  // negated: the exponent is one fma
     else if (tid < 128) stat = delp[r0 + tid - 64];
   };
   auto sstore = [&](uint8_t* buf) {
@@ -349,7 +350,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnT q, AttnT k, At
         float p[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          p[i] = fast_exp2(S[4 * j + i] * sl2 - L[i]);
+          p[i] = fast_exp2(fmaf(S[4 * j + i], sl2, L[i]));
           if (diag && (kq - 8 * j - i > 0)) p[i] = 0.f;
         }
         uint32_t w0 = pack2bf(p[0], p[1]), w1 = pack2bf(p[2], p[3]);
@@ -415,7 +416,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnT q, AttnT k, Attn
     qf[s] = *(const bf16x8*)(qp + (long)myq * q.st + 16 * s + 8 * lh);
     gf[s] = *(const bf16x8*)(gp + (long)myq * go.st + 16 * s + 8 * lh);
   }
-  const float myL = lse[(long)bh * T + myq] * LOG2E;
+  const float myL = -lse[(long)bh * T + myq] * LOG2E;
   const float myD = delta[(long)bh * T + myq];
 
   const int ntiles = (q0 + 128) / 64;
@@ -493,7 +494,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnT q, AttnT k, Attn
       uint32_t dsw[8];
 #pragma unroll
       for (int e = 0; e < 16; e += 2) {
-        float p0 = fast_exp2(S[e] * sl2 - myL), p1 = fast_exp2(S[e + 1] * sl2 - myL);
+        float p0 = fast_exp2(fmaf(S[e], sl2, myL)), p1 = fast_exp2(fmaf(S[e + 1], sl2, myL));
         if (diag && (kbase + (e >> 2) * 8 + (e & 3) > 0)) p0 = 0.f;
         if (diag && (kbase + ((e + 1) >> 2) * 8 + ((e + 1) & 3) > 0)) p1 = 0.f;
         uint32_t w = pack2bf(p0, p1);
@@ -577,7 +578,7 @@ int bwd_impl(AttnT q, AttnT k, AttnT v, AttnT o, AttnT go, AttnT dq, AttnT dk, A
 extern "C" int tfb_attn_fwd(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs, void* o,
                             const long* os, void* lse, int B, int H, int T, int D, float scale, void* stream) {
   if (!q || !k || !v || !o || !lse || !qs || !ks || !vs || !os) return TFB_ERR_ARG;
-  if (B <= 0 || H <= 0 || T <= 0 || T % 128 || D != 64) return TFB_ERR_SHAPE;  // the D = 128 instantiation is switched off (wrong results, cause not yet found)
+  if (B <= 0 || H <= 0 || T <= 0 || T % 128 || (D != 64 && D != 128)) return TFB_ERR_SHAPE;
   if (!strides_ok(qs) || !strides_ok(ks) || !strides_ok(vs) || !strides_ok(os)) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   if (D == 64) return fwd_impl<64>(mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), (float*)lse, B, H, T, scale, s);
@@ -591,7 +592,7 @@ extern "C" int tfb_attn_bwd(const void* q, const long* qs, const void* k, const 
                             float scale, void* stream) {
   if (!q || !k || !v || !o || !go || !dq || !dk || !dv || !lse || !delta) return TFB_ERR_ARG;
   if (!qs || !ks || !vs || !os || !gos || !dqs || !dks || !dvs) return TFB_ERR_ARG;
-  if (B <= 0 || H <= 0 || T <= 0 || T % 128 || D != 64) return TFB_ERR_SHAPE;  // the D = 128 instantiation is switched off (wrong results, cause not yet found)
+  if (B <= 0 || H <= 0 || T <= 0 || T % 128 || (D != 64 && D != 128)) return TFB_ERR_SHAPE;
   if (!strides_ok(qs) || !strides_ok(ks) || !strides_ok(vs) || !strides_ok(os) || !strides_ok(gos) || !strides_ok(dqs) ||
       !strides_ok(dks) || !strides_ok(dvs))
     return TFB_ERR_SHAPE;

@@ -34,14 +34,23 @@ __device__ __forceinline__ bf16_t f2bf(float f) {
   return (bf16_t)(u >> 16);
 }
 
-// Two fp32 -> packed bf16 pair (lo in bits 0..15) with gfx950's v_cvt_pk_bf16_f32 (round to nearest even).
+// Two fp32 -> packed bf16 pair (lo in bits 0..15), round to nearest even. Written as a vector conversion so that the
+// compiler selects gfx950's v_cvt_pk_bf16_f32 itself: as inline assembly the instruction is opaque to the hazard
+// recognizer, and a conversion scheduled right behind the MFMA / transcendental that feeds it read stale lanes.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack2bf(float lo, float hi) {
-  uint32_t r;
-  asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
-  return r;
+  f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 __device__ __forceinline__ float bflo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bfhi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// acc + lo + hi of a packed bf16 pair in one instruction (v_dot2c_f32_bf16 against the pair (1, 1)).
+__device__ __forceinline__ float sum2bf(uint32_t w, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), acc,
+                                         false);
+}
 
 // Round an fp32 value to the nearest bf16 and return it as fp32 (a rounding point of the
 // reference arithmetic that stays in registers).

@@ -1,12 +1,19 @@
 // MFMA GEMM core for gfx950: D[p][q] = sum_k P[p][k] * Q[q][k], fp32 accumulation.
 //
 // One workgroup of WP x WQ wavefronts owns a BP x BQ output tile. Both operand tiles are
-// staged in LDS as [row][128 bytes of k] with a 16-byte row pad (conflict-free 128-bit
-// fragment reads), double-buffered, the next k-tile's global loads in flight while the
-// MFMAs of the current one run. The P tile feeds the MFMA A operand (rows), the Q tile
-// the B operand (columns), so a lane ends up holding D[p .. p+3][q] for four consecutive
-// p: callers put the dimension that is contiguous in the output on the P side and get
-// 64- or 128-bit stores from the epilogue.
+// staged in LDS as [row][128 bytes of k], the eight 16-byte chunks of a row XOR-swizzled by
+// a function of the row so that 128-bit fragment reads, 128-bit row writes and the 64-bit
+// transposing writes are all free of bank conflicts. Staging is double-buffered (NBUF 2: the
+// next k-tile's global loads are in flight while the MFMAs of the current one run, one barrier
+// per k-tile) or single-buffered (NBUF 1: half the LDS, two barriers, more workgroups per CU).
+// The P tile feeds the MFMA A operand (rows), the Q tile the B operand (columns), so a lane
+// ends up holding D[p .. p+3][q] for four consecutive p: callers put the dimension that is
+// contiguous in the output on the P side.
+//
+// Epilogues: "staged" (default) - the accumulators go through LDS once and every thread then
+// owns 8 consecutive p of one q, so global reads/writes of the epilogue are 128-bit and
+// coalesced along the output rows; or "tile" (kTileEpilogue) - the functor gets the raw
+// accumulator registers (used when the epilogue reduces along p in registers).
 //
 // Element types: bf16 (v_mfma_f32_32x32x16_bf16, 64 k per tile) or OCP fp8
 // (v_mfma_scale_f32_32x32x64_f8f6f4 with unit scales, 128 k per tile, e4m3/e5m2 per side).
@@ -20,7 +27,7 @@
 
 #define TFB_K_CONTIG 0
 #define TFB_K_STRIDED 1
-#define TFB_LDS_ROW 144  // 128 bytes of k + 16 pad
+#define TFB_LDS_ROW 128
 
 struct GemmOperand {
   const uint8_t* base;
@@ -38,17 +45,28 @@ struct LoadIdentity {
   __device__ __forceinline__ u32x4 operator()(u32x4 v) const { return v; }
 };
 
-template <int BP_, int BQ_, int WP_, int WQ_, int ES_, int LAYP_, int LAYQ_, int FMTP_ = 0, int FMTQ_ = 0>
+// Byte offset of 16-byte chunk `chunk` of row `row` in a swizzled tile. Over any 8 consecutive rows, and over the 8
+// same-parity rows of any aligned 16, the swizzle takes 8 distinct values.
+__device__ __forceinline__ int lds_off(int row, int chunk) {
+  return row * TFB_LDS_ROW + (((chunk ^ (row + (row >> 3))) & 7) << 4);
+}
+
+template <int BP_, int BQ_, int WP_, int WQ_, int ES_, int LAYP_, int LAYQ_, int FMTP_ = 0, int FMTQ_ = 0, int NBUF_ = 2>
 struct GemmCfg {
-  static constexpr int BP = BP_, BQ = BQ_, WP = WP_, WQ = WQ_, ES = ES_;
+  static constexpr int BP = BP_, BQ = BQ_, WP = WP_, WQ = WQ_, ES = ES_, NBUF = NBUF_;
   static constexpr int LAYP = LAYP_, LAYQ = LAYQ_, FMTP = FMTP_, FMTQ = FMTQ_;
   static constexpr int NT = WP * WQ * 64;
   static constexpr int TP = BP / WP / 32, TQ = BQ / WQ / 32;
   static constexpr int BK = 128 / ES;  // elements of k per tile
-  static constexpr int LDS_BYTES = 2 * (BP + BQ) * TFB_LDS_ROW;
+  static constexpr int TILE_BYTES = (BP + BQ) * TFB_LDS_ROW;
+  static constexpr int STAGE_LD = BP + 4;  // floats per staged output row
+  static constexpr int STAGE_BYTES = BQ * STAGE_LD * 4;
+  static constexpr int LDS_BYTES = NBUF * TILE_BYTES > STAGE_BYTES ? NBUF * TILE_BYTES : STAGE_BYTES;
   static_assert(ES == 1 || ES == 2, "fp8 or bf16");
+  static_assert(NBUF == 1 || NBUF == 2, "single or double buffering");
   static_assert(ES == 2 || (LAYP == TFB_K_CONTIG && LAYQ == TFB_K_CONTIG), "fp8 operands are k-contiguous");
   static_assert((BP * 8) % NT == 0 && (BQ * 8) % NT == 0, "tile rows vs threads");
+  static_assert((BQ * BP / 8) % NT == 0, "staged epilogue chunks vs threads");
 };
 
 // ---- global -> register -> LDS staging of one operand tile ---------------------------------
@@ -73,7 +91,7 @@ struct TileLoader<ROWS, NT, TFB_K_CONTIG> {
     for (int i = 0; i < N; ++i) {
       int c = tid + i * NT;
       int row = c >> 3, cc = c & 7;
-      *(u32x4*)(lds + row * TFB_LDS_ROW + cc * 16) = pre(g[i]);
+      *(u32x4*)(lds + lds_off(row, cc)) = pre(g[i]);
     }
   }
 };
@@ -104,14 +122,15 @@ struct TileLoader<ROWS, NT, TFB_K_STRIDED> {
       u32x4 v0 = pre(g[i][0]), v1 = pre(g[i][1]), v2 = pre(g[i][2]), v3 = pre(g[i][3]);
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
-        // rows 2w (low halves) and 2w+1 (high halves) of the micro-block
+        // rows 2w (low halves) and 2w+1 (high halves) of the micro-block: 4 consecutive k each
         u32x2 lo, hi;
-        lo.x = (v0[w] & 0xffffu) | (v1[w] << 16);
-        lo.y = (v2[w] & 0xffffu) | (v3[w] << 16);
-        hi.x = (v0[w] >> 16) | (v1[w] & 0xffff0000u);
-        hi.y = (v2[w] >> 16) | (v3[w] & 0xffff0000u);
-        *(u32x2*)(lds + (8 * rg + 2 * w) * TFB_LDS_ROW + kg * 8) = lo;
-        *(u32x2*)(lds + (8 * rg + 2 * w + 1) * TFB_LDS_ROW + kg * 8) = hi;
+        lo.x = __builtin_amdgcn_perm(v1[w], v0[w], 0x05040100u);
+        lo.y = __builtin_amdgcn_perm(v3[w], v2[w], 0x05040100u);
+        hi.x = __builtin_amdgcn_perm(v1[w], v0[w], 0x07060302u);
+        hi.y = __builtin_amdgcn_perm(v3[w], v2[w], 0x07060302u);
+        const int r0 = 8 * rg + 2 * w;
+        *(u32x2*)(lds + lds_off(r0, kg >> 1) + (kg & 1) * 8) = lo;
+        *(u32x2*)(lds + lds_off(r0 + 1, kg >> 1) + (kg & 1) * 8) = hi;
       }
     }
   }
@@ -125,7 +144,7 @@ struct Frag<2> {
   bf16x8 v;
   static constexpr int KSTEPS = 4;  // 4 x 16 bf16 per 128-byte tile row
   __device__ __forceinline__ void read(const uint8_t* lds, int row, int s, int h) {
-    v = *(const bf16x8*)(lds + row * TFB_LDS_ROW + s * 32 + h * 16);
+    v = *(const bf16x8*)(lds + lds_off(row, 2 * s + h));
   }
 };
 template <>
@@ -133,8 +152,8 @@ struct Frag<1> {
   i32x8 v;
   static constexpr int KSTEPS = 2;  // 2 x 64 fp8 per 128-byte tile row
   __device__ __forceinline__ void read(const uint8_t* lds, int row, int s, int h) {
-    const i32x4* p = (const i32x4*)(lds + row * TFB_LDS_ROW + s * 64 + h * 32);
-    i32x4 a = p[0], b = p[1];
+    i32x4 a = *(const i32x4*)(lds + lds_off(row, 4 * s + 2 * h));
+    i32x4 b = *(const i32x4*)(lds + lds_off(row, 4 * s + 2 * h + 1));
     v = i32x8{a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
   }
 };
@@ -161,13 +180,13 @@ struct has_tile_epilogue : std::false_type {};
 template <class T>
 struct has_tile_epilogue<T, std::void_t<decltype(T::kTileEpilogue)>> : std::true_type {};
 
-// Epi: either  __device__ void operator()(int p, int q, f32x4 v, int split)  with v = D[p..p+3][q],
+// Epi: either  __device__ void operator()(int p, int q, const float (&v)[8], int split)  with v = D[p..p+7][q], p % 8 == 0,
 // or (with a static member kTileEpilogue)  __device__ void tile(acc, pw, qw, lr, lh, tile_id, split).
 template <class Cfg, class PreP, class PreQ, class Epi>
 __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, PreQ preq, Epi epi) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   constexpr int BP = Cfg::BP, BQ = Cfg::BQ, NT = Cfg::NT, TP = Cfg::TP, TQ = Cfg::TQ, ES = Cfg::ES;
-  constexpr int BUF = (BP + BQ) * TFB_LDS_ROW;
+  constexpr int BUF = Cfg::TILE_BYTES;
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int wp = wave % Cfg::WP, wq = wave / Cfg::WP;
@@ -196,7 +215,7 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, Pr
   __syncthreads();
 
   for (int t = 0; t < a.nkt; ++t) {
-    const uint8_t* sp = smem + (t & 1) * BUF;
+    const uint8_t* sp = smem + (Cfg::NBUF == 2 ? (t & 1) * BUF : 0);
     const uint8_t* sq = sp + BP * TFB_LDS_ROW;
     const bool more = (t + 1 < a.nkt);
     if (more) {
@@ -215,30 +234,43 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, Pr
 #pragma unroll
         for (int j = 0; j < TQ; ++j) acc[i][j] = mfma32<ES, Cfg::FMTP, Cfg::FMTQ>(fa[i], fb[j], acc[i][j]);
     }
+    if (Cfg::NBUF == 1) __syncthreads();
     if (more) {
-      uint8_t* np_ = smem + ((t + 1) & 1) * BUF;
+      uint8_t* np_ = smem + (Cfg::NBUF == 2 ? ((t + 1) & 1) * BUF : 0);
       lp.store(np_, tid, prep);
       lq.store(np_ + BP * TFB_LDS_ROW, tid, preq);
     }
     __syncthreads();
   }
 
-  const int pw = (int)p0 + wp * (TP * 32), qw = (int)q0 + wq * (TQ * 32);
+  const int pw = wp * (TP * 32), qw = wq * (TQ * 32);  // wavefront's origin inside the tile
   if constexpr (has_tile_epilogue<Epi>::value) {
     // whole-accumulator epilogue: acc[i][j][4*jj + e] = D[pw + 32 i + 8 jj + 4 lh + e][qw + 32 j + lr]
-    epi.tile(acc, pw, qw, lr, lh, lid, (int)blockIdx.z);
+    epi.tile(acc, (int)p0 + pw, (int)q0 + qw, lr, lh, lid, (int)blockIdx.z);
   } else {
+    // (the loop's last barrier has passed: every wavefront is done reading the operand tiles)
+    float* stage = (float*)smem;
+    constexpr int SLD = Cfg::STAGE_LD;
 #pragma unroll
     for (int i = 0; i < TP; ++i)
 #pragma unroll
       for (int j = 0; j < TQ; ++j)
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
-          int p = pw + i * 32 + jj * 8 + lh * 4;
-          int q = qw + j * 32 + lr;
           f32x4 v = {acc[i][j][jj * 4 + 0], acc[i][j][jj * 4 + 1], acc[i][j][jj * 4 + 2], acc[i][j][jj * 4 + 3]};
-          epi(p, q, v, (int)blockIdx.z);
+          *(f32x4*)(stage + (qw + j * 32 + lr) * SLD + pw + i * 32 + jj * 8 + lh * 4) = v;
         }
+    __syncthreads();
+    constexpr int CPR = BP / 8;  // 8-element chunks per output row
+#pragma unroll
+    for (int i = 0; i < BQ * CPR / NT; ++i) {
+      const int c = tid + i * NT;
+      const int q = c / CPR, pc = (c % CPR) * 8;
+      f32x4 lo = *(const f32x4*)(stage + q * SLD + pc);
+      f32x4 hi = *(const f32x4*)(stage + q * SLD + pc + 4);
+      const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      epi((int)p0 + pc, (int)q0 + q, v, (int)blockIdx.z);
+    }
   }
 }
 
@@ -266,4 +298,104 @@ static int gemm_launch(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes
   hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, a, prep, preq, epi);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
+}
+
+// ---- shared epilogue helpers -----------------------------------------------------------------
+__device__ __forceinline__ u32x4 pack8bf(const float (&v)[8]) {
+  u32x4 o = {pack2bf(v[0], v[1]), pack2bf(v[2], v[3]), pack2bf(v[4], v[5]), pack2bf(v[6], v[7])};
+  return o;
+}
+__device__ __forceinline__ void unpack8bf(u32x4 u, float (&v)[8]) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    v[2 * k] = bflo(u[k]);
+    v[2 * k + 1] = bfhi(u[k]);
+  }
+}
+
+// out (bf16 or fp32) [nq][ld] (+)= D
+struct EpiStore {
+  void* out;
+  long ld;  // elements
+  int f32;
+  int accumulate;
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
+    float r[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) r[k] = v[k];
+    if (f32) {
+      float* o = (float*)out + (long)q * ld + p;
+      if (accumulate) {
+        f32x4 c0 = *(const f32x4*)o, c1 = *(const f32x4*)(o + 4);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          r[k] += c0[k];
+          r[4 + k] += c1[k];
+        }
+      }
+      *(f32x4*)o = f32x4{r[0], r[1], r[2], r[3]};
+      *(f32x4*)(o + 4) = f32x4{r[4], r[5], r[6], r[7]};
+    } else {
+      bf16_t* o = (bf16_t*)out + (long)q * ld + p;
+      if (accumulate) {
+        float c[8];
+        unpack8bf(*(const u32x4*)o, c);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) r[k] += c[k];
+      }
+      *(u32x4*)o = pack8bf(r);
+    }
+  }
+};
+
+// fp32 partial of one k-split: ws [splits][nq][ld]
+struct EpiSplit {
+  float* ws;
+  long ld, slab;  // slab = nq * ld
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int split) const {
+    float* o = ws + (long)split * slab + (long)q * ld + p;
+    *(f32x4*)o = f32x4{v[0], v[1], v[2], v[3]};
+    *(f32x4*)(o + 4) = f32x4{v[4], v[5], v[6], v[7]};
+  }
+};
+
+// out (+)= sum over splits of ws, rounded once
+static __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* out, long n, int splits, int f32,
+                                            int accumulate) {
+  long i = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i >= n) return;
+  f32x4 s = *(const f32x4*)(ws + i);
+  for (int k = 1; k < splits; ++k) s += *(const f32x4*)(ws + (long)k * n + i);
+  if (f32) {
+    float* o = (float*)out + i;
+    if (accumulate) s += *(const f32x4*)o;
+    *(f32x4*)o = s;
+  } else {
+    bf16_t* o = (bf16_t*)out + i;
+    if (accumulate) {
+      u32x2 c = *(const u32x2*)o;
+      s[0] += bflo(c.x);
+      s[1] += bfhi(c.x);
+      s[2] += bflo(c.y);
+      s[3] += bfhi(c.y);
+    }
+    u32x2 r = {pack2bf(s[0], s[1]), pack2bf(s[2], s[3])};
+    *(u32x2*)o = r;
+  }
+}
+
+static inline int splitk_reduce(const float* ws, void* out, long n, int splits, int f32, int accumulate, hipStream_t s) {
+  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, s, ws, out, n, splits, f32,
+                     accumulate);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// How many k-splits a token-contraction GEMM with `tiles` output tiles and `nkt` k-tiles should use.
+static inline int choose_splits(long tiles, int nkt, long out_elems, long ws_bytes) {
+  if (tiles >= 512 || nkt < 32) return 1;
+  int splits = (int)((768 + tiles - 1) / tiles);
+  while (splits > 1 && (nkt % splits != 0 || nkt / splits < 8)) --splits;
+  if ((long)splits * out_elems * 4 > ws_bytes) splits = 1;
+  return splits;
 }

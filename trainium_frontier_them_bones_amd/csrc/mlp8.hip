@@ -286,18 +286,19 @@ struct EpiUp {  // pre = x8 @ wf8^T: r, h8
   bf16_t* r;     // [M][F]
   uint8_t* h8;   // [M][F]
   long F;
-  __device__ __forceinline__ void operator()(int p, int q, f32x4 v, int) const {
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
     const float dq = sc[SC_DQ_FC], c = sc[SC_C_H];
-    float rr[4], hh[4];
+    float rr[8], hh[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 8; ++i) {
       rr[i] = round_bf(fmaxf(v[i] * dq, 0.f));
       float rc = round_bf(fminf(rr[i] * c, H_CLAMP));
       hh[i] = rc * rc;
     }
-    u32x2 o = {pack2bf(rr[0], rr[1]), pack2bf(rr[2], rr[3])};
-    *(u32x2*)(r + (long)q * F + p) = o;
-    *(uint32_t*)(h8 + (long)q * F + p) = cvt4_fp8<TFB_FMT_E4M3>(hh[0], hh[1], hh[2], hh[3]);
+    const long off = (long)q * F + p;
+    *(u32x4*)(r + off) = pack8bf(rr);
+    u32x2 o = {cvt4_fp8<TFB_FMT_E4M3>(hh[0], hh[1], hh[2], hh[3]), cvt4_fp8<TFB_FMT_E4M3>(hh[4], hh[5], hh[6], hh[7])};
+    *(u32x2*)(h8 + off) = o;
   }
 };
 
@@ -306,10 +307,12 @@ struct EpiScaleStore {  // out = bf16(acc * sc[col])
   int col;
   bf16_t* out;
   long ld;
-  __device__ __forceinline__ void operator()(int p, int q, f32x4 v, int) const {
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
     const float dq = sc[col];
-    u32x2 o = {pack2bf(v[0] * dq, v[1] * dq), pack2bf(v[2] * dq, v[3] * dq)};
-    *(u32x2*)(out + (long)q * ld + p) = o;
+    float r[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = v[i] * dq;
+    *(u32x4*)(out + (long)q * ld + p) = pack8bf(r);
   }
 };
 
@@ -320,20 +323,21 @@ struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*
   uint8_t* dp8;     // [M][F]
   bf16_t* h;        // [M][F] or null
   long F;
-  __device__ __forceinline__ void operator()(int p, int q, f32x4 v, int) const {
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
     const float dq = sc[SC_DQ_DH2], sdp = sc[SC_S_DP];
     const long off = (long)q * F + p;
-    u32x2 ru = *(const u32x2*)(r + off);
-    float rr[4] = {bflo(ru.x), bfhi(ru.x), bflo(ru.y), bfhi(ru.y)};
-    float dp[4];
+    float rr[8], dp[8];
+    unpack8bf(*(const u32x4*)(r + off), rr);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dp[i] = round_bf((v[i] * dq) * rr[i]);
-    u32x2 o = {pack2bf(dp[0], dp[1]), pack2bf(dp[2], dp[3])};
-    *(u32x2*)(dpre + off) = o;
-    *(uint32_t*)(dp8 + off) = cvt4_fp8<TFB_FMT_E5M2>(dp[0] * sdp, dp[1] * sdp, dp[2] * sdp, dp[3] * sdp);
+    for (int i = 0; i < 8; ++i) dp[i] = round_bf((v[i] * dq) * rr[i]);
+    *(u32x4*)(dpre + off) = pack8bf(dp);
+    u32x2 o = {cvt4_fp8<TFB_FMT_E5M2>(dp[0] * sdp, dp[1] * sdp, dp[2] * sdp, dp[3] * sdp),
+               cvt4_fp8<TFB_FMT_E5M2>(dp[4] * sdp, dp[5] * sdp, dp[6] * sdp, dp[7] * sdp)};
+    *(u32x2*)(dp8 + off) = o;
     if (h) {
-      u32x2 ho = {pack2bf(rr[0] * rr[0], rr[1] * rr[1]), pack2bf(rr[2] * rr[2], rr[3] * rr[3])};
-      *(u32x2*)(h + off) = ho;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) rr[i] = rr[i] * rr[i];
+      *(u32x4*)(h + off) = pack8bf(rr);
     }
   }
 };
@@ -350,37 +354,6 @@ struct LoadSquare {
     return o;
   }
 };
-
-struct EpiSplitF32 {
-  float* ws;
-  long ld, slab;
-  __device__ __forceinline__ void operator()(int p, int q, f32x4 v, int split) const {
-    *(f32x4*)(ws + (long)split * slab + (long)q * ld + p) = v;
-  }
-};
-
-__global__ void reduce_store_kernel(const float* __restrict__ ws, void* out, long n, int splits, int f32, int accumulate) {
-  long i = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
-  if (i >= n) return;
-  f32x4 s = *(const f32x4*)(ws + i);
-  for (int k = 1; k < splits; ++k) s += *(const f32x4*)(ws + (long)k * n + i);
-  if (f32) {
-    float* o = (float*)out + i;
-    if (accumulate) s += *(const f32x4*)o;
-    *(f32x4*)o = s;
-  } else {
-    bf16_t* o = (bf16_t*)out + i;
-    if (accumulate) {
-      u32x2 c = *(const u32x2*)o;
-      s[0] += bflo(c.x);
-      s[1] += bfhi(c.x);
-      s[2] += bflo(c.y);
-      s[3] += bfhi(c.y);
-    }
-    u32x2 r = {pack2bf(s[0], s[1]), pack2bf(s[2], s[3])};
-    *(u32x2*)o = r;
-  }
-}
 
 inline bool shapes8(long M, int d, int F) { return M > 0 && M % 128 == 0 && d > 0 && d % 256 == 0 && F > 0 && F % 256 == 0; }
 
@@ -530,17 +503,14 @@ extern "C" int tfb_mlp_dw_proj(const void* dy, const void* r, void* dw, long M, 
   hipStream_t s = (hipStream_t)stream;
   using Cfg = GemmCfg<128, 128, 2, 2, 2, TFB_K_STRIDED, TFB_K_STRIDED>;
   GemmOperand P{(const uint8_t*)r, (long)F * 2}, Q{(const uint8_t*)dy, (long)d * 2};
-  const int nkt = (int)(M / 64);
   const long tiles = (long)(F / 128) * (d / 128);
-  int splits = (int)((768 + tiles - 1) / tiles);
-  while (splits > 1 && (nkt % splits != 0 || nkt / splits < 8)) --splits;
-  if (!workspace || (long)splits * d * F * 4 > workspace_bytes) return TFB_ERR_WORKSPACE;
-  EpiSplitF32 e{(float*)workspace, (long)F, (long)d * F};
+  const int splits = workspace ? choose_splits(tiles, (int)(M / 64), (long)d * F, workspace_bytes) : 1;
+  if (splits == 1) {
+    EpiStore e{dw, (long)F, out_f32, accumulate};
+    return gemm_launch<Cfg>(P, Q, F, d, M * 2, 1, LoadSquare{}, LoadIdentity{}, e, s);
+  }
+  EpiSplit e{(float*)workspace, (long)F, (long)d * F};
   int st = gemm_launch<Cfg>(P, Q, F, d, M * 2, splits, LoadSquare{}, LoadIdentity{}, e, s);
   if (st != TFB_OK) return st;
-  long nn = (long)d * F;
-  hipLaunchKernelGGL(reduce_store_kernel, dim3((unsigned)((nn / 4 + 255) / 256)), dim3(256), 0, s, (const float*)workspace, dw,
-                     nn, splits, out_f32, accumulate);
-  TFB_LAUNCH_CHECK();
-  return TFB_OK;
+  return splitk_reduce((const float*)workspace, dw, (long)d * F, splits, out_f32, accumulate, s);
 }

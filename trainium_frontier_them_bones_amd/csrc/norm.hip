@@ -161,12 +161,23 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16_t* __restri
   }
 }
 
-__global__ void colsum_kernel(const float* __restrict__ part, float* __restrict__ out, int rows, int C, int accumulate) {
-  int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= C) return;
+// out[c] (+)= sum_r part[r][c]: 64 columns x 16 row lanes per workgroup, rows interleaved over the lanes.
+__global__ __launch_bounds__(1024) void colsum_kernel(const float* __restrict__ part, float* __restrict__ out, int rows, int C,
+                                                     int accumulate) {
+  __shared__ float red[16][64];
+  const int tx = threadIdx.x, ty = threadIdx.y;
+  const int c = blockIdx.x * 64 + tx;
   float t = 0.f;
-  for (int r = 0; r < rows; ++r) t += part[(long)r * C + c];
-  out[c] = accumulate ? out[c] + t : t;
+  if (c < C)
+    for (int r = ty; r < rows; r += 16) t += part[(long)r * C + c];
+  red[ty][tx] = t;
+  __syncthreads();
+  if (ty == 0 && c < C) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s += red[i][tx];
+    out[c] = accumulate ? out[c] + s : s;
+  }
 }
 
 // ------------------------------------------------------------------------------------------ block head
@@ -329,7 +340,7 @@ extern "C" int tfb_rmsnorm_bwd(const void* gy, const void* gs, const void* s, co
 #undef CALL
   TFB_LAUNCH_CHECK();
   if (w) {
-    hipLaunchKernelGGL(colsum_kernel, dim3((C + 255) / 256), dim3(256), 0, (hipStream_t)stream, (const float*)dw_part,
+    hipLaunchKernelGGL(colsum_kernel, dim3((C + 63) / 64), dim3(64, 16), 0, (hipStream_t)stream, (const float*)dw_part,
                        (float*)dw, grid, C, dw_accumulate);
     TFB_LAUNCH_CHECK();
   }
@@ -368,7 +379,7 @@ extern "C" int tfb_block_head_bwd(const void* g_new, const void* g_norm, const v
   DISPATCH_NCH(C, CALL);
 #undef CALL
   TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(colsum_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const float*)gain_part, (float*)dgains,
+  hipLaunchKernelGGL(colsum_kernel, dim3(1), dim3(64, 16), 0, (hipStream_t)stream, (const float*)gain_part, (float*)dgains,
                      grid, 4, 0);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
