@@ -171,6 +171,66 @@ int tfb_loss_bwd(const void* logits, const void* targets, int idx64, const void*
 int tfb_lmhead_fwd(const void* x, const void* W, const void* targets, int idx64, const void* row_w, void* logits, void* part,
                    void* loss, void* lse, long rows, int d, int V, float softcap, void* stream);
 
+/* ---- mixture of experts (top-1 / top-2, all experts on this GPU, dropless ragged slots) -------------------------------
+ * Slot buffer: expert e's assignments are contiguous rows, in token order, padded to a multiple of 128 (zero rows).
+ * Tables (device int32): cnt[E], seg[E+1] padded segment offsets, tile_expert[rmax/128] (-1 beyond the extent),
+ * slot[N][topk], tok[rmax] (-1 = padding), ksel[rmax]. rmax = tfb_moe_max_rows(N, E, topk) (host helper). */
+long tfb_moe_max_rows(long N, int E, int topk);
+
+/* p = softmax(h Wr^T + bias) fp32 [N][E] (logits optional), the top-k experts by first maximum (ties low) and gates
+ * (renormalised over the two at k = 2, the probability at k = 1). h bf16 [N][d], wr fp32 [E][d]; E <= 16.
+ * Replaces the router matmul + moe_route / moe_tournament (round2/source/train.py:10505-10553, 10961). */
+int tfb_moe_route(const void* h, const void* wr, const void* bias, void* logits, void* p, void* idx, void* gate, long N, int d,
+                  int E, int topk, void* stream);
+
+/* The slot tables from idx. scratch: int32 [ceil(N/64) * E].
+ * Replaces moe_positions + moe_gather_tables (round2/source/train.py:10555-10634) without a capacity (nothing is dropped). */
+int tfb_moe_tables(const void* idx, void* cnt, void* seg, void* tile_expert, void* slot, void* tok, void* ksel, void* scratch,
+                   long N, int E, int topk, long rmax, void* stream);
+
+/* xs bf16 [rmax][d] = h[tok] (zero padding rows) and xs8 = e4m3(xs * scale) (scale_ptr device fp32 or scale_imm).
+ * Replaces MoeDispatch2.forward (round2/source/train.py:10652-10660). */
+int tfb_moe_gather(const void* h, const void* tok, const void* scale_ptr, float scale_imm, void* xs, void* xs8, long rmax, int d,
+                   void* stream);
+
+/* Grouped fp8 expert MLP: x8 [rmax][d] -> y bf16 [rmax][d], r bf16 [rmax][F]; w8 uint8 [E][4][F*d] (tfb_mlp8_precast per
+ * expert), rows fp32 [E][16]; h8 [rmax][F] byte scratch.
+ * Replaces moe_experts8_local / moe_expert8_mlp (round2/source/train.py:10731-10776). */
+int tfb_moe_mlp8_fwd(const void* x8, const void* w8, const void* rows, const void* tile_expert, void* y, void* r, void* h8,
+                     long rmax, int d, int F, void* stream);
+int tfb_moe_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* rows, const void* tile_expert, void* dx,
+                     void* dpre, void* dp8, long rmax, int d, int F, void* stream);
+
+/* dw_fc [E][F][d] (+)= dpre_e^T xs_e, dw_proj [E][d][F] (+)= dys_e^T bf16(r_e^2) over each expert's row segment.
+ * Replaces the per-expert weight_grads (round2/source/kernels/nki_mlp_fused8.py:706-711). */
+int tfb_moe_dw(const void* dpre, const void* xs, const void* dys, const void* r, const void* seg, void* dw_fc, void* dw_proj,
+               int E, int d, int F, int out_f32, int accumulate, void* stream);
+
+/* out bf16 [N][d] = sum_k bf16(gate_k) ys[slot_k] (the eager bf16 expression's roundings).
+ * Replaces MoeCombine2.forward + the gated sum (round2/source/train.py:10672-10676, 10990-10992). */
+int tfb_moe_combine(const void* ys, const void* slot, const void* gate, void* out, long N, int d, int topk, void* stream);
+
+/* dys bf16 [rmax][d] = bf16(gate_k) dout[tok]; dgate fp32 [N][topk] = sum_d dout ys.
+ * Replaces MoeCombine2.backward (round2/source/train.py:10678-10688). */
+int tfb_moe_combine_bwd(const void* dout, const void* ys, const void* tok, const void* ksel, const void* gate, void* dys,
+                        void* dgate, long rmax, int d, int topk, void* stream);
+
+/* dlogits fp32 [N][E] from dgate through the renormalisation and the softmax; dh bf16 [N][d] = dxs[slot_1] + dxs[slot_2] +
+ * dlogits Wr; dwr fp32 [E][d] (+)= dlogits^T h.
+ * Replaces MoeDispatch2.backward (round2/source/train.py:10662-10666) and autograd through moe_route / the router matmul. */
+int tfb_moe_route_bwd(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot, const void* h,
+                      const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate, long N, int d, int E, int topk,
+                      void* stream);
+
+/* rows_out fp32 [E][16] = rows_in with the backward columns filled from each expert's amax over its rows of dys
+ * (backward_scales per expert, round2/source/kernels/nki_mlp_fused8.py:803-813). amax_scratch: uint32 [E]. */
+int tfb_moe_backward_scales(const void* dys, const void* tile_expert, const void* rows_in, void* rows_out, void* amax_scratch,
+                            long rmax, int d, int E, void* stream);
+
+/* out8 = fp8(x * rows[expert of the row's tile][col]); fmt 0 e4m3, 1 e5m2; padding tiles give zero bytes. */
+int tfb_moe_quant(const void* x, const void* tile_expert, const void* rows, int col, int fmt, void* out8, long rmax, int d,
+                  void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,98 @@
+"""Mixture-of-experts oracle: router, top-k, dropless dispatch, per-expert fp8 MLPs, gated combine.
+
+Restates R2:10505-10553 (moe_tournament: first maximum, ties low; moe_route: fp32 softmax of the router logits, top-2
+gates renormalised v1 / (v1 + v2), top-1 gate = the probability), R2:10961 (logits = F.linear(h.float(), router.float())),
+R2:10652-10688 (dispatch / combine as gathers), R2:10753-10776 (moe_experts8_local: one fp8 MLP per expert with the expert's
+own scale row, rows padded with zeros to a multiple of 128) and R2:10990-10992 (out = g1.to(dt) * y1 + g2.to(dt) * y2 in the
+activations' dtype). The reference places assignments in per-sequence capacity slots and drops the overflow; with a capacity
+that drops nothing its output is this function, because a zero padding row yields a zero output row and touches no other
+row (R2:10735-10737). Gradients come from torch.autograd over these expressions with the fp8 MLP's own backward
+(oracle.mlp8), as EmulatedFusedMlp8 does.
+
+Pinned by (tests/test_oracle_moe.py): torch.topk for the selections, gates summing to one, a brute-force per-token loop
+with the bf16 expert MLP, permutation equivariance over tokens, and the reference's capacity layout computed with a cumsum
+giving the same output when nothing is dropped.
+"""
+import torch
+import torch.nn.functional as F
+
+from . import mlp8 as omlp
+
+
+def route(h2, router, topk, bias=None):
+    """(p [N, E] fp32, idx [N, k] int64, gate [N, k] fp32, logits)."""
+    logits = F.linear(h2.float(), router.float())
+    if bias is not None:
+        logits = logits + bias.float()
+    p = torch.softmax(logits, dim=-1)
+    i1 = torch.argmax(p, dim=-1)                      # first maximum: ties go to the lower index
+    v1 = p.gather(1, i1[:, None]).squeeze(1)
+    if topk == 1:
+        return p, i1[:, None], v1[:, None], logits
+    masked = p.masked_fill(F.one_hot(i1, p.shape[1]).bool(), -1.0)
+    i2 = torch.argmax(masked, dim=-1)
+    v2 = p.gather(1, i2[:, None]).squeeze(1)
+    den = v1 + v2
+    return p, torch.stack([i1, i2], 1), torch.stack([v1 / den, v2 / den], 1), logits
+
+
+def tables(idx, E):
+    """Dropless ragged layout: expert e's assignments contiguous in token order, segments padded to 128 rows.
+    Returns (slot [N, k] int64, tok [R] int64 (-1 padding), seg [E+1])."""
+    N, k = idx.shape
+    flat_e = idx.reshape(-1)
+    cnt = torch.bincount(flat_e, minlength=E)
+    pad = (cnt + 127) // 128 * 128
+    seg = torch.zeros(E + 1, dtype=torch.long)
+    seg[1:] = torch.cumsum(pad, 0)
+    onehot = F.one_hot(flat_e, E).reshape(N, k, E).sum(1)             # assignments per token per expert (0/1)
+    before = torch.cumsum(onehot, 0) - onehot                         # from earlier tokens
+    pos = before.gather(1, idx)
+    slot = seg[idx] + pos
+    tok = torch.full((int(seg[-1]),), -1, dtype=torch.long)
+    for j in range(k):
+        tok[slot[:, j]] = torch.arange(N)
+    return slot, tok, seg
+
+
+class _ExpertMlp8(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x2, w_fc, w_proj, row, x_scale):
+        y, r = omlp.forward(x2, w_fc, w_proj, row, x_scale)
+        ctx.save_for_backward(x2, r, w_fc, w_proj, row)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2, r, w_fc, w_proj, row = ctx.saved_tensors
+        dy = dy.contiguous()
+        dx, h, dpre = omlp.backward(dy, r, w_fc, w_proj, omlp.backward_scales(dy, row))
+        dw_fc, dw_proj = omlp.weight_grads(dy, x2, h, dpre)
+        return dx, dw_fc, dw_proj, None, None
+
+
+def moe_forward(h, router, w_fc, w_proj, topk, bias=None, fp8=True, e4m3_limit=240.0, x_scale=4.0):
+    """h [.., d] bf16; router [E, d]; w_fc [E, F, d]; w_proj [E, d, F]. Differentiable (autograd) in h, router, weights."""
+    d = h.shape[-1]
+    h2 = h.reshape(-1, d)
+    E = w_fc.shape[0]
+    p, idx, gate, _ = route(h2, router, topk, bias)
+    slot, tok, seg = tables(idx, E)
+    pad = torch.cat([h2, h2.new_zeros(1, d)], 0)
+    xs = pad.index_select(0, torch.where(tok >= 0, tok, torch.full_like(tok, h2.shape[0])))
+    outs = []
+    for e in range(E):
+        xe = xs[seg[e]:seg[e + 1]]
+        if xe.shape[0] == 0:
+            continue
+        if fp8:
+            row = omlp.forward_scales(w_fc[e].detach(), w_proj[e].detach(), e4m3_limit, x_scale)
+            outs.append(_ExpertMlp8.apply(xe, w_fc[e], w_proj[e], row, x_scale))
+        else:
+            outs.append(F.linear(torch.relu(F.linear(xe, w_fc[e])).square(), w_proj[e]))
+    ys = torch.cat(outs, 0)
+    dt = ys.dtype
+    out = gate[:, 0].to(dt).unsqueeze(-1) * ys.index_select(0, slot[:, 0])
+    if topk == 2:
+        out = out + gate[:, 1].to(dt).unsqueeze(-1) * ys.index_select(0, slot[:, 1])
+    return out.reshape(h.shape), {"p": p, "idx": idx, "gate": gate, "slot": slot, "tok": tok, "seg": seg}

@@ -1,0 +1,94 @@
+"""MoE layer on the HIP kernels against the oracle (BASELINE config 5 shapes in the last test)."""
+import pytest
+import torch
+
+from helpers import rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def _layer(seed, N, d, Fd, E, skew=0.0):
+    g = torch.Generator().manual_seed(seed)
+    h = torch.randn(N, d, generator=g).bfloat16()
+    router = 0.02 * torch.randn(E, d, generator=g) * 8
+    wf = (0.02 * torch.randn(E, Fd, d, generator=g)).bfloat16()
+    wp = (0.02 * torch.randn(E, d, Fd, generator=g)).bfloat16()
+    bias = torch.zeros(E)
+    bias[:2] = skew
+    return h, router, wf, wp, bias
+
+
+@pytest.mark.parametrize("topk", [2, 1])
+@pytest.mark.parametrize("skew", [0.0, 2.0])
+def test_routing_tables_bit_exact(dev, topk, skew):
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import ops
+    h, router, _, _, bias = _layer(1, 2048 + 64, 256, 512, 8, skew)
+    p, idx, gate, logits = ops.moe_route(h.to(dev), router.to(dev), topk, bias.to(dev), want_logits=True)
+    po, io, go, lo = O.route(h, router, topk, bias)
+    assert rel_l2(logits, lo) < 1e-5 and rel_l2(p, po) < 1e-5 and rel_l2(gate, go) < 1e-5
+    agree = (idx.cpu().long() == io).all(1)
+    assert agree.float().mean().item() > 0.999           # only exact near-ties may pick differently
+    tab = ops.moe_tables(idx, 8)
+    slot, tok, seg = O.tables(idx.cpu().long(), 8)       # oracle tables from the kernel's own selections
+    assert torch.equal(tab["seg"].cpu().long(), seg)
+    assert torch.equal(tab["slot"].cpu().long(), slot)
+    R = int(seg[-1])
+    assert torch.equal(tab["tok"].cpu().long()[:R], tok)
+    te = tab["tile_expert"].cpu()
+    for e in range(8):
+        assert bool((te[int(seg[e]) // 128:int(seg[e + 1]) // 128] == e).all())
+    assert bool((te[R // 128:] == -1).all())
+
+
+@pytest.mark.parametrize("shape,topk,skew", [((1024, 256, 512, 8), 2, 0.0), ((1024, 256, 512, 4), 1, 0.0),
+                                              ((2048, 512, 768, 8), 2, 2.0)])
+def test_moe_layer_forward_backward(dev, shape, topk, skew):
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import autograd as A
+    N, d, Fd, E = shape
+    h, router, wf, wp, bias = _layer(2, N, d, Fd, E, skew)
+    hd = h.to(dev).requires_grad_(True)
+    rd = router.to(dev).requires_grad_(True)
+    wfd = wf.to(dev).requires_grad_(True)
+    wpd = wp.to(dev).requires_grad_(True)
+    st = A.Moe8State()
+    st.refresh(wfd, wpd)
+    out = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, st, topk, bias.to(dev) if skew else None)
+    g = torch.randn(N, d, generator=torch.Generator().manual_seed(3)).bfloat16()
+    out.backward(g.to(dev))
+    ho, ro, wfo, wpo = (t.clone().requires_grad_(True) for t in (h, router, wf, wp))
+    oo, aux = O.moe_forward(ho, ro, wfo, wpo, topk, bias if skew else None)
+    oo.backward(g)
+    assert rel_l2(out, oo) < 2e-2
+    assert rel_l2(hd.grad, ho.grad) < 2e-2
+    assert rel_l2(wfd.grad, wfo.grad) < 2e-2 and rel_l2(wpd.grad, wpo.grad) < 2e-2
+    assert rel_l2(rd.grad, ro.grad) < 2e-2
+
+
+def test_moe_config5_full_size(dev):
+    """16384 tokens, d 1024, 8 experts top-2, FFN 2816: balanced and skewed routing; a token slice against the oracle,
+    exact equivariance under a token permutation, and load accounting."""
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import autograd as A
+    from trainium_frontier_them_bones_amd import ops
+    N, d, Fd, E = 16384, 1024, 2816, 8
+    for skew in (0.0, 2.0):
+        h, router, wf, wp, bias = _layer(5, N, d, Fd, E, skew)
+        hd, rd, wfd, wpd = (t.to(dev) for t in (h, router, wf, wp))
+        st = A.Moe8State()
+        st.refresh(wfd, wpd)
+        b = bias.to(dev) if skew else None
+        out = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, st, 2, b)
+        p, idx, gate, _ = ops.moe_route(hd, rd, 2, b)
+        tab = ops.moe_tables(idx, E)
+        assert int(tab["cnt"].sum()) == 2 * N
+        if skew:
+            assert int(tab["cnt"][:2].min()) > 1.3 * int(tab["cnt"][2:].max())     # the biased experts are hot
+        perm = torch.randperm(N, generator=torch.Generator().manual_seed(7)).to(dev)
+        out_p = A.MoeMlp8Fn.apply(hd[perm].contiguous(), rd, wfd, wpd, st, 2, b)
+        assert torch.equal(out_p, out[perm])
+        # oracle on the tokens of one expert pair: run the oracle's experts on this slice with the layer's scale rows
+        sl = slice(0, 512)
+        oo, _ = O.moe_forward(h[sl], router, wf, wp, 2, bias if skew else None)
+        assert rel_l2(out[sl], oo) < 2e-2

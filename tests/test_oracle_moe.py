@@ -1,0 +1,104 @@
+"""Pins oracle/moe.py: torch.topk, a brute-force per-token loop, invariants, and the reference's capacity layout."""
+import torch
+import torch.nn.functional as F
+
+from oracle import moe as O
+from helpers import rel_l2
+
+
+def _layer(seed, N=384, d=128, Fd=256, E=8):
+    g = torch.Generator().manual_seed(seed)
+    h = torch.randn(N, d, generator=g).bfloat16()
+    router = 0.5 * torch.randn(E, d, generator=g)
+    wf = (0.05 * torch.randn(E, Fd, d, generator=g)).bfloat16()
+    wp = (0.05 * torch.randn(E, d, Fd, generator=g)).bfloat16()
+    return h, router, wf, wp
+
+
+def test_route_matches_topk_and_gates_sum_to_one():
+    h, router, _, _ = _layer(0)
+    p, idx, gate, logits = O.route(h, router, 2)
+    tv, ti = torch.topk(p, 2, dim=-1)
+    assert torch.equal(idx, ti)
+    assert torch.allclose(gate.sum(-1), torch.ones(h.shape[0]), atol=1e-6)
+    assert torch.allclose(gate[:, 0], tv[:, 0] / tv.sum(-1))
+    p1, idx1, gate1, _ = O.route(h, router, 1)
+    assert torch.equal(idx1[:, 0], p.argmax(-1)) and torch.equal(gate1[:, 0], p.max(-1).values)
+    tie = torch.zeros(4, 8)
+    assert O.route(torch.zeros(4, 16).bfloat16(), torch.zeros(8, 16), 2)[1].tolist() == [[0, 1]] * 4    # ties go low
+    bias = torch.zeros(8)
+    bias[5] = 50.0
+    assert bool((O.route(h, router, 2, bias)[1][:, 0] == 5).all())
+
+
+def test_tables_are_a_stable_padded_partition():
+    h, router, _, _ = _layer(1)
+    _, idx, _, _ = O.route(h, router, 2)
+    slot, tok, seg = O.tables(idx, 8)
+    assert bool((seg % 128 == 0).all()) and int(seg[-1]) == tok.numel()
+    assert int((tok >= 0).sum()) == idx.numel() and slot.unique().numel() == idx.numel()
+    for e in range(8):
+        rows = tok[seg[e]:seg[e + 1]]
+        live = rows[rows >= 0]
+        assert bool((live[1:] > live[:-1]).all())                       # token order inside an expert
+        assert bool(((idx[live] == e).any(1)).all())
+        assert bool((rows[live.numel():] == -1).all())                  # padding at the end of the segment
+
+
+def test_forward_matches_brute_force_bf16_experts():
+    h, router, wf, wp = _layer(2, N=128)
+    out, aux = O.moe_forward(h, router, wf, wp, 2, fp8=False)
+    ref = torch.zeros(128, 128)
+    for n in range(128):
+        acc = None
+        for j in range(2):
+            e = int(aux["idx"][n, j])
+            y = F.linear(torch.relu(F.linear(h[n:n + 1], wf[e])).square(), wp[e])
+            term = aux["gate"][n, j].to(torch.bfloat16) * y
+            acc = term if acc is None else acc + term
+        ref[n] = acc.float()
+    assert rel_l2(out, ref) < 1e-2
+
+
+def test_token_permutation_equivariance_and_fp8_budget():
+    h, router, wf, wp = _layer(3)
+    out, _ = O.moe_forward(h, router, wf, wp, 2)
+    perm = torch.randperm(h.shape[0], generator=torch.Generator().manual_seed(1))
+    out_p, _ = O.moe_forward(h[perm], router, wf, wp, 2)
+    assert rel_l2(out_p, out[perm]) < 1e-6
+    out16, _ = O.moe_forward(h, router, wf, wp, 2, fp8=False)
+    assert rel_l2(out, out16) < 0.15
+
+
+def test_reference_capacity_layout_gives_same_output_when_nothing_drops():
+    """The reference's slots: [E][b][cap] with the position = earlier assignments to e in the same sequence (R2:10555-10600).
+    With cap = t nothing is dropped and its gather/combine gives the dropless output."""
+    h, router, wf, wp = _layer(4, N=256)
+    b, t, E = 2, 128, 8
+    _, idx, gate, _ = O.route(h, router, 2)
+    mall = F.one_hot(idx, E).sum(1).reshape(b, t, E)
+    excl = torch.cumsum(mall, 1) - mall
+    cap = t
+    row = torch.arange(b).repeat_interleave(t)
+    pos = excl.reshape(b * t, E).gather(1, idx)
+    slot = (idx * b + row[:, None]) * cap + pos
+    xs = torch.zeros(E * b * cap, h.shape[1], dtype=h.dtype)
+    for j in range(2):
+        xs[slot[:, j]] = h
+    ys = torch.stack([F.linear(torch.relu(F.linear(xs.reshape(E, b * cap, -1)[e], wf[e])).square(), wp[e]) for e in range(E)])
+    ys = ys.reshape(E * b * cap, -1)
+    out = gate[:, 0].bfloat16()[:, None] * ys[slot[:, 0]] + gate[:, 1].bfloat16()[:, None] * ys[slot[:, 1]]
+    ref, _ = O.moe_forward(h, router, wf, wp, 2, fp8=False)
+    assert torch.equal(out, ref)
+
+
+def test_backward_is_consistent_with_plain_autograd():
+    h, router, wf, wp = _layer(5, N=128)
+    hs = [h.clone().requires_grad_(True) for _ in range(2)]
+    rs = [router.clone().requires_grad_(True) for _ in range(2)]
+    g = torch.randn(128, 128, generator=torch.Generator().manual_seed(2)).bfloat16()
+    o8, _ = O.moe_forward(hs[0], rs[0], wf, wp, 2, fp8=True)
+    o16, _ = O.moe_forward(hs[1], rs[1], wf, wp, 2, fp8=False)
+    o8.backward(g)
+    o16.backward(g)
+    assert rel_l2(hs[0].grad, hs[1].grad) < 0.2 and rel_l2(rs[0].grad, rs[1].grad) < 0.2

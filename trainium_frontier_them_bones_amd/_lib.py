@@ -45,10 +45,22 @@ SIGNATURES = {
     "tfb_loss_fwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_loss_bwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_lmhead_fwd": [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _f, _vp],
+    "tfb_moe_max_rows": [_l, _i, _i],
+    "tfb_moe_route": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _i, _vp],
+    "tfb_moe_tables": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _l, _vp],
+    "tfb_moe_gather": [_vp, _vp, _vp, _f, _vp, _vp, _l, _i, _vp],
+    "tfb_moe_mlp8_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_moe_mlp8_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_moe_dw": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "tfb_moe_combine": [_vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_moe_combine_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_moe_route_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _l, _i, _i, _i, _vp],
+    "tfb_moe_backward_scales": [_vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_moe_quant": [_vp, _vp, _vp, _i, _i, _vp, _l, _i, _vp],
     "tfb_mlp_dw_proj": [_vp, _vp, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
 }
 
-_LONG_RESULT = {"tfb_mlp8_scale_scratch_floats"}
+_LONG_RESULT = {"tfb_mlp8_scale_scratch_floats", "tfb_moe_max_rows"}
 
 STATUS = {0: "ok", 1: "unsupported shape", 2: "bad argument", 3: "kernel launch failed", 4: "workspace too small"}
 

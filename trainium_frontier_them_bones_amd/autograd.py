@@ -290,3 +290,59 @@ class Relu2Fn(torch.autograd.Function):
 
 def default_scale(D):
     return 1.0 / math.sqrt(D)
+
+
+class Moe8State:
+    """Per-layer fp8 state of the experts, refreshed once per optimizer step: a scale row and an e4m3 weight pack per
+    expert (the reference's exp8_sc [E,128,16] / exp8_w8 buffers, round2/source/train.py:10900-10935)."""
+
+    def __init__(self, e4m3_limit=240.0, x_scale=4.0):
+        self.e4m3_limit, self.x_scale = e4m3_limit, x_scale
+        self.rows = None
+        self.w8 = None
+
+    def refresh(self, w_fc, w_proj):
+        E, F, d = w_fc.shape
+        rows = [ops.mlp8_forward_scales(w_fc[e].detach(), w_proj[e].detach(), self.e4m3_limit, self.x_scale) for e in range(E)]
+        self.rows = torch.stack(rows).contiguous()
+        self.w8 = torch.stack([ops.mlp8_precast(w_fc[e].detach(), w_proj[e].detach(), rows[e]) for e in range(E)]).contiguous()
+
+
+class MoeMlp8Fn(torch.autograd.Function):
+    """The routed half of MoeMLP.forward_e8 (round2/source/train.py:11003-11067) with every expert on this GPU:
+    router -> top-k -> dropless dispatch -> grouped fp8 expert MLPs -> gated combine. h [.., d] bf16, router fp32 [E, d],
+    w_fc [E, F, d], w_proj [E, d, F] bf16; router_bias fp32 [E] or None (added to the logits)."""
+
+    @staticmethod
+    def forward(ctx, h, router, w_fc, w_proj, state, topk, router_bias):
+        h2 = h.reshape(-1, h.shape[-1]).contiguous()
+        E, F, d = w_fc.shape
+        wr = router.detach().float().contiguous()
+        p, idx, gate, _ = ops.moe_route(h2, wr, topk, router_bias)
+        tab = ops.moe_tables(idx, E)
+        xs, xs8 = ops.moe_gather(h2, tab, state.x_scale)
+        ys, r = ops.moe_mlp8_fwd(xs8, state.w8, state.rows, tab, F)
+        out = ops.moe_combine(ys, tab, gate, h2.shape[0])
+        ctx.save_for_backward(h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj)
+        ctx.tab, ctx.state, ctx.hshape = tab, state, h.shape
+        return out.view(h.shape)
+
+    @staticmethod
+    def backward(ctx, gout):
+        h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj = ctx.saved_tensors
+        tab, st = ctx.tab, ctx.state
+        E = w_fc.shape[0]
+        g2 = gout.reshape(-1, gout.shape[-1]).contiguous()
+        dys, dgate = ops.moe_combine_bwd(g2, ys, tab, gate)
+        rows_b = ops.moe_backward_scales(dys, st.rows, tab)
+        dxs, dpre = ops.moe_mlp8_bwd(dys, r, st.w8, rows_b, tab)
+        bf, accf = _accumulate_into(w_fc)
+        bp, accp = _accumulate_into(w_proj)
+        if bf is not None and bp is not None:
+            ops.moe_dw(dpre, xs, dys, r, tab, E, bf, bp, accumulate=accf)
+            dw_fc = dw_proj = None
+        else:
+            dw_fc, dw_proj = ops.moe_dw(dpre, xs, dys, r, tab, E)
+        br, accr = _accumulate_into(router)
+        dh, dwr, _ = ops.moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, br, accr)
+        return dh.view(ctx.hshape), (None if br is not None else dwr.to(router.dtype)), dw_fc, dw_proj, None, None, None

@@ -72,7 +72,10 @@ struct MicroBlock {
 
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
-constexpr int TROW = 64 * 2 + 16;  // LDS row of a transposed tile: 64 tokens + pad
+// LDS row of a transposed tile: 64 tokens + 8 bytes of pad. With 32 banks and 64-bit accesses resolved per 16 lanes,
+// a 136-byte stride puts the 16 rows a half-wavefront's fragment read touches on 16 different bank pairs, and the
+// transposing writes (16 consecutive lanes along the tokens of one row) are conflict-free as well.
+constexpr int TROW = 64 * 2 + 8;
 
 // =========================================================================================== forward
 template <int D>

@@ -1,18 +1,22 @@
 // MFMA GEMM core for gfx950: D[p][q] = sum_k P[p][k] * Q[q][k], fp32 accumulation.
 //
 // One workgroup of WP x WQ wavefronts owns a BP x BQ output tile. Both operand tiles are
-// staged in LDS as [row][128 bytes of k], the eight 16-byte chunks of a row XOR-swizzled by
-// a function of the row so that 128-bit fragment reads, 128-bit row writes and the 64-bit
-// transposing writes are all free of bank conflicts. Staging is double-buffered (NBUF 2: the
+// staged in LDS as [row][128 bytes of k + 16 bytes of pad], the eight 16-byte chunks of a row
+// XOR-swizzled by (row / 8) mod 8. With the measured bank behaviour of gfx950's LDS (32 banks
+// of 4 bytes; 128-bit accesses resolved per 8 consecutive lanes, 64-bit accesses per 16) the
+// 144-byte stride makes the 128-bit fragment reads (8 consecutive rows, one chunk) conflict-free,
+// and the swizzle does the same for the 64-bit transposing writes (8 rows that are 8 apart times
+// two adjacent k-groups per 16 lanes) while global loads stay 128-byte coalesced. Staging is
+// double-buffered (NBUF 2: the
 // next k-tile's global loads are in flight while the MFMAs of the current one run, one barrier
 // per k-tile) or single-buffered (NBUF 1: half the LDS, two barriers, more workgroups per CU).
 // The P tile feeds the MFMA A operand (rows), the Q tile the B operand (columns), so a lane
 // ends up holding D[p .. p+3][q] for four consecutive p: callers put the dimension that is
 // contiguous in the output on the P side.
 //
-// Epilogues: "staged" (default) - the accumulators go through LDS once and every thread then
-// owns 8 consecutive p of one q, so global reads/writes of the epilogue are 128-bit and
-// coalesced along the output rows; or "tile" (kTileEpilogue) - the functor gets the raw
+// Epilogues: "staged" (default) - each wavefront passes its accumulators through its own LDS
+// slice, 32 output rows at a time, and every lane then owns 8 consecutive p of one q, so global
+// reads/writes of the epilogue are 128-bit and coalesced along the output rows; or "tile" (kTileEpilogue) - the functor gets the raw
 // accumulator registers (used when the epilogue reduces along p in registers).
 //
 // Element types: bf16 (v_mfma_f32_32x32x16_bf16, 64 k per tile) or OCP fp8
@@ -27,7 +31,7 @@
 
 #define TFB_K_CONTIG 0
 #define TFB_K_STRIDED 1
-#define TFB_LDS_ROW 128
+#define TFB_LDS_ROW 144  // 128 bytes of k + 16 bytes of pad
 
 struct GemmOperand {
   const uint8_t* base;
@@ -39,16 +43,19 @@ struct GemmArgs {
   int np, nq;   // output extent (multiples of BP / BQ)
   int nkt;      // k-tiles (128 bytes of k each) per split
   int ntp;      // tiles along p
+  // Grouped (ragged) launches, both optional:
+  const int* q_group;    // group id of each q tile (-1: the tile is beyond the ragged extent, the workgroup exits);
+  long p_group_stride;   //   the P operand of group g starts p_group_stride bytes * g further (per-expert weights)
+  const int* k_seg;      // [groups + 1] k offsets in elements: group = blockIdx.y contracts over k_seg[g] .. k_seg[g+1]
 };
 
 struct LoadIdentity {
   __device__ __forceinline__ u32x4 operator()(u32x4 v) const { return v; }
 };
 
-// Byte offset of 16-byte chunk `chunk` of row `row` in a swizzled tile. Over any 8 consecutive rows, and over the 8
-// same-parity rows of any aligned 16, the swizzle takes 8 distinct values.
+// Byte offset of 16-byte chunk `chunk` of row `row` in a staged tile.
 __device__ __forceinline__ int lds_off(int row, int chunk) {
-  return row * TFB_LDS_ROW + (((chunk ^ (row + (row >> 3))) & 7) << 4);
+  return row * TFB_LDS_ROW + (((chunk ^ (row >> 3)) & 7) << 4);
 }
 
 template <int BP_, int BQ_, int WP_, int WQ_, int ES_, int LAYP_, int LAYQ_, int FMTP_ = 0, int FMTQ_ = 0, int NBUF_ = 2>
@@ -59,14 +66,13 @@ struct GemmCfg {
   static constexpr int TP = BP / WP / 32, TQ = BQ / WQ / 32;
   static constexpr int BK = 128 / ES;  // elements of k per tile
   static constexpr int TILE_BYTES = (BP + BQ) * TFB_LDS_ROW;
-  static constexpr int STAGE_LD = BP + 4;  // floats per staged output row
-  static constexpr int STAGE_BYTES = BQ * STAGE_LD * 4;
+  static constexpr int STAGE_LD = TP * 32 + 4;  // floats per staged row: a wavefront's 32 x (TP*32) slice
+  static constexpr int STAGE_BYTES = WP * WQ * 32 * STAGE_LD * 4;
   static constexpr int LDS_BYTES = NBUF * TILE_BYTES > STAGE_BYTES ? NBUF * TILE_BYTES : STAGE_BYTES;
   static_assert(ES == 1 || ES == 2, "fp8 or bf16");
   static_assert(NBUF == 1 || NBUF == 2, "single or double buffering");
   static_assert(ES == 2 || (LAYP == TFB_K_CONTIG && LAYQ == TFB_K_CONTIG), "fp8 operands are k-contiguous");
   static_assert((BP * 8) % NT == 0 && (BQ * 8) % NT == 0, "tile rows vs threads");
-  static_assert((BQ * BP / 8) % NT == 0, "staged epilogue chunks vs threads");
 };
 
 // ---- global -> register -> LDS staging of one operand tile ---------------------------------
@@ -100,14 +106,16 @@ template <int ROWS, int NT>
 struct TileLoader<ROWS, NT, TFB_K_STRIDED> {
   // bf16 only: 64 k x ROWS tile, micro-blocks of 4 k x 8 rows
   static constexpr int N = ROWS * 2 / NT;
-  static_assert((ROWS * 2) % NT == 0 && N >= 1, "K_STRIDED tile rows vs threads");
+  static_assert((ROWS * 2) % NT == 0 && N >= 1 && ROWS % 64 == 0, "K_STRIDED tile rows vs threads");
   u32x4 g[N][4];
   __device__ __forceinline__ void load(const GemmOperand& o, long row0, long kbyte0, int tid) {
     const long k0 = kbyte0 >> 1;
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       int mb = tid + i * NT;
-      int rg = mb % (ROWS / 8), kg = mb / (ROWS / 8);
+      // 16 consecutive lanes = 8 row groups x 2 adjacent k groups: 128-byte coalesced loads, conflict-free writes
+      int hi = mb >> 4;
+      int rg = (mb & 7) + 8 * (hi % (ROWS / 64)), kg = ((mb >> 3) & 1) + 2 * (hi / (ROWS / 64));
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         g[i][j] = *(const u32x4*)(o.base + (k0 + 4 * kg + j) * o.ld + (row0 + 8 * rg) * 2);
@@ -118,7 +126,8 @@ struct TileLoader<ROWS, NT, TFB_K_STRIDED> {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       int mb = tid + i * NT;
-      int rg = mb % (ROWS / 8), kg = mb / (ROWS / 8);
+      int hi = mb >> 4;
+      int rg = (mb & 7) + 8 * (hi % (ROWS / 64)), kg = ((mb >> 3) & 1) + 2 * (hi / (ROWS / 64));
       u32x4 v0 = pre(g[i][0]), v1 = pre(g[i][1]), v2 = pre(g[i][2]), v3 = pre(g[i][3]);
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
@@ -176,6 +185,17 @@ __device__ __forceinline__ int xcd_remap(int pid, int nb) {
 }
 
 template <class T, class = void>
+struct has_for_group : std::false_type {};
+template <class T>
+struct has_for_group<T, std::void_t<decltype(std::declval<const T&>().for_group(0))>> : std::true_type {};
+// An epilogue with per-group state (scale row, output slab) provides  Epi for_group(int g) const.
+template <class Epi>
+__device__ __forceinline__ Epi epi_for_group(const Epi& e, int g) {
+  if constexpr (has_for_group<Epi>::value) return e.for_group(g);
+  else return e;
+}
+
+template <class T, class = void>
 struct has_tile_epilogue : std::false_type {};
 template <class T>
 struct has_tile_epilogue<T, std::void_t<decltype(T::kTileEpilogue)>> : std::true_type {};
@@ -183,7 +203,7 @@ struct has_tile_epilogue<T, std::void_t<decltype(T::kTileEpilogue)>> : std::true
 // Epi: either  __device__ void operator()(int p, int q, const float (&v)[8], int split)  with v = D[p..p+7][q], p % 8 == 0,
 // or (with a static member kTileEpilogue)  __device__ void tile(acc, pw, qw, lr, lh, tile_id, split).
 template <class Cfg, class PreP, class PreQ, class Epi>
-__global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, PreQ preq, Epi epi) {
+__global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, PreQ preq, Epi epi_in) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   constexpr int BP = Cfg::BP, BQ = Cfg::BQ, NT = Cfg::NT, TP = Cfg::TP, TQ = Cfg::TQ, ES = Cfg::ES;
   constexpr int BUF = Cfg::TILE_BYTES;
@@ -195,7 +215,20 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, Pr
   const int lid = xcd_remap(blockIdx.x, gridDim.x);
   const int tile_p = lid % a.ntp, tile_q = lid / a.ntp;
   const long p0 = (long)tile_p * BP, q0 = (long)tile_q * BQ;
-  const long kt0 = (long)blockIdx.z * a.nkt;
+  long kt0 = (long)blockIdx.z * a.nkt;
+  int group = 0;
+  if (a.q_group) {
+    group = a.q_group[tile_q];
+    if (group < 0) return;  // the whole workgroup leaves before any barrier
+    a.P.base += (long)group * a.p_group_stride;
+  }
+  if (a.k_seg) {
+    group = blockIdx.y;
+    const long k0 = a.k_seg[group], k1 = a.k_seg[group + 1];
+    kt0 = k0 * ES / 128;
+    a.nkt = (int)((k1 - k0) * ES / 128);  // may be 0: the accumulators stay zero and are still written
+  }
+  const Epi epi = epi_for_group(epi_in, group);
 
   TileLoader<BP, NT, Cfg::LAYP> lp;
   TileLoader<BQ, NT, Cfg::LAYQ> lq;
@@ -208,10 +241,12 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, Pr
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  lp.load(a.P, p0, kt0 * 128, tid);
-  lq.load(a.Q, q0, kt0 * 128, tid);
-  lp.store(smem, tid, prep);
-  lq.store(smem + BP * TFB_LDS_ROW, tid, preq);
+  if (a.nkt > 0) {
+    lp.load(a.P, p0, kt0 * 128, tid);
+    lq.load(a.Q, q0, kt0 * 128, tid);
+    lp.store(smem, tid, prep);
+    lq.store(smem + BP * TFB_LDS_ROW, tid, preq);
+  }
   __syncthreads();
 
   for (int t = 0; t < a.nkt; ++t) {
@@ -222,17 +257,28 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, Pr
       lp.load(a.P, p0, (kt0 + t + 1) * 128, tid);
       lq.load(a.Q, q0, (kt0 + t + 1) * 128, tid);
     }
+    {
+      // fragments of k-step s+1 are requested before the MFMAs of step s are issued
+      constexpr int KS = Frag<ES>::KSTEPS;
+      Frag<ES> fa[2][TP], fb[2][TQ];
 #pragma unroll
-    for (int s = 0; s < Frag<ES>::KSTEPS; ++s) {
-      Frag<ES> fa[TP], fb[TQ];
+      for (int i = 0; i < TP; ++i) fa[0][i].read(sp, wp * (TP * 32) + i * 32 + lr, 0, lh);
 #pragma unroll
-      for (int i = 0; i < TP; ++i) fa[i].read(sp, wp * (TP * 32) + i * 32 + lr, s, lh);
+      for (int j = 0; j < TQ; ++j) fb[0][j].read(sq, wq * (TQ * 32) + j * 32 + lr, 0, lh);
 #pragma unroll
-      for (int j = 0; j < TQ; ++j) fb[j].read(sq, wq * (TQ * 32) + j * 32 + lr, s, lh);
+      for (int s = 0; s < KS; ++s) {
+        if (s + 1 < KS) {
 #pragma unroll
-      for (int i = 0; i < TP; ++i)
+          for (int i = 0; i < TP; ++i) fa[(s + 1) & 1][i].read(sp, wp * (TP * 32) + i * 32 + lr, s + 1, lh);
 #pragma unroll
-        for (int j = 0; j < TQ; ++j) acc[i][j] = mfma32<ES, Cfg::FMTP, Cfg::FMTQ>(fa[i], fb[j], acc[i][j]);
+          for (int j = 0; j < TQ; ++j) fb[(s + 1) & 1][j].read(sq, wq * (TQ * 32) + j * 32 + lr, s + 1, lh);
+        }
+#pragma unroll
+        for (int i = 0; i < TP; ++i)
+#pragma unroll
+          for (int j = 0; j < TQ; ++j)
+            acc[i][j] = mfma32<ES, Cfg::FMTP, Cfg::FMTQ>(fa[s & 1][i], fb[s & 1][j], acc[i][j]);
+      }
     }
     if (Cfg::NBUF == 1) __syncthreads();
     if (more) {
@@ -248,31 +294,40 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, Pr
     // whole-accumulator epilogue: acc[i][j][4*jj + e] = D[pw + 32 i + 8 jj + 4 lh + e][qw + 32 j + lr]
     epi.tile(acc, (int)p0 + pw, (int)q0 + qw, lr, lh, lid, (int)blockIdx.z);
   } else {
-    // (the loop's last barrier has passed: every wavefront is done reading the operand tiles)
-    float* stage = (float*)smem;
+    // (the loop's last barrier has passed: every wavefront is done reading the operand tiles.) Each wavefront stages
+    // 32 output rows at a time through its own LDS slice (no workgroup barrier: LDS operations of one wavefront
+    // execute in order) and then finishes them as 8-element chunks, a row's chunks on consecutive lanes.
     constexpr int SLD = Cfg::STAGE_LD;
+    float* stage = (float*)smem + wave * (32 * SLD);
+    constexpr int CPR = TP * 4;  // 8-element chunks per staged row
 #pragma unroll
-    for (int i = 0; i < TP; ++i)
+    for (int j = 0; j < TQ; ++j) {
 #pragma unroll
-      for (int j = 0; j < TQ; ++j)
+      for (int i = 0; i < TP; ++i)
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
           f32x4 v = {acc[i][j][jj * 4 + 0], acc[i][j][jj * 4 + 1], acc[i][j][jj * 4 + 2], acc[i][j][jj * 4 + 3]};
-          *(f32x4*)(stage + (qw + j * 32 + lr) * SLD + pw + i * 32 + jj * 8 + lh * 4) = v;
+          *(f32x4*)(stage + lr * SLD + i * 32 + jj * 8 + lh * 4) = v;
         }
-    __syncthreads();
-    constexpr int CPR = BP / 8;  // 8-element chunks per output row
+      __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int i = 0; i < BQ * CPR / NT; ++i) {
-      const int c = tid + i * NT;
-      const int q = c / CPR, pc = (c % CPR) * 8;
-      f32x4 lo = *(const f32x4*)(stage + q * SLD + pc);
-      f32x4 hi = *(const f32x4*)(stage + q * SLD + pc + 4);
-      const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      epi((int)p0 + pc, (int)q0 + q, v, (int)blockIdx.z);
+      for (int k = 0; k < 32 * CPR / 64; ++k) {
+        // 8 consecutive lanes take 4 chunks of each of two rows: their 128-bit reads fall on 8 different bank groups
+        const int rest = (lane >> 3) + k * 8;
+        const int row = 2 * (rest / (CPR / 4)) + ((lane >> 2) & 1);
+        const int pc = (4 * (rest % (CPR / 4)) + (lane & 3)) * 8;
+        f32x4 lo = *(const f32x4*)(stage + row * SLD + pc);
+        f32x4 hi = *(const f32x4*)(stage + row * SLD + pc + 4);
+        const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        epi((int)p0 + pw + pc, (int)q0 + qw + j * 32 + row, v, (int)blockIdx.z);
+      }
+      __builtin_amdgcn_wave_barrier();
     }
   }
 }
+
+template <class Cfg, class PreP, class PreQ, class Epi>
+static int gemm_launch_args(GemmArgs a, int groups_y, int splits, PreP prep, PreQ preq, Epi epi, hipStream_t stream);
 
 // Host-side launch: np, nq multiples of the tile; kbytes a multiple of 128 * splits.
 template <class Cfg, class PreP, class PreQ, class Epi>
@@ -287,6 +342,15 @@ static int gemm_launch(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes
   a.nq = nq;
   a.nkt = (int)(kbytes / 128 / splits);
   a.ntp = np / Cfg::BP;
+  a.q_group = nullptr;
+  a.p_group_stride = 0;
+  a.k_seg = nullptr;
+  return gemm_launch_args<Cfg>(a, 1, splits, prep, preq, epi, stream);
+}
+
+// Launch with prepared arguments; groups_y > 1 only with a.k_seg.
+template <class Cfg, class PreP, class PreQ, class Epi>
+static int gemm_launch_args(GemmArgs a, int groups_y, int splits, PreP prep, PreQ preq, Epi epi, hipStream_t stream) {
   auto kern = gemm_kernel<Cfg, PreP, PreQ, Epi>;
   static bool attr_set = false;  // per template instantiation
   if (!attr_set) {
@@ -294,7 +358,7 @@ static int gemm_launch(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes
       return TFB_ERR_LAUNCH;
     attr_set = true;
   }
-  dim3 grid(a.ntp * (nq / Cfg::BQ), 1, splits);
+  dim3 grid(a.ntp * (a.nq / Cfg::BQ), groups_y, splits);
   hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, a, prep, preq, epi);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
@@ -346,6 +410,18 @@ struct EpiStore {
       *(u32x4*)o = pack8bf(r);
     }
   }
+};
+
+// Per-group output slabs (grouped launches): group g writes out + g * slab elements.
+struct EpiStoreGrouped {
+  EpiStore base;
+  long slab;  // elements per group
+  __device__ __forceinline__ EpiStoreGrouped for_group(int g) const {
+    EpiStoreGrouped e = *this;
+    e.base.out = base.f32 ? (void*)((float*)base.out + (long)g * slab) : (void*)((bf16_t*)base.out + (long)g * slab);
+    return e;
+  }
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int s) const { base(p, q, v, s); }
 };
 
 // fp32 partial of one k-split: ws [splits][nq][ld]

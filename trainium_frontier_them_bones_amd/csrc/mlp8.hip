@@ -286,6 +286,11 @@ struct EpiUp {  // pre = x8 @ wf8^T: r, h8
   bf16_t* r;     // [M][F]
   uint8_t* h8;   // [M][F]
   long F;
+  __device__ __forceinline__ EpiUp for_group(int g) const {
+    EpiUp e = *this;
+    e.sc = sc + g * NSC;
+    return e;
+  }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
     const float dq = sc[SC_DQ_FC], c = sc[SC_C_H];
     float rr[8], hh[8];
@@ -307,6 +312,11 @@ struct EpiScaleStore {  // out = bf16(acc * sc[col])
   int col;
   bf16_t* out;
   long ld;
+  __device__ __forceinline__ EpiScaleStore for_group(int g) const {
+    EpiScaleStore e = *this;
+    e.sc = sc + g * NSC;
+    return e;
+  }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
     const float dq = sc[col];
     float r[8];
@@ -323,6 +333,11 @@ struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*
   uint8_t* dp8;     // [M][F]
   bf16_t* h;        // [M][F] or null
   long F;
+  __device__ __forceinline__ EpiDh for_group(int g) const {
+    EpiDh e = *this;
+    e.sc = sc + g * NSC;
+    return e;
+  }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
     const float dq = sc[SC_DQ_DH2], sdp = sc[SC_S_DP];
     const long off = (long)q * F + p;
@@ -513,4 +528,88 @@ extern "C" int tfb_mlp_dw_proj(const void* dy, const void* r, void* dw, long M, 
   int st = gemm_launch<Cfg>(P, Q, F, d, M * 2, splits, LoadSquare{}, LoadIdentity{}, e, s);
   if (st != TFB_OK) return st;
   return splitk_reduce((const float*)workspace, dw, (long)d * F, splits, out_f32, accumulate, s);
+}
+
+// ================================================================================================ grouped (MoE experts)
+// The experts' rows live in one token-major buffer, expert e's rows contiguous and padded to a multiple of 128 (padding
+// rows are zero), so every 128-row tile belongs to one expert: tile_expert[t] names it (-1 beyond the ragged extent).
+// Each expert has its own weight pack (w8 + e * 4 F d bytes) and scale row (rows + e * 16).
+// Replaces moe_experts8_local / moe_expert8_mlp (round2/source/train.py:10731-10776): one fp8 MLP call per expert there,
+// one grouped launch per GEMM here, with no host-side knowledge of the experts' loads.
+namespace {
+template <class Cfg, class Epi>
+int grouped_launch(const uint8_t* wbase, long wld, long wgroup_stride, const uint8_t* act, long ald, int np, long rmax, long kbytes,
+                   const int* tile_expert, Epi e, hipStream_t s) {
+  GemmArgs a;
+  a.P = GemmOperand{wbase, wld};
+  a.Q = GemmOperand{act, ald};
+  a.np = np;
+  a.nq = (int)rmax;
+  a.nkt = (int)(kbytes / 128);
+  a.ntp = np / Cfg::BP;
+  a.q_group = tile_expert;
+  a.p_group_stride = wgroup_stride;
+  a.k_seg = nullptr;
+  return gemm_launch_args<Cfg>(a, 1, 1, LoadIdentity{}, LoadIdentity{}, e, s);
+}
+}  // namespace
+
+extern "C" int tfb_moe_mlp8_fwd(const void* x8, const void* w8, const void* rows, const void* tile_expert, void* y, void* r,
+                                void* h8, long rmax, int d, int F, void* stream) {
+  if (!x8 || !w8 || !rows || !tile_expert || !y || !r || !h8) return TFB_ERR_ARG;
+  if (!shapes8(rmax, d, F)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const uint8_t* b = (const uint8_t*)w8;
+  const long n = (long)F * d;
+  EpiUp e1{(const float*)rows, (bf16_t*)r, (uint8_t*)h8, (long)F};
+  int st = grouped_launch<Cfg8>(b, d, 4 * n, (const uint8_t*)x8, d, F, rmax, d, (const int*)tile_expert, e1, s);
+  if (st != TFB_OK) return st;
+  EpiScaleStore e2{(const float*)rows, SC_DQ_PROJ, (bf16_t*)y, (long)d};
+  return grouped_launch<Cfg8>(b + 2 * n, F, 4 * n, (const uint8_t*)h8, F, d, rmax, F, (const int*)tile_expert, e2, s);
+}
+
+extern "C" int tfb_moe_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* rows, const void* tile_expert,
+                                void* dx, void* dpre, void* dp8, long rmax, int d, int F, void* stream) {
+  if (!dy8 || !r || !w8 || !rows || !tile_expert || !dx || !dpre || !dp8) return TFB_ERR_ARG;
+  if (!shapes8(rmax, d, F)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const uint8_t* b = (const uint8_t*)w8;
+  const long n = (long)F * d;
+  EpiDh e1{(const float*)rows, (const bf16_t*)r, (bf16_t*)dpre, (uint8_t*)dp8, nullptr, (long)F};
+  int st = grouped_launch<Cfg8g>(b + 3 * n, d, 4 * n, (const uint8_t*)dy8, d, F, rmax, d, (const int*)tile_expert, e1, s);
+  if (st != TFB_OK) return st;
+  EpiScaleStore e2{(const float*)rows, SC_DQ_DX, (bf16_t*)dx, (long)d};
+  return grouped_launch<Cfg8g>(b + n, F, 4 * n, (const uint8_t*)dp8, F, d, rmax, F, (const int*)tile_expert, e2, s);
+}
+
+// Per-expert weight gradients over the expert's row segment [seg[e], seg[e+1]) of the grouped buffers:
+// dw_fc [E][F][d] (+)= dpre_e^T @ xs_e; dw_proj [E][d][F] (+)= dys_e^T @ bf16(r_e^2). bf16 or fp32 outputs.
+extern "C" int tfb_moe_dw(const void* dpre, const void* xs, const void* dys, const void* r, const void* seg, void* dw_fc,
+                          void* dw_proj, int E, int d, int F, int out_f32, int accumulate, void* stream) {
+  if (!dpre || !xs || !dys || !r || !seg || !dw_fc || !dw_proj) return TFB_ERR_ARG;
+  if (E <= 0 || d % 128 || F % 128) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  using Cfg = GemmCfg<128, 128, 2, 2, 2, TFB_K_STRIDED, TFB_K_STRIDED>;
+  GemmArgs a;
+  a.q_group = nullptr;
+  a.p_group_stride = 0;
+  a.k_seg = (const int*)seg;
+  a.nkt = 0;
+  // dw_fc[e][f][j] = sum_m dpre[m][f] xs[m][j]: output contiguous in j (d) -> P = xs, Q = dpre
+  a.P = GemmOperand{(const uint8_t*)xs, (long)d * 2};
+  a.Q = GemmOperand{(const uint8_t*)dpre, (long)F * 2};
+  a.np = d;
+  a.nq = F;
+  a.ntp = d / 128;
+  EpiStoreGrouped e1{EpiStore{dw_fc, (long)d, out_f32, accumulate}, (long)F * d};
+  int st = gemm_launch_args<Cfg>(a, E, 1, LoadIdentity{}, LoadIdentity{}, e1, s);
+  if (st != TFB_OK) return st;
+  // dw_proj[e][j][f] = sum_m dys[m][j] r[m][f]^2: output contiguous in f -> P = r (squared while staged), Q = dys
+  a.P = GemmOperand{(const uint8_t*)r, (long)F * 2};
+  a.Q = GemmOperand{(const uint8_t*)dys, (long)d * 2};
+  a.np = F;
+  a.nq = d;
+  a.ntp = F / 128;
+  EpiStoreGrouped e2{EpiStore{dw_proj, (long)F, out_f32, accumulate}, (long)F * d};
+  return gemm_launch_args<Cfg>(a, E, 1, LoadSquare{}, LoadIdentity{}, e2, s);
 }

@@ -1,0 +1,594 @@
+// Mixture-of-experts routing, dispatch and combine for gfx950 (top-1 / top-2, experts local to the GPU).
+//
+// Replaces the host-side torch graph of MoeMLP.forward (round2/source/train.py:10941-11001): moe_route / moe_tournament
+// (10505-10553: softmax of fp32 router logits, the k best experts by first-maximum, gates renormalised over the two),
+// moe_positions / moe_gather_tables (10555-10634: each assignment's slot), MoeDispatch2 / MoeCombine2 (10652-10688) and
+// the gated combine (10990-10992). The reference counts a fixed capacity per sequence and drops the overflow because
+// its compiler needs static shapes; here the slot buffer is ragged and dropless: expert e's assignments are contiguous,
+// in token order, padded to a multiple of 128 rows, and a device-side table names the expert of every 128-row tile, so
+// the grouped fp8 GEMMs need no host knowledge of the loads (no sync, no recompilation when routing is skewed).
+// With a capacity that drops nothing the reference computes the same function.
+//
+// Tables (int32, device): cnt[E]; seg[E+1] padded segment offsets; tile_expert[rmax/128]; slot[N][k]; tok[rmax] (token
+// of each row or -1); ksel[rmax] (which choice a row holds).
+#include "common.hpp"
+
+namespace {
+
+constexpr int MAXE = 16;
+
+__device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
+  u32x4 u = *(const u32x4*)p;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    v[2 * k] = bflo(u[k]);
+    v[2 * k + 1] = bfhi(u[k]);
+  }
+}
+__device__ __forceinline__ void store8(bf16_t* p, const float (&v)[8]) {
+  u32x4 u = {pack2bf(v[0], v[1]), pack2bf(v[2], v[3]), pack2bf(v[4], v[5]), pack2bf(v[6], v[7])};
+  *(u32x4*)p = u;
+}
+
+// ------------------------------------------------------------------------------------------------ router
+// One wavefront per token: logits = h . Wr[e] (+ bias) in fp32, softmax, first-maximum top-k, gates.
+__global__ __launch_bounds__(256) void moe_route_kernel(const bf16_t* __restrict__ h, const float* __restrict__ wr,
+                                                       const float* __restrict__ bias, float* __restrict__ logits_out,
+                                                       float* __restrict__ p_out, int* __restrict__ idx_out,
+                                                       float* __restrict__ gate_out, long N, int d, int E, int topk) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (long n = (long)blockIdx.x * 4 + wave; n < N; n += (long)gridDim.x * 4) {
+    float acc[MAXE];
+#pragma unroll
+    for (int e = 0; e < MAXE; ++e) acc[e] = 0.f;
+    for (int c = lane * 8; c < d; c += 512) {
+      float x[8];
+      load8(h + n * d + c, x);
+#pragma unroll
+      for (int e = 0; e < MAXE; ++e) {
+        if (e < E) {
+          const float* w = wr + (long)e * d + c;
+          f32x4 w0 = *(const f32x4*)w, w1 = *(const f32x4*)(w + 4);
+          acc[e] += x[0] * w0[0] + x[1] * w0[1] + x[2] * w0[2] + x[3] * w0[3] + x[4] * w1[0] + x[5] * w1[1] + x[6] * w1[2] +
+                    x[7] * w1[3];
+        }
+      }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < MAXE; ++e) {
+      if (e < E) {
+        acc[e] = wave_sum(acc[e]) + (bias ? bias[e] : 0.f);
+        mx = fmaxf(mx, acc[e]);
+      }
+    }
+    float p[MAXE], den = 0.f;
+#pragma unroll
+    for (int e = 0; e < MAXE; ++e) {
+      p[e] = e < E ? expf(acc[e] - mx) : 0.f;
+      den += p[e];
+    }
+    int i1 = 0, i2 = 0;
+    float v1 = -1.f, v2 = -1.f;
+#pragma unroll
+    for (int e = 0; e < MAXE; ++e) {
+      if (e < E) {
+        p[e] = p[e] / den;
+        if (p[e] > v1) {
+          v1 = p[e];
+          i1 = e;
+        }
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < MAXE; ++e) {
+      if (e < E && e != i1 && p[e] > v2) {
+        v2 = p[e];
+        i2 = e;
+      }
+    }
+    if (lane == 0) {
+      for (int e = 0; e < E; ++e) {
+        p_out[n * E + e] = p[e];
+        if (logits_out) logits_out[n * E + e] = acc[e];
+      }
+      if (topk == 2) {
+        const float s = v1 + v2;
+        idx_out[n * 2] = i1;
+        idx_out[n * 2 + 1] = i2;
+        gate_out[n * 2] = v1 / s;
+        gate_out[n * 2 + 1] = v2 / s;
+      } else {
+        idx_out[n] = i1;
+        gate_out[n] = v1;
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ slot tables
+// Per wavefront of 64 tokens: how many assignments each expert receives.
+__global__ __launch_bounds__(256) void moe_count_kernel(const int* __restrict__ idx, int* __restrict__ wave_cnt, long N, int E,
+                                                       int topk) {
+  const int lane = threadIdx.x & 63;
+  const long w = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const long n = w * 64 + lane;
+  if (w * 64 >= N) return;
+  int a0 = -1, a1 = -1;
+  if (n < N) {
+    a0 = idx[n * topk];
+    if (topk == 2) a1 = idx[n * 2 + 1];
+  }
+  for (int e = 0; e < E; ++e) {
+    int c = __popcll(__ballot(a0 == e)) + __popcll(__ballot(a1 == e));
+    if (lane == 0) wave_cnt[w * E + e] = c;
+  }
+}
+
+// One workgroup: exclusive scan of the per-wavefront counts per expert, padded segment offsets, tile -> expert table.
+__global__ __launch_bounds__(256) void moe_scan_kernel(int* __restrict__ wave_cnt, int nwaves, int E, int* __restrict__ cnt,
+                                                      int* __restrict__ seg, int* __restrict__ tile_expert, int ntiles) {
+  __shared__ int s_seg[MAXE + 1];
+  if ((int)threadIdx.x < E) {
+    int e = threadIdx.x, run = 0;
+    for (int w = 0; w < nwaves; ++w) {
+      int c = wave_cnt[(long)w * E + e];
+      wave_cnt[(long)w * E + e] = run;  // becomes the wavefront's offset inside the expert's segment
+      run += c;
+    }
+    cnt[e] = run;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int off = 0;
+    for (int e = 0; e < E; ++e) {
+      s_seg[e] = off;
+      off += (cnt[e] + 127) / 128 * 128;
+    }
+    s_seg[E] = off;
+    for (int e = 0; e <= E; ++e) seg[e] = s_seg[e];
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < ntiles; t += 256) {
+    int row = t * 128, ex = -1;
+    for (int e = 0; e < E; ++e)
+      if (row >= s_seg[e] && row < s_seg[e + 1]) ex = e;
+    tile_expert[t] = ex;
+  }
+}
+
+// Every assignment's row: seg[e] + (assignments to e from earlier wavefronts) + (from earlier lanes of this one).
+__global__ __launch_bounds__(256) void moe_place_kernel(const int* __restrict__ idx, const int* __restrict__ wave_off,
+                                                       const int* __restrict__ seg, int* __restrict__ slot,
+                                                       int* __restrict__ tok, int* __restrict__ ksel, long N, int E, int topk) {
+  const int lane = threadIdx.x & 63;
+  const long w = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const long n = w * 64 + lane;
+  if (w * 64 >= N) return;
+  int a0 = -1, a1 = -1;
+  if (n < N) {
+    a0 = idx[n * topk];
+    if (topk == 2) a1 = idx[n * 2 + 1];
+  }
+  const unsigned long long lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  int r0 = 0, r1 = 0;
+  for (int e = 0; e < E; ++e) {
+    unsigned long long b0 = __ballot(a0 == e), b1 = __ballot(a1 == e);
+    int before = __popcll(b0 & lt) + __popcll(b1 & lt);
+    if (a0 == e) r0 = before;
+    if (a1 == e) r1 = before;
+  }
+  if (n < N) {
+    int s0 = seg[a0] + wave_off[w * E + a0] + r0;
+    slot[n * topk] = s0;
+    tok[s0] = (int)n;
+    ksel[s0] = 0;
+    if (topk == 2) {
+      int s1 = seg[a1] + wave_off[w * E + a1] + r1;
+      slot[n * 2 + 1] = s1;
+      tok[s1] = (int)n;
+      ksel[s1] = 1;
+    }
+  }
+}
+
+__global__ void fill_i32_kernel(int* __restrict__ p, int val, long n) {
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) p[i] = val;
+}
+
+// ------------------------------------------------------------------------------------------------ dispatch / combine
+// xs[row] = h[tok[row]] (zero rows for padding), and its e4m3 cast at `scale`.
+__global__ __launch_bounds__(256) void moe_gather_kernel(const bf16_t* __restrict__ h, const int* __restrict__ tok,
+                                                        const float* __restrict__ scale_ptr, float scale_imm,
+                                                        bf16_t* __restrict__ xs, uint8_t* __restrict__ xs8, long rmax, int d) {
+  const float sc = scale_ptr ? *scale_ptr : scale_imm;
+  const int cpr = d / 8;
+  const long total = rmax * cpr;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    long row = i / cpr;
+    int c = (int)(i % cpr) * 8;
+    int t = tok[row];
+    float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (t >= 0) load8(h + (long)t * d + c, v);
+    store8(xs + row * d + c, v);
+    u32x2 o = {cvt4_fp8<TFB_FMT_E4M3>(v[0] * sc, v[1] * sc, v[2] * sc, v[3] * sc),
+               cvt4_fp8<TFB_FMT_E4M3>(v[4] * sc, v[5] * sc, v[6] * sc, v[7] * sc)};
+    *(u32x2*)(xs8 + row * d + c) = o;
+  }
+}
+
+// out[n] = bf16(bf16(g1) y[slot1]) + bf16(bf16(g2) y[slot2]), rounded again (the eager bf16 expression).
+__global__ __launch_bounds__(256) void moe_combine_kernel(const bf16_t* __restrict__ ys, const int* __restrict__ slot,
+                                                         const float* __restrict__ gate, bf16_t* __restrict__ out, long N,
+                                                         int d, int topk) {
+  const int cpr = d / 8;
+  const long total = N * cpr;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    long n = i / cpr;
+    int c = (int)(i % cpr) * 8;
+    float a[8], r[8];
+    load8(ys + (long)slot[n * topk] * d + c, a);
+    const float g1 = round_bf(gate[n * topk]);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) r[k] = round_bf(g1 * a[k]);
+    if (topk == 2) {
+      float b[8];
+      load8(ys + (long)slot[n * 2 + 1] * d + c, b);
+      const float g2 = round_bf(gate[n * 2 + 1]);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) r[k] += round_bf(g2 * b[k]);
+    }
+    store8(out + n * d + c, r);
+  }
+}
+
+// One wavefront per slot row: dys[row] = bf16(bf16(g_k) dout[tok]); dgate[tok][k] = bf16(sum_d dout[tok] ys[row]).
+__global__ __launch_bounds__(256) void moe_combine_bwd_kernel(const bf16_t* __restrict__ dout, const bf16_t* __restrict__ ys,
+                                                             const int* __restrict__ tok, const int* __restrict__ ksel,
+                                                             const float* __restrict__ gate, bf16_t* __restrict__ dys,
+                                                             float* __restrict__ dgate, long rmax, int d, int topk) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (long row = (long)blockIdx.x * 4 + wave; row < rmax; row += (long)gridDim.x * 4) {
+    const int t = tok[row];
+    if (t < 0) {
+      for (int c = lane * 8; c < d; c += 512) *(u32x4*)(dys + row * d + c) = u32x4{0, 0, 0, 0};
+      continue;
+    }
+    const int k = ksel[row];
+    const float g = round_bf(gate[(long)t * topk + k]);
+    float dot = 0.f;
+    for (int c = lane * 8; c < d; c += 512) {
+      float go[8], y[8], r[8];
+      load8(dout + (long)t * d + c, go);
+      load8(ys + row * d + c, y);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        r[j] = g * go[j];
+        dot += go[j] * y[j];
+      }
+      store8(dys + row * d + c, r);
+    }
+    dot = wave_sum(dot);
+    if (lane == 0) dgate[(long)t * topk + k] = round_bf(dot);
+  }
+}
+
+// dlogits[n][e] = p_e (dp_e - sum_j p_j dp_j), dp from the gate gradients through the renormalisation.
+__global__ __launch_bounds__(256) void moe_dlogits_kernel(const float* __restrict__ dgate, const float* __restrict__ p,
+                                                         const int* __restrict__ idx, float* __restrict__ dlogits, long N,
+                                                         int E, int topk) {
+  long n = (long)blockIdx.x * 256 + threadIdx.x;
+  if (n >= N) return;
+  float dp[MAXE];
+  for (int e = 0; e < E; ++e) dp[e] = 0.f;
+  if (topk == 2) {
+    const int i1 = idx[n * 2], i2 = idx[n * 2 + 1];
+    const float v1 = p[n * E + i1], v2 = p[n * E + i2], den = v1 + v2;
+    const float dg1 = dgate[n * 2], dg2 = dgate[n * 2 + 1];
+    // g1 = v1 / den, g2 = v2 / den
+    const float inv2 = 1.0f / (den * den);
+    const float dv1 = (dg1 - dg2) * v2 * inv2, dv2 = (dg2 - dg1) * v1 * inv2;
+    for (int e = 0; e < E; ++e) dp[e] = e == i1 ? dv1 : (e == i2 ? dv2 : 0.f);
+  } else {
+    const int i1 = idx[n];
+    for (int e = 0; e < E; ++e) dp[e] = e == i1 ? dgate[n] : 0.f;
+  }
+  float dot = 0.f;
+  for (int e = 0; e < E; ++e) dot += p[n * E + e] * dp[e];
+  for (int e = 0; e < E; ++e) dlogits[n * E + e] = p[n * E + e] * (dp[e] - dot);
+}
+
+// dh[n] = dxs[slot1] + dxs[slot2] + sum_e dlogits[n][e] Wr[e] (fp32 sum, one rounding).
+__global__ __launch_bounds__(256) void moe_dispatch_bwd_kernel(const bf16_t* __restrict__ dxs, const int* __restrict__ slot,
+                                                              const float* __restrict__ dlogits, const float* __restrict__ wr,
+                                                              bf16_t* __restrict__ dh, long N, int d, int E, int topk) {
+  const int cpr = d / 8;
+  const long total = N * cpr;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    long n = i / cpr;
+    int c = (int)(i % cpr) * 8;
+    float r[8];
+    load8(dxs + (long)slot[n * topk] * d + c, r);
+    if (topk == 2) {
+      float b[8];
+      load8(dxs + (long)slot[n * 2 + 1] * d + c, b);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) r[k] += b[k];
+    }
+    if (dlogits) {
+      for (int e = 0; e < E; ++e) {
+        const float g = dlogits[n * E + e];
+        const float* w = wr + (long)e * d + c;
+        f32x4 w0 = *(const f32x4*)w, w1 = *(const f32x4*)(w + 4);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          r[k] += g * w0[k];
+          r[4 + k] += g * w1[k];
+        }
+      }
+    }
+    store8(dh + n * d + c, r);
+  }
+}
+
+// dWr[e][c] (+)= sum_n dlogits[n][e] h[n][c]: a workgroup owns 64 columns, 32 row lanes stride over the tokens.
+__global__ __launch_bounds__(256) void moe_dwr_kernel(const float* __restrict__ dlogits, const bf16_t* __restrict__ h,
+                                                     float* __restrict__ dwr, long N, int d, int E, int accumulate) {
+  __shared__ float red[32][8][8];
+  const int cl = threadIdx.x & 7, rl = threadIdx.x >> 3;
+  const int c = blockIdx.x * 64 + cl * 8;
+  for (int e0 = 0; e0 < E; e0 += 8) {
+    float acc[8][8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) acc[e][k] = 0.f;
+    for (long n = rl; n < N; n += 32) {
+      float x[8];
+      load8(h + n * d + c, x);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (e0 + e < E) {
+          const float g = dlogits[n * E + e0 + e];
+#pragma unroll
+          for (int k = 0; k < 8; ++k) acc[e][k] += g * x[k];
+        }
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < 8; ++k) red[rl][cl][k] = acc[e][k];
+      __syncthreads();
+      if (rl == 0 && e0 + e < E) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          float s = 0.f;
+          for (int r = 0; r < 32; ++r) s += red[r][cl][k];
+          float* o = dwr + (long)(e0 + e) * d + c + k;
+          *o = accumulate ? *o + s : s;
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ per-expert scales
+// amax of each 128-row tile of g, merged into its expert's slot (non-negative floats order like their bit patterns).
+__global__ __launch_bounds__(256) void moe_amax_kernel(const bf16_t* __restrict__ g, const int* __restrict__ tile_expert,
+                                                      unsigned* __restrict__ amax_bits, int d) {
+  __shared__ float red[4];
+  const int e = tile_expert[blockIdx.x];
+  if (e < 0) return;
+  const bf16_t* base = g + (long)blockIdx.x * 128 * d;
+  float m = 0.f;
+  for (long i = (long)threadIdx.x * 8; i < 128L * d; i += 256 * 8) {
+    u32x4 u = *(const u32x4*)(base + i);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) m = fmaxf(m, fmaxf(fabsf(bflo(u[k])), fabsf(bfhi(u[k]))));
+  }
+  m = wave_max(m);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    atomicMax(amax_bits + e, __float_as_uint(m));
+  }
+}
+
+__device__ void pow2_le_moe(float v, float limit, int e_lo, int e_hi, float* s_out, float* inv_out) {
+  float s = ldexpf(1.0f, e_lo), inv = ldexpf(1.0f, -e_lo);
+  const float top = ldexpf(1.0f, e_hi);
+  const int span = e_hi - e_lo;
+  for (int b = 64; b >= 1; b >>= 1) {
+    if (b > span) continue;
+    float cand = s * ldexpf(1.0f, b);
+    if ((v * cand <= limit) && (cand <= top)) {
+      s = cand;
+      inv = inv * ldexpf(1.0f, -b);
+    }
+  }
+  *s_out = s;
+  *inv_out = inv;
+}
+
+// rows_out[e] = rows_in[e] with the four backward columns filled from the expert's amax(dy)
+// (round2/source/kernels/nki_mlp_fused8.py:803-813, once per expert).
+__global__ void moe_backward_scales_kernel(const unsigned* __restrict__ amax_bits, const float* __restrict__ rows_in,
+                                           float* __restrict__ rows_out, int E, float dp_factor) {
+  int e = threadIdx.x;
+  if (e >= E) return;
+  const float* in = rows_in + e * 16;
+  float* out = rows_out + e * 16;
+  for (int i = 0; i < 16; ++i) out[i] = in[i];
+  const float amax_dy = __uint_as_float(amax_bits[e]);
+  float s_dy, i_dy, s_dp, i_dp;
+  pow2_le_moe(amax_dy, TFB_E5M2_MAX / 2.0f, -40, 60, &s_dy, &i_dy);
+  float bound = sqrtf(in[9] * in[10]) * amax_dy * dp_factor;
+  pow2_le_moe(bound, TFB_E5M2_MAX, -40, 60, &s_dp, &i_dp);
+  out[5] = s_dy;
+  out[6] = i_dy * in[12] * 2.0f;
+  out[7] = s_dp;
+  out[8] = i_dp * in[11];
+}
+
+// out8[row] = fp8(x[row] * rows[expert of row][col]) for the rows of live tiles; padding tiles are zero-filled.
+template <int FMT>
+__global__ __launch_bounds__(256) void moe_quant_kernel(const bf16_t* __restrict__ x, const int* __restrict__ tile_expert,
+                                                       const float* __restrict__ rows, int col, uint8_t* __restrict__ out,
+                                                       long rmax, int d) {
+  const int cpr = d / 8;
+  const long total = rmax * cpr;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    long row = i / cpr;
+    int c = (int)(i % cpr) * 8;
+    int e = tile_expert[row >> 7];
+    u32x2 o = {0, 0};
+    if (e >= 0) {
+      const float s = rows[e * 16 + col];
+      float v[8];
+      load8(x + row * d + c, v);
+      o.x = cvt4_fp8<FMT>(v[0] * s, v[1] * s, v[2] * s, v[3] * s);
+      o.y = cvt4_fp8<FMT>(v[4] * s, v[5] * s, v[6] * s, v[7] * s);
+    }
+    *(u32x2*)(out + row * d + c) = o;
+  }
+}
+
+inline int nblocks(long n, int cap = 8192) {
+  long b = (n + 255) / 256;
+  return (int)(b < 1 ? 1 : (b < cap ? b : cap));
+}
+
+}  // namespace
+
+// Upper bound of the padded slot rows for N tokens: every expert's segment rounds up to 128 (host helper).
+extern "C" long tfb_moe_max_rows(long N, int E, int topk) { return (N * topk + (long)E * 127) / 128 * 128; }
+
+// h bf16 [N][d], wr fp32 [E][d], bias fp32 [E] or NULL -> logits (optional) / p fp32 [N][E], idx int32 [N][topk],
+// gate fp32 [N][topk]. E <= 16, topk 1 or 2, d % 8 == 0.
+// Replaces F.linear(h.float(), router.float()) + moe_route (round2/source/train.py:10525-10553, 10961).
+extern "C" int tfb_moe_route(const void* h, const void* wr, const void* bias, void* logits, void* p, void* idx, void* gate, long N,
+                             int d, int E, int topk, void* stream) {
+  if (!h || !wr || !p || !idx || !gate) return TFB_ERR_ARG;
+  if (N <= 0 || d <= 0 || d % 8 || E < 2 || E > MAXE || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_route_kernel, dim3(nblocks(N * 64)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)h,
+                     (const float*)wr, (const float*)bias, (float*)logits, (float*)p, (int*)idx, (float*)gate, N, d, E, topk);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// idx int32 [N][topk] -> cnt [E], seg [E+1], tile_expert [rmax/128], slot [N][topk], tok [rmax], ksel [rmax];
+// scratch: int32 [ceil(N/64) * E]. rmax = tfb_moe_max_rows(N, E, topk).
+// Replaces moe_positions + moe_gather_tables (round2/source/train.py:10555-10634), dropless.
+extern "C" int tfb_moe_tables(const void* idx, void* cnt, void* seg, void* tile_expert, void* slot, void* tok, void* ksel,
+                              void* scratch, long N, int E, int topk, long rmax, void* stream) {
+  if (!idx || !cnt || !seg || !tile_expert || !slot || !tok || !ksel || !scratch) return TFB_ERR_ARG;
+  if (N <= 0 || E < 2 || E > MAXE || (topk != 1 && topk != 2) || rmax % 128 || rmax < tfb_moe_max_rows(N, E, topk))
+    return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const int nwaves = (int)((N + 63) / 64);
+  const int nb = (nwaves + 3) / 4;
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(nblocks(rmax)), dim3(256), 0, s, (int*)tok, -1, rmax);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_count_kernel, dim3(nb), dim3(256), 0, s, (const int*)idx, (int*)scratch, N, E, topk);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(256), 0, s, (int*)scratch, nwaves, E, (int*)cnt, (int*)seg,
+                     (int*)tile_expert, (int)(rmax / 128));
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_place_kernel, dim3(nb), dim3(256), 0, s, (const int*)idx, (const int*)scratch, (const int*)seg,
+                     (int*)slot, (int*)tok, (int*)ksel, N, E, topk);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// xs bf16 [rmax][d] = h[tok] (zero padding rows), xs8 = e4m3(xs * scale). Replaces MoeDispatch2.forward (10652-10660).
+extern "C" int tfb_moe_gather(const void* h, const void* tok, const void* scale_ptr, float scale_imm, void* xs, void* xs8,
+                              long rmax, int d, void* stream) {
+  if (!h || !tok || !xs || !xs8) return TFB_ERR_ARG;
+  if (rmax <= 0 || d <= 0 || d % 8) return TFB_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_gather_kernel, dim3(nblocks(rmax * (d / 8))), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)h,
+                     (const int*)tok, (const float*)scale_ptr, scale_imm, (bf16_t*)xs, (uint8_t*)xs8, rmax, d);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// out bf16 [N][d] = sum_k bf16(gate_k) ys[slot_k]. Replaces MoeCombine2.forward + the gated sum (10672-10676, 10990-10992).
+extern "C" int tfb_moe_combine(const void* ys, const void* slot, const void* gate, void* out, long N, int d, int topk,
+                               void* stream) {
+  if (!ys || !slot || !gate || !out) return TFB_ERR_ARG;
+  if (N <= 0 || d <= 0 || d % 8 || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(nblocks(N * (d / 8))), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)ys,
+                     (const int*)slot, (const float*)gate, (bf16_t*)out, N, d, topk);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// dys bf16 [rmax][d], dgate fp32 [N][topk] from dout bf16 [N][d]. Replaces MoeCombine2.backward (10678-10688).
+extern "C" int tfb_moe_combine_bwd(const void* dout, const void* ys, const void* tok, const void* ksel, const void* gate,
+                                   void* dys, void* dgate, long rmax, int d, int topk, void* stream) {
+  if (!dout || !ys || !tok || !ksel || !gate || !dys || !dgate) return TFB_ERR_ARG;
+  if (rmax <= 0 || d <= 0 || d % 8 || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_combine_bwd_kernel, dim3(nblocks(rmax * 64)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)dout,
+                     (const bf16_t*)ys, (const int*)tok, (const int*)ksel, (const float*)gate, (bf16_t*)dys, (float*)dgate, rmax,
+                     d, topk);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// Router backward + dispatch backward: dlogits fp32 [N][E] (scratch/output), dh bf16 [N][d] = dxs[slots] + dlogits Wr,
+// dwr fp32 [E][d] (+)= dlogits^T h. Replaces MoeDispatch2.backward (10662-10666) and autograd through moe_route.
+extern "C" int tfb_moe_route_bwd(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot,
+                                 const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate, long N,
+                                 int d, int E, int topk, void* stream) {
+  if (!dgate || !p || !idx || !dxs || !slot || !h || !wr || !dlogits || !dh || !dwr) return TFB_ERR_ARG;
+  if (N <= 0 || d <= 0 || d % 64 || E < 2 || E > MAXE || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(moe_dlogits_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, (const float*)dgate,
+                     (const float*)p, (const int*)idx, (float*)dlogits, N, E, topk);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_dispatch_bwd_kernel, dim3(nblocks(N * (d / 8))), dim3(256), 0, s, (const bf16_t*)dxs, (const int*)slot,
+                     (const float*)dlogits, (const float*)wr, (bf16_t*)dh, N, d, E, topk);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_dwr_kernel, dim3(d / 64), dim3(256), 0, s, (const float*)dlogits, (const bf16_t*)h, (float*)dwr, N, d, E,
+                     dwr_accumulate);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// rows_out fp32 [E][16]: each expert's backward scale row from the amax of its rows of dys; amax_scratch: uint32 [E].
+extern "C" int tfb_moe_backward_scales(const void* dys, const void* tile_expert, const void* rows_in, void* rows_out,
+                                       void* amax_scratch, long rmax, int d, int E, void* stream) {
+  if (!dys || !tile_expert || !rows_in || !rows_out || !amax_scratch) return TFB_ERR_ARG;
+  if (rmax <= 0 || rmax % 128 || d % 8 || E < 1 || E > MAXE) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(256), 0, s, (int*)amax_scratch, 0, (long)E);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_amax_kernel, dim3((unsigned)(rmax / 128)), dim3(256), 0, s, (const bf16_t*)dys, (const int*)tile_expert,
+                     (unsigned*)amax_scratch, d);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_backward_scales_kernel, dim3(1), dim3(64), 0, s, (const unsigned*)amax_scratch, (const float*)rows_in,
+                     (float*)rows_out, E, (float)(36.16 * (double)d));
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// out8 = fp8(x * rows[expert][col]) row-wise by the tile's expert (fmt 0 e4m3, 1 e5m2).
+extern "C" int tfb_moe_quant(const void* x, const void* tile_expert, const void* rows, int col, int fmt, void* out8, long rmax,
+                             int d, void* stream) {
+  if (!x || !tile_expert || !rows || !out8) return TFB_ERR_ARG;
+  if (rmax <= 0 || rmax % 128 || d % 8 || col < 0 || col >= 16) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  int nb = nblocks(rmax * (d / 8));
+  if (fmt == TFB_FMT_E4M3)
+    hipLaunchKernelGGL(moe_quant_kernel<TFB_FMT_E4M3>, dim3(nb), dim3(256), 0, s, (const bf16_t*)x, (const int*)tile_expert,
+                       (const float*)rows, col, (uint8_t*)out8, rmax, d);
+  else if (fmt == TFB_FMT_E5M2)
+    hipLaunchKernelGGL(moe_quant_kernel<TFB_FMT_E5M2>, dim3(nb), dim3(256), 0, s, (const bf16_t*)x, (const int*)tile_expert,
+                       (const float*)rows, col, (uint8_t*)out8, rmax, d);
+  else
+    return TFB_ERR_ARG;
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}

@@ -413,3 +413,136 @@ def lmhead_fwd(x2, W, targets, softcap=None, row_w=None):
     _lib.call("tfb_lmhead_fwd", _p(x2), _p(W), _p(tg), int(tg.dtype == torch.int64), _p(row_w), _p(logits), _p(part), _p(loss),
               _p(lse), N, d, V, float(softcap or 0.0), _stream())
     return logits, loss, lse
+
+
+# ------------------------------------------------------------------------------------------ mixture of experts
+def moe_max_rows(N, E, topk):
+    return _lib.lib().tfb_moe_max_rows(N, E, topk)
+
+
+def moe_route(h2, wr, topk, bias=None, want_logits=False):
+    """(p fp32 [N,E], idx int32 [N,topk], gate fp32 [N,topk], logits or None) from h2 bf16 [N,d], wr fp32 [E,d]."""
+    _chk(h2), _chk(wr, torch.float32), _chk(bias, torch.float32)
+    N, d = h2.shape
+    E = wr.shape[0]
+    dev = h2.device
+    p = torch.empty(N, E, dtype=torch.float32, device=dev)
+    idx = torch.empty(N, topk, dtype=torch.int32, device=dev)
+    gate = torch.empty(N, topk, dtype=torch.float32, device=dev)
+    logits = torch.empty(N, E, dtype=torch.float32, device=dev) if want_logits else None
+    _lib.call("tfb_moe_route", _p(h2), _p(wr), _p(bias), _p(logits), _p(p), _p(idx), _p(gate), N, d, E, topk, _stream())
+    return p, idx, gate, logits
+
+
+def moe_tables(idx, E):
+    """Slot tables for the dropless ragged layout: dict(cnt, seg, tile_expert, slot, tok, ksel, rmax)."""
+    _chk(idx, torch.int32)
+    N, topk = idx.shape
+    dev = idx.device
+    rmax = moe_max_rows(N, E, topk)
+    i32 = dict(dtype=torch.int32, device=dev)
+    t = {"cnt": torch.empty(E, **i32), "seg": torch.empty(E + 1, **i32), "tile_expert": torch.empty(rmax // 128, **i32),
+         "slot": torch.empty(N, topk, **i32), "tok": torch.empty(rmax, **i32), "ksel": torch.empty(rmax, **i32), "rmax": rmax}
+    scratch = torch.empty(((N + 63) // 64) * E, **i32)
+    _lib.call("tfb_moe_tables", _p(idx), _p(t["cnt"]), _p(t["seg"]), _p(t["tile_expert"]), _p(t["slot"]), _p(t["tok"]),
+              _p(t["ksel"]), _p(scratch), N, E, topk, rmax, _stream())
+    return t
+
+
+def moe_gather(h2, tab, x_scale=4.0):
+    """(xs bf16 [rmax,d], xs8 uint8 [rmax,d])."""
+    _chk(h2)
+    d = h2.shape[1]
+    rmax = tab["rmax"]
+    xs = torch.empty(rmax, d, dtype=bf16, device=h2.device)
+    xs8 = torch.empty(rmax, d, dtype=torch.uint8, device=h2.device)
+    if isinstance(x_scale, torch.Tensor):
+        _lib.call("tfb_moe_gather", _p(h2), _p(tab["tok"]), _p(x_scale), 0.0, _p(xs), _p(xs8), rmax, d, _stream())
+    else:
+        _lib.call("tfb_moe_gather", _p(h2), _p(tab["tok"]), None, float(x_scale), _p(xs), _p(xs8), rmax, d, _stream())
+    return xs, xs8
+
+
+def moe_mlp8_fwd(xs8, w8, rows, tab, F):
+    """Grouped fp8 expert MLP forward: (ys bf16 [rmax,d], r bf16 [rmax,F]). w8 uint8 [E,4,F*d], rows fp32 [E,16]."""
+    _chk(xs8, torch.uint8), _chk(w8, torch.uint8), _chk(rows, torch.float32)
+    rmax, d = xs8.shape
+    ys = torch.empty(rmax, d, dtype=bf16, device=xs8.device)
+    r = torch.empty(rmax, F, dtype=bf16, device=xs8.device)
+    h8 = torch.empty(rmax, F, dtype=torch.uint8, device=xs8.device)
+    _lib.call("tfb_moe_mlp8_fwd", _p(xs8), _p(w8), _p(rows), _p(tab["tile_expert"]), _p(ys), _p(r), _p(h8), rmax, d, F, _stream())
+    return ys, r
+
+
+def moe_backward_scales(dys, rows, tab):
+    _chk(dys), _chk(rows, torch.float32)
+    E = rows.shape[0]
+    out = torch.empty_like(rows)
+    scratch = torch.empty(E, dtype=torch.int32, device=dys.device)
+    _lib.call("tfb_moe_backward_scales", _p(dys), _p(tab["tile_expert"]), _p(rows), _p(out), _p(scratch), dys.shape[0],
+              dys.shape[1], E, _stream())
+    return out
+
+
+def moe_quant(x, rows, col, fmt, tab):
+    _chk(x), _chk(rows, torch.float32)
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    _lib.call("tfb_moe_quant", _p(x), _p(tab["tile_expert"]), _p(rows), col, fmt, _p(out), x.shape[0], x.shape[1], _stream())
+    return out
+
+
+def moe_mlp8_bwd(dys, r, w8, rows_bwd, tab):
+    """(dxs bf16 [rmax,d], dpre bf16 [rmax,F]) from dys; rows_bwd from moe_backward_scales."""
+    _chk(dys), _chk(r)
+    rmax, d = dys.shape
+    F = r.shape[1]
+    dy8 = moe_quant(dys, rows_bwd, 5, FMT_E5M2, tab)
+    dxs = torch.empty(rmax, d, dtype=bf16, device=dys.device)
+    dpre = torch.empty(rmax, F, dtype=bf16, device=dys.device)
+    dp8 = torch.empty(rmax, F, dtype=torch.uint8, device=dys.device)
+    _lib.call("tfb_moe_mlp8_bwd", _p(dy8), _p(r), _p(w8), _p(rows_bwd), _p(tab["tile_expert"]), _p(dxs), _p(dpre), _p(dp8), rmax, d,
+              F, _stream())
+    return dxs, dpre
+
+
+def moe_dw(dpre, xs, dys, r, tab, E, dw_fc=None, dw_proj=None, accumulate=False, out_dtype=bf16):
+    """(dw_fc [E,F,d], dw_proj [E,d,F]) over each expert's row segment."""
+    d, F = xs.shape[1], r.shape[1]
+    if dw_fc is None:
+        dw_fc = torch.empty(E, F, d, dtype=out_dtype, device=xs.device)
+        dw_proj = torch.empty(E, d, F, dtype=out_dtype, device=xs.device)
+    _lib.call("tfb_moe_dw", _p(dpre), _p(xs), _p(dys), _p(r), _p(tab["seg"]), _p(dw_fc), _p(dw_proj), E, d, F,
+              int(dw_fc.dtype == torch.float32), int(accumulate), _stream())
+    return dw_fc, dw_proj
+
+
+def moe_combine(ys, tab, gate, N):
+    _chk(ys), _chk(gate, torch.float32)
+    d = ys.shape[1]
+    out = torch.empty(N, d, dtype=bf16, device=ys.device)
+    _lib.call("tfb_moe_combine", _p(ys), _p(tab["slot"]), _p(gate), _p(out), N, d, gate.shape[1], _stream())
+    return out
+
+
+def moe_combine_bwd(dout, ys, tab, gate):
+    _chk(dout), _chk(ys), _chk(gate, torch.float32)
+    rmax, d = ys.shape
+    dys = torch.empty_like(ys)
+    dgate = torch.empty_like(gate)
+    _lib.call("tfb_moe_combine_bwd", _p(dout), _p(ys), _p(tab["tok"]), _p(tab["ksel"]), _p(gate), _p(dys), _p(dgate), rmax, d,
+              gate.shape[1], _stream())
+    return dys, dgate
+
+
+def moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, dwr=None, accumulate=False):
+    """(dh bf16 [N,d], dwr fp32 [E,d], dlogits fp32 [N,E])."""
+    N, d = h2.shape
+    E = wr.shape[0]
+    dlogits = torch.empty(N, E, dtype=torch.float32, device=h2.device)
+    dh = torch.empty_like(h2)
+    if dwr is None:
+        dwr = torch.empty(E, d, dtype=torch.float32, device=h2.device)
+        accumulate = False
+    _lib.call("tfb_moe_route_bwd", _p(dgate), _p(p), _p(idx), _p(dxs), _p(tab["slot"]), _p(h2), _p(wr), _p(dlogits), _p(dh),
+              _p(dwr), int(accumulate), N, d, E, idx.shape[1], _stream())
+    return dh, dwr, dlogits
