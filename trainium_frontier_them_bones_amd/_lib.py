@@ -7,7 +7,7 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libtfb_hip.so")
+LIB_PATH = os.environ.get("TFB_LIB_PATH") or os.path.join(HERE, "libtfb_hip.so")  # override: another build of the same ABI
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int

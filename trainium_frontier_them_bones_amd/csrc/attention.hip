@@ -21,6 +21,22 @@
 // contiguous, so q/k/v may be thirds of a fused qkv [B,T,3C] buffer and o / dO are [B,T,H,D].
 #include "common.hpp"
 
+#ifndef TFB_FWD_WPE
+#define TFB_FWD_WPE 3  // wavefronts per SIMD the forward kernel is compiled for (register budget 512 / WPE)
+#endif
+#ifndef TFB_DKDV_WPE
+#define TFB_DKDV_WPE 2
+#endif
+#ifndef TFB_BWD_NBUF
+#define TFB_BWD_NBUF 1  // LDS buffers of the backward kernels' staged tiles
+#endif
+#ifndef TFB_DQ_WPE
+#define TFB_DQ_WPE 2
+#endif
+#ifndef TFB_FWD_QG2
+#define TFB_FWD_QG2 0  // two query groups per wavefront: measured slower (373 VGPRs, one wavefront per SIMD)
+#endif
+
 namespace {
 
 struct AttnT {
@@ -78,12 +94,15 @@ constexpr float LN2 = 0.6931471805599453f;
 constexpr int TROW = 64 * 2 + 8;
 
 // =========================================================================================== forward
-template <int D>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(AttnT q, AttnT k, AttnT v, AttnT o, float* __restrict__ lse, int T,
+// QG = query groups of 32 per wavefront. With QG = 2 every K / V^T fragment read from LDS feeds two MFMAs (half the LDS
+// traffic per flop) and the two groups' softmax arithmetic and MFMAs are independent instruction streams that co-execute.
+template <int D, int QG>
+__global__ __launch_bounds__(256, (D == 64 && QG == 1) ? TFB_FWD_WPE : 1) void attn_fwd_kernel(AttnT q, AttnT k, AttnT v, AttnT o, float* __restrict__ lse, int T,
                                                       int H, float sl2) {
   constexpr int DS = D / 16, DT = D / 32, NV = D / 64;
   constexpr int KROW = D * 2 + 16;
   constexpr int KBYTES = 64 * KROW, VBYTES = D * TROW, BUF = KBYTES + VBYTES;
+  constexpr int QB = 128 * QG, QW = 32 * QG;  // queries per workgroup / per wavefront
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int qb = gridDim.x - 1 - blockIdx.x;  // longest rows first
@@ -92,13 +111,15 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnT q, AttnT k, AttnT v
   const bf16_t* kp = k.p + b * k.sb + h * k.sh;
   const bf16_t* vp = v.p + b * v.sb + h * v.sh;
   bf16_t* op = o.p + b * o.sb + h * o.sh;
-  const int q0 = qb * 128, qw0 = q0 + wave * 32, myq = qw0 + lr;
+  const int q0 = qb * QB, qw0 = q0 + wave * QW;
 
-  bf16x8 qf[DS];
+  bf16x8 qf[QG][DS];
 #pragma unroll
-  for (int s = 0; s < DS; ++s) qf[s] = *(const bf16x8*)(qp + (long)myq * q.st + 16 * s + 8 * lh);
+  for (int g = 0; g < QG; ++g)
+#pragma unroll
+    for (int s = 0; s < DS; ++s) qf[g][s] = *(const bf16x8*)(qp + (long)(qw0 + 32 * g + lr) * q.st + 16 * s + 8 * lh);
 
-  const int ntiles = (q0 + 128) / 64;
+  const int ntiles = (q0 + QB) / 64;
   const bool vrole = wave < 2;
   const int t2 = tid & 127;
   MicroBlock mb[NV];  // V micro-blocks (waves 0,1) or DS K chunks (waves 2,3) share these registers
@@ -137,12 +158,17 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnT q, AttnT k, AttnT v
     }
   };
 
-  f32x16 oacc[DT];
+  f32x16 oacc[QG][DT];
+  float m[QG], l[QG];
 #pragma unroll
-  for (int i = 0; i < DT; ++i)
+  for (int g = 0; g < QG; ++g) {
+    m[g] = -1e30f;  // running maximum of the raw scores
+    l[g] = 0.f;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) oacc[i][e] = 0.f;
-  float m = -1e30f, l = 0.f;
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) oacc[g][i][e] = 0.f;
+  }
 
   gload(0);
   sstore(smem);
@@ -153,75 +179,93 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnT q, AttnT k, AttnT v
     const bool more = t + 1 < ntiles;
     if (more) gload(t + 1);
     const int k0 = t * 64;
-    if (k0 <= qw0 + 31) {
-      f32x16 st[2];
+    if (k0 <= qw0 + QW - 1) {
+      f32x16 st[QG][2];
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
+      for (int g = 0; g < QG; ++g)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) st[kt][e] = 0.f;
+        for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int s = 0; s < DS; ++s)
-          st[kt] = mfma_bf16(lds16(cur, (kt * 32 + lr) * KROW + s * 32 + lh * 16), qf[s], st[kt]);
-      }
-      const bool diag = k0 + 63 > qw0;
-      const int kbase = k0 + lh * 4 - myq;  // key - q for element (kt, e) is kbase + kt*32 + (e>>2)*8 + (e&3)
-      float mx = m;                         // running maximum of the raw scores
+          for (int e = 0; e < 16; ++e) st[g][kt][e] = 0.f;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          if (diag && (kbase + kt * 32 + (e >> 2) * 8 + (e & 3) > 0)) st[kt][e] = -INFINITY;
-          mx = fmaxf(mx, st[kt][e]);
-        }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      if (__builtin_amdgcn_ballot_w64(mx > m) != 0) {  // some row's maximum moved: rescale (wavefront-uniform branch)
-        const float alpha = fast_exp2((m - mx) * sl2);
-        l *= alpha;
+        for (int s = 0; s < DS; ++s) {
+          bf16x8 a = lds16(cur, (kt * 32 + lr) * KROW + s * 32 + lh * 16);
 #pragma unroll
-        for (int i = 0; i < DT; ++i)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) oacc[i][e] *= alpha;
-      }
-      m = mx;
-      const float negm = -mx * sl2;
-      uint32_t pk[2][8];
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int e = 0; e < 16; e += 2) {
-          float p0 = fast_exp2(fmaf(st[kt][e], sl2, negm)), p1 = fast_exp2(fmaf(st[kt][e + 1], sl2, negm));
-          uint32_t w = pack2bf(p0, p1);
-          l = sum2bf(w, l);  // the row sum runs over the rounded values
-          pk[kt][e >> 1] = w;
+          for (int g = 0; g < QG; ++g) st[g][kt] = mfma_bf16(a, qf[g][s], st[g][kt]);
         }
       const uint8_t* vt = cur + KBYTES;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+      for (int g = 0; g < QG; ++g) {
+        const int qg0 = qw0 + 32 * g;
+        const bool diag = k0 + 63 > qg0;
+        const int kbase = k0 + lh * 4 - (qg0 + lr);  // key - q for element (kt, e) is kbase + kt*32 + (e>>2)*8 + (e&3)
+        float mx = m[g];
+        if (diag) {  // wavefront-uniform; the per-element masking below is branch-free selects
+#pragma unroll
+          for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+              const bool future = kbase + kt * 32 + (e >> 2) * 8 + (e & 3) > 0;
+              st[g][kt][e] = future ? -INFINITY : st[g][kt][e];
+            }
+        }
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int e = 0; e < 16; e += 2) mx = fmaxf(fmaxf(mx, st[g][kt][e]), st[g][kt][e + 1]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float alpha = fast_exp2((m[g] - mx) * sl2);
+        m[g] = mx;
+        l[g] *= alpha;
+#pragma unroll
+        for (int i = 0; i < DT; ++i)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) oacc[g][i][e] *= alpha;
+        const float negm = -mx * sl2;
+        // 16 keys at a time: exponentials and packing (VALU) of one chunk run beside the PV MFMAs of the previous one
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
           for (int hf = 0; hf < 2; ++hf) {
-            bf16x8 a = lds8x2(vt, (dt * 32 + lr) * TROW + (kt * 32 + 16 * hf + 4 * lh) * 2);
-            bf16x8 bb = frag_from(pk[kt][4 * hf], pk[kt][4 * hf + 1], pk[kt][4 * hf + 2], pk[kt][4 * hf + 3]);
-            oacc[dt] = mfma_bf16(a, bb, oacc[dt]);
+            uint32_t w[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+              const int e = 8 * hf + 2 * x;
+              float p0 = fast_exp2(fmaf(st[g][kt][e], sl2, negm)), p1 = fast_exp2(fmaf(st[g][kt][e + 1], sl2, negm));
+              w[x] = pack2bf(p0, p1);
+              l[g] = sum2bf(w[x], l[g]);  // the row sum runs over the rounded values
+            }
+            const bf16x8 bb = frag_from(w[0], w[1], w[2], w[3]);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+              bf16x8 a = lds8x2(vt, (dt * 32 + lr) * TROW + (kt * 32 + 16 * hf + 4 * lh) * 2);
+              oacc[g][dt] = mfma_bf16(a, bb, oacc[g][dt]);
+            }
           }
+      }
     }
     if (more) sstore(smem + ((t + 1) & 1) * BUF);
     __syncthreads();
   }
 
-  l += __shfl_xor(l, 32, 64);
-  const float inv = 1.0f / l;
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+  for (int g = 0; g < QG; ++g) {
+    const int myq = qw0 + 32 * g + lr;
+    float lt = l[g] + __shfl_xor(l[g], 32, 64);
+    const float inv = 1.0f / lt;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      int d = dt * 32 + 8 * j + 4 * lh;
-      u32x2 w = {pack2bf(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
-                 pack2bf(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv)};
-      *(u32x2*)(op + (long)myq * o.st + d) = w;
-    }
-  if (lh == 0) lse[(long)bh * T + myq] = (m * sl2 + log2f(l)) * LN2;  // m is the raw-score maximum
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int d = dt * 32 + 8 * j + 4 * lh;
+        u32x2 w = {pack2bf(oacc[g][dt][4 * j] * inv, oacc[g][dt][4 * j + 1] * inv),
+                   pack2bf(oacc[g][dt][4 * j + 2] * inv, oacc[g][dt][4 * j + 3] * inv)};
+        *(u32x2*)(op + (long)myq * o.st + d) = w;
+      }
+    if (lh == 0) lse[(long)bh * T + myq] = (m[g] * sl2 + log2f(lt)) * LN2;  // m is the raw-score maximum
+  }
 }
 
 // =========================================================================================== delta
@@ -255,7 +299,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(AttnT o, AttnT go, floa
 
 // =========================================================================================== dK / dV
 template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dk, AttnT dv,
+__global__ __launch_bounds__(256, D == 64 ? TFB_DKDV_WPE : 1) void attn_bwd_dkdv_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dk, AttnT dv,
                                                            const float* __restrict__ lse, const float* __restrict__ delta,
                                                            int T, int H, float scale, float sl2) {
   constexpr int DS = D / 16, DT = D / 32, NV = D / 64;
@@ -324,7 +368,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnT q, AttnT k, At
   __syncthreads();
 
   for (int qt = qt0; qt < nqt; ++qt) {
-    const uint8_t* cur = smem + ((qt - qt0) & 1) * BUF;
+    const uint8_t* cur = smem + (TFB_BWD_NBUF == 2 ? ((qt - qt0) & 1) * BUF : 0);
     const bool more = qt + 1 < nqt;
     if (more) gload(qt + 1);
     const float* ls = (const float*)(cur + OFF_L);
@@ -345,6 +389,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnT q, AttnT k, At
       }
       const bool diag = kw0 + 31 > qlo;
       const int kq = mykey - (qlo + 4 * lh);  // key - q for element e is kq - (e>>2)*8 - (e&3)
+      if (diag) {  // wavefront-uniform; masked scores become -inf (P = 0) through branch-free selects
+#pragma unroll
+        for (int e = 0; e < 16; ++e) S[e] = (kq - 8 * (e >> 2) - (e & 3) > 0) ? -INFINITY : S[e];
+      }
       uint32_t pw[8], dsw[8];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -354,7 +402,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnT q, AttnT k, At
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           p[i] = fast_exp2(fmaf(S[4 * j + i], sl2, L[i]));
-          if (diag && (kq - 8 * j - i > 0)) p[i] = 0.f;
         }
         uint32_t w0 = pack2bf(p[0], p[1]), w1 = pack2bf(p[2], p[3]);
         pw[2 * j] = w0;
@@ -375,7 +422,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnT q, AttnT k, At
           dka[dt] = mfma_bf16(lds8x2(cur + OFF_QT, off), db, dka[dt]);
         }
     }
-    if (more) sstore(smem + ((qt + 1 - qt0) & 1) * BUF);
+    if (TFB_BWD_NBUF == 1) __syncthreads();
+    if (more) sstore(smem + (TFB_BWD_NBUF == 2 ? ((qt + 1 - qt0) & 1) * BUF : 0));
     __syncthreads();
   }
 
@@ -396,7 +444,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnT q, AttnT k, At
 
 // =========================================================================================== dQ
 template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dq,
+__global__ __launch_bounds__(256, D == 64 ? TFB_DQ_WPE : 1) void attn_bwd_dq_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dq,
                                                          const float* __restrict__ lse, const float* __restrict__ delta,
                                                          int T, int H, float scale, float sl2) {
   constexpr int DS = D / 16, DT = D / 32, NV = D / 64;
@@ -473,7 +521,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnT q, AttnT k, Attn
   __syncthreads();
 
   for (int t = 0; t < ntiles; ++t) {
-    const uint8_t* cur = smem + (t & 1) * BUF;
+    const uint8_t* cur = smem + (TFB_BWD_NBUF == 2 ? (t & 1) * BUF : 0);
     const bool more = t + 1 < ntiles;
     if (more) gload(t + 1);
     const int k0 = t * 64;
@@ -494,12 +542,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnT q, AttnT k, Attn
       }
       const bool diag = klo + 31 > qw0;
       const int kbase = klo + lh * 4 - myq;
+      if (diag) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) S[e] = (kbase + (e >> 2) * 8 + (e & 3) > 0) ? -INFINITY : S[e];
+      }
       uint32_t dsw[8];
 #pragma unroll
       for (int e = 0; e < 16; e += 2) {
         float p0 = fast_exp2(fmaf(S[e], sl2, myL)), p1 = fast_exp2(fmaf(S[e + 1], sl2, myL));
-        if (diag && (kbase + (e >> 2) * 8 + (e & 3) > 0)) p0 = 0.f;
-        if (diag && (kbase + ((e + 1) >> 2) * 8 + ((e + 1) & 3) > 0)) p1 = 0.f;
         uint32_t w = pack2bf(p0, p1);
         dsw[e >> 1] = pack2bf(bflo(w) * (dP[e] - myD), bfhi(w) * (dP[e + 1] - myD));
       }
@@ -512,7 +562,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnT q, AttnT k, Attn
           dqa[dt] = mfma_bf16(a, bb, dqa[dt]);
         }
     }
-    if (more) sstore(smem + ((t + 1) & 1) * BUF);
+    if (TFB_BWD_NBUF == 1) __syncthreads();
+    if (more) sstore(smem + (TFB_BWD_NBUF == 2 ? ((t + 1) & 1) * BUF : 0));
     __syncthreads();
   }
 
@@ -538,17 +589,25 @@ AttnT mk(const void* p, const long* s) { return AttnT{(bf16_t*)p, s[0], s[1], s[
 
 bool strides_ok(const long* s) { return s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0; }
 
-template <int D>
-int fwd_impl(AttnT q, AttnT k, AttnT v, AttnT o, float* lse, int B, int H, int T, float scale, hipStream_t s) {
+template <int D, int QG>
+int fwd_launch(AttnT q, AttnT k, AttnT v, AttnT o, float* lse, int B, int H, int T, float scale, hipStream_t s) {
   constexpr int BUF = 64 * (D * 2 + 16) + D * TROW;
   static bool once = false;
   if (!once) {
-    if (set_lds(attn_fwd_kernel<D>, 2 * BUF) != TFB_OK) return TFB_ERR_LAUNCH;
+    if (set_lds(attn_fwd_kernel<D, QG>, 2 * BUF) != TFB_OK) return TFB_ERR_LAUNCH;
     once = true;
   }
-  hipLaunchKernelGGL(attn_fwd_kernel<D>, dim3(T / 128, B * H), dim3(256), 2 * BUF, s, q, k, v, o, lse, T, H, scale * LOG2E);
+  hipLaunchKernelGGL((attn_fwd_kernel<D, QG>), dim3(T / (128 * QG), B * H), dim3(256), 2 * BUF, s, q, k, v, o, lse, T, H,
+                     scale * LOG2E);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
+}
+
+template <int D>
+int fwd_impl(AttnT q, AttnT k, AttnT v, AttnT o, float* lse, int B, int H, int T, float scale, hipStream_t s) {
+  // two query groups per wavefront when the sequence splits into 256-query blocks and the registers allow (D = 64)
+  if (TFB_FWD_QG2 && D == 64 && T % 256 == 0) return fwd_launch<D, (D == 64 ? 2 : 1)>(q, k, v, o, lse, B, H, T, scale, s);
+  return fwd_launch<D, 1>(q, k, v, o, lse, B, H, T, scale, s);
 }
 
 template <int D>
@@ -558,17 +617,17 @@ int bwd_impl(AttnT q, AttnT k, AttnT v, AttnT o, AttnT go, AttnT dq, AttnT dk, A
   constexpr int BUF1 = 2 * NB + 2 * TB + 512, BUF2 = 2 * NB + TB;
   static bool once = false;
   if (!once) {
-    if (set_lds(attn_bwd_dkdv_kernel<D>, 2 * BUF1) != TFB_OK) return TFB_ERR_LAUNCH;
-    if (set_lds(attn_bwd_dq_kernel<D>, 2 * BUF2) != TFB_OK) return TFB_ERR_LAUNCH;
+    if (set_lds(attn_bwd_dkdv_kernel<D>, TFB_BWD_NBUF * BUF1) != TFB_OK) return TFB_ERR_LAUNCH;
+    if (set_lds(attn_bwd_dq_kernel<D>, TFB_BWD_NBUF * BUF2) != TFB_OK) return TFB_ERR_LAUNCH;
     once = true;
   }
   const long rows = (long)B * H * T;
   hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)((rows * 4 + 255) / 256)), dim3(256), 0, s, o, go, delta, T, H, rows);
   TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(attn_bwd_dkdv_kernel<D>, dim3(T / 128, B * H), dim3(256), 2 * BUF1, s, q, k, v, go, dk, dv, lse, delta, T, H,
+  hipLaunchKernelGGL(attn_bwd_dkdv_kernel<D>, dim3(T / 128, B * H), dim3(256), TFB_BWD_NBUF * BUF1, s, q, k, v, go, dk, dv, lse, delta, T, H,
                      scale, scale * LOG2E);
   TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(attn_bwd_dq_kernel<D>, dim3(T / 128, B * H), dim3(256), 2 * BUF2, s, q, k, v, go, dq, lse, delta, T, H, scale,
+  hipLaunchKernelGGL(attn_bwd_dq_kernel<D>, dim3(T / 128, B * H), dim3(256), TFB_BWD_NBUF * BUF2, s, q, k, v, go, dq, lse, delta, T, H, scale,
                      scale * LOG2E);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
