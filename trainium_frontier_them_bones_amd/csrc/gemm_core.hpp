@@ -1,29 +1,28 @@
 // MFMA GEMM core for gfx950: D[p][q] = sum_k P[p][k] * Q[q][k], fp32 accumulation.
 //
-// One workgroup of WP x WQ wavefronts owns a BP x BQ output tile. Both operand tiles are
-// staged in LDS as [row][128 bytes of k + 16 bytes of pad], the eight 16-byte chunks of a row
-// XOR-swizzled by (row / 8) mod 8. With the measured bank behaviour of gfx950's LDS (32 banks
-// of 4 bytes; 128-bit accesses resolved per 8 consecutive lanes, 64-bit accesses per 16) the
-// 144-byte stride makes the 128-bit fragment reads (8 consecutive rows, one chunk) conflict-free,
-// and the swizzle does the same for the 64-bit transposing writes (8 rows that are 8 apart times
-// two adjacent k-groups per 16 lanes) while global loads stay 128-byte coalesced. Staging is
-// double-buffered (NBUF 2: the
-// next k-tile's global loads are in flight while the MFMAs of the current one run, one barrier
-// per k-tile) or single-buffered (NBUF 1: half the LDS, two barriers, more workgroups per CU).
-// The P tile feeds the MFMA A operand (rows), the Q tile the B operand (columns), so a lane
-// ends up holding D[p .. p+3][q] for four consecutive p: callers put the dimension that is
-// contiguous in the output on the P side.
+// One workgroup of WP x WQ wavefronts owns a BP x BQ output tile; a wavefront owns TP x TQ MFMA tiles of 32 x 32.
+// Operand tiles (128 bytes of k per row: 64 bf16 or 128 fp8) go from global memory straight into LDS with
+// global_load_lds_dwordx4 (no staging registers, no VALU work): one instruction moves 1 KB, lane l filling bytes
+// 16 l .. 16 l + 15, so the LDS layout is chosen by which 16-byte global chunk each lane fetches:
+//   K_CONTIG  [rows][K]:  LDS row = 128 bytes of k, chunk c of row r at slot c ^ ((r + r / 8) & 7). The 128-bit
+//             fragment reads of 16 consecutive rows then fall on 16 different 16-byte bank groups (LDS here has
+//             64 banks of 4 bytes, measured 256 B/clk for ds_read_b128).
+//   K_STRIDED [K][rows]:  (bf16) LDS row = one k with the tile's rows contiguous, 16-byte chunk c of k-row k at slot
+//             c ^ (4 (k & 3)); fragments are fetched with ds_read_b64_tr_b16, whose 16-lane transpose hands lane i
+//             four consecutive k of row i when lane j points at (k0 + j / 4, row0 + 4 (j % 4)).
+// Two LDS buffers (separate __shared__ objects, so the compiler can tell a fragment read of one from the loads in
+// flight into the other and does not wait for them), loads of k-tile t+1 in flight during the MFMAs of tile t, one
+// barrier per k-tile, fragments of k-step s+1 requested between the MFMAs of step s.
+// The P tile feeds the MFMA A operand (rows), the Q tile the B operand (columns), so a lane ends up holding
+// D[p .. p+3][q] for four consecutive p: callers put the dimension that is contiguous in the output on the P side.
 //
-// Epilogues: "staged" (default) - each wavefront passes its accumulators through its own LDS
-// slice, 32 output rows at a time, and every lane then owns 8 consecutive p of one q, so global
-// reads/writes of the epilogue are 128-bit and coalesced along the output rows; or "tile" (kTileEpilogue) - the functor gets the raw
-// accumulator registers (used when the epilogue reduces along p in registers).
+// Epilogues: "staged" (default) - each wavefront passes its accumulators through its own LDS slice, 32 output rows
+// at a time, and every lane then owns 8 consecutive p of one q, so global reads/writes of the epilogue are 128-bit
+// and coalesced along the output rows; or "tile" (kTileEpilogue) - the functor gets the raw accumulator registers
+// (used when the epilogue reduces along p in registers).
 //
-// Element types: bf16 (v_mfma_f32_32x32x16_bf16, 64 k per tile) or OCP fp8
-// (v_mfma_scale_f32_32x32x64_f8f6f4 with unit scales, 128 k per tile, e4m3/e5m2 per side).
-// Operand layouts: K_CONTIG = [rows][K] (k contiguous); K_STRIDED = [K][rows] (bf16 only,
-// transposed on the way into LDS through 4k x 8row register micro-blocks), which is what
-// the weight-gradient GEMMs (contraction over tokens) read.
+// Element types: bf16 (v_mfma_f32_32x32x16_bf16) or OCP fp8 (v_mfma_scale_f32_32x32x64_f8f6f4 with unit scales,
+// e4m3/e5m2 per side; k-contiguous only).
 #pragma once
 #include <type_traits>
 
@@ -31,7 +30,6 @@
 
 #define TFB_K_CONTIG 0
 #define TFB_K_STRIDED 1
-#define TFB_LDS_ROW 144  // 128 bytes of k + 16 bytes of pad
 
 struct GemmOperand {
   const uint8_t* base;
@@ -49,131 +47,158 @@ struct GemmArgs {
   const int* k_seg;      // [groups + 1] k offsets in elements: group = blockIdx.y contracts over k_seg[g] .. k_seg[g+1]
 };
 
+// Operand pre-operation, applied to a fragment (8 bf16 along k of one row) on its way into the MFMA.
 struct LoadIdentity {
-  __device__ __forceinline__ u32x4 operator()(u32x4 v) const { return v; }
+  template <class T>
+  __device__ __forceinline__ T operator()(T v) const { return v; }
 };
 
-// Byte offset of 16-byte chunk `chunk` of row `row` in a staged tile.
-__device__ __forceinline__ int lds_off(int row, int chunk) {
-  return row * TFB_LDS_ROW + (((chunk ^ (row >> 3)) & 7) << 4);
-}
+typedef __attribute__((address_space(3))) void tfb_lds_void_t;
+typedef const __attribute__((address_space(1))) void tfb_glb_void_t;
+typedef short tfb_s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) tfb_s16x4 tfb_lds_s16x4_t;
 
-template <int BP_, int BQ_, int WP_, int WQ_, int ES_, int LAYP_, int LAYQ_, int FMTP_ = 0, int FMTQ_ = 0, int NBUF_ = 2>
+template <int BP_, int BQ_, int WP_, int WQ_, int ES_, int LAYP_, int LAYQ_, int FMTP_ = 0, int FMTQ_ = 0, int OCC_ = 0>
 struct GemmCfg {
-  static constexpr int BP = BP_, BQ = BQ_, WP = WP_, WQ = WQ_, ES = ES_, NBUF = NBUF_;
+  static constexpr int BP = BP_, BQ = BQ_, WP = WP_, WQ = WQ_, ES = ES_;
   static constexpr int LAYP = LAYP_, LAYQ = LAYQ_, FMTP = FMTP_, FMTQ = FMTQ_;
-  static constexpr int NT = WP * WQ * 64;
+  static constexpr int NW = WP * WQ, NT = NW * 64;
   static constexpr int TP = BP / WP / 32, TQ = BQ / WQ / 32;
-  static constexpr int BK = 128 / ES;  // elements of k per tile
-  static constexpr int TILE_BYTES = (BP + BQ) * TFB_LDS_ROW;
-  static constexpr int STAGE_LD = TP * 32 + 4;  // floats per staged row: a wavefront's 32 x (TP*32) slice
-  static constexpr int STAGE_BYTES = WP * WQ * 32 * STAGE_LD * 4;
-  static constexpr int LDS_BYTES = NBUF * TILE_BYTES > STAGE_BYTES ? NBUF * TILE_BYTES : STAGE_BYTES;
+  static constexpr int BK = 128 / ES;                  // elements of k per tile
+  static constexpr int STAGE_BYTES = (BP + BQ) * 128;  // one k-tile of both operands
+  // epilogue staging: a wavefront's slice is 32 rows x (ETP * 32) floats (+ 4 of pad); ETP of the TP tiles per pass
+  static constexpr int ETP = (TP >= 2 && NW * 32 * (TP * 32 + 4) * 4 > 72 * 1024) ? TP / 2 : TP;
+  static constexpr int STAGE_LD = ETP * 32 + 4;
+  static constexpr int EPI_BYTES = NW * 32 * STAGE_LD * 4;
+  static constexpr int BUF0_BYTES = STAGE_BYTES > EPI_BYTES ? STAGE_BYTES : EPI_BYTES;
+  static constexpr int LDS_BYTES = BUF0_BYTES + STAGE_BYTES;
+  // wavefronts per SIMD the kernel is compiled for: two workgroups per CU when registers and LDS allow it
+  static constexpr int OCC = OCC_ > 0 ? OCC_ : ((NT <= 256 && 2 * LDS_BYTES <= 160 * 1024 && TP * TQ <= 4) ? 2 : 1);
   static_assert(ES == 1 || ES == 2, "fp8 or bf16");
-  static_assert(NBUF == 1 || NBUF == 2, "single or double buffering");
   static_assert(ES == 2 || (LAYP == TFB_K_CONTIG && LAYQ == TFB_K_CONTIG), "fp8 operands are k-contiguous");
-  static_assert((BP * 8) % NT == 0 && (BQ * 8) % NT == 0, "tile rows vs threads");
+  static_assert(NW >= 4 && (NW & (NW - 1)) == 0, "4, 8 or 16 wavefronts");
+  static_assert((BP / 8) % NW == 0 && (BQ / 8) % NW == 0, "1 KB load instructions vs wavefronts");
+  static_assert(LAYP == TFB_K_CONTIG || BP == 128 || BP == 256, "K_STRIDED tiles are 128 or 256 rows");
+  static_assert(LAYQ == TFB_K_CONTIG || BQ == 128 || BQ == 256, "K_STRIDED tiles are 128 or 256 rows");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS");
 };
 
-// ---- global -> register -> LDS staging of one operand tile ---------------------------------
-template <int ROWS, int NT, int LAY>
-struct TileLoader;
+// ---- global -> LDS (one operand tile, this wavefront's share) ---------------------------------------------------
+template <int ROWS, int NW, int LAY>
+struct TileDma;
 
-template <int ROWS, int NT>
-struct TileLoader<ROWS, NT, TFB_K_CONTIG> {
-  static constexpr int N = ROWS * 8 / NT;
-  u32x4 g[N];
-  __device__ __forceinline__ void load(const GemmOperand& o, long row0, long kbyte0, int tid) {
+template <int ROWS, int NW>
+struct TileDma<ROWS, NW, TFB_K_CONTIG> {
+  static constexpr int NI = ROWS / 8 / NW;            // instructions per wavefront: 8 rows x 128 bytes each
+  static constexpr int NV = NW >= 8 ? 1 : 8 / NW;     // distinct per-lane offsets over the instructions
+  const uint8_t* base;  // wavefront-uniform
+  long step;            // bytes between this wavefront's consecutive instructions
+  uint32_t voff[NV];
+  __device__ __forceinline__ void init(const GemmOperand& o, long row0, long k0_bytes, int wave, int lane) {
+    const int lrow = lane >> 3;
+    base = o.base + (row0 + wave * 8) * o.ld + k0_bytes;
+    step = 8L * NW * o.ld;
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-      int c = tid + i * NT;
-      int row = c >> 3, cc = c & 7;
-      g[i] = *(const u32x4*)(o.base + (row0 + row) * o.ld + kbyte0 + cc * 16);
+    for (int v = 0; v < NV; ++v) {
+      // rows 8 g .. 8 g + 7 with g = i * NW + wave; slot (lane & 7) of row r holds chunk slot ^ ((r + g) & 7)
+      const int ch = (lane & 7) ^ ((lrow + v * NW + wave) & 7);
+      voff[v] = (uint32_t)(lrow * o.ld + ch * 16);
     }
   }
-  template <class Pre>
-  __device__ __forceinline__ void store(uint8_t* lds, int tid, const Pre& pre) {
+  // k-tile t of the split (128 bytes of k further per tile)
+  __device__ __forceinline__ void issue(uint8_t* lds, int t, int wave) const {
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-      int c = tid + i * NT;
-      int row = c >> 3, cc = c & 7;
-      *(u32x4*)(lds + lds_off(row, cc)) = pre(g[i]);
-    }
+    for (int i = 0; i < NI; ++i)
+      __builtin_amdgcn_global_load_lds((tfb_glb_void_t*)(base + i * step + (long)t * 128 + (size_t)voff[i % NV]),
+                                       (tfb_lds_void_t*)(lds + (i * NW + wave) * 1024), 16, 0, 0);
   }
 };
 
-template <int ROWS, int NT>
-struct TileLoader<ROWS, NT, TFB_K_STRIDED> {
-  // bf16 only: 64 k x ROWS tile, micro-blocks of 4 k x 8 rows
-  static constexpr int N = ROWS * 2 / NT;
-  static_assert((ROWS * 2) % NT == 0 && N >= 1 && ROWS % 64 == 0, "K_STRIDED tile rows vs threads");
-  u32x4 g[N][4];
-  __device__ __forceinline__ void load(const GemmOperand& o, long row0, long kbyte0, int tid) {
-    const long k0 = kbyte0 >> 1;
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-      int mb = tid + i * NT;
-      // 16 consecutive lanes = 8 row groups x 2 adjacent k groups: 128-byte coalesced loads, conflict-free writes
-      int hi = mb >> 4;
-      int rg = (mb & 7) + 8 * (hi % (ROWS / 64)), kg = ((mb >> 3) & 1) + 2 * (hi / (ROWS / 64));
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        g[i][j] = *(const u32x4*)(o.base + (k0 + 4 * kg + j) * o.ld + (row0 + 8 * rg) * 2);
-    }
+template <int ROWS, int NW>
+struct TileDma<ROWS, NW, TFB_K_STRIDED> {
+  static constexpr int LPR = ROWS / 8;       // lanes (16-byte chunks) per k-row
+  static constexpr int RPI = 64 / LPR;       // k-rows per instruction
+  static constexpr int NI = ROWS / 8 / NW;   // 64 k-rows / RPI / NW
+  static_assert((NW * RPI) % 4 == 0, "k & 3 must not depend on the instruction index");
+  const uint8_t* base;
+  long step, tstep;
+  uint32_t voff;
+  __device__ __forceinline__ void init(const GemmOperand& o, long row0, long k0_bytes, int wave, int lane) {
+    const int kl = lane / LPR, slot = lane % LPR;
+    const long k0 = k0_bytes >> 1;  // elements
+    base = o.base + (k0 + (long)wave * RPI) * o.ld + row0 * 2;
+    step = (long)NW * RPI * o.ld;
+    tstep = 64 * o.ld;
+    const int k = wave * RPI + kl;  // k & 3 of the k-row this lane fills, the same for every instruction
+    voff = (uint32_t)(kl * o.ld + ((slot ^ (4 * (k & 3))) * 16));
   }
-  template <class Pre>
-  __device__ __forceinline__ void store(uint8_t* lds, int tid, const Pre& pre) {
+  __device__ __forceinline__ void issue(uint8_t* lds, int t, int wave) const {
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-      int mb = tid + i * NT;
-      int hi = mb >> 4;
-      int rg = (mb & 7) + 8 * (hi % (ROWS / 64)), kg = ((mb >> 3) & 1) + 2 * (hi / (ROWS / 64));
-      u32x4 v0 = pre(g[i][0]), v1 = pre(g[i][1]), v2 = pre(g[i][2]), v3 = pre(g[i][3]);
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        // rows 2w (low halves) and 2w+1 (high halves) of the micro-block: 4 consecutive k each
-        u32x2 lo, hi;
-        lo.x = __builtin_amdgcn_perm(v1[w], v0[w], 0x05040100u);
-        lo.y = __builtin_amdgcn_perm(v3[w], v2[w], 0x05040100u);
-        hi.x = __builtin_amdgcn_perm(v1[w], v0[w], 0x07060302u);
-        hi.y = __builtin_amdgcn_perm(v3[w], v2[w], 0x07060302u);
-        const int r0 = 8 * rg + 2 * w;
-        *(u32x2*)(lds + lds_off(r0, kg >> 1) + (kg & 1) * 8) = lo;
-        *(u32x2*)(lds + lds_off(r0 + 1, kg >> 1) + (kg & 1) * 8) = hi;
-      }
-    }
+    for (int i = 0; i < NI; ++i)
+      __builtin_amdgcn_global_load_lds((tfb_glb_void_t*)(base + i * step + t * tstep + (size_t)voff),
+                                       (tfb_lds_void_t*)(lds + (i * NW + wave) * 1024), 16, 0, 0);
   }
 };
 
-// ---- MFMA fragments ------------------------------------------------------------------------
-template <int ES>
-struct Frag;
-template <>
-struct Frag<2> {
-  bf16x8 v;
-  static constexpr int KSTEPS = 4;  // 4 x 16 bf16 per 128-byte tile row
-  __device__ __forceinline__ void read(const uint8_t* lds, int row, int s, int h) {
-    v = *(const bf16x8*)(lds + lds_off(row, 2 * s + h));
+// ---- LDS -> MFMA fragments ---------------------------------------------------------------------------------------
+// Per-lane addressing of one operand: off(i, s) = byte offset of the lane's fragment of MFMA tile i, k-step s.
+template <int ROWS, int ES, int LAY>
+struct FragReader;
+
+template <int ROWS>
+struct FragReader<ROWS, 2, TFB_K_CONTIG> {
+  static constexpr int KSTEPS = 4;
+  typedef bf16x8 frag_t;
+  int row, lh;
+  __device__ __forceinline__ void init(int wave_row0, int lane) { row = wave_row0 + (lane & 31); lh = lane >> 5; }
+  __device__ __forceinline__ frag_t read(const uint8_t* lds, int i, int s) const {
+    const int r = row + 32 * i;
+    return *(const bf16x8*)(lds + r * 128 + ((((2 * s + lh) ^ (r + (r >> 3))) & 7) << 4));
   }
 };
-template <>
-struct Frag<1> {
-  i32x8 v;
-  static constexpr int KSTEPS = 2;  // 2 x 64 fp8 per 128-byte tile row
-  __device__ __forceinline__ void read(const uint8_t* lds, int row, int s, int h) {
-    i32x4 a = *(const i32x4*)(lds + lds_off(row, 4 * s + 2 * h));
-    i32x4 b = *(const i32x4*)(lds + lds_off(row, 4 * s + 2 * h + 1));
-    v = i32x8{a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+template <int ROWS>
+struct FragReader<ROWS, 1, TFB_K_CONTIG> {
+  static constexpr int KSTEPS = 2;
+  typedef i32x8 frag_t;
+  int row, lh;
+  __device__ __forceinline__ void init(int wave_row0, int lane) { row = wave_row0 + (lane & 31); lh = lane >> 5; }
+  __device__ __forceinline__ frag_t read(const uint8_t* lds, int i, int s) const {
+    const int r = row + 32 * i, f = r + (r >> 3);
+    const i32x4 a = *(const i32x4*)(lds + r * 128 + ((((4 * s + 2 * lh) ^ f) & 7) << 4));
+    const i32x4 b = *(const i32x4*)(lds + r * 128 + ((((4 * s + 2 * lh + 1) ^ f) & 7) << 4));
+    return i32x8{a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+  }
+};
+template <int ROWS>
+struct FragReader<ROWS, 2, TFB_K_STRIDED> {
+  static constexpr int KSTEPS = 4;
+  typedef bf16x8 frag_t;
+  static constexpr int PITCH = ROWS * 2;
+  int wave_row0, lane;
+  __device__ __forceinline__ void init(int wave_row0_, int lane_) { wave_row0 = wave_row0_; lane = lane_; }
+  __device__ __forceinline__ frag_t read(const uint8_t* lds, int i, int s) const {
+    // 16-lane group g4: rows 16 (g4 & 1) .. + 15 of the MFMA tile, k-group g4 >> 1; lane j of the group points at
+    // k-row j / 4 (of four consecutive k), rows 4 (j % 4) .. + 3
+    const int g4 = lane >> 4, j = lane & 15;
+    const int p = wave_row0 + 32 * i + 16 * (g4 & 1) + 4 * (j & 3);
+    const int kq = j >> 2;  // = k & 3
+    const int k = 16 * s + 8 * (g4 >> 1) + kq;
+    const int off = k * PITCH + ((((p >> 3) ^ (4 * kq)) << 4) | ((p & 4) << 1));
+    const tfb_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tfb_lds_s16x4_t*)(lds + off));
+    const tfb_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tfb_lds_s16x4_t*)(lds + off + 4 * PITCH));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    const s16x8 v = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    return __builtin_bit_cast(bf16x8, v);
   }
 };
 
-template <int ES, int FMTP, int FMTQ>
-__device__ __forceinline__ f32x16 mfma32(const Frag<ES>& a, const Frag<ES>& b, f32x16 c) {
+template <int ES, int FMTP, int FMTQ, class FA, class FB>
+__device__ __forceinline__ f32x16 mfma32(const FA& a, const FB& b, f32x16 c) {
   if constexpr (ES == 2) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   } else {
     // formats: 0 = e4m3, 1 = e5m2; E8M0 scale byte 127 = 2^0
-    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a.v, b.v, c, FMTP, FMTQ, 0, 127, 0, 127);
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, FMTP, FMTQ, 0, 127, 0, 127);
   }
 }
 
@@ -203,12 +228,12 @@ struct has_tile_epilogue<T, std::void_t<decltype(T::kTileEpilogue)>> : std::true
 // Epi: either  __device__ void operator()(int p, int q, const float (&v)[8], int split)  with v = D[p..p+7][q], p % 8 == 0,
 // or (with a static member kTileEpilogue)  __device__ void tile(acc, pw, qw, lr, lh, tile_id, split).
 template <class Cfg, class PreP, class PreQ, class Epi>
-__global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, PreQ preq, Epi epi_in) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  constexpr int BP = Cfg::BP, BQ = Cfg::BQ, NT = Cfg::NT, TP = Cfg::TP, TQ = Cfg::TQ, ES = Cfg::ES;
-  constexpr int BUF = Cfg::TILE_BYTES;
+__global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, PreP prep, PreQ preq, Epi epi_in) {
+  constexpr int BP = Cfg::BP, BQ = Cfg::BQ, NW = Cfg::NW, TP = Cfg::TP, TQ = Cfg::TQ, ES = Cfg::ES;
+  __shared__ __attribute__((aligned(1024))) uint8_t buf0[Cfg::BUF0_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t buf1[Cfg::STAGE_BYTES];
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int wp = wave % Cfg::WP, wq = wave / Cfg::WP;
   const int lr = lane & 31, lh = lane >> 5;
 
@@ -229,9 +254,18 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, Pr
     a.nkt = (int)((k1 - k0) * ES / 128);  // may be 0: the accumulators stay zero and are still written
   }
   const Epi epi = epi_for_group(epi_in, group);
+  const int nkt = a.nkt;
 
-  TileLoader<BP, NT, Cfg::LAYP> lp;
-  TileLoader<BQ, NT, Cfg::LAYQ> lq;
+  TileDma<BP, NW, Cfg::LAYP> dp;
+  TileDma<BQ, NW, Cfg::LAYQ> dq;
+  dp.init(a.P, p0, kt0 * 128, wave, lane);
+  dq.init(a.Q, q0, kt0 * 128, wave, lane);
+  typedef FragReader<BP, ES, Cfg::LAYP> RP;
+  typedef FragReader<BQ, ES, Cfg::LAYQ> RQ;
+  RP rp;
+  RQ rq;
+  rp.init(wp * (TP * 32), lane);
+  rq.init(wq * (TQ * 32), lane);
 
   f32x16 acc[TP][TQ];
 #pragma unroll
@@ -241,87 +275,96 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_kernel(GemmArgs a, PreP prep, Pr
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  if (a.nkt > 0) {
-    lp.load(a.P, p0, kt0 * 128, tid);
-    lq.load(a.Q, q0, kt0 * 128, tid);
-    lp.store(smem, tid, prep);
-    lq.store(smem + BP * TFB_LDS_ROW, tid, preq);
-  }
-  __syncthreads();
-
-  for (int t = 0; t < a.nkt; ++t) {
-    const uint8_t* sp = smem + (Cfg::NBUF == 2 ? (t & 1) * BUF : 0);
-    const uint8_t* sq = sp + BP * TFB_LDS_ROW;
-    const bool more = (t + 1 < a.nkt);
-    if (more) {
-      lp.load(a.P, p0, (kt0 + t + 1) * 128, tid);
-      lq.load(a.Q, q0, (kt0 + t + 1) * 128, tid);
-    }
-    {
-      // fragments of k-step s+1 are requested before the MFMAs of step s are issued
-      constexpr int KS = Frag<ES>::KSTEPS;
-      Frag<ES> fa[2][TP], fb[2][TQ];
+  auto issue = [&](uint8_t* buf, int t) {
+    dp.issue(buf, t, wave);
+    dq.issue(buf + BP * 128, t, wave);
+  };
+  auto compute = [&](const uint8_t* buf) {
+    const uint8_t* sp = buf;
+    const uint8_t* sq = buf + BP * 128;
+    constexpr int KS = RP::KSTEPS;
+    constexpr int NR = TP + TQ, NM = TP * TQ;
+    typename RP::frag_t fa[2][TP];
+    typename RQ::frag_t fb[2][TQ];
+    // fragments are requested in the order the MFMAs below first need them: P tile 0, all Q tiles, P tiles 1..
+    auto rd = [&](int nb, int s, int r) {
+      if (r == 0) fa[nb][0] = prep(rp.read(sp, 0, s));
+      else if (r <= TQ) fb[nb][r - 1] = preq(rq.read(sq, r - 1, s));
+      else fa[nb][r - TQ] = prep(rp.read(sp, r - TQ, s));
+    };
 #pragma unroll
-      for (int i = 0; i < TP; ++i) fa[0][i].read(sp, wp * (TP * 32) + i * 32 + lr, 0, lh);
+    for (int r = 0; r < NR; ++r) rd(0, 0, r);
 #pragma unroll
-      for (int j = 0; j < TQ; ++j) fb[0][j].read(sq, wq * (TQ * 32) + j * 32 + lr, 0, lh);
+    for (int s = 0; s < KS; ++s) {
+      int m = 0, r = 0;
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        if (s + 1 < KS) {
+      for (int i = 0; i < TP; ++i)
 #pragma unroll
-          for (int i = 0; i < TP; ++i) fa[(s + 1) & 1][i].read(sp, wp * (TP * 32) + i * 32 + lr, s + 1, lh);
-#pragma unroll
-          for (int j = 0; j < TQ; ++j) fb[(s + 1) & 1][j].read(sq, wq * (TQ * 32) + j * 32 + lr, s + 1, lh);
+        for (int j = 0; j < TQ; ++j) {
+          acc[i][j] = mfma32<ES, Cfg::FMTP, Cfg::FMTQ>(fa[s & 1][i], fb[s & 1][j], acc[i][j]);
+          ++m;
+          if (s + 1 < KS) {
+            // the next k-step's fragment reads are spread evenly between this step's MFMAs
+            while (r < NR && r * NM < m * NR) {
+              rd((s + 1) & 1, s + 1, r);
+              ++r;
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          }
         }
-#pragma unroll
-        for (int i = 0; i < TP; ++i)
-#pragma unroll
-          for (int j = 0; j < TQ; ++j)
-            acc[i][j] = mfma32<ES, Cfg::FMTP, Cfg::FMTQ>(fa[s & 1][i], fb[s & 1][j], acc[i][j]);
-      }
     }
-    if (Cfg::NBUF == 1) __syncthreads();
-    if (more) {
-      uint8_t* np_ = smem + (Cfg::NBUF == 2 ? ((t + 1) & 1) * BUF : 0);
-      lp.store(np_, tid, prep);
-      lq.store(np_ + BP * TFB_LDS_ROW, tid, preq);
-    }
+  };
+
+  if (nkt > 0) issue(buf0, 0);
+  __syncthreads();
+  for (int t = 0; t + 2 <= nkt; t += 2) {
+    issue(buf1, t + 1);
+    compute(buf0);
+    __syncthreads();
+    issue(buf0, t + 2 < nkt ? t + 2 : nkt - 1);  // (the last pair re-fetches a tile nobody reads: no branch in the loop)
+    compute(buf1);
     __syncthreads();
   }
+  if (nkt & 1) compute(buf0);
+  __syncthreads();
 
   const int pw = wp * (TP * 32), qw = wq * (TQ * 32);  // wavefront's origin inside the tile
   if constexpr (has_tile_epilogue<Epi>::value) {
     // whole-accumulator epilogue: acc[i][j][4*jj + e] = D[pw + 32 i + 8 jj + 4 lh + e][qw + 32 j + lr]
     epi.tile(acc, (int)p0 + pw, (int)q0 + qw, lr, lh, lid, (int)blockIdx.z);
   } else {
-    // (the loop's last barrier has passed: every wavefront is done reading the operand tiles.) Each wavefront stages
+    // (the barrier above has passed: every wavefront is done reading the operand tiles.) Each wavefront stages
     // 32 output rows at a time through its own LDS slice (no workgroup barrier: LDS operations of one wavefront
     // execute in order) and then finishes them as 8-element chunks, a row's chunks on consecutive lanes.
-    constexpr int SLD = Cfg::STAGE_LD;
-    float* stage = (float*)smem + wave * (32 * SLD);
-    constexpr int CPR = TP * 4;  // 8-element chunks per staged row
+    constexpr int SLD = Cfg::STAGE_LD, ETP = Cfg::ETP;
+    float* stage = (float*)buf0 + wave * (32 * SLD);
+    constexpr int CPR = ETP * 4;  // 8-element chunks per staged row
 #pragma unroll
     for (int j = 0; j < TQ; ++j) {
 #pragma unroll
-      for (int i = 0; i < TP; ++i)
+      for (int i0 = 0; i0 < TP; i0 += ETP) {
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          f32x4 v = {acc[i][j][jj * 4 + 0], acc[i][j][jj * 4 + 1], acc[i][j][jj * 4 + 2], acc[i][j][jj * 4 + 3]};
-          *(f32x4*)(stage + lr * SLD + i * 32 + jj * 8 + lh * 4) = v;
+        for (int i = 0; i < ETP; ++i)
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj) {
+            f32x4 v = {acc[i0 + i][j][jj * 4 + 0], acc[i0 + i][j][jj * 4 + 1], acc[i0 + i][j][jj * 4 + 2],
+                       acc[i0 + i][j][jj * 4 + 3]};
+            *(f32x4*)(stage + lr * SLD + i * 32 + jj * 8 + lh * 4) = v;
+          }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int k = 0; k < 32 * CPR / 64; ++k) {
+          // 8 consecutive lanes take 4 chunks of each of two rows: their 128-bit reads fall on 8 different bank groups
+          const int rest = (lane >> 3) + k * 8;
+          const int row = 2 * (rest / (CPR / 4)) + ((lane >> 2) & 1);
+          const int pc = (4 * (rest % (CPR / 4)) + (lane & 3)) * 8;
+          f32x4 lo = *(const f32x4*)(stage + row * SLD + pc);
+          f32x4 hi = *(const f32x4*)(stage + row * SLD + pc + 4);
+          const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          epi((int)p0 + pw + i0 * 32 + pc, (int)q0 + qw + j * 32 + row, v, (int)blockIdx.z);
         }
-      __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int k = 0; k < 32 * CPR / 64; ++k) {
-        // 8 consecutive lanes take 4 chunks of each of two rows: their 128-bit reads fall on 8 different bank groups
-        const int rest = (lane >> 3) + k * 8;
-        const int row = 2 * (rest / (CPR / 4)) + ((lane >> 2) & 1);
-        const int pc = (4 * (rest % (CPR / 4)) + (lane & 3)) * 8;
-        f32x4 lo = *(const f32x4*)(stage + row * SLD + pc);
-        f32x4 hi = *(const f32x4*)(stage + row * SLD + pc + 4);
-        const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        epi((int)p0 + pw + pc, (int)q0 + qw + j * 32 + row, v, (int)blockIdx.z);
+        __builtin_amdgcn_wave_barrier();
       }
-      __builtin_amdgcn_wave_barrier();
     }
   }
 }
@@ -351,19 +394,14 @@ static int gemm_launch(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes
 // Launch with prepared arguments; groups_y > 1 only with a.k_seg.
 template <class Cfg, class PreP, class PreQ, class Epi>
 static int gemm_launch_args(GemmArgs a, int groups_y, int splits, PreP prep, PreQ preq, Epi epi, hipStream_t stream) {
-  auto kern = gemm_kernel<Cfg, PreP, PreQ, Epi>;
-  static bool attr_set = false;  // per template instantiation
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES) != hipSuccess)
-      return TFB_ERR_LAUNCH;
-    attr_set = true;
-  }
+  // the per-lane part of a load address is a 32-bit offset: 8 rows (K_CONTIG) or 8 k-rows (K_STRIDED) of the operand
+  if (a.P.ld <= 0 || a.Q.ld <= 0 || a.P.ld > (1L << 28) || a.Q.ld > (1L << 28)) return TFB_ERR_SHAPE;
+  if (((uintptr_t)a.P.base | (uintptr_t)a.Q.base | (uintptr_t)a.P.ld | (uintptr_t)a.Q.ld) & 15) return TFB_ERR_ARG;
   dim3 grid(a.ntp * (a.nq / Cfg::BQ), groups_y, splits);
-  hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, a, prep, preq, epi);
+  hipLaunchKernelGGL((gemm_kernel<Cfg, PreP, PreQ, Epi>), grid, dim3(Cfg::NT), 0, stream, a, prep, preq, epi);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
-
 // ---- shared epilogue helpers -----------------------------------------------------------------
 __device__ __forceinline__ u32x4 pack8bf(const float (&v)[8]) {
   u32x4 o = {pack2bf(v[0], v[1]), pack2bf(v[2], v[3]), pack2bf(v[4], v[5]), pack2bf(v[6], v[7])};

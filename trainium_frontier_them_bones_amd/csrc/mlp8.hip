@@ -357,16 +357,13 @@ struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*
   }
 };
 
-// h = bf16(r^2) applied to the 8 bf16 of a 128-bit load (the dW_proj GEMM reads r, not h).
+// h = bf16(r^2) applied to a fragment of 8 bf16 on its way into the MFMA (the dW_proj GEMM reads r, not h).
 struct LoadSquare {
-  __device__ __forceinline__ u32x4 operator()(u32x4 v) const {
-    u32x4 o;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      float a = bflo(v[k]), b = bfhi(v[k]);
-      o[k] = pack2bf(a * a, b * b);
-    }
-    return o;
+  __device__ __forceinline__ bf16x8 operator()(bf16x8 v) const {
+    typedef float f32x8_t __attribute__((ext_vector_type(8)));
+    f32x8_t f = __builtin_convertvector(v, f32x8_t);
+    f = f * f;
+    return __builtin_convertvector(f, bf16x8);
   }
 };
 
@@ -516,7 +513,8 @@ extern "C" int tfb_mlp_dw_proj(const void* dy, const void* r, void* dw, long M, 
   if (!dy || !r || !dw) return TFB_ERR_ARG;
   if (M <= 0 || M % 64 || d % 128 || F % 128) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
-  using Cfg = GemmCfg<128, 128, 2, 2, 2, TFB_K_STRIDED, TFB_K_STRIDED>;
+  // 4 x 1 wavefronts: each wavefront squares one P fragment per k-step and every element of r is squared once
+  using Cfg = GemmCfg<128, 128, 4, 1, 2, TFB_K_STRIDED, TFB_K_STRIDED>;
   GemmOperand P{(const uint8_t*)r, (long)F * 2}, Q{(const uint8_t*)dy, (long)d * 2};
   const long tiles = (long)(F / 128) * (d / 128);
   const int splits = workspace ? choose_splits(tiles, (int)(M / 64), (long)d * F, workspace_bytes) : 1;
@@ -611,5 +609,6 @@ extern "C" int tfb_moe_dw(const void* dpre, const void* xs, const void* dys, con
   a.nq = d;
   a.ntp = F / 128;
   EpiStoreGrouped e2{EpiStore{dw_proj, (long)F, out_f32, accumulate}, (long)F * d};
-  return gemm_launch_args<Cfg>(a, E, 1, LoadSquare{}, LoadIdentity{}, e2, s);
+  using CfgSq = GemmCfg<128, 128, 4, 1, 2, TFB_K_STRIDED, TFB_K_STRIDED>;
+  return gemm_launch_args<CfgSq>(a, E, 1, LoadSquare{}, LoadIdentity{}, e2, s);
 }
