@@ -79,6 +79,12 @@ int tfb_resmix_bwd(const void* g, const void* x, const void* x0, const void* ab,
 int tfb_embedding_fwd(const void* idx, int idx64, const void* w, void* out, long n, int C, void* stream);
 /* dw_f32[idx[i]] += dy[i] (fp32 atomics). Replaces _emb_bwd_kernel (round1/source/train.py:8303). */
 int tfb_embedding_bwd(const void* idx, int idx64, const void* dy, void* dw_f32, long n, int C, void* stream);
+/* The same sum with the rows grouped by token first (counting sort on the device, then a segmented sum), so that the
+ * frequent tokens of a Zipf batch do not serialize on atomics; idx values must lie in [0, V). scratch: int32
+ * [tfb_embedding_bwd_scratch_ints(n, V)]. Replaces _emb_bwd_kernel (round1/source/train.py:8303). */
+long tfb_embedding_bwd_scratch_ints(long n, int V);
+int tfb_embedding_bwd_grouped(const void* idx, int idx64, const void* dy, void* dw_f32, long n, int C, int V, void* scratch,
+                              void* stream);
 
 /* One AdamW update in place on fp32 p, m, v from g (fp32 if g_f32 else bf16); optional bf16 copy of p.
  * p *= 1 - lr wd; m = lerp(m, g, 1-b1); v = lerp(v, g^2, 1-b2); p -= lr (m / bias1) / (sqrt(v / bias2) + eps).

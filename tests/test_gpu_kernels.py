@@ -131,6 +131,12 @@ def test_relu2_rope_resmix_embedding_bit_exact(ops, dev):
     ops.embedding_bwd(idx.to(dev), dy.to(dev), dw)
     want = torch.zeros(1000, 768).index_add_(0, idx.reshape(-1), dy.float().reshape(-1, 768))
     assert rel_l2(dw, want) < 1e-6
+    # ragged row count, int32 ids, accumulation into a non-zero dW, Zipf-like skew
+    idx2 = (torch.rand(1237, generator=g) ** 4 * 1000).long().clamp_(0, 999)
+    dy2 = torch.randn(1237, 768, generator=g).bfloat16()
+    ops.embedding_bwd(idx2.int().to(dev), dy2.to(dev), dw)
+    want.index_add_(0, idx2, dy2.float())
+    assert rel_l2(dw, want) < 1e-6
 
 
 def test_adamw(ops, dev):

@@ -40,6 +40,8 @@ SIGNATURES = {
     "tfb_resmix_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _vp],
     "tfb_embedding_fwd": [_vp, _i, _vp, _vp, _l, _i, _vp],
     "tfb_embedding_bwd": [_vp, _i, _vp, _vp, _l, _i, _vp],
+    "tfb_embedding_bwd_scratch_ints": [_l, _i],
+    "tfb_embedding_bwd_grouped": [_vp, _i, _vp, _vp, _l, _i, _i, _vp, _vp],
     "tfb_adamw": [_vp, _vp, _i, _vp, _vp, _vp, _l, _f, _f, _f, _f, _f, _f, _f, _vp],
     "tfb_fill_f32": [_vp, _f, _l, _vp],
     "tfb_loss_fwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
@@ -60,7 +62,7 @@ SIGNATURES = {
     "tfb_mlp_dw_proj": [_vp, _vp, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
 }
 
-_LONG_RESULT = {"tfb_mlp8_scale_scratch_floats", "tfb_moe_max_rows"}
+_LONG_RESULT = {"tfb_mlp8_scale_scratch_floats", "tfb_moe_max_rows", "tfb_embedding_bwd_scratch_ints"}
 
 STATUS = {0: "ok", 1: "unsupported shape", 2: "bad argument", 3: "kernel launch failed", 4: "workspace too small"}
 

@@ -168,6 +168,93 @@ __global__ __launch_bounds__(256) void embedding_bwd_kernel(const IDX* __restric
   }
 }
 
+// ---- embedding backward without contended atomics: rows grouped by token (counting sort), then a segmented sum.
+__global__ __launch_bounds__(256) void emb_zero_kernel(int* __restrict__ p, long n) {
+  long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+template <typename IDX>
+__global__ __launch_bounds__(256) void emb_count_kernel(const IDX* __restrict__ idx, int* __restrict__ count, long n) {
+  long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) atomicAdd(count + (long)idx[i], 1);
+}
+// One workgroup: cursor[v] = exclusive prefix sum of count[v] (count is left untouched).
+__global__ __launch_bounds__(1024) void emb_scan_kernel(const int* __restrict__ count, int* __restrict__ cursor, int V) {
+  __shared__ int wsum[16];
+  __shared__ int carry;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) carry = 0;
+  __syncthreads();
+  for (int base = 0; base < V; base += 1024) {
+    const int v = base + tid;
+    const int c = v < V ? count[v] : 0;
+    int x = c;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      int y = __shfl_up(x, o, 64);
+      if (lane >= o) x += y;
+    }
+    if (lane == 63) wsum[wave] = x;
+    __syncthreads();
+    int before = carry;
+    for (int w = 0; w < wave; ++w) before += wsum[w];
+    if (v < V) cursor[v] = before + x - c;
+    __syncthreads();
+    if (tid == 1023) carry = before + x;
+    __syncthreads();
+  }
+}
+template <typename IDX>
+__global__ __launch_bounds__(256) void emb_place_kernel(const IDX* __restrict__ idx, int* __restrict__ cursor,
+                                                       int* __restrict__ order, long n) {
+  long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) order[atomicAdd(cursor + (long)idx[i], 1)] = (int)i;
+}
+// A workgroup sums EMB_SEG consecutive rows of the token-grouped order, thread t owning columns 8t .. 8t+7. A run of
+// equal tokens that lies inside the segment has a single owner and is added with plain loads/stores; the first and the
+// last run may continue in the neighbouring segments and use atomics.
+constexpr int EMB_SEG = 32;
+template <typename IDX>
+__global__ __launch_bounds__(128) void emb_reduce_kernel(const IDX* __restrict__ idx, const int* __restrict__ order,
+                                                        const bf16_t* __restrict__ dy, float* __restrict__ dw, long n, int C) {
+  __shared__ int rows[EMB_SEG];
+  __shared__ int toks[EMB_SEG];
+  const long pos0 = (long)blockIdx.x * EMB_SEG;
+  const int cnt = (int)min((long)EMB_SEG, n - pos0);
+  if (threadIdx.x < cnt) {
+    const int r = order[pos0 + threadIdx.x];
+    rows[threadIdx.x] = r;
+    toks[threadIdx.x] = (int)idx[r];
+  }
+  __syncthreads();
+  const int c = (blockIdx.y * 128 + threadIdx.x) * 8;
+  if (c >= C) return;
+  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  int run_start = 0;
+  for (int i = 0; i < cnt; ++i) {
+    u32x4 u = *(const u32x4*)(dy + (long)rows[i] * C + c);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      acc[2 * k] += bflo(u[k]);
+      acc[2 * k + 1] += bfhi(u[k]);
+    }
+    if (i + 1 == cnt || toks[i + 1] != toks[i]) {
+      float* d = dw + (long)toks[i] * C + c;
+      if (run_start == 0 || i + 1 == cnt) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) atomicAdd(d + k, acc[k]);
+      } else {
+        f32x4 a0 = *(const f32x4*)d, a1 = *(const f32x4*)(d + 4);
+        *(f32x4*)d = f32x4{a0[0] + acc[0], a0[1] + acc[1], a0[2] + acc[2], a0[3] + acc[3]};
+        *(f32x4*)(d + 4) = f32x4{a1[0] + acc[4], a1[1] + acc[5], a1[2] + acc[6], a1[3] + acc[7]};
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) acc[k] = 0.f;
+      run_start = i + 1;
+    }
+  }
+}
+
 struct AdamScalars {
   float lr, wd, omb1, omb2, eps, bias1, bias2;
 };
@@ -283,6 +370,32 @@ extern "C" int tfb_embedding_bwd(const void* idx, int idx64, const void* dy, voi
   int nb = blocks_for(n * (C / 8));
   if (idx64) hipLaunchKernelGGL(embedding_bwd_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, (const bf16_t*)dy, (float*)dw_f32, n, C);
   else hipLaunchKernelGGL(embedding_bwd_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, (const bf16_t*)dy, (float*)dw_f32, n, C);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// Scratch (int32 elements) of tfb_embedding_bwd_grouped.
+extern "C" long tfb_embedding_bwd_scratch_ints(long n, int V) { return 2L * V + n; }
+
+// The same sum as tfb_embedding_bwd, rows grouped by token first: hot tokens (a Zipf batch) no longer serialize on atomics.
+extern "C" int tfb_embedding_bwd_grouped(const void* idx, int idx64, const void* dy, void* dw_f32, long n, int C, int V,
+                                         void* scratch, void* stream) {
+  if (!idx || !dy || !dw_f32 || !scratch) return TFB_ERR_ARG;
+  if (n <= 0 || n > 0x7fffffffL || C <= 0 || C % 8 || V <= 0) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  int* count = (int*)scratch;
+  int* cursor = count + V;
+  int* order = cursor + V;
+  const unsigned nb = (unsigned)((n + 255) / 256);
+  hipLaunchKernelGGL(emb_zero_kernel, dim3((unsigned)((V + 255) / 256)), dim3(256), 0, s, count, (long)V);
+  if (idx64) hipLaunchKernelGGL(emb_count_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, count, n);
+  else hipLaunchKernelGGL(emb_count_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, count, n);
+  hipLaunchKernelGGL(emb_scan_kernel, dim3(1), dim3(1024), 0, s, count, cursor, V);
+  if (idx64) hipLaunchKernelGGL(emb_place_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, cursor, order, n);
+  else hipLaunchKernelGGL(emb_place_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, cursor, order, n);
+  dim3 grid((unsigned)((n + EMB_SEG - 1) / EMB_SEG), (unsigned)((C / 8 + 127) / 128));
+  if (idx64) hipLaunchKernelGGL(emb_reduce_kernel<long>, grid, dim3(128), 0, s, (const long*)idx, order, (const bf16_t*)dy, (float*)dw_f32, n, C);
+  else hipLaunchKernelGGL(emb_reduce_kernel<int>, grid, dim3(128), 0, s, (const int*)idx, order, (const bf16_t*)dy, (float*)dw_f32, n, C);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

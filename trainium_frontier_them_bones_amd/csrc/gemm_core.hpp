@@ -39,7 +39,7 @@ struct GemmOperand {
 struct GemmArgs {
   GemmOperand P, Q;
   int np, nq;   // output extent (multiples of BP / BQ)
-  int nkt;      // k-tiles (128 bytes of k each) per split
+  int nkt;      // k-tiles (128 bytes of k each) in all; split z of gridDim.z takes tiles [z nkt / Z, (z + 1) nkt / Z)
   int ntp;      // tiles along p
   // Grouped (ragged) launches, both optional:
   const int* q_group;    // group id of each q tile (-1: the tile is beyond the ragged extent, the workgroup exits);
@@ -240,7 +240,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   const int lid = xcd_remap(blockIdx.x, gridDim.x);
   const int tile_p = lid % a.ntp, tile_q = lid / a.ntp;
   const long p0 = (long)tile_p * BP, q0 = (long)tile_q * BQ;
-  long kt0 = (long)blockIdx.z * a.nkt;
+  long kt0 = (long)blockIdx.z * a.nkt / gridDim.z;
+  a.nkt = (int)((long)(blockIdx.z + 1) * a.nkt / gridDim.z - kt0);
   int group = 0;
   if (a.q_group) {
     group = a.q_group[tile_q];
@@ -372,18 +373,19 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
 template <class Cfg, class PreP, class PreQ, class Epi>
 static int gemm_launch_args(GemmArgs a, int groups_y, int splits, PreP prep, PreQ preq, Epi epi, hipStream_t stream);
 
-// Host-side launch: np, nq multiples of the tile; kbytes a multiple of 128 * splits.
+// Host-side launch: np, nq multiples of the tile; kbytes a multiple of 128; the k-tiles are dealt to the splits evenly
+// to within one tile.
 template <class Cfg, class PreP, class PreQ, class Epi>
 static int gemm_launch(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes, int splits, PreP prep, PreQ preq,
                        Epi epi, hipStream_t stream) {
   if (np <= 0 || nq <= 0 || kbytes <= 0 || splits <= 0) return TFB_ERR_SHAPE;
-  if (np % Cfg::BP || nq % Cfg::BQ || kbytes % (128L * splits)) return TFB_ERR_SHAPE;
+  if (np % Cfg::BP || nq % Cfg::BQ || kbytes % 128 || splits > kbytes / 128) return TFB_ERR_SHAPE;
   GemmArgs a;
   a.P = P;
   a.Q = Q;
   a.np = np;
   a.nq = nq;
-  a.nkt = (int)(kbytes / 128 / splits);
+  a.nkt = (int)(kbytes / 128);
   a.ntp = np / Cfg::BP;
   a.q_group = nullptr;
   a.p_group_stride = 0;
@@ -505,11 +507,22 @@ static inline int splitk_reduce(const float* ws, void* out, long n, int splits, 
   return TFB_OK;
 }
 
-// How many k-splits a token-contraction GEMM with `tiles` output tiles and `nkt` k-tiles should use.
+// How many k-splits a token-contraction GEMM with `tiles` output tiles and `nkt` k-tiles should use. Cost model in
+// units of one k-tile of one workgroup: rounds over the 512 workgroup slots (256 CUs x 2 resident workgroups) x
+// (k-tiles per split + 10 for prologue and epilogue) + the fp32 partials' round trip through memory (8 bytes per
+// output element and split at ~4 TB/s, one k-tile ~0.7 us).
 static inline int choose_splits(long tiles, int nkt, long out_elems, long ws_bytes) {
-  if (tiles >= 512 || nkt < 32) return 1;
-  int splits = (int)((768 + tiles - 1) / tiles);
-  while (splits > 1 && (nkt % splits != 0 || nkt / splits < 8)) --splits;
-  if ((long)splits * out_elems * 4 > ws_bytes) splits = 1;
-  return splits;
+  if (tiles >= 1024 || nkt < 32) return 1;
+  int best = 1;
+  double best_cost = 1e30;
+  for (int sp = 1; sp <= 32; ++sp) {
+    if (sp > 1 && (nkt / sp < 16 || (long)sp * out_elems * 4 > ws_bytes)) break;
+    const long rounds = (tiles * sp + 511) / 512;
+    const double cost = (double)rounds * ((double)nkt / sp + 10.0) + (sp > 1 ? sp * (double)out_elems * 2e-6 / 0.7 : 0.0);
+    if (cost < best_cost) {
+      best_cost = cost;
+      best = sp;
+    }
+  }
+  return best;
 }

@@ -129,18 +129,22 @@ __global__ __launch_bounds__(256) void row_stats_kernel(const bf16_t* __restrict
   if (threadIdx.x == 0) amax_part[blockIdx.x] = m;
 }
 
-// Column sums of squares of w [rows][cols]: a workgroup owns 512 columns (64 lanes x 8), its 4
-// wavefronts take interleaved rows; amax partial per workgroup.
+// Column sums of squares of w [rows][cols]: a workgroup owns 512 columns (64 lanes x 8) of one slice of the rows
+// (blockIdx.y of COL_SLICES), its 4 wavefronts take interleaved rows; the slices' partial sums go to
+// colss_part [COL_SLICES][cols] and are added in slice order by the scale kernel; amax partial per workgroup.
+constexpr int COL_SLICES = 32;
 __global__ __launch_bounds__(256) void col_stats_kernel(const bf16_t* __restrict__ w, int rows, int cols,
-                                                       float* __restrict__ colss, float* __restrict__ amax_part) {
+                                                       float* __restrict__ colss_part, float* __restrict__ amax_part) {
   __shared__ float red[4];
   __shared__ float acc[4][512];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = blockIdx.x * 512 + lane * 8;
+  const int per = (rows + gridDim.y - 1) / gridDim.y;
+  const int r0 = blockIdx.y * per, r1 = min(rows, r0 + per);
   float ss[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   float m = 0.f;
   if (c < cols) {
-    for (int r = wave; r < rows; r += 4) {
+    for (int r = r0 + wave; r < r1; r += 4) {
       u32x4 u = *(const u32x4*)(w + (long)r * cols + c);
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
@@ -156,9 +160,19 @@ __global__ __launch_bounds__(256) void col_stats_kernel(const bf16_t* __restrict
   m = block_max(m, red);  // contains the barriers that publish acc
   for (int i = threadIdx.x; i < 512; i += 256) {
     int cc = blockIdx.x * 512 + i;
-    if (cc < cols) colss[cc] = acc[0][i] + acc[1][i] + acc[2][i] + acc[3][i];
+    if (cc < cols) colss_part[(long)blockIdx.y * cols + cc] = acc[0][i] + acc[1][i] + acc[2][i] + acc[3][i];
   }
-  if (threadIdx.x == 0) amax_part[blockIdx.x] = m;
+  if (threadIdx.x == 0) amax_part[blockIdx.y * gridDim.x + blockIdx.x] = m;
+}
+
+// colss[c] = sum over the row slices, in slice order
+__global__ __launch_bounds__(256) void col_finish_kernel(const float* __restrict__ part, int n, int slices,
+                                                        float* __restrict__ colss) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float t = 0.f;
+  for (int sl = 0; sl < slices; ++sl) t += part[(long)sl * n + i];
+  colss[i] = t;
 }
 
 __device__ float reduce_max_array(const float* a, int n, float* red) {
@@ -384,7 +398,7 @@ constexpr int AMAX_BLOCKS = 1024;
 }  // namespace
 
 // Scratch the scale kernels need (fp32 elements): partial maxima and the per-row / per-column norms.
-extern "C" long tfb_mlp8_scale_scratch_floats(int F) { return 2L * F + 4L * AMAX_BLOCKS; }
+extern "C" long tfb_mlp8_scale_scratch_floats(int F) { return (2L + COL_SLICES) * F + 4L * AMAX_BLOCKS; }
 
 // row_out: fp32 [16] device. e4m3_limit: 240 reproduces the reference's rows; 448 is the OCP maximum.
 extern "C" int tfb_mlp8_forward_scales(const void* w_fc, const void* w_proj, void* row_out, void* scratch, int F, int d,
@@ -394,17 +408,22 @@ extern "C" int tfb_mlp8_forward_scales(const void* w_fc, const void* w_proj, voi
   hipStream_t s = (hipStream_t)stream;
   float* rowss = (float*)scratch;
   float* colss = rowss + F;
-  float* pa = colss + F;
+  float* colpart = colss + F;
+  float* pa = colpart + (long)COL_SLICES * F;
   float* pb = pa + AMAX_BLOCKS;
   int nfc = (F + 3) / 4;
   if (nfc > AMAX_BLOCKS) nfc = AMAX_BLOCKS;
   int npj = (F + 511) / 512;
   hipLaunchKernelGGL(row_stats_kernel, dim3(nfc), dim3(256), 0, s, (const bf16_t*)w_fc, F, d, rowss, pa);
   TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(col_stats_kernel, dim3(npj), dim3(256), 0, s, (const bf16_t*)w_proj, d, F, colss, pb);
+  int slices = AMAX_BLOCKS / npj < COL_SLICES ? AMAX_BLOCKS / npj : COL_SLICES;
+  if (slices < 1) return TFB_ERR_SHAPE;
+  hipLaunchKernelGGL(col_stats_kernel, dim3(npj, slices), dim3(256), 0, s, (const bf16_t*)w_proj, d, F, colpart, pb);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(col_finish_kernel, dim3((F + 255) / 256), dim3(256), 0, s, colpart, F, slices, colss);
   TFB_LAUNCH_CHECK();
   const float h_bound = (float)(1.3 * (double)d);
-  hipLaunchKernelGGL(forward_scales_kernel, dim3(1), dim3(256), 0, s, rowss, F, pa, nfc, colss, pb, npj, e4m3_limit, h_bound,
+  hipLaunchKernelGGL(forward_scales_kernel, dim3(1), dim3(256), 0, s, rowss, F, pa, nfc, colss, pb, npj * slices, e4m3_limit, h_bound,
                      (float)(1.0 / (double)x_scale), (float*)row_out);
   TFB_LAUNCH_CHECK();
   return TFB_OK;

@@ -348,7 +348,10 @@ def embedding_bwd(idx, dy, dw):
     """dw (fp32 [V, C]) += scatter of dy rows by idx."""
     _chk(dy), _chk(dw, torch.float32)
     idx = idx.contiguous()
-    _lib.call("tfb_embedding_bwd", _p(idx), int(idx.dtype == torch.int64), _p(dy), _p(dw), idx.numel(), dy.shape[-1], _stream())
+    n, V = idx.numel(), dw.shape[0]
+    scr = _scratch(dw.device, _lib.lib().tfb_embedding_bwd_scratch_ints(n, V))  # 4-byte elements, used as int32
+    _lib.call("tfb_embedding_bwd_grouped", _p(idx), int(idx.dtype == torch.int64), _p(dy), _p(dw), n, dy.shape[-1], V,
+              _p(scr), _stream())
     return dw
 
 
