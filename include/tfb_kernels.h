@@ -151,7 +151,7 @@ int tfb_attn_fwd(const void* q, const long* q_strides, const void* k, const long
                  const long* v_strides, void* o, const long* o_strides, void* lse, int B, int H, int T, int D, float scale,
                  void* stream);
 
-/* dq, dk, dv from (q, k, v, o, do, lse); delta fp32 [B*H][T] scratch.
+/* dq, dk, dv from (q, k, v, o, do, lse); delta fp32 [2][B*H][T] scratch.
  * Replaces _attn_bwd_kernel / NkiAttnFn.backward (round1/source/train.py:7591, 8036). */
 int tfb_attn_bwd(const void* q, const long* q_strides, const void* k, const long* k_strides, const void* v,
                  const long* v_strides, const void* o, const long* o_strides, const void* d_o, const long* do_strides,

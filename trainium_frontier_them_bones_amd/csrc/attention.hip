@@ -86,6 +86,11 @@ struct MicroBlock {
   }
 };
 
+// s_waitcnt vmcnt(0) before a main loop: the register fragments loaded from global memory ahead of the loop are then
+// known to have arrived, and the compiler does not repeat (in every iteration, against the tile loads in flight) the
+// waits it would otherwise keep for them.
+__device__ __forceinline__ void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
 // LDS row of a transposed tile: 64 tokens + 8 bytes of pad. With 32 banks and 64-bit accesses resolved per 16 lanes,
@@ -172,6 +177,7 @@ __global__ __launch_bounds__(256, (D == 64 && QG == 1) ? TFB_FWD_WPE : 1) void a
 
   gload(0);
   sstore(smem);
+  wait_all_loads();
   __syncthreads();
 
   for (int t = 0; t < ntiles; ++t) {
@@ -331,6 +337,7 @@ __global__ __launch_bounds__(256, D == 64 ? TFB_DKDV_WPE : 1) void attn_bwd_dkdv
   const int t2 = tid & 127;
   MicroBlock mb[NV];
   float stat = 0.f;
+  const float* statp = tid < 64 ? lsep : delp;  // wavefront 0 stages lse, the others delta (wavefront 1's copy is stored)
 
   auto gload = [&](int qt) {
     const int r0 = qt * 64;
@@ -341,8 +348,8 @@ __global__ __launch_bounds__(256, D == 64 ? TFB_DKDV_WPE : 1) void attn_bwd_dkdv
       int m = t2 + i * 128;
       mb[i].load(src, st_, r0 + 4 * (m & 15), 8 * (m >> 4));
     }
-    if (tid < 64) stat = -lsep[r0 + tid] * LOG2E;  // negated: the exponent is one fma
-    else if (tid < 128) stat = delp[r0 + tid - 64];
+    // raw value only: any arithmetic here would make the wavefront wait for the loads it has just issued
+    stat = statp[r0 + (tid & 63)];
   };
   auto sstore = [&](uint8_t* buf) {
 #pragma unroll
@@ -351,7 +358,7 @@ __global__ __launch_bounds__(256, D == 64 ? TFB_DKDV_WPE : 1) void attn_bwd_dkdv
       mb[i].store_normal(buf + (qrole ? OFF_QN : OFF_GN), KROW, 4 * (m & 15), 8 * (m >> 4));
       mb[i].store_transposed(buf + (qrole ? OFF_QT : OFF_GT), TROW, 4 * (m & 15), 8 * (m >> 4));
     }
-    if (tid < 128) ((float*)(buf + OFF_L))[tid] = stat;
+    if (tid < 128) ((float*)(buf + OFF_L))[tid] = tid < 64 ? -stat * LOG2E : stat;  // negated lse: the exponent is one fma
   };
 
   f32x16 dka[DT], dva[DT];
@@ -365,6 +372,7 @@ __global__ __launch_bounds__(256, D == 64 ? TFB_DKDV_WPE : 1) void attn_bwd_dkdv
 
   gload(qt0);
   sstore(smem);
+  wait_all_loads();
   __syncthreads();
 
   for (int qt = qt0; qt < nqt; ++qt) {
@@ -518,6 +526,7 @@ __global__ __launch_bounds__(256, D == 64 ? TFB_DQ_WPE : 1) void attn_bwd_dq_ker
 
   gload(0);
   sstore(smem);
+  wait_all_loads();
   __syncthreads();
 
   for (int t = 0; t < ntiles; ++t) {
@@ -635,6 +644,14 @@ int bwd_impl(AttnT q, AttnT k, AttnT v, AttnT o, AttnT go, AttnT dq, AttnT dk, A
 
 }  // namespace
 
+// D = 64 runs the kernels of attention64.hip (direct-to-LDS tile loads, transposed LDS fragment reads).
+int tfb_attn64_fwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs, void* o,
+                        const long* os, float* lse, int B, int H, int T, float scale, hipStream_t s);
+int tfb_attn64_bwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
+                        const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs, void* dk,
+                        const long* dks, void* dv, const long* dvs, const float* lse, float* stats, int B, int H, int T,
+                        float scale, hipStream_t s);
+
 // Every tensor argument comes with long[3] element strides (batch, head, token); the head dimension is contiguous.
 // lse: fp32 [B*H][T].
 extern "C" int tfb_attn_fwd(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs, void* o,
@@ -643,11 +660,11 @@ extern "C" int tfb_attn_fwd(const void* q, const long* qs, const void* k, const 
   if (B <= 0 || H <= 0 || T <= 0 || T % 128 || (D != 64 && D != 128)) return TFB_ERR_SHAPE;
   if (!strides_ok(qs) || !strides_ok(ks) || !strides_ok(vs) || !strides_ok(os)) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
-  if (D == 64) return fwd_impl<64>(mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), (float*)lse, B, H, T, scale, s);
+  if (D == 64) return tfb_attn64_fwd_impl(q, qs, k, ks, v, vs, o, os, (float*)lse, B, H, T, scale, s);
   return fwd_impl<128>(mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), (float*)lse, B, H, T, scale, s);
 }
 
-// delta: fp32 [B*H][T] scratch. dq, dk, dv may alias thirds of one dqkv buffer.
+// delta: fp32 [2][B*H][T] scratch (row dot products, then -lse log2 e). dq, dk, dv may alias thirds of one dqkv buffer.
 extern "C" int tfb_attn_bwd(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
                             const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs, void* dk,
                             const long* dks, void* dv, const long* dvs, const void* lse, void* delta, int B, int H, int T, int D,
@@ -660,8 +677,8 @@ extern "C" int tfb_attn_bwd(const void* q, const long* qs, const void* k, const 
     return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   if (D == 64)
-    return bwd_impl<64>(mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), mk(go, gos), mk(dq, dqs), mk(dk, dks), mk(dv, dvs),
-                        (const float*)lse, (float*)delta, B, H, T, scale, s);
+    return tfb_attn64_bwd_impl(q, qs, k, ks, v, vs, o, os, go, gos, dq, dqs, dk, dks, dv, dvs, (const float*)lse, (float*)delta,
+                               B, H, T, scale, s);
   return bwd_impl<128>(mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), mk(go, gos), mk(dq, dqs), mk(dk, dks), mk(dv, dvs),
                        (const float*)lse, (float*)delta, B, H, T, scale, s);
 }

@@ -1,0 +1,564 @@
+// Causal flash attention for head dimension 64 on gfx950: the kernels the C-ABI entry points in attention.hip run for
+// D = 64 (their arithmetic contract and the reference citations are stated there).
+//
+// Data movement: a 64-token x 64-element bf16 tile is 64 rows of 128 bytes. Tiles go from global memory straight
+// into LDS with global_load_lds_dwordx4 (8 tokens per instruction, no staging registers); 16-byte chunk c of token t
+// sits at slot c ^ swz(t), swz(t) = 4 ((t >> 1) & 1) | ((t >> 2) & 3). One copy of a tile then serves both MFMA
+// operand forms without bank conflicts (LDS: 64 banks of 4 bytes):
+//   * token-major fragments (token = MFMA row, contraction over d): one ds_read_b128 per lane; 16 consecutive tokens
+//     of one chunk fall on 16 different 16-byte bank groups;
+//   * transposed fragments (d = MFMA row, contraction over tokens): two ds_read_b64_tr_b16 per lane, whose 16-lane
+//     transpose hands lane i four consecutive tokens of element i when lane j points at (token0 + j / 4, d0 + 4 (j % 4));
+//     the four tokens of a 32-lane access fall on four different 64-byte bank quarters.
+// Two LDS stages (separate __shared__ objects: the compiler can tell reads of one stage from the loads in flight into
+// the other), one barrier per tile.
+//
+// Work layout: a wavefront owns 32 queries (forward, dQ) or 32 keys (dK/dV) as the MFMA column index, so every row
+// statistic is one scalar per lane and the packed score registers are directly the B operand of the next product.
+#include "common.hpp"
+
+// wavefronts per SIMD the kernels are compiled for (register budget 512 / n)
+#ifndef TFB_DQ64_WPE
+#define TFB_DQ64_WPE 2
+#endif
+#ifndef TFB_FWD64_WPE
+#define TFB_FWD64_WPE 2
+#endif
+
+namespace {
+
+struct AttnT {
+  bf16_t* p;
+  long sb, sh, st;
+};
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef const __attribute__((address_space(1))) void glb_void_t;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4_t;
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+constexpr int TILE = 64 * 128;  // bytes of one staged tile
+
+__device__ __forceinline__ f32x16 mfma_bf16(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ bf16x8 frag_from(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  u32x4 v = {a, b, c, d};
+  return __builtin_bit_cast(bf16x8, v);
+}
+__device__ __forceinline__ void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // s_waitcnt vmcnt(0)
+
+__device__ __forceinline__ int swz(int t) { return (((t >> 1) & 1) << 2) | ((t >> 2) & 3); }
+
+// This wavefront's share (2 of the 8 instructions) of a 64-token tile load. `rows` points at token 0 of the tile,
+// `stride` = bytes between tokens.
+struct TileLoad {
+  uint32_t voff;
+  int wave;
+  __device__ __forceinline__ void init(long stride, int wave_, int lane) {
+    wave = wave_;
+    const int lrow = lane >> 3;
+    // token = 8 g + lrow with g = wave or wave + 4: swz depends on g only through g & 1 = wave & 1
+    const int chunk = (lane & 7) ^ swz(8 * wave + lrow);
+    voff = (uint32_t)(lrow * stride + chunk * 16);
+  }
+  __device__ __forceinline__ void issue(const uint8_t* rows, long stride, uint8_t* lds) const {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int g = wave + 4 * i;
+      __builtin_amdgcn_global_load_lds((glb_void_t*)(rows + 8L * g * stride + (size_t)voff), (lds_void_t*)(lds + g * 1024), 16,
+                                       0, 0);
+    }
+  }
+};
+
+// token-major fragment: token = 32 * half + (lane & 31), elements 16 s + 8 (lane >> 5) .. + 7
+__device__ __forceinline__ bf16x8 frag_rows(const uint8_t* tile, int half, int s, int lr, int lh) {
+  const int t = 32 * half + lr;
+  return *(const bf16x8*)(tile + t * 128 + (((2 * s + lh) ^ swz(t)) << 4));
+}
+// transposed fragment: element (MFMA row) 32 dt + (lane & 31); tokens tok0 + 4 lh + {0..3} and tok0 + 8 + 4 lh + {0..3}
+// (the order in which a lane's packed score registers hold a 16-token block)
+__device__ __forceinline__ bf16x8 frag_cols(const uint8_t* tile, int dt, int tok0, int lane) {
+  const int g4 = lane >> 4, j = lane & 15;
+  const int d = 32 * dt + 16 * (g4 & 1) + 4 * (j & 3);
+  const int t = tok0 + 4 * (g4 >> 1) + (j >> 2);
+  const int off0 = t * 128 + ((((d >> 3) ^ swz(t))) << 4) + ((d & 4) << 1);
+  const int off1 = (t + 8) * 128 + ((((d >> 3) ^ swz(t + 8))) << 4) + ((d & 4) << 1);
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(tile + off0));
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(tile + off1));
+  const s16x8 v = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+// =========================================================================================== forward
+__global__ __launch_bounds__(256, TFB_FWD64_WPE) void attn64_fwd_kernel(AttnT q, AttnT k, AttnT v, AttnT o, float* __restrict__ lse,
+                                                            int T, int H, float sl2) {
+  __shared__ __attribute__((aligned(1024))) uint8_t st0[2 * TILE];
+  __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
+  const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int qb = gridDim.x - 1 - blockIdx.x;  // longest rows first
+  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  const bf16_t* qp = q.p + b * q.sb + h * q.sh;
+  const uint8_t* kp = (const uint8_t*)(k.p + b * k.sb + h * k.sh);
+  const uint8_t* vp = (const uint8_t*)(v.p + b * v.sb + h * v.sh);
+  bf16_t* op = o.p + b * o.sb + h * o.sh;
+  const int q0 = qb * 128, qw0 = q0 + wave * 32;
+  const long kst = k.st * 2, vst = v.st * 2;
+
+  bf16x8 qf[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) qf[s] = *(const bf16x8*)(qp + (long)(qw0 + lr) * q.st + 16 * s + 8 * lh);
+
+  TileLoad lk, lv;
+  lk.init(kst, wave, lane);
+  lv.init(vst, wave, lane);
+  auto issue = [&](uint8_t* st, int tile) {
+    lk.issue(kp + (long)tile * 64 * kst, kst, st);
+    lv.issue(vp + (long)tile * 64 * vst, vst, st + TILE);
+  };
+
+  f32x16 oacc[2];
+  float m = -1e30f, l = 0.f;  // running maximum of the raw scores, running sum
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) oacc[i][e] = 0.f;
+
+  auto compute = [&](const uint8_t* st, int tile) {
+    const int k0 = tile * 64;
+    if (k0 > qw0 + 31) return;  // the whole tile is in this wavefront's future
+    const uint8_t* kt_ = st;
+    const uint8_t* vt_ = st + TILE;
+    f32x16 sc[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) sc[kt][e] = 0.f;
+    bf16x8 ka[2][4];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int s = 0; s < 4; ++s) ka[kt][s] = frag_rows(kt_, kt, s, lr, lh);
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) sc[kt] = mfma_bf16(ka[kt][s], qf[s], sc[kt]);
+    // V^T fragments do not depend on the softmax: requested now, they arrive while the exponentials run
+    bf16x8 va[2][2][2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) va[kt][hf][dt] = frag_cols(vt_, dt, kt * 32 + 16 * hf, lane);
+    const bool diag = k0 + 63 > qw0;
+    const int kbase = k0 + lh * 4 - (qw0 + lr);  // key - q for element (kt, e) is kbase + kt*32 + (e>>2)*8 + (e&3)
+    float mx = m;
+    if (diag) {  // wavefront-uniform; the per-element masking is branch-free selects
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const bool future = kbase + kt * 32 + (e >> 2) * 8 + (e & 3) > 0;
+          sc[kt][e] = future ? -INFINITY : sc[kt][e];
+        }
+    }
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int e = 0; e < 16; e += 2) mx = fmaxf(fmaxf(mx, sc[kt][e]), sc[kt][e + 1]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float alpha = fast_exp2((m - mx) * sl2);
+    m = mx;
+    l *= alpha;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) oacc[i][e] *= alpha;
+    const float negm = -mx * sl2;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        uint32_t w[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          const int e = 8 * hf + 2 * x;
+          float p0 = fast_exp2(fmaf(sc[kt][e], sl2, negm)), p1 = fast_exp2(fmaf(sc[kt][e + 1], sl2, negm));
+          w[x] = pack2bf(p0, p1);
+          l = sum2bf(w[x], l);  // the row sum runs over the rounded values
+        }
+        const bf16x8 bb = frag_from(w[0], w[1], w[2], w[3]);
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) oacc[dt] = mfma_bf16(va[kt][hf][dt], bb, oacc[dt]);
+      }
+  };
+
+  const int n = (q0 + 128) / 64;
+  issue(st0, 0);
+  wait_all_loads();
+  __syncthreads();
+  for (int t = 0; t + 2 <= n; t += 2) {
+    issue(st1, t + 1);
+    compute(st0, t);
+    __syncthreads();
+    issue(st0, t + 2 < n ? t + 2 : n - 1);
+    compute(st1, t + 1);
+    __syncthreads();
+  }
+  // n is even (128 queries per workgroup, 64-key tiles)
+
+  const int myq = qw0 + lr;
+  const float lt = l + __shfl_xor(l, 32, 64);
+  const float inv = 1.0f / lt;
+#pragma unroll
+  for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int d = dt * 32 + 8 * j + 4 * lh;
+      u32x2 w = {pack2bf(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
+                 pack2bf(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv)};
+      *(u32x2*)(op + (long)myq * o.st + d) = w;
+    }
+  if (lh == 0) lse[(long)bh * T + myq] = (m * sl2 + log2f(lt)) * LN2;  // m is the raw-score maximum
+}
+
+// =========================================================================================== delta
+// stats[0][bh][t] = -sum_d dO * O (fp32 of the bf16 values); stats[1][bh][t] = -lse / scale; 4 lanes per row. Both are
+// the values the backward kernels start their dP and S accumulators from: the MFMAs then deliver dP - delta and
+// S - lse / scale, and P = exp2(scale log2(e) (S - lse / scale)) needs no further row term.
+__global__ __launch_bounds__(256) void attn64_delta_kernel(AttnT o, AttnT go, const float* __restrict__ lse,
+                                                           float* __restrict__ stats, int T, int H, long rows, float inv_scale) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  const long row = idx >> 2;
+  const int part = (int)(idx & 3);
+  if (row >= rows) return;
+  const int t = (int)(row % T);
+  const long bh = row / T;
+  const int b = (int)(bh / H), h = (int)(bh % H);
+  const bf16_t* op = o.p + b * o.sb + h * o.sh + (long)t * o.st + part * 16;
+  const bf16_t* gp = go.p + b * go.sb + h * go.sh + (long)t * go.st + part * 16;
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    u32x4 a = *(const u32x4*)(op + 8 * i);
+    u32x4 g = *(const u32x4*)(gp + 8 * i);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      s += bflo(a[w]) * bflo(g[w]);
+      s += bfhi(a[w]) * bfhi(g[w]);
+    }
+  }
+  s += __shfl_xor(s, 1, 64);
+  s += __shfl_xor(s, 2, 64);
+  if (part == 0) {
+    stats[row] = -s;
+    stats[rows + row] = -lse[row] * inv_scale;
+  }
+}
+
+// =========================================================================================== dK / dV
+__global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dk, AttnT dv,
+                                                             const float* __restrict__ stats, long rows, int T, int H,
+                                                             float scale, float sl2) {
+  constexpr int STAGE = 2 * TILE + 512;  // Q tile, dO tile, 64 x (-lse / scale), 64 x (-delta)
+  __shared__ __attribute__((aligned(1024))) uint8_t st0[STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t st1[STAGE];
+  const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kb = blockIdx.x;  // low key blocks see the most query tiles: already longest first
+  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  const uint8_t* qp = (const uint8_t*)(q.p + b * q.sb + h * q.sh);
+  const uint8_t* gp = (const uint8_t*)(go.p + b * go.sb + h * go.sh);
+  const bf16_t* kp = k.p + b * k.sb + h * k.sh;
+  const bf16_t* vp = v.p + b * v.sb + h * v.sh;
+  const float* delp = stats + (long)bh * T;
+  const float* nlp = stats + rows + (long)bh * T;
+  const int kw0 = kb * 128 + wave * 32, mykey = kw0 + lr;
+  const long qst = q.st * 2, gst = go.st * 2;
+
+  bf16x8 kf[4], vf[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    kf[s] = *(const bf16x8*)(kp + (long)mykey * k.st + 16 * s + 8 * lh);
+    vf[s] = *(const bf16x8*)(vp + (long)mykey * v.st + 16 * s + 8 * lh);
+  }
+
+  TileLoad lq, lg;
+  lq.init(qst, wave, lane);
+  lg.init(gst, wave, lane);
+  const int qt0 = kb * 2, n = T / 64 - qt0;
+  auto issue = [&](uint8_t* st, int i) {
+    const long r0 = (long)(qt0 + i) * 64;
+    lq.issue(qp + r0 * qst, qst, st);
+    lg.issue(gp + r0 * gst, gst, st + TILE);
+    // the row statistics: 64 floats each, one 4-byte load per lane (wavefront 0: -lse / scale, wavefront 1: -delta)
+    if (wave < 2) {
+      const float* src = (wave == 0 ? nlp : delp) + r0;
+      __builtin_amdgcn_global_load_lds((glb_void_t*)(src + lane), (lds_void_t*)(st + 2 * TILE + wave * 256), 4, 0, 0);
+    }
+  };
+
+  f32x16 dka[2], dva[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      dka[i][e] = 0.f;
+      dva[i][e] = 0.f;
+    }
+
+  auto compute = [&](const uint8_t* st, int i) {
+    const uint8_t* qt_ = st;
+    const uint8_t* gt_ = st + TILE;
+    const float* ls = (const float*)(st + 2 * TILE);
+    const int qbase = (qt0 + i) * 64;
+#pragma unroll
+    for (int qs = 0; qs < 2; ++qs) {
+      const int qlo = qbase + qs * 32;
+      if (qlo + 31 < kw0) continue;  // every key of this wavefront is in the future of these queries
+      bf16x8 qa[4], ga[4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        qa[s] = frag_rows(qt_, qs, s, lr, lh);
+        ga[s] = frag_rows(gt_, qs, s, lr, lh);
+      }
+      // the accumulators start from the rows' -lse / scale and -delta
+      f32x16 S, dP;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const f32x4 L = *(const f32x4*)(ls + qs * 32 + 8 * j + 4 * lh);
+        const f32x4 Dl = *(const f32x4*)(ls + 64 + qs * 32 + 8 * j + 4 * lh);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          S[4 * j + x] = L[x];
+          dP[4 * j + x] = Dl[x];
+        }
+      }
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        S = mfma_bf16(qa[s], kf[s], S);
+        dP = mfma_bf16(ga[s], vf[s], dP);
+      }
+      // transposed fragments for the second pair of products: independent of the arithmetic below, so they are
+      // requested first and arrive while the exponentials run
+      bf16x8 gT[2][2], qT[2][2];
+#pragma unroll
+      for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          gT[dt][ks] = frag_cols(gt_, dt, qs * 32 + 16 * ks, lane);
+          qT[dt][ks] = frag_cols(qt_, dt, qs * 32 + 16 * ks, lane);
+        }
+      const int kq = mykey - (qlo + 4 * lh);  // key - q for element e is kq - (e>>2)*8 - (e&3)
+      if (kw0 + 31 > qlo) {  // wavefront-uniform; masked scores become -inf (P = 0) through branch-free selects
+#pragma unroll
+        for (int e = 0; e < 16; ++e) S[e] = (kq - 8 * (e >> 2) - (e & 3) > 0) ? -INFINITY : S[e];
+      }
+      uint32_t pw[8], dsw[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float p[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) p[x] = fast_exp2(S[4 * j + x] * sl2);
+        const uint32_t w0 = pack2bf(p[0], p[1]), w1 = pack2bf(p[2], p[3]);
+        pw[2 * j] = w0;
+        pw[2 * j + 1] = w1;
+        const float d0 = bflo(w0) * dP[4 * j], d1 = bfhi(w0) * dP[4 * j + 1];
+        const float d2 = bflo(w1) * dP[4 * j + 2], d3 = bfhi(w1) * dP[4 * j + 3];
+        dsw[2 * j] = pack2bf(d0, d1);
+        dsw[2 * j + 1] = pack2bf(d2, d3);
+      }
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const bf16x8 pb = frag_from(pw[4 * ks], pw[4 * ks + 1], pw[4 * ks + 2], pw[4 * ks + 3]);
+        const bf16x8 db = frag_from(dsw[4 * ks], dsw[4 * ks + 1], dsw[4 * ks + 2], dsw[4 * ks + 3]);
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) {
+          dva[dt] = mfma_bf16(gT[dt][ks], pb, dva[dt]);
+          dka[dt] = mfma_bf16(qT[dt][ks], db, dka[dt]);
+        }
+      }
+    }
+  };
+
+  issue(st0, 0);
+  wait_all_loads();
+  __syncthreads();
+  for (int t = 0; t + 2 <= n; t += 2) {
+    issue(st1, t + 1);
+    compute(st0, t);
+    __syncthreads();
+    issue(st0, t + 2 < n ? t + 2 : n - 1);
+    compute(st1, t + 1);
+    __syncthreads();
+  }
+  // n = T / 64 - 2 kb is even
+
+  bf16_t* dkp = dk.p + b * dk.sb + h * dk.sh + (long)mykey * dk.st;
+  bf16_t* dvp = dv.p + b * dv.sb + h * dv.sh + (long)mykey * dv.st;
+#pragma unroll
+  for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int d = dt * 32 + 8 * j + 4 * lh;
+      u32x2 wk = {pack2bf(dka[dt][4 * j] * scale, dka[dt][4 * j + 1] * scale),
+                  pack2bf(dka[dt][4 * j + 2] * scale, dka[dt][4 * j + 3] * scale)};
+      u32x2 wv = {pack2bf(dva[dt][4 * j], dva[dt][4 * j + 1]), pack2bf(dva[dt][4 * j + 2], dva[dt][4 * j + 3])};
+      *(u32x2*)(dkp + d) = wk;
+      *(u32x2*)(dvp + d) = wv;
+    }
+}
+
+// =========================================================================================== dQ
+__global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dq,
+                                                           const float* __restrict__ stats, long rows, int T, int H,
+                                                           float scale, float sl2) {
+  __shared__ __attribute__((aligned(1024))) uint8_t st0[2 * TILE];
+  __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
+  const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int qb = gridDim.x - 1 - blockIdx.x;
+  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  const bf16_t* qp = q.p + b * q.sb + h * q.sh;
+  const bf16_t* gp = go.p + b * go.sb + h * go.sh;
+  const uint8_t* kp = (const uint8_t*)(k.p + b * k.sb + h * k.sh);
+  const uint8_t* vp = (const uint8_t*)(v.p + b * v.sb + h * v.sh);
+  const int q0 = qb * 128, qw0 = q0 + wave * 32, myq = qw0 + lr;
+  const long kst = k.st * 2, vst = v.st * 2;
+
+  bf16x8 qf[4], gf[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    qf[s] = *(const bf16x8*)(qp + (long)myq * q.st + 16 * s + 8 * lh);
+    gf[s] = *(const bf16x8*)(gp + (long)myq * go.st + 16 * s + 8 * lh);
+  }
+  const float myD = stats[(long)bh * T + myq];
+  const float myL = stats[rows + (long)bh * T + myq];
+
+  TileLoad lk, lv;
+  lk.init(kst, wave, lane);
+  lv.init(vst, wave, lane);
+  auto issue = [&](uint8_t* st, int tile) {
+    lk.issue(kp + (long)tile * 64 * kst, kst, st);
+    lv.issue(vp + (long)tile * 64 * vst, vst, st + TILE);
+  };
+
+  f32x16 dqa[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) dqa[i][e] = 0.f;
+
+  auto compute = [&](const uint8_t* st, int tile) {
+    const uint8_t* kt_ = st;
+    const uint8_t* vt_ = st + TILE;
+    const int k0 = tile * 64;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      const int klo = k0 + kt * 32;
+      if (klo > qw0 + 31) continue;
+      bf16x8 ka[4], va[4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        ka[s] = frag_rows(kt_, kt, s, lr, lh);
+        va[s] = frag_rows(vt_, kt, s, lr, lh);
+      }
+      f32x16 S, dP;  // started from the query's -lse / scale and -delta
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        S[e] = myL;
+        dP[e] = myD;
+      }
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        S = mfma_bf16(ka[s], qf[s], S);
+        dP = mfma_bf16(va[s], gf[s], dP);
+      }
+      bf16x8 kT[2][2];  // requested before the arithmetic they do not depend on
+#pragma unroll
+      for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) kT[dt][ks] = frag_cols(kt_, dt, kt * 32 + 16 * ks, lane);
+      const int kbase = klo + lh * 4 - myq;
+      if (klo + 31 > qw0) {  // wavefront-uniform
+#pragma unroll
+        for (int e = 0; e < 16; ++e) S[e] = (kbase + (e >> 2) * 8 + (e & 3) > 0) ? -INFINITY : S[e];
+      }
+      uint32_t dsw[8];
+#pragma unroll
+      for (int e = 0; e < 16; e += 2) {
+        const float p0 = fast_exp2(S[e] * sl2), p1 = fast_exp2(S[e + 1] * sl2);
+        const uint32_t w = pack2bf(p0, p1);
+        dsw[e >> 1] = pack2bf(bflo(w) * dP[e], bfhi(w) * dP[e + 1]);
+      }
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const bf16x8 db = frag_from(dsw[4 * ks], dsw[4 * ks + 1], dsw[4 * ks + 2], dsw[4 * ks + 3]);
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) dqa[dt] = mfma_bf16(kT[dt][ks], db, dqa[dt]);
+      }
+    }
+  };
+
+  const int n = (q0 + 128) / 64;
+  issue(st0, 0);
+  wait_all_loads();
+  __syncthreads();
+  for (int t = 0; t + 2 <= n; t += 2) {
+    issue(st1, t + 1);
+    compute(st0, t);
+    __syncthreads();
+    issue(st0, t + 2 < n ? t + 2 : n - 1);
+    compute(st1, t + 1);
+    __syncthreads();
+  }
+
+  bf16_t* dqp = dq.p + b * dq.sb + h * dq.sh + (long)myq * dq.st;
+#pragma unroll
+  for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int d = dt * 32 + 8 * j + 4 * lh;
+      u32x2 w = {pack2bf(dqa[dt][4 * j] * scale, dqa[dt][4 * j + 1] * scale),
+                 pack2bf(dqa[dt][4 * j + 2] * scale, dqa[dt][4 * j + 3] * scale)};
+      *(u32x2*)(dqp + d) = w;
+    }
+}
+
+AttnT mk(const void* p, const long* s) { return AttnT{(bf16_t*)p, s[0], s[1], s[2]}; }
+
+}  // namespace
+
+// Called by tfb_attn_fwd / tfb_attn_bwd for D = 64 (arguments already validated there: T % 128 == 0, strides % 8 == 0).
+int tfb_attn64_fwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs, void* o,
+                        const long* os, float* lse, int B, int H, int T, float scale, hipStream_t s) {
+  hipLaunchKernelGGL(attn64_fwd_kernel, dim3(T / 128, B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), lse,
+                     T, H, scale * LOG2E);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// stats: fp32 [2][B*H][T] scratch (-delta, then -lse / scale).
+int tfb_attn64_bwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
+                        const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs, void* dk,
+                        const long* dks, void* dv, const long* dvs, const float* lse, float* stats, int B, int H, int T,
+                        float scale, hipStream_t s) {
+  const long rows = (long)B * H * T;
+  hipLaunchKernelGGL(attn64_delta_kernel, dim3((unsigned)((rows * 4 + 255) / 256)), dim3(256), 0, s, mk(o, os), mk(go, gos), lse,
+                     stats, T, H, rows, 1.0f / scale);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(attn64_dkdv_kernel, dim3(T / 128, B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
+                     mk(dk, dks), mk(dv, dvs), stats, rows, T, H, scale, scale * LOG2E);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(attn64_dq_kernel, dim3(T / 128, B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
+                     mk(dq, dqs), stats, rows, T, H, scale, scale * LOG2E);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}

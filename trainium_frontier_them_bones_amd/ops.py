@@ -280,7 +280,7 @@ def attn_bwd(q, k, v, o, do, lse, scale, layout="bhtd", dq=None, dk=None, dv=Non
         dk = torch.empty(B, H, T, D, dtype=bf16, device=q.device)
         dv = torch.empty(B, T, H, D, dtype=bf16, device=q.device).permute(0, 2, 1, 3)
         out_layout = "bhtd"
-    delta = torch.empty(B, H, T, dtype=torch.float32, device=q.device)
+    delta = torch.empty(2, B, H, T, dtype=torch.float32, device=q.device)
     _lib.call("tfb_attn_bwd", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o), _bht(o, "bthd"),
               _p(do), _bht(do, "bthd"), _p(dq), _bht(dq, out_layout), _p(dk), _bht(dk, out_layout), _p(dv),
               _bht(dv, out_layout), _p(lse), _p(delta), B, H, T, D, float(scale), _stream())
