@@ -101,7 +101,7 @@ def main():
                    "step_tflops": round(flops_per_token(cfg) * tokens / 1e12, 2),
                    "model_tflops_per_s": round(flops_per_token(cfg) * tokens / (dt / args.steps) / 1e12, 1),
                    "final_loss": round(float(loss.item()), 4)},
-        "roofline": {"kernel": "attention backward (attn_bwd_dkdv + attn_bwd_dq + delta), B16 H12 T2048 D64", "bound": "mfma",
+        "roofline": {"kernel": "attention backward (tfb_attn_bwd: attn64_delta + attn64_dkdv + attn64_dq), B16 H12 T2048 D64", "bound": "mfma",
                      "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
                      "launch_ms": round(k_ms, 4), "launches_timed": len(rec)},
