@@ -3,6 +3,9 @@ HIP kernels, with the roofline position of the dominant kernel and the CPU oracl
 
 python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
 Prints ONE JSON line.
+
+python bench.py --traffic-probe   (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: a 256 MiB device copy as the
+counters' calibration, then attention forward + backward at the benchmark shape; prints nothing)
 """
 import argparse
 import json
@@ -15,6 +18,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0
+# HBM-side bytes one tfb_attn_bwd call moves at B16 H12 T2048 D64 (delta + dkdv + dq kernels), from the FETCH_SIZE and
+# WRITE_SIZE counters scaled by a 256 MiB copy (profiles/attn_c2_hbm_traffic.md): 1,820 MB fetched + 155 MB written.
+ATTN_BWD_TRAFFIC_BYTES = 1.974e9
 
 
 def flops_per_token(cfg):
@@ -40,16 +46,39 @@ def cpu_baseline(cfg, init_values):
             "sample": "1 of the 16 sequences (2048 tokens) through the full 12-layer model, fwd+bwd+AdamW, 1 repetition"}
 
 
+def traffic_probe():
+    import torch
+    from trainium_frontier_them_bones_amd import ops
+    dev = torch.device("cuda:0")
+    B, H, T, D = 16, 12, 2048, 64
+    torch.manual_seed(0)
+    q = torch.randn(B, H, T, D, device=dev).bfloat16()
+    k, v = torch.randn_like(q), torch.randn_like(q)
+    do = torch.randn(B, T, H, D, device=dev).bfloat16()
+    src = torch.randn(64 * 1024 * 1024, device=dev)   # 256 MiB fp32
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)                                 # calibration: reads 256 MiB, writes 256 MiB
+        o, lse = ops.attn_fwd(q, k, v, 0.125)
+        ops.attn_bwd(q, k, v, o, do, lse, 0.125)
+    torch.cuda.synchronize()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
+
+    if args.traffic_probe:
+        traffic_probe()
+        return
 
     import torch
     from trainium_frontier_them_bones_amd import _lib
@@ -103,7 +132,7 @@ def main():
                    "final_loss": round(float(loss.item()), 4)},
         "roofline": {"kernel": "attention backward (tfb_attn_bwd: attn64_delta + attn64_dkdv + attn64_dq), B16 H12 T2048 D64", "bound": "mfma",
                      "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": ATTN_BWD_TRAFFIC_BYTES,
                      "launch_ms": round(k_ms, 4), "launches_timed": len(rec)},
     }
     if not args.no_cpu:
