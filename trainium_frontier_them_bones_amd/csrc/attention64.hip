@@ -52,6 +52,21 @@ __device__ __forceinline__ bf16x8 frag_from(uint32_t a, uint32_t b, uint32_t c, 
 }
 __device__ __forceinline__ void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // s_waitcnt vmcnt(0)
 
+// Workgroup -> (block along the sequence, batch*head): consecutive workgroup ids are dealt round-robin to the 8 XCDs,
+// each with its own L2, so the ids are re-dealt to keep all sequence blocks of one (batch, head) - which stream the same
+// K/V (or Q/dO) tiles - on one XCD. nx = blocks per (batch, head), nbh = batch*head count.
+__device__ __forceinline__ void xcd_block(int nx, int nbh, int& bx, int& bh) {
+  const int lin = blockIdx.y * nx + blockIdx.x;
+  if (nbh % 8 == 0) {
+    const int xcd = lin & 7, idx = lin >> 3;
+    bh = xcd + 8 * (idx / nx);
+    bx = idx % nx;
+  } else {
+    bh = blockIdx.y;
+    bx = blockIdx.x;
+  }
+}
+
 __device__ __forceinline__ int swz(int t) { return (((t >> 1) & 1) << 2) | ((t >> 2) & 3); }
 
 // This wavefront's share (2 of the 8 instructions) of a 64-token tile load. `rows` points at token 0 of the tile,
@@ -102,8 +117,10 @@ __global__ __launch_bounds__(256, TFB_FWD64_WPE) void attn64_fwd_kernel(AttnT q,
   __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int qb = gridDim.x - 1 - blockIdx.x;  // longest rows first
-  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  int bx, bh;
+  xcd_block(gridDim.x, gridDim.y, bx, bh);
+  const int qb = gridDim.x - 1 - bx;  // longest rows first
+  const int b = bh / H, h = bh % H;
   const bf16_t* qp = q.p + b * q.sb + h * q.sh;
   const uint8_t* kp = (const uint8_t*)(k.p + b * k.sb + h * k.sh);
   const uint8_t* vp = (const uint8_t*)(v.p + b * v.sb + h * v.sh);
@@ -272,8 +289,9 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
   __shared__ __attribute__((aligned(1024))) uint8_t st1[STAGE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int kb = blockIdx.x;  // low key blocks see the most query tiles: already longest first
-  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  int kb, bh;  // low key blocks see the most query tiles: already longest first
+  xcd_block(gridDim.x, gridDim.y, kb, bh);
+  const int b = bh / H, h = bh % H;
   const uint8_t* qp = (const uint8_t*)(q.p + b * q.sb + h * q.sh);
   const uint8_t* gp = (const uint8_t*)(go.p + b * go.sb + h * go.sh);
   const bf16_t* kp = k.p + b * k.sb + h * k.sh;
@@ -424,8 +442,10 @@ __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, A
   __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int qb = gridDim.x - 1 - blockIdx.x;
-  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  int bx, bh;
+  xcd_block(gridDim.x, gridDim.y, bx, bh);
+  const int qb = gridDim.x - 1 - bx;
+  const int b = bh / H, h = bh % H;
   const bf16_t* qp = q.p + b * q.sb + h * q.sh;
   const bf16_t* gp = go.p + b * go.sb + h * go.sh;
   const uint8_t* kp = (const uint8_t*)(k.p + b * k.sb + h * k.sh);
