@@ -96,18 +96,20 @@ def main():
     torch.cuda.synchronize()
 
     rec = []
-    _lib.TIMED["tfb_attn_bwd"] = rec
+    _lib.TIMED["tfb_attn_bwd_rope"] = rec
     t0 = time.perf_counter()
     for _ in range(args.steps):
         loss = model.train_step(idx, tg)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    del _lib.TIMED["tfb_attn_bwd"]
+    del _lib.TIMED["tfb_attn_bwd_rope"]
     tokens = B * cfg.seq_len
     ms = dt / args.steps * 1e3
 
     # dominant entry point: attention backward (three launches: D = sum dO*O, dK/dV, dQ), timed with events on its stream
-    k_ms = sum(s.elapsed_time(e) for s, e in rec) / max(len(rec), 1)
+    if not rec:
+        raise RuntimeError("the timed entry point was never called: roofline.achieved would be meaningless")
+    k_ms = sum(s.elapsed_time(e) for s, e in rec) / len(rec)
     H, D, T = cfg.n_head, cfg.head_dim, cfg.seq_len
     k_flops = 5 * B * H * T * T * D   # causal-halved: 5 matmuls x 2 flop x 1/2
     achieved = k_flops / (k_ms * 1e-3) / 1e12 if k_ms > 0 else 0.0
@@ -130,7 +132,7 @@ def main():
                    "step_tflops": round(flops_per_token(cfg) * tokens / 1e12, 2),
                    "model_tflops_per_s": round(flops_per_token(cfg) * tokens / (dt / args.steps) / 1e12, 1),
                    "final_loss": round(float(loss.item()), 4)},
-        "roofline": {"kernel": "attention backward (tfb_attn_bwd: attn64_delta + attn64_dkdv + attn64_dq), B16 H12 T2048 D64", "bound": "mfma",
+        "roofline": {"kernel": "attention backward (tfb_attn_bwd_rope: attn64_delta + attn64_dkdv + attn64_dq), B16 H12 T2048 D64", "bound": "mfma",
                      "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": ATTN_BWD_TRAFFIC_BYTES,
                      "launch_ms": round(k_ms, 4), "launches_timed": len(rec)},

@@ -141,6 +141,13 @@ int tfb_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* row
 int tfb_mlp_dw_proj(const void* dy, const void* r, void* dw, long M, int d, int F, int out_f32, int accumulate,
                     void* workspace, long workspace_bytes, void* stream);
 
+/* qkv [M][N] = rope(x [M][K] @ w [N][K]^T): the fused attention projection with the rotary embedding (half-split,
+ * heads of 64) of its first rot_cols columns applied in the GEMM epilogue; row m is token m % T; cos_t, sin_t bf16
+ * [T][32]. Equals tfb_gemm_bf16 followed by tfb_rope bit for bit. Replaces the c_attn projection + the rotation inside
+ * nki_rope_attention (round1/source/train.py:8197, 4188-4193) as one launch. */
+int tfb_qkv_rope_fwd(const void* x, const void* w, const void* cos_t, const void* sin_t, void* out, int M, int N, int K, int T,
+                     int rot_cols, void* stream);
+
 /* ---- attention ----------------------------------------------------------------------------------------------------
  * Causal flash attention, bf16. Every tensor comes with host long[3] element strides (batch, head, token); head dim
  * contiguous; so q/k/v can be [B,H,T,D], [B,T,H,D] or thirds of a fused [B,T,3C] projection. lse fp32 [B*H][T].
@@ -157,6 +164,14 @@ int tfb_attn_bwd(const void* q, const long* q_strides, const void* k, const long
                  const long* v_strides, const void* o, const long* o_strides, const void* d_o, const long* do_strides,
                  void* dq, const long* dq_strides, void* dk, const long* dk_strides, void* dv, const long* dv_strides,
                  const void* lse, void* delta, int B, int H, int T, int D, float scale, void* stream);
+/* The same, with the inverse RoPE rotation (cos_t, sin_t bf16 [T][D/2]) applied to dq and dk on their way out: the
+ * backward half of attention over a rotated fused projection. D == 64; TFB_ERR_SHAPE otherwise (caller runs tfb_rope).
+ * Replaces NkiRopeAttnFn.backward / s2attn::rope_attn_bwd (round1/source/train.py:8135; round2/source/train.py:5040). */
+int tfb_attn_bwd_rope(const void* q, const long* q_strides, const void* k, const long* k_strides, const void* v,
+                      const long* v_strides, const void* o, const long* o_strides, const void* d_o, const long* do_strides,
+                      void* dq, const long* dq_strides, void* dk, const long* dk_strides, void* dv, const long* dv_strides,
+                      const void* lse, void* delta, const void* cos_t, const void* sin_t, int B, int H, int T, int D,
+                      float scale, void* stream);
 
 /* ---- loss head ------------------------------------------------------------------------------------------------------
  * loss[row] = row_w[row] * (lse - s_target), lse[row] = log sum exp(s), s = softcap tanh(x / softcap) (softcap <= 0:

@@ -280,6 +280,15 @@ def test_attention_strided_qkv_and_rejects(ops, dev):
     dqo, dko, dvo = O.backward(q4, k4, v4, o.cpu(), do, lse.cpu(), 0.125)
     want = torch.cat([t.permute(0, 2, 1, 3).reshape(B, T, H * D) for t in (dqo, dko, dvo)], dim=-1)
     assert rel_l2(dqkv, want) < BF16_TOL
+    # inverse RoPE fused into the backward stores == the separate rotation pass over the bf16 gradient, bit for bit
+    cos, sin = O.rope_tables(T, D)
+    cosd, sind = cos.to(dev), sin.to(dev)
+    unfused = dqkv.clone()
+    ops.rope_(unfused.view(B * T, 3 * H * D), cosd, sind, T, 2 * H, D, inverse=True)
+    fused = torch.empty_like(qd)
+    fq, fk, fv = (t.view(B, T, H, D) for t in fused.split(H * D, dim=-1))
+    ops.attn_bwd(q, k, v, o, do.to(dev), lse, 0.125, "bthd", fq, fk, fv, "bthd", rope=(cosd, sind))
+    assert torch.equal(fused, unfused)
     with pytest.raises(TfbError):
         ops.attn_fwd(q[:, :100], k[:, :100], v[:, :100], 0.125, layout="bthd")       # T % 128 != 0
 
@@ -369,3 +378,27 @@ def test_lmhead_softcap_matches_materialised_path(ops, dev):
     assert torch.equal(logits, ops.matmul(x, W, trans_b=True))
     rows2, lse2 = ops.loss_fwd(logits, t, 15.0)
     assert rel_l2(rows, rows2) < 1e-5 and rel_l2(lse, lse2) < 1e-6
+
+
+def test_qkv_rope_projection_fused_equals_unfused(ops, dev):
+    """The projection with the rotary embedding in its epilogue, and the autograd node built on it, against the
+    separate GEMM / rotation / attention launches: bit for bit."""
+    from oracle import attention as O
+    from trainium_frontier_them_bones_amd import autograd as A
+    B, T, H, D, Cin = 2, 256, 4, 64, 256
+    g = _g(21)
+    x = torch.randn(B, T, Cin, generator=g).bfloat16().to(dev)
+    w = (0.05 * torch.randn(3 * H * D, Cin, generator=g)).bfloat16().to(dev)
+    cos, sin = (t.to(dev) for t in O.rope_tables(T, D))
+    fused = ops.qkv_rope(x.view(B * T, Cin), w, cos, sin, T, 2 * H * D)
+    plain = ops.matmul(x.view(B * T, Cin), w, trans_b=True)
+    ops.rope_(plain, cos, sin, T, 2 * H, D)
+    assert torch.equal(fused, plain)
+    go = torch.randn(B, T, H * D, generator=g).bfloat16().to(dev)
+    x1, w1 = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    y1 = A.QkvRopeAttentionFn.apply(x1, w1, cos, sin, H, 0.125)
+    y1.backward(go)
+    x2, w2 = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    y2 = A.RopeAttentionFn.apply(A.LinearFn.apply(x2, w2), cos, sin, H, 0.125)
+    y2.backward(go)
+    assert torch.equal(y1, y2) and torch.equal(x1.grad, x2.grad) and torch.equal(w1.grad, w2.grad)

@@ -157,9 +157,51 @@ class RopeAttentionFn(torch.autograd.Function):
         q, k, v = (t.view(B, T, H, D) for t in qkv.split(C, dim=-1))
         dqkv = torch.empty_like(qkv)
         dq, dk, dv = (t.view(B, T, H, D) for t in dqkv.split(C, dim=-1))
-        ops.attn_bwd(q, k, v, o, go.contiguous().view(B, T, H, D), lse, ctx.scale, "bthd", dq, dk, dv, "bthd")
-        ops.rope_(dqkv.view(B * T, C3), cos, sin, T, 2 * H, D, inverse=True)
+        if D == 64:  # the inverse rotation of dq, dk rides the backward kernels' stores
+            ops.attn_bwd(q, k, v, o, go.contiguous().view(B, T, H, D), lse, ctx.scale, "bthd", dq, dk, dv, "bthd", rope=(cos, sin))
+        else:
+            ops.attn_bwd(q, k, v, o, go.contiguous().view(B, T, H, D), lse, ctx.scale, "bthd", dq, dk, dv, "bthd")
+            ops.rope_(dqkv.view(B * T, C3), cos, sin, T, 2 * H, D, inverse=True)
         return dqkv, None, None, None, None
+
+
+class QkvRopeAttentionFn(torch.autograd.Function):
+    """Attention block core in one autograd node: qkv = rope(x @ w_qkv^T) (rotation in the projection's epilogue), causal
+    attention on the thirds, and in backward the inverse rotation inside the attention kernels' stores followed by the
+    projection's dX and dW (accumulated into w_qkv.grad_buf when present). Head dimension 64."""
+
+    @staticmethod
+    def forward(ctx, x, w_qkv, cos, sin, n_head, scale):
+        B, T, Cin = x.shape
+        C3 = w_qkv.shape[0]
+        C = C3 // 3
+        D = C // n_head
+        x2 = x.reshape(B * T, Cin).contiguous()
+        qkv = ops.qkv_rope(x2, w_qkv, cos, sin, T, 2 * C).view(B, T, C3)
+        q, k, v = (t.view(B, T, n_head, D) for t in qkv.split(C, dim=-1))
+        o, lse = ops.attn_fwd(q, k, v, scale, "bthd")
+        ctx.save_for_backward(x2, w_qkv, qkv, o, lse, cos, sin)
+        ctx.n_head, ctx.scale, ctx.xshape = n_head, scale, x.shape
+        return o.view(B, T, C)
+
+    @staticmethod
+    def backward(ctx, go):
+        x2, w, qkv, o, lse, cos, sin = ctx.saved_tensors
+        B, T, C3 = qkv.shape
+        C = C3 // 3
+        H = ctx.n_head
+        D = C // H
+        q, k, v = (t.view(B, T, H, D) for t in qkv.split(C, dim=-1))
+        dqkv = torch.empty_like(qkv)
+        dq, dk, dv = (t.view(B, T, H, D) for t in dqkv.split(C, dim=-1))
+        ops.attn_bwd(q, k, v, o, go.contiguous().view(B, T, H, D), lse, ctx.scale, "bthd", dq, dk, dv, "bthd", rope=(cos, sin))
+        g2 = dqkv.view(B * T, C3)
+        dx = ops.matmul(g2, w).view(ctx.xshape)
+        buf, acc = _accumulate_into(w)
+        if buf is not None:
+            ops.matmul(g2, x2, trans_a=True, out=buf, accumulate=acc)
+            return dx, None, None, None, None, None
+        return dx, ops.matmul(g2, x2, trans_a=True), None, None, None, None
 
 
 class Mlp8State:

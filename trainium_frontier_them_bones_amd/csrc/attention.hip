@@ -650,7 +650,7 @@ int tfb_attn64_fwd_impl(const void* q, const long* qs, const void* k, const long
 int tfb_attn64_bwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
                         const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs, void* dk,
                         const long* dks, void* dv, const long* dvs, const float* lse, float* stats, int B, int H, int T,
-                        float scale, hipStream_t s);
+                        float scale, const void* cos_t, const void* sin_t, hipStream_t s);
 
 // Every tensor argument comes with long[3] element strides (batch, head, token); the head dimension is contiguous.
 // lse: fp32 [B*H][T].
@@ -665,20 +665,33 @@ extern "C" int tfb_attn_fwd(const void* q, const long* qs, const void* k, const 
 }
 
 // delta: fp32 [2][B*H][T] scratch (row dot products, then -lse log2 e). dq, dk, dv may alias thirds of one dqkv buffer.
-extern "C" int tfb_attn_bwd(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
-                            const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs, void* dk,
-                            const long* dks, void* dv, const long* dvs, const void* lse, void* delta, int B, int H, int T, int D,
-                            float scale, void* stream) {
+// cos_t / sin_t (bf16 [T][D/2], both or neither): dq and dk come out with the inverse RoPE rotation applied, i.e. as
+// gradients of the projections the rotation was applied to (D = 64 only; otherwise TFB_ERR_SHAPE and the caller runs
+// tfb_rope itself).
+extern "C" int tfb_attn_bwd_rope(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
+                                 const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs,
+                                 void* dk, const long* dks, void* dv, const long* dvs, const void* lse, void* delta,
+                                 const void* cos_t, const void* sin_t, int B, int H, int T, int D, float scale, void* stream) {
   if (!q || !k || !v || !o || !go || !dq || !dk || !dv || !lse || !delta) return TFB_ERR_ARG;
   if (!qs || !ks || !vs || !os || !gos || !dqs || !dks || !dvs) return TFB_ERR_ARG;
+  if ((cos_t == nullptr) != (sin_t == nullptr)) return TFB_ERR_ARG;
   if (B <= 0 || H <= 0 || T <= 0 || T % 128 || (D != 64 && D != 128)) return TFB_ERR_SHAPE;
+  if (cos_t && D != 64) return TFB_ERR_SHAPE;
   if (!strides_ok(qs) || !strides_ok(ks) || !strides_ok(vs) || !strides_ok(os) || !strides_ok(gos) || !strides_ok(dqs) ||
       !strides_ok(dks) || !strides_ok(dvs))
     return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   if (D == 64)
     return tfb_attn64_bwd_impl(q, qs, k, ks, v, vs, o, os, go, gos, dq, dqs, dk, dks, dv, dvs, (const float*)lse, (float*)delta,
-                               B, H, T, scale, s);
+                               B, H, T, scale, cos_t, sin_t, s);
   return bwd_impl<128>(mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), mk(go, gos), mk(dq, dqs), mk(dk, dks), mk(dv, dvs),
                        (const float*)lse, (float*)delta, B, H, T, scale, s);
+}
+
+extern "C" int tfb_attn_bwd(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
+                            const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs, void* dk,
+                            const long* dks, void* dv, const long* dvs, const void* lse, void* delta, int B, int H, int T, int D,
+                            float scale, void* stream) {
+  return tfb_attn_bwd_rope(q, qs, k, ks, v, vs, o, os, go, gos, dq, dqs, dk, dks, dv, dvs, lse, delta, nullptr, nullptr, B, H, T,
+                           D, scale, stream);
 }

@@ -110,6 +110,37 @@ __device__ __forceinline__ bf16x8 frag_cols(const uint8_t* tile, int dt, int tok
   return __builtin_bit_cast(bf16x8, v);
 }
 
+// Store one token's gradient row from the two 32-element halves a lane's accumulators hold (elements 8 j + 4 lh + i of
+// each half), scaled and rounded once to bf16; with cos / sin tables ([T][32] bf16) the inverse RoPE rotation
+// (y1 = x1 c - x2 s, y2 = x2 c + x1 s on the rounded values, rounded again: what a separate pass over the bf16
+// gradient computes) is applied on the way out.
+__device__ __forceinline__ void store_grad_row(const f32x16 (&acc)[2], float scale, bf16_t* row, const bf16_t* cs,
+                                               const bf16_t* sn, int tok, int lh) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int d = 8 * j + 4 * lh;
+    u32x2 w1 = {pack2bf(acc[0][4 * j] * scale, acc[0][4 * j + 1] * scale),
+                pack2bf(acc[0][4 * j + 2] * scale, acc[0][4 * j + 3] * scale)};
+    u32x2 w2 = {pack2bf(acc[1][4 * j] * scale, acc[1][4 * j + 1] * scale),
+                pack2bf(acc[1][4 * j + 2] * scale, acc[1][4 * j + 3] * scale)};
+    if (cs) {
+      const u32x2 c = *(const u32x2*)(cs + (long)tok * 32 + d), s = *(const u32x2*)(sn + (long)tok * 32 + d);
+      u32x2 o1, o2;
+#pragma unroll
+      for (int x = 0; x < 2; ++x) {
+        const float a0 = bflo(w1[x]), a1 = bfhi(w1[x]), b0 = bflo(w2[x]), b1 = bfhi(w2[x]);
+        const float c0 = bflo(c[x]), c1 = bfhi(c[x]), s0 = -bflo(s[x]), s1 = -bfhi(s[x]);
+        o1[x] = pack2bf(a0 * c0 + b0 * s0, a1 * c1 + b1 * s1);
+        o2[x] = pack2bf(b0 * c0 - a0 * s0, b1 * c1 - a1 * s1);
+      }
+      w1 = o1;
+      w2 = o2;
+    }
+    *(u32x2*)(row + d) = w1;
+    *(u32x2*)(row + 32 + d) = w2;
+  }
+}
+
 // =========================================================================================== forward
 __global__ __launch_bounds__(256, TFB_FWD64_WPE) void attn64_fwd_kernel(AttnT q, AttnT k, AttnT v, AttnT o, float* __restrict__ lse,
                                                             int T, int H, float sl2) {
@@ -283,7 +314,8 @@ __global__ __launch_bounds__(256) void attn64_delta_kernel(AttnT o, AttnT go, co
 // =========================================================================================== dK / dV
 __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dk, AttnT dv,
                                                              const float* __restrict__ stats, long rows, int T, int H,
-                                                             float scale, float sl2) {
+                                                             float scale, float sl2, const bf16_t* __restrict__ cs,
+                                                             const bf16_t* __restrict__ sn) {
   constexpr int STAGE = 2 * TILE + 512;  // Q tile, dO tile, 64 x (-lse / scale), 64 x (-delta)
   __shared__ __attribute__((aligned(1024))) uint8_t st0[STAGE];
   __shared__ __attribute__((aligned(1024))) uint8_t st1[STAGE];
@@ -421,23 +453,15 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
 
   bf16_t* dkp = dk.p + b * dk.sb + h * dk.sh + (long)mykey * dk.st;
   bf16_t* dvp = dv.p + b * dv.sb + h * dv.sh + (long)mykey * dv.st;
-#pragma unroll
-  for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int d = dt * 32 + 8 * j + 4 * lh;
-      u32x2 wk = {pack2bf(dka[dt][4 * j] * scale, dka[dt][4 * j + 1] * scale),
-                  pack2bf(dka[dt][4 * j + 2] * scale, dka[dt][4 * j + 3] * scale)};
-      u32x2 wv = {pack2bf(dva[dt][4 * j], dva[dt][4 * j + 1]), pack2bf(dva[dt][4 * j + 2], dva[dt][4 * j + 3])};
-      *(u32x2*)(dkp + d) = wk;
-      *(u32x2*)(dvp + d) = wv;
-    }
+  store_grad_row(dka, scale, dkp, cs, sn, mykey, lh);
+  store_grad_row(dva, 1.0f, dvp, nullptr, nullptr, mykey, lh);
 }
 
 // =========================================================================================== dQ
 __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dq,
                                                            const float* __restrict__ stats, long rows, int T, int H,
-                                                           float scale, float sl2) {
+                                                           float scale, float sl2, const bf16_t* __restrict__ cs,
+                                                           const bf16_t* __restrict__ sn) {
   __shared__ __attribute__((aligned(1024))) uint8_t st0[2 * TILE];
   __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
@@ -541,15 +565,7 @@ __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, A
   }
 
   bf16_t* dqp = dq.p + b * dq.sb + h * dq.sh + (long)myq * dq.st;
-#pragma unroll
-  for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int d = dt * 32 + 8 * j + 4 * lh;
-      u32x2 w = {pack2bf(dqa[dt][4 * j] * scale, dqa[dt][4 * j + 1] * scale),
-                 pack2bf(dqa[dt][4 * j + 2] * scale, dqa[dt][4 * j + 3] * scale)};
-      *(u32x2*)(dqp + d) = w;
-    }
+  store_grad_row(dqa, scale, dqp, cs, sn, myq, lh);
 }
 
 AttnT mk(const void* p, const long* s) { return AttnT{(bf16_t*)p, s[0], s[1], s[2]}; }
@@ -565,20 +581,21 @@ int tfb_attn64_fwd_impl(const void* q, const long* qs, const void* k, const long
   return TFB_OK;
 }
 
-// stats: fp32 [2][B*H][T] scratch (-delta, then -lse / scale).
+// stats: fp32 [2][B*H][T] scratch (-delta, then -lse / scale). cos_t / sin_t: bf16 [T][32] or null; when given, dq and dk
+// leave the kernels with the inverse RoPE rotation applied (the gradient w.r.t. the un-rotated projections).
 int tfb_attn64_bwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
                         const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs, void* dk,
                         const long* dks, void* dv, const long* dvs, const float* lse, float* stats, int B, int H, int T,
-                        float scale, hipStream_t s) {
+                        float scale, const void* cos_t, const void* sin_t, hipStream_t s) {
   const long rows = (long)B * H * T;
   hipLaunchKernelGGL(attn64_delta_kernel, dim3((unsigned)((rows * 4 + 255) / 256)), dim3(256), 0, s, mk(o, os), mk(go, gos), lse,
                      stats, T, H, rows, 1.0f / scale);
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(attn64_dkdv_kernel, dim3(T / 128, B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
-                     mk(dk, dks), mk(dv, dvs), stats, rows, T, H, scale, scale * LOG2E);
+                     mk(dk, dks), mk(dv, dvs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t);
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(attn64_dq_kernel, dim3(T / 128, B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
-                     mk(dq, dqs), stats, rows, T, H, scale, scale * LOG2E);
+                     mk(dq, dqs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

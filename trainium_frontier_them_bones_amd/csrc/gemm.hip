@@ -23,6 +23,35 @@ int run(GemmOperand P, GemmOperand Q, int N, int M, int K, void* C, int out_f32,
   return splitk_reduce(ws, C, (long)M * N, splits, out_f32, accumulate, stream);
 }
 
+// out [q][ld] = bf16(D) with the rotary embedding applied to the first rot_cols columns (heads of 64: y1 = x1 c + x2 s,
+// y2 = x2 c - x1 s on the bf16-rounded products, rounded again - what tfb_rope computes from the stored projection).
+struct EpiStoreRope {
+  static constexpr bool kPartner32 = true;
+  bf16_t* out;
+  long ld;
+  const bf16_t* cs;  // [T][32]
+  const bf16_t* sn;
+  int T, rot_cols;
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const float (&vp)[8], int) const {
+    u32x4 x = pack8bf(v);
+    if (p < rot_cols) {
+      const u32x4 y = pack8bf(vp);
+      const int t = q % T, idx = p & 31;
+      const bool low = (p & 32) == 0;
+      const u32x4 c = *(const u32x4*)(cs + (long)t * 32 + idx), s = *(const u32x4*)(sn + (long)t * 32 + idx);
+      u32x4 o;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float x0 = bflo(x[k]), x1 = bfhi(x[k]), y0 = bflo(y[k]), y1 = bfhi(y[k]);
+        const float c0 = bflo(c[k]), c1 = bfhi(c[k]), s0 = bflo(s[k]), s1 = bfhi(s[k]);
+        o[k] = low ? pack2bf(x0 * c0 + y0 * s0, x1 * c1 + y1 * s1) : pack2bf(x0 * c0 - y0 * s0, x1 * c1 - y1 * s1);
+      }
+      x = o;
+    }
+    *(u32x4*)(out + (long)q * ld + p) = x;
+  }
+};
+
 }  // namespace
 
 extern "C" int tfb_gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int trans_a, int trans_b,
@@ -41,4 +70,18 @@ extern "C" int tfb_gemm_bf16(const void* A, const void* B, void* C, int M, int N
   if (!trans_b && !trans_a) return run<TFB_K_STRIDED, TFB_K_CONTIG>(P, Q, N, M, K, C, out_f32, accumulate, ws, workspace_bytes, s);
   if (!trans_b && trans_a) return run<TFB_K_STRIDED, TFB_K_STRIDED>(P, Q, N, M, K, C, out_f32, accumulate, ws, workspace_bytes, s);
   return run<TFB_K_CONTIG, TFB_K_STRIDED>(P, Q, N, M, K, C, out_f32, accumulate, ws, workspace_bytes, s);
+}
+
+// qkv [M][N] = rope(x [M][K] @ w [N][K]^T): the fused attention projection with the rotary embedding of the q and k
+// thirds (the first rot_cols columns, heads of 64 elements) applied in the GEMM epilogue; row m is token m % T.
+// cos_t, sin_t: bf16 [T][32]. The output equals tfb_gemm_bf16 followed by tfb_rope bit for bit.
+extern "C" int tfb_qkv_rope_fwd(const void* x, const void* w, const void* cos_t, const void* sin_t, void* out, int M, int N,
+                                int K, int T, int rot_cols, void* stream) {
+  if (!x || !w || !cos_t || !sin_t || !out) return TFB_ERR_ARG;
+  if (M <= 0 || N <= 0 || K <= 0 || M % 128 || N % 128 || K % 64 || T <= 0 || rot_cols < 0 || rot_cols > N || rot_cols % 64)
+    return TFB_ERR_SHAPE;
+  using Cfg = GemmCfg<128, 128, 2, 2, 2, TFB_K_CONTIG, TFB_K_CONTIG>;
+  GemmOperand P{(const uint8_t*)w, (long)K * 2}, Q{(const uint8_t*)x, (long)K * 2};
+  EpiStoreRope e{(bf16_t*)out, (long)N, (const bf16_t*)cos_t, (const bf16_t*)sin_t, T, rot_cols};
+  return gemm_launch<Cfg>(P, Q, N, M, (long)K * 2, 1, LoadIdentity{}, LoadIdentity{}, e, (hipStream_t)stream);
 }

@@ -224,6 +224,14 @@ __device__ __forceinline__ Epi epi_for_group(const Epi& e, int g) {
   else return e;
 }
 
+// A staged epilogue with the static member kPartner32 also receives the 8 values 32 output columns away (p ^ 32: the
+// other half of a 64-wide head, for rotary embeddings): operator()(p, q, v, v_partner, split). Needs a wavefront slice
+// of exactly 64 staged columns.
+template <class T, class = void>
+struct has_partner32 : std::false_type {};
+template <class T>
+struct has_partner32<T, std::void_t<decltype(T::kPartner32)>> : std::true_type {};
+
 template <class T, class = void>
 struct has_tile_epilogue : std::false_type {};
 template <class T>
@@ -242,8 +250,12 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   const int wp = wave % Cfg::WP, wq = wave / Cfg::WP;
   const int lr = lane & 31, lh = lane >> 5;
 
+  // An XCD's run of tiles walks the smaller operand's tiles fastest: the run then shares few rows of the larger
+  // operand (which is thereby partitioned over the XCDs' L2s) and re-reads the smaller one.
   const int lid = xcd_remap(blockIdx.x, gridDim.x);
-  const int tile_p = lid % a.ntp, tile_q = lid / a.ntp;
+  const int ntq = a.nq / BQ;
+  const bool p_fast = a.np <= a.nq || a.q_group;
+  const int tile_p = p_fast ? lid % a.ntp : lid / ntq, tile_q = p_fast ? lid / a.ntp : lid % ntq;
   const long p0 = (long)tile_p * BP, q0 = (long)tile_q * BQ;
   long kt0 = (long)blockIdx.z * a.nkt / gridDim.z;
   a.nkt = (int)((long)(blockIdx.z + 1) * a.nkt / gridDim.z - kt0);
@@ -397,7 +409,15 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
           f32x4 lo = *(const f32x4*)(stage + row * SLD + pc);
           f32x4 hi = *(const f32x4*)(stage + row * SLD + pc + 4);
           const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          epi((int)p0 + pw + i0 * 32 + pc, (int)q0 + qw + j * 32 + row, v, (int)blockIdx.z);
+          if constexpr (has_partner32<Epi>::value) {
+            static_assert(ETP == 2 && TP == 2, "partner epilogue: 64 staged columns per wavefront");
+            f32x4 plo = *(const f32x4*)(stage + row * SLD + (pc ^ 32));
+            f32x4 phi = *(const f32x4*)(stage + row * SLD + (pc ^ 32) + 4);
+            const float vp[8] = {plo[0], plo[1], plo[2], plo[3], phi[0], phi[1], phi[2], phi[3]};
+            epi((int)p0 + pw + pc, (int)q0 + qw + j * 32 + row, v, vp, (int)blockIdx.z);
+          } else {
+            epi((int)p0 + pw + i0 * 32 + pc, (int)q0 + qw + j * 32 + row, v, (int)blockIdx.z);
+          }
         }
         __builtin_amdgcn_wave_barrier();
       }

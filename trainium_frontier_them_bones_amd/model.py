@@ -138,8 +138,11 @@ class GPT:
         x = A.EmbeddingFn.apply(idx, p["wte"])
         h = A.RMSNormFn.apply(x, p["norm1.0"], cfg.norm_eps)
         for i in range(cfg.n_layer):
-            qkv = A.LinearFn.apply(h, p["w_qkv.%d" % i])
-            att = A.RopeAttentionFn.apply(qkv, self.cos[:T], self.sin[:T], cfg.n_head, scale)
+            if cfg.head_dim == 64:   # rotation fused into the projection's epilogue and the backward kernels' stores
+                att = A.QkvRopeAttentionFn.apply(h, p["w_qkv.%d" % i], self.cos[:T], self.sin[:T], cfg.n_head, scale)
+            else:
+                qkv = A.LinearFn.apply(h, p["w_qkv.%d" % i])
+                att = A.RopeAttentionFn.apply(qkv, self.cos[:T], self.sin[:T], cfg.n_head, scale)
             att = A.LinearFn.apply(att, p["w_o.%d" % i])
             x, h = A.AddRMSNormFn.apply(x, att, p["norm2.%d" % i], cfg.norm_eps)
             m = A.Mlp8Fn.apply(h, p["w_fc.%d" % i], p["w_proj.%d" % i], self.mlp_state[i])

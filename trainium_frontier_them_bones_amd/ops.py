@@ -64,6 +64,17 @@ def matmul(a, b, trans_a=False, trans_b=False, out=None, accumulate=False, out_d
     return out
 
 
+def qkv_rope(x2, w, cos, sin, T, rot_cols):
+    """rope(x2 @ w^T): the fused attention projection [M, N] with the rotary embedding of its first rot_cols columns
+    (heads of 64) applied in the GEMM epilogue; row m is token m % T."""
+    _chk(x2), _chk(w), _chk(cos), _chk(sin)
+    M, K = x2.shape
+    N = w.shape[0]
+    out = torch.empty(M, N, dtype=bf16, device=x2.device)
+    _lib.call("tfb_qkv_rope_fwd", _p(x2), _p(w), _p(cos), _p(sin), _p(out), M, N, K, T, rot_cols, _stream())
+    return out
+
+
 # ------------------------------------------------------------------------------------------ norms
 def rmsnorm_fwd(x, weight=None, eps=2.0 ** -23, res=None):
     """y = RMSNorm(s) * weight with s = x (res None) or bf16(x + res). Returns (s, y, inv[rows] fp32)."""
@@ -266,9 +277,10 @@ def attn_fwd(q, k, v, scale, layout="bhtd"):
     return o, lse
 
 
-def attn_bwd(q, k, v, o, do, lse, scale, layout="bhtd", dq=None, dk=None, dv=None, out_layout="bhtd"):
+def attn_bwd(q, k, v, o, do, lse, scale, layout="bhtd", dq=None, dk=None, dv=None, out_layout="bhtd", rope=None):
     """Gradients of attn_fwd. o, do are [B,T,H,D]. dq/dk/dv may be given as (strided) views with `out_layout`;
-    otherwise dq, dk are allocated [B,H,T,D] and dv [B,T,H,D] (returned as a [B,H,T,D] view), as the reference returns."""
+    otherwise dq, dk are allocated [B,H,T,D] and dv [B,T,H,D] (returned as a [B,H,T,D] view), as the reference returns.
+    rope = (cos, sin) (bf16 [T, D/2]): dq and dk come back with the inverse rotation applied (D = 64)."""
     for t in (q, k, v, o, do):
         _attn_chk(t)
     if layout == "bhtd":
@@ -281,9 +293,11 @@ def attn_bwd(q, k, v, o, do, lse, scale, layout="bhtd", dq=None, dk=None, dv=Non
         dv = torch.empty(B, T, H, D, dtype=bf16, device=q.device).permute(0, 2, 1, 3)
         out_layout = "bhtd"
     delta = torch.empty(2, B, H, T, dtype=torch.float32, device=q.device)
-    _lib.call("tfb_attn_bwd", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o), _bht(o, "bthd"),
-              _p(do), _bht(do, "bthd"), _p(dq), _bht(dq, out_layout), _p(dk), _bht(dk, out_layout), _p(dv),
-              _bht(dv, out_layout), _p(lse), _p(delta), B, H, T, D, float(scale), _stream())
+    cos, sin = rope if rope is not None else (None, None)
+    _chk(cos), _chk(sin)
+    _lib.call("tfb_attn_bwd_rope", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o),
+              _bht(o, "bthd"), _p(do), _bht(do, "bthd"), _p(dq), _bht(dq, out_layout), _p(dk), _bht(dk, out_layout), _p(dv),
+              _bht(dv, out_layout), _p(lse), _p(delta), _p(cos), _p(sin), B, H, T, D, float(scale), _stream())
     return dq, dk, dv
 
 
