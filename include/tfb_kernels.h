@@ -136,6 +136,16 @@ int tfb_mlp8_fwd(const void* x8, const void* w8, const void* row, void* y, void*
 int tfb_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* row, void* dx, void* h, void* dpre, void* dp8,
                  long M, int d, int F, void* stream);
 
+/* ---- fp8 projections (attention QKV / output projection in fp8) -----------------------------------------------------
+ * out8 [R][C], outT8 [C][R] = e4m3(w [R][C] * *scale_ptr): a weight pre-cast once per optimizer step in both byte layouts.
+ * Replaces precast_ref (round2/source/kernels/nki_attn_tt8g.py:795). */
+int tfb_precast8(const void* w, const void* scale_ptr, void* out8, void* outT8, int R, int C, void* stream);
+/* out [M][N] bf16 = bf16((a8 [M][K] @ b8 [N][K]^T) * dq), a8 e4m3 (fmt_a 0) or e5m2 (fmt_a 1), b8 e4m3;
+ * dq = dq_imm * *dq_a * *dq_b (device fp32 scalars or NULL). M, N, K % 128 == 0.
+ * Replaces _proj8_fwd_kernel / _proj8_bwd_kernel (emulate_fwd, emulate_bwd: nki_attn_tt8g.py:745-757). */
+int tfb_gemm_fp8(const void* a8, int fmt_a, const void* b8, const void* dq_a, const void* dq_b, float dq_imm, void* out,
+                 long M, int N, int K, void* stream);
+
 /* dw [d][F] (+)= dy^T @ bf16(r^2) (bf16 GEMM over the tokens, h never materialised). workspace fp32 split-K scratch.
  * Replaces the dw_proj half of weight_grads (nki_mlp_fused8.py:706-711) / l4_weight_grads (nki_mlp_l4t.py:932). */
 int tfb_mlp_dw_proj(const void* dy, const void* r, void* dw, long M, int d, int F, int out_f32, int accumulate,

@@ -37,6 +37,8 @@ SIGNATURES = {
     "tfb_attn_bwd_rope": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _vp, _vp, _vp,
                           _i, _i, _i, _i, _f, _vp],
     "tfb_qkv_rope_fwd": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "tfb_precast8": [_vp, _vp, _vp, _vp, _i, _i, _vp],
+    "tfb_gemm_fp8": [_vp, _i, _vp, _vp, _vp, _f, _vp, _l, _i, _i, _vp],
     "tfb_relu2": [_vp, _vp, _vp, _l, _i, _vp],
     "tfb_rope": [_vp, _vp, _vp, _vp, _l, _i, _i, _i, _l, _l, _i, _vp],
     "tfb_resmix_bwd_blocks": [_l],

@@ -204,6 +204,56 @@ class QkvRopeAttentionFn(torch.autograd.Function):
         return dx, ops.matmul(g2, x2, trans_a=True), None, None, None, None
 
 
+class Linear8State:
+    """Per-weight fp8 state of a projection, refreshed once per optimizer step: the weight's power-of-two scale
+    (s, 1/s, amax on the device) and its e4m3 bytes in both layouts (forward_scales / precast_ref,
+    round2/source/kernels/nki_attn_tt8g.py:700, 795)."""
+
+    def __init__(self, limit=240.0):
+        self.limit = limit
+        self.sc = None
+        self.w8 = self.w8t = None
+
+    def refresh(self, w):
+        self.sc = ops.amax_scale(w.detach(), self.limit, -24, 40)
+        self.w8, self.w8t = ops.precast8(w.detach(), self.sc[0:1])
+
+
+class Linear8Fn(torch.autograd.Function):
+    """y = x @ w^T with the forward in e4m3 x e4m3 and the input gradient in e5m2 x e4m3 (per-tensor power-of-two
+    scales, fp32 accumulation, one bf16 rounding), the weight gradient in bf16 (accumulated into w.grad_buf when
+    present). x_scale: the reference's constant (4 for an RMSNorm output) or None for the per-tensor amax scale of x.
+    The arithmetic of emulate_fwd / emulate_bwd (nki_attn_tt8g.py:745-757)."""
+
+    @staticmethod
+    def forward(ctx, x, w, state, x_scale):
+        x2 = x.reshape(-1, x.shape[-1]).contiguous()
+        if x_scale is None:
+            sx = ops.amax_scale(x2, state.limit, -24, 40)
+            x8 = ops.quant_fp8(x2, sx[0:1], ops.FMT_E4M3)
+            y = ops.gemm_fp8(x8, state.w8, ops.FMT_E4M3, sx[1:2], state.sc[1:2])
+        else:
+            x8 = ops.quant_fp8(x2, float(x_scale), ops.FMT_E4M3)
+            y = ops.gemm_fp8(x8, state.w8, ops.FMT_E4M3, None, state.sc[1:2], 1.0 / float(x_scale))
+        ctx.save_for_backward(x2, w)
+        ctx.state, ctx.xshape = state, x.shape
+        return y.view(*x.shape[:-1], w.shape[0])
+
+    @staticmethod
+    def backward(ctx, gy):
+        x2, w = ctx.saved_tensors
+        st = ctx.state
+        g2 = gy.reshape(-1, gy.shape[-1]).contiguous()
+        sg = ops.amax_scale(g2, 57344.0 / 2.0, -40, 60)
+        g8 = ops.quant_fp8(g2, sg[0:1], ops.FMT_E5M2)
+        dx = ops.gemm_fp8(g8, st.w8t, ops.FMT_E5M2, sg[1:2], st.sc[1:2]).view(ctx.xshape)
+        buf, acc = _accumulate_into(w)
+        if buf is not None:
+            ops.matmul(g2, x2, trans_a=True, out=buf, accumulate=acc)
+            return dx, None, None, None
+        return dx, ops.matmul(g2, x2, trans_a=True), None, None
+
+
 class Mlp8State:
     """Per-layer fp8 state refreshed once per optimizer step: the scale row and the e4m3 weight pack
     (round2/source/train.py:6617 fp8_refresh_weights, 7003 mlp8_scales_into, 7267 mlp8_precast_into)."""

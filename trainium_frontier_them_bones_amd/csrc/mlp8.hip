@@ -340,6 +340,23 @@ struct EpiScaleStore {  // out = bf16(acc * sc[col])
   }
 };
 
+struct EpiDescale {  // out = bf16(acc * dq), dq = dq_imm * *dq_a * *dq_b (absent factors are 1)
+  const float* dq_a;
+  const float* dq_b;
+  float dq_imm;
+  bf16_t* out;
+  long ld;
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
+    float dq = dq_imm;
+    if (dq_a) dq *= *dq_a;
+    if (dq_b) dq *= *dq_b;
+    float r[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = v[i] * dq;
+    *(u32x4*)(out + (long)q * ld + p) = pack8bf(r);
+  }
+};
+
 struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*s_dp), optional h = bf16(r^2)
   const float* sc;
   const bf16_t* r;  // [M][F]
@@ -487,8 +504,34 @@ extern "C" int tfb_mlp8_precast(const void* w_fc, const void* w_proj, const void
   return TFB_OK;
 }
 
+// w [R][C] bf16 -> out8 [R][C] and outT8 [C][R], both e4m3(w * *scale_ptr): the two byte layouts a projection's forward
+// (contraction over C) and input-gradient (contraction over R) GEMMs read k-contiguously.
+extern "C" int tfb_precast8(const void* w, const void* scale_ptr, void* out8, void* outT8, int R, int C, void* stream) {
+  if (!w || !scale_ptr || !out8 || !outT8) return TFB_ERR_ARG;
+  if (R <= 0 || C <= 0 || R % 64 || C % 64) return TFB_ERR_SHAPE;
+  hipLaunchKernelGGL(precast_kernel, dim3(C / 64, R / 64), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)w,
+                     (const float*)scale_ptr, (uint8_t*)out8, (uint8_t*)outT8, R, C);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
 using Cfg8 = GemmCfg<128, 128, 2, 2, 1, TFB_K_CONTIG, TFB_K_CONTIG, TFB_FMT_E4M3, TFB_FMT_E4M3>;
 using Cfg8g = GemmCfg<128, 128, 2, 2, 1, TFB_K_CONTIG, TFB_K_CONTIG, TFB_FMT_E4M3, TFB_FMT_E5M2>;
+
+// out [M][N] bf16 = bf16((a8 [M][K] @ b8 [N][K]^T) * dq): the fp8 projection GEMM. a8 is e4m3 (fmt_a 0: forward
+// activations) or e5m2 (fmt_a 1: gradients); b8 is e4m3 (a pre-cast weight layout). dq = dq_imm * *dq_a * *dq_b, the
+// pointers being device fp32 scalars (inverse power-of-two scales) or null.
+extern "C" int tfb_gemm_fp8(const void* a8, int fmt_a, const void* b8, const void* dq_a, const void* dq_b, float dq_imm,
+                            void* out, long M, int N, int K, void* stream) {
+  if (!a8 || !b8 || !out) return TFB_ERR_ARG;
+  if (fmt_a != TFB_FMT_E4M3 && fmt_a != TFB_FMT_E5M2) return TFB_ERR_ARG;
+  if (M <= 0 || N <= 0 || K <= 0 || M % 128 || N % 128 || K % 128 || M > 0x7fffffffL) return TFB_ERR_SHAPE;
+  GemmOperand P{(const uint8_t*)b8, (long)K}, Q{(const uint8_t*)a8, (long)K};
+  EpiDescale e{(const float*)dq_a, (const float*)dq_b, dq_imm, (bf16_t*)out, (long)N};
+  if (fmt_a == TFB_FMT_E4M3)
+    return gemm_launch<Cfg8>(P, Q, N, (int)M, (long)K, 1, LoadIdentity{}, LoadIdentity{}, e, (hipStream_t)stream);
+  return gemm_launch<Cfg8g>(P, Q, N, (int)M, (long)K, 1, LoadIdentity{}, LoadIdentity{}, e, (hipStream_t)stream);
+}
 
 // Forward: x8 [M][d] e4m3 (already cast at s_x), w8 pack, row -> y [M][d] bf16, r [M][F] bf16, h8 [M][F] e4m3 scratch.
 extern "C" int tfb_mlp8_fwd(const void* x8, const void* w8, const void* row, void* y, void* r, void* h8, long M, int d, int F,

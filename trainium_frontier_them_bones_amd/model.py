@@ -32,6 +32,7 @@ class GPTConfig:
     init_std: float = 0.02
     e4m3_limit: float = 240.0     # fp8 scale search limit (240 = the reference's rows, 448 = OCP maximum)
     x_scale: float = 4.0          # constant activation scale of the fp8 MLP input (a unit-RMS norm output)
+    fp8_attn_proj: bool = False   # QKV and output projections in fp8 (e4m3 forward, e5m2 dX, bf16 dW); off in BASELINE C4
 
     @property
     def head_dim(self):
@@ -105,6 +106,8 @@ class GPT:
         self.p.update(self.mats.params)
         self.p.update(self.others.params)
         self.mlp_state = [A.Mlp8State(cfg.e4m3_limit, cfg.x_scale) for _ in range(L)]
+        self.qkv_state = [A.Linear8State(cfg.e4m3_limit) for _ in range(L)] if cfg.fp8_attn_proj else None
+        self.wo_state = [A.Linear8State(cfg.e4m3_limit) for _ in range(L)] if cfg.fp8_attn_proj else None
         self.cos, self.sin = rope_tables(cfg.seq_len, cfg.head_dim, cfg.rope_base, device)
         self.step_count = 0
         self.init_weights(seed)
@@ -130,6 +133,10 @@ class GPT:
         """Per-optimizer-step refresh of each layer's fp8 scale row and e4m3 weight pack."""
         for i, st in enumerate(self.mlp_state):
             st.refresh(self.p["w_fc.%d" % i], self.p["w_proj.%d" % i])
+        if self.qkv_state is not None:
+            for i in range(self.cfg.n_layer):
+                self.qkv_state[i].refresh(self.p["w_qkv.%d" % i])
+                self.wo_state[i].refresh(self.p["w_o.%d" % i])
 
     def forward(self, idx, targets):
         cfg, p = self.cfg, self.p
@@ -138,12 +145,17 @@ class GPT:
         x = A.EmbeddingFn.apply(idx, p["wte"])
         h = A.RMSNormFn.apply(x, p["norm1.0"], cfg.norm_eps)
         for i in range(cfg.n_layer):
-            if cfg.head_dim == 64:   # rotation fused into the projection's epilogue and the backward kernels' stores
-                att = A.QkvRopeAttentionFn.apply(h, p["w_qkv.%d" % i], self.cos[:T], self.sin[:T], cfg.n_head, scale)
-            else:
-                qkv = A.LinearFn.apply(h, p["w_qkv.%d" % i])
+            if cfg.fp8_attn_proj:    # h is an RMSNorm output (constant scale 4); the attention output takes its amax scale
+                qkv = A.Linear8Fn.apply(h, p["w_qkv.%d" % i], self.qkv_state[i], cfg.x_scale)
                 att = A.RopeAttentionFn.apply(qkv, self.cos[:T], self.sin[:T], cfg.n_head, scale)
-            att = A.LinearFn.apply(att, p["w_o.%d" % i])
+                att = A.Linear8Fn.apply(att, p["w_o.%d" % i], self.wo_state[i], None)
+            else:
+                if cfg.head_dim == 64:   # rotation fused into the projection's epilogue and the backward kernels' stores
+                    att = A.QkvRopeAttentionFn.apply(h, p["w_qkv.%d" % i], self.cos[:T], self.sin[:T], cfg.n_head, scale)
+                else:
+                    qkv = A.LinearFn.apply(h, p["w_qkv.%d" % i])
+                    att = A.RopeAttentionFn.apply(qkv, self.cos[:T], self.sin[:T], cfg.n_head, scale)
+                att = A.LinearFn.apply(att, p["w_o.%d" % i])
             x, h = A.AddRMSNormFn.apply(x, att, p["norm2.%d" % i], cfg.norm_eps)
             m = A.Mlp8Fn.apply(h, p["w_fc.%d" % i], p["w_proj.%d" % i], self.mlp_state[i])
             nw = p["norm1.%d" % (i + 1)] if i + 1 < cfg.n_layer else p["norm_f"]

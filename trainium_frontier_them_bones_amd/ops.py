@@ -193,6 +193,29 @@ def quant_fp8(x, scale, fmt=FMT_E4M3):
     return out
 
 
+def precast8(w, scale):
+    """(w8 [R,C], w8T [C,R]) uint8: e4m3(w * scale) in both byte layouts; scale a 1-element fp32 device tensor."""
+    _chk(w), _chk(scale, torch.float32)
+    R, C = w.shape
+    w8 = torch.empty(R, C, dtype=torch.uint8, device=w.device)
+    w8t = torch.empty(C, R, dtype=torch.uint8, device=w.device)
+    _lib.call("tfb_precast8", _p(w), _p(scale), _p(w8), _p(w8t), R, C, _stream())
+    return w8, w8t
+
+
+def gemm_fp8(a8, b8, fmt_a=FMT_E4M3, dq_a=None, dq_b=None, dq=1.0):
+    """bf16 [M,N] = (a8 [M,K] @ b8 [N,K]^T) * dq * dq_a * dq_b; a8 e4m3 or e5m2 bytes, b8 e4m3 bytes; dq_a, dq_b
+    1-element fp32 device tensors (or None)."""
+    _chk(a8, torch.uint8), _chk(b8, torch.uint8), _chk(dq_a, torch.float32), _chk(dq_b, torch.float32)
+    M, K = a8.shape
+    N = b8.shape[0]
+    if b8.shape[1] != K:
+        raise ValueError("inner dimensions differ")
+    out = torch.empty(M, N, dtype=bf16, device=a8.device)
+    _lib.call("tfb_gemm_fp8", _p(a8), int(fmt_a), _p(b8), _p(dq_a), _p(dq_b), float(dq), _p(out), M, N, K, _stream())
+    return out
+
+
 def mlp8_precast(w_fc, w_proj, row):
     """uint8 [4, F*d]: w_fc and w_proj cast once to e4m3 at the row's scales, each in both byte layouts."""
     _chk(w_fc), _chk(w_proj), _chk(row, torch.float32)
