@@ -18,6 +18,9 @@
 #include "common.hpp"
 
 // wavefronts per SIMD the kernels are compiled for (register budget 512 / n)
+#ifndef TFB_DKDV64_QT
+#define TFB_DKDV64_QT 2
+#endif
 #ifndef TFB_DQ64_WPE
 #define TFB_DQ64_WPE 2
 #endif
@@ -69,21 +72,22 @@ __device__ __forceinline__ void xcd_block(int nx, int nbh, int& bx, int& bh) {
 
 __device__ __forceinline__ int swz(int t) { return (((t >> 1) & 1) << 2) | ((t >> 2) & 3); }
 
-// This wavefront's share (2 of the 8 instructions) of a 64-token tile load. `rows` points at token 0 of the tile,
-// `stride` = bytes between tokens.
+// This wavefront's share (NI of the 4 NI instructions) of a (32 NI)-token tile load. `rows` points at token 0 of the
+// tile, `stride` = bytes between tokens.
+template <int NI>
 struct TileLoad {
   uint32_t voff;
   int wave;
   __device__ __forceinline__ void init(long stride, int wave_, int lane) {
     wave = wave_;
     const int lrow = lane >> 3;
-    // token = 8 g + lrow with g = wave or wave + 4: swz depends on g only through g & 1 = wave & 1
+    // token = 8 g + lrow with g = wave + 4 i: swz depends on g only through g & 1 = wave & 1
     const int chunk = (lane & 7) ^ swz(8 * wave + lrow);
     voff = (uint32_t)(lrow * stride + chunk * 16);
   }
   __device__ __forceinline__ void issue(const uint8_t* rows, long stride, uint8_t* lds) const {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NI; ++i) {
       const int g = wave + 4 * i;
       __builtin_amdgcn_global_load_lds((glb_void_t*)(rows + 8L * g * stride + (size_t)voff), (lds_void_t*)(lds + g * 1024), 16,
                                        0, 0);
@@ -163,7 +167,7 @@ __global__ __launch_bounds__(256, TFB_FWD64_WPE) void attn64_fwd_kernel(AttnT q,
 #pragma unroll
   for (int s = 0; s < 4; ++s) qf[s] = *(const bf16x8*)(qp + (long)(qw0 + lr) * q.st + 16 * s + 8 * lh);
 
-  TileLoad lk, lv;
+  TileLoad<2> lk, lv;
   lk.init(kst, wave, lane);
   lv.init(vst, wave, lane);
   auto issue = [&](uint8_t* st, int tile) {
@@ -316,7 +320,9 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
                                                              const float* __restrict__ stats, long rows, int T, int H,
                                                              float scale, float sl2, const bf16_t* __restrict__ cs,
                                                              const bf16_t* __restrict__ sn) {
-  constexpr int STAGE = 2 * TILE + 512;  // Q tile, dO tile, 64 x (-lse / scale), 64 x (-delta)
+  constexpr int QT = TFB_DKDV64_QT;       // 64-query tiles per LDS stage (one barrier per stage)
+  constexpr int R = 64 * QT, RT = R * 128;  // rows and bytes of a staged Q (dO) tile
+  constexpr int STAGE = 2 * RT + 8 * R;    // Q tile, dO tile, R x (-lse / scale), R x (-delta)
   __shared__ __attribute__((aligned(1024))) uint8_t st0[STAGE];
   __shared__ __attribute__((aligned(1024))) uint8_t st1[STAGE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
@@ -340,18 +346,21 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
     vf[s] = *(const bf16x8*)(vp + (long)mykey * v.st + 16 * s + 8 * lh);
   }
 
-  TileLoad lq, lg;
+  TileLoad<2 * QT> lq, lg;
   lq.init(qst, wave, lane);
   lg.init(gst, wave, lane);
-  const int qt0 = kb * 2, n = T / 64 - qt0;
+  const int qt0 = kb * 2, n = (T / 64 - qt0) / QT;  // T / 64 - 2 kb is even
   auto issue = [&](uint8_t* st, int i) {
-    const long r0 = (long)(qt0 + i) * 64;
+    const long r0 = (long)qt0 * 64 + (long)i * R;
     lq.issue(qp + r0 * qst, qst, st);
-    lg.issue(gp + r0 * gst, gst, st + TILE);
-    // the row statistics: 64 floats each, one 4-byte load per lane (wavefront 0: -lse / scale, wavefront 1: -delta)
+    lg.issue(gp + r0 * gst, gst, st + RT);
+    // the row statistics: R floats each, 4-byte loads (wavefront 0: -lse / scale, wavefront 1: -delta)
     if (wave < 2) {
       const float* src = (wave == 0 ? nlp : delp) + r0;
-      __builtin_amdgcn_global_load_lds((glb_void_t*)(src + lane), (lds_void_t*)(st + 2 * TILE + wave * 256), 4, 0, 0);
+#pragma unroll
+      for (int x = 0; x < QT; ++x)
+        __builtin_amdgcn_global_load_lds((glb_void_t*)(src + 64 * x + lane), (lds_void_t*)(st + 2 * RT + wave * 4 * R + 256 * x),
+                                         4, 0, 0);
     }
   };
 
@@ -366,11 +375,11 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
 
   auto compute = [&](const uint8_t* st, int i) {
     const uint8_t* qt_ = st;
-    const uint8_t* gt_ = st + TILE;
-    const float* ls = (const float*)(st + 2 * TILE);
-    const int qbase = (qt0 + i) * 64;
+    const uint8_t* gt_ = st + RT;
+    const float* ls = (const float*)(st + 2 * RT);
+    const int qbase = qt0 * 64 + i * R;
 #pragma unroll
-    for (int qs = 0; qs < 2; ++qs) {
+    for (int qs = 0; qs < 2 * QT; ++qs) {
       const int qlo = qbase + qs * 32;
       if (qlo + 31 < kw0) continue;  // every key of this wavefront is in the future of these queries
       bf16x8 qa[4], ga[4];
@@ -384,7 +393,7 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const f32x4 L = *(const f32x4*)(ls + qs * 32 + 8 * j + 4 * lh);
-        const f32x4 Dl = *(const f32x4*)(ls + 64 + qs * 32 + 8 * j + 4 * lh);
+        const f32x4 Dl = *(const f32x4*)(ls + R + qs * 32 + 8 * j + 4 * lh);
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
           S[4 * j + x] = L[x];
@@ -449,7 +458,7 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
     compute(st1, t + 1);
     __syncthreads();
   }
-  // n = T / 64 - 2 kb is even
+  if (n & 1) compute(st0, n - 1);
 
   bf16_t* dkp = dk.p + b * dk.sb + h * dk.sh + (long)mykey * dk.st;
   bf16_t* dvp = dv.p + b * dv.sb + h * dv.sh + (long)mykey * dv.st;
@@ -486,7 +495,7 @@ __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, A
   const float myD = stats[(long)bh * T + myq];
   const float myL = stats[rows + (long)bh * T + myq];
 
-  TileLoad lk, lv;
+  TileLoad<2> lk, lv;
   lk.init(kst, wave, lane);
   lv.init(vst, wave, lane);
   auto issue = [&](uint8_t* st, int tile) {
