@@ -136,6 +136,22 @@ int tfb_mlp8_fwd(const void* x8, const void* w8, const void* row, void* y, void*
 int tfb_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* row, void* dx, void* h, void* dpre, void* dp8,
                  long M, int d, int F, void* stream);
 
+/* tfb_mlp8_bwd that also writes hq8 [M][F] = e4m3(min(bf16(r^2) * s_h, hq_limit)) (NULL to skip): the g-side operand of
+ * the fp8 weight gradient of w_proj (format E4M3C of nki_dw8.py:312-320; round2/source/train.py:8226). */
+int tfb_mlp8_bwd_q(const void* dy8, const void* r, const void* w8, const void* row, void* dx, void* h, void* dpre, void* dp8,
+                   void* hq8, float hq_limit, long M, int d, int F, void* stream);
+
+/* Both MLP weight gradients in fp8 from byte tensors the forward and backward already hold (token-major [M][.]):
+ * dw_fc [F][d] = ((dp8^T @ x8) / (s_dp * x_scale)), dp8 = e5m2(dpre s_dp) from tfb_mlp8_bwd, x8 = e4m3(x x_scale);
+ * dw_proj [d][F] = ((dy8^T @ hq8) / (s_dy * s_h)), dy8 = e5m2(dy s_dy), hq8 from tfb_mlp8_bwd_q. row = the backward row.
+ * Outputs bf16 (out_f32 = 0) or fp32, optionally accumulated into (one rounding); fp32 accumulation over all tokens;
+ * workspace >= splits * d * F * 4 bytes (256 MB always suffices). Shapes as tfb_mlp8_fwd.
+ * Replaces mlp8_weight_grads under the fp8 weight-gradient switch (round2/source/train.py:8209-8229: dw8_grad twice,
+ * nki_dw8.py:323 emulate_dw / _dw8_kernel) and R1's fp8 dW rows (round1/source/train.py:3182 run_tn_fp8). */
+int tfb_mlp8_dw8(const void* x8, const void* dp8, const void* hq8, const void* dy8, const void* row, float x_scale, void* dw_fc,
+                 void* dw_proj, long M, int d, int F, int out_f32, int accumulate, void* workspace, long workspace_bytes,
+                 void* stream);
+
 /* ---- fp8 projections (attention QKV / output projection in fp8) -----------------------------------------------------
  * out8 [R][C], outT8 [C][R] = e4m3(w [R][C] * *scale_ptr): a weight pre-cast once per optimizer step in both byte layouts.
  * Replaces precast_ref (round2/source/kernels/nki_attn_tt8g.py:795). */

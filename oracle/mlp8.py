@@ -10,7 +10,10 @@ plain bf16 relu(x @ w)^2 (R1:2128-2133), which is `reference_forward` here.
 Pinned by (tests/test_oracle_mlp8.py): the scale search against the closed form 2^floor(log2(limit / v))
 clipped to the exponent window by brute force over exponents and mantissas; s * (1/s) == 1; every e4m3 value up
 to 240 surviving a bf16 round trip; the fp8 cast against an independent bit-level rounding routine; the fp8
-MLP against the bf16 MLP within the fp8 error budget; weight gradients against torch.autograd of the bf16 form.
+MLP against the bf16 MLP within the fp8 error budget; weight gradients against torch.autograd of the bf16 form; the
+fp8 weight gradients against an independent route (operands decoded byte by byte through the format tables, one
+fp64 matmul), against the bf16 weight gradients within the fp8 budget, and by exact invariance under power-of-two
+rescaling of the operands.
 """
 import torch
 
@@ -174,3 +177,15 @@ def fp8_weight_grad(g2, a2, s_g, s_a, dq, fmt_g, fmt_a, clamp_g=None):
     if clamp_g is not None:
         g = torch.clamp_max(g, clamp_g)
     return ((fp8_round(g, fmt_g).t() @ fp8_round(a2.float() * s_a, fmt_a)) * dq).to(g2.dtype)
+
+
+def weight_grads_fp8(x2, dy2, h, dpre, row, x_scale=X_SCALE, e4m3_limit=E4M3_LIMIT_REF):
+    """(dw_fc [F, d], dw_proj [d, F]) in fp8 (round2/source/train.py:8209-8229 mlp8_weight_grads under its fp8
+    weight-gradient switch): dw_fc = dpre^T x with dpre e5m2 at s_dp (the bytes the backward's second GEMM
+    multiplies) and x e4m3 at x_scale (the forward's), dw_proj = (h^T dy)^T with h e4m3 at s_h clamped at the format's
+    limit and dy e5m2 at s_dy; descales are the exact inverse powers of two. row = the backward row."""
+    s_dp, s_h, s_dy = row[COL["s_dp"]], row[COL["s_h"]], row[COL["s_dy"]]
+    dw_fc = fp8_weight_grad(dpre, x2, s_dp, x_scale, 1.0 / (s_dp * x_scale), 1, 0)
+    dw_pt = fp8_weight_grad(h, dy2, s_h, s_dy, 1.0 / (s_h * s_dy), 0, 1, clamp_g=e4m3_limit)
+    return dw_fc, dw_pt.t().contiguous()
+

@@ -216,6 +216,52 @@ def test_mlp8_scales_precast_forward_backward(ops, dev, shape, limit):
     assert st[0].item() == rowb_o[5].item() and st[2].item() == dy.float().abs().max().item()
 
 
+@pytest.mark.parametrize("shape", [(256, 256, 512), (1024, 768, 3072), (4096, 768, 3072)])
+@pytest.mark.parametrize("limit", [240.0, 448.0])
+def test_mlp8_fp8_weight_grads(ops, dev, shape, limit):
+    """tfb_mlp8_bwd_q + tfb_mlp8_dw8 against the oracle's fp8 weight gradients; the operand bytes bit for bit."""
+    from oracle import mlp8 as O
+    from helpers import fp8_table
+    M, d, F = shape
+    g = _g(7 * M + d + F)
+    x = torch.randn(M, d, generator=g).bfloat16()
+    wf = (0.02 * torch.randn(F, d, generator=g)).bfloat16()
+    wp = (0.02 * torch.randn(d, F, generator=g)).bfloat16()
+    dy = torch.randn(M, d, generator=g).bfloat16()
+    xd, wfd, wpd, dyd = x.to(dev), wf.to(dev), wp.to(dev), dy.to(dev)
+    row = ops.mlp8_forward_scales(wfd, wpd, limit)
+    w8 = ops.mlp8_precast(wfd, wpd, row)
+    y, r, x8 = ops.mlp8_fwd(xd, w8, row, F, want_x8=True)
+    rowb = ops.mlp8_backward_scales(dyd, row)
+    dx, dpre, dp8, hq8, dy8 = ops.mlp8_bwd_q(dyd, r, w8, rowb, limit)
+    dx0, _, dpre0 = ops.mlp8_bwd(dyd, r, w8, rowb, want_h=False)
+    assert torch.equal(dx, dx0) and torch.equal(dpre, dpre0)                       # the extra output changes nothing else
+    rb = rowb.cpu()
+    s_dp, s_h, s_dy = (rb[O.COL[k]] for k in ("s_dp", "s_h", "s_dy"))
+    hb = (r.cpu().float() * r.cpu().float()).bfloat16()
+    assert torch.equal(x8.cpu(), O.fp8_bytes(x.float() * 4.0, 0))
+    assert torch.equal(dy8.cpu(), O.fp8_bytes(dy.float() * s_dy, 1))
+    assert torch.equal(dp8.cpu(), O.fp8_bytes(dpre.cpu().float() * s_dp, 1))
+    assert torch.equal(hq8.cpu(), O.fp8_bytes(torch.clamp_max(hb.float() * s_h, limit), 0))
+    dw_fc, dw_proj = ops.mlp8_dw8(x8, dp8, hq8, dy8, rowb)
+    # the oracle on the same saved activations (r and dpre as the device produced them)
+    o_fc, o_pj = O.weight_grads_fp8(x, dy, hb, dpre.cpu(), rb, e4m3_limit=limit)
+    assert rel_l2(dw_fc, o_fc) < 2e-3 and rel_l2(dw_proj, o_pj) < 2e-3             # summation order + one bf16 rounding
+    # and through the byte tables, in fp64
+    t4, t5 = fp8_table("e4m3fn"), fp8_table("e5m2")
+    ref_fc = (t5[dp8.cpu().long()].t() @ t4[x8.cpu().long()]) / float(s_dp * 4.0)
+    ref_pj = (t5[dy8.cpu().long()].t() @ t4[hq8.cpu().long()]) / float(s_dy * s_h)
+    assert rel_l2(dw_fc, ref_fc) < 3e-3 and rel_l2(dw_proj, ref_pj) < 3e-3
+    # within the fp8 budget of the bf16 weight gradients
+    b_fc, b_pj = O.weight_grads(dy, x, hb, dpre.cpu())
+    assert rel_l2(dw_fc, b_fc) < 0.08 and rel_l2(dw_proj, b_pj) < 0.08
+    # fp32 outputs, accumulated into
+    acc_fc = torch.randn(F, d, generator=g)
+    acc_pj = torch.randn(d, F, generator=g)
+    a_fc, a_pj = ops.mlp8_dw8(x8, dp8, hq8, dy8, rowb, dw_fc=acc_fc.to(dev).clone(), dw_proj=acc_pj.to(dev).clone(), accumulate=True)
+    assert rel_l2(a_fc, ref_fc + acc_fc) < 1e-4 and rel_l2(a_pj, ref_pj + acc_pj) < 1e-4
+
+
 def test_mlp8_full_size_properties(ops, dev):
     """BASELINE config 3 sizes: exact equivariance under a permutation of the tokens and agreement of 512-row slices
     with the oracle."""

@@ -124,3 +124,41 @@ def test_fp8_weight_grad_close_to_bf16_weight_grad():
     out = O.fp8_weight_grad(dy, x, s_g, 4.0, 1.0 / (s_g * 4.0), 1, 0)
     ref = (dy.float().t() @ x.float()).bfloat16()
     assert rel_l2(out, ref) < 0.1
+
+
+def _decode(bytes_u8, fmt):
+    """fp8 bytes -> fp64 values through the format tables (decoded from the format definitions, not by torch's cast)."""
+    from helpers import fp8_table
+    return fp8_table("e5m2" if fmt == 1 else "e4m3fn")[bytes_u8.long()]
+
+
+def test_fp8_weight_grads_independent_route_budget_and_invariance():
+    x, wf, wp, dy = _layer(5, M=256, d=256, F=512)
+    row = O.forward_scales(wf, wp)
+    y, r = O.forward(x, wf, wp, row)
+    rowb = O.backward_scales(dy, row)
+    dx, h, dpre = O.backward(dy, r, wf, wp, rowb)
+    dw_fc, dw_proj = O.weight_grads_fp8(x, dy, h, dpre, rowb)
+    assert dw_fc.shape == wf.shape and dw_proj.shape == wp.shape and dw_fc.dtype == x.dtype
+    # (1) independent route: the operand bytes decoded through the tables, one fp64 product, the inverse scales applied
+    s_dp, s_h, s_dy = (float(rowb[O.COL[k]]) for k in ("s_dp", "s_h", "s_dy"))
+    g8 = _decode(O.fp8_bytes(dpre.float() * s_dp, 1), 1)
+    a8 = _decode(O.fp8_bytes(x.float() * 4.0, 0), 0)
+    ref_fc = (g8.t() @ a8) / (s_dp * 4.0)
+    hq = _decode(O.fp8_bytes(torch.clamp_max(h.float() * s_h, 240.0), 0), 0)
+    d8 = _decode(O.fp8_bytes(dy.float() * s_dy, 1), 1)
+    ref_pj = (d8.t() @ hq) / (s_dy * s_h)
+    assert rel_l2(dw_fc, ref_fc) < 3e-3 and rel_l2(dw_proj, ref_pj) < 3e-3   # one bf16 rounding + fp32 summation
+    # (2) the fp8 budget against the bf16 weight gradients (the reference quotes ~6 % mean relative)
+    b_fc, b_pj = O.weight_grads(dy, x, h, dpre)
+    assert rel_l2(dw_fc, b_fc) < 0.08 and rel_l2(dw_proj, b_pj) < 0.08
+    # (3) a dropped or doubled scale factor, or swapped formats, would break these: exact power-of-two covariance
+    dw2 = O.fp8_weight_grad(dpre * 4.0, x, s_dp / 4.0, 4.0, 1.0 / (s_dp * 4.0), 1, 0)
+    assert torch.equal(dw2, dw_fc)
+    dw3 = O.fp8_weight_grad(dpre, x, s_dp, 4.0, 2.0 / (s_dp * 4.0), 1, 0)
+    assert torch.equal(dw3.float(), dw_fc.float() * 2.0)
+    # (4) the clamp is on the g side only and only above the limit: a tiny limit changes dw_proj, a huge one does not
+    same = O.weight_grads_fp8(x, dy, h, dpre, rowb, e4m3_limit=448.0)[1]
+    assert torch.equal(same, dw_proj) or float((h.float() * s_h).max()) > 240.0
+    small = O.weight_grads_fp8(x, dy, h, dpre, rowb, e4m3_limit=1.0)[1]
+    assert not torch.equal(small, dw_proj)

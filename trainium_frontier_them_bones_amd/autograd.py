@@ -258,8 +258,9 @@ class Mlp8State:
     """Per-layer fp8 state refreshed once per optimizer step: the scale row and the e4m3 weight pack
     (round2/source/train.py:6617 fp8_refresh_weights, 7003 mlp8_scales_into, 7267 mlp8_precast_into)."""
 
-    def __init__(self, e4m3_limit=240.0, x_scale=4.0):
+    def __init__(self, e4m3_limit=240.0, x_scale=4.0, dw_fp8=False):
         self.e4m3_limit, self.x_scale = e4m3_limit, x_scale
+        self.dw_fp8 = dw_fp8   # weight gradients in fp8 too (round2/source/train.py:8209 under its switch 9k; R1 DW_ROWS)
         self.row = None
         self.w8 = None
 
@@ -269,13 +270,19 @@ class Mlp8State:
 
 
 class Mlp8Fn(torch.autograd.Function):
-    """y = c_proj(relu(c_fc(x))^2) with the four activation GEMMs in fp8 and bf16 weight gradients."""
+    """y = c_proj(relu(c_fc(x))^2) with the four activation GEMMs in fp8 and the weight gradients in bf16
+    (K/nki_mlp_fused8.py:706 weight_grads) or, with state.dw_fp8, in fp8 from the bytes the other GEMMs multiplied
+    (round2/source/train.py:8209 mlp8_weight_grads)."""
 
     @staticmethod
     def forward(ctx, x, w_fc, w_proj, state):
         x2 = x.reshape(-1, x.shape[-1]).contiguous()
-        y, r = ops.mlp8_fwd(x2, state.w8, state.row, w_fc.shape[0], state.x_scale)
-        ctx.save_for_backward(x2, r, w_fc, w_proj)
+        if state.dw_fp8:
+            y, r, x8 = ops.mlp8_fwd(x2, state.w8, state.row, w_fc.shape[0], state.x_scale, want_x8=True)
+            ctx.save_for_backward(x8, r, w_fc, w_proj)
+        else:
+            y, r = ops.mlp8_fwd(x2, state.w8, state.row, w_fc.shape[0], state.x_scale)
+            ctx.save_for_backward(x2, r, w_fc, w_proj)
         ctx.state = state
         ctx.xshape = x.shape
         return y.view(x.shape)
@@ -286,6 +293,16 @@ class Mlp8Fn(torch.autograd.Function):
         st = ctx.state
         g2 = gy.reshape(-1, gy.shape[-1]).contiguous()
         rowb = ops.mlp8_backward_scales(g2, st.row)
+        if st.dw_fp8:
+            dx, _, dp8, hq8, dy8 = ops.mlp8_bwd_q(g2, r, st.w8, rowb, st.e4m3_limit)
+            (bf, af), (bp, ap) = _accumulate_into(w_fc), _accumulate_into(w_proj)
+            if (bf is None) != (bp is None) or af != ap:
+                raise RuntimeError("the fp8 weight gradients write both MLP weights' gradient buffers in one call")
+            if bf is not None:
+                ops.mlp8_dw8(x2, dp8, hq8, dy8, rowb, st.x_scale, dw_fc=bf, dw_proj=bp, accumulate=af)
+                return dx.view(ctx.xshape), None, None, None
+            dw_fc, dw_proj = ops.mlp8_dw8(x2, dp8, hq8, dy8, rowb, st.x_scale)
+            return dx.view(ctx.xshape), dw_fc, dw_proj, None
         dx, _, dpre = ops.mlp8_bwd(g2, r, st.w8, rowb, want_h=False)
         buf, acc = _accumulate_into(w_fc)
         if buf is not None:

@@ -7,9 +7,11 @@
 //   K_CONTIG  [rows][K]:  LDS row = 128 bytes of k, chunk c of row r at slot c ^ ((r + r / 8) & 7). The 128-bit
 //             fragment reads of 16 consecutive rows then fall on 16 different 16-byte bank groups (LDS here has
 //             64 banks of 4 bytes, measured 256 B/clk for ds_read_b128).
-//   K_STRIDED [K][rows]:  (bf16) LDS row = one k with the tile's rows contiguous, 16-byte chunk c of k-row k at slot
+//   K_STRIDED [K][rows]:  LDS row = one k with the tile's rows contiguous. bf16: 16-byte chunk c of k-row k at slot
 //             c ^ (4 (k & 3)); fragments are fetched with ds_read_b64_tr_b16, whose 16-lane transpose hands lane i
-//             four consecutive k of row i when lane j points at (k0 + j / 4, row0 + 4 (j % 4)).
+//             four consecutive k of row i when lane j points at (k0 + j / 4, row0 + 4 (j % 4)). fp8 (128-row tiles):
+//             slot c ^ (2 ((k >> 1) & 3)) and ds_read_b64_tr_b8 (lane j at (k0 + j / 2, row0 + 8 (j % 2)) gives lane i
+//             eight consecutive k of row i).
 // Two LDS buffers (separate __shared__ objects, so the compiler can tell a fragment read of one from the loads in
 // flight into the other and does not wait for them), loads of k-tile t+1 in flight during the MFMAs of tile t, one
 // barrier per k-tile, fragments of k-step s+1 requested between the MFMAs of step s.
@@ -22,7 +24,7 @@
 // (used when the epilogue reduces along p in registers).
 //
 // Element types: bf16 (v_mfma_f32_32x32x16_bf16) or OCP fp8 (v_mfma_scale_f32_32x32x64_f8f6f4 with unit scales,
-// e4m3/e5m2 per side; k-contiguous only).
+// e4m3/e5m2 per side).
 #pragma once
 #include <type_traits>
 
@@ -80,7 +82,6 @@ struct GemmCfg {
   // wavefronts per SIMD the kernel is compiled for: two workgroups per CU when registers and LDS allow it
   static constexpr int OCC = OCC_ > 0 ? OCC_ : ((NT <= 256 && 2 * LDS_BYTES <= 160 * 1024 && TP * TQ <= 4) ? 2 : 1);
   static_assert(ES == 1 || ES == 2, "fp8 or bf16");
-  static_assert(ES == 2 || (LAYP == TFB_K_CONTIG && LAYQ == TFB_K_CONTIG), "fp8 operands are k-contiguous");
   static_assert(NW >= 4 && (NW & (NW - 1)) == 0, "4, 8 or 16 wavefronts");
   static_assert((BP / 8) % NW == 0 && (BQ / 8) % NW == 0, "1 KB load instructions vs wavefronts");
   static_assert(LAYP == TFB_K_CONTIG || BP == 128 || BP == 256, "K_STRIDED tiles are 128 or 256 rows");
@@ -90,11 +91,11 @@ struct GemmCfg {
 };
 
 // ---- global -> LDS (one operand tile, this wavefront's share) ---------------------------------------------------
-template <int ROWS, int NW, int LAY>
+template <int ROWS, int NW, int LAY, int ES = 2>
 struct TileDma;
 
-template <int ROWS, int NW>
-struct TileDma<ROWS, NW, TFB_K_CONTIG> {
+template <int ROWS, int NW, int ES>
+struct TileDma<ROWS, NW, TFB_K_CONTIG, ES> {
   static constexpr int NI = ROWS / 8 / NW;            // instructions per wavefront: 8 rows x 128 bytes each
   static constexpr int NV = NW >= 8 ? 1 : 8 / NW;     // distinct per-lane offsets over the instructions
   const uint8_t* base;  // wavefront-uniform
@@ -120,23 +121,27 @@ struct TileDma<ROWS, NW, TFB_K_CONTIG> {
   }
 };
 
-template <int ROWS, int NW>
-struct TileDma<ROWS, NW, TFB_K_STRIDED> {
-  static constexpr int LPR = ROWS / 8;       // lanes (16-byte chunks) per k-row
-  static constexpr int RPI = 64 / LPR;       // k-rows per instruction
-  static constexpr int NI = ROWS / 8 / NW;   // 64 k-rows / RPI / NW
-  static_assert((NW * RPI) % 4 == 0, "k & 3 must not depend on the instruction index");
+template <int ROWS, int NW, int ES>
+struct TileDma<ROWS, NW, TFB_K_STRIDED, ES> {
+  static constexpr int LPR = ROWS * ES / 16;   // lanes (16-byte chunks) per k-row
+  static constexpr int RPI = 64 / LPR;         // k-rows per instruction
+  static constexpr int KROWS = 128 / ES;       // k-rows per tile
+  static constexpr int NI = KROWS / RPI / NW;  // = ROWS / 8 / NW
+  // the swizzle term (k & 3 for bf16, (k >> 1) & 3 for fp8) must not depend on the instruction index
+  static_assert((NW * RPI) % (ES == 2 ? 4 : 8) == 0, "swizzle phase vs instruction index");
+  static_assert(ES == 2 || ROWS == 128, "fp8 K_STRIDED tiles are 128 rows");
   const uint8_t* base;
   long step, tstep;
   uint32_t voff;
   __device__ __forceinline__ void init(const GemmOperand& o, long row0, long k0_bytes, int wave, int lane) {
     const int kl = lane / LPR, slot = lane % LPR;
-    const long k0 = k0_bytes >> 1;  // elements
-    base = o.base + (k0 + (long)wave * RPI) * o.ld + row0 * 2;
+    const long k0 = k0_bytes / ES;  // elements
+    base = o.base + (k0 + (long)wave * RPI) * o.ld + row0 * ES;
     step = (long)NW * RPI * o.ld;
-    tstep = 64 * o.ld;
-    const int k = wave * RPI + kl;  // k & 3 of the k-row this lane fills, the same for every instruction
-    voff = (uint32_t)(kl * o.ld + ((slot ^ (4 * (k & 3))) * 16));
+    tstep = (long)KROWS * o.ld;
+    const int k = wave * RPI + kl;  // the swizzle phase of the k-row this lane fills, the same for every instruction
+    const int sw = ES == 2 ? 4 * (k & 3) : 2 * ((k >> 1) & 3);
+    voff = (uint32_t)(kl * o.ld + ((slot ^ sw) * 16));
   }
   __device__ __forceinline__ void issue(uint8_t* lds, int t, int wave) const {
 #pragma unroll
@@ -195,6 +200,36 @@ struct FragReader<ROWS, 2, TFB_K_STRIDED> {
     typedef short s16x8 __attribute__((ext_vector_type(8)));
     const s16x8 v = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     return __builtin_bit_cast(bf16x8, v);
+  }
+};
+
+// fp8, one k per LDS row of ROWS bytes: ds_read_b64_tr_b8 hands lane i of a 16-lane group the bytes
+// src[2 e + (i >> 3)][i & 7], e = 0..7, of the 16 x 8 bytes its lanes point at; with lane j pointing at
+// (k0 + j / 2, row0 + 8 (j % 2)) lane i receives 8 consecutive k of row row0 + i. 16-byte chunk c of k-row k sits at
+// slot c ^ (2 ((k >> 1) & 3)): the 8 k-rows x 2 chunks that 32 lanes read together then cover all 64 banks once.
+template <int ROWS>
+struct FragReader<ROWS, 1, TFB_K_STRIDED> {
+  static constexpr int KSTEPS = 2;
+  typedef i32x8 frag_t;
+  static constexpr int PITCH = ROWS;
+  int wave_row0, lane;
+  __device__ __forceinline__ void init(int wave_row0_, int lane_) { wave_row0 = wave_row0_; lane = lane_; }
+  __device__ __forceinline__ frag_t read(const uint8_t* lds, int i, int s) const {
+    typedef int tfb_i32x2 __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(3))) tfb_i32x2 tfb_lds_i32x2_t;
+    const int g4 = lane >> 4, j = lane & 15;
+    const int p = wave_row0 + 32 * i + 16 * (g4 & 1) + 8 * (j & 1);  // first of this lane's 8 source rows
+    const int kq = j >> 1;                                           // k offset of the source lane, 0..7
+    const int k = 64 * s + 32 * (g4 >> 1) + kq;
+    const int off = k * PITCH + ((((p >> 4) ^ (2 * ((kq >> 1) & 3))) << 4) | (p & 8));
+    frag_t v;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const tfb_i32x2 t = __builtin_amdgcn_ds_read_tr8_b64_v2i32((tfb_lds_i32x2_t*)(lds + off + 8 * q * PITCH));
+      v[2 * q] = t.x;
+      v[2 * q + 1] = t.y;
+    }
+    return v;
   }
 };
 
@@ -314,8 +349,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   const Epi epi = epi_for_group(epi_in, group);
   const int nkt = a.nkt;
 
-  TileDma<BP, NW, Cfg::LAYP> dp;
-  TileDma<BQ, NW, Cfg::LAYQ> dq;
+  TileDma<BP, NW, Cfg::LAYP, ES> dp;
+  TileDma<BQ, NW, Cfg::LAYQ, ES> dq;
   dp.init(a.P, p0, kt0 * 128, wave, lane);
   dq.init(a.Q, q0, kt0 * 128, wave, lane);
   typedef FragReader<BP, ES, Cfg::LAYP> RP;
@@ -391,7 +426,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
     // have landed, barrier (every wavefront's share of tile t is in LDS, and everyone is done reading the stage that
     // is refilled next), start the load of tile t + 2, multiply tile t. The barrier is the bare instruction: a
     // __syncthreads() fence would wait for the loads still in flight.
-    constexpr int NI = TileDma<BP, NW, Cfg::LAYP>::NI + TileDma<BQ, NW, Cfg::LAYQ>::NI;  // load instructions per tile
+    constexpr int NI = TileDma<BP, NW, Cfg::LAYP, ES>::NI + TileDma<BQ, NW, Cfg::LAYQ, ES>::NI;  // load instructions per tile
     constexpr int WAIT_OLDER = (NI & 15) | (7 << 4) | (0 << 8) | ((NI >> 4) << 14);      // vmcnt(NI) lgkmcnt(0)
     auto step = [&](const uint8_t* cur, uint8_t* refill, int t) {
       __builtin_amdgcn_s_waitcnt(WAIT_OLDER);
@@ -584,13 +619,20 @@ struct EpiSplit {
   }
 };
 
-// out (+)= sum over splits of ws, rounded once
+// out (+)= scale * (sum over splits of ws), rounded once; scale = imm / (*sa * *sb) (absent factors are 1: the fp8
+// GEMMs' power-of-two descale, exact)
 static __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* out, long n, int splits, int f32,
-                                            int accumulate) {
+                                            int accumulate, const float* sa, const float* sb, float imm) {
   long i = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (i >= n) return;
   f32x4 s = *(const f32x4*)(ws + i);
   for (int k = 1; k < splits; ++k) s += *(const f32x4*)(ws + (long)k * n + i);
+  if (sa || sb || imm != 1.0f) {
+    float d = 1.0f;
+    if (sa) d *= *sa;
+    if (sb) d *= *sb;
+    s *= imm / d;
+  }
   if (f32) {
     float* o = (float*)out + i;
     if (accumulate) s += *(const f32x4*)o;
@@ -609,9 +651,10 @@ static __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* 
   }
 }
 
-static inline int splitk_reduce(const float* ws, void* out, long n, int splits, int f32, int accumulate, hipStream_t s) {
+static inline int splitk_reduce(const float* ws, void* out, long n, int splits, int f32, int accumulate, hipStream_t s,
+                                const float* sa = nullptr, const float* sb = nullptr, float imm = 1.0f) {
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, s, ws, out, n, splits, f32,
-                     accumulate);
+                     accumulate, sa, sb, imm);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

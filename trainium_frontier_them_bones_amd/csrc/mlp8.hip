@@ -357,12 +357,15 @@ struct EpiDescale {  // out = bf16(acc * dq), dq = dq_imm * *dq_a * *dq_b (absen
   }
 };
 
-struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*s_dp), optional h = bf16(r^2)
+struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*s_dp), optional h = bf16(r^2) and
+                // hq8 = e4m3(min(h*s_h, limit)) (the fp8 weight gradient's operand)
   const float* sc;
   const bf16_t* r;  // [M][F]
   bf16_t* dpre;     // [M][F]
   uint8_t* dp8;     // [M][F]
   bf16_t* h;        // [M][F] or null
+  uint8_t* hq8;     // [M][F] or null
+  float hq_limit;
   long F;
   __device__ __forceinline__ EpiDh for_group(int g) const {
     EpiDh e = *this;
@@ -380,10 +383,17 @@ struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*
     u32x2 o = {cvt4_fp8<TFB_FMT_E5M2>(dp[0] * sdp, dp[1] * sdp, dp[2] * sdp, dp[3] * sdp),
                cvt4_fp8<TFB_FMT_E5M2>(dp[4] * sdp, dp[5] * sdp, dp[6] * sdp, dp[7] * sdp)};
     *(u32x2*)(dp8 + off) = o;
-    if (h) {
+    if (h || hq8) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) rr[i] = rr[i] * rr[i];
-      *(u32x4*)(h + off) = pack8bf(rr);
+      for (int i = 0; i < 8; ++i) rr[i] = round_bf(rr[i] * rr[i]);
+      if (h) *(u32x4*)(h + off) = pack8bf(rr);
+      if (hq8) {
+        const float sh = sc[SC_S_H];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) rr[i] = fminf(rr[i] * sh, hq_limit);
+        u32x2 q = {cvt4_fp8<TFB_FMT_E4M3>(rr[0], rr[1], rr[2], rr[3]), cvt4_fp8<TFB_FMT_E4M3>(rr[4], rr[5], rr[6], rr[7])};
+        *(u32x2*)(hq8 + off) = q;
+      }
     }
   }
 };
@@ -552,20 +562,59 @@ extern "C" int tfb_mlp8_fwd(const void* x8, const void* w8, const void* row, voi
 
 // Backward: dy8 [M][d] e5m2 (cast at the row's s_dy), r [M][F] -> dx [M][d], dpre [M][F] bf16, h [M][F] bf16 (optional,
 // may be NULL), dp8 [M][F] e5m2 scratch.
-extern "C" int tfb_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* row, void* dx, void* h, void* dpre,
-                            void* dp8, long M, int d, int F, void* stream) {
+// hq8 (optional, may be NULL) [M][F] = e4m3(min(bf16(r^2) * s_h, hq_limit)): the g-side operand of the fp8 weight
+// gradient of w_proj (K/nki_dw8.py:323 with format E4M3C, round2/source/train.py:8226).
+extern "C" int tfb_mlp8_bwd_q(const void* dy8, const void* r, const void* w8, const void* row, void* dx, void* h, void* dpre,
+                              void* dp8, void* hq8, float hq_limit, long M, int d, int F, void* stream) {
   if (!dy8 || !r || !w8 || !row || !dx || !dpre || !dp8) return TFB_ERR_ARG;
   if (!shapes8(M, d, F)) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   const uint8_t* b = (const uint8_t*)w8;
   const long n = (long)F * d;
   GemmOperand Pw{b + 3 * n, (long)d}, Qg{(const uint8_t*)dy8, (long)d};  // wp8T [F][d]
-  EpiDh e1{(const float*)row, (const bf16_t*)r, (bf16_t*)dpre, (uint8_t*)dp8, (bf16_t*)h, (long)F};
+  EpiDh e1{(const float*)row, (const bf16_t*)r, (bf16_t*)dpre, (uint8_t*)dp8, (bf16_t*)h, (uint8_t*)hq8, hq_limit, (long)F};
   int st = gemm_launch<Cfg8g>(Pw, Qg, F, (int)M, (long)d, 1, LoadIdentity{}, LoadIdentity{}, e1, s);
   if (st != TFB_OK) return st;
   GemmOperand Pf{b + n, (long)F}, Qd{(const uint8_t*)dp8, (long)F};  // wf8T [d][F]
   EpiScaleStore e2{(const float*)row, SC_DQ_DX, (bf16_t*)dx, (long)d};
   return gemm_launch<Cfg8g>(Pf, Qd, d, (int)M, (long)F, 1, LoadIdentity{}, LoadIdentity{}, e2, s);
+}
+extern "C" int tfb_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* row, void* dx, void* h, void* dpre,
+                            void* dp8, long M, int d, int F, void* stream) {
+  return tfb_mlp8_bwd_q(dy8, r, w8, row, dx, h, dpre, dp8, nullptr, 0.f, M, d, F, stream);
+}
+
+// The two weight gradients in fp8, from byte tensors the forward and backward already hold (token-major, contraction
+// over the M tokens): dw_fc [F][d] = bf16((dp8^T @ x8) / (s_dp x_scale)) with dp8 = e5m2(dpre s_dp) and x8 = e4m3(x x_scale);
+// dw_proj [d][F] = bf16((dy8^T @ hq8) / (s_dy s_h)) with dy8 = e5m2(dy s_dy) and hq8 from tfb_mlp8_bwd_q. row = the
+// backward call's scale row. Outputs bf16 or fp32, optionally accumulated into; split-K through the workspace.
+// Replaces mlp8_weight_grads under switch 9k (round2/source/train.py:8209-8229) = K/nki_dw8.py:323 emulate_dw.
+extern "C" int tfb_mlp8_dw8(const void* x8, const void* dp8, const void* hq8, const void* dy8, const void* row, float x_scale,
+                            void* dw_fc, void* dw_proj, long M, int d, int F, int out_f32, int accumulate, void* workspace,
+                            long workspace_bytes, void* stream) {
+  if (!x8 || !dp8 || !hq8 || !dy8 || !row || !dw_fc || !dw_proj || !workspace) return TFB_ERR_ARG;
+  if (!shapes8(M, d, F) || !(x_scale > 0.f)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  using Cfg = GemmCfg<128, 128, 2, 2, 1, TFB_K_STRIDED, TFB_K_STRIDED, TFB_FMT_E4M3, TFB_FMT_E5M2>;
+  const float* sc = (const float*)row;
+  const long n = (long)d * F;
+  const int splits = choose_splits(n / (128 * 128), (int)(M / 128), n, workspace_bytes);
+  if ((long)splits * n * 4 > workspace_bytes) return TFB_ERR_SHAPE;
+  float* ws = (float*)workspace;
+  {  // D[p = dd][q = f] = sum_m x8[m][dd] dp8[m][f] -> dw_fc[f][dd]
+    GemmOperand P{(const uint8_t*)x8, (long)d}, Q{(const uint8_t*)dp8, (long)F};
+    EpiSplit e{ws, (long)d, n};
+    int st = gemm_launch<Cfg>(P, Q, d, F, M, splits, LoadIdentity{}, LoadIdentity{}, e, s);
+    if (st != TFB_OK) return st;
+    st = splitk_reduce(ws, dw_fc, n, splits, out_f32, accumulate, s, sc + SC_S_DP, nullptr, 1.0f / x_scale);
+    if (st != TFB_OK) return st;
+  }
+  // D[p = f][q = dd] = sum_m hq8[m][f] dy8[m][dd] -> dw_proj[dd][f]
+  GemmOperand P{(const uint8_t*)hq8, (long)F}, Q{(const uint8_t*)dy8, (long)d};
+  EpiSplit e{ws, (long)F, n};
+  int st = gemm_launch<Cfg>(P, Q, F, d, M, splits, LoadIdentity{}, LoadIdentity{}, e, s);
+  if (st != TFB_OK) return st;
+  return splitk_reduce(ws, dw_proj, n, splits, out_f32, accumulate, s, sc + SC_S_H, sc + SC_S_DY, 1.0f);
 }
 
 // dW_proj [d][F] (+)= dy^T @ bf16(r^2): the token-contraction GEMM with the square applied while r is staged, so h
@@ -635,7 +684,7 @@ extern "C" int tfb_moe_mlp8_bwd(const void* dy8, const void* r, const void* w8, 
   hipStream_t s = (hipStream_t)stream;
   const uint8_t* b = (const uint8_t*)w8;
   const long n = (long)F * d;
-  EpiDh e1{(const float*)rows, (const bf16_t*)r, (bf16_t*)dpre, (uint8_t*)dp8, nullptr, (long)F};
+  EpiDh e1{(const float*)rows, (const bf16_t*)r, (bf16_t*)dpre, (uint8_t*)dp8, nullptr, nullptr, 0.f, (long)F};
   int st = grouped_launch<Cfg8g>(b + 3 * n, d, 4 * n, (const uint8_t*)dy8, d, F, rmax, d, (const int*)tile_expert, e1, s);
   if (st != TFB_OK) return st;
   EpiScaleStore e2{(const float*)rows, SC_DQ_DX, (bf16_t*)dx, (long)d};

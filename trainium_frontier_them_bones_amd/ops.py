@@ -225,8 +225,9 @@ def mlp8_precast(w_fc, w_proj, row):
     return w8
 
 
-def mlp8_fwd(x2, w8, row, F, x_scale=4.0):
-    """y [M,d], r [M,F] (bf16): the fp8 forward. x_scale: python float (the reference's constant 4) or a device scalar."""
+def mlp8_fwd(x2, w8, row, F, x_scale=4.0, want_x8=False):
+    """y [M,d], r [M,F] (bf16): the fp8 forward. x_scale: python float (the reference's constant 4) or a device scalar.
+    want_x8 also returns x8 = e4m3(x x_scale) [M,d] bytes (the fp8 weight gradient's operand)."""
     _chk(x2), _chk(w8, torch.uint8), _chk(row, torch.float32)
     M, d = x2.shape
     x8 = quant_fp8(x2, x_scale, FMT_E4M3)
@@ -234,7 +235,7 @@ def mlp8_fwd(x2, w8, row, F, x_scale=4.0):
     r = torch.empty(M, F, dtype=bf16, device=x2.device)
     h8 = torch.empty(M, F, dtype=torch.uint8, device=x2.device)
     _lib.call("tfb_mlp8_fwd", _p(x8), _p(w8), _p(row), _p(y), _p(r), _p(h8), M, d, F, _stream())
-    return y, r
+    return (y, r, x8) if want_x8 else (y, r)
 
 
 def mlp8_bwd(dy2, r, w8, row, want_h=True):
@@ -249,6 +250,51 @@ def mlp8_bwd(dy2, r, w8, row, want_h=True):
     dp8 = torch.empty(M, F, dtype=torch.uint8, device=dy2.device)
     _lib.call("tfb_mlp8_bwd", _p(dy8), _p(r), _p(w8), _p(row), _p(dx), _p(h), _p(dpre), _p(dp8), M, d, F, _stream())
     return dx, h, dpre
+
+
+def mlp8_bwd_q(dy2, r, w8, row, e4m3_limit=240.0):
+    """The fp8 backward keeping the byte tensors of the fp8 weight gradients: (dx [M,d], dpre [M,F], dp8 [M,F] e5m2 bytes,
+    hq8 [M,F] = e4m3(min(bf16(r^2) s_h, e4m3_limit)) bytes, dy8 [M,d] e5m2 bytes)."""
+    _chk(dy2), _chk(r), _chk(w8, torch.uint8), _chk(row, torch.float32)
+    M, d = dy2.shape
+    F = r.shape[1]
+    dy8 = quant_fp8(dy2, row[5:6], FMT_E5M2)
+    dx = torch.empty(M, d, dtype=bf16, device=dy2.device)
+    dpre = torch.empty(M, F, dtype=bf16, device=dy2.device)
+    dp8 = torch.empty(M, F, dtype=torch.uint8, device=dy2.device)
+    hq8 = torch.empty(M, F, dtype=torch.uint8, device=dy2.device)
+    _lib.call("tfb_mlp8_bwd_q", _p(dy8), _p(r), _p(w8), _p(row), _p(dx), None, _p(dpre), _p(dp8), _p(hq8), float(e4m3_limit),
+              M, d, F, _stream())
+    return dx, dpre, dp8, hq8, dy8
+
+
+def mlp8_dw8(x8, dp8, hq8, dy8, row, x_scale=4.0, dw_fc=None, dw_proj=None, accumulate=False, out_dtype=bf16):
+    """(dw_fc [F,d], dw_proj [d,F]) (+)= the fp8 weight gradients from the forward's x8 and the backward's dp8, hq8, dy8
+    (mlp8_weight_grads under the fp8 weight-gradient switch, round2/source/train.py:8209)."""
+    for t in (x8, dp8, hq8, dy8):
+        _chk(t, torch.uint8)
+    _chk(row, torch.float32)
+    M, d = x8.shape
+    F = dp8.shape[1]
+    if tuple(hq8.shape) != (M, F) or tuple(dy8.shape) != (M, d):
+        raise ValueError("operand shapes")
+    if (dw_fc is None) != (dw_proj is None):
+        raise ValueError("give both outputs or neither")
+    if dw_fc is None:
+        if accumulate:
+            raise ValueError("accumulate needs the outputs")
+        dw_fc = torch.empty(F, d, dtype=out_dtype, device=x8.device)
+        dw_proj = torch.empty(d, F, dtype=out_dtype, device=x8.device)
+    else:
+        _chk(dw_fc, dw_fc.dtype), _chk(dw_proj, dw_proj.dtype)
+        if dw_fc.dtype != dw_proj.dtype or dw_fc.dtype not in (bf16, torch.float32):
+            raise ValueError("bad outputs")
+        if tuple(dw_fc.shape) != (F, d) or tuple(dw_proj.shape) != (d, F):
+            raise ValueError("bad output shapes")
+    ws = _workspace(x8.device)
+    _lib.call("tfb_mlp8_dw8", _p(x8), _p(dp8), _p(hq8), _p(dy8), _p(row), float(x_scale), _p(dw_fc), _p(dw_proj), M, d, F,
+              int(dw_fc.dtype == torch.float32), int(accumulate), _p(ws), ws.numel() * 4, _stream())
+    return dw_fc, dw_proj
 
 
 def mlp_dw_proj(dy2, r, out=None, accumulate=False, out_dtype=bf16):
