@@ -136,6 +136,15 @@ int tfb_mlp8_fwd(const void* x8, const void* w8, const void* row, void* y, void*
 int tfb_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* row, void* dx, void* h, void* dpre, void* dp8,
                  long M, int d, int F, void* stream);
 
+/* out [O][D] (+)= (g8 [M][O]^T @ a8 [M][D]) * imm / (*s_g * *s_a): one weight gradient in fp8 from two token-major byte
+ * tensors, contraction over the M tokens (fp32 accumulation over all of them, one rounding). (fmt_g, fmt_a) = (1, 0): an
+ * e5m2 gradient against the forward's e4m3 activation bytes, or (0, 1). s_g, s_a: device fp32 scalars (the power-of-two
+ * scales the bytes were cast at; NULL = 1). out bf16 (out_f32 = 0) or fp32, accumulate = 1 adds into it.
+ * M, O, D multiples of 128; workspace >= splits * O * D * 4 bytes (256 MB always suffices).
+ * Replaces dw8_grad (round2/source/train.py:8185; attn8_weight_grad 8232) = nki_dw8.py:323 emulate_dw / _dw8_kernel. */
+int tfb_gemm_fp8_tn(const void* g8, int fmt_g, const void* a8, int fmt_a, const void* s_g, const void* s_a, float imm, void* out,
+                    long M, int O, int D, int out_f32, int accumulate, void* workspace, long workspace_bytes, void* stream);
+
 /* tfb_mlp8_bwd that also writes hq8 [M][F] = e4m3(min(bf16(r^2) * s_h, hq_limit)) (NULL to skip): the g-side operand of
  * the fp8 weight gradient of w_proj (format E4M3C of nki_dw8.py:312-320; round2/source/train.py:8226). */
 int tfb_mlp8_bwd_q(const void* dy8, const void* r, const void* w8, const void* row, void* dx, void* h, void* dpre, void* dp8,

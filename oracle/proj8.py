@@ -11,7 +11,8 @@ bound, e.g. the attention output) the per-tensor amax scale found by the same se
 Pinned by (tests/test_oracle_proj8.py): the scale search is the one pinned in tests/test_oracle_mlp8.py (brute force
 against 2^floor(log2(limit / v))); the casts against the bit-level fp8 tables; forward and input gradient against the
 bf16 projection F.linear and its autograd within the fp8 error budget; exact invariance of the forward under
-power-of-two rescaling of the weight (the scale search absorbs it).
+power-of-two rescaling of the weight (the scale search absorbs it); the fp8 weight gradient against autograd's within
+the e5m2 budget and against an fp64 product of the operands decoded through the byte tables.
 """
 import torch
 
@@ -57,6 +58,13 @@ def backward_input(g2, w, s_g, s_w):
 def weight_grad(g2, a2):
     """dw [N, K] = bf16(g2^T @ a2), fp32 accumulation (the bf16 weight gradient this build keeps for the projections)."""
     return (g2.float().t() @ a2.float()).to(a2.dtype)
+
+
+def weight_grad_fp8(g2, a2, s_g, s_a):
+    """dw [N, K] = bf16((e5m2(g2 s_g)^T @ e4m3(a2 s_a)) / (s_g s_a)): the projection's weight gradient in fp8
+    (round2/source/train.py:8232 attn8_weight_grad -> dw8_grad 8185 -> nki_dw8.py:323 emulate_dw): the g side at the
+    scale the input gradient was cast with, the a side at its forward's."""
+    return mlp8.fp8_weight_grad(g2, a2, s_g, s_a, (1.0 / s_g) * (1.0 / s_a), 1, 0)
 
 
 def reference_forward(a2, w):

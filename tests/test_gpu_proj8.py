@@ -40,6 +40,15 @@ def test_projection_forward_backward(dev, shape):
         s_g, _ = O.grad_scale(gy)
         assert rel_l2(xd.grad, O.backward_input(gy, w, s_g, s_w)) < 2e-3
         assert rel_l2(wd.grad, O.weight_grad(gy, x)) < 5e-3
+        # the weight gradient in fp8 from the same e5m2 gradient bytes and the forward's activation bytes
+        st8 = A.Linear8State(dw_fp8=True)
+        st8.refresh(w.to(dev))
+        xd8, wd8 = x.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+        y8 = A.Linear8Fn.apply(xd8, wd8, st8, x_scale)
+        y8.backward(gy.to(dev))
+        assert torch.equal(y8, y) and torch.equal(xd8.grad, xd.grad)
+        assert rel_l2(wd8.grad, O.weight_grad_fp8(gy, x, s_g, s_a)) < 2e-3
+        assert rel_l2(wd8.grad, O.weight_grad(gy, x)) < 8e-2
 
 
 def test_model_with_fp8_projections_tracks_the_bf16_model(dev):

@@ -50,6 +50,27 @@ def test_forward_and_input_gradient_against_the_bf16_projection():
     assert rel_l2(proj8.weight_grad(gy, a), wf.grad) < 5e-3
 
 
+def test_fp8_weight_gradient_against_autograd_and_the_byte_tables():
+    from helpers import fp8_table
+    g = _g(5)
+    M, K, N = 512, 256, 384
+    a = torch.randn(M, K, generator=g).bfloat16()
+    gy = (1e-2 * torch.randn(M, N, generator=g)).bfloat16()
+    s_g, _ = proj8.grad_scale(gy)
+    dw = proj8.weight_grad_fp8(gy, a, s_g, proj8.X_SCALE)
+    assert dw.shape == (N, K)
+    assert rel_l2(dw, proj8.weight_grad(gy, a)) < 8e-2                    # e5m2 gradient x e4m3 activation
+    g8 = fp8_table("e5m2")[mlp8.fp8_bytes(gy.float() * s_g, 1).long()]
+    a8 = fp8_table("e4m3fn")[mlp8.fp8_bytes(a.float() * proj8.X_SCALE, 0).long()]
+    assert rel_l2(dw, (g8.t() @ a8) / float(s_g * proj8.X_SCALE)) < 3e-3   # one bf16 rounding + fp32 summation
+    s_a, _ = proj8.act_scale(a)
+    dw2 = proj8.weight_grad_fp8(gy, a, s_g, s_a)
+    assert rel_l2(dw2, proj8.weight_grad(gy, a)) < 8e-2
+    # a gradient 16 times larger gets a scale 16 times smaller: identical bytes, the result exactly 16 times larger
+    gy16 = (gy.float() * 16).bfloat16()
+    assert torch.equal(proj8.weight_grad_fp8(gy16, a, proj8.grad_scale(gy16)[0], proj8.X_SCALE).float(), dw.float() * 16)
+
+
 def test_forward_is_exactly_invariant_under_power_of_two_weight_rescaling():
     g = _g(4)
     a = torch.randn(256, 128, generator=g).bfloat16()

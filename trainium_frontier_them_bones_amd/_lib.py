@@ -32,6 +32,7 @@ SIGNATURES = {
     "tfb_mlp8_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_mlp8_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_mlp8_bwd_q": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _l, _i, _i, _vp],
+    "tfb_gemm_fp8_tn": [_vp, _i, _vp, _i, _vp, _vp, _f, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
     "tfb_mlp8_dw8": [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
     "tfb_attn_fwd": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _i, _i, _i, _i, _f, _vp],
     "tfb_attn_bwd": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _vp, _i, _i, _i, _i,

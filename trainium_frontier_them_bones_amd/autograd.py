@@ -209,8 +209,9 @@ class Linear8State:
     (s, 1/s, amax on the device) and its e4m3 bytes in both layouts (forward_scales / precast_ref,
     round2/source/kernels/nki_attn_tt8g.py:700, 795)."""
 
-    def __init__(self, limit=240.0):
+    def __init__(self, limit=240.0, dw_fp8=False):
         self.limit = limit
+        self.dw_fp8 = dw_fp8   # the weight gradient in fp8 too (attn8_weight_grad, round2/source/train.py:8232)
         self.sc = None
         self.w8 = self.w8t = None
 
@@ -221,9 +222,10 @@ class Linear8State:
 
 class Linear8Fn(torch.autograd.Function):
     """y = x @ w^T with the forward in e4m3 x e4m3 and the input gradient in e5m2 x e4m3 (per-tensor power-of-two
-    scales, fp32 accumulation, one bf16 rounding), the weight gradient in bf16 (accumulated into w.grad_buf when
-    present). x_scale: the reference's constant (4 for an RMSNorm output) or None for the per-tensor amax scale of x.
-    The arithmetic of emulate_fwd / emulate_bwd (nki_attn_tt8g.py:745-757)."""
+    scales, fp32 accumulation, one bf16 rounding); the weight gradient in bf16, or with state.dw_fp8 in fp8 from the
+    gradient's e5m2 bytes and the forward's e4m3 activation bytes (round2/source/train.py:8232 attn8_weight_grad);
+    either is accumulated into w.grad_buf when present. x_scale: the reference's constant (4 for an RMSNorm output) or
+    None for the per-tensor amax scale of x. The arithmetic of emulate_fwd / emulate_bwd (nki_attn_tt8g.py:745-757)."""
 
     @staticmethod
     def forward(ctx, x, w, state, x_scale):
@@ -232,26 +234,29 @@ class Linear8Fn(torch.autograd.Function):
             sx = ops.amax_scale(x2, state.limit, -24, 40)
             x8 = ops.quant_fp8(x2, sx[0:1], ops.FMT_E4M3)
             y = ops.gemm_fp8(x8, state.w8, ops.FMT_E4M3, sx[1:2], state.sc[1:2])
+            ctx.sx, ctx.sx_imm = sx[0:1], 1.0
         else:
             x8 = ops.quant_fp8(x2, float(x_scale), ops.FMT_E4M3)
             y = ops.gemm_fp8(x8, state.w8, ops.FMT_E4M3, None, state.sc[1:2], 1.0 / float(x_scale))
-        ctx.save_for_backward(x2, w)
+            ctx.sx, ctx.sx_imm = None, 1.0 / float(x_scale)
+        ctx.save_for_backward(x8 if state.dw_fp8 else x2, w)
         ctx.state, ctx.xshape = state, x.shape
         return y.view(*x.shape[:-1], w.shape[0])
 
     @staticmethod
     def backward(ctx, gy):
-        x2, w = ctx.saved_tensors
+        xa, w = ctx.saved_tensors
         st = ctx.state
         g2 = gy.reshape(-1, gy.shape[-1]).contiguous()
         sg = ops.amax_scale(g2, 57344.0 / 2.0, -40, 60)
         g8 = ops.quant_fp8(g2, sg[0:1], ops.FMT_E5M2)
         dx = ops.gemm_fp8(g8, st.w8t, ops.FMT_E5M2, sg[1:2], st.sc[1:2]).view(ctx.xshape)
         buf, acc = _accumulate_into(w)
-        if buf is not None:
-            ops.matmul(g2, x2, trans_a=True, out=buf, accumulate=acc)
-            return dx, None, None, None
-        return dx, ops.matmul(g2, x2, trans_a=True), None, None
+        if st.dw_fp8:
+            dw = ops.gemm_fp8_tn(g8, xa, ops.FMT_E5M2, ops.FMT_E4M3, sg[0:1], ctx.sx, ctx.sx_imm, out=buf, accumulate=acc)
+        else:
+            dw = ops.matmul(g2, xa, trans_a=True, out=buf, accumulate=acc)
+        return dx, (None if buf is not None else dw), None, None
 
 
 class Mlp8State:

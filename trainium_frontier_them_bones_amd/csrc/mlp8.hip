@@ -543,6 +543,35 @@ extern "C" int tfb_gemm_fp8(const void* a8, int fmt_a, const void* b8, const voi
   return gemm_launch<Cfg8g>(P, Q, N, (int)M, (long)K, 1, LoadIdentity{}, LoadIdentity{}, e, (hipStream_t)stream);
 }
 
+// out [O][D] (+)= ((g8 [M][O]^T @ a8 [M][D]) * imm / (*s_g * *s_a)): the fp8 weight gradient of a projection, contraction
+// over the M tokens of two token-major byte tensors (fp32 accumulation over all tokens, one rounding; bf16 or fp32
+// output, optionally accumulated into). (fmt_g, fmt_a) = (e5m2, e4m3): a gradient against the forward's activation
+// bytes; (e4m3, e5m2): an activation on the g side (the MLP's h against dy). s_g, s_a: device fp32 scalars (the
+// power-of-two scales the bytes were cast at) or null. Split-K through the workspace.
+// Replaces dw8_grad (round2/source/train.py:8185) = K/nki_dw8.py:323 emulate_dw / _dw8_kernel.
+extern "C" int tfb_gemm_fp8_tn(const void* g8, int fmt_g, const void* a8, int fmt_a, const void* s_g, const void* s_a, float imm,
+                               void* out, long M, int O, int D, int out_f32, int accumulate, void* workspace,
+                               long workspace_bytes, void* stream) {
+  if (!g8 || !a8 || !out || !workspace) return TFB_ERR_ARG;
+  const bool ga = fmt_g == TFB_FMT_E5M2 && fmt_a == TFB_FMT_E4M3, ag = fmt_g == TFB_FMT_E4M3 && fmt_a == TFB_FMT_E5M2;
+  if (!ga && !ag) return TFB_ERR_ARG;
+  if (M <= 0 || O <= 0 || D <= 0 || M % 128 || O % 128 || D % 128) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const long n = (long)O * D;
+  const int splits = choose_splits(n / (128 * 128), (int)(M / 128), n, workspace_bytes);
+  if ((long)splits * n * 4 > workspace_bytes) return TFB_ERR_SHAPE;
+  float* ws = (float*)workspace;
+  // D[p = dd][q = o] = sum_m a8[m][dd] g8[m][o] -> out[o][dd]
+  GemmOperand P{(const uint8_t*)a8, (long)D}, Q{(const uint8_t*)g8, (long)O};
+  EpiSplit e{ws, (long)D, n};
+  int st = ga ? gemm_launch<GemmCfg<128, 128, 2, 2, 1, TFB_K_STRIDED, TFB_K_STRIDED, TFB_FMT_E4M3, TFB_FMT_E5M2>>(
+                    P, Q, D, O, M, splits, LoadIdentity{}, LoadIdentity{}, e, s)
+              : gemm_launch<GemmCfg<128, 128, 2, 2, 1, TFB_K_STRIDED, TFB_K_STRIDED, TFB_FMT_E5M2, TFB_FMT_E4M3>>(
+                    P, Q, D, O, M, splits, LoadIdentity{}, LoadIdentity{}, e, s);
+  if (st != TFB_OK) return st;
+  return splitk_reduce(ws, out, n, splits, out_f32, accumulate, s, (const float*)s_g, (const float*)s_a, imm);
+}
+
 // Forward: x8 [M][d] e4m3 (already cast at s_x), w8 pack, row -> y [M][d] bf16, r [M][F] bf16, h8 [M][F] e4m3 scratch.
 extern "C" int tfb_mlp8_fwd(const void* x8, const void* w8, const void* row, void* y, void* r, void* h8, long M, int d, int F,
                             void* stream) {
@@ -594,27 +623,14 @@ extern "C" int tfb_mlp8_dw8(const void* x8, const void* dp8, const void* hq8, co
                             long workspace_bytes, void* stream) {
   if (!x8 || !dp8 || !hq8 || !dy8 || !row || !dw_fc || !dw_proj || !workspace) return TFB_ERR_ARG;
   if (!shapes8(M, d, F) || !(x_scale > 0.f)) return TFB_ERR_SHAPE;
-  hipStream_t s = (hipStream_t)stream;
-  using Cfg = GemmCfg<128, 128, 2, 2, 1, TFB_K_STRIDED, TFB_K_STRIDED, TFB_FMT_E4M3, TFB_FMT_E5M2>;
   const float* sc = (const float*)row;
-  const long n = (long)d * F;
-  const int splits = choose_splits(n / (128 * 128), (int)(M / 128), n, workspace_bytes);
-  if ((long)splits * n * 4 > workspace_bytes) return TFB_ERR_SHAPE;
-  float* ws = (float*)workspace;
-  {  // D[p = dd][q = f] = sum_m x8[m][dd] dp8[m][f] -> dw_fc[f][dd]
-    GemmOperand P{(const uint8_t*)x8, (long)d}, Q{(const uint8_t*)dp8, (long)F};
-    EpiSplit e{ws, (long)d, n};
-    int st = gemm_launch<Cfg>(P, Q, d, F, M, splits, LoadIdentity{}, LoadIdentity{}, e, s);
-    if (st != TFB_OK) return st;
-    st = splitk_reduce(ws, dw_fc, n, splits, out_f32, accumulate, s, sc + SC_S_DP, nullptr, 1.0f / x_scale);
-    if (st != TFB_OK) return st;
-  }
-  // D[p = f][q = dd] = sum_m hq8[m][f] dy8[m][dd] -> dw_proj[dd][f]
-  GemmOperand P{(const uint8_t*)hq8, (long)F}, Q{(const uint8_t*)dy8, (long)d};
-  EpiSplit e{ws, (long)F, n};
-  int st = gemm_launch<Cfg>(P, Q, F, d, M, splits, LoadIdentity{}, LoadIdentity{}, e, s);
+  // dw_fc[f][dd] = sum_m dp8[m][f] x8[m][dd]: g = dp8 (e5m2), a = x8 (e4m3)
+  int st = tfb_gemm_fp8_tn(dp8, TFB_FMT_E5M2, x8, TFB_FMT_E4M3, sc + SC_S_DP, nullptr, 1.0f / x_scale, dw_fc, M, F, d, out_f32,
+                           accumulate, workspace, workspace_bytes, stream);
   if (st != TFB_OK) return st;
-  return splitk_reduce(ws, dw_proj, n, splits, out_f32, accumulate, s, sc + SC_S_H, sc + SC_S_DY, 1.0f);
+  // dw_proj[dd][f] = sum_m dy8[m][dd] hq8[m][f]: g = dy8 (e5m2), a = hq8 (e4m3)
+  return tfb_gemm_fp8_tn(dy8, TFB_FMT_E5M2, hq8, TFB_FMT_E4M3, sc + SC_S_DY, sc + SC_S_H, 1.0f, dw_proj, M, d, F, out_f32,
+                         accumulate, workspace, workspace_bytes, stream);
 }
 
 // dW_proj [d][F] (+)= dy^T @ bf16(r^2): the token-contraction GEMM with the square applied while r is staged, so h

@@ -33,6 +33,7 @@ class GPTConfig:
     e4m3_limit: float = 240.0     # fp8 scale search limit (240 = the reference's rows, 448 = OCP maximum)
     x_scale: float = 4.0          # constant activation scale of the fp8 MLP input (a unit-RMS norm output)
     fp8_attn_proj: bool = False   # QKV and output projections in fp8 (e4m3 forward, e5m2 dX, bf16 dW); off in BASELINE C4
+    fp8_attn_dw: bool = False     # with fp8_attn_proj: their weight gradients in fp8 as well (R2_DW8_SET=qkv,proj)
     fp8_mlp_dw: bool = False      # the MLP's two weight gradients in fp8 as well (R1's DW_ROWS recipe); off in BASELINE C4
 
     @property
@@ -107,8 +108,8 @@ class GPT:
         self.p.update(self.mats.params)
         self.p.update(self.others.params)
         self.mlp_state = [A.Mlp8State(cfg.e4m3_limit, cfg.x_scale, cfg.fp8_mlp_dw) for _ in range(L)]
-        self.qkv_state = [A.Linear8State(cfg.e4m3_limit) for _ in range(L)] if cfg.fp8_attn_proj else None
-        self.wo_state = [A.Linear8State(cfg.e4m3_limit) for _ in range(L)] if cfg.fp8_attn_proj else None
+        self.qkv_state = [A.Linear8State(cfg.e4m3_limit, cfg.fp8_attn_dw) for _ in range(L)] if cfg.fp8_attn_proj else None
+        self.wo_state = [A.Linear8State(cfg.e4m3_limit, cfg.fp8_attn_dw) for _ in range(L)] if cfg.fp8_attn_proj else None
         self.cos, self.sin = rope_tables(cfg.seq_len, cfg.head_dim, cfg.rope_base, device)
         self.step_count = 0
         self.init_weights(seed)

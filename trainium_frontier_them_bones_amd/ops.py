@@ -216,6 +216,29 @@ def gemm_fp8(a8, b8, fmt_a=FMT_E4M3, dq_a=None, dq_b=None, dq=1.0):
     return out
 
 
+def gemm_fp8_tn(g8, a8, fmt_g=FMT_E5M2, fmt_a=FMT_E4M3, s_g=None, s_a=None, imm=1.0, out=None, accumulate=False,
+                out_dtype=bf16):
+    """[O,D] (+)= (g8 [M,O]^T @ a8 [M,D]) * imm / (s_g s_a): a weight gradient in fp8 (dw8_grad,
+    round2/source/train.py:8185). s_g, s_a: 1-element fp32 device tensors (the scales the bytes were cast at) or None."""
+    _chk(g8, torch.uint8), _chk(a8, torch.uint8), _chk(s_g, torch.float32), _chk(s_a, torch.float32)
+    M, O = g8.shape
+    D = a8.shape[1]
+    if a8.shape[0] != M:
+        raise ValueError("token counts differ")
+    if out is None:
+        if accumulate:
+            raise ValueError("accumulate needs out")
+        out = torch.empty(O, D, dtype=out_dtype, device=g8.device)
+    else:
+        _chk(out, out.dtype)
+        if out.dtype not in (bf16, torch.float32) or tuple(out.shape) != (O, D):
+            raise ValueError("bad out")
+    ws = _workspace(g8.device)
+    _lib.call("tfb_gemm_fp8_tn", _p(g8), int(fmt_g), _p(a8), int(fmt_a), _p(s_g), _p(s_a), float(imm), _p(out), M, O, D,
+              int(out.dtype == torch.float32), int(accumulate), _p(ws), ws.numel() * 4, _stream())
+    return out
+
+
 def mlp8_precast(w_fc, w_proj, row):
     """uint8 [4, F*d]: w_fc and w_proj cast once to e4m3 at the row's scales, each in both byte layouts."""
     _chk(w_fc), _chk(w_proj), _chk(row, torch.float32)
