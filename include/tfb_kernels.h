@@ -68,6 +68,19 @@ int tfb_relu2(const void* a, const void* b, void* out, long n, int mode, void* s
 int tfb_rope(const void* x, const void* cos_t, const void* sin_t, void* out, long rows, int T, int nheads, int D,
              long row_stride, long out_stride, int inverse, void* stream);
 
+/* RoPE followed by the parameter-free RMSNorm of every head (the attention block's QK-norm): r = bf16(rope(x)) (NULL to
+ * skip), inv [rows][nheads] fp32 = rsqrt(mean_D(r^2) + eps), y = bf16(r inv). Head layout as tfb_rope; D = 64 or 128;
+ * strides in elements (multiples of 8). Replaces rope_norm(x, cos, sin) (round1/source/train.py:4447; eager form 4184-4196)
+ * and the rotation + QK-norm prologue of nki_rope_attention (round1/source/train.py:8197; r5 / inv3 of
+ * round2/source/kernels/nki_attn_bandpro.py:1850). */
+int tfb_rope_norm_fwd(const void* x, const void* cos_t, const void* sin_t, void* r, void* y, void* inv, long rows, int T,
+                      int nheads, int D, long x_stride, long r_stride, long y_stride, float eps, void* stream);
+
+/* dx = the gradient of tfb_rope_norm_fwd's input: dr = bf16(inv (g - rh (g . rh) / D)), rh = r inv, then the transposed
+ * rotation. dx may alias g. Replaces the backward of rope_norm (round1/source/train.py:4339 _rope_norm_bwd_kernel; forward kernel 4308). */
+int tfb_rope_norm_bwd(const void* g, const void* r, const void* inv, const void* cos_t, const void* sin_t, void* dx, long rows,
+                      int T, int nheads, int D, long g_stride, long r_stride, long dx_stride, void* stream);
+
 int tfb_resmix_bwd_blocks(long n);
 /* dx = g bf16(a), dx0 = g bf16(b), dab fp32 [2] = (sum bf16(g x), sum bf16(g x0)); ab fp32 [2] device;
  * part: fp32 [2 * tfb_resmix_bwd_blocks(n)] scratch.
@@ -220,6 +233,20 @@ int tfb_loss_fwd(const void* logits, const void* targets, int idx64, const void*
  * Replaces _loss_bwd_kernel (round1/source/train.py:4584) / _lh_bwd_kernel (round2/source/train.py:5297). */
 int tfb_loss_bwd(const void* logits, const void* targets, int idx64, const void* lse, const void* grow, void* dlogits,
                  long rows, int V, float softcap, void* stream);
+
+/* Several targets per row and / or label smoothing: targets [K][rows] (int64 or int32; < 0 = weight 0), row_w fp32
+ * [K][rows], 1 <= K <= 8, 0 <= eps < 1:  loss[row] = sum_k row_w[k][row] (lse - (1 - eps) s_{t_k} - (eps / V) sum_v s_v).
+ * K > 1, eps = 0 replaces _loss_multi_fwd_kernel behind fused_loss_multi(logits, tg, rw, softcap)
+ * (round1/source/train.py:4725, 4908); K = 1, eps > 0 replaces _lh_fwd_ls_kernel (round2/source/train.py:5697; host
+ * chunked_loss_mean(smooth=True) 6364, the mean and per-token weights being row weights). */
+int tfb_loss_multi_fwd(const void* logits, const void* targets, int idx64, const void* row_w, int K, float eps, void* loss,
+                       void* lse, long rows, int V, float softcap, void* stream);
+
+/* dlogits = g[row] (1 - tanh^2) (W softmax - (1 - eps) sum_k row_w[k][row] [v = t_k] - W eps / V), W = sum_k row_w[k][row];
+ * bf16, may alias logits. Replaces _loss_multi_bwd_kernel (round1/source/train.py:4778) and _lh_bwd_ls_kernel
+ * (round2/source/train.py:5767). */
+int tfb_loss_multi_bwd(const void* logits, const void* targets, int idx64, const void* row_w, int K, float eps, const void* lse,
+                       const void* g, void* dlogits, long rows, int V, float softcap, void* stream);
 
 /* logits = x @ W^T (x [rows][d], W [V][d]) with the row log-sum-exp reduced in the GEMM epilogue, then loss / lse as
  * tfb_loss_fwd. part: fp32 [rows][V/64][2] scratch. rows, V multiples of 128, d of 64.

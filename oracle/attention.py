@@ -94,3 +94,27 @@ def rope_backward(gy, cos, sin):
     s = sin.float()[None, :, None, :]
     g1, g2 = gy.float()[..., : D // 2], gy.float()[..., D // 2:]
     return torch.cat((g1 * c - g2 * s, g2 * c + g1 * s), dim=-1).to(gy.dtype)
+
+
+QK_NORM_EPS = 2.0 ** -23
+
+
+def rope_norm(x, cos, sin, eps=QK_NORM_EPS):
+    """(y, r, inv): r = rope(x) rounded to x's dtype, inv = rsqrt(mean_D(r^2) + eps) fp32 [..., 1], y = (r inv) rounded:
+    the rotation followed by the parameter-free per-head RMSNorm, norm(apply_rotary_emb(x, cos, sin)) of
+    round1/source/train.py:4184-4196 (kernel :4308; eps :4172), before its transpose(1, 2). x [B, T, H, D]."""
+    r = rope(x, cos, sin)
+    rf = r.float()
+    inv = torch.rsqrt(rf.pow(2).mean(-1, keepdim=True) + eps)
+    return (rf * inv).to(x.dtype), r, inv
+
+
+def rope_norm_backward(g, r, inv, cos, sin):
+    """Gradient of rope_norm's input (round1/source/train.py:4353-4381): u = g - r inv^2 (g . r) / D, gr = (u inv)
+    rounded to g's dtype, then the transposed rotation."""
+    gf, rf = g.float(), r.float()
+    D = g.shape[-1]
+    coef = inv * inv * (gf * rf).sum(-1, keepdim=True) / D
+    gr = ((gf - rf * coef) * inv).to(g.dtype)
+    return rope_backward(gr, cos, sin)
+

@@ -54,27 +54,30 @@ def add_rmsnorm_backward(gs, gy, s, inv, weight=None):
 
 
 def block_head(x, x0, l1, l2, skip=None, l3=None, eps=RMS_EPS):
-    """x_new = dtype(l1*x + l2*x0 [+ l3*skip]) in fp32 from fp32 gains; x_norm = norm(x_new); inv."""
-    v = l1.float() * x.float() + l2.float() * x0.float()
+    """x_new = dtype(l1*(x [+ l3*skip]) + l2*x0) in fp32 from fp32 gains (the skip joins the stream BEFORE the block
+    head: round1/source/train.py:5644-5647 eager form, kernel 5743-5744); x_norm = norm(x_new); inv."""
+    s = x.float()
     if skip is not None:
-        v = v + l3.float() * skip.float()
+        s = s + l3.float() * skip.float()
+    v = l1.float() * s + l2.float() * x0.float()
     x_new = v.to(x.dtype)
     x_norm, inv = rmsnorm(x_new, None, eps)
     return x_new, x_norm, inv
 
 
 def block_head_backward(g_new, g_norm, x, x0, x_new, inv, l1, l2, skip=None, l3=None):
-    """(dx, dx0, dskip, dl1, dl2, dl3) with G = g_new + J^T(g_norm); gain grads fp32 sums of G * input."""
+    """(dx, dx0, dskip, dl1, dl2, dl3) with G = g_new + J^T(g_norm): dx = l1 G, dx0 = l2 G, dskip = l1 l3 G; gain
+    grads fp32 sums G.(x + l3 skip), G.x0, l1 G.skip (round1/source/train.py:5794-5795)."""
     jt, _ = rmsnorm_backward(g_norm, x_new, inv, None)
     G = jt if g_new is None else jt + g_new.float()
     dt = x.dtype
     dx = (l1.float() * G).to(dt)
     dx0 = (l2.float() * G).to(dt)
-    dl1 = (G * x.float()).sum()
     dl2 = (G * x0.float()).sum()
     if skip is None:
-        return dx, dx0, None, dl1, dl2, None
-    return dx, dx0, (l3.float() * G).to(dt), dl1, dl2, (G * skip.float()).sum()
+        return dx, dx0, None, (G * x.float()).sum(), dl2, None
+    gs = (G * skip.float()).sum()
+    return dx, dx0, (l1.float() * l3.float() * G).to(dt), (G * x.float()).sum() + l3.float() * gs, dl2, l1.float() * gs
 
 
 def relu2(x):

@@ -1,0 +1,227 @@
+"""The reference-named host functions (trainium_frontier_them_bones_amd/train_api.py) called the way the reference's
+train.py calls them, checked against the oracle on the same seeded inputs. bf16 paths: rel-L2 <= 5e-3; fp8: <= 2e-2;
+loss: <= 1e-3 relative."""
+import math
+
+import pytest
+import torch
+
+from helpers import rel_l2
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL, FP8_TOL, LOSS_TOL = 5e-3, 2e-2, 1e-3
+
+
+def _g(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+@pytest.fixture(scope="module")
+def api():
+    from trainium_frontier_them_bones_amd import train_api
+    return train_api
+
+
+def test_nki_attn_fn_and_rope_norm(api, dev):
+    from oracle import attention as O
+    B, H, T, D = 2, 3, 256, 64
+    g = _g(1)
+    q, k, v = (torch.randn(B, H, T, D, generator=g).bfloat16() for _ in range(3))
+    go = torch.randn(B, T, H, D, generator=g).bfloat16()
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    y = api.nki_attn_fn(qd, kd, vd)                                       # scale=None -> 1 / sqrt(D)
+    assert y.shape == (B, T, H, D)
+    y.backward(go.to(dev))
+    o, lse = O.forward(q, k, v, 1.0 / math.sqrt(D))
+    dq, dk, dv = O.backward(q, k, v, o, go, lse, 1.0 / math.sqrt(D))
+    assert rel_l2(y, o) < BF16_TOL
+    assert rel_l2(qd.grad, dq) < BF16_TOL and rel_l2(kd.grad, dk) < BF16_TOL and rel_l2(vd.grad, dv) < BF16_TOL
+    assert y.data_ptr() != qd.data_ptr() and torch.equal(qd.detach().cpu(), q)   # inputs untouched
+    # rope_norm: [B, T, H, D] in, [B, H, T, D] out, tables in the reference's [1, T, 1, D/2] shape
+    for Dh in (64, 128):
+        x = torch.randn(B, T, H, Dh, generator=g).bfloat16()
+        cos, sin = O.rope_tables(T, Dh)
+        gy = torch.randn(B, H, T, Dh, generator=g).bfloat16()
+        xd = x.to(dev).requires_grad_(True)
+        yn = api.rope_norm(xd, cos.to(dev)[None, :, None, :], sin.to(dev)[None, :, None, :])
+        assert yn.shape == (B, H, T, Dh)
+        yn.backward(gy.to(dev))
+        yo, r, inv = O.rope_norm(x, cos, sin)
+        assert rel_l2(yn, yo.transpose(1, 2)) < 1e-3
+        assert float((yn.detach().cpu().float() - yo.transpose(1, 2).float()).abs().max()) <= 2.0 ** -6   # one bf16 ulp near 2
+        dxo = O.rope_norm_backward(gy.transpose(1, 2).contiguous(), r, inv, cos, sin)
+        assert rel_l2(xd.grad, dxo) < 2e-3
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_nki_rope_attention_with_qk_norm(api, dev, D):
+    from oracle import attention as O
+    B, T, H = 2, 256, 3
+    C = H * D
+    g = _g(2 + D)
+    qkv = torch.randn(B, T, 3 * C, generator=g).bfloat16()
+    go = torch.randn(B, T, H, D, generator=g).bfloat16()
+    cos, sin = O.rope_tables(T, D)
+    xd = qkv.to(dev).requires_grad_(True)
+    y = api.nki_rope_attention(xd, cos.to(dev), sin.to(dev), H, scale=0.11)
+    assert y.shape == (B, T, H, D)
+    y.backward(go.to(dev))
+    assert torch.equal(xd.detach().cpu(), qkv)                            # the fused projection output is not modified
+    # oracle: the unfused chain rope_norm -> causal attention, and its backward
+    q, k, v = (t.view(B, T, H, D) for t in qkv.split(C, dim=-1))
+    qn, rq, iq = O.rope_norm(q, cos, sin)
+    kn, rk, ik = O.rope_norm(k, cos, sin)
+    q4, k4, v4 = (t.transpose(1, 2).contiguous() for t in (qn, kn, v))
+    o, lse = O.forward(q4, k4, v4, 0.11)
+    assert rel_l2(y, o) < BF16_TOL
+    dq4, dk4, dv4 = O.backward(q4, k4, v4, o, go, lse, 0.11)
+    dq = O.rope_norm_backward(dq4.transpose(1, 2).contiguous(), rq, iq, cos, sin)
+    dk = O.rope_norm_backward(dk4.transpose(1, 2).contiguous(), rk, ik, cos, sin)
+    want = torch.cat([dq.reshape(B, T, C), dk.reshape(B, T, C), dv4.transpose(1, 2).reshape(B, T, C)], dim=-1)
+    assert rel_l2(xd.grad, want) < BF16_TOL
+    # "None = not done": a head size the kernels do not take
+    assert api.nki_rope_attention(torch.zeros(1, 128, 3 * 2 * 32, dtype=torch.bfloat16, device=dev), cos.to(dev), sin.to(dev), 2) is None
+
+
+def test_fused_loss_family(api, dev):
+    from oracle import loss as O
+    g = _g(5)
+    B, T, V, K = 2, 128, 1024, 3
+    N = B * T
+    x = (3 * torch.randn(B, T, V, generator=g)).bfloat16()
+    t = torch.randint(0, V, (B, T), generator=g)
+    t[0, 3] = -1
+    for red in ("mean", "sum", "none"):
+        xd = x.to(dev).requires_grad_(True)
+        got = api.fused_loss(xd, t.to(dev), red)
+        want = O.fused_loss(x, t, red, 15.0)
+        if red == "none":
+            assert got.shape == t.shape and rel_l2(got, want) < LOSS_TOL
+            got.sum().backward()
+        else:
+            assert abs(got.item() - want.item()) < LOSS_TOL * abs(want.item())
+            got.backward()
+        rows, lse = O.loss_rows(x.reshape(N, V), t, 15.0)
+        grow = O.row_weights(t, "mean") if red == "mean" else (t.reshape(-1) >= 0).float()
+        assert rel_l2(xd.grad.reshape(N, V), O.loss_backward(x.reshape(N, V), t, lse, grow, 15.0)) < BF16_TOL
+    # several targets per row (multi-token prediction)
+    tg = torch.randint(0, V, (K, N), generator=g)
+    tg[1, 7] = -1
+    rw = torch.rand(K, N, generator=g)
+    xd = x.to(dev).requires_grad_(True)
+    got = api.fused_loss_multi(xd, tg.to(dev), rw.to(dev))
+    rows, lse = O.loss_multi_rows(x.reshape(N, V), tg, rw, 15.0)
+    assert abs(got.item() - rows.sum().item()) < LOSS_TOL * rows.sum().item()
+    got.backward()
+    assert rel_l2(xd.grad.reshape(N, V), O.loss_multi_backward(x.reshape(N, V), tg, rw, lse, torch.ones(N), 15.0)) < BF16_TOL
+    assert api.fused_loss_multi(xd, tg.to(dev).repeat(4, 1), rw.to(dev).repeat(4, 1)) is None      # K = 12: not taken
+    # label smoothing and per-token weights (R2's chunked_loss_mean)
+    tok_w = 1.0 + torch.rand(B, T, generator=g)
+    for smooth, eps in ((False, 0.0), (True, 0.1)):
+        xd = x.to(dev).requires_grad_(True)
+        got = api.chunked_loss_mean(xd, t.to(dev), smooth=smooth, tok_w=tok_w.to(dev), eps=eps)
+        w = (O.row_weights(t, "mean") * tok_w.reshape(-1)).view(1, N)
+        rows, lse = O.loss_multi_rows(x.reshape(N, V), t.view(1, N), w, 15.0, eps)
+        assert abs(got.item() - rows.sum().item()) < LOSS_TOL * rows.sum().item()
+        got.backward()
+        want = O.loss_multi_backward(x.reshape(N, V), t.view(1, N), w, lse, torch.ones(N), 15.0, eps)
+        assert rel_l2(xd.grad.reshape(N, V), want) < BF16_TOL
+    s = 15.0 * torch.tanh(x.float().reshape(N, V) / 15.0)
+    lib = torch.nn.functional.cross_entropy(s, t.reshape(-1), ignore_index=-1, label_smoothing=0.1)
+    got = api.chunked_loss_mean(x.to(dev), t.to(dev), smooth=True, eps=0.1)
+    assert abs(got.item() - lib.item()) < LOSS_TOL * lib.item()
+
+
+def test_norm_blocks_and_relu2(api, dev):
+    from oracle import norm as O
+    g = _g(6)
+    shape = (2, 128, 768)
+    x, x0, sk, a, gn, gy = (torch.randn(*shape, generator=g).bfloat16() for _ in range(6))
+    l1, l2, l3 = (torch.tensor([v]) for v in (0.9, 0.25, -0.4))
+    ld = [t.to(dev).requires_grad_(True) for t in (l1, l2, l3)]
+    xd, x0d, skd = (t.to(dev).requires_grad_(True) for t in (x, x0, sk))
+    xn, xnorm = api.head_skip(xd, x0d, skd, *ld)
+    (xn.float() * gn.to(dev).float()).sum().backward(retain_graph=True)
+    (xnorm.float() * gy.to(dev).float()).sum().backward()
+    o = O.block_head(x.view(-1, 768), x0.view(-1, 768), l1[0], l2[0], sk.view(-1, 768), l3[0])
+    assert rel_l2(xn, o[0].view(shape)) < 1e-3 and rel_l2(xnorm, o[1].view(shape)) < 1e-3
+    eager = (x + l3.to(x.dtype) * sk)                                   # R1:5646, then the block head
+    assert rel_l2(xn, (l1 * eager.float() + l2 * x0.float())) < BF16_TOL
+    ob = O.block_head_backward(gn.view(-1, 768), gy.view(-1, 768), x.view(-1, 768), x0.view(-1, 768), o[0], o[2], l1[0], l2[0],
+                               sk.view(-1, 768), l3[0])
+    assert rel_l2(xd.grad, ob[0].view(shape)) < BF16_TOL and rel_l2(x0d.grad, ob[1].view(shape)) < BF16_TOL
+    assert rel_l2(skd.grad, ob[2].view(shape)) < BF16_TOL
+    for got, want in zip(ld, ob[3:]):
+        assert abs(got.grad.item() - want.item()) < 1e-3 * abs(want.item()) + 0.05
+    xn2, xnorm2 = api.block_head(x.to(dev), x0.to(dev), l1.to(dev), l2.to(dev))
+    o2 = O.block_head(x, x0, l1[0], l2[0])
+    assert rel_l2(xn2, o2[0]) < 1e-3 and rel_l2(xnorm2, o2[1]) < 1e-3
+    assert rel_l2(api.rmsnorm_fast(x.to(dev)), O.rmsnorm(x, None, O.RMS_EPS)[0]) < 1e-3
+    s1, y = api.tail_norm2(x.to(dev), a.to(dev))
+    so, yo, _ = O.add_rmsnorm(x, a)
+    assert torch.equal(s1.cpu(), so) and rel_l2(y, yo) < 1e-3
+    assert rel_l2(api.final_norm(x.to(dev), a.to(dev)), yo) < 1e-3
+    assert torch.equal(api.relu_squared(x.to(dev)).cpu(), O.relu2(x))
+
+
+def test_gemm_glue_and_mlp_fused8(api, dev):
+    from oracle import mlp8 as O8
+    g = _g(7)
+    M, d, F = 384, 256, 512
+    x = torch.randn(3, 128, d, generator=g).bfloat16()
+    w = (0.05 * torch.randn(d, F, generator=g)).bfloat16()                # LinearT [in, out]
+    xd, wd = x.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+    h = api.fused_fc_relu2(xd, wd)
+    ref = torch.relu(x.float().reshape(M, d) @ w.float()).bfloat16().float().square().bfloat16()
+    assert h.shape == (3, 128, F) and rel_l2(h, ref.view(3, 128, F)) < BF16_TOL
+    gh = torch.randn(3, 128, F, generator=g).bfloat16()
+    h.backward(gh.to(dev))
+    xf, wf = x.float().reshape(M, d).requires_grad_(True), w.float().requires_grad_(True)
+    (torch.relu(xf @ wf).square() * gh.float().reshape(M, F)).sum().backward()
+    assert rel_l2(xd.grad.reshape(M, d), xf.grad) < 1e-2 and rel_l2(wd.grad, wf.grad) < 1e-2
+    # inplace=True: the weight gradient is summed into an existing w.grad, the op answers None for it
+    wd2 = w.to(dev).requires_grad_(True)
+    wd2.grad = torch.ones_like(wd2)
+    api.fused_fc_relu2(x.to(dev), wd2, inplace=True).backward(gh.to(dev))
+    assert rel_l2(wd2.grad, wf.grad + 1.0) < 1e-2
+    a2, b2 = torch.randn(M, d, generator=g).bfloat16(), torch.randn(M, F, generator=g).bfloat16()
+    assert rel_l2(api.nki_matmul(a2.to(dev), b2.to(dev), trans_a=True), a2.float().t() @ b2.float()) < BF16_TOL
+    assert rel_l2(api.dw_matmul(a2.to(dev), b2.to(dev)), a2.float().t() @ b2.float()) < BF16_TOL
+    assert api.dw_matmul(a2.to(dev)[:, :100].contiguous(), b2.to(dev)) is None
+    # the fp8 MLP on a module with c_fc / c_proj, 300 tokens (padded to 384 inside)
+    mlp = torch.nn.Module()
+    mlp.c_fc = torch.nn.Linear(d, F, bias=False)
+    mlp.c_proj = torch.nn.Linear(F, d, bias=False)
+    wf8 = (0.05 * torch.randn(F, d, generator=g)).bfloat16()
+    wp8 = (0.05 * torch.randn(d, F, generator=g)).bfloat16()
+    mlp.c_fc.weight.data, mlp.c_proj.weight.data = wf8.clone(), wp8.clone()
+    mlp = mlp.to(dev)
+    xm = torch.randn(3, 100, d, generator=g).bfloat16()
+    xmd = xm.to(dev).requires_grad_(True)
+    y = api.mlp_fused8(mlp, xmd)
+    row = O8.forward_scales(wf8, wp8)
+    yo, ro = O8.forward(xm.reshape(300, d), wf8, wp8, row)
+    assert y.shape == xm.shape and rel_l2(y.reshape(300, d), yo) < FP8_TOL
+    gy = torch.randn(3, 100, d, generator=g).bfloat16()
+    y.backward(gy.to(dev))
+    gpad = torch.cat([gy.reshape(300, d), torch.zeros(84, d, dtype=torch.bfloat16)])   # the amax of dy ignores zero rows
+    dxo, ho, dpo = O8.backward(gy.reshape(300, d), ro, wf8, wp8, O8.backward_scales(gpad, row))
+    assert rel_l2(xmd.grad.reshape(300, d), dxo) < FP8_TOL
+    dwf, dwp = O8.weight_grads(gy.reshape(300, d), xm.reshape(300, d), ho, dpo)
+    assert rel_l2(mlp.c_fc.weight.grad, dwf) < FP8_TOL and rel_l2(mlp.c_proj.weight.grad, dwp) < FP8_TOL
+    assert torch.equal(api.forward_scales(wf8.to(dev), wp8.to(dev)).cpu()[[0, 3, 13]], row[[0, 3, 13]])
+
+
+def test_embedding_fwd(api, dev):
+    g = _g(8)
+    V, C = 1024, 256
+    w = torch.randn(V, C, generator=g).bfloat16()
+    idx = torch.randint(0, V, (2, 128), generator=g)
+    wd = w.to(dev).requires_grad_(True)
+    e = api.embedding_fwd(idx.to(dev), wd, torch.bfloat16)
+    assert torch.equal(e.cpu(), w[idx])
+    gy = torch.randn(2, 128, C, generator=g).bfloat16()
+    e.backward(gy.to(dev))
+    want = torch.zeros(V, C).index_add_(0, idx.reshape(-1), gy.float().reshape(-1, C))
+    assert rel_l2(wd.grad, want) < BF16_TOL

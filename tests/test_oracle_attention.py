@@ -93,3 +93,31 @@ def test_rope_is_a_rotation():
     xr = x.clone().requires_grad_(True)
     O.rope(xr, cos, sin).backward(y)
     assert torch.allclose(xr.grad, O.rope_backward(y, cos, sin), atol=1e-6)
+
+
+def test_rope_norm_is_library_rms_norm_of_the_rotation_and_autograd():
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(6)
+    B, T, H, D = 2, 64, 3, 64
+    x = torch.randn(B, T, H, D, generator=g).bfloat16()
+    cos, sin = O.rope_tables(T, D)
+    y, r, inv = O.rope_norm(x, cos, sin)
+    assert torch.equal(r, O.rope(x, cos, sin))
+    # the library routine on the rounded rotation (fp32 in, the oracle's eps), one rounding
+    assert torch.equal(y, F.rms_norm(r.float(), (D,), eps=O.QK_NORM_EPS).to(x.dtype))
+    assert torch.allclose(y.float().pow(2).mean(-1), torch.ones(B, T, H), atol=2e-2)   # unit RMS per head
+    assert torch.allclose(inv.squeeze(-1), 1.0 / r.float().pow(2).mean(-1).sqrt(), rtol=1e-5)
+    # gradient: autograd of rms_norm(rope(x)) in fp64 (no intermediate roundings there)
+    gy = torch.randn(B, T, H, D, generator=g).bfloat16()
+    xd = x.double().requires_grad_(True)
+    c, s = cos.double()[None, :, None, :], sin.double()[None, :, None, :]
+    x1, x2 = xd[..., : D // 2], xd[..., D // 2:]
+    rd = torch.cat((x1 * c + x2 * s, x2 * c - x1 * s), dim=-1)
+    F.rms_norm(rd, (D,), eps=O.QK_NORM_EPS).backward(gy.double())
+    dx = O.rope_norm_backward(gy, r, inv, cos, sin)
+    assert rel_l2(dx, xd.grad) < 6e-3                                                   # bf16 roundings of r, gr, dx
+    # the norm's Jacobian annihilates the radial direction: a gradient along y itself gives (almost) nothing
+    dx_rad = O.rope_norm_backward(y, r, inv, cos, sin)
+    assert float(dx_rad.float().abs().max()) < 2e-2 * float(dx.float().abs().max())
+    # scale invariance: rope_norm(4 x) == rope_norm(x) bit for bit (powers of two commute with every rounding)
+    assert torch.equal(O.rope_norm((x.float() * 4).bfloat16(), cos, sin, eps=O.QK_NORM_EPS * 16)[0], y)

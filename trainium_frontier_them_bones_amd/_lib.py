@@ -44,6 +44,8 @@ SIGNATURES = {
     "tfb_gemm_fp8": [_vp, _i, _vp, _vp, _vp, _f, _vp, _l, _i, _i, _vp],
     "tfb_relu2": [_vp, _vp, _vp, _l, _i, _vp],
     "tfb_rope": [_vp, _vp, _vp, _vp, _l, _i, _i, _i, _l, _l, _i, _vp],
+    "tfb_rope_norm_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _i, _l, _l, _l, _f, _vp],
+    "tfb_rope_norm_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _i, _l, _l, _l, _vp],
     "tfb_resmix_bwd_blocks": [_l],
     "tfb_resmix_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _vp],
     "tfb_embedding_fwd": [_vp, _i, _vp, _vp, _l, _i, _vp],
@@ -54,6 +56,8 @@ SIGNATURES = {
     "tfb_fill_f32": [_vp, _f, _l, _vp],
     "tfb_loss_fwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_loss_bwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
+    "tfb_loss_multi_fwd": [_vp, _vp, _i, _vp, _i, _f, _vp, _vp, _l, _i, _f, _vp],
+    "tfb_loss_multi_bwd": [_vp, _vp, _i, _vp, _i, _f, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_lmhead_fwd": [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _f, _vp],
     "tfb_moe_max_rows": [_l, _i, _i],
     "tfb_moe_route": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _i, _vp],

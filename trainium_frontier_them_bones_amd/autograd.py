@@ -165,6 +165,64 @@ class RopeAttentionFn(torch.autograd.Function):
         return dqkv, None, None, None, None
 
 
+class RopeNormFn(torch.autograd.Function):
+    """norm(apply_rotary_emb(x, cos, sin)) for x [B, T, H, D]: RoPE then the parameter-free per-head RMSNorm
+    (round1/source/train.py:4411 RopeNormFn; rope_norm 4447 returns this transposed to [B, H, T, D])."""
+
+    @staticmethod
+    def forward(ctx, x, cos, sin, eps):
+        B, T, H, D = x.shape
+        x = x.contiguous()
+        y, r, inv = ops.rope_norm_fwd(x.view(B * T, H * D), cos, sin, T, H, D, eps)
+        ctx.save_for_backward(r, inv, cos, sin)
+        ctx.dims = (B, T, H, D)
+        return y.view(B, T, H, D)
+
+    @staticmethod
+    def backward(ctx, gy):
+        r, inv, cos, sin = ctx.saved_tensors
+        B, T, H, D = ctx.dims
+        dx = ops.rope_norm_bwd(gy.contiguous().view(B * T, H * D), r, inv, cos, sin, T, H, D)
+        return dx.view(B, T, H, D), None, None, None
+
+
+class RopeNormAttentionFn(torch.autograd.Function):
+    """nki_rope_attention(qkv, cos, sin, n_head, scale) (round1/source/train.py:8197, NkiRopeAttnFn 8135): causal
+    SDPA(QKnorm(RoPE(q)), QKnorm(RoPE(k)), v) straight from the fused projection output qkv [B, T, 3C], one dqkv
+    [B, T, 3C] back. The input is not modified: the normalised q and k go to a fresh buffer, v is read in place through
+    strides; saved for backward: qkv's v third, the rotated q, k (r5), their inverse RMS (inv3), o, lse."""
+
+    @staticmethod
+    def forward(ctx, qkv, cos, sin, n_head, scale, eps):
+        B, T, C3 = qkv.shape
+        C = C3 // 3
+        D = C // n_head
+        qkv = qkv.contiguous()
+        qk, r, inv = ops.rope_norm_fwd(qkv.view(B * T, C3), cos, sin, T, 2 * n_head, D, eps)
+        q, k = (t.view(B, T, n_head, D) for t in qk.view(B, T, 2 * C).split(C, dim=-1))
+        v = qkv[..., 2 * C:].view(B, T, n_head, D)
+        o, lse = ops.attn_fwd(q, k, v, scale, "bthd")
+        ctx.save_for_backward(qkv, qk, r, inv, o, lse, cos, sin)
+        ctx.n_head, ctx.scale = n_head, scale
+        return o.view(B, T, C)
+
+    @staticmethod
+    def backward(ctx, go):
+        qkv, qk, r, inv, o, lse, cos, sin = ctx.saved_tensors
+        B, T, C3 = qkv.shape
+        C = C3 // 3
+        H = ctx.n_head
+        D = C // H
+        q, k = (t.view(B, T, H, D) for t in qk.view(B, T, 2 * C).split(C, dim=-1))
+        v = qkv[..., 2 * C:].view(B, T, H, D)
+        dqkv = torch.empty_like(qkv)
+        dq, dk, dv = (t.view(B, T, H, D) for t in dqkv.split(C, dim=-1))
+        ops.attn_bwd(q, k, v, o, go.contiguous().view(B, T, H, D), lse, ctx.scale, "bthd", dq, dk, dv, "bthd")
+        g2 = dqkv.view(B * T, C3)
+        ops.rope_norm_bwd(g2, r, inv, cos, sin, T, 2 * H, D, out=g2)   # in place on the q and k thirds
+        return dqkv, None, None, None, None, None
+
+
 class QkvRopeAttentionFn(torch.autograd.Function):
     """Attention block core in one autograd node: qkv = rope(x @ w_qkv^T) (rotation in the projection's epilogue), causal
     attention on the thirds, and in backward the inverse rotation inside the attention kernels' stores followed by the
@@ -367,6 +425,23 @@ class FusedLossFn(torch.autograd.Function):
     def backward(ctx, grows):
         logits2, targets, lse = ctx.saved_tensors
         return ops.loss_bwd(logits2, targets, lse, grows.contiguous().float(), ctx.softcap), None, None
+
+
+class FusedLossMultiFn(torch.autograd.Function):
+    """rows [N] = sum_k rw[k] (lse - (1 - eps) s_{t_k} - eps mean_v s_v) on materialised logits: several targets per row
+    (round1/source/train.py:4870 LossMultiFn) and / or label smoothing (round2/source/train.py:6344 ChunkedLossHeadLS)."""
+
+    @staticmethod
+    def forward(ctx, logits2, tg, rw, softcap, eps):
+        rows, lse = ops.loss_multi_fwd(logits2, tg, rw, softcap, eps)
+        ctx.save_for_backward(logits2, tg, rw, lse)
+        ctx.softcap, ctx.eps = softcap, eps
+        return rows
+
+    @staticmethod
+    def backward(ctx, grows):
+        logits2, tg, rw, lse = ctx.saved_tensors
+        return ops.loss_multi_bwd(logits2, tg, rw, lse, grows.contiguous().float(), ctx.softcap, ctx.eps), None, None, None, None
 
 
 class EmbeddingFn(torch.autograd.Function):

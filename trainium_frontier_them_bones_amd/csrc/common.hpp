@@ -56,6 +56,19 @@ __device__ __forceinline__ float sum2bf(uint32_t w, float acc) {
 // reference arithmetic that stays in registers).
 __device__ __forceinline__ float round_bf(float f) { return bf2f(f2bf(f)); }
 
+// 8 fp32 values <-> 8 bf16 in four 32-bit words (one 128-bit access)
+__device__ __forceinline__ u32x4 pack8bf(const float (&v)[8]) {
+  u32x4 o = {pack2bf(v[0], v[1]), pack2bf(v[2], v[3]), pack2bf(v[4], v[5]), pack2bf(v[6], v[7])};
+  return o;
+}
+__device__ __forceinline__ void unpack8bf(u32x4 u, float (&v)[8]) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    v[2 * k] = bflo(u[k]);
+    v[2 * k + 1] = bfhi(u[k]);
+  }
+}
+
 // fp32 -> OCP fp8 bytes (gfx950's v_cvt_pk_*_f32 are OCP e4m3fn / e5m2, round to nearest
 // even). Inputs are clamped to the format's finite range first, so a value beyond it
 // saturates instead of becoming NaN/Inf; inside the range the bytes are torch's

@@ -84,6 +84,116 @@ __global__ __launch_bounds__(256) void rope_kernel(const bf16_t* __restrict__ x,
   }
 }
 
+// RoPE followed by the parameter-free RMSNorm of each head (the attention block's QK-norm): r = bf16(rope(x)),
+// inv = rsqrt(mean(r^2) + eps) over the head's D elements, y = bf16(r inv). D / 16 lanes share a head (a lane holds 8
+// elements of each half); heads laid out as in rope_kernel. r_out may be NULL.
+__global__ __launch_bounds__(256) void rope_norm_fwd_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ cs,
+                                                           const bf16_t* __restrict__ sn, bf16_t* __restrict__ r_out,
+                                                           bf16_t* __restrict__ y_out, float* __restrict__ inv_out, long rows,
+                                                           int T, int nheads, int D, long x_stride, long r_stride,
+                                                           long y_stride, float eps) {
+  const int hc = D / 16;  // lanes per head: 4 (D = 64) or 8 (D = 128), a power of two
+  const long per_row = (long)nheads * hc;
+  const long total = rows * per_row;
+  const long span = ((total + 63) / 64) * 64;  // whole wavefronts stay in the loop for the shuffles
+  for (long idx = (long)blockIdx.x * 256 + threadIdx.x; idx < span; idx += (long)gridDim.x * 256) {
+    const bool live = idx < total;
+    const long id = live ? idx : total - 1;
+    const long row = id / per_row;
+    const int rem = (int)(id % per_row);
+    const int head = rem / hc, c = rem % hc;
+    const int t = (int)(row % T);
+    const bf16_t* p1 = x + row * x_stride + (long)head * D + c * 8;
+    const u32x4 a = *(const u32x4*)p1, b = *(const u32x4*)(p1 + D / 2);
+    const u32x4 cc = *(const u32x4*)(cs + (long)t * (D / 2) + c * 8), ss = *(const u32x4*)(sn + (long)t * (D / 2) + c * 8);
+    float r1[8], r2[8], sq = 0.f;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float a0 = bflo(a[k]), a1 = bfhi(a[k]), b0 = bflo(b[k]), b1 = bfhi(b[k]);
+      const float c0 = bflo(cc[k]), c1 = bfhi(cc[k]), s0 = bflo(ss[k]), s1 = bfhi(ss[k]);
+      r1[2 * k] = round_bf(a0 * c0 + b0 * s0);
+      r1[2 * k + 1] = round_bf(a1 * c1 + b1 * s1);
+      r2[2 * k] = round_bf(b0 * c0 - a0 * s0);
+      r2[2 * k + 1] = round_bf(b1 * c1 - a1 * s1);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) sq += r1[k] * r1[k] + r2[k] * r2[k];
+    for (int o = 1; o < hc; o <<= 1) sq += __shfl_xor(sq, o, 64);
+    const float inv = rsqrtf(sq / (float)D + eps);
+    if (!live) continue;
+    if (r_out) {
+      bf16_t* q = r_out + row * r_stride + (long)head * D + c * 8;
+      *(u32x4*)q = pack8bf(r1);
+      *(u32x4*)(q + D / 2) = pack8bf(r2);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      r1[k] *= inv;
+      r2[k] *= inv;
+    }
+    bf16_t* q = y_out + row * y_stride + (long)head * D + c * 8;
+    *(u32x4*)q = pack8bf(r1);
+    *(u32x4*)(q + D / 2) = pack8bf(r2);
+    if (c == 0) inv_out[row * nheads + head] = inv;
+  }
+}
+
+// Gradient of rope_norm_fwd: rh = r inv, dr = bf16(inv (g - rh (g . rh) / D)), then the transposed rotation
+// dx1 = dr1 c - dr2 s, dx2 = dr2 c + dr1 s, one rounding.
+__global__ __launch_bounds__(256) void rope_norm_bwd_kernel(const bf16_t* __restrict__ g, const bf16_t* __restrict__ r,
+                                                           const float* __restrict__ inv_in, const bf16_t* __restrict__ cs,
+                                                           const bf16_t* __restrict__ sn, bf16_t* __restrict__ dx, long rows,
+                                                           int T, int nheads, int D, long g_stride, long r_stride,
+                                                           long dx_stride) {
+  const int hc = D / 16;
+  const long per_row = (long)nheads * hc;
+  const long total = rows * per_row;
+  const long span = ((total + 63) / 64) * 64;
+  for (long idx = (long)blockIdx.x * 256 + threadIdx.x; idx < span; idx += (long)gridDim.x * 256) {
+    const bool live = idx < total;
+    const long id = live ? idx : total - 1;
+    const long row = id / per_row;
+    const int rem = (int)(id % per_row);
+    const int head = rem / hc, c = rem % hc;
+    const int t = (int)(row % T);
+    const long off = (long)head * D + c * 8;
+    const u32x4 ga = *(const u32x4*)(g + row * g_stride + off), gb = *(const u32x4*)(g + row * g_stride + off + D / 2);
+    const u32x4 ra = *(const u32x4*)(r + row * r_stride + off), rb = *(const u32x4*)(r + row * r_stride + off + D / 2);
+    const float inv = inv_in[row * nheads + head];
+    float g1[8], g2[8], h1[8], h2[8], dot = 0.f;
+    unpack8bf(ga, g1);
+    unpack8bf(gb, g2);
+    unpack8bf(ra, h1);
+    unpack8bf(rb, h2);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      h1[k] *= inv;
+      h2[k] *= inv;
+      dot += g1[k] * h1[k] + g2[k] * h2[k];
+    }
+    for (int o = 1; o < hc; o <<= 1) dot += __shfl_xor(dot, o, 64);
+    if (!live) continue;
+    const float coef = dot / (float)D;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      g1[k] = round_bf(inv * (g1[k] - h1[k] * coef));
+      g2[k] = round_bf(inv * (g2[k] - h2[k] * coef));
+    }
+    const u32x4 cc = *(const u32x4*)(cs + (long)t * (D / 2) + c * 8), ss = *(const u32x4*)(sn + (long)t * (D / 2) + c * 8);
+    float cf[8], sf[8], o1[8], o2[8];
+    unpack8bf(cc, cf);
+    unpack8bf(ss, sf);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      o1[k] = g1[k] * cf[k] - g2[k] * sf[k];
+      o2[k] = g2[k] * cf[k] + g1[k] * sf[k];
+    }
+    bf16_t* q = dx + row * dx_stride + off;
+    *(u32x4*)q = pack8bf(o1);
+    *(u32x4*)(q + D / 2) = pack8bf(o2);
+  }
+}
+
 // dx = g * bf16(a), dx0 = g * bf16(b) (products rounded to bf16), partial sums of bf16(g x) and bf16(g x0) in fp32.
 __global__ __launch_bounds__(256) void resmix_bwd_kernel(const bf16_t* __restrict__ g, const bf16_t* __restrict__ x,
                                                         const bf16_t* __restrict__ x0, const float* __restrict__ ab,
@@ -331,6 +441,36 @@ extern "C" int tfb_rope(const void* x, const void* cos_t, const void* sin_t, voi
   long total = rows * nheads * (D / 16);
   hipLaunchKernelGGL(rope_kernel, dim3(blocks_for(total)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x,
                      (const bf16_t*)cos_t, (const bf16_t*)sin_t, (bf16_t*)out, rows, T, nheads, D, row_stride, out_stride, inverse);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// x [rows][x_stride] holds nheads heads of D elements from column 0 (row = token, row % T its position): y = the
+// RMS-normalised rotation, r (NULL to skip) the rotation before the norm, inv fp32 [rows][nheads]. D = 64 or 128.
+extern "C" int tfb_rope_norm_fwd(const void* x, const void* cos_t, const void* sin_t, void* r, void* y, void* inv, long rows, int T,
+                                 int nheads, int D, long x_stride, long r_stride, long y_stride, float eps, void* stream) {
+  if (!x || !cos_t || !sin_t || !y || !inv) return TFB_ERR_ARG;
+  if (rows <= 0 || T <= 0 || nheads <= 0 || (D != 64 && D != 128) || x_stride % 8 || r_stride % 8 || y_stride % 8)
+    return TFB_ERR_SHAPE;
+  const long total = rows * nheads * (D / 16);
+  hipLaunchKernelGGL(rope_norm_fwd_kernel, dim3(blocks_for(total)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x,
+                     (const bf16_t*)cos_t, (const bf16_t*)sin_t, (bf16_t*)r, (bf16_t*)y, (float*)inv, rows, T, nheads, D,
+                     x_stride, r_stride, y_stride, eps);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// dx = gradient of tfb_rope_norm_fwd's input from g = gradient of y, the saved r and inv. dx may alias g.
+extern "C" int tfb_rope_norm_bwd(const void* g, const void* r, const void* inv, const void* cos_t, const void* sin_t, void* dx,
+                                 long rows, int T, int nheads, int D, long g_stride, long r_stride, long dx_stride,
+                                 void* stream) {
+  if (!g || !r || !inv || !cos_t || !sin_t || !dx) return TFB_ERR_ARG;
+  if (rows <= 0 || T <= 0 || nheads <= 0 || (D != 64 && D != 128) || g_stride % 8 || r_stride % 8 || dx_stride % 8)
+    return TFB_ERR_SHAPE;
+  const long total = rows * nheads * (D / 16);
+  hipLaunchKernelGGL(rope_norm_bwd_kernel, dim3(blocks_for(total)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)g,
+                     (const bf16_t*)r, (const float*)inv, (const bf16_t*)cos_t, (const bf16_t*)sin_t, (bf16_t*)dx, rows, T,
+                     nheads, D, g_stride, r_stride, dx_stride);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

@@ -549,17 +549,6 @@ static int gemm_launch_args(GemmArgs a, int groups_y, int splits, PreP prep, Pre
   return TFB_OK;
 }
 // ---- shared epilogue helpers -----------------------------------------------------------------
-__device__ __forceinline__ u32x4 pack8bf(const float (&v)[8]) {
-  u32x4 o = {pack2bf(v[0], v[1]), pack2bf(v[2], v[3]), pack2bf(v[4], v[5]), pack2bf(v[6], v[7])};
-  return o;
-}
-__device__ __forceinline__ void unpack8bf(u32x4 u, float (&v)[8]) {
-#pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    v[2 * k] = bflo(u[k]);
-    v[2 * k + 1] = bfhi(u[k]);
-  }
-}
 
 // out (bf16 or fp32) [nq][ld] (+)= D
 struct EpiStore {

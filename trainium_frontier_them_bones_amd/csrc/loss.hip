@@ -137,6 +137,137 @@ __global__ __launch_bounds__(256) void loss_bwd_kernel(const bf16_t* __restrict_
   }
 }
 
+// ------------------------------------------------------------------------------------ several targets / label smoothing
+// loss_row = sum_k rw_k (lse - (1 - eps) s_{t_k} - (eps / V) sum_v s_v), targets tg [K][rows] and weights rw [K][rows]
+// (a target < 0 counts with weight 0). K > 1 is the multi-token-prediction loss (round1/source/train.py:4725), eps > 0
+// the label-smoothed loss (round2/source/train.py:5697); K = 1, eps = 0 is loss_fwd_kernel with row weights.
+// d x_v = g (1 - tanh^2) (W softmax_v - (1 - eps) sum_k rw_k [v = t_k] - W eps / V), W = sum_k rw_k.
+constexpr int LOSS_KMAX = 8;
+
+template <typename IDX>
+__global__ __launch_bounds__(256) void loss_multi_fwd_kernel(const bf16_t* __restrict__ x, const IDX* __restrict__ tg,
+                                                            const float* __restrict__ rw, int K, long rows,
+                                                            float* __restrict__ loss, float* __restrict__ lse, int V, float cap,
+                                                            float eps) {
+  __shared__ float rm[4], rs[4], rt[4];
+  const long row = blockIdx.x;
+  const bf16_t* xr = x + row * V;
+  const float icap = cap > 0.f ? 1.0f / cap : 0.f;
+  MS a{-1e30f, 0.f};
+  float ssum = 0.f;  // sum_v s_v (label smoothing)
+  for (int i = threadIdx.x * 8; i < V; i += 256 * 8) {
+    u32x4 u = *(const u32x4*)(xr + i);
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      v[2 * k] = bflo(u[k]);
+      v[2 * k + 1] = bfhi(u[k]);
+    }
+    if (cap > 0.f) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const float sv = cap * tanh_fast(v[k] * icap);
+        ssum += sv;
+        a.s += fexp(sv - cap);
+      }
+      a.m = cap;
+    } else {
+      float mx = a.m;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) mx = fmaxf(mx, v[k]);
+      float sc = fexp(a.m - mx), t = 0.f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        t += fexp(v[k] - mx);
+        ssum += v[k];
+      }
+      a.s = a.s * sc + t;
+      a.m = mx;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    MS b{__shfl_xor(a.m, o, 64), __shfl_xor(a.s, o, 64)};
+    a = ms_merge(a, b);
+    ssum += __shfl_xor(ssum, o, 64);
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    rm[wave] = a.m;
+    rs[wave] = a.s;
+    rt[wave] = ssum;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    MS t{rm[0], rs[0]};
+    for (int i = 1; i < 4; ++i) t = ms_merge(t, MS{rm[i], rs[i]});
+    const float l = t.m + logf(t.s);
+    const float mean_s = (rt[0] + rt[1] + rt[2] + rt[3]) / (float)V;
+    lse[row] = l;
+    float out = 0.f;
+    for (int k = 0; k < K; ++k) {
+      const long tt = (long)tg[(long)k * rows + row];
+      if (tt < 0) continue;
+      const float xt = bf2f(xr[tt]);
+      const float st = cap > 0.f ? cap * tanh_fast(xt * icap) : xt;
+      out += rw[(long)k * rows + row] * (l - (1.0f - eps) * st - eps * mean_s);
+    }
+    loss[row] = out;
+  }
+}
+
+template <typename IDX>
+__global__ __launch_bounds__(256) void loss_multi_bwd_kernel(const bf16_t* __restrict__ x, const IDX* __restrict__ tg,
+                                                            const float* __restrict__ rw, int K, long rows,
+                                                            const float* __restrict__ lse, const float* __restrict__ g,
+                                                            bf16_t* __restrict__ dx, int V, float cap, float eps) {
+  const long row = blockIdx.x;
+  const bf16_t* xr = x + row * V;
+  bf16_t* dr = dx + row * V;
+  long tk[LOSS_KMAX];
+  float wk[LOSS_KMAX];
+  float W = 0.f;
+#pragma unroll
+  for (int k = 0; k < LOSS_KMAX; ++k) {
+    tk[k] = -1;
+    wk[k] = 0.f;
+    if (k < K) {
+      tk[k] = (long)tg[(long)k * rows + row];
+      if (tk[k] >= 0) {
+        wk[k] = rw[(long)k * rows + row];
+        W += wk[k];
+      }
+    }
+  }
+  const float gr = g[row];
+  const float l = lse[row];
+  const float icap = cap > 0.f ? 1.0f / cap : 0.f;
+  const float flat = W * eps / (float)V, keep = 1.0f - eps;
+  for (int i = threadIdx.x * 8; i < V; i += 256 * 8) {
+    u32x4 u = *(const u32x4*)(xr + i);
+    float v[8], d[8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      v[2 * k] = bflo(u[k]);
+      v[2 * k + 1] = bfhi(u[k]);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float hot = 0.f;
+#pragma unroll
+      for (int k = 0; k < LOSS_KMAX; ++k) hot += (i + e == tk[k]) ? wk[k] : 0.f;
+      if (cap > 0.f) {
+        const float t = tanh_fast(v[e] * icap);
+        d[e] = gr * (W * fexp(cap * t - l) - keep * hot - flat) * (1.0f - t * t);
+      } else {
+        d[e] = gr * (W * fexp(v[e] - l) - keep * hot - flat);
+      }
+    }
+    u32x4 o = {pack2bf(d[0], d[1]), pack2bf(d[2], d[3]), pack2bf(d[4], d[5]), pack2bf(d[6], d[7])};
+    *(u32x4*)(dr + i) = o;
+  }
+}
+
 // ------------------------------------------------------------------------------------ LM head GEMM + lse partials
 struct EpiLmHead {
   static constexpr bool kTileEpilogue = true;
@@ -259,6 +390,40 @@ extern "C" int tfb_loss_bwd(const void* logits, const void* targets, int idx64, 
   else
     hipLaunchKernelGGL(loss_bwd_kernel<int>, dim3((unsigned)rows), dim3(256), 0, s, (const bf16_t*)logits, (const int*)targets,
                        (const float*)lse, (const float*)grow, (bf16_t*)dlogits, V, softcap);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// Several targets per row and / or label smoothing: targets [K][rows], row_w fp32 [K][rows], 1 <= K <= 8, 0 <= eps < 1.
+extern "C" int tfb_loss_multi_fwd(const void* logits, const void* targets, int idx64, const void* row_w, int K, float eps,
+                                  void* loss, void* lse, long rows, int V, float softcap, void* stream) {
+  if (!logits || !targets || !row_w || !loss || !lse) return TFB_ERR_ARG;
+  if (rows <= 0 || V <= 0 || V % 8 || K < 1 || K > LOSS_KMAX || !(eps >= 0.f && eps < 1.f)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  if (idx64)
+    hipLaunchKernelGGL(loss_multi_fwd_kernel<long>, dim3((unsigned)rows), dim3(256), 0, s, (const bf16_t*)logits,
+                       (const long*)targets, (const float*)row_w, K, rows, (float*)loss, (float*)lse, V, softcap, eps);
+  else
+    hipLaunchKernelGGL(loss_multi_fwd_kernel<int>, dim3((unsigned)rows), dim3(256), 0, s, (const bf16_t*)logits,
+                       (const int*)targets, (const float*)row_w, K, rows, (float*)loss, (float*)lse, V, softcap, eps);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// g fp32 [rows] = upstream gradient of each row's loss (the weights are applied here). dlogits may alias logits.
+extern "C" int tfb_loss_multi_bwd(const void* logits, const void* targets, int idx64, const void* row_w, int K, float eps,
+                                  const void* lse, const void* g, void* dlogits, long rows, int V, float softcap, void* stream) {
+  if (!logits || !targets || !row_w || !lse || !g || !dlogits) return TFB_ERR_ARG;
+  if (rows <= 0 || V <= 0 || V % 8 || K < 1 || K > LOSS_KMAX || !(eps >= 0.f && eps < 1.f)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  if (idx64)
+    hipLaunchKernelGGL(loss_multi_bwd_kernel<long>, dim3((unsigned)rows), dim3(256), 0, s, (const bf16_t*)logits,
+                       (const long*)targets, (const float*)row_w, K, rows, (const float*)lse, (const float*)g,
+                       (bf16_t*)dlogits, V, softcap, eps);
+  else
+    hipLaunchKernelGGL(loss_multi_bwd_kernel<int>, dim3((unsigned)rows), dim3(256), 0, s, (const bf16_t*)logits,
+                       (const int*)targets, (const float*)row_w, K, rows, (const float*)lse, (const float*)g,
+                       (bf16_t*)dlogits, V, softcap, eps);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

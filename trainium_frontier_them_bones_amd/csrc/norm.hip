@@ -199,7 +199,7 @@ __global__ __launch_bounds__(256) void block_head_fwd_kernel(const bf16_t* __res
 #pragma unroll
       for (int i = 0; i < NCH; ++i)
 #pragma unroll
-        for (int k = 0; k < 8; ++k) a.v[i][k] = round_bf(l1 * a.v[i][k] + l2 * b.v[i][k] + l3 * c.v[i][k]);
+        for (int k = 0; k < 8; ++k) a.v[i][k] = round_bf(l1 * (a.v[i][k] + l3 * c.v[i][k]) + l2 * b.v[i][k]);
     } else {
 #pragma unroll
       for (int i = 0; i < NCH; ++i)
@@ -218,8 +218,8 @@ __global__ __launch_bounds__(256) void block_head_fwd_kernel(const bf16_t* __res
   }
 }
 
-// G = g_new + inv * (g_norm - x_new * (g_norm . x_new) * inv^2 / C);
-// dx = l1 G, dx0 = l2 G, dskip = l3 G; gain partials [gridDim.x][4] = sum G.x, G.x0, G.skip, 0
+// x_new = l1 (x + l3 skip) + l2 x0. G = g_new + inv * (g_norm - x_new * (g_norm . x_new) * inv^2 / C);
+// dx = l1 G, dx0 = l2 G, dskip = l1 l3 G; gain partials [gridDim.x][4] = sum G.(x + l3 skip), G.x0, l1 G.skip, 0
 template <int NCH>
 __global__ __launch_bounds__(256) void block_head_bwd_kernel(const bf16_t* __restrict__ g_new,
                                                             const bf16_t* __restrict__ g_norm,
@@ -255,6 +255,13 @@ __global__ __launch_bounds__(256) void block_head_bwd_kernel(const bf16_t* __res
     // g is G (fp32)
     t.load(x + row * C, C, lane);
     s1 += row_dot(g, t);
+    if (skip) {
+      Row<NCH> sk;
+      sk.load(skip + row * C, C, lane);
+      const float gs = row_dot(g, sk);
+      s1 += l3 * gs;
+      s3 += l1 * gs;
+    }
 #pragma unroll
     for (int i = 0; i < NCH; ++i)
 #pragma unroll
@@ -268,12 +275,11 @@ __global__ __launch_bounds__(256) void block_head_bwd_kernel(const bf16_t* __res
       for (int k = 0; k < 8; ++k) t.v[i][k] = l2 * g.v[i][k];
     t.store(dx0 + row * C, C, lane);
     if (skip) {
-      t.load(skip + row * C, C, lane);
-      s3 += row_dot(g, t);
+      const float l13 = l1 * l3;
 #pragma unroll
       for (int i = 0; i < NCH; ++i)
 #pragma unroll
-        for (int k = 0; k < 8; ++k) t.v[i][k] = l3 * g.v[i][k];
+        for (int k = 0; k < 8; ++k) t.v[i][k] = l13 * g.v[i][k];
       t.store(dskip + row * C, C, lane);
     }
   }
@@ -363,7 +369,7 @@ extern "C" int tfb_block_head_fwd(const void* x, const void* x0, const void* ski
   return TFB_OK;
 }
 
-// gain_part: fp32 [tfb_norm_bwd_blocks(nrows)][4] scratch; dgains: fp32 [4] (sum G.x, G.x0, G.skip, 0)
+// gain_part: fp32 [tfb_norm_bwd_blocks(nrows)][4] scratch; dgains: fp32 [4] (sum G.(x + l3 skip), G.x0, l1 G.skip, 0)
 extern "C" int tfb_block_head_bwd(const void* g_new, const void* g_norm, const void* x, const void* x0, const void* skip,
                                   const void* x_new, const void* inv, const void* gains, void* dx, void* dx0,
                                   void* dskip, void* gain_part, void* dgains, long nrows, int C, void* stream) {

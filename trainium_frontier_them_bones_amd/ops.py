@@ -428,6 +428,39 @@ def rope_(x, cos, sin, T, nheads, D, inverse=False, out=None):
     return x if out is None else out
 
 
+def _rows2d(x):
+    if not x.is_cuda or x.dtype != bf16 or x.stride(-1) != 1:
+        raise TypeError("expected a bf16 device tensor with contiguous rows")
+    return x.reshape(-1, x.shape[-1]) if x.is_contiguous() else x
+
+
+def rope_norm_fwd(x, cos, sin, T, nheads, D, eps=2.0 ** -23, want_r=True):
+    """RoPE then parameter-free RMSNorm of each of the first `nheads` heads (D columns each) of every row of x
+    ([rows, row_stride] view). Returns (y [rows, nheads*D] normalised, r [rows, nheads*D] rotated or None,
+    inv [rows, nheads] fp32)."""
+    _chk(cos), _chk(sin)
+    x2 = _rows2d(x)
+    rows = x2.shape[0]
+    y = torch.empty(rows, nheads * D, dtype=bf16, device=x.device)
+    r = torch.empty(rows, nheads * D, dtype=bf16, device=x.device) if want_r else None
+    inv = torch.empty(rows, nheads, dtype=torch.float32, device=x.device)
+    _lib.call("tfb_rope_norm_fwd", _p(x2), _p(cos), _p(sin), _p(r), _p(y), _p(inv), rows, T, nheads, D, x2.stride(0),
+              nheads * D, nheads * D, float(eps), _stream())
+    return y, r, inv
+
+
+def rope_norm_bwd(g, r, inv, cos, sin, T, nheads, D, out=None):
+    """The gradient of rope_norm_fwd's input from g (gradient of y; [rows, row_stride] view), the saved r and inv; written
+    into `out` ([rows, row_stride] view) or a fresh [rows, nheads*D] tensor."""
+    _chk(cos), _chk(sin), _chk(r), _chk(inv, torch.float32)
+    g2 = _rows2d(g)
+    rows = g2.shape[0]
+    o = torch.empty(rows, nheads * D, dtype=bf16, device=g.device) if out is None else _rows2d(out)
+    _lib.call("tfb_rope_norm_bwd", _p(g2), _p(r), _p(inv), _p(cos), _p(sin), _p(o), rows, T, nheads, D, g2.stride(0),
+              r.stride(0), o.stride(0), _stream())
+    return o if out is None else out
+
+
 def resmix_bwd(g, x, x0, ab):
     """dx = g*a, dx0 = g*b, dab = (sum g*x, sum g*x0) for x_new = a*x + b*x0; ab: fp32 device [2]."""
     _chk(g), _chk(x), _chk(x0), _chk(ab, torch.float32)
@@ -505,6 +538,34 @@ def loss_bwd(logits2, targets, lse, grow, softcap=15.0, inplace=False):
     out = logits2 if inplace else torch.empty_like(logits2)
     _lib.call("tfb_loss_bwd", _p(logits2), _p(tg), int(tg.dtype == torch.int64), _p(lse), _p(grow), _p(out), N, V,
               float(softcap or 0.0), _stream())
+    return out
+
+
+def loss_multi_fwd(logits2, targets, row_w, softcap=15.0, eps=0.0):
+    """Row losses sum_k row_w[k] (lse - (1 - eps) s_{t_k} - eps mean_v s_v) and lse; targets [K, N] (int64 / int32, < 0 =
+    weight 0), row_w fp32 [K, N]."""
+    _chk(logits2), _chk(row_w, torch.float32)
+    tg = _tg(targets)
+    K, N = tg.shape
+    V = logits2.shape[1]
+    if tuple(row_w.shape) != (K, N) or logits2.shape[0] != N:
+        raise ValueError("targets [K, N], row_w [K, N], logits [N, V]")
+    loss = torch.empty(N, dtype=torch.float32, device=logits2.device)
+    lse = torch.empty(N, dtype=torch.float32, device=logits2.device)
+    _lib.call("tfb_loss_multi_fwd", _p(logits2), _p(tg), int(tg.dtype == torch.int64), _p(row_w), K, float(eps), _p(loss),
+              _p(lse), N, V, float(softcap or 0.0), _stream())
+    return loss, lse
+
+
+def loss_multi_bwd(logits2, targets, row_w, lse, g, softcap=15.0, eps=0.0, inplace=False):
+    """dlogits bf16 [N, V] of loss_multi_fwd; g fp32 [N] = d(total)/d(row loss)."""
+    _chk(logits2), _chk(row_w, torch.float32), _chk(lse, torch.float32), _chk(g, torch.float32)
+    tg = _tg(targets)
+    K, N = tg.shape
+    V = logits2.shape[1]
+    out = logits2 if inplace else torch.empty_like(logits2)
+    _lib.call("tfb_loss_multi_bwd", _p(logits2), _p(tg), int(tg.dtype == torch.int64), _p(row_w), K, float(eps), _p(lse),
+              _p(g), _p(out), N, V, float(softcap or 0.0), _stream())
     return out
 
 

@@ -1,0 +1,289 @@
+"""The reference training loop's call signatures on the HIP kernels.
+
+Every function here has the name, argument order, argument meaning and result layout of the wrapper the reference's
+`train.py` calls (round1/source/train.py, cited as R1; round2/source/train.py, R2), so a call site switches over by
+changing its import. Differences that a caller can see, all of them in the error behaviour:
+  * there is no eager fallback: on a CPU tensor, a dtype other than bf16 or a shape the kernels do not take the call
+    raises (`TypeError` / `_lib.TfbError`), which is R2's policy (R2:6947 "a shape the kernels do not take ... raises");
+  * the three wrappers whose contract is "None = not done, run your own line" (`nki_rope_attention` R1:8197,
+    `fused_loss_multi` R1:4908, `dw_matmul` R1:3486) return None exactly when the library answers "shape not taken".
+Inputs are never modified; outputs are fresh tensors, except `inplace=True` weight gradients, which are accumulated into
+`w.grad` (R1:8463-8472) and answered with a None gradient.
+"""
+import math
+
+import torch
+
+from . import autograd as A
+from . import ops
+from ._lib import TfbError
+
+bf16 = torch.bfloat16
+LOGIT_SOFTCAP = 15.0          # R1:81
+RMS_EPS = 2.0 ** -23          # R1:5153, 4172
+_SHAPE = 1                    # the library's "shape not taken" status
+
+
+def _none_if_shape(fn, *args):
+    try:
+        return fn(*args)
+    except TfbError as err:
+        if err.status == _SHAPE:
+            return None
+        raise
+
+
+# ------------------------------------------------------------------------------------------ attention (R1:8069-8210)
+def nki_causal_attention(q, k, v, scale=None):
+    """Causal SDPA(q, k, v) for [B, H, T, D] inputs, returned as [B, T, H, D] (R1:8069)."""
+    sc = float(scale) if scale is not None else 1.0 / math.sqrt(q.shape[-1])
+    return A.CausalAttentionFn.apply(q, k, v, sc)
+
+
+nki_attn_fn = nki_causal_attention   # R1:8207
+
+
+def rope_norm(x, cos, sin):
+    """norm(apply_rotary_emb(x, cos, sin)).transpose(1, 2): x [B, T, H, D] -> [B, H, T, D] (R1:4447). cos, sin hold
+    T x D/2 values (any leading singleton shape, as the reference's [1, T, 1, D/2] buffers)."""
+    B, T, H, D = x.shape
+    c, s = _tables_2d(cos, sin, T, D // 2)
+    return A.RopeNormFn.apply(x, c, s, RMS_EPS).transpose(1, 2)
+
+
+def _tables_2d(cos, sin, T, half):
+    c = cos.reshape(-1, half)[:T].to(bf16).contiguous()
+    s = sin.reshape(-1, half)[:T].to(bf16).contiguous()
+    if c.shape[0] != T:
+        raise ValueError("rotary tables shorter than the sequence")
+    return c, s
+
+
+def nki_rope_attention(qkv, cos, sin, n_head, scale=None):
+    """y [B, T, H, D] = causal SDPA(QKnorm(RoPE(q)), QKnorm(RoPE(k)), v) straight from the fused projection output qkv
+    [B, T, 3C]; None when the fused path does not apply (R1:8197)."""
+    if qkv.dim() != 3 or qkv.shape[-1] % (3 * n_head):
+        return None
+    B, T, C3 = qkv.shape
+    D = C3 // 3 // n_head
+    if D not in (64, 128):
+        return None
+    sc = float(scale) if scale is not None else 1.0 / math.sqrt(D)
+    c, s = _tables_2d(cos, sin, T, D // 2)
+    y = _none_if_shape(A.RopeNormAttentionFn.apply, qkv, c, s, n_head, sc, RMS_EPS)
+    return None if y is None else y.view(B, T, n_head, D)
+
+
+# ------------------------------------------------------------------------------------------ loss head (R1:4691, 4908; R2:6364)
+def fused_loss(logits, targets, reduction="mean", softcap=LOGIT_SOFTCAP):
+    """The static cross-entropy chain on the raw lm_head output (R1:4691): softcap * tanh(logits / softcap), log-softmax,
+    ignore_index -1; reduction "mean" (over the targets not ignored), "sum" or "none" (rows in targets' shape)."""
+    V = logits.shape[-1]
+    x2 = logits.reshape(-1, V).contiguous()
+    t = targets.reshape(-1)
+    rows = A.FusedLossFn.apply(x2, t, softcap)
+    if reduction == "none":
+        return rows.view(targets.shape)
+    if reduction == "sum":
+        return rows.sum()
+    if reduction != "mean":
+        raise ValueError("reduction must be 'mean', 'sum' or 'none'")
+    return rows.sum() / (t >= 0).sum().clamp_min(1).to(rows.dtype)
+
+
+def fused_loss_multi(logits, tg, rw, softcap=LOGIT_SOFTCAP, ref=None):
+    """0-dim fp32 sum_i sum_k rw[k, i] nll(logits_i, tg[k, i]) through one kernel pair, or None when the kernels do not
+    take the call (R1:4908). tg [K, N] integer targets, rw [K, N] weights; `ref` (the reference's self-check input) is
+    accepted and unused."""
+    V = logits.shape[-1]
+    K, N = tg.shape
+    if logits.numel() != N * V or not (1 <= K <= 8):
+        return None
+    rows = _none_if_shape(A.FusedLossMultiFn.apply, logits.reshape(N, V).contiguous(), tg.contiguous(),
+                          rw.float().contiguous(), softcap, 0.0)
+    return None if rows is None else rows.sum()
+
+
+def chunked_loss_mean(logits, targets, smooth=False, tok_w=None, eps=0.0):
+    """F.cross_entropy(softcap * tanh(logits.float() / softcap), targets, ignore_index=-1, reduction="mean") through the
+    kernels (R2:6364): the mean and the ignored targets are row weights, `tok_w` (per-target weights) multiplies them,
+    `smooth` selects the label-smoothed pair with the reference's R2_LABEL_SMOOTH passed here as `eps`."""
+    b, t, v = logits.shape
+    n = b * t
+    y = targets.reshape(n)
+    valid = y >= 0
+    w = valid.to(torch.float32) / valid.sum().clamp_min(1).to(torch.float32)
+    if tok_w is not None:
+        w = w * tok_w.reshape(n).to(torch.float32)
+    x2 = logits.reshape(n, v).contiguous()
+    rows = A.FusedLossMultiFn.apply(x2, y.view(1, n).contiguous(), w.view(1, n).contiguous(), LOGIT_SOFTCAP,
+                                    float(eps) if smooth else 0.0)
+    return rows.sum()
+
+
+# ------------------------------------------------------------------------------------------ norm / residual blocks (R1:5578-6834)
+def _gain(l, like):
+    return l if torch.is_tensor(l) else torch.tensor([float(l)], dtype=torch.float32, device=like.device)
+
+
+def block_head(x, x0, l1, l2):
+    """(l1*x + l2*x0, norm(l1*x + l2*x0)) (R1:5578); l1, l2 one-element tensors (the model's learnable gains)."""
+    C = x.shape[-1]
+    x_new, x_norm = A.BlockHeadFn.apply(x.reshape(-1, C), x0.reshape(-1, C), _gain(l1, x), _gain(l2, x), None, None, RMS_EPS)
+    return x_new.view(x.shape), x_norm.view(x.shape)
+
+
+def head_skip(x, x0, skip, l1, l2, l3):
+    """Block head with the U-net skip folded in: head(x + l3*skip, x0) = (l1*(x + l3*skip) + l2*x0, its norm) (R1:6106,
+    eager form 5644-5647). skip None = the plain block head."""
+    if skip is None:
+        return block_head(x, x0, l1, l2)
+    C = x.shape[-1]
+    x_new, x_norm = A.BlockHeadFn.apply(x.reshape(-1, C), x0.reshape(-1, C), _gain(l1, x), _gain(l2, x),
+                                        skip.reshape(-1, C), _gain(l3, x), RMS_EPS)
+    return x_new.view(x.shape), x_norm.view(x.shape)
+
+
+def rmsnorm_fast(x):
+    """F.rms_norm(x, (C,)) (R1:5594)."""
+    C = x.shape[-1]
+    return A.RMSNormFn.apply(x.reshape(-1, C), None, RMS_EPS).view(x.shape)
+
+
+def tail_norm2(x_new, attn_out):
+    """(x_new + attn_out, norm(x_new + attn_out)) (R1:6117)."""
+    C = x_new.shape[-1]
+    s1, y = A.AddRMSNormFn.apply(x_new.reshape(-1, C), attn_out.reshape(-1, C), None, RMS_EPS)
+    return s1.view(x_new.shape), y.view(x_new.shape)
+
+
+def final_norm(s1, mo):
+    """norm(s1 + mo): the last block's residual add and the final RMSNorm (R1:6826)."""
+    C = s1.shape[-1]
+    _, y = A.AddRMSNormFn.apply(s1.reshape(-1, C), mo.reshape(-1, C), None, RMS_EPS)
+    return y.view(s1.shape)
+
+
+def relu_squared(x):
+    """relu(x)**2 (R1:4161)."""
+    return A.Relu2Fn.apply(x)
+
+
+# ------------------------------------------------------------------------------------------ GEMM glue (R1:1137, 1231, 8407)
+def nki_matmul(a, b, trans_a=False, trans_b=False):
+    """out = op(a) @ op(b), fp32 accumulation, one rounding (R1:1137). No autograd, as in the reference (its callers are
+    autograd Functions)."""
+    return ops.matmul(a.contiguous(), b.contiguous(), trans_a=trans_a, trans_b=trans_b)
+
+
+class _LinearTFn(torch.autograd.Function):
+    """y = x @ w with w [in, out] (the reference's LinearT layout, R1:8419-8711)."""
+
+    @staticmethod
+    def forward(ctx, x2, w, inplace):
+        ctx.save_for_backward(x2, w)
+        ctx.inplace = inplace
+        return ops.matmul(x2, w)
+
+    @staticmethod
+    def backward(ctx, gy):
+        x2, w = ctx.saved_tensors
+        g2 = gy.contiguous()
+        dx = ops.matmul(g2, w, trans_b=True)
+        if ctx.inplace and w.grad is not None and w.grad.dtype in (bf16, torch.float32) and w.grad.is_contiguous():
+            ops.matmul(x2, g2, trans_a=True, out=w.grad, accumulate=True)     # R1:8463-8472: summed in the GEMM's output stage
+            return dx, None, None
+        return dx, ops.matmul(x2, g2, trans_a=True), None
+
+
+def fused_fc_relu2(x, w, inplace=False):
+    """relu(x @ w)^2 for any leading shape, w [in, out]; with inplace=True the c_fc dW goes straight into w.grad when it
+    exists (R1:1231)."""
+    K = x.shape[-1]
+    h = A.Relu2Fn.apply(_LinearTFn.apply(x.reshape(-1, K).contiguous(), w, inplace))
+    return h.view(*x.shape[:-1], w.shape[1])
+
+
+def dw_matmul(a2d, b2d, row=None, key=None):
+    """a2d^T @ b2d [Ka, N] from two token-major matrices, or None when the kernels do not take the shape (R1:3486: the
+    weight-gradient GEMM; `row` and `key` select the reference's fp8 scale row and plan cache and are unused here)."""
+    return _none_if_shape(lambda: ops.matmul(a2d.contiguous(), b2d.contiguous(), trans_a=True))
+
+
+def embedding_fwd(idx, weight, out_dtype, shadow=None):
+    """wte(idx).to(out_dtype) with the kernels' backward (R1:8407). `shadow` (the table already in out_dtype) is used for
+    the forward gather when given."""
+    if out_dtype != bf16:
+        raise TypeError("the embedding kernels produce bf16")
+    if shadow is not None:
+        return _EmbeddingShadowFn.apply(idx, weight, shadow)
+    return A.EmbeddingFn.apply(idx, weight if weight.dtype == bf16 else weight.to(bf16))
+
+
+class _EmbeddingShadowFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, idx, weight, shadow):
+        ctx.save_for_backward(idx, weight)
+        return ops.embedding_fwd(idx, shadow)
+
+    @staticmethod
+    def backward(ctx, gy):
+        idx, weight = ctx.saved_tensors
+        dw = ops.fill_f32_(torch.empty(weight.shape, dtype=torch.float32, device=weight.device), 0.0)
+        ops.embedding_bwd(idx, gy.contiguous(), dw)
+        return None, dw.to(weight.dtype), None
+
+
+# ------------------------------------------------------------------------------------------ fp8 fused MLP (R2:6617, 6947)
+def fp8_refresh_weights(mlps, e4m3_limit=240.0, x_scale=4.0, dw_fp8=False):
+    """Once per optimizer step: every MLP's scale row and e4m3 weight bytes (R2:6617 fp8_refresh_weights; the reference
+    keeps them on the module as mlp8_sc / mlp8_w8, here as mlp.tfb_mlp8)."""
+    for mlp in mlps:
+        st = getattr(mlp, "tfb_mlp8", None)
+        if st is None:
+            st = mlp.tfb_mlp8 = A.Mlp8State(e4m3_limit, x_scale, dw_fp8)
+        st.refresh(mlp.c_fc.weight.detach().to(bf16), mlp.c_proj.weight.detach().to(bf16))
+
+
+def mlp_fused8(mlp, x):
+    """MLP.forward on [b, t, n_embd] with the four activation GEMMs in fp8 (R2:6947): c_proj(relu(c_fc(x))^2), weights
+    mlp.c_fc.weight [F, d] and mlp.c_proj.weight [d, F]; rows are padded with zeros to a multiple of 128 (a zero row
+    touches no other row). The scale row and weight bytes come from fp8_refresh_weights (made here on first use)."""
+    if getattr(mlp, "tfb_mlp8", None) is None or mlp.tfb_mlp8.row is None:
+        fp8_refresh_weights([mlp])
+    b, t, c = x.shape
+    x2 = x.reshape(b * t, c)
+    m = x2.shape[0]
+    pad = (-m) % 128
+    if pad:
+        x2 = torch.nn.functional.pad(x2, (0, 0, 0, pad))
+    w_fc = mlp.c_fc.weight if mlp.c_fc.weight.dtype == bf16 else mlp.c_fc.weight.to(bf16)
+    w_proj = mlp.c_proj.weight if mlp.c_proj.weight.dtype == bf16 else mlp.c_proj.weight.to(bf16)
+    y = A.Mlp8Fn.apply(x2, w_fc, w_proj, mlp.tfb_mlp8)
+    if pad:
+        y = y[:m]
+    return y.reshape(b, t, c)
+
+
+def forward_scales(w_fc, w_proj):
+    """The forward's 16-column scale row from the two weights (K/nki_mlp_fused8.py:782)."""
+    return ops.mlp8_forward_scales(w_fc, w_proj)
+
+
+def backward_scales(dy2, row):
+    """The backward call's row: the forward row with this call's gradient scales filled in (K/nki_mlp_fused8.py:803)."""
+    return ops.mlp8_backward_scales(dy2, row)
+
+
+def dw8_grad(g2, a2, s_g, i_g, s_a, i_a, fg, fa):
+    """One weight gradient g2^T a2 [O, D] in fp8 (R2:8185): the g side cast at s_g into format fg, the a side at s_a into
+    fa (0 = e4m3, 1 = e5m2, 2 = e4m3 with g * s_g clamped at 240 first), the descale i_g * i_a. The scales are
+    one-element fp32 device tensors and powers of two; i_g, i_a are their exact inverses, which the kernel forms itself.
+    One side must be e5m2 and the other e4m3 (the two pairings the reference registers, R2:8156)."""
+    f8 = {0: ops.FMT_E4M3, 1: ops.FMT_E5M2, 2: ops.FMT_E4M3}
+    sg, sa = s_g.reshape(1).float(), s_a.reshape(1).float()
+    if fg == 2:   # clamp(g s_g, 240) = s_g clamp(g, 240 / s_g): exact, s_g is a power of two
+        g2 = torch.minimum(g2, (240.0 / sg).to(g2.dtype))
+    g8 = ops.quant_fp8(g2.contiguous(), sg, f8[fg])
+    a8 = ops.quant_fp8(a2.contiguous(), sa, f8[fa])
+    return ops.gemm_fp8_tn(g8, a8, f8[fg], f8[fa], sg, sa)
