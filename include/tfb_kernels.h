@@ -45,7 +45,15 @@ int tfb_rmsnorm_fwd(const void* x, const void* res, const void* w, void* s_out, 
 int tfb_rmsnorm_bwd(const void* gy, const void* gs, const void* s, const void* w, const void* inv, void* dx, void* dw_part,
                     void* dw, int dw_accumulate, long nrows, int C, void* stream);
 
-/* x_new = bf16(l1 x + l2 x0 [+ l3 skip]); x_norm = RMSNorm(x_new); gains = fp32 [3] device (l1, l2, l3).
+/* tfb_rmsnorm_bwd with dw = NULL leaves the weight gradient as per-workgroup partial sums in dw_part; this call finishes
+ * `count` of them in one launch: dw[i][c] (+)= sum_r dw_part[i][r][c], i < count, r < tfb_norm_bwd_blocks(nrows)
+ * (part_stride, dw_stride: floats between consecutive i). The sums are taken in a fixed order (bit-reproducible).
+ * Has no counterpart in the reference, whose wrappers finish each gain gradient with a torch .sum
+ * (round1/source/train.py:6039); it exists because 25 separate 12-workgroup reductions cost 0.5 ms of the step. */
+int tfb_norm_dw_finish(const void* dw_part, void* dw, int count, long part_stride, long dw_stride, int dw_accumulate,
+                       long nrows, int C, void* stream);
+
+/* x_new = bf16(l1 (x [+ l3 skip]) + l2 x0); x_norm = RMSNorm(x_new); gains = fp32 [3] device (l1, l2, l3).
  * Replaces block_head (round1/source/train.py:5578, kernel 5257) and head_skip (6106, kernel 5743). */
 int tfb_block_head_fwd(const void* x, const void* x0, const void* skip, const void* gains, void* x_new, void* x_norm,
                        void* inv, long nrows, int C, float eps, void* stream);

@@ -74,6 +74,29 @@ def test_rmsnorm_fwd_bwd(ops, dev, C, weighted):
     assert rel_l2(y1, O.rmsnorm(x, w, eps)[0]) < 1e-3
 
 
+def test_norm_weight_gradients_finished_in_one_launch(ops, dev):
+    """rmsnorm_bwd(part=...) + norm_dw_finish equals the per-call weight gradient bit for bit (same partials, same
+    order of summation), also when added into."""
+    g = _g(21)
+    rows, C, n = 2048, 768, 3
+    xs = [torch.randn(rows, C, generator=g).bfloat16().to(dev) for _ in range(n)]
+    gys = [torch.randn(rows, C, generator=g).bfloat16().to(dev) for _ in range(n)]
+    w = (1 + 0.02 * torch.randn(C, generator=g)).bfloat16().to(dev)
+    parts = torch.empty(n, ops.norm_bwd_blocks(rows), C, dtype=torch.float32, device=dev)
+    want, dxs = [], []
+    for i in range(n):
+        _, _, inv = ops.rmsnorm_fwd(xs[i], w, 1e-6)
+        dx, dw = ops.rmsnorm_bwd(gys[i], xs[i], inv, w)
+        dx2, none = ops.rmsnorm_bwd(gys[i], xs[i], inv, w, part=parts[i])
+        assert none is None and torch.equal(dx, dx2)
+        want.append(dw)
+    out = torch.full((n, C), 7.0, dtype=torch.float32, device=dev)
+    ops.norm_dw_finish(parts, out, rows)
+    assert torch.equal(out, torch.stack(want))
+    ops.norm_dw_finish(parts, out, rows, accumulate=True)
+    assert torch.equal(out, 2 * torch.stack(want))
+
+
 def test_block_head(ops, dev):
     from oracle import norm as O
     g = _g(11)

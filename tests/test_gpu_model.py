@@ -15,7 +15,7 @@ def test_small_model_losses_and_gradients_track_oracle(dev):
     o = OracleGPT(cfg, m.init_values)
     idx, tg = zipf_tokens(2, 256, cfg.vocab, seed=3)
     loss = m.forward(idx.to(dev), tg.to(dev))
-    loss.backward()
+    m.backward(loss)
     lo = o.forward(idx, tg)
     lo.backward()
     assert abs(loss.item() - lo.item()) < 1e-3 * lo.item()
@@ -40,9 +40,9 @@ def test_gradient_accumulation_in_place(dev):
     idx, tg = zipf_tokens(4, 128, cfg.vocab, seed=4)
     idx, tg = idx.to(dev), tg.to(dev)
     m.zero_grad()
-    m.forward(idx, tg).backward()
+    m.backward(m.forward(idx, tg))
     once = {k: p.grad_buf.clone() for k, p in m.p.items()}
-    m.forward(idx, tg).backward()                                   # second micro-step adds into the same buffers
+    m.backward(m.forward(idx, tg))                                  # second micro-step adds into the same buffers
     for k, p in m.p.items():
         assert rel_l2(p.grad_buf, 2 * once[k].float()) < 1e-2, k
 

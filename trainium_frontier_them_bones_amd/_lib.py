@@ -21,6 +21,7 @@ SIGNATURES = {
     "tfb_norm_bwd_blocks": [_l],
     "tfb_rmsnorm_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_rmsnorm_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _l, _i, _vp],
+    "tfb_norm_dw_finish": [_vp, _vp, _i, _l, _l, _i, _l, _i, _vp],
     "tfb_block_head_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_block_head_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _vp],
     "tfb_mlp8_scale_scratch_floats": [_i],

@@ -36,6 +36,9 @@ class RMSNormFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, gy):
         x, inv, weight = ctx.saved_tensors
+        part = getattr(weight, "dw_part", None)
+        if part is not None:   # the weight gradient is finished later, with the other norms', by ops.norm_dw_finish
+            return ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, None, part=part)[0], None, None
         buf, acc = (None, False) if weight is None else _accumulate_into(weight)
         dx, dw = ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, None, buf, acc)
         if weight is None or buf is not None:
@@ -56,6 +59,10 @@ class AddRMSNormFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, gs, gy):
         s, inv, weight = ctx.saved_tensors
+        part = getattr(weight, "dw_part", None)
+        if part is not None and gy is not None:
+            dx = ops.rmsnorm_bwd(gy.contiguous(), s, inv, weight, None if gs is None else gs.contiguous(), part=part)[0]
+            return dx, dx, None, None
         buf, acc = (None, False) if weight is None else _accumulate_into(weight)
         if gy is None:
             return gs, gs, None, None

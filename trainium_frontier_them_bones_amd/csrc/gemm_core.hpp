@@ -65,7 +65,7 @@ typedef __attribute__((address_space(3))) tfb_s16x4 tfb_lds_s16x4_t;
 template <int BP_, int BQ_, int WP_, int WQ_, int ES_, int LAYP_, int LAYQ_, int FMTP_ = 0, int FMTQ_ = 0, int OCC_ = 0,
           int NSTAGE_ = 2>
 struct GemmCfg {
-  static constexpr int NSTAGE = NSTAGE_;  // LDS stages: 2 (one k-tile of loads in flight) or 3 (two in flight)
+  static constexpr int NSTAGE = NSTAGE_;  // LDS stages: 2 (one k-tile of loads in flight)
   static constexpr int BP = BP_, BQ = BQ_, WP = WP_, WQ = WQ_, ES = ES_;
   static constexpr int LAYP = LAYP_, LAYQ = LAYQ_, FMTP = FMTP_, FMTQ = FMTQ_;
   static constexpr int NW = WP * WQ, NT = NW * 64;
@@ -73,7 +73,7 @@ struct GemmCfg {
   static constexpr int BK = 128 / ES;                  // elements of k per tile
   static constexpr int STAGE_BYTES = (BP + BQ) * 128;  // one k-tile of both operands
   // epilogue staging: a wavefront's slice is 32 rows x (ETP * 32) floats (+ 4 of pad); ETP of the TP tiles per pass
-  static constexpr int EPI_LIMIT = NSTAGE_ == 3 ? STAGE_BYTES : 72 * 1024;
+  static constexpr int EPI_LIMIT = 72 * 1024;
   static constexpr int ETP = (TP >= 2 && NW * 32 * (TP * 32 + 4) * 4 > EPI_LIMIT) ? TP / 2 : TP;
   static constexpr int STAGE_LD = ETP * 32 + 4;
   static constexpr int EPI_BYTES = NW * 32 * STAGE_LD * 4;
@@ -87,7 +87,7 @@ struct GemmCfg {
   static_assert(LAYP == TFB_K_CONTIG || BP == 128 || BP == 256, "K_STRIDED tiles are 128 or 256 rows");
   static_assert(LAYQ == TFB_K_CONTIG || BQ == 128 || BQ == 256, "K_STRIDED tiles are 128 or 256 rows");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS");
-  static_assert(NSTAGE == 2 || NSTAGE == 3, "stages");
+  static_assert(NSTAGE == 2, "two LDS stages (a three-stage loop was measured no faster and removed)");
 };
 
 // ---- global -> LDS (one operand tile, this wavefront's share) ---------------------------------------------------
@@ -281,7 +281,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   constexpr int BP = Cfg::BP, BQ = Cfg::BQ, NW = Cfg::NW, TP = Cfg::TP, TQ = Cfg::TQ, ES = Cfg::ES;
   __shared__ __attribute__((aligned(1024))) uint8_t buf0[Cfg::BUF0_BYTES];
   __shared__ __attribute__((aligned(1024))) uint8_t buf1[Cfg::STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t buf2[Cfg::NSTAGE == 3 ? Cfg::STAGE_BYTES : 16];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int wp = wave % Cfg::WP, wq = wave / Cfg::WP;
@@ -408,7 +407,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
     }
   };
 
-  if constexpr (Cfg::NSTAGE == 2) {
+  {
     if (nkt > 0) issue(buf0, 0);
     __syncthreads();
     for (int t = 0; t + 2 <= nkt; t += 2) {
@@ -421,34 +420,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
     }
     if (nkt & 1) compute(buf0);
     __syncthreads();
-  } else {
-    // Three stages, two k-tiles of loads in flight. Each step: wait until all but this wavefront's newest tile load
-    // have landed, barrier (every wavefront's share of tile t is in LDS, and everyone is done reading the stage that
-    // is refilled next), start the load of tile t + 2, multiply tile t. The barrier is the bare instruction: a
-    // __syncthreads() fence would wait for the loads still in flight.
-    constexpr int NI = TileDma<BP, NW, Cfg::LAYP, ES>::NI + TileDma<BQ, NW, Cfg::LAYQ, ES>::NI;  // load instructions per tile
-    constexpr int WAIT_OLDER = (NI & 15) | (7 << 4) | (0 << 8) | ((NI >> 4) << 14);      // vmcnt(NI) lgkmcnt(0)
-    auto step = [&](const uint8_t* cur, uint8_t* refill, int t) {
-      __builtin_amdgcn_s_waitcnt(WAIT_OLDER);
-      __atomic_signal_fence(__ATOMIC_SEQ_CST);
-      __builtin_amdgcn_s_barrier();
-      __atomic_signal_fence(__ATOMIC_SEQ_CST);
-      issue(refill, t + 2 < nkt ? t + 2 : nkt - 1);  // past the end: re-fetch the last tile, keeps the count uniform
-      compute(cur);
-    };
-    if (nkt > 0) {
-      issue(buf0, 0);
-      issue(buf1, nkt > 1 ? 1 : 0);
-      const int n3 = nkt / 3 * 3;
-      for (int t = 0; t < n3; t += 3) {
-        step(buf0, buf2, t);
-        step(buf1, buf0, t + 1);
-        step(buf2, buf1, t + 2);
-      }
-      if (nkt - n3 >= 1) step(buf0, buf2, n3);
-      if (nkt - n3 == 2) step(buf1, buf0, n3 + 1);
-    }
-    __syncthreads();  // all loads landed, all fragment reads done: the stages can be reused by the epilogue
   }
 
   const int pw = wp * (TP * 32), qw = wq * (TQ * 32);  // wavefront's origin inside the tile

@@ -162,11 +162,14 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16_t* __restri
 }
 
 // out[c] (+)= sum_r part[r][c]: 64 columns x 16 row lanes per workgroup, rows interleaved over the lanes.
+// blockIdx.y selects one of several independent sums (part + y * part_stride -> out + y * out_stride).
 __global__ __launch_bounds__(1024) void colsum_kernel(const float* __restrict__ part, float* __restrict__ out, int rows, int C,
-                                                     int accumulate) {
+                                                     int accumulate, long part_stride = 0, long out_stride = 0) {
   __shared__ float red[16][64];
   const int tx = threadIdx.x, ty = threadIdx.y;
   const int c = blockIdx.x * 64 + tx;
+  part += (long)blockIdx.y * part_stride;
+  out += (long)blockIdx.y * out_stride;
   float t = 0.f;
   if (c < C)
     for (int r = ty; r < rows; r += 16) t += part[(long)r * C + c];
@@ -335,7 +338,7 @@ extern "C" int tfb_rmsnorm_fwd(const void* x, const void* res, const void* w, vo
 extern "C" int tfb_rmsnorm_bwd(const void* gy, const void* gs, const void* s, const void* w, const void* inv, void* dx,
                                void* dw_part, void* dw, int dw_accumulate, long nrows, int C, void* stream) {
   if (!gy || !s || !inv || !dx) return TFB_ERR_ARG;
-  if (w && (!dw_part || !dw)) return TFB_ERR_ARG;
+  if (w && !dw_part) return TFB_ERR_ARG;
   if (!norm_shape_ok(nrows, C)) return TFB_ERR_SHAPE;
   int grid = grid_for(nrows, 1024);
 #define CALL(N)                                                                                                        \
@@ -345,11 +348,24 @@ extern "C" int tfb_rmsnorm_bwd(const void* gy, const void* gs, const void* s, co
   DISPATCH_NCH(C, CALL);
 #undef CALL
   TFB_LAUNCH_CHECK();
-  if (w) {
+  if (w && dw) {
     hipLaunchKernelGGL(colsum_kernel, dim3((C + 63) / 64), dim3(64, 16), 0, (hipStream_t)stream, (const float*)dw_part,
-                       (float*)dw, grid, C, dw_accumulate);
+                       (float*)dw, grid, C, dw_accumulate, 0L, 0L);
     TFB_LAUNCH_CHECK();
   }
+  return TFB_OK;
+}
+
+// Finish `count` weight gradients at once: dw[i][c] (+)= sum_r part[i][r][c], part = count blocks of
+// tfb_norm_bwd_blocks(nrows) x C floats as left by tfb_rmsnorm_bwd calls made with dw = NULL (part_stride, dw_stride in
+// floats). One launch instead of one 12-workgroup launch per norm.
+extern "C" int tfb_norm_dw_finish(const void* dw_part, void* dw, int count, long part_stride, long dw_stride, int dw_accumulate,
+                                  long nrows, int C, void* stream) {
+  if (!dw_part || !dw) return TFB_ERR_ARG;
+  if (count <= 0 || count > 65535 || !norm_shape_ok(nrows, C) || part_stride < 0 || dw_stride < 0) return TFB_ERR_SHAPE;
+  hipLaunchKernelGGL(colsum_kernel, dim3((C + 63) / 64, count), dim3(64, 16), 0, (hipStream_t)stream, (const float*)dw_part,
+                     (float*)dw, grid_for(nrows, 1024), C, dw_accumulate, part_stride, dw_stride);
+  TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
 

@@ -111,6 +111,14 @@ class GPT:
         self.qkv_state = [A.Linear8State(cfg.e4m3_limit, cfg.fp8_attn_dw) for _ in range(L)] if cfg.fp8_attn_proj else None
         self.wo_state = [A.Linear8State(cfg.e4m3_limit, cfg.fp8_attn_dw) for _ in range(L)] if cfg.fp8_attn_proj else None
         self.cos, self.sin = rope_tables(cfg.seq_len, cfg.head_dim, cfg.rope_base, device)
+        # The 2 L + 1 norm weights sit side by side in the flat fp32 buffer: their gradients are left as per-workgroup
+        # partial sums by every norm backward and finished by ONE launch after the backward pass (norm_rows fixes the
+        # partial buffer's shape on first use).
+        self.norm_names = [n for n in self.others.names if n.startswith("norm")]
+        o0 = self.others.offsets[self.norm_names[0]][0]
+        assert all(self.others.offsets[n] == (o0 + i * d, d) for i, n in enumerate(self.norm_names))
+        self.norm_grads = self.others.grad[o0:o0 + len(self.norm_names) * d].view(len(self.norm_names), d)
+        self.norm_parts, self.norm_rows, self.norm_fresh = None, 0, True
         self.step_count = 0
         self.init_weights(seed)
 
@@ -140,9 +148,24 @@ class GPT:
                 self.qkv_state[i].refresh(self.p["w_qkv.%d" % i])
                 self.wo_state[i].refresh(self.p["w_o.%d" % i])
 
+    def _norm_partials(self, rows):
+        if self.norm_rows != rows:
+            nb = ops.norm_bwd_blocks(rows)
+            self.norm_parts = torch.empty(len(self.norm_names), nb, self.cfg.d_model, dtype=torch.float32, device=self.device)
+            self.norm_rows = rows
+            for i, n in enumerate(self.norm_names):
+                self.p[n].dw_part = self.norm_parts[i]
+
+    def finish_norm_grads(self):
+        """The norm weights' gradients from the partial sums of this backward pass (added to what earlier micro-steps
+        left when the gradients are not fresh)."""
+        ops.norm_dw_finish(self.norm_parts, self.norm_grads, self.norm_rows, accumulate=not self.norm_fresh)
+        self.norm_fresh = False
+
     def forward(self, idx, targets):
         cfg, p = self.cfg, self.p
         B, T = idx.shape
+        self._norm_partials(B * T)
         scale = 1.0 / math.sqrt(cfg.head_dim)
         x = A.EmbeddingFn.apply(idx, p["wte"])
         h = A.RMSNormFn.apply(x, p["norm1.0"], cfg.norm_eps)
@@ -167,6 +190,11 @@ class GPT:
     def zero_grad(self):
         self.mats.mark_fresh()
         self.others.mark_fresh()
+        self.norm_fresh = True
+
+    def backward(self, loss):
+        loss.backward()
+        self.finish_norm_grads()
 
     def optimizer_step(self, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1):
         self.step_count += 1
@@ -178,7 +206,7 @@ class GPT:
     def train_step(self, idx, targets, **opt):
         """One fwd + bwd + AdamW step; returns the loss tensor (no host sync)."""
         loss = self.forward(idx, targets)
-        loss.backward()
+        self.backward(loss)
         self.optimizer_step(**opt)
         return loss
 

@@ -89,15 +89,19 @@ def rmsnorm_fwd(x, weight=None, eps=2.0 ** -23, res=None):
     return s, y, inv
 
 
-def rmsnorm_bwd(gy, s, inv, weight=None, gs=None, dw=None, accumulate=False):
+def rmsnorm_bwd(gy, s, inv, weight=None, gs=None, dw=None, accumulate=False, part=None):
     """dx = gs + J^T(gy) for y = RMSNorm(s) * weight. Returns (dx, dw fp32 [C] or None); a given dw is written, or
-    added into with accumulate=True."""
+    added into with accumulate=True. With `part` (fp32 [tfb_norm_bwd_blocks(rows), C]) the weight gradient is left there
+    as partial sums for norm_dw_finish and None is returned for it."""
     _chk(gy), _chk(s), _chk(weight), _chk(gs), _chk(inv, torch.float32)
     C = s.shape[-1]
     rows = s.numel() // C
     dx = torch.empty_like(s)
-    part = None
     acc = 0
+    if weight is not None and part is not None:
+        _chk(part, torch.float32)
+        _lib.call("tfb_rmsnorm_bwd", _p(gy), _p(gs), _p(s), _p(weight), _p(inv), _p(dx), _p(part), None, 0, rows, C, _stream())
+        return dx, None
     if weight is not None:
         nb = _lib.lib().tfb_norm_bwd_blocks(rows)
         part = torch.empty(nb, C, dtype=torch.float32, device=s.device)
@@ -109,6 +113,21 @@ def rmsnorm_bwd(gy, s, inv, weight=None, gs=None, dw=None, accumulate=False):
     _lib.call("tfb_rmsnorm_bwd", _p(gy), _p(gs), _p(s), _p(weight), _p(inv), _p(dx), _p(part), _p(dw), acc, rows, C,
               _stream())
     return dx, dw
+
+
+def norm_bwd_blocks(rows):
+    return int(_lib.lib().tfb_norm_bwd_blocks(rows))
+
+
+def norm_dw_finish(parts, dw, rows, accumulate=False):
+    """dw [count, C] fp32 (+)= the weight gradients whose partial sums rmsnorm_bwd(part=parts[i]) left in parts
+    [count, blocks, C]: one launch for all of them."""
+    _chk(parts, torch.float32), _chk(dw, torch.float32)
+    count, nb, C = parts.shape
+    if tuple(dw.shape) != (count, C) or nb != norm_bwd_blocks(rows):
+        raise ValueError("parts [count, blocks, C], dw [count, C]")
+    _lib.call("tfb_norm_dw_finish", _p(parts), _p(dw), count, nb * C, C, int(accumulate), rows, C, _stream())
+    return dw
 
 
 def block_head_fwd(x, x0, gains, skip=None, eps=2.0 ** -23):
