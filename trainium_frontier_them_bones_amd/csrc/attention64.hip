@@ -72,6 +72,19 @@ __device__ __forceinline__ void xcd_block(int nx, int nbh, int& bx, int& bh) {
 
 __device__ __forceinline__ int swz(int t) { return (((t >> 1) & 1) << 2) | ((t >> 2) & 3); }
 
+// Of the two workgroups that start together on a CU, the one in an odd wavefront slot (HW_ID.wave_id bit 0) begins
+// ~3.6 us late, once, in the first round: the pair then alternates between its memory-bound and MFMA-bound phases
+// instead of running them in lockstep (measured -0.17 ms per training step over the three kernels).
+#ifndef TFB_ATTN_STAGGER
+#define TFB_ATTN_STAGGER 1
+#endif
+__device__ __forceinline__ void stagger_start() {
+  if (TFB_ATTN_STAGGER > 0 && blockIdx.x + gridDim.x * blockIdx.y < 512) {
+    if (__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 4) & 1)  // getreg(size 4, offset 0, HW_REG_HW_ID)
+      for (int i = 0; i < TFB_ATTN_STAGGER; ++i) __builtin_amdgcn_s_sleep(127);
+  }
+}
+
 // This wavefront's share (NI of the 4 NI instructions) of a (32 NI)-token tile load. `rows` points at token 0 of the
 // tile, `stride` = bytes between tokens.
 template <int NI>
@@ -152,6 +165,7 @@ __global__ __launch_bounds__(256, TFB_FWD64_WPE) void attn64_fwd_kernel(AttnT q,
   __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  stagger_start();
   int bx, bh;
   xcd_block(gridDim.x, gridDim.y, bx, bh);
   const int qb = gridDim.x - 1 - bx;  // longest rows first
@@ -327,6 +341,7 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
   __shared__ __attribute__((aligned(1024))) uint8_t st1[STAGE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  stagger_start();
   int kb, bh;  // low key blocks see the most query tiles: already longest first
   xcd_block(gridDim.x, gridDim.y, kb, bh);
   const int b = bh / H, h = bh % H;
@@ -475,6 +490,7 @@ __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, A
   __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  stagger_start();
   int bx, bh;
   xcd_block(gridDim.x, gridDim.y, bx, bh);
   const int qb = gridDim.x - 1 - bx;

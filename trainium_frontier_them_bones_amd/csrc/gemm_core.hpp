@@ -283,6 +283,21 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   __shared__ __attribute__((aligned(1024))) uint8_t buf1[Cfg::STAGE_BYTES];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  // Two workgroups share a CU. Launched together they run in lockstep: both in the k-loop (each at half the MFMA rate),
+  // then both in the epilogue (MFMA idle, memory busy). The one that landed in an odd wavefront slot (HW_ID.wave_id
+  // bit 0) therefore starts ~7 us late, once, in the first round of workgroups: from then on one's epilogue runs
+  // under the other's MFMAs (measured -0.5 to -1.3 ms per training step; delaying both costs +0.65 ms, none is the
+  // old behaviour). Only where there is a second round to overlap with and no k-split (long k-loops, small epilogues).
+#ifndef TFB_STAGGER_SLEEPS
+#define TFB_STAGGER_SLEEPS 2
+#endif
+#ifndef TFB_STAGGER_SPLITK
+#define TFB_STAGGER_SPLITK 0
+#endif
+  if (Cfg::OCC == 2 && TFB_STAGGER_SLEEPS > 0 && (a.splits == 1 || TFB_STAGGER_SPLITK) && blockIdx.x < 512 && gridDim.x >= 1024) {
+    if (__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 4) & 1)  // getreg(size 4, offset 0, HW_REG_HW_ID): wave_id
+      for (int i = 0; i < TFB_STAGGER_SLEEPS; ++i) __builtin_amdgcn_s_sleep(127);  // 127 x 64 clocks each
+  }
   const int wp = wave % Cfg::WP, wq = wave / Cfg::WP;
   const int lr = lane & 31, lh = lane >> 5;
 
