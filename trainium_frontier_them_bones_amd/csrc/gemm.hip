@@ -32,13 +32,25 @@ struct EpiStoreRope {
   const bf16_t* cs;  // [T][32]
   const bf16_t* sn;
   int T, rot_cols;
-  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const float (&vp)[8], int) const {
+  struct pre_t {  // the chunk's cos / sin values, requested before the k-loop
+    u32x4 c, s;
+  };
+  __device__ __forceinline__ pre_t prefetch(int p, int q) const {
+    pre_t r = {};
+    if (p < rot_cols) {
+      const int t = q % T, idx = p & 31;
+      r.c = *(const u32x4*)(cs + (long)t * 32 + idx);
+      r.s = *(const u32x4*)(sn + (long)t * 32 + idx);
+    }
+    return r;
+  }
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const float (&vp)[8], const pre_t& tab,
+                                             int) const {
     u32x4 x = pack8bf(v);
     if (p < rot_cols) {
       const u32x4 y = pack8bf(vp);
-      const int t = q % T, idx = p & 31;
       const bool low = (p & 32) == 0;
-      const u32x4 c = *(const u32x4*)(cs + (long)t * 32 + idx), s = *(const u32x4*)(sn + (long)t * 32 + idx);
+      const u32x4 c = tab.c, s = tab.s;
       u32x4 o;
 #pragma unroll
       for (int k = 0; k < 4; ++k) {

@@ -274,6 +274,30 @@ struct has_tile_epilogue : std::false_type {};
 template <class T>
 struct has_tile_epilogue<T, std::void_t<decltype(T::kTileEpilogue)>> : std::true_type {};
 
+#ifndef TFB_STAGGER_SLEEPS
+#define TFB_STAGGER_SLEEPS 2
+#endif
+#ifndef TFB_STAGGER_SPLITK
+#define TFB_STAGGER_SPLITK 0
+#endif
+template <class T, class = void>
+struct stagger_sleeps : std::integral_constant<int, TFB_STAGGER_SLEEPS> {};
+template <class T>
+struct stagger_sleeps<T, std::void_t<decltype(T::kStaggerSleeps)>> : std::integral_constant<int, T::kStaggerSleeps> {};
+
+// A staged epilogue that reads an operand of its own (the saved activation of the fp8 MLP's backward) declares
+//   typedef ... pre_t;  pre_t prefetch(int p, int q) const;  void operator()(p, q, v, const pre_t&, split) const;
+// prefetch is called for every 8-element chunk the lane will finish BEFORE the k-loop, so those loads are in flight
+// under the MFMAs instead of being eight dependent load-use chains at the end of the tile.
+template <class T, class = void>
+struct has_prefetch : std::false_type {};
+template <class T>
+struct has_prefetch<T, std::void_t<typename T::pre_t>> : std::true_type {};
+template <class T, bool = has_prefetch<T>::value>
+struct prefetch_type { typedef int type; };
+template <class T>
+struct prefetch_type<T, true> { typedef typename T::pre_t type; };
+
 // Epi: either  __device__ void operator()(int p, int q, const float (&v)[8], int split)  with v = D[p..p+7][q], p % 8 == 0,
 // or (with a static member kTileEpilogue)  __device__ void tile(acc, pw, qw, lr, lh, tile_id, split).
 template <class Cfg, class PreP, class PreQ, class Epi>
@@ -288,15 +312,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   // bit 0) therefore starts ~7 us late, once, in the first round of workgroups: from then on one's epilogue runs
   // under the other's MFMAs (measured -0.5 to -1.3 ms per training step; delaying both costs +0.65 ms, none is the
   // old behaviour). Only where there is a second round to overlap with and no k-split (long k-loops, small epilogues).
-#ifndef TFB_STAGGER_SLEEPS
-#define TFB_STAGGER_SLEEPS 2
-#endif
-#ifndef TFB_STAGGER_SPLITK
-#define TFB_STAGGER_SPLITK 0
-#endif
-  if (Cfg::OCC == 2 && TFB_STAGGER_SLEEPS > 0 && (a.splits == 1 || TFB_STAGGER_SPLITK) && blockIdx.x < 512 && gridDim.x >= 1024) {
+  constexpr int kSleeps = stagger_sleeps<Epi>::value;  // an epilogue may name its own count (static kStaggerSleeps)
+  if (Cfg::OCC == 2 && kSleeps > 0 && (a.splits == 1 || TFB_STAGGER_SPLITK) && blockIdx.x < 512 && gridDim.x >= 1024) {
     if (__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 4) & 1)  // getreg(size 4, offset 0, HW_REG_HW_ID): wave_id
-      for (int i = 0; i < TFB_STAGGER_SLEEPS; ++i) __builtin_amdgcn_s_sleep(127);  // 127 x 64 clocks each
+      for (int i = 0; i < kSleeps; ++i) __builtin_amdgcn_s_sleep(127);  // 127 x 64 clocks each
   }
   const int wp = wave % Cfg::WP, wq = wave / Cfg::WP;
   const int lr = lane & 31, lh = lane >> 5;
@@ -382,6 +401,20 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
+  // the staged epilogue's chunk of pass k, column block j: row and first column inside the wavefront's 32-row slice
+  constexpr bool kPrefetch = has_prefetch<Epi>::value && !has_tile_epilogue<Epi>::value && Cfg::ETP == TP;
+  constexpr int EPI_CPR = Cfg::ETP * 4, EPI_NK = 32 * EPI_CPR / 64;
+  auto chunk_row = [&](int k) { return 2 * (((lane >> 3) + k * 8) / (EPI_CPR / 4)) + ((lane >> 2) & 1); };
+  auto chunk_col = [&](int k) { return (4 * (((lane >> 3) + k * 8) % (EPI_CPR / 4)) + (lane & 3)) * 8; };
+  [[maybe_unused]] typename prefetch_type<Epi>::type pre[TQ][EPI_NK];
+  if constexpr (kPrefetch) {
+#pragma unroll
+    for (int j = 0; j < TQ; ++j)
+#pragma unroll
+      for (int k = 0; k < EPI_NK; ++k)
+        pre[j][k] = epi.prefetch((int)p0 + wp * (TP * 32) + chunk_col(k), (int)q0 + wq * (TQ * 32) + j * 32 + chunk_row(k));
+  }
+
   auto issue = [&](uint8_t* buf, int t) {
     dp.issue(buf, t, wave);
     dq.issue(buf + BP * 128, t, wave);
@@ -447,7 +480,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
     // execute in order) and then finishes them as 8-element chunks, a row's chunks on consecutive lanes.
     constexpr int SLD = Cfg::STAGE_LD, ETP = Cfg::ETP;
     float* stage = (float*)buf0 + wave * (32 * SLD);
-    constexpr int CPR = ETP * 4;  // 8-element chunks per staged row
+    constexpr int CPR = EPI_CPR;  // 8-element chunks per staged row
 #pragma unroll
     for (int j = 0; j < TQ; ++j) {
 #pragma unroll
@@ -464,9 +497,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
 #pragma unroll
         for (int k = 0; k < 32 * CPR / 64; ++k) {
           // 8 consecutive lanes take 4 chunks of each of two rows: their 128-bit reads fall on 8 different bank groups
-          const int rest = (lane >> 3) + k * 8;
-          const int row = 2 * (rest / (CPR / 4)) + ((lane >> 2) & 1);
-          const int pc = (4 * (rest % (CPR / 4)) + (lane & 3)) * 8;
+          const int row = chunk_row(k), pc = chunk_col(k);
           f32x4 lo = *(const f32x4*)(stage + row * SLD + pc);
           f32x4 hi = *(const f32x4*)(stage + row * SLD + pc + 4);
           const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -475,7 +506,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
             f32x4 plo = *(const f32x4*)(stage + row * SLD + (pc ^ 32));
             f32x4 phi = *(const f32x4*)(stage + row * SLD + (pc ^ 32) + 4);
             const float vp[8] = {plo[0], plo[1], plo[2], plo[3], phi[0], phi[1], phi[2], phi[3]};
-            epi((int)p0 + pw + pc, (int)q0 + qw + j * 32 + row, v, vp, split);
+            if constexpr (kPrefetch) epi((int)p0 + pw + pc, (int)q0 + qw + j * 32 + row, v, vp, pre[j][k], split);
+            else epi((int)p0 + pw + pc, (int)q0 + qw + j * 32 + row, v, vp, split);
+          } else if constexpr (kPrefetch) {
+            epi((int)p0 + pw + pc, (int)q0 + qw + j * 32 + row, v, pre[j][k], split);
           } else {
             epi((int)p0 + pw + i0 * 32 + pc, (int)q0 + qw + j * 32 + row, v, split);
           }

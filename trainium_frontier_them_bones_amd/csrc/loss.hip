@@ -435,15 +435,14 @@ extern "C" int tfb_lmhead_fwd(const void* x, const void* W, const void* targets,
   if (!x || !W || !targets || !logits || !part || !loss || !lse) return TFB_ERR_ARG;
   if (rows <= 0 || rows % 128 || V <= 0 || V % 128 || d <= 0 || d % 64) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
-  // 256 vocabulary columns x 256 rows per workgroup of 8 wavefronts when the shape allows it (half the operand bytes
-  // per flop of the 128 x 128 tile: measured ~15 % faster at V = 32768), else 128 x 128; a wavefront spans 64
-  // vocabulary columns in both.
+  // 128 x 128 tiles, two workgroups per CU started half a tile apart (gemm_core.hpp): the epilogue of one (2.1 GB of
+  // logits written, exp / max / sum per element) runs under the other's MFMAs. Measured at V = 32768, 32768 rows:
+  // 2.08 ms, against 2.26 ms for 256 x 256 tiles on 8 wavefronts (half the operand bytes per flop, but one resident
+  // workgroup and nothing to hide its epilogue behind); a wavefront spans 64 vocabulary columns.
   using Cfg = GemmCfg<128, 128, 2, 2, 2, TFB_K_CONTIG, TFB_K_CONTIG>;
-  using CfgWide = GemmCfg<256, 256, 4, 2, 2, TFB_K_CONTIG, TFB_K_CONTIG>;
   GemmOperand P{(const uint8_t*)W, (long)d * 2}, Q{(const uint8_t*)x, (long)d * 2};
   EpiLmHead e{(bf16_t*)logits, (float*)part, (long)V, V / 64, softcap};
-  int st = (rows % 256 == 0 && V % 256 == 0) ? gemm_launch<CfgWide>(P, Q, V, (int)rows, (long)d * 2, 1, LoadIdentity{}, LoadIdentity{}, e, s)
-                           : gemm_launch<Cfg>(P, Q, V, (int)rows, (long)d * 2, 1, LoadIdentity{}, LoadIdentity{}, e, s);
+  int st = gemm_launch<Cfg>(P, Q, V, (int)rows, (long)d * 2, 1, LoadIdentity{}, LoadIdentity{}, e, s);
   if (st != TFB_OK) return st;
   unsigned nb = (unsigned)((rows + 3) / 4);
   if (idx64)

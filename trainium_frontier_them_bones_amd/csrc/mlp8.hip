@@ -372,11 +372,13 @@ struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*
     e.sc = sc + g * NSC;
     return e;
   }
-  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
+  typedef u32x4 pre_t;  // the 8 values of r this chunk needs, requested before the k-loop
+  __device__ __forceinline__ pre_t prefetch(int p, int q) const { return *(const u32x4*)(r + (long)q * F + p); }
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const pre_t& rv, int) const {
     const float dq = sc[SC_DQ_DH2], sdp = sc[SC_S_DP];
     const long off = (long)q * F + p;
     float rr[8], dp[8];
-    unpack8bf(*(const u32x4*)(r + off), rr);
+    unpack8bf(rv, rr);
 #pragma unroll
     for (int i = 0; i < 8; ++i) dp[i] = round_bf((v[i] * dq) * rr[i]);
     *(u32x4*)(dpre + off) = pack8bf(dp);
