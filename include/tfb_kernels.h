@@ -143,6 +143,14 @@ int tfb_quant_fp8(const void* x, const void* scale_ptr, float scale_imm, int fmt
  * Replaces _precast8_kernel / precast_ref (round2/source/kernels/nki_mlp_l4t.py:392, 948-970). */
 int tfb_mlp8_precast(const void* w_fc, const void* w_proj, const void* row, void* w8, int F, int d, void* stream);
 
+/* tfb_mlp8_forward_scales + tfb_mlp8_precast for `layers` MLPs in six launches: rows fp32 [layers][16], w8 uint8
+ * [layers][4][F*d], from weights laid out with one stride (layer i's w_fc at w_fc + i * layer_stride elements, its
+ * w_proj at w_proj + i * layer_stride). scratch: layers * tfb_mlp8_scale_scratch_floats(F) floats. F, d multiples of 64.
+ * Replaces the loop over layers of fp8_refresh_weights (round2/source/train.py:6617: mlp8_scales_into 7003 +
+ * mlp8_precast_into 7267 per layer). */
+int tfb_mlp8_refresh_layers(const void* w_fc, const void* w_proj, long layer_stride, int layers, void* rows, void* w8,
+                            void* scratch, int F, int d, float e4m3_limit, float x_scale, void* stream);
+
 /* Forward from x8 = e4m3(x s_x) [M][d]: y bf16 [M][d], r bf16 [M][F] (saved for backward), h8 [M][F] byte scratch.
  * M % 128 == 0, d % 256 == 0, F % 256 == 0 (the reference's shapes_apply8, nki_mlp_fused8.py:666).
  * Replaces _mlp8_fwd_kernel / _mlp8_fwd_pc_kernel (nki_mlp_fused8.py:509, nki_mlp_l4t.py:434); op s2mlp8::fwd

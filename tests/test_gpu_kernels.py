@@ -285,6 +285,20 @@ def test_mlp8_fp8_weight_grads(ops, dev, shape, limit):
     assert rel_l2(a_fc, ref_fc + acc_fc) < 1e-4 and rel_l2(a_pj, ref_pj + acc_pj) < 1e-4
 
 
+def test_mlp8_refresh_of_all_layers_equals_per_layer_calls(ops, dev):
+    g = _g(31)
+    L, d, F = 3, 256, 512
+    per = 2 * F * d + 1024                                                 # w_fc, w_proj and some other parameters
+    flat = (0.05 * torch.randn(L * per, generator=g)).bfloat16().to(dev)
+    wfc = [flat[i * per:i * per + F * d].view(F, d) for i in range(L)]
+    wpj = [flat[i * per + F * d:i * per + 2 * F * d].view(d, F) for i in range(L)]
+    rows, w8 = ops.mlp8_refresh_layers(wfc[0], wpj[0], per, L, 448.0, 4.0)
+    for i in range(L):
+        row = ops.mlp8_forward_scales(wfc[i], wpj[i], 448.0, 4.0)
+        assert torch.equal(rows[i], row)
+        assert torch.equal(w8[i], ops.mlp8_precast(wfc[i], wpj[i], row))
+
+
 def test_mlp8_full_size_properties(ops, dev):
     """BASELINE config 3 sizes: exact equivariance under a permutation of the tokens and agreement of 512-row slices
     with the oracle."""

@@ -30,6 +30,7 @@ SIGNATURES = {
     "tfb_amax_scale": [_vp, _l, _f, _i, _i, _vp, _vp, _vp],
     "tfb_quant_fp8": [_vp, _vp, _f, _i, _vp, _l, _vp],
     "tfb_mlp8_precast": [_vp, _vp, _vp, _vp, _i, _i, _vp],
+    "tfb_mlp8_refresh_layers": [_vp, _vp, _l, _i, _vp, _vp, _vp, _i, _i, _f, _f, _vp],
     "tfb_mlp8_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_mlp8_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_mlp8_bwd_q": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _l, _i, _i, _vp],

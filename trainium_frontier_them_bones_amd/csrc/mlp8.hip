@@ -105,10 +105,15 @@ __global__ __launch_bounds__(256) void amax_partial_kernel(const bf16_t* __restr
 }
 
 // One wavefront per row of w [rows][cols]: sum of squares per row; amax partial per workgroup.
+// blockIdx.z = layer of a batched refresh: w advances by wz elements, the outputs by their per-layer sizes (oz floats).
 __global__ __launch_bounds__(256) void row_stats_kernel(const bf16_t* __restrict__ w, int rows, int cols,
-                                                       float* __restrict__ rowss, float* __restrict__ amax_part) {
+                                                       float* __restrict__ rowss, float* __restrict__ amax_part, long wz,
+                                                       long oz) {
   __shared__ float red[4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  w += blockIdx.z * wz;
+  rowss += blockIdx.z * oz;
+  amax_part += blockIdx.z * oz;
   float m = 0.f;
   for (int r = blockIdx.x * 4 + wave; r < rows; r += gridDim.x * 4) {
     float ss = 0.f;
@@ -134,10 +139,14 @@ __global__ __launch_bounds__(256) void row_stats_kernel(const bf16_t* __restrict
 // colss_part [COL_SLICES][cols] and are added in slice order by the scale kernel; amax partial per workgroup.
 constexpr int COL_SLICES = 32;
 __global__ __launch_bounds__(256) void col_stats_kernel(const bf16_t* __restrict__ w, int rows, int cols,
-                                                       float* __restrict__ colss_part, float* __restrict__ amax_part) {
+                                                       float* __restrict__ colss_part, float* __restrict__ amax_part, long wz,
+                                                       long oz) {
   __shared__ float red[4];
   __shared__ float acc[4][512];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  w += blockIdx.z * wz;
+  colss_part += blockIdx.z * oz;
+  amax_part += blockIdx.z * oz;
   const int c = blockIdx.x * 512 + lane * 8;
   const int per = (rows + gridDim.y - 1) / gridDim.y;
   const int r0 = blockIdx.y * per, r1 = min(rows, r0 + per);
@@ -167,9 +176,11 @@ __global__ __launch_bounds__(256) void col_stats_kernel(const bf16_t* __restrict
 
 // colss[c] = sum over the row slices, in slice order
 __global__ __launch_bounds__(256) void col_finish_kernel(const float* __restrict__ part, int n, int slices,
-                                                        float* __restrict__ colss) {
+                                                        float* __restrict__ colss, long oz) {
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
+  part += blockIdx.z * oz;
+  colss += blockIdx.z * oz;
   float t = 0.f;
   for (int sl = 0; sl < slices; ++sl) t += part[(long)sl * n + i];
   colss[i] = t;
@@ -185,8 +196,13 @@ __device__ float reduce_max_array(const float* a, int n, float* red) {
 __global__ __launch_bounds__(256) void forward_scales_kernel(const float* rowss, int F, const float* amax_fc_part, int nfc,
                                                             const float* colss, const float* amax_pj_part, int npj,
                                                             float e4m3_limit, float h_bound, float inv_x_scale,
-                                                            float* row_out) {
+                                                            float* row_out, long oz) {
   __shared__ float red[4];
+  rowss += blockIdx.z * oz;
+  amax_fc_part += blockIdx.z * oz;
+  colss += blockIdx.z * oz;
+  amax_pj_part += blockIdx.z * oz;
+  row_out += blockIdx.z * NSC;
   float rho2 = reduce_max_array(rowss, F, red);
   float kappa2 = reduce_max_array(colss, F, red);
   float amax_fc = reduce_max_array(amax_fc_part, nfc, red);
@@ -264,8 +280,13 @@ __global__ __launch_bounds__(256) void quant_kernel(const bf16_t* __restrict__ x
 
 // w [R][C] bf16 -> out [R][C] e4m3 and outT [C][R] e4m3, 64 x 64 tiles through LDS.
 __global__ __launch_bounds__(256) void precast_kernel(const bf16_t* __restrict__ w, const float* __restrict__ scale_ptr,
-                                                     uint8_t* __restrict__ out, uint8_t* __restrict__ outT, int R, int C) {
+                                                     uint8_t* __restrict__ out, uint8_t* __restrict__ outT, int R, int C,
+                                                     long wz, long sz, long bz) {
   __shared__ uint8_t t[64][80];
+  w += blockIdx.z * wz;
+  scale_ptr += blockIdx.z * sz;
+  out += blockIdx.z * bz;
+  outT += blockIdx.z * bz;
   const float s = *scale_ptr;
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
 #pragma unroll
@@ -430,11 +451,11 @@ constexpr int AMAX_BLOCKS = 1024;
 extern "C" long tfb_mlp8_scale_scratch_floats(int F) { return (2L + COL_SLICES) * F + 4L * AMAX_BLOCKS; }
 
 // row_out: fp32 [16] device. e4m3_limit: 240 reproduces the reference's rows; 448 is the OCP maximum.
-extern "C" int tfb_mlp8_forward_scales(const void* w_fc, const void* w_proj, void* row_out, void* scratch, int F, int d,
-                                       float e4m3_limit, float x_scale, void* stream) {
-  if (!w_fc || !w_proj || !row_out || !scratch) return TFB_ERR_ARG;
-  if (F <= 0 || d <= 0 || F % 8 || d % 8) return TFB_ERR_SHAPE;
-  hipStream_t s = (hipStream_t)stream;
+// The forward scale rows of `layers` MLPs whose weights sit `wz` elements apart (w_fc and w_proj alike): four launches
+// whatever the layer count. scratch: layers x tfb_mlp8_scale_scratch_floats(F) floats; row_out: layers x 16 floats.
+static int launch_forward_scales(const void* w_fc, const void* w_proj, void* row_out, void* scratch, int F, int d,
+                                 float e4m3_limit, float x_scale, int layers, long wz, hipStream_t s) {
+  const long oz = tfb_mlp8_scale_scratch_floats(F);
   float* rowss = (float*)scratch;
   float* colss = rowss + F;
   float* colpart = colss + F;
@@ -443,19 +464,28 @@ extern "C" int tfb_mlp8_forward_scales(const void* w_fc, const void* w_proj, voi
   int nfc = (F + 3) / 4;
   if (nfc > AMAX_BLOCKS) nfc = AMAX_BLOCKS;
   int npj = (F + 511) / 512;
-  hipLaunchKernelGGL(row_stats_kernel, dim3(nfc), dim3(256), 0, s, (const bf16_t*)w_fc, F, d, rowss, pa);
+  hipLaunchKernelGGL(row_stats_kernel, dim3(nfc, 1, layers), dim3(256), 0, s, (const bf16_t*)w_fc, F, d, rowss, pa, wz, oz);
   TFB_LAUNCH_CHECK();
   int slices = AMAX_BLOCKS / npj < COL_SLICES ? AMAX_BLOCKS / npj : COL_SLICES;
   if (slices < 1) return TFB_ERR_SHAPE;
-  hipLaunchKernelGGL(col_stats_kernel, dim3(npj, slices), dim3(256), 0, s, (const bf16_t*)w_proj, d, F, colpart, pb);
+  hipLaunchKernelGGL(col_stats_kernel, dim3(npj, slices, layers), dim3(256), 0, s, (const bf16_t*)w_proj, d, F, colpart, pb, wz,
+                     oz);
   TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(col_finish_kernel, dim3((F + 255) / 256), dim3(256), 0, s, colpart, F, slices, colss);
+  hipLaunchKernelGGL(col_finish_kernel, dim3((F + 255) / 256, 1, layers), dim3(256), 0, s, colpart, F, slices, colss, oz);
   TFB_LAUNCH_CHECK();
   const float h_bound = (float)(1.3 * (double)d);
-  hipLaunchKernelGGL(forward_scales_kernel, dim3(1), dim3(256), 0, s, rowss, F, pa, nfc, colss, pb, npj * slices, e4m3_limit, h_bound,
-                     (float)(1.0 / (double)x_scale), (float*)row_out);
+  hipLaunchKernelGGL(forward_scales_kernel, dim3(1, 1, layers), dim3(256), 0, s, rowss, F, pa, nfc, colss, pb, npj * slices,
+                     e4m3_limit, h_bound, (float)(1.0 / (double)x_scale), (float*)row_out, oz);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
+}
+
+extern "C" int tfb_mlp8_forward_scales(const void* w_fc, const void* w_proj, void* row_out, void* scratch, int F, int d,
+                                       float e4m3_limit, float x_scale, void* stream) {
+  if (!w_fc || !w_proj || !row_out || !scratch) return TFB_ERR_ARG;
+  if (F <= 0 || d <= 0 || F % 8 || d % 8) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  return launch_forward_scales(w_fc, w_proj, row_out, scratch, F, d, e4m3_limit, x_scale, 1, 0, s);
 }
 
 extern "C" int tfb_mlp8_backward_scales(const void* dy, const void* row_in, void* row_out, void* scratch, long M, int d,
@@ -507,11 +537,35 @@ extern "C" int tfb_mlp8_precast(const void* w_fc, const void* w_proj, const void
   hipStream_t s = (hipStream_t)stream;
   uint8_t* b = (uint8_t*)w8;
   const long n = (long)F * d;
-  hipLaunchKernelGGL(precast_kernel, dim3(d / 64, F / 64), dim3(256), 0, s, (const bf16_t*)w_fc,
-                     (const float*)row + SC_S_WFC, b, b + n, F, d);
+  hipLaunchKernelGGL(precast_kernel, dim3(d / 64, F / 64, 1), dim3(256), 0, s, (const bf16_t*)w_fc,
+                     (const float*)row + SC_S_WFC, b, b + n, F, d, 0L, 0L, 0L);
   TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(precast_kernel, dim3(F / 64, d / 64), dim3(256), 0, s, (const bf16_t*)w_proj,
-                     (const float*)row + SC_S_WPROJ, b + 2 * n, b + 3 * n, d, F);
+  hipLaunchKernelGGL(precast_kernel, dim3(F / 64, d / 64, 1), dim3(256), 0, s, (const bf16_t*)w_proj,
+                     (const float*)row + SC_S_WPROJ, b + 2 * n, b + 3 * n, d, F, 0L, 0L, 0L);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// The per-optimizer-step refresh of `layers` MLPs in six launches: scale rows [layers][16] and e4m3 packs [layers][4 F d]
+// (layouts as tfb_mlp8_forward_scales / tfb_mlp8_precast) from weights laid out with one stride: layer i's w_fc at
+// w_fc + i * layer_stride elements, its w_proj at w_proj + i * layer_stride. scratch: layers x
+// tfb_mlp8_scale_scratch_floats(F) floats. The per-layer calls cost ~45 us of small launches each.
+extern "C" int tfb_mlp8_refresh_layers(const void* w_fc, const void* w_proj, long layer_stride, int layers, void* rows, void* w8,
+                                       void* scratch, int F, int d, float e4m3_limit, float x_scale, void* stream) {
+  if (!w_fc || !w_proj || !rows || !w8 || !scratch) return TFB_ERR_ARG;
+  if (F <= 0 || d <= 0 || F % 64 || d % 64 || layers <= 0 || layers > 65535 || layer_stride < 0 || layer_stride % 8 ||
+      !(x_scale > 0.f))
+    return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  int st = launch_forward_scales(w_fc, w_proj, rows, scratch, F, d, e4m3_limit, x_scale, layers, layer_stride, s);
+  if (st != TFB_OK) return st;
+  uint8_t* b = (uint8_t*)w8;
+  const long n = (long)F * d;
+  hipLaunchKernelGGL(precast_kernel, dim3(d / 64, F / 64, layers), dim3(256), 0, s, (const bf16_t*)w_fc,
+                     (const float*)rows + SC_S_WFC, b, b + n, F, d, layer_stride, (long)NSC, 4 * n);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(precast_kernel, dim3(F / 64, d / 64, layers), dim3(256), 0, s, (const bf16_t*)w_proj,
+                     (const float*)rows + SC_S_WPROJ, b + 2 * n, b + 3 * n, d, F, layer_stride, (long)NSC, 4 * n);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
@@ -521,8 +575,8 @@ extern "C" int tfb_mlp8_precast(const void* w_fc, const void* w_proj, const void
 extern "C" int tfb_precast8(const void* w, const void* scale_ptr, void* out8, void* outT8, int R, int C, void* stream) {
   if (!w || !scale_ptr || !out8 || !outT8) return TFB_ERR_ARG;
   if (R <= 0 || C <= 0 || R % 64 || C % 64) return TFB_ERR_SHAPE;
-  hipLaunchKernelGGL(precast_kernel, dim3(C / 64, R / 64), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)w,
-                     (const float*)scale_ptr, (uint8_t*)out8, (uint8_t*)outT8, R, C);
+  hipLaunchKernelGGL(precast_kernel, dim3(C / 64, R / 64, 1), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)w,
+                     (const float*)scale_ptr, (uint8_t*)out8, (uint8_t*)outT8, R, C, 0L, 0L, 0L);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

@@ -141,8 +141,21 @@ class GPT:
 
     def refresh_fp8(self):
         """Per-optimizer-step refresh of each layer's fp8 scale row and e4m3 weight pack."""
-        for i, st in enumerate(self.mlp_state):
-            st.refresh(self.p["w_fc.%d" % i], self.p["w_proj.%d" % i])
+        L = self.cfg.n_layer
+        o_fc = [self.mats.offsets["w_fc.%d" % i][0] for i in range(L)]
+        o_pj = [self.mats.offsets["w_proj.%d" % i][0] for i in range(L)]
+        stride = o_fc[1] - o_fc[0] if L > 1 else 0
+        if all(o_fc[i] - o_fc[0] == i * stride and o_pj[i] - o_pj[0] == i * stride for i in range(L)):
+            # the layers' weights sit one stride apart in the flat buffer: one batched refresh (six launches)
+            st0 = self.mlp_state[0]
+            self._mlp_rows, self._mlp_w8 = ops.mlp8_refresh_layers(
+                self.p["w_fc.0"].detach(), self.p["w_proj.0"].detach(), stride, L, st0.e4m3_limit, st0.x_scale,
+                getattr(self, "_mlp_rows", None), getattr(self, "_mlp_w8", None))
+            for i, st in enumerate(self.mlp_state):
+                st.row, st.w8 = self._mlp_rows[i], self._mlp_w8[i]
+        else:
+            for i, st in enumerate(self.mlp_state):
+                st.refresh(self.p["w_fc.%d" % i], self.p["w_proj.%d" % i])
         if self.qkv_state is not None:
             for i in range(self.cfg.n_layer):
                 self.qkv_state[i].refresh(self.p["w_qkv.%d" % i])

@@ -182,6 +182,26 @@ def mlp8_forward_scales(w_fc, w_proj, e4m3_limit=240.0, x_scale=4.0):
     return row
 
 
+def mlp8_refresh_layers(w_fc0, w_proj0, layer_stride, layers, e4m3_limit=240.0, x_scale=4.0, rows=None, w8=None):
+    """Scale rows [layers, 16] and e4m3 packs [layers, 4, F*d] of `layers` MLPs whose weights share one flat buffer:
+    layer i's w_fc [F, d] starts layer_stride elements after layer i-1's (w_fc0, w_proj0: layer 0's), likewise w_proj.
+    Six launches whatever the layer count; rows / w8 may be given to be overwritten."""
+    _chk(w_fc0), _chk(w_proj0)
+    F, d = w_fc0.shape
+    if tuple(w_proj0.shape) != (d, F):
+        raise ValueError("w_proj must be [d, F]")
+    dev = w_fc0.device
+    if rows is None:
+        rows = torch.empty(layers, NSC, dtype=torch.float32, device=dev)
+    if w8 is None:
+        w8 = torch.empty(layers, 4, F * d, dtype=torch.uint8, device=dev)
+    _chk(rows, torch.float32), _chk(w8, torch.uint8)
+    scr = _scratch(dev, layers * _lib.lib().tfb_mlp8_scale_scratch_floats(F))
+    _lib.call("tfb_mlp8_refresh_layers", _p(w_fc0), _p(w_proj0), int(layer_stride), int(layers), _p(rows), _p(w8), _p(scr),
+              F, d, float(e4m3_limit), float(x_scale), _stream())
+    return rows, w8
+
+
 def mlp8_backward_scales(dy2, row):
     _chk(dy2), _chk(row, torch.float32)
     M, d = dy2.shape
