@@ -344,6 +344,26 @@ def test_attention_fwd_bwd(ops, dev, shape):
     assert rel_l2(dq, dqo) < BF16_TOL and rel_l2(dk, dko) < BF16_TOL and rel_l2(dv, dvo) < BF16_TOL
 
 
+@pytest.mark.parametrize("ramp", [0.5, 3.0, 12.0])
+def test_attention_growing_row_maximum(ops, dev, ramp):
+    """Scores whose row maximum keeps growing along the keys (slowly, by a few powers of two per tile, and by far more
+    than the range of one tile): the forward's reference point of the exponentials has to follow at every rate, and the
+    output and log-sum-exp must not depend on when it does."""
+    from oracle import attention as O
+    B, H, T, D = 1, 2, 1024, 64
+    g = _g(31)
+    q = torch.randn(B, H, T, D, generator=g).abs().bfloat16()
+    k = torch.randn(B, H, T, D, generator=g).abs()
+    k = (k * (1.0 + ramp * torch.arange(T).float()[None, None, :, None] / T)).bfloat16()   # q.k > 0 and growing with the key
+    k[:, :, 700:] *= 0.25                                                                    # ... then far below the maximum
+    v = torch.randn(B, H, T, D, generator=g).bfloat16()
+    o, lse = ops.attn_fwd(q.to(dev), k.to(dev), v.to(dev), 0.125)
+    oo, lo = O.forward(q, k, v, 0.125)
+    assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
+    assert rel_l2(o, oo) < BF16_TOL and rel_l2(lse, lo) < 1e-4
+    assert rel_l2(o, O.sdpa_reference(q, k, v, 0.125)) < BF16_TOL
+
+
 def test_attention_strided_qkv_and_rejects(ops, dev):
     from oracle import attention as O
     from trainium_frontier_them_bones_amd._lib import TfbError

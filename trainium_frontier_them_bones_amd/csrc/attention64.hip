@@ -70,6 +70,19 @@ __device__ __forceinline__ void xcd_block(int nx, int nbh, int& bx, int& bh) {
   }
 }
 
+// Causal work per 128-token block grows linearly along the sequence, and workgroups are dispatched in id order: with one
+// block per workgroup the heaviest blocks of the last (batch, head) pairs start when most of the grid has drained and
+// run on alone (for 16 blocks x 192 pairs on 512 slots: 17 % of the kernel's time). When the block count nx is even a
+// workgroup therefore does block i and then block nx - 1 - i (gridDim.x = nx / 2): every workgroup carries the same
+// work. `heavy_last` = the work grows with the block index (query blocks) rather than falls (key blocks); the heavier
+// block of the pair runs first either way.
+__device__ __forceinline__ int paired_passes(int nx) { return (int)gridDim.x * 2 == nx ? 2 : 1; }
+__device__ __forceinline__ int paired_block(int nx, int bx, int pass, bool heavy_last) {
+  const int first = heavy_last ? nx - 1 - bx : bx;
+  return pass == 0 ? first : nx - 1 - first;
+}
+__host__ inline unsigned paired_grid(int nx) { return (unsigned)(nx % 2 == 0 ? nx / 2 : nx); }
+
 __device__ __forceinline__ int swz(int t) { return (((t >> 1) & 1) << 2) | ((t >> 2) & 3); }
 
 // Of the two workgroups that start together on a CU, the one in an odd wavefront slot (HW_ID.wave_id bit 0) begins
@@ -168,12 +181,14 @@ __global__ __launch_bounds__(256, TFB_FWD64_WPE) void attn64_fwd_kernel(AttnT q,
   stagger_start();
   int bx, bh;
   xcd_block(gridDim.x, gridDim.y, bx, bh);
-  const int qb = gridDim.x - 1 - bx;  // longest rows first
   const int b = bh / H, h = bh % H;
   const bf16_t* qp = q.p + b * q.sb + h * q.sh;
   const uint8_t* kp = (const uint8_t*)(k.p + b * k.sb + h * k.sh);
   const uint8_t* vp = (const uint8_t*)(v.p + b * v.sb + h * v.sh);
   bf16_t* op = o.p + b * o.sb + h * o.sh;
+  const int nx = T / 128, npass = paired_passes(nx);
+  for (int pass = 0; pass < npass; ++pass) {
+  const int qb = paired_block(nx, bx, pass, true);
   const int q0 = qb * 128, qw0 = q0 + wave * 32;
   const long kst = k.st * 2, vst = v.st * 2;
 
@@ -240,14 +255,20 @@ __global__ __launch_bounds__(256, TFB_FWD64_WPE) void attn64_fwd_kernel(AttnT q,
 #pragma unroll
       for (int e = 0; e < 16; e += 2) mx = fmaxf(fmaxf(mx, sc[kt][e]), sc[kt][e + 1]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float alpha = fast_exp2((m - mx) * sl2);
-    m = mx;
-    l *= alpha;
+    // The reference point m of the exponentials only has to keep them in range: it follows the running maximum when
+    // some row's maximum has grown by more than 2^8 (always on a row's first tile, m = -inf), which after the first few
+    // tiles is rare, and the 33 multiplications that rescale l and the output accumulators are skipped otherwise.
+    // O = sum p v / sum p and lse = m + log(sum p) do not depend on the reference point.
+    if (__builtin_amdgcn_ballot_w64((mx - m) * sl2 > 8.0f)) {
+      const float alpha = fast_exp2((m - mx) * sl2);
+      m = mx;
+      l *= alpha;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) oacc[i][e] *= alpha;
-    const float negm = -mx * sl2;
+        for (int e = 0; e < 16; ++e) oacc[i][e] *= alpha;
+    }
+    const float negm = -m * sl2;
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -293,6 +314,8 @@ __global__ __launch_bounds__(256, TFB_FWD64_WPE) void attn64_fwd_kernel(AttnT q,
       *(u32x2*)(op + (long)myq * o.st + d) = w;
     }
   if (lh == 0) lse[(long)bh * T + myq] = (m * sl2 + log2f(lt)) * LN2;  // m is the raw-score maximum
+  __syncthreads();  // the stages are free for the partner block
+  }
 }
 
 // =========================================================================================== delta
@@ -342,8 +365,8 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   stagger_start();
-  int kb, bh;  // low key blocks see the most query tiles: already longest first
-  xcd_block(gridDim.x, gridDim.y, kb, bh);
+  int bx, bh;
+  xcd_block(gridDim.x, gridDim.y, bx, bh);
   const int b = bh / H, h = bh % H;
   const uint8_t* qp = (const uint8_t*)(q.p + b * q.sb + h * q.sh);
   const uint8_t* gp = (const uint8_t*)(go.p + b * go.sb + h * go.sh);
@@ -351,6 +374,9 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
   const bf16_t* vp = v.p + b * v.sb + h * v.sh;
   const float* delp = stats + (long)bh * T;
   const float* nlp = stats + rows + (long)bh * T;
+  const int nx = T / 128, npass = paired_passes(nx);
+  for (int pass = 0; pass < npass; ++pass) {
+  const int kb = paired_block(nx, bx, pass, false);  // low key blocks see the most query tiles
   const int kw0 = kb * 128 + wave * 32, mykey = kw0 + lr;
   const long qst = q.st * 2, gst = go.st * 2;
 
@@ -479,6 +505,8 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
   bf16_t* dvp = dv.p + b * dv.sb + h * dv.sh + (long)mykey * dv.st;
   store_grad_row(dka, scale, dkp, cs, sn, mykey, lh);
   store_grad_row(dva, 1.0f, dvp, nullptr, nullptr, mykey, lh);
+  __syncthreads();  // the stages are free for the partner block
+  }
 }
 
 // =========================================================================================== dQ
@@ -493,12 +521,14 @@ __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, A
   stagger_start();
   int bx, bh;
   xcd_block(gridDim.x, gridDim.y, bx, bh);
-  const int qb = gridDim.x - 1 - bx;
   const int b = bh / H, h = bh % H;
   const bf16_t* qp = q.p + b * q.sb + h * q.sh;
   const bf16_t* gp = go.p + b * go.sb + h * go.sh;
   const uint8_t* kp = (const uint8_t*)(k.p + b * k.sb + h * k.sh);
   const uint8_t* vp = (const uint8_t*)(v.p + b * v.sb + h * v.sh);
+  const int nx = T / 128, npass = paired_passes(nx);
+  for (int pass = 0; pass < npass; ++pass) {
+  const int qb = paired_block(nx, bx, pass, true);
   const int q0 = qb * 128, qw0 = q0 + wave * 32, myq = qw0 + lr;
   const long kst = k.st * 2, vst = v.st * 2;
 
@@ -591,6 +621,8 @@ __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, A
 
   bf16_t* dqp = dq.p + b * dq.sb + h * dq.sh + (long)myq * dq.st;
   store_grad_row(dqa, scale, dqp, cs, sn, myq, lh);
+  __syncthreads();  // the stages are free for the partner block
+  }
 }
 
 AttnT mk(const void* p, const long* s) { return AttnT{(bf16_t*)p, s[0], s[1], s[2]}; }
@@ -600,7 +632,7 @@ AttnT mk(const void* p, const long* s) { return AttnT{(bf16_t*)p, s[0], s[1], s[
 // Called by tfb_attn_fwd / tfb_attn_bwd for D = 64 (arguments already validated there: T % 128 == 0, strides % 8 == 0).
 int tfb_attn64_fwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs, void* o,
                         const long* os, float* lse, int B, int H, int T, float scale, hipStream_t s) {
-  hipLaunchKernelGGL(attn64_fwd_kernel, dim3(T / 128, B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), lse,
+  hipLaunchKernelGGL(attn64_fwd_kernel, dim3(paired_grid(T / 128), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), lse,
                      T, H, scale * LOG2E);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
@@ -616,10 +648,10 @@ int tfb_attn64_bwd_impl(const void* q, const long* qs, const void* k, const long
   hipLaunchKernelGGL(attn64_delta_kernel, dim3((unsigned)((rows * 4 + 255) / 256)), dim3(256), 0, s, mk(o, os), mk(go, gos), lse,
                      stats, T, H, rows, 1.0f / scale);
   TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(attn64_dkdv_kernel, dim3(T / 128, B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
+  hipLaunchKernelGGL(attn64_dkdv_kernel, dim3(paired_grid(T / 128), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
                      mk(dk, dks), mk(dv, dvs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t);
   TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(attn64_dq_kernel, dim3(T / 128, B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
+  hipLaunchKernelGGL(attn64_dq_kernel, dim3(paired_grid(T / 128), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
                      mk(dq, dqs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
