@@ -15,6 +15,17 @@
 //
 // Work layout: a wavefront owns 32 queries (forward, dQ) or 32 keys (dK/dV) as the MFMA column index, so every row
 // statistic is one scalar per lane and the packed score registers are directly the B operand of the next product.
+//
+// What bounds these kernels is the SIMD's vector issue port, not the matrix pipe: measured on gfx950 with one
+// wavefront issuing MFMAs and another VALU instructions on the same SIMD, a 32x32x16 MFMA costs the port about 18
+// cycles, a v_exp_f32 8 and any other VALU instruction 4, and the main loops below run at 80-93 % of the time that sum
+// predicts (dQ: 12 MFMA + 16 exp + 66 other per 32x32 block = 608 cycles against 384 cycles of matrix pipe). The
+// forward and dQ main loops are therefore software-pipelined: the scores of the next block are issued while the vector
+// ALU turns the current block's into P (dS), dealt out 1 MFMA : ~10 VALU by scheduling-group barriers, so the matrix
+// pipe's work hides under the vector work inside one wavefront instead of depending on the other resident wavefront
+// being in the opposite phase. dK/dV has no registers left for a second set of scores at two wavefronts per SIMD and
+// keeps the plain loop.
+#include <type_traits>
 #include "common.hpp"
 
 // wavefronts per SIMD the kernels are compiled for (register budget 512 / n)
@@ -23,6 +34,12 @@
 #endif
 #ifndef TFB_DQ64_WPE
 #define TFB_DQ64_WPE 2
+#endif
+#ifndef TFB_DQ64_VALU_PER_MFMA
+#define TFB_DQ64_VALU_PER_MFMA 10
+#endif
+#ifndef TFB_FWD64_VALU_PER_MFMA
+#define TFB_FWD64_VALU_PER_MFMA 12
 #endif
 #ifndef TFB_FWD64_WPE
 #define TFB_FWD64_WPE 2
@@ -211,54 +228,46 @@ __global__ __launch_bounds__(256, TFB_FWD64_WPE) void attn64_fwd_kernel(AttnT q,
 #pragma unroll
     for (int e = 0; e < 16; ++e) oacc[i][e] = 0.f;
 
-  auto compute = [&](const uint8_t* st, int tile) {
-    const int k0 = tile * 64;
-    if (k0 > qw0 + 31) return;  // the whole tile is in this wavefront's future
-    const uint8_t* kt_ = st;
-    const uint8_t* vt_ = st + TILE;
-    f32x16 sc[2];
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) sc[kt][e] = 0.f;
+  // One 64-key tile against the wavefront's 32 queries, in steps that the main loop overlaps across tiles.
+  // (1) raw scores S = K Q^T (key = MFMA row: a lane holds 32 keys of one query)
+  auto scores = [&](const uint8_t* st, f32x16 (&sc)[2]) {
     bf16x8 ka[2][4];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int s = 0; s < 4; ++s) ka[kt][s] = frag_rows(kt_, kt, s, lr, lh);
+      for (int s = 0; s < 4; ++s) ka[kt][s] = frag_rows(st, kt, s, lr, lh);
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) sc[kt][e] = 0.f;
 #pragma unroll
     for (int s = 0; s < 4; ++s)
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt) sc[kt] = mfma_bf16(ka[kt][s], qf[s], sc[kt]);
-    // V^T fragments do not depend on the softmax: requested now, they arrive while the exponentials run
-    bf16x8 va[2][2][2];
+  };
+  // (2) the V^T fragments of the second product
+  auto load_vT = [&](const uint8_t* st, bf16x8 (&va)[2][2][2]) {
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
-        for (int dt = 0; dt < 2; ++dt) va[kt][hf][dt] = frag_cols(vt_, dt, kt * 32 + 16 * hf, lane);
-    const bool diag = k0 + 63 > qw0;
-    const int kbase = k0 + lh * 4 - (qw0 + lr);  // key - q for element (kt, e) is kbase + kt*32 + (e>>2)*8 + (e&3)
+        for (int dt = 0; dt < 2; ++dt) va[kt][hf][dt] = frag_cols(st + TILE, dt, kt * 32 + 16 * hf, lane);
+  };
+  // (3) the row maximum including this tile
+  auto row_max = [&](const f32x16 (&sc)[2]) {
     float mx = m;
-    if (diag) {  // wavefront-uniform; the per-element masking is branch-free selects
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const bool future = kbase + kt * 32 + (e >> 2) * 8 + (e & 3) > 0;
-          sc[kt][e] = future ? -INFINITY : sc[kt][e];
-        }
-    }
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int e = 0; e < 16; e += 2) mx = fmaxf(fmaxf(mx, sc[kt][e]), sc[kt][e + 1]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    // The reference point m of the exponentials only has to keep them in range: it follows the running maximum when
-    // some row's maximum has grown by more than 2^8 (always on a row's first tile, m = -inf), which after the first few
-    // tiles is rare, and the 33 multiplications that rescale l and the output accumulators are skipped otherwise.
-    // O = sum p v / sum p and lse = m + log(sum p) do not depend on the reference point.
+    return fmaxf(mx, __shfl_xor(mx, 32, 64));
+  };
+  // (4) The reference point m of the exponentials only has to keep them in range: it follows the running maximum when
+  // some row's maximum has grown by more than 2^8 (always on a row's first tile, m = -1e30), which after the first few
+  // tiles is rare, and the 33 multiplications that rescale l and the output accumulators are skipped otherwise.
+  // O = sum p v / sum p and lse = m + log(sum p) do not depend on the reference point.
+  auto follow_max = [&](float mx) {
     if (__builtin_amdgcn_ballot_w64((mx - m) * sl2 > 8.0f)) {
       const float alpha = fast_exp2((m - mx) * sl2);
       m = mx;
@@ -268,38 +277,108 @@ __global__ __launch_bounds__(256, TFB_FWD64_WPE) void attn64_fwd_kernel(AttnT q,
 #pragma unroll
         for (int e = 0; e < 16; ++e) oacc[i][e] *= alpha;
     }
+  };
+  // (5) P = exp2(sl2 (S - m)) rounded to bf16 and packed as B operands; the row sum runs over the rounded values
+  auto softmax = [&](const f32x16 (&sc)[2], uint32_t (&pw)[2][2][4]) {
     const float negm = -m * sl2;
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        uint32_t w[4];
+      for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
           const int e = 8 * hf + 2 * x;
-          float p0 = fast_exp2(fmaf(sc[kt][e], sl2, negm)), p1 = fast_exp2(fmaf(sc[kt][e + 1], sl2, negm));
-          w[x] = pack2bf(p0, p1);
-          l = sum2bf(w[x], l);  // the row sum runs over the rounded values
+          const float p0 = fast_exp2(fmaf(sc[kt][e], sl2, negm)), p1 = fast_exp2(fmaf(sc[kt][e + 1], sl2, negm));
+          pw[kt][hf][x] = pack2bf(p0, p1);
+          l = sum2bf(pw[kt][hf][x], l);
         }
-        const bf16x8 bb = frag_from(w[0], w[1], w[2], w[3]);
+  };
+  // (6) O += P V
+  auto accumulate = [&](const bf16x8 (&va)[2][2][2], const uint32_t (&pw)[2][2][4]) {
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        const bf16x8 bb = frag_from(pw[kt][hf][0], pw[kt][hf][1], pw[kt][hf][2], pw[kt][hf][3]);
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt) oacc[dt] = mfma_bf16(va[kt][hf][dt], bb, oacc[dt]);
       }
   };
+  // MFMA and VALU instructions of one scheduling region dealt out alternately (8 MFMAs, `per` VALU instructions each)
+  auto interleave = [&](auto per) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x402, decltype(per)::value, 0);
+    }
+  };
 
-  const int n = (q0 + 128) / 64;
+  // State carried between tiles: the scores of the tile about to be normalised (computed one step ahead, while the
+  // previous tile's exponentials ran) and the P / V^T operands of the previous tile, whose product into O runs under
+  // this tile's row maximum.
+  f32x16 scA[2], scB[2];
+  bf16x8 pva[2][2][2];
+  uint32_t ppw[2][2][4];
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+#pragma unroll
+      for (int x = 0; x < 4; ++x) ppw[kt][hf][x] = 0u;
+#pragma unroll
+      for (int dt = 0; dt < 2; ++dt) pva[kt][hf][dt] = bf16x8{};
+    }
+  // a tile with all keys before the workgroup's queries: `cur` holds tile t (scores in scC), `nxt` tile t + 1 (scores
+  // left in scN); tile t + 2 replaces t
+  auto full_tile = [&](uint8_t* cur, const uint8_t* nxt, int t, f32x16 (&scC)[2], f32x16 (&scN)[2]) {
+    const float mx = row_max(scC);
+    accumulate(pva, ppw);
+    interleave(std::integral_constant<int, 3>{});
+    follow_max(mx);
+    load_vT(cur, pva);
+    __syncthreads();  // tile t + 1 has landed; every wavefront has its fragments of tile t
+    issue(cur, t + 2);
+    scores(nxt, scN);
+    softmax(scC, ppw);
+    interleave(std::integral_constant<int, TFB_FWD64_VALU_PER_MFMA>{});
+  };
+  // one of the two tiles over the workgroup's own tokens: skipped when in the wavefront's future, masked on its diagonal
+  auto diagonal_tile = [&](const uint8_t* st, int tile, f32x16 (&sc)[2]) {
+    const int k0 = tile * 64;
+    if (k0 > qw0 + 31) return;
+    bf16x8 va[2][2][2];
+    uint32_t pw[2][2][4];
+    load_vT(st, va);
+    if (k0 + 63 > qw0) {  // wavefront-uniform; the per-element masking is branch-free selects
+      const int kbase = k0 + lh * 4 - (qw0 + lr);  // key - q for element (kt, e) is kbase + kt*32 + (e>>2)*8 + (e&3)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const bool future = kbase + kt * 32 + (e >> 2) * 8 + (e & 3) > 0;
+          sc[kt][e] = future ? -INFINITY : sc[kt][e];
+        }
+    }
+    follow_max(row_max(sc));
+    softmax(sc, pw);
+    accumulate(va, pw);
+  };
+
+  const int n = (q0 + 128) / 64;  // even; tiles n - 2 and n - 1 cover the workgroup's own 128 tokens
   issue(st0, 0);
   wait_all_loads();
   __syncthreads();
-  for (int t = 0; t + 2 <= n; t += 2) {
-    issue(st1, t + 1);
-    compute(st0, t);
-    __syncthreads();
-    issue(st0, t + 2 < n ? t + 2 : n - 1);
-    compute(st1, t + 1);
-    __syncthreads();
+  issue(st1, 1);
+  scores(st0, scA);
+  for (int t = 0; t + 2 < n; t += 2) {
+    full_tile(st0, st1, t, scA, scB);
+    full_tile(st1, st0, t + 1, scB, scA);
   }
-  // n is even (128 queries per workgroup, 64-key tiles)
+  accumulate(pva, ppw);  // the last full tile's product (zeros when there was none)
+  diagonal_tile(st0, n - 2, scA);
+  __syncthreads();
+  scores(st1, scB);
+  diagonal_tile(st1, n - 1, scB);
 
   const int myq = qw0 + lr;
   const float lt = l + __shfl_xor(l, 32, 64);
@@ -555,69 +634,115 @@ __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, A
 #pragma unroll
     for (int e = 0; e < 16; ++e) dqa[i][e] = 0.f;
 
-  auto compute = [&](const uint8_t* st, int tile) {
-    const uint8_t* kt_ = st;
-    const uint8_t* vt_ = st + TILE;
-    const int k0 = tile * 64;
+  // One 32-key block of the tile at `st`, in four steps that the main loop overlaps across blocks.
+  // (1) S and dP, started from the query's -lse / scale and -delta
+  auto scores = [&](const uint8_t* st, int kt, f32x16& S, f32x16& dP) {
+    bf16x8 ka[4], va[4];
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
-      const int klo = k0 + kt * 32;
-      if (klo > qw0 + 31) continue;
-      bf16x8 ka[4], va[4];
+    for (int s = 0; s < 4; ++s) {
+      ka[s] = frag_rows(st, kt, s, lr, lh);
+      va[s] = frag_rows(st + TILE, kt, s, lr, lh);
+    }
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        ka[s] = frag_rows(kt_, kt, s, lr, lh);
-        va[s] = frag_rows(vt_, kt, s, lr, lh);
-      }
-      f32x16 S, dP;  // started from the query's -lse / scale and -delta
+    for (int e = 0; e < 16; ++e) {
+      S[e] = myL;
+      dP[e] = myD;
+    }
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        S[e] = myL;
-        dP[e] = myD;
-      }
+    for (int s = 0; s < 4; ++s) {
+      S = mfma_bf16(ka[s], qf[s], S);
+      dP = mfma_bf16(va[s], gf[s], dP);
+    }
+  };
+  // (2) the K^T fragments of the last product
+  auto load_kT = [&](const uint8_t* st, int kt, bf16x8 (&kT)[2][2]) {
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        S = mfma_bf16(ka[s], qf[s], S);
-        dP = mfma_bf16(va[s], gf[s], dP);
-      }
-      bf16x8 kT[2][2];  // requested before the arithmetic they do not depend on
+    for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
-      for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) kT[dt][ks] = frag_cols(kt_, dt, kt * 32 + 16 * ks, lane);
+      for (int ks = 0; ks < 2; ++ks) kT[dt][ks] = frag_cols(st, dt, kt * 32 + 16 * ks, lane);
+  };
+  // (3) dS = bf16(P) (dP - delta), packed as the B operand; `klo` = first key of the block when it can reach past the
+  // wavefront's queries (masked scores become -inf, P = 0, through branch-free selects), -1 when it cannot
+  auto softmax_ds = [&](f32x16& S, const f32x16& dP, uint32_t (&dsw)[8], int klo) {
+    if (klo >= 0) {
       const int kbase = klo + lh * 4 - myq;
-      if (klo + 31 > qw0) {  // wavefront-uniform
 #pragma unroll
-        for (int e = 0; e < 16; ++e) S[e] = (kbase + (e >> 2) * 8 + (e & 3) > 0) ? -INFINITY : S[e];
-      }
-      uint32_t dsw[8];
+      for (int e = 0; e < 16; ++e) S[e] = (kbase + (e >> 2) * 8 + (e & 3) > 0) ? -INFINITY : S[e];
+    }
 #pragma unroll
-      for (int e = 0; e < 16; e += 2) {
-        const float p0 = fast_exp2(S[e] * sl2), p1 = fast_exp2(S[e + 1] * sl2);
-        const uint32_t w = pack2bf(p0, p1);
-        dsw[e >> 1] = pack2bf(bflo(w) * dP[e], bfhi(w) * dP[e + 1]);
-      }
+    for (int e = 0; e < 16; e += 2) {
+      const float p0 = fast_exp2(S[e] * sl2), p1 = fast_exp2(S[e + 1] * sl2);
+      const uint32_t w = pack2bf(p0, p1);  // the reference multiplies dP - delta by the rounded P
+      dsw[e >> 1] = pack2bf(bflo(w) * dP[e], bfhi(w) * dP[e + 1]);
+    }
+  };
+  // (4) dQ += dS K
+  auto accumulate = [&](const bf16x8 (&kT)[2][2], const uint32_t (&dsw)[8]) {
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        const bf16x8 db = frag_from(dsw[4 * ks], dsw[4 * ks + 1], dsw[4 * ks + 2], dsw[4 * ks + 3]);
+    for (int ks = 0; ks < 2; ++ks) {
+      const bf16x8 db = frag_from(dsw[4 * ks], dsw[4 * ks + 1], dsw[4 * ks + 2], dsw[4 * ks + 3]);
 #pragma unroll
-        for (int dt = 0; dt < 2; ++dt) dqa[dt] = mfma_bf16(kT[dt][ks], db, dqa[dt]);
-      }
+      for (int dt = 0; dt < 2; ++dt) dqa[dt] = mfma_bf16(kT[dt][ks], db, dqa[dt]);
+    }
+  };
+  // MFMA and VALU instructions of one scheduling region dealt out alternately: the matrix pipe works on the next block's
+  // scores while the vector ALU turns the current block's into dS
+  auto interleave = [&]() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x402, TFB_DQ64_VALU_PER_MFMA, 0);
     }
   };
 
-  const int n = (q0 + 128) / 64;
+  f32x16 Sa, dPa;  // the scores of the next tile's first block, computed one step ahead
+  // a tile with all keys before the workgroup's queries: `cur` holds tile t, `nxt` tile t + 1; tile t + 2 replaces t
+  auto full_tile = [&](uint8_t* cur, const uint8_t* nxt, int t) {
+    bf16x8 kTa[2][2], kTb[2][2];
+    uint32_t dsa[8], dsb[8];
+    f32x16 Sb, dPb;
+    load_kT(cur, 0, kTa);
+    scores(cur, 1, Sb, dPb);
+    softmax_ds(Sa, dPa, dsa, -1);
+    interleave();
+    accumulate(kTa, dsa);
+    load_kT(cur, 1, kTb);
+    __syncthreads();  // tile t + 1 has landed; every wavefront has its fragments of tile t
+    issue(cur, t + 2);
+    scores(nxt, 0, Sa, dPa);
+    softmax_ds(Sb, dPb, dsb, -1);
+    interleave();
+    accumulate(kTb, dsb);
+  };
+  // one of the two tiles over the workgroup's own tokens: blocks in the wavefront's future are skipped, its diagonal
+  // block masked; `first_ready`: block 0's scores are already in Sa / dPa
+  auto diagonal_tile = [&](const uint8_t* st, int tile, bool first_ready) {
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      const int klo = tile * 64 + kt * 32;
+      if (klo > qw0 + 31) continue;
+      if (!(first_ready && kt == 0)) scores(st, kt, Sa, dPa);
+      bf16x8 kT[2][2];
+      uint32_t dsw[8];
+      load_kT(st, kt, kT);
+      softmax_ds(Sa, dPa, dsw, klo + 31 > qw0 ? klo : -1);
+      accumulate(kT, dsw);
+    }
+  };
+
+  const int n = (q0 + 128) / 64;  // even; tiles n - 2 and n - 1 cover the workgroup's own 128 tokens
   issue(st0, 0);
   wait_all_loads();
   __syncthreads();
-  for (int t = 0; t + 2 <= n; t += 2) {
-    issue(st1, t + 1);
-    compute(st0, t);
-    __syncthreads();
-    issue(st0, t + 2 < n ? t + 2 : n - 1);
-    compute(st1, t + 1);
-    __syncthreads();
+  issue(st1, 1);
+  scores(st0, 0, Sa, dPa);
+  for (int t = 0; t + 2 < n; t += 2) {
+    full_tile(st0, st1, t);
+    full_tile(st1, st0, t + 1);
   }
+  diagonal_tile(st0, n - 2, true);
+  __syncthreads();
+  diagonal_tile(st1, n - 1, false);
 
   bf16_t* dqp = dq.p + b * dq.sb + h * dq.sh + (long)myq * dq.st;
   store_grad_row(dqa, scale, dqp, cs, sn, myq, lh);
