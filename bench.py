@@ -1,9 +1,10 @@
 """Benchmark: train tokens/s of the 12-layer d768 T2048 step (fwd + bwd + AdamW) on one MI355X, entirely on the
 HIP kernels, with the roofline position of the dominant kernel and the CPU oracle timed beside it.
 
-python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--fp8-dw]
+python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--fp8-dw] [--unfused-residual]
 Prints ONE JSON line. --fp8-dw (not the default, not the headline configuration) also runs the MLP's two weight-gradient
-GEMMs in fp8, as the reference's round-1 recipe does; the line's config then says so.
+GEMMs in fp8, as the reference's round-1 recipe does; the line's config then says so. --unfused-residual runs the same
+arithmetic with the residual adds and the MLP's fp8 operand cast as passes of their own (for comparison; same values).
 
 python bench.py --traffic-probe   (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: a 256 MiB device copy as the
 counters' calibration, then attention forward + backward at the benchmark shape; prints nothing)
@@ -73,6 +74,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true")
     ap.add_argument("--fp8-dw", action="store_true")
+    ap.add_argument("--unfused-residual", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -90,6 +92,7 @@ def main():
     dev = torch.device("cuda:0")
     cfg = GPTConfig()
     cfg.fp8_mlp_dw = bool(args.fp8_dw)
+    cfg.fuse_residual = not args.unfused_residual
     model = GPT(cfg, dev, seed=0)
     B = 16
     idx, tg = zipf_tokens(B, cfg.seq_len, cfg.vocab, seed=0)
@@ -131,7 +134,9 @@ def main():
         "data": "synthetic: Zipf(1.1) token ids, N(0, 0.02) random-init weights",
         "config": {"workload": "C4 full step: 12 layers, d_model 768, 12 heads x 64, MLP 3072 squared-ReLU fp8, RMSNorm "
                                "pre-norm, RoPE, untied head, vocab 32768; batch 16 x 2048 tokens; fwd+bwd+AdamW"
-                               + ("; MLP weight gradients in fp8 too (--fp8-dw)" if args.fp8_dw else ""),
+                               + ("; MLP weight gradients in fp8 too (--fp8-dw)" if args.fp8_dw else "")
+                               + ("; residual adds and fp8 casts as separate passes (--unfused-residual)"
+                                  if args.unfused_residual else ""),
                    "global_batch": B, "seq_len": cfg.seq_len, "params": model.num_params(),
                    "step_tflops": round(flops_per_token(cfg) * tokens / 1e12, 2),
                    "model_tflops_per_s": round(flops_per_token(cfg) * tokens / (dt / args.steps) / 1e12, 1),

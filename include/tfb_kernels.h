@@ -26,6 +26,10 @@ extern "C" {
  * weight-gradient accumulate of round1/source/train.py:8463-8509. */
 int tfb_gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int trans_a, int trans_b, int out_f32,
                   int accumulate, void* workspace, long workspace_bytes, void* stream);
+/* C [M,N] = bf16(res + bf16(A [M,K] @ op(B))), res [M,N] bf16: a projection with the residual add that follows it made in
+ * the GEMM's store; equal to tfb_gemm_bf16 followed by a bf16 add, bit for bit. B is [K,N] (trans_b=0) or [N,K].
+ * The bf16 form of _proj8_fwd_ra_kernel (round2/source/kernels/nki_attn_nr8.py:1003: out = bf16(res + bf16(acc dq))). */
+int tfb_gemm_bf16_res(const void* A, const void* B, const void* res, void* C, int M, int N, int K, int trans_b, void* stream);
 
 /* ---- RMSNorm family --------------------------------------------------------------------------------------------
  * Number of partial-sum rows the backward kernels write for `nrows` rows (host helper, no GPU work). */
@@ -37,6 +41,12 @@ int tfb_norm_bwd_blocks(long nrows);
  * (6826) and nf_norm_rows (round2/source/train.py:8805). */
 int tfb_rmsnorm_fwd(const void* x, const void* res, const void* w, void* s_out, void* y, void* inv, long nrows, int C,
                     float eps, void* stream);
+/* tfb_rmsnorm_fwd that also writes y8 [nrows][C] = e4m3(bf16(y) * y8_scale): the operand cast of the fp8 GEMM that
+ * consumes y (tfb_mlp8_fwd's x8 at the constant scale 4, tfb_gemm_fp8's a8), made in the norm's pass instead of one of
+ * its own. Replaces the norm prologue of _mlp8_fwd_nr_kernel (round2/source/kernels/nki_mlp_nr8.py:1032: xn, rs and the
+ * casts at X_SCALE) and of _proj8_fwd_nm_kernel (round2/source/kernels/nki_attn_nr8.py:929). */
+int tfb_rmsnorm_fwd_q(const void* x, const void* res, const void* w, void* s_out, void* y, void* inv, void* y8,
+                      float y8_scale, long nrows, int C, float eps, void* stream);
 
 /* dx = gs + inv * (gh - s * (gh . s) * inv^2 / C), gh = gy * w; dw fp32 [C] (+)= sum_rows gy * s * inv.
  * dw_part: fp32 [tfb_norm_bwd_blocks(nrows)][C] scratch (needed only with w).
@@ -157,6 +167,11 @@ int tfb_mlp8_refresh_layers(const void* w_fc, const void* w_proj, long layer_str
  * (round2/source/train.py:6858). r is token-major [M][F] (the reference returns its transpose rT [F][M]). */
 int tfb_mlp8_fwd(const void* x8, const void* w8, const void* row, void* y, void* r, void* h8, long M, int d, int F,
                  void* stream);
+/* tfb_mlp8_fwd with the block's residual add in the second GEMM's store: y = bf16(res + bf16(MLP(x))), res [M][d] bf16;
+ * equal to tfb_mlp8_fwd followed by a bf16 add, bit for bit. Replaces the residual evacuation of _mlp8_fwd_nr_kernel
+ * (round2/source/kernels/nki_mlp_nr8.py:1032: xo = bf16(x1 + y)). */
+int tfb_mlp8_fwd_res(const void* x8, const void* w8, const void* row, const void* res, void* y, void* r, void* h8, long M,
+                     int d, int F, void* stream);
 
 /* Backward from dy8 = e5m2(dy s_dy) [M][d]: dx bf16 [M][d], dpre bf16 [M][F], h = bf16(r^2) [M][F] (NULL to skip),
  * dp8 [M][F] byte scratch. row = the backward row.
@@ -199,6 +214,10 @@ int tfb_precast8(const void* w, const void* scale_ptr, void* out8, void* outT8, 
  * Replaces _proj8_fwd_kernel / _proj8_bwd_kernel (emulate_fwd, emulate_bwd: nki_attn_tt8g.py:745-757). */
 int tfb_gemm_fp8(const void* a8, int fmt_a, const void* b8, const void* dq_a, const void* dq_b, float dq_imm, void* out,
                  long M, int N, int K, void* stream);
+/* tfb_gemm_fp8 (e4m3 activations) with the residual add in the store: out = bf16(res + bf16((a8 @ b8^T) * dq)).
+ * Replaces _proj8_fwd_ra_kernel (round2/source/kernels/nki_attn_nr8.py:1003). */
+int tfb_gemm_fp8_res(const void* a8, const void* b8, const void* dq_a, const void* dq_b, float dq_imm, const void* res,
+                     void* out, long M, int N, int K, void* stream);
 
 /* dw [d][F] (+)= dy^T @ bf16(r^2) (bf16 GEMM over the tokens, h never materialised). workspace fp32 split-K scratch.
  * Replaces the dw_proj half of weight_grads (nki_mlp_fused8.py:706-711) / l4_weight_grads (nki_mlp_l4t.py:932). */

@@ -74,6 +74,48 @@ def test_rmsnorm_fwd_bwd(ops, dev, C, weighted):
     assert rel_l2(y1, O.rmsnorm(x, w, eps)[0]) < 1e-3
 
 
+def test_norm_with_fp8_cast_and_projections_with_residual_equal_the_separate_passes(ops, dev):
+    """The folded forms (norm that also writes the next GEMM's e4m3 operand; projections and the MLP with the residual add
+    in their store) against the separate passes they replace, bit for bit, and against the oracle's composition."""
+    from oracle import mlp8 as OM, norm as ON
+    g = _g(33)
+    M, d, F = 512, 768, 3072
+    x, res = (torch.randn(M, d, generator=g).bfloat16() for _ in range(2))
+    w = (1 + 0.02 * torch.randn(d, generator=g)).bfloat16()
+    xd, rd, wd = x.to(dev), res.to(dev), w.to(dev)
+    # norm + cast
+    for r_ in (None, rd):
+        s0, y0, inv0 = ops.rmsnorm_fwd(xd, wd, 1e-6, res=r_)
+        s1, y1, inv1, y8 = ops.rmsnorm_fwd_q(xd, wd, 1e-6, res=r_, y8_scale=4.0)
+        assert torch.equal(s0, s1) and torch.equal(y0, y1) and torch.equal(inv0, inv1)
+        assert torch.equal(y8, ops.quant_fp8(y0, 4.0, ops.FMT_E4M3))
+        assert torch.equal(y8.cpu().view(torch.float8_e4m3fn).float(), (y0.cpu().float() * 4.0).to(torch.float8_e4m3fn).float())
+    # bf16 projection + residual
+    wo = (0.02 * torch.randn(d, d, generator=g)).bfloat16().to(dev)
+    assert torch.equal(ops.matmul_res(xd, wo, rd, trans_b=True), ops.matmul(xd, wo, trans_b=True) + rd)
+    assert torch.equal(ops.matmul_res(xd, wo, rd), ops.matmul(xd, wo) + rd)
+    # fp8 projection + residual
+    x8 = ops.quant_fp8(xd, 4.0, ops.FMT_E4M3)
+    sw = torch.tensor([64.0, 1.0 / 64.0], device=dev)
+    w8 = ops.quant_fp8(wo, sw[0:1], ops.FMT_E4M3)
+    assert torch.equal(ops.gemm_fp8_res(x8, w8, rd, None, sw[1:2], 0.25), ops.gemm_fp8(x8, w8, ops.FMT_E4M3, None, sw[1:2], 0.25) + rd)
+    # fp8 MLP from the norm's bytes, residual in the second GEMM's store
+    wf = (0.02 * torch.randn(F, d, generator=g)).bfloat16()
+    wp = (0.02 * torch.randn(d, F, generator=g)).bfloat16()
+    row = ops.mlp8_forward_scales(wf.to(dev), wp.to(dev))
+    pack = ops.mlp8_precast(wf.to(dev), wp.to(dev), row)
+    _, h, _, h8 = ops.rmsnorm_fwd_q(xd, wd, 1e-6, y8_scale=4.0)
+    y_sep, r_sep = ops.mlp8_fwd(h, pack, row, F)
+    y_fold, r_fold = ops.mlp8_fwd(h, pack, row, F, x8=h8, res=xd)
+    assert torch.equal(r_fold, r_sep) and torch.equal(y_fold, y_sep + xd)
+    ho = ON.rmsnorm(x, w, 1e-6)[0]
+    yo, _ = OM.forward(ho, wf, wp, OM.forward_scales(wf, wp))
+    assert rel_l2(y_fold, (yo + x).bfloat16()) < FP8_TOL
+    from trainium_frontier_them_bones_amd._lib import TfbError
+    with pytest.raises(TfbError):
+        ops.matmul_res(xd[:100], wo, rd[:100], trans_b=True)                      # rows % 128 != 0
+
+
 def test_norm_weight_gradients_finished_in_one_launch(ops, dev):
     """rmsnorm_bwd(part=...) + norm_dw_finish equals the per-call weight gradient bit for bit (same partials, same
     order of summation), also when added into."""

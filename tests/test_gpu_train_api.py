@@ -213,6 +213,53 @@ def test_gemm_glue_and_mlp_fused8(api, dev):
     assert torch.equal(api.forward_scales(wf8.to(dev), wp8.to(dev)).cpu()[[0, 3, 13]], row[[0, 3, 13]])
 
 
+def test_nr_mlp_and_projection_with_residual(api, dev):
+    """nr_mlp(mlp, x1) = x1 + MLP(rms_norm(x1)) (R2:9202) against the oracle's composition norm -> fp8 MLP -> add, forward
+    and backward (the norm's backward plus the residual gradient, R2:9199), and the projection with its residual."""
+    from oracle import mlp8 as O8, norm as ON
+    g = _g(12)
+    d, F = 256, 512
+    mlp = torch.nn.Module()
+    mlp.c_fc = torch.nn.Linear(d, F, bias=False)
+    mlp.c_proj = torch.nn.Linear(F, d, bias=False)
+    wf8 = (0.05 * torch.randn(F, d, generator=g)).bfloat16()
+    wp8 = (0.05 * torch.randn(d, F, generator=g)).bfloat16()
+    mlp.c_fc.weight.data, mlp.c_proj.weight.data = wf8.clone(), wp8.clone()
+    mlp = mlp.to(dev)
+    x1 = torch.randn(3, 100, d, generator=g).bfloat16()
+    x1d = x1.to(dev).requires_grad_(True)
+    xo = api.nr_mlp(mlp, x1d)
+    x2 = x1.reshape(300, d)
+    xn, inv = ON.rmsnorm(x2, None, ON.RMS_EPS)
+    row = O8.forward_scales(wf8, wp8)
+    yo, ro = O8.forward(xn, wf8, wp8, row)
+    assert xo.shape == x1.shape and rel_l2(xo.reshape(300, d), (x2.float() + yo.float()).bfloat16()) < FP8_TOL
+    assert rel_l2(xo.reshape(300, d).float() - x2.to(dev).float(), yo) < FP8_TOL          # the MLP term itself, not hidden by x1
+    gy = torch.randn(3, 100, d, generator=g).bfloat16()
+    xo.backward(gy.to(dev))
+    gpad = torch.cat([gy.reshape(300, d), torch.zeros(84, d, dtype=torch.bfloat16)])
+    dxn, ho, dpo = O8.backward(gy.reshape(300, d), ro, wf8, wp8, O8.backward_scales(gpad, row))
+    gxo = ON.add_rmsnorm_backward(gy.reshape(300, d), dxn, x2, inv, None)[0]
+    assert rel_l2(x1d.grad.reshape(300, d), gxo) < FP8_TOL
+    assert rel_l2(x1d.grad.reshape(300, d).float() - gy.reshape(300, d).to(dev).float(),
+                  gxo.float() - gy.reshape(300, d).float()) < 2 * FP8_TOL                  # the norm-path term alone
+    dwf, dwp = O8.weight_grads(gy.reshape(300, d), xn, ho, dpo)
+    assert rel_l2(mlp.c_fc.weight.grad, dwf) < FP8_TOL and rel_l2(mlp.c_proj.weight.grad, dwp) < FP8_TOL
+    # projection + residual
+    a = torch.randn(2, 128, d, generator=g).bfloat16()
+    res = torch.randn(2, 128, d, generator=g).bfloat16()
+    w = (0.05 * torch.randn(d, d, generator=g)).bfloat16()
+    ad, rd, wd = (t.to(dev).requires_grad_(True) for t in (a, res, w))
+    out = api.proj_residual(ad, wd, rd)
+    want = ((a.float() @ w.float().t()).bfloat16().float() + res.float()).bfloat16()
+    assert rel_l2(out, want) < 1e-3
+    go = torch.randn(2, 128, d, generator=g).bfloat16()
+    out.backward(go.to(dev))
+    assert torch.equal(rd.grad.cpu(), go)
+    assert rel_l2(ad.grad, go.float() @ w.float()) < BF16_TOL
+    assert rel_l2(wd.grad, go.float().reshape(256, d).t() @ a.float().reshape(256, d)) < BF16_TOL
+
+
 def test_embedding_fwd(api, dev):
     g = _g(8)
     V, C = 1024, 256

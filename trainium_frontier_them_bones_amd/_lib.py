@@ -18,8 +18,10 @@ _lp = ctypes.POINTER(ctypes.c_long)
 # name -> argtypes (restype is always int status unless listed in _RESTYPE)
 SIGNATURES = {
     "tfb_gemm_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _vp],
+    "tfb_gemm_bf16_res": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "tfb_norm_bwd_blocks": [_l],
     "tfb_rmsnorm_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _f, _vp],
+    "tfb_rmsnorm_fwd_q": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _l, _i, _f, _vp],
     "tfb_rmsnorm_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _l, _i, _vp],
     "tfb_norm_dw_finish": [_vp, _vp, _i, _l, _l, _i, _l, _i, _vp],
     "tfb_block_head_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _f, _vp],
@@ -32,6 +34,7 @@ SIGNATURES = {
     "tfb_mlp8_precast": [_vp, _vp, _vp, _vp, _i, _i, _vp],
     "tfb_mlp8_refresh_layers": [_vp, _vp, _l, _i, _vp, _vp, _vp, _i, _i, _f, _f, _vp],
     "tfb_mlp8_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_mlp8_fwd_res": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_mlp8_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_mlp8_bwd_q": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _l, _i, _i, _vp],
     "tfb_gemm_fp8_tn": [_vp, _i, _vp, _i, _vp, _vp, _f, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
@@ -44,6 +47,7 @@ SIGNATURES = {
     "tfb_qkv_rope_fwd": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "tfb_precast8": [_vp, _vp, _vp, _vp, _i, _i, _vp],
     "tfb_gemm_fp8": [_vp, _i, _vp, _vp, _vp, _f, _vp, _l, _i, _i, _vp],
+    "tfb_gemm_fp8_res": [_vp, _vp, _vp, _vp, _f, _vp, _vp, _l, _i, _i, _vp],
     "tfb_relu2": [_vp, _vp, _vp, _l, _i, _vp],
     "tfb_rope": [_vp, _vp, _vp, _vp, _l, _i, _i, _i, _l, _l, _i, _vp],
     "tfb_rope_norm_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _i, _l, _l, _l, _f, _vp],

@@ -23,6 +23,12 @@ def _accumulate_into(w):
     return buf, not fresh
 
 
+def _tail_grads(ctx, gy):
+    """Gradients of the optional trailing (x8, res) inputs of Linear8Fn / Mlp8Fn: none for the bytes, the output's
+    gradient itself for the residual (the add's other operand)."""
+    return (None, gy) if ctx.has_res else (None, None)
+
+
 class RMSNormFn(torch.autograd.Function):
     """y = RMSNorm(x) * weight (weight optional)."""
 
@@ -44,6 +50,41 @@ class RMSNormFn(torch.autograd.Function):
         if weight is None or buf is not None:
             return dx, None, None
         return dx, dw.to(weight.dtype), None
+
+
+class RMSNormPassFn(torch.autograd.Function):
+    """(x, y[, y8]) = (x, RMSNorm(x) * weight[, e4m3(y * y8_scale)]) for a residual stream whose adds are made in the
+    stores of the projections (LinearFn / Linear8Fn / Mlp8Fn with `res`): x is handed through so that the stream's
+    gradient and the norm's meet in ONE backward launch (dx = g_x + J^T g_y), as in AddRMSNormFn. y8 is the operand cast
+    of the fp8 GEMM that consumes y, made in the norm's pass (the norm prologue of round2/source/kernels/nki_mlp_nr8.py:1032
+    and nki_attn_nr8.py:929)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, eps, y8_scale=None):
+        x = x.contiguous()
+        if y8_scale is None:
+            _, y, inv = ops.rmsnorm_fwd(x, weight, eps)
+            outs = (x, y)
+        else:
+            _, y, inv, y8 = ops.rmsnorm_fwd_q(x, weight, eps, None, float(y8_scale))
+            ctx.mark_non_differentiable(y8)
+            outs = (x, y, y8)
+        ctx.save_for_backward(x, inv, weight)
+        return outs
+
+    @staticmethod
+    def backward(ctx, gs, gy, g8=None):
+        x, inv, weight = ctx.saved_tensors
+        gs = None if gs is None else gs.contiguous()
+        if gy is None:
+            return gs, None, None, None
+        part = getattr(weight, "dw_part", None)
+        if part is not None:
+            return ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, gs, part=part)[0], None, None, None
+        buf, acc = (None, False) if weight is None else _accumulate_into(weight)
+        dx, dw = ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, gs, buf, acc)
+        gw = dw.to(weight.dtype) if (weight is not None and buf is None) else None
+        return dx, gw, None, None
 
 
 class AddRMSNormFn(torch.autograd.Function):
@@ -99,11 +140,14 @@ class LinearFn(torch.autograd.Function):
     """y = x @ w^T with w [out, in] (nn.Linear layout); dW accumulates into w.grad_buf when present."""
 
     @staticmethod
-    def forward(ctx, x, w):
+    def forward(ctx, x, w, res=None):
         x2 = x.reshape(-1, x.shape[-1]).contiguous()
-        y = ops.matmul(x2, w, trans_b=True)
+        if res is None:
+            y = ops.matmul(x2, w, trans_b=True)
+        else:   # bf16(res + bf16(x @ w^T)): the residual add made in the GEMM's store (nki_attn_nr8.py:1003)
+            y = ops.matmul_res(x2, w, res.reshape(-1, w.shape[0]).contiguous(), trans_b=True)
         ctx.save_for_backward(x2, w)
-        ctx.xshape = x.shape
+        ctx.xshape, ctx.has_res = x.shape, res is not None
         return y.view(*x.shape[:-1], w.shape[0])
 
     @staticmethod
@@ -114,8 +158,10 @@ class LinearFn(torch.autograd.Function):
         buf, acc = _accumulate_into(w)
         if buf is not None:
             ops.matmul(g2, x2, trans_a=True, out=buf, accumulate=acc)
-            return dx, None
-        return dx, ops.matmul(g2, x2, trans_a=True)
+            dw = None
+        else:
+            dw = ops.matmul(g2, x2, trans_a=True)
+        return (dx, dw, gy) if ctx.has_res else (dx, dw)
 
 
 class CausalAttentionFn(torch.autograd.Function):
@@ -293,19 +339,27 @@ class Linear8Fn(torch.autograd.Function):
     None for the per-tensor amax scale of x. The arithmetic of emulate_fwd / emulate_bwd (nki_attn_tt8g.py:745-757)."""
 
     @staticmethod
-    def forward(ctx, x, w, state, x_scale):
+    def forward(ctx, x, w, state, x_scale, x8=None, res=None):
+        """x8: the bytes e4m3(x * x_scale) when the norm that made x already cast them (RMSNormPassFn); res: a residual
+        added in the GEMM's store, bf16(res + bf16(x @ w^T)) (nki_attn_nr8.py:1003)."""
         x2 = x.reshape(-1, x.shape[-1]).contiguous()
+        r2 = None if res is None else res.reshape(-1, w.shape[0]).contiguous()
         if x_scale is None:
             sx = ops.amax_scale(x2, state.limit, -24, 40)
             x8 = ops.quant_fp8(x2, sx[0:1], ops.FMT_E4M3)
-            y = ops.gemm_fp8(x8, state.w8, ops.FMT_E4M3, sx[1:2], state.sc[1:2])
+            dq_a, dq = sx[1:2], 1.0
             ctx.sx, ctx.sx_imm = sx[0:1], 1.0
         else:
-            x8 = ops.quant_fp8(x2, float(x_scale), ops.FMT_E4M3)
-            y = ops.gemm_fp8(x8, state.w8, ops.FMT_E4M3, None, state.sc[1:2], 1.0 / float(x_scale))
+            x8 = ops.quant_fp8(x2, float(x_scale), ops.FMT_E4M3) if x8 is None else x8.reshape(x2.shape)
+            dq_a, dq = None, 1.0 / float(x_scale)
             ctx.sx, ctx.sx_imm = None, 1.0 / float(x_scale)
+        if r2 is None:
+            y = ops.gemm_fp8(x8, state.w8, ops.FMT_E4M3, dq_a, state.sc[1:2], dq)
+        else:
+            y = ops.gemm_fp8_res(x8, state.w8, r2, dq_a, state.sc[1:2], dq)
         ctx.save_for_backward(x8 if state.dw_fp8 else x2, w)
-        ctx.state, ctx.xshape = state, x.shape
+        ctx.state, ctx.xshape, ctx.nin = state, x.shape, 4 + (x8 is not None) + (res is not None)
+        ctx.has_res = res is not None
         return y.view(*x.shape[:-1], w.shape[0])
 
     @staticmethod
@@ -321,7 +375,7 @@ class Linear8Fn(torch.autograd.Function):
             dw = ops.gemm_fp8_tn(g8, xa, ops.FMT_E5M2, ops.FMT_E4M3, sg[0:1], ctx.sx, ctx.sx_imm, out=buf, accumulate=acc)
         else:
             dw = ops.matmul(g2, xa, trans_a=True, out=buf, accumulate=acc)
-        return dx, (None if buf is not None else dw), None, None
+        return (dx, (None if buf is not None else dw), None, None) + _tail_grads(ctx, gy)
 
 
 class Mlp8State:
@@ -345,16 +399,20 @@ class Mlp8Fn(torch.autograd.Function):
     (round2/source/train.py:8209 mlp8_weight_grads)."""
 
     @staticmethod
-    def forward(ctx, x, w_fc, w_proj, state):
+    def forward(ctx, x, w_fc, w_proj, state, x8=None, res=None):
+        """x8: the bytes e4m3(x * state.x_scale) when the norm that made x already cast them (RMSNormPassFn); res: the
+        block's residual, added in the second GEMM's store: y = bf16(res + bf16(MLP(x))) (nki_mlp_nr8.py:1032)."""
         x2 = x.reshape(-1, x.shape[-1]).contiguous()
+        x8 = None if x8 is None else x8.reshape(x2.shape)
+        r2 = None if res is None else res.reshape(x2.shape).contiguous()
         if state.dw_fp8:
-            y, r, x8 = ops.mlp8_fwd(x2, state.w8, state.row, w_fc.shape[0], state.x_scale, want_x8=True)
+            y, r, x8 = ops.mlp8_fwd(x2, state.w8, state.row, w_fc.shape[0], state.x_scale, want_x8=True, x8=x8, res=r2)
             ctx.save_for_backward(x8, r, w_fc, w_proj)
         else:
-            y, r = ops.mlp8_fwd(x2, state.w8, state.row, w_fc.shape[0], state.x_scale)
+            y, r = ops.mlp8_fwd(x2, state.w8, state.row, w_fc.shape[0], state.x_scale, x8=x8, res=r2)
             ctx.save_for_backward(x2, r, w_fc, w_proj)
         ctx.state = state
-        ctx.xshape = x.shape
+        ctx.xshape, ctx.has_res = x.shape, res is not None
         return y.view(x.shape)
 
     @staticmethod
@@ -370,9 +428,9 @@ class Mlp8Fn(torch.autograd.Function):
                 raise RuntimeError("the fp8 weight gradients write both MLP weights' gradient buffers in one call")
             if bf is not None:
                 ops.mlp8_dw8(x2, dp8, hq8, dy8, rowb, st.x_scale, dw_fc=bf, dw_proj=bp, accumulate=af)
-                return dx.view(ctx.xshape), None, None, None
+                return (dx.view(ctx.xshape), None, None, None) + _tail_grads(ctx, gy)
             dw_fc, dw_proj = ops.mlp8_dw8(x2, dp8, hq8, dy8, rowb, st.x_scale)
-            return dx.view(ctx.xshape), dw_fc, dw_proj, None
+            return (dx.view(ctx.xshape), dw_fc, dw_proj, None) + _tail_grads(ctx, gy)
         dx, _, dpre = ops.mlp8_bwd(g2, r, st.w8, rowb, want_h=False)
         buf, acc = _accumulate_into(w_fc)
         if buf is not None:
@@ -386,7 +444,38 @@ class Mlp8Fn(torch.autograd.Function):
             dw_proj = None
         else:
             dw_proj = ops.mlp_dw_proj(g2, r)
-        return dx.view(ctx.xshape), dw_fc, dw_proj, None
+        return (dx.view(ctx.xshape), dw_fc, dw_proj, None) + _tail_grads(ctx, gy)
+
+
+class NrMlpFn(torch.autograd.Function):
+    """x_out = x1 + MLP(rms_norm(x1)) for a dense block on rows x1 [M, d] (round2/source/train.py:9168 NrMlp): the norm
+    (parameter-free, eps 2^-23) also writes the MLP's e4m3 operand, the residual add is made in the second GEMM's store,
+    and in the backward the norm's backward and the residual gradient's add are one launch (gx = g + J^T dxn)."""
+
+    @staticmethod
+    def forward(ctx, x2, w_fc, w_proj, state, eps=2.0 ** -23):
+        x2 = x2.contiguous()
+        _, xn, inv, x8 = ops.rmsnorm_fwd_q(x2, None, eps, None, state.x_scale)
+        xo, r = ops.mlp8_fwd(xn, state.w8, state.row, w_fc.shape[0], state.x_scale, x8=x8, res=x2)
+        ctx.save_for_backward(x2, x8 if state.dw_fp8 else xn, inv, r, w_fc, w_proj)
+        ctx.state = state
+        return xo
+
+    @staticmethod
+    def backward(ctx, g):
+        x2, xa, inv, r, w_fc, w_proj = ctx.saved_tensors
+        st = ctx.state
+        g = g.contiguous()
+        rowb = ops.mlp8_backward_scales(g, st.row)
+        if st.dw_fp8:
+            dxn, _, dp8, hq8, dy8 = ops.mlp8_bwd_q(g, r, st.w8, rowb, st.e4m3_limit)
+            dw_fc, dw_proj = ops.mlp8_dw8(xa, dp8, hq8, dy8, rowb, st.x_scale)
+        else:
+            dxn, _, dpre = ops.mlp8_bwd(g, r, st.w8, rowb, want_h=False)
+            dw_fc = ops.matmul(dpre, xa, trans_a=True)
+            dw_proj = ops.mlp_dw_proj(g, r)
+        gx = ops.rmsnorm_bwd(dxn, x2, inv, None, g)[0]
+        return gx, dw_fc, dw_proj, None, None
 
 
 class LmHeadLossFn(torch.autograd.Function):

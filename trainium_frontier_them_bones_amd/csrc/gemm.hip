@@ -84,6 +84,22 @@ extern "C" int tfb_gemm_bf16(const void* A, const void* B, void* C, int M, int N
   return run<TFB_K_CONTIG, TFB_K_STRIDED>(P, Q, N, M, K, C, out_f32, accumulate, ws, workspace_bytes, s);
 }
 
+// C [M][N] = bf16(res + bf16(A [M][K] @ op(B))), B [N][K] (trans_b) or [K][N]: a projection with the residual add that
+// follows it made in the store. Equal to tfb_gemm_bf16 followed by a bf16 add, bit for bit. The bf16 form of the
+// reference's projection-with-residual forward (round2/source/kernels/nki_attn_nr8.py:1003).
+extern "C" int tfb_gemm_bf16_res(const void* A, const void* B, const void* res, void* C, int M, int N, int K, int trans_b,
+                                 void* stream) {
+  if (!A || !B || !res || !C) return TFB_ERR_ARG;
+  if (M <= 0 || N <= 0 || K <= 0 || M % 128 || N % 128 || K % 64) return TFB_ERR_SHAPE;
+  GemmOperand P{(const uint8_t*)B, trans_b ? (long)K * 2 : (long)N * 2}, Q{(const uint8_t*)A, (long)K * 2};
+  EpiStoreRes e{(bf16_t*)C, (const bf16_t*)res, (long)N};
+  if (trans_b)
+    return gemm_launch<GemmCfg<128, 128, 2, 2, 2, TFB_K_CONTIG, TFB_K_CONTIG>>(P, Q, N, M, (long)K * 2, 1, LoadIdentity{},
+                                                                               LoadIdentity{}, e, (hipStream_t)stream);
+  return gemm_launch<GemmCfg<128, 128, 2, 2, 2, TFB_K_STRIDED, TFB_K_CONTIG>>(P, Q, N, M, (long)K * 2, 1, LoadIdentity{},
+                                                                              LoadIdentity{}, e, (hipStream_t)stream);
+}
+
 // qkv [M][N] = rope(x [M][K] @ w [N][K]^T): the fused attention projection with the rotary embedding of the q and k
 // thirds (the first rot_cols columns, heads of 64 elements) applied in the GEMM epilogue; row m is token m % T.
 // cos_t, sin_t: bf16 [T][32]. The output equals tfb_gemm_bf16 followed by tfb_rope bit for bit.

@@ -571,6 +571,24 @@ static int gemm_launch_args(GemmArgs a, int groups_y, int splits, PreP prep, Pre
 // ---- shared epilogue helpers -----------------------------------------------------------------
 
 // out (bf16 or fp32) [nq][ld] (+)= D
+// out = bf16(res + bf16(D)): the residual add that follows a projection, made where the product leaves the accumulators
+// (two roundings, as the separate add of the bf16 product makes them). The residual chunk is requested before the k-loop.
+struct EpiStoreRes {
+  bf16_t* out;
+  const bf16_t* res;
+  long ld;  // elements, of both
+  using pre_t = u32x4;
+  __device__ __forceinline__ pre_t prefetch(int p, int q) const { return *(const u32x4*)(res + (long)q * ld + p); }
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const pre_t& r, int) const {
+    float a[8], b[8];
+    unpack8bf(pack8bf(v), a);
+    unpack8bf(r, b);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) a[k] += b[k];
+    *(u32x4*)(out + (long)q * ld + p) = pack8bf(a);
+  }
+};
+
 struct EpiStore {
   void* out;
   long ld;  // elements

@@ -361,6 +361,40 @@ struct EpiScaleStore {  // out = bf16(acc * sc[col])
   }
 };
 
+// out = bf16(res + bf16(acc * dq)): EpiScaleStore / EpiDescale with the residual add that follows the projection made in
+// the same store (the reference's projection-with-residual forward, K/nki_attn_nr8.py:1003, and the residual half of
+// K/nki_mlp_nr8.py:1032); dq = sc[col] when sc is given, else dq_imm * *dq_a * *dq_b. Two roundings, as the separate add.
+struct EpiDescaleRes {
+  const float* sc;
+  int col;
+  const float* dq_a;
+  const float* dq_b;
+  float dq_imm;
+  const bf16_t* res;
+  bf16_t* out;
+  long ld;
+  using pre_t = u32x4;
+  __device__ __forceinline__ pre_t prefetch(int p, int q) const { return *(const u32x4*)(res + (long)q * ld + p); }
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const pre_t& rv, int) const {
+    float dq;
+    if (sc) {
+      dq = sc[col];
+    } else {
+      dq = dq_imm;
+      if (dq_a) dq *= *dq_a;
+      if (dq_b) dq *= *dq_b;
+    }
+    float r[8], a[8], b[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = v[i] * dq;
+    unpack8bf(pack8bf(r), a);
+    unpack8bf(rv, b);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a[i] += b[i];
+    *(u32x4*)(out + (long)q * ld + p) = pack8bf(a);
+  }
+};
+
 struct EpiDescale {  // out = bf16(acc * dq), dq = dq_imm * *dq_a * *dq_b (absent factors are 1)
   const float* dq_a;
   const float* dq_b;
@@ -599,6 +633,18 @@ extern "C" int tfb_gemm_fp8(const void* a8, int fmt_a, const void* b8, const voi
   return gemm_launch<Cfg8g>(P, Q, N, (int)M, (long)K, 1, LoadIdentity{}, LoadIdentity{}, e, (hipStream_t)stream);
 }
 
+// tfb_gemm_fp8 with the residual add in the store: out = bf16(res + bf16((a8 @ b8^T) * dq)), res [M][N] bf16; e4m3
+// activations only (a forward projection). Equal to tfb_gemm_fp8 followed by a bf16 add, bit for bit.
+// Replaces _proj8_fwd_ra_kernel (round2/source/kernels/nki_attn_nr8.py:1003).
+extern "C" int tfb_gemm_fp8_res(const void* a8, const void* b8, const void* dq_a, const void* dq_b, float dq_imm, const void* res,
+                                void* out, long M, int N, int K, void* stream) {
+  if (!a8 || !b8 || !res || !out) return TFB_ERR_ARG;
+  if (M <= 0 || N <= 0 || K <= 0 || M % 128 || N % 128 || K % 128 || M > 0x7fffffffL) return TFB_ERR_SHAPE;
+  GemmOperand P{(const uint8_t*)b8, (long)K}, Q{(const uint8_t*)a8, (long)K};
+  EpiDescaleRes e{nullptr, 0, (const float*)dq_a, (const float*)dq_b, dq_imm, (const bf16_t*)res, (bf16_t*)out, (long)N};
+  return gemm_launch<Cfg8>(P, Q, N, (int)M, (long)K, 1, LoadIdentity{}, LoadIdentity{}, e, (hipStream_t)stream);
+}
+
 // out [O][D] (+)= ((g8 [M][O]^T @ a8 [M][D]) * imm / (*s_g * *s_a)): the fp8 weight gradient of a projection, contraction
 // over the M tokens of two token-major byte tensors (fp32 accumulation over all tokens, one rounding; bf16 or fp32
 // output, optionally accumulated into). (fmt_g, fmt_a) = (e5m2, e4m3): a gradient against the forward's activation
@@ -642,6 +688,26 @@ extern "C" int tfb_mlp8_fwd(const void* x8, const void* w8, const void* row, voi
   if (st != TFB_OK) return st;
   GemmOperand Pp{b + 2 * n, (long)F}, Qh{(const uint8_t*)h8, (long)F};
   EpiScaleStore e2{(const float*)row, SC_DQ_PROJ, (bf16_t*)y, (long)d};
+  return gemm_launch<Cfg8>(Pp, Qh, d, (int)M, (long)F, 1, LoadIdentity{}, LoadIdentity{}, e2, s);
+}
+
+// tfb_mlp8_fwd with the block's residual add in the second GEMM's store: y = bf16(res + bf16(MLP(x))), res [M][d] bf16 (the
+// MLP's input before its norm). Equal to tfb_mlp8_fwd followed by a bf16 add, bit for bit.
+// Replaces the residual half of _mlp8_fwd_nr_kernel (round2/source/kernels/nki_mlp_nr8.py:1032); its norm half is
+// tfb_rmsnorm_fwd_q, which hands this call its x8.
+extern "C" int tfb_mlp8_fwd_res(const void* x8, const void* w8, const void* row, const void* res, void* y, void* r, void* h8,
+                                long M, int d, int F, void* stream) {
+  if (!x8 || !w8 || !row || !res || !y || !r || !h8) return TFB_ERR_ARG;
+  if (!shapes8(M, d, F)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const uint8_t* b = (const uint8_t*)w8;
+  const long n = (long)F * d;
+  GemmOperand Pw{b, (long)d}, Qx{(const uint8_t*)x8, (long)d};
+  EpiUp e1{(const float*)row, (bf16_t*)r, (uint8_t*)h8, (long)F};
+  int st = gemm_launch<Cfg8>(Pw, Qx, F, (int)M, (long)d, 1, LoadIdentity{}, LoadIdentity{}, e1, s);
+  if (st != TFB_OK) return st;
+  GemmOperand Pp{b + 2 * n, (long)F}, Qh{(const uint8_t*)h8, (long)F};
+  EpiDescaleRes e2{(const float*)row, SC_DQ_PROJ, nullptr, nullptr, 1.0f, (const bf16_t*)res, (bf16_t*)y, (long)d};
   return gemm_launch<Cfg8>(Pp, Qh, d, (int)M, (long)F, 1, LoadIdentity{}, LoadIdentity{}, e2, s);
 }
 

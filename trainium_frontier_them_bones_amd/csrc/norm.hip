@@ -77,7 +77,7 @@ template <int NCH>
 __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ res,
                                                          const bf16_t* __restrict__ w, bf16_t* __restrict__ s_out,
                                                          bf16_t* __restrict__ y, float* __restrict__ inv, long nrows,
-                                                         int C, float eps) {
+                                                         int C, float eps, uint8_t* __restrict__ y8, float y8_scale) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   Row<NCH> wr;
   if (w) wr.load(w, C, lane);
@@ -100,6 +100,19 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16_t* __restri
 #pragma unroll
       for (int k = 0; k < 8; ++k) a.v[i][k] = w ? a.v[i][k] * rs * wr.v[i][k] : a.v[i][k] * rs;
     a.store(y + row * C, C, lane);
+    if (y8) {  // e4m3(bf16(y) * scale): the cast the fp8 GEMM that consumes y would otherwise make in a pass of its own
+      a.round();
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        const int c = (lane + 64 * i) * 8;
+        if (c < C) {
+          u32x2 o;
+          o.x = cvt4_fp8<TFB_FMT_E4M3>(a.v[i][0] * y8_scale, a.v[i][1] * y8_scale, a.v[i][2] * y8_scale, a.v[i][3] * y8_scale);
+          o.y = cvt4_fp8<TFB_FMT_E4M3>(a.v[i][4] * y8_scale, a.v[i][5] * y8_scale, a.v[i][6] * y8_scale, a.v[i][7] * y8_scale);
+          *(u32x2*)(y8 + row * C + c) = o;
+        }
+      }
+    }
     if (inv && lane == 0) inv[row] = rs;
   }
 }
@@ -319,19 +332,31 @@ static bool norm_shape_ok(long nrows, int C) { return nrows > 0 && C > 0 && C % 
 
 extern "C" int tfb_norm_bwd_blocks(long nrows) { return grid_for(nrows, 1024); }
 
-extern "C" int tfb_rmsnorm_fwd(const void* x, const void* res, const void* w, void* s_out, void* y, void* inv, long nrows,
-                               int C, float eps, void* stream) {
+// y8 (optional): e4m3(bf16(y) * y8_scale), [nrows][C] bytes - the operand cast of the fp8 GEMM that consumes y, made here
+// instead of in a pass of its own.
+static int rmsnorm_fwd_impl(const void* x, const void* res, const void* w, void* s_out, void* y, void* inv, void* y8,
+                            float y8_scale, long nrows, int C, float eps, void* stream) {
   if (!x || !y) return TFB_ERR_ARG;
   if (res && !s_out) return TFB_ERR_ARG;
   if (!norm_shape_ok(nrows, C)) return TFB_ERR_SHAPE;
   int grid = grid_for(nrows, 8192);
 #define CALL(N)                                                                                                       \
   hipLaunchKernelGGL(rmsnorm_fwd_kernel<N>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x,          \
-                     (const bf16_t*)res, (const bf16_t*)w, (bf16_t*)s_out, (bf16_t*)y, (float*)inv, nrows, C, eps)
+                     (const bf16_t*)res, (const bf16_t*)w, (bf16_t*)s_out, (bf16_t*)y, (float*)inv, nrows, C, eps,    \
+                     (uint8_t*)y8, y8_scale)
   DISPATCH_NCH(C, CALL);
 #undef CALL
   TFB_LAUNCH_CHECK();
   return TFB_OK;
+}
+extern "C" int tfb_rmsnorm_fwd(const void* x, const void* res, const void* w, void* s_out, void* y, void* inv, long nrows,
+                               int C, float eps, void* stream) {
+  return rmsnorm_fwd_impl(x, res, w, s_out, y, inv, nullptr, 0.f, nrows, C, eps, stream);
+}
+extern "C" int tfb_rmsnorm_fwd_q(const void* x, const void* res, const void* w, void* s_out, void* y, void* inv, void* y8,
+                                 float y8_scale, long nrows, int C, float eps, void* stream) {
+  if (!y8) return TFB_ERR_ARG;
+  return rmsnorm_fwd_impl(x, res, w, s_out, y, inv, y8, y8_scale, nrows, C, eps, stream);
 }
 
 // dw_part: fp32 [tfb_norm_bwd_blocks(nrows)][C] scratch (only when w != NULL); dw: fp32 [C].

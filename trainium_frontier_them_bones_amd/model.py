@@ -35,6 +35,7 @@ class GPTConfig:
     fp8_attn_proj: bool = False   # QKV and output projections in fp8 (e4m3 forward, e5m2 dX, bf16 dW); off in BASELINE C4
     fp8_attn_dw: bool = False     # with fp8_attn_proj: their weight gradients in fp8 as well (R2_DW8_SET=qkv,proj)
     fp8_mlp_dw: bool = False      # the MLP's two weight gradients in fp8 as well (R1's DW_ROWS recipe); off in BASELINE C4
+    fuse_residual: bool = True    # residual adds in the projections' stores, fp8 operand casts in the norms (same values)
 
     @property
     def head_dim(self):
@@ -181,6 +182,8 @@ class GPT:
         self._norm_partials(B * T)
         scale = 1.0 / math.sqrt(cfg.head_dim)
         x = A.EmbeddingFn.apply(idx, p["wte"])
+        if cfg.fuse_residual:
+            return self._forward_fused(x, targets, T, scale)
         h = A.RMSNormFn.apply(x, p["norm1.0"], cfg.norm_eps)
         for i in range(cfg.n_layer):
             if cfg.fp8_attn_proj:    # h is an RMSNorm output (constant scale 4); the attention output takes its amax scale
@@ -198,6 +201,32 @@ class GPT:
             m = A.Mlp8Fn.apply(h, p["w_fc.%d" % i], p["w_proj.%d" % i], self.mlp_state[i])
             nw = p["norm1.%d" % (i + 1)] if i + 1 < cfg.n_layer else p["norm_f"]
             x, h = A.AddRMSNormFn.apply(x, m, nw, cfg.norm_eps)
+        return A.LmHeadLossFn.apply(h, p["lm_head"], targets, cfg.softcap, "mean")
+
+    def _forward_fused(self, x, targets, T, scale):
+        """The same network with the residual adds made in the stores of the output projection and of the MLP's second
+        GEMM, and the MLP's (with fp8 attention projections also the QKV projection's) fp8 operand cast made by the norm
+        that precedes it (round2/source/kernels/nki_attn_nr8.py, nki_mlp_nr8.py): bit-identical activations, two
+        elementwise passes per layer fewer."""
+        cfg, p = self.cfg, self.p
+        q8 = cfg.x_scale if cfg.fp8_attn_proj else None
+        x, h, *h8 = A.RMSNormPassFn.apply(x, p["norm1.0"], cfg.norm_eps, q8)
+        for i in range(cfg.n_layer):
+            if cfg.fp8_attn_proj:
+                qkv = A.Linear8Fn.apply(h, p["w_qkv.%d" % i], self.qkv_state[i], cfg.x_scale, h8[0])
+                att = A.RopeAttentionFn.apply(qkv, self.cos[:T], self.sin[:T], cfg.n_head, scale)
+                x = A.Linear8Fn.apply(att, p["w_o.%d" % i], self.wo_state[i], None, None, x)
+            else:
+                if cfg.head_dim == 64:
+                    att = A.QkvRopeAttentionFn.apply(h, p["w_qkv.%d" % i], self.cos[:T], self.sin[:T], cfg.n_head, scale)
+                else:
+                    qkv = A.LinearFn.apply(h, p["w_qkv.%d" % i])
+                    att = A.RopeAttentionFn.apply(qkv, self.cos[:T], self.sin[:T], cfg.n_head, scale)
+                x = A.LinearFn.apply(att, p["w_o.%d" % i], x)
+            x, h, h8m = A.RMSNormPassFn.apply(x, p["norm2.%d" % i], cfg.norm_eps, cfg.x_scale)
+            x = A.Mlp8Fn.apply(h, p["w_fc.%d" % i], p["w_proj.%d" % i], self.mlp_state[i], h8m, x)
+            nw = p["norm1.%d" % (i + 1)] if i + 1 < cfg.n_layer else p["norm_f"]
+            x, h, *h8 = A.RMSNormPassFn.apply(x, nw, cfg.norm_eps, q8 if i + 1 < cfg.n_layer else None)
         return A.LmHeadLossFn.apply(h, p["lm_head"], targets, cfg.softcap, "mean")
 
     def zero_grad(self):

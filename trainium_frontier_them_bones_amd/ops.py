@@ -64,6 +64,19 @@ def matmul(a, b, trans_a=False, trans_b=False, out=None, accumulate=False, out_d
     return out
 
 
+def matmul_res(a, b, res, trans_b=False):
+    """bf16(res + bf16(a @ op(b))): a projection with the residual add that follows it made in the GEMM's store (equal to
+    matmul followed by a bf16 add, bit for bit). a [M,K]; b [K,N] or, with trans_b, [N,K]; res [M,N]."""
+    _chk(a), _chk(b), _chk(res)
+    M, K = a.shape
+    Kb, N = (b.shape[1], b.shape[0]) if trans_b else (b.shape[0], b.shape[1])
+    if K != Kb or tuple(res.shape) != (M, N):
+        raise ValueError("shapes differ")
+    out = torch.empty(M, N, dtype=bf16, device=a.device)
+    _lib.call("tfb_gemm_bf16_res", _p(a), _p(b), _p(res), _p(out), M, N, K, int(trans_b), _stream())
+    return out
+
+
 def qkv_rope(x2, w, cos, sin, T, rot_cols):
     """rope(x2 @ w^T): the fused attention projection [M, N] with the rotary embedding of its first rot_cols columns
     (heads of 64) applied in the GEMM epilogue; row m is token m % T."""
@@ -87,6 +100,21 @@ def rmsnorm_fwd(x, weight=None, eps=2.0 ** -23, res=None):
     _lib.call("tfb_rmsnorm_fwd", _p(x), _p(res), _p(weight), _p(s) if res is not None else None, _p(y), _p(inv),
               rows, C, float(eps), _stream())
     return s, y, inv
+
+
+def rmsnorm_fwd_q(x, weight=None, eps=2.0 ** -23, res=None, y8_scale=4.0):
+    """rmsnorm_fwd that also returns y8 = e4m3(bf16(y) * y8_scale) bytes, the operand cast of the fp8 GEMM that consumes y
+    (equal to quant_fp8(y, y8_scale), bit for bit). Returns (s, y, inv, y8)."""
+    _chk(x), _chk(res), _chk(weight)
+    C = x.shape[-1]
+    rows = x.numel() // C
+    y = torch.empty_like(x)
+    s = torch.empty_like(x) if res is not None else x
+    inv = torch.empty(rows, dtype=torch.float32, device=x.device)
+    y8 = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    _lib.call("tfb_rmsnorm_fwd_q", _p(x), _p(res), _p(weight), _p(s) if res is not None else None, _p(y), _p(inv), _p(y8),
+              float(y8_scale), rows, C, float(eps), _stream())
+    return s, y, inv, y8
 
 
 def rmsnorm_bwd(gy, s, inv, weight=None, gs=None, dw=None, accumulate=False, part=None):
@@ -255,6 +283,19 @@ def gemm_fp8(a8, b8, fmt_a=FMT_E4M3, dq_a=None, dq_b=None, dq=1.0):
     return out
 
 
+def gemm_fp8_res(a8, b8, res, dq_a=None, dq_b=None, dq=1.0):
+    """bf16(res + bf16((a8 [M,K] @ b8 [N,K]^T) * dq * dq_a * dq_b)): gemm_fp8 (e4m3 activations) with the residual add
+    in the store, equal to gemm_fp8 followed by a bf16 add bit for bit."""
+    _chk(a8, torch.uint8), _chk(b8, torch.uint8), _chk(dq_a, torch.float32), _chk(dq_b, torch.float32), _chk(res)
+    M, K = a8.shape
+    N = b8.shape[0]
+    if b8.shape[1] != K or tuple(res.shape) != (M, N):
+        raise ValueError("shapes differ")
+    out = torch.empty(M, N, dtype=bf16, device=a8.device)
+    _lib.call("tfb_gemm_fp8_res", _p(a8), _p(b8), _p(dq_a), _p(dq_b), float(dq), _p(res), _p(out), M, N, K, _stream())
+    return out
+
+
 def gemm_fp8_tn(g8, a8, fmt_g=FMT_E5M2, fmt_a=FMT_E4M3, s_g=None, s_a=None, imm=1.0, out=None, accumulate=False,
                 out_dtype=bf16):
     """[O,D] (+)= (g8 [M,O]^T @ a8 [M,D]) * imm / (s_g s_a): a weight gradient in fp8 (dw8_grad,
@@ -287,16 +328,26 @@ def mlp8_precast(w_fc, w_proj, row):
     return w8
 
 
-def mlp8_fwd(x2, w8, row, F, x_scale=4.0, want_x8=False):
+def mlp8_fwd(x2, w8, row, F, x_scale=4.0, want_x8=False, x8=None, res=None):
     """y [M,d], r [M,F] (bf16): the fp8 forward. x_scale: python float (the reference's constant 4) or a device scalar.
-    want_x8 also returns x8 = e4m3(x x_scale) [M,d] bytes (the fp8 weight gradient's operand)."""
-    _chk(x2), _chk(w8, torch.uint8), _chk(row, torch.float32)
+    want_x8 also returns x8 = e4m3(x x_scale) [M,d] bytes (the fp8 weight gradient's operand). A given x8 (from
+    rmsnorm_fwd_q) is used instead of casting x2; with res [M,d], y = bf16(res + bf16(MLP(x))) (the block's residual add
+    made in the second GEMM's store)."""
+    _chk(x2), _chk(w8, torch.uint8), _chk(row, torch.float32), _chk(x8, torch.uint8), _chk(res)
     M, d = x2.shape
-    x8 = quant_fp8(x2, x_scale, FMT_E4M3)
+    if x8 is None:
+        x8 = quant_fp8(x2, x_scale, FMT_E4M3)
+    elif tuple(x8.shape) != (M, d):
+        raise ValueError("x8 shape")
     y = torch.empty(M, d, dtype=bf16, device=x2.device)
     r = torch.empty(M, F, dtype=bf16, device=x2.device)
     h8 = torch.empty(M, F, dtype=torch.uint8, device=x2.device)
-    _lib.call("tfb_mlp8_fwd", _p(x8), _p(w8), _p(row), _p(y), _p(r), _p(h8), M, d, F, _stream())
+    if res is None:
+        _lib.call("tfb_mlp8_fwd", _p(x8), _p(w8), _p(row), _p(y), _p(r), _p(h8), M, d, F, _stream())
+    else:
+        if tuple(res.shape) != (M, d):
+            raise ValueError("res shape")
+        _lib.call("tfb_mlp8_fwd_res", _p(x8), _p(w8), _p(row), _p(res), _p(y), _p(r), _p(h8), M, d, F, _stream())
     return (y, r, x8) if want_x8 else (y, r)
 
 

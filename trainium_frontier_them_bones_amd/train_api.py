@@ -265,6 +265,35 @@ def mlp_fused8(mlp, x):
     return y.reshape(b, t, c)
 
 
+def nr_mlp(mlp, x1):
+    """x1 + MLP(rms_norm(x1)) on [b, t, n_embd] with the norm and the residual add folded into the fp8 MLP's two calls
+    (R2:9202 nr_mlp / 9168 NrMlp; kernels K/nki_mlp_nr8.py:1032): the norm's pass also writes the e4m3 operand, the add
+    is made in the second GEMM's store, the backward's norm gradient and residual add are one launch. Rows are padded
+    with zeros to a multiple of 128 (a zero row normalises to zero and adds zero)."""
+    if getattr(mlp, "tfb_mlp8", None) is None or mlp.tfb_mlp8.row is None:
+        fp8_refresh_weights([mlp])
+    b, t, c = x1.shape
+    x2 = x1.reshape(b * t, c)
+    if x2.dtype != bf16:
+        raise RuntimeError("the folded MLP takes bf16 rows, not %s" % x2.dtype)
+    m = x2.shape[0]
+    pad = (-m) % 128
+    if pad:
+        x2 = torch.nn.functional.pad(x2, (0, 0, 0, pad))
+    w_fc = mlp.c_fc.weight if mlp.c_fc.weight.dtype == bf16 else mlp.c_fc.weight.to(bf16)
+    w_proj = mlp.c_proj.weight if mlp.c_proj.weight.dtype == bf16 else mlp.c_proj.weight.to(bf16)
+    xo = A.NrMlpFn.apply(x2, w_fc, w_proj, mlp.tfb_mlp8)
+    if pad:
+        xo = xo[:m]
+    return xo.reshape(b, t, c)
+
+
+def proj_residual(x, w, res):
+    """res + x @ w^T with the add made in the GEMM's store (the bf16 form of _proj8_fwd_ra_kernel,
+    K/nki_attn_nr8.py:1003; R2:9293 NrAttnOut): w [out, in], any leading shape, rows a multiple of 128."""
+    return A.LinearFn.apply(x, w, res)
+
+
 def forward_scales(w_fc, w_proj):
     """The forward's 16-column scale row from the two weights (K/nki_mlp_fused8.py:782)."""
     return ops.mlp8_forward_scales(w_fc, w_proj)
