@@ -6,6 +6,9 @@ Prints ONE JSON line. --fp8-dw (not the default, not the headline configuration)
 GEMMs in fp8, as the reference's round-1 recipe does; the line's config then says so. --unfused-residual runs the same
 arithmetic with the residual adds and the MLP's fp8 operand cast as passes of their own (for comparison; same values).
 
+python bench.py --ns-probe        (Muon's Newton-Schulz call on the benchmark model's four stacks of 12 hidden matrices:
+one line per stack with its time and flop rate; not part of the AdamW step the headline line times)
+
 python bench.py --traffic-probe   (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: a 256 MiB device copy as the
 counters' calibration, then attention forward + backward at the benchmark shape; prints nothing)
 """
@@ -66,6 +69,27 @@ def traffic_probe():
     torch.cuda.synchronize()
 
 
+def ns_probe():
+    import torch
+    from trainium_frontier_them_bones_amd import ops
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    for (K, r, c) in ((12, 3072, 768), (12, 768, 3072), (12, 2304, 768), (12, 768, 768)):
+        g = torch.randn(K, r, c, device=dev) * 0.02
+        d = g.bfloat16().norm(dim=(-2, -1)) * 1.01 + 1e-6
+        for _ in range(3):
+            ops.ns5(g, d)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            ops.ns5(g, d)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / 10
+        M, N = max(r, c), min(r, c)
+        flop = 5 * K * (4 * M * N * N + 2 * N * N * N)   # per iteration: X^T X, X B (2 M N^2 each) and G G (2 N^3)
+        print("ns5 K=%d %dx%d: %.3f ms, %.0f TFLOP/s" % (K, r, c, dt * 1e3, flop / dt / 1e12), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -73,6 +97,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true")
+    ap.add_argument("--ns-probe", action="store_true")
     ap.add_argument("--fp8-dw", action="store_true")
     ap.add_argument("--unfused-residual", action="store_true")
     args = ap.parse_args()
@@ -82,6 +107,9 @@ def main():
 
     if args.traffic_probe:
         traffic_probe()
+        return
+    if args.ns_probe:
+        ns_probe()
         return
 
     import torch

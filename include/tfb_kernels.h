@@ -349,6 +349,18 @@ int tfb_moe_backward_scales(const void* dys, const void* tile_expert, const void
 int tfb_moe_quant(const void* x, const void* tile_expert, const void* rows, int col, int fmt, void* out8, long rmax, int d,
                   void* stream);
 
+/* ---- Muon: Newton-Schulz ("Polar Express") orthogonalisation of a stack of gradient matrices -------------------------
+ * Per matrix, held tall X [M][N] (M >= N): X0 = bf16(bf16(g) / d), then five times G = bf16(X^T X),
+ * B = bf16(c G G + b G), X = bf16(X B + a X) with the (a, b, c) of `coeffs` (15 host floats), fp32 accumulation;
+ * y = X5 in g's layout, v [K][M] = the sums of X5^2 along the N-long side (the NorMuon row statistic times N).
+ * g fp32 [K][M][N] (wide 0) or [K][N][M] (wide 1: handled as the transposes); inv_d fp32 [K] device (1 / d). M, N % 128.
+ * workspace: tfb_ns5_workspace_bytes(K, M, N) bytes of device memory. The whole stack takes 3 grouped GEMM launches per
+ * iteration. Replaces _nsk_kernel(ga, gb, sc) -> ya, yb, va, vb (round2/source/kernels/nki_nsk.py:370; arithmetic
+ * emulate_nsk :452) = the loop of muon_math_body (reference_ns :471); one call per stack. */
+long tfb_ns5_workspace_bytes(int K, int M, int N);
+int tfb_ns5(const void* g, const void* inv_d, const float* coeffs, void* y, void* v, int K, int M, int N, int wide,
+            void* workspace, long workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

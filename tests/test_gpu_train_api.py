@@ -272,3 +272,20 @@ def test_embedding_fwd(api, dev):
     e.backward(gy.to(dev))
     want = torch.zeros(V, C).index_add_(0, idx.reshape(-1), gy.float().reshape(-1, C))
     assert rel_l2(wd.grad, want) < BF16_TOL
+
+
+def test_nsk_both_stacks(api, dev):
+    """nsk(ga, gb, d_a, d_b) (K/nki_nsk.py:370): the tall and the wide stack of one Muon step against the oracle's
+    restatement of emulate_nsk; tolerance as explained in tests/test_gpu_kernels.py (chained iterations)."""
+    from oracle import muon as O
+    g = _g(13)
+    ga = torch.randn(2, 512, 256, generator=g) * 0.02
+    gb = torch.randn(3, 256, 512, generator=g) * 0.02
+    da, db = O.muon_denominator(ga), O.muon_denominator(gb)
+    ya, yb, va, vb = api.nsk(ga.to(dev), gb.to(dev), da.to(dev), db.to(dev))
+    yao, vao = O.ns5(ga, da)
+    ybo, vbo = O.ns5(gb, db)
+    assert ya.shape == ga.shape and yb.shape == gb.shape and va.shape == (2, 512) and vb.shape == (3, 512)
+    assert rel_l2(ya, yao) < 2e-2 and rel_l2(yb, ybo) < 2e-2 and rel_l2(va, vao) < 2e-2 and rel_l2(vb, vbo) < 2e-2
+    e = api.nsk(ga.to(dev)[:0], gb.to(dev), da.to(dev)[:0], db.to(dev))
+    assert e[0].shape == (0, 512, 256) and torch.equal(e[1], yb)

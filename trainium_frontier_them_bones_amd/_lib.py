@@ -77,10 +77,12 @@ SIGNATURES = {
     "tfb_moe_route_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _l, _i, _i, _i, _vp],
     "tfb_moe_backward_scales": [_vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_moe_quant": [_vp, _vp, _vp, _i, _i, _vp, _l, _i, _vp],
+    "tfb_ns5_workspace_bytes": [_i, _i, _i],
+    "tfb_ns5": [_vp, _vp, ctypes.POINTER(ctypes.c_float), _vp, _vp, _i, _i, _i, _i, _vp, _l, _vp],
     "tfb_mlp_dw_proj": [_vp, _vp, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
 }
 
-_LONG_RESULT = {"tfb_mlp8_scale_scratch_floats", "tfb_moe_max_rows", "tfb_embedding_bwd_scratch_ints"}
+_LONG_RESULT = {"tfb_mlp8_scale_scratch_floats", "tfb_moe_max_rows", "tfb_embedding_bwd_scratch_ints", "tfb_ns5_workspace_bytes"}
 
 STATUS = {0: "ok", 1: "unsupported shape", 2: "bad argument", 3: "kernel launch failed", 4: "workspace too small"}
 

@@ -570,7 +570,6 @@ static int gemm_launch_args(GemmArgs a, int groups_y, int splits, PreP prep, Pre
 }
 // ---- shared epilogue helpers -----------------------------------------------------------------
 
-// out (bf16 or fp32) [nq][ld] (+)= D
 // out = bf16(res + bf16(D)): the residual add that follows a projection, made where the product leaves the accumulators
 // (two roundings, as the separate add of the bf16 product makes them). The residual chunk is requested before the k-loop.
 struct EpiStoreRes {
@@ -589,6 +588,7 @@ struct EpiStoreRes {
   }
 };
 
+// out (bf16 or fp32) [nq][ld] (+)= D
 struct EpiStore {
   void* out;
   long ld;  // elements

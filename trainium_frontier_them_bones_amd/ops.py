@@ -806,3 +806,40 @@ def moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, dwr=None, accumulate=False):
     _lib.call("tfb_moe_route_bwd", _p(dgate), _p(p), _p(idx), _p(dxs), _p(tab["slot"]), _p(h2), _p(wr), _p(dlogits), _p(dh),
               _p(dwr), int(accumulate), N, d, E, idx.shape[1], _stream())
     return dh, dwr, dlogits
+
+
+# ------------------------------------------------------------------------------------------ Muon Newton-Schulz
+# the kit's POLAR_EXPRESS_COEFFS as the reference's kernel module holds them (round2/source/kernels/nki_nsk.py:82-88)
+NS_COEFFS = (
+    (8.156554524902461, -22.48329292557795, 15.878769915207462),
+    (4.042929935166739, -2.808917465908714, 0.5000178451051316),
+    (3.8916678022926607, -2.772484153217685, 0.5060648178503393),
+    (3.285753657755655, -2.3681294933425376, 0.46449024233003106),
+    (2.3465413258596377, -1.7097828382687081, 0.42323551169305323),
+)
+_NS_WS = {}
+
+
+def ns5(g, d, coeffs=NS_COEFFS):
+    """Five Newton-Schulz iterations on a stack g fp32 [K, r, c] (tall r >= c, or wide: handled as the transposes) from
+    X0 = bf16(bf16(g) / d), d [K] (any float dtype; the reciprocal is taken in fp32 as the reference's sc_tile does).
+    Returns (y bf16 [K, r, c], v fp32 [K, max(r, c)] = the sums of y^2 along the short side)."""
+    import ctypes
+    _chk(g, torch.float32)
+    K, r, c = g.shape
+    wide = r < c
+    M, N = (c, r) if wide else (r, c)
+    inv = (1.0 / d.reshape(-1).float()).contiguous()
+    if inv.numel() != K:
+        raise ValueError("one denominator per matrix")
+    _chk(inv, torch.float32)
+    need = _lib.lib().tfb_ns5_workspace_bytes(K, M, N)
+    key = (g.device, need)
+    ws = _NS_WS.get(key)
+    if ws is None:
+        ws = _NS_WS[key] = torch.empty(max(need, 256), dtype=torch.uint8, device=g.device)
+    y = torch.empty(K, r, c, dtype=bf16, device=g.device)
+    v = torch.empty(K, M, dtype=torch.float32, device=g.device)
+    co = (ctypes.c_float * 15)(*[float(x) for t in coeffs for x in t])
+    _lib.call("tfb_ns5", _p(g), _p(inv), co, _p(y), _p(v), K, M, N, int(wide), _p(ws), ws.numel(), _stream())
+    return y, v

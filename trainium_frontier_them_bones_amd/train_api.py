@@ -316,3 +316,20 @@ def dw8_grad(g2, a2, s_g, i_g, s_a, i_a, fg, fa):
     g8 = ops.quant_fp8(g2.contiguous(), sg, f8[fg])
     a8 = ops.quant_fp8(a2.contiguous(), sa, f8[fa])
     return ops.gemm_fp8_tn(g8, a8, f8[fg], f8[fa], sg, sa)
+
+
+# ------------------------------------------------------------------------------------------ Muon Newton-Schulz (K/nki_nsk.py)
+def nsk(ga, gb, d_a, d_b, coeffs=ops.NS_COEFFS):
+    """(ya, yb, va, vb) = the five Polar Express iterations of both stacks of a Muon step (K/nki_nsk.py:370 _nsk_kernel,
+    arithmetic :452 emulate_nsk): ga fp32 [K, M, N] tall, gb fp32 [K2, N, M] wide, after the optimizer's two lerps; d_a, d_b
+    the matrices' denominators bf16(bf16(||bf16(g)||) * 1.01 + 1e-6) ([K] or [K, 1, 1], any float dtype; the reciprocal is
+    taken in fp32 as sc_tile does, :406). ya, yb bf16 in the inputs' layouts; va [K, M], vb [K2, M] fp32 = the sums of x^2
+    along the N-long side (the caller divides by N). An empty stack is skipped, as in the reference."""
+    def one(g, d):
+        if g.shape[0] == 0:
+            return (torch.empty(g.shape, dtype=bf16, device=g.device),
+                    torch.empty(0, max(g.shape[1], g.shape[2]), dtype=torch.float32, device=g.device))
+        return ops.ns5(g.contiguous(), d)
+    ya, va = one(ga, d_a)
+    yb, vb = one(gb, d_b)
+    return ya, yb, va, vb
