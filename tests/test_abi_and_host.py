@@ -48,7 +48,7 @@ def test_binding_table_matches_header():
         assert len(sig) == len(args), name
         for a, c in zip(args, sig):
             if "*" in a:
-                assert c in (ctypes.c_void_p, _lib._lp), (name, a)
+                assert c in (ctypes.c_void_p, _lib._lp, _lib._fp), (name, a)
             elif a.startswith("float"):
                 assert c is ctypes.c_float, (name, a)
             elif a.startswith("long"):

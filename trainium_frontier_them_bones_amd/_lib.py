@@ -14,6 +14,7 @@ _i = ctypes.c_int
 _l = ctypes.c_long
 _f = ctypes.c_float
 _lp = ctypes.POINTER(ctypes.c_long)
+_fp = ctypes.POINTER(ctypes.c_float)   # a HOST array of floats (tfb_ns5's coefficients)
 
 # name -> argtypes (restype is always int status unless listed in _RESTYPE)
 SIGNATURES = {
@@ -78,7 +79,7 @@ SIGNATURES = {
     "tfb_moe_backward_scales": [_vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_moe_quant": [_vp, _vp, _vp, _i, _i, _vp, _l, _i, _vp],
     "tfb_ns5_workspace_bytes": [_i, _i, _i],
-    "tfb_ns5": [_vp, _vp, ctypes.POINTER(ctypes.c_float), _vp, _vp, _i, _i, _i, _i, _vp, _l, _vp],
+    "tfb_ns5": [_vp, _vp, _fp, _vp, _vp, _i, _i, _i, _i, _vp, _l, _vp],
     "tfb_mlp_dw_proj": [_vp, _vp, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
 }
 
