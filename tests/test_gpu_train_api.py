@@ -289,3 +289,39 @@ def test_nsk_both_stacks(api, dev):
     assert rel_l2(ya, yao) < 2e-2 and rel_l2(yb, ybo) < 2e-2 and rel_l2(va, vao) < 2e-2 and rel_l2(vb, vbo) < 2e-2
     e = api.nsk(ga.to(dev)[:0], gb.to(dev), da.to(dev)[:0], db.to(dev))
     assert e[0].shape == (0, 512, 256) and torch.equal(e[1], yb)
+
+
+def test_head2_and_adamw_fused_step(api, dev):
+    from oracle import norm as ON
+    g = _g(14)
+    s1, mo, x0, sk = (torch.randn(2, 128, 256, generator=g).bfloat16() for _ in range(4))
+    l1, l2, l3 = torch.tensor([0.9]), torch.tensor([0.25]), torch.tensor([-0.4])
+    d = lambda t: t.to(dev)
+    # the pair form with an external skip, emitting the block input
+    x_new, x_norm, x_in, x0p = api.head2((d(s1), d(mo)), d(x0), d(sk), d(l1), d(l2), d(l3), emit=True)
+    xt = s1 + mo
+    o = ON.block_head(xt.reshape(-1, 256), x0.reshape(-1, 256), l1[0], l2[0], sk.reshape(-1, 256), l3[0])
+    assert torch.equal(x_in.cpu(), xt) and torch.equal(x_new.cpu().reshape(-1, 256), o[0]) and x0p.data_ptr() == x0p.data_ptr()
+    assert rel_l2(x_norm.reshape(-1, 256), o[1]) < 1e-3
+    # the self-skip form on a plain tensor, nothing emitted
+    x_new2, _, none, _ = api.head2(d(xt), d(x0), api.SELF_SKIP, d(l1), d(l2), d(l3))
+    o2 = ON.block_head(xt.reshape(-1, 256), x0.reshape(-1, 256), l1[0], l2[0], xt.reshape(-1, 256), l3[0])
+    assert none is None and torch.equal(x_new2.cpu().reshape(-1, 256), o2[0])
+    # AdamW: three steps against torch.optim.AdamW on the same parameters and gradients
+    ps = [torch.randn(300, 64, generator=g), torch.randn(1000, generator=g)]
+    ref = [p.clone().requires_grad_(True) for p in ps]
+    mine = [p.clone().to(dev).requires_grad_(True) for p in ps]
+    kw = dict(lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    o_ref, o_mine = torch.optim.AdamW(ref, **kw), torch.optim.AdamW(mine, **kw)
+    for step in range(3):
+        for a, b in zip(ref, mine):
+            gr = torch.randn(a.shape, generator=g)
+            a.grad, b.grad = gr.clone(), gr.to(dev)
+        o_ref.step()
+        assert api.adamw_fused_step(o_mine) is True
+    for a, b in zip(ref, mine):
+        assert rel_l2(b, a) < 1e-6
+        assert rel_l2(o_mine.state[b]["exp_avg_sq"], o_ref.state[a]["exp_avg_sq"]) < 1e-6
+    mine[0].grad = mine[0].grad.t().contiguous().t()                         # a strided gradient is not the kernel's layout: nothing is done
+    before = mine[1].detach().clone()
+    assert api.adamw_fused_step(o_mine) is False and torch.equal(mine[1].detach(), before)

@@ -144,6 +144,20 @@ def head_skip(x, x0, skip, l1, l2, l3):
     return x_new.view(x.shape), x_norm.view(x.shape)
 
 
+SELF_SKIP = object()   # head2's marker: the skip is the block's own (materialised) input (R1: mblk_SELF_SKIP)
+
+
+def head2(x, x0, skip, l1, l2, l3, emit=False, key=None):
+    """Block head whose input may be the previous block's (s1, mlp_out) pair (R1:6778): x_in = s1 + mlp_out (or x itself),
+    then head_skip(x_in, x0, skip, l1, l2, l3) with skip None | tensor | SELF_SKIP (= x_in). Returns (x_new, x_norm,
+    x_in when emit else None, x0). The pair's add is one bf16 pass in front of the block-head kernel (the reference's own
+    composition when its folded kernel does not apply, R1:6803-6807); `key` (its gain-gradient bookkeeping) is unused."""
+    x_t = x[0] + x[1] if isinstance(x, (tuple, list)) else x
+    sk = x_t if skip is SELF_SKIP else skip
+    x_new, x_norm = head_skip(x_t, x0, sk, l1, l2, l3)
+    return x_new, x_norm, (x_t if emit else None), x0
+
+
 def rmsnorm_fast(x):
     """F.rms_norm(x, (C,)) (R1:5594)."""
     C = x.shape[-1]
@@ -333,3 +347,40 @@ def nsk(ga, gb, d_a, d_b, coeffs=ops.NS_COEFFS):
     ya, va = one(ga, d_a)
     yb, vb = one(gb, d_b)
     return ya, yb, va, vb
+
+
+# ------------------------------------------------------------------------------------------ fused AdamW step (R1:1573)
+@torch.no_grad()
+def adamw_fused_step(opt) -> bool:
+    """One AdamW step of every parameter group of `opt` (a torch.optim.AdamW-shaped object: param_groups with lr, betas,
+    eps, weight_decay; state with step, exp_avg, exp_avg_sq) through the fused kernel, in place (R1:1573
+    adamw_fused_step; update rule R1:9670-9677: p *= 1 - lr wd; m.lerp_(g, 1 - b1); v.lerp_(g^2, 1 - b2);
+    p -= lr (m / bias1) / (sqrt(v / bias2) + eps)). Returns True when the groups were updated (the caller skips its own
+    step), False - with nothing touched - when a parameter is not the kernel's layout (fp32 device parameter, contiguous
+    fp32 or bf16 gradient of its shape): the reference's "not done, run your own line" convention."""
+    todo = []
+    for g in opt.param_groups:
+        if g.get("amsgrad") or g.get("maximize"):
+            return False
+        for p in g["params"]:
+            if p.grad is None:
+                continue
+            gr = p.grad
+            if (not p.is_cuda or p.dtype != torch.float32 or not p.is_contiguous() or not gr.is_contiguous()
+                    or gr.shape != p.shape or gr.dtype not in (torch.float32, bf16)):
+                return False
+            todo.append((g, p))
+    for g, p in todo:
+        st = opt.state[p]
+        if len(st) == 0:
+            st["step"] = torch.zeros((), dtype=torch.float32)
+            st["exp_avg"] = torch.zeros_like(p)
+            st["exp_avg_sq"] = torch.zeros_like(p)
+        n = int(st["step"]) + 1
+        b1, b2 = g["betas"]
+        ops.adamw_(p, p.grad, st["exp_avg"], st["exp_avg_sq"], n, float(g["lr"]), b1, b2, g["eps"], g["weight_decay"])
+        if torch.is_tensor(st["step"]):
+            st["step"] += 1
+        else:
+            st["step"] = n
+    return True
