@@ -325,3 +325,48 @@ def test_head2_and_adamw_fused_step(api, dev):
     mine[0].grad = mine[0].grad.t().contiguous().t()                         # a strided gradient is not the kernel's layout: nothing is done
     before = mine[1].detach().clone()
     assert api.adamw_fused_step(o_mine) is False and torch.equal(mine[1].detach(), before)
+
+
+def test_r1_fp8_rows(api, dev):
+    """The round-1 fixed-scale fp8 rows (R1:2169 fused_fc_relu2_fp8, 4097 fused_fc_relu2_nn, 3728 c_proj, 3412 row_matmul,
+    3486 dw_matmul, 2059 begin_step) against the oracle's restatement: each row alone, then the MLP forward + backward with
+    the in-place weight-gradient convention."""
+    from oracle import r1fp8 as O
+    nn8 = api.nki_gemm_fp8_nn
+    g = _g(15)
+    M, d, F = 384, 256, 512
+    x = torch.randn(M, d, generator=g).bfloat16()
+    w1 = (0.5 * torch.randn(d, F, generator=g)).bfloat16()                  # LinearT [in, out]
+    w2 = (0.05 * torch.randn(d, F, generator=g)).bfloat16()                 # [out, in]
+    dy = (1e-7 * torch.randn(M, d, generator=g)).bfloat16()
+    xd, w1d, w2d, dyd = (t.to(dev) for t in (x, w1, w2, dy))
+    nn8.begin_step()
+    pre = nn8.row_matmul(xd, w1d, 1)
+    assert rel_l2(pre, O.row_matmul(x, w1, 1)) < 1e-3
+    h = (torch.relu(pre.float()) * pre.float()).bfloat16()
+    assert rel_l2(nn8.row_matmul(h, w2d, 2), O.row_matmul(h.cpu(), w2, 2)) < 1e-3
+    assert rel_l2(nn8.row_matmul(dyd, w2d, 4), O.row_matmul(dy, w2, 4)) < 1e-3
+    dpre = (1e-7 * torch.randn(M, F, generator=g)).bfloat16()
+    assert rel_l2(nn8.row_matmul(dpre.to(dev), w1d, 3), O.row_matmul(dpre, w1, 3)) < 1e-3
+    assert rel_l2(nn8.dw_matmul(xd, dpre.to(dev), 5), O.dw_matmul(x, dpre, 5)) < 1e-3
+    assert rel_l2(nn8.dw_matmul(dyd, h, 6), O.dw_matmul(dy, h.cpu(), 6)) < 1e-3
+    assert nn8.dw_matmul(xd.float(), dpre.to(dev), 5) is None and nn8.dw_matmul(xd[:100], dpre.to(dev)[:100], 5) is None
+    # the weight cache: one fp8 copy per step, a new one after begin_step or after the parameter is written
+    a = api.nki_gemm_fp8.quantised_weight(w1d, 64.0, False)
+    assert api.nki_gemm_fp8.quantised_weight(w1d, 64.0, False) is a
+    nn8.begin_step()
+    assert api.nki_gemm_fp8.quantised_weight(w1d, 64.0, False) is not a
+    # the MLP through the reference's two calls, inplace: gradients are summed into existing .grad tensors
+    x3 = x.view(3, 128, d).to(dev).requires_grad_(True)
+    p1, p2 = w1d.clone().requires_grad_(True), w2d.clone().requires_grad_(True)
+    g1 = (1e-5 * torch.randn(d, F, generator=g)).bfloat16()              # what an earlier micro-step left in .grad
+    p1.grad, p2.grad = g1.to(dev).clone(), g1.to(dev).clone()
+    hh = nn8.fused_fc_relu2_nn(x3, p1, inplace=True)
+    y = nn8.c_proj(hh, p2, True)
+    y.backward(dy.view(3, 128, d).to(dev))
+    yo, dxo, dw1o, dw2o = O.mlp_forward_backward(x, w1, w2, dy)
+    assert y.shape == (3, 128, d) and rel_l2(y.reshape(M, d), yo) < 2e-3
+    assert rel_l2(x3.grad.reshape(M, d), dxo) < 2e-2
+    assert rel_l2(p1.grad, g1.float() + dw1o.float()) < 2e-2 and rel_l2(p2.grad, g1.float() + dw2o.float()) < 2e-2
+    assert rel_l2(p1.grad.float() - g1.to(dev).float(), dw1o) < 5e-2       # the row-5 product itself, not hidden by g1
+    assert api.nki_gemm_fp8.active(True) and not api.nki_gemm_fp8.active(False)

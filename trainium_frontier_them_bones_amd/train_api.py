@@ -384,3 +384,7 @@ def adamw_fused_step(opt) -> bool:
         else:
             st["step"] = n
     return True
+
+
+# ------------------------------------------------------------------------------------------ R1 fp8 MLP rows (R1:1780-4140)
+from .r1_fp8 import nki_gemm_fp8, nki_gemm_fp8_nn  # noqa: E402  (namespaces, as the reference uses its modules)
