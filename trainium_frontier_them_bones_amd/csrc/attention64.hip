@@ -706,6 +706,7 @@ __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, A
     softmax_ds(Sa, dPa, dsa, -1);
     interleave();
     accumulate(kTa, dsa);
+    __builtin_amdgcn_sched_barrier(0);  // the second block's fragments are not requested while the first's are live
     load_kT(cur, 1, kTb);
     __syncthreads();  // tile t + 1 has landed; every wavefront has its fragments of tile t
     issue(cur, t + 2);
