@@ -3,7 +3,7 @@ HIP kernels, with the roofline position of the dominant kernel and the CPU oracl
 
 python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--fp8-dw] [--unfused-residual]
 Prints ONE JSON line. --fp8-dw (not the default, not the headline configuration) also runs the MLP's two weight-gradient
-GEMMs in fp8, as the reference's round-1 recipe does; the line's config then says so. --unfused-residual runs the same
+GEMMs in fp8, as the recipe of the reference's round1 sources does; the line's config then says so. --unfused-residual runs the same
 arithmetic with the residual adds and the MLP's fp8 operand cast as passes of their own (for comparison; same values).
 
 python bench.py --ns-probe        (Muon's Newton-Schulz call on the benchmark model's four stacks of 12 hidden matrices:

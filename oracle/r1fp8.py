@@ -1,4 +1,4 @@
-"""CPU restatement of the round-1 fp8 MLP rows (fixed power-of-two scales). TEST INFRASTRUCTURE ONLY.
+"""CPU restatement of the fp8 MLP rows of the reference's round1 sources (fixed power-of-two scales). TEST INFRASTRUCTURE ONLY.
 
 Follows round1/source/train.py: clip_bound 2272-2283, ROW_SPEC 2300, the constants 1758-1759 and 2234-2243, and the
 arithmetic stated in the module text at 1746 ("out = (s_a A)^T (s_w W) / (s_a s_w), both operands rounded to e4m3 after

@@ -1,4 +1,4 @@
-"""The torch.library registration of the kernel calls (the reference's round-2 form, round2/source/train.py:4988-5036,
+"""The torch.library registration of the kernel calls (the form of the reference's round2 sources, round2/source/train.py:4988-5036,
 6858-6913): the ops against the autograd.Function wrappers they mirror, their fake implementations and schemas."""
 import pytest
 import torch

@@ -328,7 +328,7 @@ def test_head2_and_adamw_fused_step(api, dev):
 
 
 def test_r1_fp8_rows(api, dev):
-    """The round-1 fixed-scale fp8 rows (R1:2169 fused_fc_relu2_fp8, 4097 fused_fc_relu2_nn, 3728 c_proj, 3412 row_matmul,
+    """The fixed-scale fp8 rows of the reference's round1 sources (R1:2169 fused_fc_relu2_fp8, 4097 fused_fc_relu2_nn, 3728 c_proj, 3412 row_matmul,
     3486 dw_matmul, 2059 begin_step) against the oracle's restatement: each row alone, then the MLP forward + backward with
     the in-place weight-gradient convention."""
     from oracle import r1fp8 as O

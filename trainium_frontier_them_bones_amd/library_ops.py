@@ -1,4 +1,4 @@
-"""torch.library registration of the kernel calls, in the reference's round-2 form: `torch.library.custom_op(name,
+"""torch.library registration of the kernel calls, in the form of the reference's round2 sources: `torch.library.custom_op(name,
 mutates_args=())` + `register_fake` (the op's own output allocations) + `register_autograd` with a `setup_context` that
 marks the auxiliary outputs non-differentiable and switches gradient materialisation off
 (round2/source/train.py:4988-5036 s2attn::*, 6858-6913 s2mlp8::*, 7127-7160 s2mlp8l::*, 6145-6156 s2b::loss_head_*).

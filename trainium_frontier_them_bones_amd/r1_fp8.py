@@ -1,4 +1,4 @@
-"""The round-1 recipe of the fp8 MLP: six GEMM "rows" with FIXED power-of-two scales, in the reference's call style
+"""The fp8 MLP recipe of the reference's round1 sources: six GEMM "rows" with FIXED power-of-two scales, in the reference's call style
 (round1/source/train.py: nki_gemm_fp8 1780-2265 = row 1, nki_gemm_fp8_nn 2269-4140 = rows 2-6).
 
     row 1  c_fc forward    x [M, d] @ W1 [d, F]        x e4m3 @ 4        W1 e4m3 @ 64      (1758-1759)
