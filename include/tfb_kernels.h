@@ -339,6 +339,17 @@ int tfb_moe_combine_bwd(const void* dout, const void* ys, const void* tok, const
 int tfb_moe_route_bwd(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot, const void* h,
                       const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate, long N, int d, int E, int topk,
                       void* stream);
+/* tfb_moe_route_bwd with the gradient of the auxiliary router terms folded into dlogits: the weighted sum
+ * alpha lb + beta z of tfb_moe_aux_fwd received the gradient *gaux (device fp32 scalar); terms, lse as that call left them. */
+int tfb_moe_route_bwd_aux(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot, const void* h,
+                          const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate, const void* terms,
+                          const void* lse, const void* gaux, float alpha, float beta, long N, int d, int E, int topk, void* stream);
+/* The router's auxiliary loss terms: terms fp32 [2 + E] = (lb = E sum_e f_e P_e, z = mean_n logsumexp(logits_n)^2, f_e),
+ * f_e = cnt_e / (N topk) the share of the assignments that chose e (cnt: the slot tables' counts; no gradient), P_e the
+ * mean router probability; lse fp32 [N] is kept for the backward; scratch fp32 [64 * 17].
+ * Replaces moe_aux_terms (round2/source/train.py:10779-10793); its per-sequence variant (R2_MOE_AUX_SEQ) is not built. */
+int tfb_moe_aux_fwd(const void* p, const void* logits, const void* cnt, void* terms, void* lse, void* scratch, long N, int E,
+                    int topk, void* stream);
 
 /* rows_out fp32 [E][16] = rows_in with the backward columns filled from each expert's amax over its rows of dys
  * (backward_scales per expert, round2/source/kernels/nki_mlp_fused8.py:803-813). amax_scratch: uint32 [E]. */

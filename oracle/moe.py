@@ -96,3 +96,16 @@ def moe_forward(h, router, w_fc, w_proj, topk, bias=None, fp8=True, e4m3_limit=2
     if topk == 2:
         out = out + gate[:, 1].to(dt).unsqueeze(-1) * ys.index_select(0, slot[:, 1])
     return out.reshape(h.shape), {"p": p, "idx": idx, "gate": gate, "slot": slot, "tok": tok, "seg": seg}
+
+
+def aux_terms(p, logits, idx, topk):
+    """(lb, z, f): the Switch load-balance term E sum_e f_e P_e (f_e the share of the k N assignments that chose e, no
+    gradient; P_e the mean router probability) and the router z term mean(logsumexp(logits)^2)
+    (round2/source/train.py:10779-10788 moe_aux_terms without its per-sequence variant)."""
+    N, E = p.shape
+    mall = torch.zeros(N, E, dtype=p.dtype)
+    mall.scatter_add_(1, idx.long(), torch.ones(idx.shape, dtype=p.dtype))
+    f = mall.mean(0) / topk
+    lb = E * (f * p.mean(0)).sum()
+    z = torch.logsumexp(logits, dim=-1).square().mean()
+    return lb, z, f

@@ -92,3 +92,32 @@ def test_moe_config5_full_size(dev):
         sl = slice(0, 512)
         oo, _ = O.moe_forward(h[sl], router, wf, wp, 2, bias if skew else None)
         assert rel_l2(out[sl], oo) < 2e-2
+
+
+def test_moe_auxiliary_router_terms(dev):
+    """moe_aux_terms (round2/source/train.py:10779): lb, z and the load shares against the oracle, and their gradient
+    joining the router's: with the layer output's gradient zero the router and input gradients are those of the weighted
+    auxiliary sum alone."""
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import autograd as A
+    N, d, Fd, E, topk = 2048, 256, 512, 8, 2
+    h, router, wf, wp, bias = _layer(5, N, d, Fd, E, 1.0)
+    hd, rd = h.to(dev).requires_grad_(True), router.to(dev).requires_grad_(True)
+    wfd, wpd = wf.to(dev).requires_grad_(True), wp.to(dev).requires_grad_(True)
+    st = A.Moe8State()
+    st.refresh(wfd, wpd)
+    alpha, beta = 0.01, 0.001
+    out, aux, terms = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, st, topk, bias.to(dev), (alpha, beta))
+    ho, ro = h.clone().float().requires_grad_(True), router.clone().float().requires_grad_(True)
+    po, idxo, _, lo = O.route(ho, ro, topk, bias)
+    lb, z, f = O.aux_terms(po, lo, idxo, topk)
+    assert abs(terms[0].item() - lb.item()) < 1e-4 * abs(lb.item()) and abs(terms[1].item() - z.item()) < 1e-4 * abs(z.item())
+    assert rel_l2(terms[2:], f) < 1e-3                                  # (a near-tie may select differently)
+    assert abs(aux.item() - (alpha * lb + beta * z).item()) < 1e-4 * abs(aux.item())
+    out0 = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, st, topk, bias.to(dev))
+    assert torch.equal(out, out0)                                       # the layer's output does not depend on the switch
+    (aux * 3.0).backward()
+    (3.0 * (alpha * lb + beta * z)).backward()
+    assert rel_l2(rd.grad, ro.grad) < 1e-2
+    assert rel_l2(hd.grad, ho.grad) < 2e-2                              # one bf16 rounding of dh
+    assert float(wfd.grad.abs().max()) == 0.0                           # no gradient reaches the experts through aux

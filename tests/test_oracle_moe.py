@@ -102,3 +102,31 @@ def test_backward_is_consistent_with_plain_autograd():
     o8.backward(g)
     o16.backward(g)
     assert rel_l2(hs[0].grad, hs[1].grad) < 0.2 and rel_l2(rs[0].grad, rs[1].grad) < 0.2
+
+
+def test_aux_terms_closed_forms_and_gradient():
+    """The auxiliary router terms: a uniform router gives lb = 1 and z = log(E)^2 whatever the selections; all tokens on
+    one expert with all probability there gives lb = E; the gradient of lb wrt the logits is the softmax Jacobian of
+    E f / N (f constant), checked by fp64 autograd."""
+    import math
+    from oracle import moe as O
+    N, E = 64, 8
+    logits = torch.zeros(N, E, dtype=torch.float64)
+    p = torch.softmax(logits, -1)
+    idx = torch.stack([torch.arange(N) % E, (torch.arange(N) + 1) % E], 1)
+    lb, z, f = O.aux_terms(p, logits, idx, 2)
+    assert abs(lb.item() - 1.0) < 1e-12 and abs(z.item() - math.log(E) ** 2) < 1e-12 and abs(f.sum().item() - 1.0) < 1e-12
+    logits = torch.full((N, E), -50.0, dtype=torch.float64)
+    logits[:, 3] = 50.0
+    lb, z, f = O.aux_terms(torch.softmax(logits, -1), logits, torch.full((N, 1), 3), 1)
+    assert abs(lb.item() - E) < 1e-9 and abs(z.item() - 2500.0) < 1e-6 and f[3] == 1.0
+    g = torch.Generator().manual_seed(0)
+    logits = torch.randn(N, E, generator=g, dtype=torch.float64, requires_grad=True)
+    p = torch.softmax(logits, -1)
+    idx = torch.topk(p, 2, dim=-1).indices
+    lb, z, f = O.aux_terms(p, logits, idx, 2)
+    (0.3 * lb + 0.7 * z).backward()
+    pd = p.detach()
+    dp = 0.3 * E * f / N
+    want = pd * (dp - (pd * dp).sum(-1, keepdim=True)) + 0.7 * 2.0 / N * torch.logsumexp(logits.detach(), -1, keepdim=True) * pd
+    assert torch.allclose(logits.grad, want, atol=1e-12)

@@ -599,24 +599,41 @@ class MoeMlp8Fn(torch.autograd.Function):
     w_fc [E, F, d], w_proj [E, d, F] bf16; router_bias fp32 [E] or None (added to the logits)."""
 
     @staticmethod
-    def forward(ctx, h, router, w_fc, w_proj, state, topk, router_bias):
+    def forward(ctx, h, router, w_fc, w_proj, state, topk, router_bias, aux_weights=None):
+        """aux_weights = (alpha, beta): also returns (aux, stats) with aux = alpha lb + beta z, the router's weighted
+        load-balance and z terms (round2/source/train.py:10779 moe_aux_terms; differentiable, its gradient joins the
+        router's in the backward), and stats fp32 [2 + E] = (lb, z, the experts' load shares f_e)."""
         h2 = h.reshape(-1, h.shape[-1]).contiguous()
         E, F, d = w_fc.shape
         wr = router.detach().float().contiguous()
-        p, idx, gate, _ = ops.moe_route(h2, wr, topk, router_bias)
+        p, idx, gate, logits = ops.moe_route(h2, wr, topk, router_bias, want_logits=aux_weights is not None)
         tab = ops.moe_tables(idx, E)
         xs, xs8 = ops.moe_gather(h2, tab, state.x_scale)
         ys, r = ops.moe_mlp8_fwd(xs8, state.w8, state.rows, tab, F)
         out = ops.moe_combine(ys, tab, gate, h2.shape[0])
-        ctx.save_for_backward(h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj)
-        ctx.tab, ctx.state, ctx.hshape = tab, state, h.shape
-        return out.view(h.shape)
+        ctx.tab, ctx.state, ctx.hshape, ctx.aux_weights = tab, state, h.shape, aux_weights
+        if aux_weights is None:
+            ctx.save_for_backward(h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj)
+            return out.view(h.shape)
+        terms, lse = ops.moe_aux_fwd(p, logits, tab, topk)
+        ctx.save_for_backward(h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj, terms, lse)
+        aux = float(aux_weights[0]) * terms[0] + float(aux_weights[1]) * terms[1]
+        ctx.mark_non_differentiable(terms)
+        return out.view(h.shape), aux, terms
 
     @staticmethod
-    def backward(ctx, gout):
-        h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj = ctx.saved_tensors
+    def backward(ctx, gout, gaux=None, _gterms=None):
+        if ctx.aux_weights is None:
+            h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj = ctx.saved_tensors
+            aux = None
+        else:
+            h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj, terms, lse = ctx.saved_tensors
+            ga = torch.zeros(1, dtype=torch.float32, device=h2.device) if gaux is None else gaux.reshape(1).float().contiguous()
+            aux = (terms, lse, ga, ctx.aux_weights[0], ctx.aux_weights[1])
         tab, st = ctx.tab, ctx.state
         E = w_fc.shape[0]
+        if gout is None:
+            gout = torch.zeros(ctx.hshape, dtype=h2.dtype, device=h2.device)
         g2 = gout.reshape(-1, gout.shape[-1]).contiguous()
         dys, dgate = ops.moe_combine_bwd(g2, ys, tab, gate)
         rows_b = ops.moe_backward_scales(dys, st.rows, tab)
@@ -629,5 +646,5 @@ class MoeMlp8Fn(torch.autograd.Function):
         else:
             dw_fc, dw_proj = ops.moe_dw(dpre, xs, dys, r, tab, E)
         br, accr = _accumulate_into(router)
-        dh, dwr, _ = ops.moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, br, accr)
-        return dh.view(ctx.hshape), (None if br is not None else dwr.to(router.dtype)), dw_fc, dw_proj, None, None, None
+        dh, dwr, _ = ops.moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, br, accr, aux=aux)
+        return dh.view(ctx.hshape), (None if br is not None else dwr.to(router.dtype)), dw_fc, dw_proj, None, None, None, None

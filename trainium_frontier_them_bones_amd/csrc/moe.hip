@@ -274,9 +274,14 @@ __global__ __launch_bounds__(256) void moe_combine_bwd_kernel(const bf16_t* __re
 }
 
 // dlogits[n][e] = p_e (dp_e - sum_j p_j dp_j), dp from the gate gradients through the renormalisation.
+// With the auxiliary router terms (terms != NULL: [0] lb, [1] z, [2..] f_e as left by moe_aux_finish_kernel; lse[n]; g =
+// *gaux, the gradient arriving at the weighted sum alpha lb + beta z): dp_e += g alpha (E / N) f_e (f carries no
+// gradient) and, after the softmax Jacobian, dlogits_e += g beta (2 / N) lse_n p_e.
 __global__ __launch_bounds__(256) void moe_dlogits_kernel(const float* __restrict__ dgate, const float* __restrict__ p,
                                                          const int* __restrict__ idx, float* __restrict__ dlogits, long N,
-                                                         int E, int topk) {
+                                                         int E, int topk, const float* __restrict__ terms,
+                                                         const float* __restrict__ lse, const float* __restrict__ gaux,
+                                                         float alpha, float beta) {
   long n = (long)blockIdx.x * 256 + threadIdx.x;
   if (n >= N) return;
   float dp[MAXE];
@@ -293,9 +298,69 @@ __global__ __launch_bounds__(256) void moe_dlogits_kernel(const float* __restric
     const int i1 = idx[n];
     for (int e = 0; e < E; ++e) dp[e] = e == i1 ? dgate[n] : 0.f;
   }
+  float zc = 0.f;
+  if (terms) {
+    const float g = *gaux;
+    const float ca = g * alpha * (float)E / (float)N;
+    for (int e = 0; e < E; ++e) dp[e] += ca * terms[2 + e];
+    zc = g * beta * 2.0f / (float)N * lse[n];
+  }
   float dot = 0.f;
   for (int e = 0; e < E; ++e) dot += p[n * E + e] * dp[e];
-  for (int e = 0; e < E; ++e) dlogits[n * E + e] = p[n * E + e] * (dp[e] - dot);
+  for (int e = 0; e < E; ++e) dlogits[n * E + e] = p[n * E + e] * (dp[e] - dot + zc);
+}
+
+// Auxiliary router terms (round2/source/train.py:10779 moe_aux_terms): partial column sums of p and of lse^2, lse[n] =
+// logsumexp(logits[n]); part [gridDim.x][MAXE + 1].
+__global__ __launch_bounds__(256) void moe_aux_partial_kernel(const float* __restrict__ p, const float* __restrict__ logits,
+                                                             float* __restrict__ lse_out, float* __restrict__ part, long N,
+                                                             int E) {
+  __shared__ float red[4][MAXE + 1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float acc[MAXE + 1];
+#pragma unroll
+  for (int e = 0; e <= MAXE; ++e) acc[e] = 0.f;
+  for (long n = (long)blockIdx.x * 256 + threadIdx.x; n < N; n += (long)gridDim.x * 256) {
+    float mx = -INFINITY;
+    for (int e = 0; e < E; ++e) mx = fmaxf(mx, logits[n * E + e]);
+    float den = 0.f;
+    for (int e = 0; e < E; ++e) den += expf(logits[n * E + e] - mx);
+    const float l = mx + logf(den);
+    lse_out[n] = l;
+    acc[MAXE] += l * l;
+#pragma unroll
+    for (int e = 0; e < MAXE; ++e)
+      if (e < E) acc[e] += p[n * E + e];
+  }
+#pragma unroll
+  for (int e = 0; e <= MAXE; ++e) {
+    const float v = wave_sum(acc[e]);
+    if (lane == 0) red[wave][e] = v;
+  }
+  __syncthreads();
+  if (threadIdx.x <= MAXE)
+    part[(long)blockIdx.x * (MAXE + 1) + threadIdx.x] = red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x];
+}
+// terms[0] = lb = E sum_e f_e P_e, terms[1] = z = mean lse^2, terms[2 + e] = f_e = cnt_e / (N topk), P_e = mean_n p[n][e]
+__global__ void moe_aux_finish_kernel(const float* __restrict__ part, int nparts, const int* __restrict__ cnt,
+                                      float* __restrict__ terms, long N, int E, int topk) {
+  __shared__ float tot[MAXE + 1];
+  if (threadIdx.x <= MAXE) {
+    float s = 0.f;
+    for (int b = 0; b < nparts; ++b) s += part[(long)b * (MAXE + 1) + threadIdx.x];
+    tot[threadIdx.x] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float lb = 0.f;
+    for (int e = 0; e < E; ++e) {
+      const float f = (float)cnt[e] / ((float)N * (float)topk);
+      terms[2 + e] = f;
+      lb += f * (tot[e] / (float)N);
+    }
+    terms[0] = (float)E * lb;
+    terms[1] = tot[MAXE] / (float)N;
+  }
 }
 
 // dh[n] = dxs[slot1] + dxs[slot2] + sum_e dlogits[n][e] Wr[e] (fp32 sum, one rounding).
@@ -539,20 +604,58 @@ extern "C" int tfb_moe_combine_bwd(const void* dout, const void* ys, const void*
 
 // Router backward + dispatch backward: dlogits fp32 [N][E] (scratch/output), dh bf16 [N][d] = dxs[slots] + dlogits Wr,
 // dwr fp32 [E][d] (+)= dlogits^T h. Replaces MoeDispatch2.backward (10662-10666) and autograd through moe_route.
-extern "C" int tfb_moe_route_bwd(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot,
-                                 const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate, long N,
-                                 int d, int E, int topk, void* stream) {
+static int moe_route_bwd_impl(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot,
+                              const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate, long N,
+                              int d, int E, int topk, const void* terms, const void* lse, const void* gaux, float alpha,
+                              float beta, void* stream) {
   if (!dgate || !p || !idx || !dxs || !slot || !h || !wr || !dlogits || !dh || !dwr) return TFB_ERR_ARG;
   if (N <= 0 || d <= 0 || d % 64 || E < 2 || E > MAXE || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(moe_dlogits_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, (const float*)dgate,
-                     (const float*)p, (const int*)idx, (float*)dlogits, N, E, topk);
+                     (const float*)p, (const int*)idx, (float*)dlogits, N, E, topk, (const float*)terms, (const float*)lse,
+                     (const float*)gaux, alpha, beta);
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(moe_dispatch_bwd_kernel, dim3(nblocks(N * (d / 8))), dim3(256), 0, s, (const bf16_t*)dxs, (const int*)slot,
                      (const float*)dlogits, (const float*)wr, (bf16_t*)dh, N, d, E, topk);
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(moe_dwr_kernel, dim3(d / 64), dim3(256), 0, s, (const float*)dlogits, (const bf16_t*)h, (float*)dwr, N, d, E,
                      dwr_accumulate);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+extern "C" int tfb_moe_route_bwd(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot,
+                                 const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate, long N,
+                                 int d, int E, int topk, void* stream) {
+  return moe_route_bwd_impl(dgate, p, idx, dxs, slot, h, wr, dlogits, dh, dwr, dwr_accumulate, N, d, E, topk, nullptr, nullptr,
+                            nullptr, 0.f, 0.f, stream);
+}
+// tfb_moe_route_bwd with the gradient of the auxiliary router terms folded into dlogits: the weighted sum
+// alpha lb + beta z of tfb_moe_aux_fwd received the gradient *gaux (device fp32 scalar); terms and lse as that call left them.
+extern "C" int tfb_moe_route_bwd_aux(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot,
+                                     const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate,
+                                     const void* terms, const void* lse, const void* gaux, float alpha, float beta, long N, int d,
+                                     int E, int topk, void* stream) {
+  if (!terms || !lse || !gaux) return TFB_ERR_ARG;
+  return moe_route_bwd_impl(dgate, p, idx, dxs, slot, h, wr, dlogits, dh, dwr, dwr_accumulate, N, d, E, topk, terms, lse, gaux,
+                            alpha, beta, stream);
+}
+
+// The router's auxiliary terms: terms fp32 [2 + E] = (lb = E sum_e f_e P_e, z = mean_n logsumexp(logits_n)^2, f_e) with
+// f_e = cnt_e / (N topk) the share of the assignments that chose e (from the slot tables' counts) and P_e the mean
+// router probability; lse fp32 [N] (kept for the backward); scratch: fp32 [64][17].
+// Replaces moe_aux_terms (round2/source/train.py:10779-10793; its per-sequence variant is not built).
+extern "C" int tfb_moe_aux_fwd(const void* p, const void* logits, const void* cnt, void* terms, void* lse, void* scratch, long N,
+                               int E, int topk, void* stream) {
+  if (!p || !logits || !cnt || !terms || !lse || !scratch) return TFB_ERR_ARG;
+  if (N <= 0 || E < 2 || E > MAXE || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const int nb = (int)((N + 255) / 256 < 64 ? (N + 255) / 256 : 64);
+  hipLaunchKernelGGL(moe_aux_partial_kernel, dim3(nb), dim3(256), 0, s, (const float*)p, (const float*)logits, (float*)lse,
+                     (float*)scratch, N, E);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_aux_finish_kernel, dim3(1), dim3(64), 0, s, (const float*)scratch, nb, (const int*)cnt, (float*)terms, N,
+                     E, topk);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

@@ -794,8 +794,9 @@ def moe_combine_bwd(dout, ys, tab, gate):
     return dys, dgate
 
 
-def moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, dwr=None, accumulate=False):
-    """(dh bf16 [N,d], dwr fp32 [E,d], dlogits fp32 [N,E])."""
+def moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, dwr=None, accumulate=False, aux=None):
+    """(dh bf16 [N,d], dwr fp32 [E,d], dlogits fp32 [N,E]). aux = (terms, lse, gaux, alpha, beta): the gradient gaux
+    (1-element fp32 device tensor) of the weighted auxiliary terms alpha lb + beta z of moe_aux_fwd is folded into dlogits."""
     N, d = h2.shape
     E = wr.shape[0]
     dlogits = torch.empty(N, E, dtype=torch.float32, device=h2.device)
@@ -803,9 +804,28 @@ def moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, dwr=None, accumulate=False):
     if dwr is None:
         dwr = torch.empty(E, d, dtype=torch.float32, device=h2.device)
         accumulate = False
-    _lib.call("tfb_moe_route_bwd", _p(dgate), _p(p), _p(idx), _p(dxs), _p(tab["slot"]), _p(h2), _p(wr), _p(dlogits), _p(dh),
-              _p(dwr), int(accumulate), N, d, E, idx.shape[1], _stream())
+    if aux is None:
+        _lib.call("tfb_moe_route_bwd", _p(dgate), _p(p), _p(idx), _p(dxs), _p(tab["slot"]), _p(h2), _p(wr), _p(dlogits), _p(dh),
+                  _p(dwr), int(accumulate), N, d, E, idx.shape[1], _stream())
+    else:
+        terms, lse, gaux, alpha, beta = aux
+        _chk(terms, torch.float32), _chk(lse, torch.float32), _chk(gaux, torch.float32)
+        _lib.call("tfb_moe_route_bwd_aux", _p(dgate), _p(p), _p(idx), _p(dxs), _p(tab["slot"]), _p(h2), _p(wr), _p(dlogits),
+                  _p(dh), _p(dwr), int(accumulate), _p(terms), _p(lse), _p(gaux), float(alpha), float(beta), N, d, E,
+                  idx.shape[1], _stream())
     return dh, dwr, dlogits
+
+
+def moe_aux_fwd(p, logits, tab, topk):
+    """(terms fp32 [2 + E] = (lb, z, f_e), lse fp32 [N]): the router's load-balance term E sum_e f_e P_e, its z term
+    mean(logsumexp(logits)^2) and the experts' load shares (round2/source/train.py:10779 moe_aux_terms)."""
+    _chk(p, torch.float32), _chk(logits, torch.float32)
+    N, E = p.shape
+    terms = torch.empty(2 + E, dtype=torch.float32, device=p.device)
+    lse = torch.empty(N, dtype=torch.float32, device=p.device)
+    scr = torch.empty(64 * 17, dtype=torch.float32, device=p.device)
+    _lib.call("tfb_moe_aux_fwd", _p(p), _p(logits), _p(tab["cnt"]), _p(terms), _p(lse), _p(scr), N, E, topk, _stream())
+    return terms, lse
 
 
 # ------------------------------------------------------------------------------------------ Muon Newton-Schulz
