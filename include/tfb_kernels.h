@@ -255,6 +255,19 @@ int tfb_attn_bwd_rope(const void* q, const long* q_strides, const void* k, const
                       void* dq, const long* dq_strides, void* dk, const long* dk_strides, void* dv, const long* dv_strides,
                       const void* lse, void* delta, const void* cos_t, const void* sin_t, int B, int H, int T, int D,
                       float scale, void* stream);
+/* The tile band of the reference's windowed layers (band_mask, round2/source/kernels/nki_attn_bandpro.py:1654-1658;
+ * kernels _attn_rope_fwd_kernel_band / _attn_rope_bwd_kernel_band, ops s2attn::rope_attn_fwd_band / _bwd_band
+ * round2/source/train.py:4925, 5040-5068): with nw > 0 a query of 128-token tile i sees the keys k <= q of tiles
+ * i - nw + 1 .. i only (the key loops start later / end earlier; the diagonal tile stays causally masked); nw = 0 is
+ * tfb_attn_fwd / tfb_attn_bwd_rope. Other arguments as there. */
+int tfb_attn_fwd_band(const void* q, const long* q_strides, const void* k, const long* k_strides, const void* v,
+                      const long* v_strides, void* o, const long* o_strides, void* lse, int B, int H, int T, int D, float scale,
+                      int nw, void* stream);
+int tfb_attn_bwd_band(const void* q, const long* q_strides, const void* k, const long* k_strides, const void* v,
+                      const long* v_strides, const void* o, const long* o_strides, const void* go, const long* go_strides,
+                      void* dq, const long* dq_strides, void* dk, const long* dk_strides, void* dv, const long* dv_strides,
+                      const void* lse, void* delta, const void* cos_t, const void* sin_t, int B, int H, int T, int D, float scale,
+                      int nw, void* stream);
 
 /* ---- loss head ------------------------------------------------------------------------------------------------------
  * loss[row] = row_w[row] * (lse - s_target), lse[row] = log sum exp(s), s = softcap tanh(x / softcap) (softcap <= 0:

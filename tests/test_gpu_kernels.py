@@ -406,6 +406,39 @@ def test_attention_growing_row_maximum(ops, dev, ramp):
     assert rel_l2(o, O.sdpa_reference(q, k, v, 0.125)) < BF16_TOL
 
 
+@pytest.mark.parametrize("shape,nw", [((1, 2, 1024, 64), 1), ((2, 2, 1024, 64), 3), ((1, 2, 1024, 64), 4), ((1, 1, 768, 128), 2),
+                                      ((1, 2, 512, 128), 4), ((1, 1, 512, 64), 9)])
+def test_attention_tile_band(ops, dev, shape, nw):
+    """The reference's windowed layers (band_mask, K/nki_attn_bandpro.py:1654): a query of 128-token tile i sees the keys
+    k <= q of tiles i - nw + 1 .. i. Forward and backward against the oracle with the same mask; a band as wide as the
+    sequence equals the full causal kernels bit for bit."""
+    from oracle import attention as O
+    B, H, T, D = shape
+    g = _g(T + D + nw)
+    q, k, v = (torch.randn(B, H, T, D, generator=g).bfloat16() for _ in range(3))
+    do = torch.randn(B, T, H, D, generator=g).bfloat16()
+    scale = 1.0 / math.sqrt(D)
+    qd, kd, vd, dod = q.to(dev), k.to(dev), v.to(dev), do.to(dev)
+    o, lse = ops.attn_fwd(qd, kd, vd, scale, band=nw)
+    oo, lo = O.forward(q, k, v, scale, band_tiles=nw)
+    assert rel_l2(o, oo) < BF16_TOL and rel_l2(lse, lo) < 1e-4
+    dq, dk, dv = ops.attn_bwd(qd, kd, vd, o, dod, lse, scale, band=nw)
+    dqo, dko, dvo = O.backward(q, k, v, o.cpu(), do, lse.cpu(), scale, band_tiles=nw)
+    assert rel_l2(dq, dqo) < BF16_TOL and rel_l2(dk, dko) < BF16_TOL and rel_l2(dv, dvo) < BF16_TOL
+    if nw * 128 >= T:
+        o2, lse2 = ops.attn_fwd(qd, kd, vd, scale)
+        dq2, dk2, dv2 = ops.attn_bwd(qd, kd, vd, o2, dod, lse2, scale)
+        assert torch.equal(o, o2) and torch.equal(lse, lse2) and torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
+    else:
+        # keys before the band do not matter: perturbing them changes nothing for the last tile's queries
+        k2, v2 = kd.clone(), vd.clone()
+        first = T - nw * 128
+        k2[:, :, :first] += 1.0
+        v2[:, :, :first] -= 1.0
+        o3, _ = ops.attn_fwd(qd, k2, v2, scale, band=nw)
+        assert torch.equal(o3[:, T - 128:], o[:, T - 128:])
+
+
 def test_attention_strided_qkv_and_rejects(ops, dev):
     from oracle import attention as O
     from trainium_frontier_them_bones_amd._lib import TfbError

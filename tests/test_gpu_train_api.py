@@ -370,3 +370,33 @@ def test_r1_fp8_rows(api, dev):
     assert rel_l2(p1.grad, g1.float() + dw1o.float()) < 2e-2 and rel_l2(p2.grad, g1.float() + dw2o.float()) < 2e-2
     assert rel_l2(p1.grad.float() - g1.to(dev).float(), dw1o) < 5e-2       # the row-5 product itself, not hidden by g1
     assert api.nki_gemm_fp8.active(True) and not api.nki_gemm_fp8.active(False)
+
+
+def test_band_attention_through_the_reference_calls(api, dev):
+    """nki_causal_attention(..., nw) and nki_rope_attention(..., nw) (R2:4925 fused_rope_attention_band) against the
+    oracle's composition with the band mask (K/nki_attn_bandpro.py:1654), forward and gradients."""
+    from oracle import attention as O
+    g = _g(16)
+    B, H, T, D, nw = 1, 2, 512, 128, 2
+    qkv = torch.randn(B, T, 3 * H * D, generator=g).bfloat16()
+    cos, sin = O.rope_tables(T, D)
+    qd = qkv.to(dev).requires_grad_(True)
+    y = api.nki_rope_attention(qd, cos.to(dev), sin.to(dev), H, nw=nw)
+    gy = torch.randn(B, T, H, D, generator=g).bfloat16()
+    y.backward(gy.to(dev))
+    q, k, v = (t.view(B, T, H, D) for t in qkv.split(H * D, dim=-1))
+    qn, rq, iq = O.rope_norm(q, cos, sin)
+    kn, rk, ik = O.rope_norm(k, cos, sin)
+    q4, k4, v4 = qn.permute(0, 2, 1, 3), kn.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3)
+    scale = 1.0 / math.sqrt(D)
+    yo, lo = O.forward(q4, k4, v4, scale, band_tiles=nw)
+    assert y.shape == (B, T, H, D) and rel_l2(y, yo) < BF16_TOL
+    dq4, dk4, dv4 = O.backward(q4, k4, v4, yo, gy, lo, scale, band_tiles=nw)
+    dq = O.rope_norm_backward(dq4.permute(0, 2, 1, 3), rq, iq, cos, sin)
+    dk = O.rope_norm_backward(dk4.permute(0, 2, 1, 3), rk, ik, cos, sin)
+    want = torch.cat([t.reshape(B, T, H * D) for t in (dq, dk, dv4.permute(0, 2, 1, 3))], dim=-1)
+    assert rel_l2(qd.grad, want) < 2 * BF16_TOL
+    q64 = torch.randn(1, 2, 512, 64, generator=g).bfloat16().to(dev)
+    a = api.nki_causal_attention(q64, q64, q64, nw=4)
+    b = api.nki_causal_attention(q64, q64, q64)
+    assert torch.equal(a, b)                                                     # a band as wide as the sequence

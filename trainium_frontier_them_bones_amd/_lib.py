@@ -41,6 +41,9 @@ SIGNATURES = {
     "tfb_gemm_fp8_tn": [_vp, _i, _vp, _i, _vp, _vp, _f, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
     "tfb_mlp8_dw8": [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
     "tfb_attn_fwd": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _i, _i, _i, _i, _f, _vp],
+    "tfb_attn_fwd_band": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _i, _i, _i, _i, _f, _i, _vp],
+    "tfb_attn_bwd_band": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _vp, _vp, _vp,
+                          _i, _i, _i, _i, _f, _i, _vp],
     "tfb_attn_bwd": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _vp, _i, _i, _i, _i,
                      _f, _vp],
     "tfb_attn_bwd_rope": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _vp, _vp, _vp,

@@ -168,18 +168,19 @@ class CausalAttentionFn(torch.autograd.Function):
     """nki_causal_attention(q, k, v, scale): q, k, v [B, H, T, D] -> [B, T, H, D] (round1/source/train.py:8069)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, scale):
+    def forward(ctx, q, k, v, scale, band=0):
+        """band = nw > 0: the reference's tile band (K/nki_attn_bandpro.py:1654): keys of the last nw 128-token tiles."""
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        o, lse = ops.attn_fwd(q, k, v, scale, "bhtd")
+        o, lse = ops.attn_fwd(q, k, v, scale, "bhtd", band)
         ctx.save_for_backward(q, k, v, o, lse)
-        ctx.scale = scale
+        ctx.scale, ctx.band = scale, band
         return o
 
     @staticmethod
     def backward(ctx, go):
         q, k, v, o, lse = ctx.saved_tensors
-        dq, dk, dv = ops.attn_bwd(q, k, v, o, go.contiguous(), lse, ctx.scale, "bhtd")
-        return dq, dk, dv, None
+        dq, dk, dv = ops.attn_bwd(q, k, v, o, go.contiguous(), lse, ctx.scale, "bhtd", band=ctx.band)
+        return dq, dk, dv, None, None
 
 
 class RopeAttentionFn(torch.autograd.Function):
@@ -246,7 +247,8 @@ class RopeNormAttentionFn(torch.autograd.Function):
     strides; saved for backward: qkv's v third, the rotated q, k (r5), their inverse RMS (inv3), o, lse."""
 
     @staticmethod
-    def forward(ctx, qkv, cos, sin, n_head, scale, eps):
+    def forward(ctx, qkv, cos, sin, n_head, scale, eps, band=0):
+        """band = nw > 0: the tile-band form (round2/source/train.py:4925 fused_rope_attention_band)."""
         B, T, C3 = qkv.shape
         C = C3 // 3
         D = C // n_head
@@ -254,9 +256,9 @@ class RopeNormAttentionFn(torch.autograd.Function):
         qk, r, inv = ops.rope_norm_fwd(qkv.view(B * T, C3), cos, sin, T, 2 * n_head, D, eps)
         q, k = (t.view(B, T, n_head, D) for t in qk.view(B, T, 2 * C).split(C, dim=-1))
         v = qkv[..., 2 * C:].view(B, T, n_head, D)
-        o, lse = ops.attn_fwd(q, k, v, scale, "bthd")
+        o, lse = ops.attn_fwd(q, k, v, scale, "bthd", band)
         ctx.save_for_backward(qkv, qk, r, inv, o, lse, cos, sin)
-        ctx.n_head, ctx.scale = n_head, scale
+        ctx.n_head, ctx.scale, ctx.band = n_head, scale, band
         return o.view(B, T, C)
 
     @staticmethod
@@ -270,10 +272,10 @@ class RopeNormAttentionFn(torch.autograd.Function):
         v = qkv[..., 2 * C:].view(B, T, H, D)
         dqkv = torch.empty_like(qkv)
         dq, dk, dv = (t.view(B, T, H, D) for t in dqkv.split(C, dim=-1))
-        ops.attn_bwd(q, k, v, o, go.contiguous().view(B, T, H, D), lse, ctx.scale, "bthd", dq, dk, dv, "bthd")
+        ops.attn_bwd(q, k, v, o, go.contiguous().view(B, T, H, D), lse, ctx.scale, "bthd", dq, dk, dv, "bthd", band=ctx.band)
         g2 = dqkv.view(B * T, C3)
         ops.rope_norm_bwd(g2, r, inv, cos, sin, T, 2 * H, D, out=g2)   # in place on the q and k thirds
-        return dqkv, None, None, None, None, None
+        return dqkv, None, None, None, None, None, None
 
 
 class QkvRopeAttentionFn(torch.autograd.Function):

@@ -103,7 +103,7 @@ constexpr int TROW = 64 * 2 + 8;
 // traffic per flop) and the two groups' softmax arithmetic and MFMAs are independent instruction streams that co-execute.
 template <int D, int QG>
 __global__ __launch_bounds__(256, (D == 64 && QG == 1) ? TFB_FWD_WPE : 1) void attn_fwd_kernel(AttnT q, AttnT k, AttnT v, AttnT o, float* __restrict__ lse, int T,
-                                                      int H, float sl2) {
+                                                      int H, float sl2, int nw) {
   constexpr int DS = D / 16, DT = D / 32, NV = D / 64;
   constexpr int KROW = D * 2 + 16;
   constexpr int KBYTES = 64 * KROW, VBYTES = D * TROW, BUF = KBYTES + VBYTES;
@@ -175,12 +175,14 @@ __global__ __launch_bounds__(256, (D == 64 && QG == 1) ? TFB_FWD_WPE : 1) void a
       for (int e = 0; e < 16; ++e) oacc[g][i][e] = 0.f;
   }
 
-  gload(0);
+  // band (nw > 0, QG = 1): the queries of 128-token tile qb see key tiles qb - nw + 1 .. qb only
+  const int t0 = nw > 0 ? 2 * (qb - nw + 1 > 0 ? qb - nw + 1 : 0) : 0;
+  gload(t0);
   sstore(smem);
   wait_all_loads();
   __syncthreads();
 
-  for (int t = 0; t < ntiles; ++t) {
+  for (int t = t0; t < ntiles; ++t) {
     const uint8_t* cur = smem + (t & 1) * BUF;
     const bool more = t + 1 < ntiles;
     if (more) gload(t + 1);
@@ -307,7 +309,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(AttnT o, AttnT go, floa
 template <int D>
 __global__ __launch_bounds__(256, D == 64 ? TFB_DKDV_WPE : 1) void attn_bwd_dkdv_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dk, AttnT dv,
                                                            const float* __restrict__ lse, const float* __restrict__ delta,
-                                                           int T, int H, float scale, float sl2) {
+                                                           int T, int H, float scale, float sl2, int nw) {
   constexpr int DS = D / 16, DT = D / 32, NV = D / 64;
   constexpr int KROW = D * 2 + 16;
   constexpr int NBYTES = 64 * KROW, TBYTES = D * TROW;
@@ -332,7 +334,8 @@ __global__ __launch_bounds__(256, D == 64 ? TFB_DKDV_WPE : 1) void attn_bwd_dkdv
     vf[s] = *(const bf16x8*)(vp + (long)mykey * v.st + 16 * s + 8 * lh);
   }
 
-  const int qt0 = kb * 2, nqt = T / 64;
+  // band (nw > 0): key tile kb is seen by the queries of tiles kb .. kb + nw - 1 only
+  const int qt0 = kb * 2, nqt = nw > 0 && (kb + nw) * 2 < T / 64 ? (kb + nw) * 2 : T / 64;
   const bool qrole = wave < 2;
   const int t2 = tid & 127;
   MicroBlock mb[NV];
@@ -454,7 +457,7 @@ __global__ __launch_bounds__(256, D == 64 ? TFB_DKDV_WPE : 1) void attn_bwd_dkdv
 template <int D>
 __global__ __launch_bounds__(256, D == 64 ? TFB_DQ_WPE : 1) void attn_bwd_dq_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dq,
                                                          const float* __restrict__ lse, const float* __restrict__ delta,
-                                                         int T, int H, float scale, float sl2) {
+                                                         int T, int H, float scale, float sl2, int nw) {
   constexpr int DS = D / 16, DT = D / 32, NV = D / 64;
   constexpr int KROW = D * 2 + 16;
   constexpr int NBYTES = 64 * KROW, TBYTES = D * TROW;
@@ -524,12 +527,13 @@ __global__ __launch_bounds__(256, D == 64 ? TFB_DQ_WPE : 1) void attn_bwd_dq_ker
 #pragma unroll
     for (int e = 0; e < 16; ++e) dqa[i][e] = 0.f;
 
-  gload(0);
+  const int t0 = nw > 0 ? 2 * (qb - nw + 1 > 0 ? qb - nw + 1 : 0) : 0;  // band: key tiles qb - nw + 1 .. qb
+  gload(t0);
   sstore(smem);
   wait_all_loads();
   __syncthreads();
 
-  for (int t = 0; t < ntiles; ++t) {
+  for (int t = t0; t < ntiles; ++t) {
     const uint8_t* cur = smem + (TFB_BWD_NBUF == 2 ? (t & 1) * BUF : 0);
     const bool more = t + 1 < ntiles;
     if (more) gload(t + 1);
@@ -599,7 +603,7 @@ AttnT mk(const void* p, const long* s) { return AttnT{(bf16_t*)p, s[0], s[1], s[
 bool strides_ok(const long* s) { return s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0; }
 
 template <int D, int QG>
-int fwd_launch(AttnT q, AttnT k, AttnT v, AttnT o, float* lse, int B, int H, int T, float scale, hipStream_t s) {
+int fwd_launch(AttnT q, AttnT k, AttnT v, AttnT o, float* lse, int B, int H, int T, float scale, int nw, hipStream_t s) {
   constexpr int BUF = 64 * (D * 2 + 16) + D * TROW;
   static bool once = false;
   if (!once) {
@@ -607,21 +611,23 @@ int fwd_launch(AttnT q, AttnT k, AttnT v, AttnT o, float* lse, int B, int H, int
     once = true;
   }
   hipLaunchKernelGGL((attn_fwd_kernel<D, QG>), dim3(T / (128 * QG), B * H), dim3(256), 2 * BUF, s, q, k, v, o, lse, T, H,
-                     scale * LOG2E);
+                     scale * LOG2E, nw);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
 
 template <int D>
-int fwd_impl(AttnT q, AttnT k, AttnT v, AttnT o, float* lse, int B, int H, int T, float scale, hipStream_t s) {
-  // two query groups per wavefront when the sequence splits into 256-query blocks and the registers allow (D = 64)
-  if (TFB_FWD_QG2 && D == 64 && T % 256 == 0) return fwd_launch<D, (D == 64 ? 2 : 1)>(q, k, v, o, lse, B, H, T, scale, s);
-  return fwd_launch<D, 1>(q, k, v, o, lse, B, H, T, scale, s);
+int fwd_impl(AttnT q, AttnT k, AttnT v, AttnT o, float* lse, int B, int H, int T, float scale, int nw, hipStream_t s) {
+  // two query groups per wavefront when the sequence splits into 256-query blocks and the registers allow (D = 64);
+  // a band needs one 128-token tile per workgroup
+  if (TFB_FWD_QG2 && D == 64 && T % 256 == 0 && nw <= 0)
+    return fwd_launch<D, (D == 64 ? 2 : 1)>(q, k, v, o, lse, B, H, T, scale, 0, s);
+  return fwd_launch<D, 1>(q, k, v, o, lse, B, H, T, scale, nw, s);
 }
 
 template <int D>
 int bwd_impl(AttnT q, AttnT k, AttnT v, AttnT o, AttnT go, AttnT dq, AttnT dk, AttnT dv, const float* lse, float* delta, int B,
-             int H, int T, float scale, hipStream_t s) {
+             int H, int T, float scale, int nw, hipStream_t s) {
   constexpr int NB = 64 * (D * 2 + 16), TB = D * TROW;
   constexpr int BUF1 = 2 * NB + 2 * TB + 512, BUF2 = 2 * NB + TB;
   static bool once = false;
@@ -634,10 +640,10 @@ int bwd_impl(AttnT q, AttnT k, AttnT v, AttnT o, AttnT go, AttnT dq, AttnT dk, A
   hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((unsigned)((rows * 4 + 255) / 256)), dim3(256), 0, s, o, go, delta, T, H, rows);
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(attn_bwd_dkdv_kernel<D>, dim3(T / 128, B * H), dim3(256), TFB_BWD_NBUF * BUF1, s, q, k, v, go, dk, dv, lse, delta, T, H,
-                     scale, scale * LOG2E);
+                     scale, scale * LOG2E, nw);
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(attn_bwd_dq_kernel<D>, dim3(T / 128, B * H), dim3(256), TFB_BWD_NBUF * BUF2, s, q, k, v, go, dq, lse, delta, T, H, scale,
-                     scale * LOG2E);
+                     scale * LOG2E, nw);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
@@ -646,36 +652,44 @@ int bwd_impl(AttnT q, AttnT k, AttnT v, AttnT o, AttnT go, AttnT dq, AttnT dk, A
 
 // D = 64 runs the kernels of attention64.hip (direct-to-LDS tile loads, transposed LDS fragment reads).
 int tfb_attn64_fwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs, void* o,
-                        const long* os, float* lse, int B, int H, int T, float scale, hipStream_t s);
+                        const long* os, float* lse, int B, int H, int T, float scale, int nw, hipStream_t s);
 int tfb_attn64_bwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
                         const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs, void* dk,
                         const long* dks, void* dv, const long* dvs, const float* lse, float* stats, int B, int H, int T,
-                        float scale, const void* cos_t, const void* sin_t, hipStream_t s);
+                        float scale, const void* cos_t, const void* sin_t, int nw, hipStream_t s);
 
 // Every tensor argument comes with long[3] element strides (batch, head, token); the head dimension is contiguous.
 // lse: fp32 [B*H][T].
-extern "C" int tfb_attn_fwd(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs, void* o,
-                            const long* os, void* lse, int B, int H, int T, int D, float scale, void* stream) {
+// nw > 0: the tile band of the reference's windowed layers (band_mask, round2/source/kernels/nki_attn_bandpro.py:1654):
+// a query of 128-token tile i sees the keys k <= q of tiles i - nw + 1 .. i; nw = 0: all keys k <= q.
+extern "C" int tfb_attn_fwd_band(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
+                                 void* o, const long* os, void* lse, int B, int H, int T, int D, float scale, int nw,
+                                 void* stream) {
   if (!q || !k || !v || !o || !lse || !qs || !ks || !vs || !os) return TFB_ERR_ARG;
-  if (B <= 0 || H <= 0 || T <= 0 || T % 128 || (D != 64 && D != 128)) return TFB_ERR_SHAPE;
+  if (B <= 0 || H <= 0 || T <= 0 || T % 128 || (D != 64 && D != 128) || nw < 0) return TFB_ERR_SHAPE;
   if (!strides_ok(qs) || !strides_ok(ks) || !strides_ok(vs) || !strides_ok(os)) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
-  if (D == 64) return tfb_attn64_fwd_impl(q, qs, k, ks, v, vs, o, os, (float*)lse, B, H, T, scale, s);
-  return fwd_impl<128>(mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), (float*)lse, B, H, T, scale, s);
+  if (D == 64) return tfb_attn64_fwd_impl(q, qs, k, ks, v, vs, o, os, (float*)lse, B, H, T, scale, nw, s);
+  return fwd_impl<128>(mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), (float*)lse, B, H, T, scale, nw, s);
+}
+extern "C" int tfb_attn_fwd(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs, void* o,
+                            const long* os, void* lse, int B, int H, int T, int D, float scale, void* stream) {
+  return tfb_attn_fwd_band(q, qs, k, ks, v, vs, o, os, lse, B, H, T, D, scale, 0, stream);
 }
 
 // delta: fp32 [2][B*H][T] scratch (row dot products, then -lse log2 e). dq, dk, dv may alias thirds of one dqkv buffer.
 // cos_t / sin_t (bf16 [T][D/2], both or neither): dq and dk come out with the inverse RoPE rotation applied, i.e. as
 // gradients of the projections the rotation was applied to (D = 64 only; otherwise TFB_ERR_SHAPE and the caller runs
 // tfb_rope itself).
-extern "C" int tfb_attn_bwd_rope(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
+extern "C" int tfb_attn_bwd_band(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
                                  const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs,
                                  void* dk, const long* dks, void* dv, const long* dvs, const void* lse, void* delta,
-                                 const void* cos_t, const void* sin_t, int B, int H, int T, int D, float scale, void* stream) {
+                                 const void* cos_t, const void* sin_t, int B, int H, int T, int D, float scale, int nw,
+                                 void* stream) {
   if (!q || !k || !v || !o || !go || !dq || !dk || !dv || !lse || !delta) return TFB_ERR_ARG;
   if (!qs || !ks || !vs || !os || !gos || !dqs || !dks || !dvs) return TFB_ERR_ARG;
   if ((cos_t == nullptr) != (sin_t == nullptr)) return TFB_ERR_ARG;
-  if (B <= 0 || H <= 0 || T <= 0 || T % 128 || (D != 64 && D != 128)) return TFB_ERR_SHAPE;
+  if (B <= 0 || H <= 0 || T <= 0 || T % 128 || (D != 64 && D != 128) || nw < 0) return TFB_ERR_SHAPE;
   if (cos_t && D != 64) return TFB_ERR_SHAPE;
   if (!strides_ok(qs) || !strides_ok(ks) || !strides_ok(vs) || !strides_ok(os) || !strides_ok(gos) || !strides_ok(dqs) ||
       !strides_ok(dks) || !strides_ok(dvs))
@@ -683,9 +697,16 @@ extern "C" int tfb_attn_bwd_rope(const void* q, const long* qs, const void* k, c
   hipStream_t s = (hipStream_t)stream;
   if (D == 64)
     return tfb_attn64_bwd_impl(q, qs, k, ks, v, vs, o, os, go, gos, dq, dqs, dk, dks, dv, dvs, (const float*)lse, (float*)delta,
-                               B, H, T, scale, cos_t, sin_t, s);
+                               B, H, T, scale, cos_t, sin_t, nw, s);
   return bwd_impl<128>(mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), mk(go, gos), mk(dq, dqs), mk(dk, dks), mk(dv, dvs),
-                       (const float*)lse, (float*)delta, B, H, T, scale, s);
+                       (const float*)lse, (float*)delta, B, H, T, scale, nw, s);
+}
+extern "C" int tfb_attn_bwd_rope(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
+                                 const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs,
+                                 void* dk, const long* dks, void* dv, const long* dvs, const void* lse, void* delta,
+                                 const void* cos_t, const void* sin_t, int B, int H, int T, int D, float scale, void* stream) {
+  return tfb_attn_bwd_band(q, qs, k, ks, v, vs, o, os, go, gos, dq, dqs, dk, dks, dv, dvs, lse, delta, cos_t, sin_t, B, H, T, D,
+                           scale, 0, stream);
 }
 
 extern "C" int tfb_attn_bwd(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,

@@ -98,6 +98,9 @@ __device__ __forceinline__ int paired_block(int nx, int bx, int pass, bool heavy
   const int first = heavy_last ? nx - 1 - bx : bx;
   return pass == 0 ? first : nx - 1 - first;
 }
+// First 64-key tile a 128-token query tile qb sees under a band of nw key tiles (a query of tile i sees the keys k <= q
+// of tiles i - nw + 1 .. i: band_mask, round2/source/kernels/nki_attn_bandpro.py:1654); 0 without a band (nw <= 0).
+__device__ __forceinline__ int band_first_tile(int qb, int nw) { return nw > 0 && qb - nw + 1 > 0 ? 2 * (qb - nw + 1) : 0; }
 __host__ inline unsigned paired_grid(int nx) { return (unsigned)(nx % 2 == 0 ? nx / 2 : nx); }
 
 __device__ __forceinline__ int swz(int t) { return (((t >> 1) & 1) << 2) | ((t >> 2) & 3); }
@@ -190,7 +193,7 @@ __device__ __forceinline__ void store_grad_row(const f32x16 (&acc)[2], float sca
 
 // =========================================================================================== forward
 __global__ __launch_bounds__(256, TFB_FWD64_WPE) void attn64_fwd_kernel(AttnT q, AttnT k, AttnT v, AttnT o, float* __restrict__ lse,
-                                                            int T, int H, float sl2) {
+                                                            int T, int H, float sl2, int nw) {
   __shared__ __attribute__((aligned(1024))) uint8_t st0[2 * TILE];
   __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
@@ -365,12 +368,13 @@ __global__ __launch_bounds__(256, TFB_FWD64_WPE) void attn64_fwd_kernel(AttnT q,
   };
 
   const int n = (q0 + 128) / 64;  // even; tiles n - 2 and n - 1 cover the workgroup's own 128 tokens
-  issue(st0, 0);
+  const int t0 = band_first_tile(qb, nw);  // even; 0 without a band
+  issue(st0, t0);
   wait_all_loads();
   __syncthreads();
-  issue(st1, 1);
+  issue(st1, t0 + 1);
   scores(st0, scA);
-  for (int t = 0; t + 2 < n; t += 2) {
+  for (int t = t0; t + 2 < n; t += 2) {
     full_tile(st0, st1, t, scA, scB);
     full_tile(st1, st0, t + 1, scB, scA);
   }
@@ -435,7 +439,7 @@ __global__ __launch_bounds__(256) void attn64_delta_kernel(AttnT o, AttnT go, co
 __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dk, AttnT dv,
                                                              const float* __restrict__ stats, long rows, int T, int H,
                                                              float scale, float sl2, const bf16_t* __restrict__ cs,
-                                                             const bf16_t* __restrict__ sn) {
+                                                             const bf16_t* __restrict__ sn, int nw) {
   constexpr int QT = TFB_DKDV64_QT;       // 64-query tiles per LDS stage (one barrier per stage)
   constexpr int R = 64 * QT, RT = R * 128;  // rows and bytes of a staged Q (dO) tile
   constexpr int STAGE = 2 * RT + 8 * R;    // Q tile, dO tile, R x (-lse / scale), R x (-delta)
@@ -469,7 +473,9 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
   TileLoad<2 * QT> lq, lg;
   lq.init(qst, wave, lane);
   lg.init(gst, wave, lane);
-  const int qt0 = kb * 2, n = (T / 64 - qt0) / QT;  // T / 64 - 2 kb is even
+  // T / 64 - 2 kb is even; with a band the keys of tile kb are seen by the queries of tiles kb .. kb + nw - 1 only
+  const int qt0 = kb * 2, nall = (T / 64 - qt0) / QT, n = nw > 0 && nw < nall ? nw : nall;
+  static_assert(QT == 2, "a stage is one 128-token tile of queries");
   auto issue = [&](uint8_t* st, int i) {
     const long r0 = (long)qt0 * 64 + (long)i * R;
     lq.issue(qp + r0 * qst, qst, st);
@@ -592,7 +598,7 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
 __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dq,
                                                            const float* __restrict__ stats, long rows, int T, int H,
                                                            float scale, float sl2, const bf16_t* __restrict__ cs,
-                                                           const bf16_t* __restrict__ sn) {
+                                                           const bf16_t* __restrict__ sn, int nw) {
   __shared__ __attribute__((aligned(1024))) uint8_t st0[2 * TILE];
   __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
@@ -732,12 +738,13 @@ __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, A
   };
 
   const int n = (q0 + 128) / 64;  // even; tiles n - 2 and n - 1 cover the workgroup's own 128 tokens
-  issue(st0, 0);
+  const int t0 = band_first_tile(qb, nw);  // even; 0 without a band
+  issue(st0, t0);
   wait_all_loads();
   __syncthreads();
-  issue(st1, 1);
+  issue(st1, t0 + 1);
   scores(st0, 0, Sa, dPa);
-  for (int t = 0; t + 2 < n; t += 2) {
+  for (int t = t0; t + 2 < n; t += 2) {
     full_tile(st0, st1, t);
     full_tile(st1, st0, t + 1);
   }
@@ -757,9 +764,9 @@ AttnT mk(const void* p, const long* s) { return AttnT{(bf16_t*)p, s[0], s[1], s[
 
 // Called by tfb_attn_fwd / tfb_attn_bwd for D = 64 (arguments already validated there: T % 128 == 0, strides % 8 == 0).
 int tfb_attn64_fwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs, void* o,
-                        const long* os, float* lse, int B, int H, int T, float scale, hipStream_t s) {
+                        const long* os, float* lse, int B, int H, int T, float scale, int nw, hipStream_t s) {
   hipLaunchKernelGGL(attn64_fwd_kernel, dim3(paired_grid(T / 128), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), lse,
-                     T, H, scale * LOG2E);
+                     T, H, scale * LOG2E, nw);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
@@ -769,16 +776,16 @@ int tfb_attn64_fwd_impl(const void* q, const long* qs, const void* k, const long
 int tfb_attn64_bwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
                         const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs, void* dk,
                         const long* dks, void* dv, const long* dvs, const float* lse, float* stats, int B, int H, int T,
-                        float scale, const void* cos_t, const void* sin_t, hipStream_t s) {
+                        float scale, const void* cos_t, const void* sin_t, int nw, hipStream_t s) {
   const long rows = (long)B * H * T;
   hipLaunchKernelGGL(attn64_delta_kernel, dim3((unsigned)((rows * 4 + 255) / 256)), dim3(256), 0, s, mk(o, os), mk(go, gos), lse,
                      stats, T, H, rows, 1.0f / scale);
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(attn64_dkdv_kernel, dim3(paired_grid(T / 128), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
-                     mk(dk, dks), mk(dv, dvs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t);
+                     mk(dk, dks), mk(dv, dvs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t, nw);
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(attn64_dq_kernel, dim3(paired_grid(T / 128), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
-                     mk(dq, dqs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t);
+                     mk(dq, dqs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t, nw);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

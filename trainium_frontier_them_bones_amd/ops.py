@@ -443,9 +443,10 @@ def _attn_chk(t):
         raise TypeError("attention takes bf16 device tensors")
 
 
-def attn_fwd(q, k, v, scale, layout="bhtd"):
+def attn_fwd(q, k, v, scale, layout="bhtd", band=0):
     """q, k, v: 4-D views [B,H,T,D] ("bhtd") or [B,T,H,D] ("bthd"), arbitrary batch/head/token strides.
-    Returns o [B,T,H,D] contiguous and lse [B,H,T] fp32."""
+    Returns o [B,T,H,D] contiguous and lse [B,H,T] fp32. band = nw > 0: the reference's tile band (a query of 128-token
+    tile i sees the keys k <= q of tiles i - nw + 1 .. i; K/nki_attn_bandpro.py:1654); 0: all keys k <= q."""
     for t in (q, k, v):
         _attn_chk(t)
     if layout == "bhtd":
@@ -454,12 +455,12 @@ def attn_fwd(q, k, v, scale, layout="bhtd"):
         B, T, H, D = q.shape
     o = torch.empty(B, T, H, D, dtype=bf16, device=q.device)
     lse = torch.empty(B, H, T, dtype=torch.float32, device=q.device)
-    _lib.call("tfb_attn_fwd", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o), _bht(o, "bthd"),
-              _p(lse), B, H, T, D, float(scale), _stream())
+    _lib.call("tfb_attn_fwd_band", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o),
+              _bht(o, "bthd"), _p(lse), B, H, T, D, float(scale), int(band), _stream())
     return o, lse
 
 
-def attn_bwd(q, k, v, o, do, lse, scale, layout="bhtd", dq=None, dk=None, dv=None, out_layout="bhtd", rope=None):
+def attn_bwd(q, k, v, o, do, lse, scale, layout="bhtd", dq=None, dk=None, dv=None, out_layout="bhtd", rope=None, band=0):
     """Gradients of attn_fwd. o, do are [B,T,H,D]. dq/dk/dv may be given as (strided) views with `out_layout`;
     otherwise dq, dk are allocated [B,H,T,D] and dv [B,T,H,D] (returned as a [B,H,T,D] view), as the reference returns.
     rope = (cos, sin) (bf16 [T, D/2]): dq and dk come back with the inverse rotation applied (D = 64)."""
@@ -477,9 +478,9 @@ def attn_bwd(q, k, v, o, do, lse, scale, layout="bhtd", dq=None, dk=None, dv=Non
     delta = torch.empty(2, B, H, T, dtype=torch.float32, device=q.device)
     cos, sin = rope if rope is not None else (None, None)
     _chk(cos), _chk(sin)
-    _lib.call("tfb_attn_bwd_rope", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o),
+    _lib.call("tfb_attn_bwd_band", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o),
               _bht(o, "bthd"), _p(do), _bht(do, "bthd"), _p(dq), _bht(dq, out_layout), _p(dk), _bht(dk, out_layout), _p(dv),
-              _bht(dv, out_layout), _p(lse), _p(delta), _p(cos), _p(sin), B, H, T, D, float(scale), _stream())
+              _bht(dv, out_layout), _p(lse), _p(delta), _p(cos), _p(sin), B, H, T, D, float(scale), int(band), _stream())
     return dq, dk, dv
 
 

@@ -34,10 +34,12 @@ def _none_if_shape(fn, *args):
 
 
 # ------------------------------------------------------------------------------------------ attention (R1:8069-8210)
-def nki_causal_attention(q, k, v, scale=None):
-    """Causal SDPA(q, k, v) for [B, H, T, D] inputs, returned as [B, T, H, D] (R1:8069)."""
+def nki_causal_attention(q, k, v, scale=None, nw=None):
+    """Causal SDPA(q, k, v) for [B, H, T, D] inputs, returned as [B, T, H, D] (R1:8069). nw (the reference's band
+    kernels' last argument, K/nki_attn_bandpro.py:1654; R2:4925 fused_rope_attention_band): a query of 128-token tile i
+    sees the keys k <= q of tiles i - nw + 1 .. i only."""
     sc = float(scale) if scale is not None else 1.0 / math.sqrt(q.shape[-1])
-    return A.CausalAttentionFn.apply(q, k, v, sc)
+    return A.CausalAttentionFn.apply(q, k, v, sc, int(nw) if nw else 0)
 
 
 nki_attn_fn = nki_causal_attention   # R1:8207
@@ -59,9 +61,10 @@ def _tables_2d(cos, sin, T, half):
     return c, s
 
 
-def nki_rope_attention(qkv, cos, sin, n_head, scale=None):
+def nki_rope_attention(qkv, cos, sin, n_head, scale=None, nw=None):
     """y [B, T, H, D] = causal SDPA(QKnorm(RoPE(q)), QKnorm(RoPE(k)), v) straight from the fused projection output qkv
-    [B, T, 3C]; None when the fused path does not apply (R1:8197)."""
+    [B, T, 3C]; None when the fused path does not apply (R1:8197). nw: the tile band of the reference's windowed layers
+    (R2:4925 fused_rope_attention_band; kernels' last argument)."""
     if qkv.dim() != 3 or qkv.shape[-1] % (3 * n_head):
         return None
     B, T, C3 = qkv.shape
@@ -70,7 +73,7 @@ def nki_rope_attention(qkv, cos, sin, n_head, scale=None):
         return None
     sc = float(scale) if scale is not None else 1.0 / math.sqrt(D)
     c, s = _tables_2d(cos, sin, T, D // 2)
-    y = _none_if_shape(A.RopeNormAttentionFn.apply, qkv, c, s, n_head, sc, RMS_EPS)
+    y = _none_if_shape(A.RopeNormAttentionFn.apply, qkv, c, s, n_head, sc, RMS_EPS, int(nw) if nw else 0)
     return None if y is None else y.view(B, T, n_head, D)
 
 
