@@ -211,6 +211,9 @@ def test_gemm_glue_and_mlp_fused8(api, dev):
     dwf, dwp = O8.weight_grads(gy.reshape(300, d), xm.reshape(300, d), ho, dpo)
     assert rel_l2(mlp.c_fc.weight.grad, dwf) < FP8_TOL and rel_l2(mlp.c_proj.weight.grad, dwp) < FP8_TOL
     assert torch.equal(api.forward_scales(wf8.to(dev), wp8.to(dev)).cpu()[[0, 3, 13]], row[[0, 3, 13]])
+    tile = api.sc_tile(api.forward_scales(wf8.to(dev), wp8.to(dev)))
+    assert tile.shape == (128, 16) and torch.equal(tile[77].cpu()[[0, 3, 13]], row[[0, 3, 13]])
+    assert api.shapes_apply8(384, 256, 512) and not api.shapes_apply8(300, 256, 512) and not api.shapes_apply8(384, 128, 512)
 
 
 def test_nr_mlp_and_projection_with_residual(api, dev):

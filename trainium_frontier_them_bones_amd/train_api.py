@@ -311,6 +311,18 @@ def proj_residual(x, w, res):
     return A.LinearFn.apply(x, w, res)
 
 
+def shapes_apply8(m, d, f, tb=None):
+    """The shapes the fp8 MLP kernels take (K/nki_mlp_fused8.py:666 shapes_apply8): M a multiple of 128, d and F multiples
+    of 256. tb, the reference's token-block knob, has no counterpart here and is ignored."""
+    return m > 0 and m % 128 == 0 and d > 0 and d % 256 == 0 and f > 0 and f % 256 == 0
+
+
+def sc_tile(row):
+    """[128, 16] fp32: the scale row down every partition, the form the reference's kernels take (K/nki_mlp_fused8.py:816).
+    The entry points here read the 16-float row itself (`sc_tile(row)[0]`)."""
+    return row.float().reshape(1, 16).expand(128, 16).contiguous()
+
+
 def forward_scales(w_fc, w_proj):
     """The forward's 16-column scale row from the two weights (K/nki_mlp_fused8.py:782)."""
     return ops.mlp8_forward_scales(w_fc, w_proj)
