@@ -9,6 +9,9 @@ arithmetic with the residual adds and the MLP's fp8 operand cast as passes of th
 python bench.py --ns-probe        (Muon's Newton-Schulz call on the benchmark model's four stacks of 12 hidden matrices:
 one line per stack with its time and flop rate; not part of the AdamW step the headline line times)
 
+python bench.py --config-probe c1|c2|c3|c5|all   (the standalone configurations beside the full step, fwd + bwd each:
+one line per configuration; run under rocprofv3 --kernel-trace --stats for the per-kernel durations)
+
 python bench.py --traffic-probe   (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: a 256 MiB device copy as the
 counters' calibration, then attention forward + backward at the benchmark shape; prints nothing)
 """
@@ -90,6 +93,97 @@ def ns_probe():
         print("ns5 K=%d %dx%d: %.3f ms, %.0f TFLOP/s" % (K, r, c, dt * 1e3, flop / dt / 1e12), flush=True)
 
 
+def config_probe(which):
+    """The standalone configurations beside the full step, each fwd + bwd through the autograd layer, 3 untimed and 5 timed
+    repetitions: c1 RMSNorm -> LM head -> cross-entropy on 8192 tokens; c2 causal attention 16 x 12 x 2048 x 64; c3 the
+    fp8 MLP on 16384 tokens with a per-tensor amax activation scale; c5 the 8-expert top-2 fp8 layer on 16384 tokens,
+    balanced and with +2.0 on two experts' router logits. Prints one line per configuration with its time per repetition."""
+    import torch
+    from trainium_frontier_them_bones_amd import autograd as A
+    from trainium_frontier_them_bones_amd import ops
+    dev = torch.device("cuda:0")
+    bf = torch.bfloat16
+
+    def timed(name, fn, flop):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / 5
+        print("%s: %.3f ms per fwd+bwd, %.0f TFLOP/s of algorithmic work" % (name, dt * 1e3, flop / dt / 1e12), flush=True)
+
+    def leaf(t):
+        return t.to(dev).requires_grad_(True)
+
+    def clear(*ts):
+        for t in ts:
+            t.grad = None
+
+    if which in ("c1", "all"):
+        g = torch.Generator().manual_seed(20261)
+        N, d, V = 8192, 768, 32768
+        x = leaf(torch.randn(N, d, generator=g).to(bf))
+        nw = leaf((1 + 0.02 * torch.randn(d, generator=g)).to(bf))
+        W = leaf((0.02 * torch.randn(V, d, generator=g)).to(bf))
+        t = torch.randint(0, V, (N,), generator=g).to(dev)
+
+        def c1():
+            clear(x, nw, W)
+            A.LmHeadLossFn.apply(A.RMSNormFn.apply(x, nw, 1e-6), W, t, 0.0, "mean").backward()
+        timed("c1 norm + LM head + loss, 8192 tokens", c1, 3 * 2.0 * N * d * V)
+        del x, W
+    if which in ("c2", "all"):
+        g = torch.Generator().manual_seed(20262)
+        B, H, T, D = 16, 12, 2048, 64
+        q, k, v = (leaf(torch.randn(B, H, T, D, generator=g).to(bf)) for _ in range(3))
+        do = torch.randn(B, T, H, D, generator=g).to(bf).to(dev)
+
+        def c2():
+            clear(q, k, v)
+            A.CausalAttentionFn.apply(q, k, v, 0.125).backward(do)
+        timed("c2 causal attention 16x12x2048x64", c2, 7.0 * B * H * T * T * D)
+        del q, k, v, do
+    if which in ("c3", "all"):
+        g = torch.Generator().manual_seed(20263)
+        M, d, F = 16384, 768, 3072
+        x = leaf(torch.randn(M, d, generator=g).to(bf))
+        wf = leaf((0.02 * torch.randn(d, F, generator=g)).to(bf).t().contiguous())
+        wp = leaf((0.02 * torch.randn(F, d, generator=g)).to(bf).t().contiguous())
+        dy = torch.randn(M, d, generator=g).to(bf).to(dev)
+        st = A.Mlp8State(e4m3_limit=448.0)
+
+        def c3():
+            clear(x, wf, wp)
+            st.x_scale = float(ops.amax_scale(x.detach(), 448.0, -20, 20)[0].item())   # power of two under amax
+            st.refresh(wf, wp)
+            A.Mlp8Fn.apply(x, wf, wp, st).backward(dy)
+        timed("c3 fp8 MLP, 16384 tokens (scales and weight packs refreshed inside)", c3, 6 * 2.0 * M * d * F)
+        del x, dy
+    if which in ("c5", "all"):
+        N, d, Fd, E = 16384, 1024, 2816, 8
+        for skew in (0.0, 2.0):
+            g = torch.Generator().manual_seed(20265)
+            h = leaf(torch.randn(N, d, generator=g).to(bf))
+            router = leaf(0.02 * torch.randn(E, d, generator=g))
+            wf = leaf((0.02 * torch.randn(E, Fd, d, generator=g)).to(bf))
+            wp = leaf((0.02 * torch.randn(E, d, Fd, generator=g)).to(bf))
+            dy = torch.randn(N, d, generator=g).to(bf).to(dev)
+            bias = torch.zeros(E)
+            bias[:2] = skew
+            b = bias.to(dev) if skew else None
+            st = A.Moe8State()
+
+            def c5():
+                clear(h, router, wf, wp)
+                st.refresh(wf, wp)
+                A.MoeMlp8Fn.apply(h, router, wf, wp, st, 2, b).backward(dy)
+            timed("c5 MoE layer, 16384 tokens top-2 of 8, router bias %+.1f on two experts" % skew, c5,
+                  6 * 2.0 * (2 * N) * d * Fd)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -98,6 +192,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true")
     ap.add_argument("--ns-probe", action="store_true")
+    ap.add_argument("--config-probe", choices=("c1", "c2", "c3", "c5", "all"))
     ap.add_argument("--fp8-dw", action="store_true")
     ap.add_argument("--unfused-residual", action="store_true")
     args = ap.parse_args()
@@ -110,6 +205,9 @@ def main():
         return
     if args.ns_probe:
         ns_probe()
+        return
+    if args.config_probe:
+        config_probe(args.config_probe)
         return
 
     import torch

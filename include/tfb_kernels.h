@@ -347,16 +347,17 @@ int tfb_moe_combine_bwd(const void* dout, const void* ys, const void* tok, const
                         void* dgate, long rmax, int d, int topk, void* stream);
 
 /* dlogits fp32 [N][E] from dgate through the renormalisation and the softmax; dh bf16 [N][d] = dxs[slot_1] + dxs[slot_2] +
- * dlogits Wr; dwr fp32 [E][d] (+)= dlogits^T h.
+ * dlogits Wr; dwr fp32 [E][d] (+)= dlogits^T h, summed over 64 token chunks in a fixed order through scratch fp32 [64][E][d].
  * Replaces MoeDispatch2.backward (round2/source/train.py:10662-10666) and autograd through moe_route / the router matmul. */
 int tfb_moe_route_bwd(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot, const void* h,
-                      const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate, long N, int d, int E, int topk,
-                      void* stream);
+                      const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate, void* scratch, long N, int d, int E,
+                      int topk, void* stream);
 /* tfb_moe_route_bwd with the gradient of the auxiliary router terms folded into dlogits: the weighted sum
  * alpha lb + beta z of tfb_moe_aux_fwd received the gradient *gaux (device fp32 scalar); terms, lse as that call left them. */
 int tfb_moe_route_bwd_aux(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot, const void* h,
-                          const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate, const void* terms,
-                          const void* lse, const void* gaux, float alpha, float beta, long N, int d, int E, int topk, void* stream);
+                          const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate, void* scratch,
+                          const void* terms, const void* lse, const void* gaux, float alpha, float beta, long N, int d, int E,
+                          int topk, void* stream);
 /* The router's auxiliary loss terms: terms fp32 [2 + E] = (lb = E sum_e f_e P_e, z = mean_n logsumexp(logits_n)^2, f_e),
  * f_e = cnt_e / (N topk) the share of the assignments that chose e (cnt: the slot tables' counts; no gradient), P_e the
  * mean router probability; lse fp32 [N] is kept for the backward; scratch fp32 [64 * 17].

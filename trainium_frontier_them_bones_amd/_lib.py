@@ -78,8 +78,8 @@ SIGNATURES = {
     "tfb_moe_dw": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "tfb_moe_combine": [_vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_moe_combine_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
-    "tfb_moe_route_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _l, _i, _i, _i, _vp],
-    "tfb_moe_route_bwd_aux": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _f, _f, _l, _i, _i, _i, _vp],
+    "tfb_moe_route_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _l, _i, _i, _i, _vp],
+    "tfb_moe_route_bwd_aux": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _f, _f, _l, _i, _i, _i, _vp],
     "tfb_moe_aux_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_moe_backward_scales": [_vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_moe_quant": [_vp, _vp, _vp, _i, _i, _vp, _l, _i, _vp],

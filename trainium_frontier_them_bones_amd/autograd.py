@@ -590,9 +590,13 @@ class Moe8State:
 
     def refresh(self, w_fc, w_proj):
         E, F, d = w_fc.shape
-        rows = [ops.mlp8_forward_scales(w_fc[e].detach(), w_proj[e].detach(), self.e4m3_limit, self.x_scale) for e in range(E)]
+        wf, wp = w_fc.detach(), w_proj.detach()
+        if wf.is_contiguous() and wp.is_contiguous():      # the experts as E layers of one flat buffer: six launches
+            self.rows, self.w8 = ops.mlp8_refresh_layers(wf[0], wp[0], F * d, E, self.e4m3_limit, self.x_scale)
+            return
+        rows = [ops.mlp8_forward_scales(wf[e], wp[e], self.e4m3_limit, self.x_scale) for e in range(E)]
         self.rows = torch.stack(rows).contiguous()
-        self.w8 = torch.stack([ops.mlp8_precast(w_fc[e].detach(), w_proj[e].detach(), rows[e]) for e in range(E)]).contiguous()
+        self.w8 = torch.stack([ops.mlp8_precast(wf[e], wp[e], rows[e]) for e in range(E)]).contiguous()
 
 
 class MoeMlp8Fn(torch.autograd.Function):

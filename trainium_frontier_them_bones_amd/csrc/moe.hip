@@ -396,19 +396,23 @@ __global__ __launch_bounds__(256) void moe_dispatch_bwd_kernel(const bf16_t* __r
   }
 }
 
-// dWr[e][c] (+)= sum_n dlogits[n][e] h[n][c]: a workgroup owns 64 columns, 32 row lanes stride over the tokens.
-__global__ __launch_bounds__(256) void moe_dwr_kernel(const float* __restrict__ dlogits, const bf16_t* __restrict__ h,
-                                                     float* __restrict__ dwr, long N, int d, int E, int accumulate) {
-  __shared__ float red[32][8][8];
+// dWr[e][c] (+)= sum_n dlogits[n][e] h[n][c] in two launches with a fixed summation order: workgroup (x, y) owns 64 columns
+// and the y-th chunk of the tokens (32 row lanes stride over it) and leaves its sums in part[y][e][c]; the finish adds the
+// chunks in order. DWR_CHUNKS chunks at most: part is fp32 [DWR_CHUNKS][E][d].
+constexpr int DWR_CHUNKS = 64;
+__global__ __launch_bounds__(256) void moe_dwr_partial_kernel(const float* __restrict__ dlogits, const bf16_t* __restrict__ h,
+                                                             float* __restrict__ part, long N, long chunk, int d, int E) {
+  __shared__ float red[32][8][9];
   const int cl = threadIdx.x & 7, rl = threadIdx.x >> 3;
   const int c = blockIdx.x * 64 + cl * 8;
+  const long n0 = blockIdx.y * chunk, n1 = n0 + chunk < N ? n0 + chunk : N;
   for (int e0 = 0; e0 < E; e0 += 8) {
     float acc[8][8];
 #pragma unroll
     for (int e = 0; e < 8; ++e)
 #pragma unroll
       for (int k = 0; k < 8; ++k) acc[e][k] = 0.f;
-    for (long n = rl; n < N; n += 32) {
+    for (long n = n0 + rl; n < n1; n += 32) {
       float x[8];
       load8(h + n * d + c, x);
 #pragma unroll
@@ -426,17 +430,22 @@ __global__ __launch_bounds__(256) void moe_dwr_kernel(const float* __restrict__ 
 #pragma unroll
       for (int k = 0; k < 8; ++k) red[rl][cl][k] = acc[e][k];
       __syncthreads();
-      if (rl == 0 && e0 + e < E) {
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-          float s = 0.f;
-          for (int r = 0; r < 32; ++r) s += red[r][cl][k];
-          float* o = dwr + (long)(e0 + e) * d + c + k;
-          *o = accumulate ? *o + s : s;
-        }
+      if (rl < 8 && e0 + e < E) {   // row lane rl adds column k = rl of this thread's eight
+        float s = 0.f;
+        for (int r = 0; r < 32; ++r) s += red[r][cl][rl];
+        part[((long)blockIdx.y * E + e0 + e) * d + c + rl] = s;
       }
     }
   }
+}
+
+__global__ __launch_bounds__(256) void moe_dwr_finish_kernel(const float* __restrict__ part, float* __restrict__ dwr, int chunks,
+                                                            long ED, int accumulate) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= ED) return;
+  float s = accumulate ? dwr[i] : 0.f;
+  for (int y = 0; y < chunks; ++y) s += part[y * ED + i];
+  dwr[i] = s;
 }
 
 // ------------------------------------------------------------------------------------------------ per-expert scales
@@ -605,10 +614,10 @@ extern "C" int tfb_moe_combine_bwd(const void* dout, const void* ys, const void*
 // Router backward + dispatch backward: dlogits fp32 [N][E] (scratch/output), dh bf16 [N][d] = dxs[slots] + dlogits Wr,
 // dwr fp32 [E][d] (+)= dlogits^T h. Replaces MoeDispatch2.backward (10662-10666) and autograd through moe_route.
 static int moe_route_bwd_impl(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot,
-                              const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate, long N,
-                              int d, int E, int topk, const void* terms, const void* lse, const void* gaux, float alpha,
-                              float beta, void* stream) {
-  if (!dgate || !p || !idx || !dxs || !slot || !h || !wr || !dlogits || !dh || !dwr) return TFB_ERR_ARG;
+                              const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate,
+                              void* scratch, long N, int d, int E, int topk, const void* terms, const void* lse,
+                              const void* gaux, float alpha, float beta, void* stream) {
+  if (!dgate || !p || !idx || !dxs || !slot || !h || !wr || !dlogits || !dh || !dwr || !scratch) return TFB_ERR_ARG;
   if (N <= 0 || d <= 0 || d % 64 || E < 2 || E > MAXE || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(moe_dlogits_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, (const float*)dgate,
@@ -618,27 +627,32 @@ static int moe_route_bwd_impl(const void* dgate, const void* p, const void* idx,
   hipLaunchKernelGGL(moe_dispatch_bwd_kernel, dim3(nblocks(N * (d / 8))), dim3(256), 0, s, (const bf16_t*)dxs, (const int*)slot,
                      (const float*)dlogits, (const float*)wr, (bf16_t*)dh, N, d, E, topk);
   TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(moe_dwr_kernel, dim3(d / 64), dim3(256), 0, s, (const float*)dlogits, (const bf16_t*)h, (float*)dwr, N, d, E,
-                     dwr_accumulate);
+  const long chunk = ((N + DWR_CHUNKS - 1) / DWR_CHUNKS + 31) / 32 * 32;
+  const int chunks = (int)((N + chunk - 1) / chunk);
+  hipLaunchKernelGGL(moe_dwr_partial_kernel, dim3(d / 64, chunks), dim3(256), 0, s, (const float*)dlogits, (const bf16_t*)h,
+                     (float*)scratch, N, chunk, d, E);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_dwr_finish_kernel, dim3(nblocks((long)E * d)), dim3(256), 0, s, (const float*)scratch, (float*)dwr,
+                     chunks, (long)E * d, dwr_accumulate);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
 
 extern "C" int tfb_moe_route_bwd(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot,
-                                 const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate, long N,
-                                 int d, int E, int topk, void* stream) {
-  return moe_route_bwd_impl(dgate, p, idx, dxs, slot, h, wr, dlogits, dh, dwr, dwr_accumulate, N, d, E, topk, nullptr, nullptr,
-                            nullptr, 0.f, 0.f, stream);
+                                 const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate,
+                                 void* scratch, long N, int d, int E, int topk, void* stream) {
+  return moe_route_bwd_impl(dgate, p, idx, dxs, slot, h, wr, dlogits, dh, dwr, dwr_accumulate, scratch, N, d, E, topk, nullptr,
+                            nullptr, nullptr, 0.f, 0.f, stream);
 }
 // tfb_moe_route_bwd with the gradient of the auxiliary router terms folded into dlogits: the weighted sum
 // alpha lb + beta z of tfb_moe_aux_fwd received the gradient *gaux (device fp32 scalar); terms and lse as that call left them.
 extern "C" int tfb_moe_route_bwd_aux(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot,
                                      const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate,
-                                     const void* terms, const void* lse, const void* gaux, float alpha, float beta, long N, int d,
-                                     int E, int topk, void* stream) {
+                                     void* scratch, const void* terms, const void* lse, const void* gaux, float alpha,
+                                     float beta, long N, int d, int E, int topk, void* stream) {
   if (!terms || !lse || !gaux) return TFB_ERR_ARG;
-  return moe_route_bwd_impl(dgate, p, idx, dxs, slot, h, wr, dlogits, dh, dwr, dwr_accumulate, N, d, E, topk, terms, lse, gaux,
-                            alpha, beta, stream);
+  return moe_route_bwd_impl(dgate, p, idx, dxs, slot, h, wr, dlogits, dh, dwr, dwr_accumulate, scratch, N, d, E, topk, terms,
+                            lse, gaux, alpha, beta, stream);
 }
 
 // The router's auxiliary terms: terms fp32 [2 + E] = (lb = E sum_e f_e P_e, z = mean_n logsumexp(logits_n)^2, f_e) with

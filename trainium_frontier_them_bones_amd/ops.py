@@ -805,14 +805,15 @@ def moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, dwr=None, accumulate=False, a
     if dwr is None:
         dwr = torch.empty(E, d, dtype=torch.float32, device=h2.device)
         accumulate = False
+    scr = _scratch(h2.device, 64 * E * d)
     if aux is None:
         _lib.call("tfb_moe_route_bwd", _p(dgate), _p(p), _p(idx), _p(dxs), _p(tab["slot"]), _p(h2), _p(wr), _p(dlogits), _p(dh),
-                  _p(dwr), int(accumulate), N, d, E, idx.shape[1], _stream())
+                  _p(dwr), int(accumulate), _p(scr), N, d, E, idx.shape[1], _stream())
     else:
         terms, lse, gaux, alpha, beta = aux
         _chk(terms, torch.float32), _chk(lse, torch.float32), _chk(gaux, torch.float32)
         _lib.call("tfb_moe_route_bwd_aux", _p(dgate), _p(p), _p(idx), _p(dxs), _p(tab["slot"]), _p(h2), _p(wr), _p(dlogits),
-                  _p(dh), _p(dwr), int(accumulate), _p(terms), _p(lse), _p(gaux), float(alpha), float(beta), N, d, E,
+                  _p(dh), _p(dwr), int(accumulate), _p(scr), _p(terms), _p(lse), _p(gaux), float(alpha), float(beta), N, d, E,
                   idx.shape[1], _stream())
     return dh, dwr, dlogits
 
