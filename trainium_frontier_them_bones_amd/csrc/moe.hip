@@ -125,25 +125,41 @@ __global__ __launch_bounds__(256) void moe_count_kernel(const int* __restrict__ 
   }
 }
 
-// One workgroup: exclusive scan of the per-wavefront counts per expert, padded segment offsets, tile -> expert table.
+// One workgroup: exclusive scan of the per-wavefront counts per expert (a wavefront per expert, each lane a run of
+// consecutive entries), padded segment offsets, tile -> expert table.
 __global__ __launch_bounds__(256) void moe_scan_kernel(int* __restrict__ wave_cnt, int nwaves, int E, int* __restrict__ cnt,
                                                       int* __restrict__ seg, int* __restrict__ tile_expert, int ntiles) {
   __shared__ int s_seg[MAXE + 1];
-  if ((int)threadIdx.x < E) {
-    int e = threadIdx.x, run = 0;
-    for (int w = 0; w < nwaves; ++w) {
-      int c = wave_cnt[(long)w * E + e];
+  __shared__ int s_cnt[MAXE];
+  const int lane = threadIdx.x & 63;
+  const int run_len = (nwaves + 63) / 64;
+  const int w0 = lane * run_len < nwaves ? lane * run_len : nwaves;
+  const int w1 = w0 + run_len < nwaves ? w0 + run_len : nwaves;
+  for (int e = threadIdx.x >> 6; e < E; e += 4) {
+    int tot = 0;
+    for (int w = w0; w < w1; ++w) tot += wave_cnt[(long)w * E + e];
+    int inc = tot;
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_up(inc, o);
+      if (lane >= o) inc += t;
+    }
+    int run = inc - tot;
+    for (int w = w0; w < w1; ++w) {
+      const int c = wave_cnt[(long)w * E + e];
       wave_cnt[(long)w * E + e] = run;  // becomes the wavefront's offset inside the expert's segment
       run += c;
     }
-    cnt[e] = run;
+    if (lane == 63) {
+      cnt[e] = inc;
+      s_cnt[e] = inc;
+    }
   }
   __syncthreads();
   if (threadIdx.x == 0) {
     int off = 0;
     for (int e = 0; e < E; ++e) {
       s_seg[e] = off;
-      off += (cnt[e] + 127) / 128 * 128;
+      off += (s_cnt[e] + 127) / 128 * 128;
     }
     s_seg[E] = off;
     for (int e = 0; e <= E; ++e) seg[e] = s_seg[e];
@@ -444,20 +460,29 @@ __global__ __launch_bounds__(256) void moe_dwr_finish_kernel(const float* __rest
   const long i = (long)blockIdx.x * 256 + threadIdx.x;
   if (i >= ED) return;
   float s = accumulate ? dwr[i] : 0.f;
-  for (int y = 0; y < chunks; ++y) s += part[y * ED + i];
+  int y = 0;
+  for (; y + 8 <= chunks; y += 8) {   // eight loads in flight, added in order
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = part[(y + j) * ED + i];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s += v[j];
+  }
+  for (; y < chunks; ++y) s += part[y * ED + i];
   dwr[i] = s;
 }
 
 // ------------------------------------------------------------------------------------------------ per-expert scales
-// amax of each 128-row tile of g, merged into its expert's slot (non-negative floats order like their bit patterns).
+// amax of each 128-row tile of g (four workgroups of 32 rows each), merged into its expert's slot (non-negative floats order
+// like their bit patterns).
 __global__ __launch_bounds__(256) void moe_amax_kernel(const bf16_t* __restrict__ g, const int* __restrict__ tile_expert,
                                                       unsigned* __restrict__ amax_bits, int d) {
   __shared__ float red[4];
   const int e = tile_expert[blockIdx.x];
   if (e < 0) return;
-  const bf16_t* base = g + (long)blockIdx.x * 128 * d;
+  const bf16_t* base = g + ((long)blockIdx.x * 128 + blockIdx.y * 32) * d;
   float m = 0.f;
-  for (long i = (long)threadIdx.x * 8; i < 128L * d; i += 256 * 8) {
+  for (long i = (long)threadIdx.x * 8; i < 32L * d; i += 256 * 8) {
     u32x4 u = *(const u32x4*)(base + i);
 #pragma unroll
     for (int k = 0; k < 4; ++k) m = fmaxf(m, fmaxf(fabsf(bflo(u[k])), fabsf(bfhi(u[k]))));
@@ -682,7 +707,7 @@ extern "C" int tfb_moe_backward_scales(const void* dys, const void* tile_expert,
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(256), 0, s, (int*)amax_scratch, 0, (long)E);
   TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(moe_amax_kernel, dim3((unsigned)(rmax / 128)), dim3(256), 0, s, (const bf16_t*)dys, (const int*)tile_expert,
+  hipLaunchKernelGGL(moe_amax_kernel, dim3((unsigned)(rmax / 128), 4), dim3(256), 0, s, (const bf16_t*)dys, (const int*)tile_expert,
                      (unsigned*)amax_scratch, d);
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(moe_backward_scales_kernel, dim3(1), dim3(64), 0, s, (const unsigned*)amax_scratch, (const float*)rows_in,
