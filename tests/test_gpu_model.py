@@ -80,3 +80,27 @@ def test_full_size_step_runs_and_loss_is_sane(dev):
     for _ in range(3):
         l = m.train_step(idx.to(dev), tg.to(dev)).item()
     assert l < l0 and math.isfinite(l)
+
+
+def test_benchmark_line_on_a_short_run(dev):
+    """bench.py end to end (2 steps, no CPU leg): one JSON line with the contract's fields, and the entry point it times
+    with events is one the step really calls (roofline.launch_ms > 0)."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--steps", "2", "--warmup", "1", "--no-cpu"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    out = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline"):
+        assert key in out, key
+    assert out["n_gpus"] == 1 and out["steps"] == 2 and out["value"] > 0 and out["vs_baseline"] is None
+    rf = out["roofline"]
+    assert rf["bound"] == "mfma" and rf["launch_ms"] > 0 and 0 < rf["frac"] < 1 and abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-3
+    r2 = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=60)
+    assert r2.returncode != 0 and "one GPU" in r2.stderr

@@ -133,6 +133,8 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16_t* __restri
     Row<NCH> g, a;
     g.load(gy + row * C, C, lane);
     a.load(s + row * C, C, lane);
+    Row<NCH> r;
+    if (gs) r.load(gs + row * C, C, lane);   // issued with the other two loads
     const float rs = inv[row];
     if (w) {
 #pragma unroll
@@ -150,8 +152,6 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16_t* __restri
 #pragma unroll
       for (int k = 0; k < 8; ++k) g.v[i][k] = rs * (g.v[i][k] - a.v[i][k] * coef);
     if (gs) {
-      Row<NCH> r;
-      r.load(gs + row * C, C, lane);
 #pragma unroll
       for (int i = 0; i < NCH; ++i)
 #pragma unroll

@@ -455,8 +455,12 @@ def attn_fwd(q, k, v, scale, layout="bhtd", band=0):
         B, T, H, D = q.shape
     o = torch.empty(B, T, H, D, dtype=bf16, device=q.device)
     lse = torch.empty(B, H, T, dtype=torch.float32, device=q.device)
-    _lib.call("tfb_attn_fwd_band", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o),
-              _bht(o, "bthd"), _p(lse), B, H, T, D, float(scale), int(band), _stream())
+    if band:
+        _lib.call("tfb_attn_fwd_band", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o),
+                  _bht(o, "bthd"), _p(lse), B, H, T, D, float(scale), int(band), _stream())
+    else:
+        _lib.call("tfb_attn_fwd", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o),
+                  _bht(o, "bthd"), _p(lse), B, H, T, D, float(scale), _stream())
     return o, lse
 
 
@@ -478,9 +482,13 @@ def attn_bwd(q, k, v, o, do, lse, scale, layout="bhtd", dq=None, dk=None, dv=Non
     delta = torch.empty(2, B, H, T, dtype=torch.float32, device=q.device)
     cos, sin = rope if rope is not None else (None, None)
     _chk(cos), _chk(sin)
-    _lib.call("tfb_attn_bwd_band", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o),
-              _bht(o, "bthd"), _p(do), _bht(do, "bthd"), _p(dq), _bht(dq, out_layout), _p(dk), _bht(dk, out_layout), _p(dv),
-              _bht(dv, out_layout), _p(lse), _p(delta), _p(cos), _p(sin), B, H, T, D, float(scale), int(band), _stream())
+    args = (_p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o), _bht(o, "bthd"), _p(do),
+            _bht(do, "bthd"), _p(dq), _bht(dq, out_layout), _p(dk), _bht(dk, out_layout), _p(dv), _bht(dv, out_layout), _p(lse),
+            _p(delta), _p(cos), _p(sin), B, H, T, D, float(scale))
+    if band:
+        _lib.call("tfb_attn_bwd_band", *args, int(band), _stream())
+    else:
+        _lib.call("tfb_attn_bwd_rope", *args, _stream())     # cos = sin = NULL: no rotation (what tfb_attn_bwd forwards to)
     return dq, dk, dv
 
 
