@@ -558,6 +558,29 @@ def test_lmhead_softcap_matches_materialised_path(ops, dev):
     assert rel_l2(rows, rows2) < 1e-5 and rel_l2(lse, lse2) < 1e-6
 
 
+def test_lmhead_loss_with_every_target_ignored_and_with_one_valid_row(ops, dev):
+    """ignore_index rows carry neither loss nor gradient: with all of them ignored the mean loss and every gradient are
+    exactly zero; with one valid row the loss is that row's cross-entropy (torch's on the kernel's own logits)."""
+    from trainium_frontier_them_bones_amd import autograd as A
+    g = _g(23)
+    N, d, V = 256, 256, 1024
+    x = torch.randn(N, d, generator=g).bfloat16().to(dev).requires_grad_(True)
+    W = (0.05 * torch.randn(V, d, generator=g)).bfloat16().to(dev).requires_grad_(True)
+    t = torch.full((N,), -1, dtype=torch.long, device=dev)
+    loss = A.LmHeadLossFn.apply(x, W, t, 15.0, "mean")
+    loss.backward()
+    assert loss.item() == 0.0 and float(x.grad.float().abs().max()) == 0.0 and float(W.grad.float().abs().max()) == 0.0
+    x.grad = W.grad = None
+    t[77] = 5
+    loss = A.LmHeadLossFn.apply(x, W, t, 15.0, "mean")
+    loss.backward()
+    z = 15.0 * torch.tanh(ops.matmul(x.detach(), W.detach(), trans_b=True)[77].float() / 15.0)
+    want = torch.nn.functional.cross_entropy(z[None], t[77:78])
+    assert abs(loss.item() - want.item()) < 1e-3 * want.item()
+    rows = x.grad.float().abs().sum(1)
+    assert float(rows[77]) > 0 and float(rows.sum() - rows[77]) == 0.0          # only the valid row has a gradient
+
+
 def test_qkv_rope_projection_fused_equals_unfused(ops, dev):
     """The projection with the rotary embedding in its epilogue, and the autograd node built on it, against the
     separate GEMM / rotation / attention launches: bit for bit."""

@@ -66,6 +66,36 @@ def test_moe_layer_forward_backward(dev, shape, topk, skew):
     assert rel_l2(rd.grad, ro.grad) < 2e-2
 
 
+def test_moe_starved_expert_and_ragged_token_count(dev):
+    """One expert's router bias keeps every token away from it (empty segment, zero weight gradient, finite scales) and the
+    token count is not a multiple of the 64-token counting groups."""
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import autograd as A
+    from trainium_frontier_them_bones_amd import ops
+    N, d, Fd, E = 1000, 256, 512, 4
+    h, router, wf, wp, bias = _layer(11, N, d, Fd, E)
+    bias[2] = -1e4
+    hd, rd, wfd, wpd = (t.to(dev).requires_grad_(True) for t in (h, router, wf, wp))
+    st = A.Moe8State()
+    st.refresh(wfd, wpd)
+    out = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, st, 2, bias.to(dev))
+    g = torch.randn(N, d, generator=torch.Generator().manual_seed(5)).bfloat16()
+    out.backward(g.to(dev))
+    _, idx, _, _ = ops.moe_route(hd.detach(), rd.detach(), 2, bias.to(dev))
+    tab = ops.moe_tables(idx, E)
+    assert int(tab["cnt"][2]) == 0 and int(tab["cnt"].sum()) == 2 * N
+    assert int(tab["seg"][3]) == int(tab["seg"][2])                              # an empty segment takes no rows
+    ho, ro, wfo, wpo = (t.clone().requires_grad_(True) for t in (h, router, wf, wp))
+    oo, _ = O.moe_forward(ho, ro, wfo, wpo, 2, bias)
+    oo.backward(g)
+    assert rel_l2(out, oo) < 2e-2 and rel_l2(hd.grad, ho.grad) < 2e-2 and rel_l2(rd.grad, ro.grad) < 2e-2
+    assert float(wfd.grad[2].float().abs().max()) == 0.0 and float(wpd.grad[2].float().abs().max()) == 0.0
+    keep = [0, 1, 3]
+    assert rel_l2(wfd.grad[keep], wfo.grad[keep]) < 2e-2 and rel_l2(wpd.grad[keep], wpo.grad[keep]) < 2e-2
+    for t in (out, hd.grad, rd.grad, wfd.grad, wpd.grad):
+        assert bool(torch.isfinite(t.float()).all())
+
+
 def test_moe_config5_full_size(dev):
     """16384 tokens, d 1024, 8 experts top-2, FFN 2816: balanced and skewed routing; a token slice against the oracle,
     exact equivariance under a token permutation, and load accounting."""
