@@ -1,5 +1,5 @@
 """Loss-head oracle: softcap + log-softmax + cross-entropy on the raw LM-head output, and the composition
-final RMSNorm -> LM-head GEMM -> loss that BASELINE config 1 times.
+final RMSNorm -> LM-head GEMM -> loss that configuration 1 of BASELINE.json times.
 
 Restates R1:4481-4495 (eager loss rows: logits.float(), softcap * tanh(logits / softcap), log_softmax, one-hot
 pick), the gradient stated in the R1 loss-head docstring (R1:4466: d x = g (softmax - onehot) (1 - tanh^2)),

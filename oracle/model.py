@@ -1,5 +1,5 @@
 """The benchmark model in plain PyTorch on the CPU: the path the reference takes off-device (eager expressions and
-the kernels' torch emulations behind autograd Functions), restated for the BASELINE configuration (12 layers, d 768,
+the kernels' torch emulations behind autograd Functions), restated for the full-step configuration of BASELINE.json (12 layers, d 768,
 12 heads of 64, fp8 squared-ReLU MLP 3072, weighted RMSNorm pre-norm, RoPE, untied head, vocab 32768).
 
 Follows the reference's Block / GPT forward order (R1:8826-8867, 9163-9228; R2:11094-11123, 11612-11709): norm ->

@@ -3,7 +3,7 @@
 Restates R1:5165-5168 (eager block head: x_new = l1*x + l2*x0, norm(x_new)), R1:5594 (rmsnorm_fast),
 R1:6106-6159 (head_skip / tail_norm2 / final_norm eager forms), R2:8805-8825 (nf_norm_rows and its
 backward: upcast, rs = rsqrt(mean(x^2) + eps), one rounding per output; G = inv * (g - x * (g.x) * inv^2 / C)).
-The optional per-channel weight and eps are BASELINE config 1's generalisation (reference: no weight, eps 2^-23).
+The optional per-channel weight and eps are configuration 1 of BASELINE.json's generalisation (reference: no weight, eps 2^-23).
 
 Pinned by: torch.nn.functional.rms_norm (forward), torch.autograd on an fp64 restatement (backward),
 the invariant that J^T(g) is orthogonal to x when weight is None.

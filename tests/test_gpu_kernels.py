@@ -342,7 +342,7 @@ def test_mlp8_refresh_of_all_layers_equals_per_layer_calls(ops, dev):
 
 
 def test_mlp8_full_size_properties(ops, dev):
-    """BASELINE config 3 sizes: exact equivariance under a permutation of the tokens and agreement of 512-row slices
+    """configuration 3 of BASELINE.json sizes: exact equivariance under a permutation of the tokens and agreement of 512-row slices
     with the oracle."""
     from oracle import mlp8 as O
     M, d, F = 16384, 768, 3072
@@ -472,7 +472,7 @@ def test_attention_strided_qkv_and_rejects(ops, dev):
 
 
 def test_attention_full_size_properties(ops, dev):
-    """BASELINE config 2 (B16 H12 T2048 D64, RoPE'd q and k): two (b, h) pairs against the oracle, causality by
+    """configuration 2 of BASELINE.json (B16 H12 T2048 D64, RoPE'd q and k): two (b, h) pairs against the oracle, causality by
     perturbing the future, and dV with dO = 1 equal to the column sums of P."""
     from oracle import attention as O
     B, H, T, D = 16, 12, 2048, 64
@@ -526,7 +526,7 @@ def test_loss_fwd_bwd(ops, dev, cap):
 
 
 def test_lmhead_config1(ops, dev):
-    """BASELINE config 1 at full size through the autograd layer: RMSNorm -> LM-head GEMM (+lse) -> CE, fwd + bwd."""
+    """configuration 1 of BASELINE.json at full size through the autograd layer: RMSNorm -> LM-head GEMM (+lse) -> CE, fwd + bwd."""
     from oracle import loss as O
     from trainium_frontier_them_bones_amd import autograd as A
     g = _g(20261)

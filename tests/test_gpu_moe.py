@@ -1,4 +1,4 @@
-"""MoE layer on the HIP kernels against the oracle (BASELINE config 5 shapes in the last test)."""
+"""MoE layer on the HIP kernels against the oracle (configuration 5 of BASELINE.json shapes in the last test)."""
 import pytest
 import torch
 

@@ -32,9 +32,9 @@ class GPTConfig:
     init_std: float = 0.02
     e4m3_limit: float = 240.0     # fp8 scale search limit (240 = the reference's rows, 448 = OCP maximum)
     x_scale: float = 4.0          # constant activation scale of the fp8 MLP input (a unit-RMS norm output)
-    fp8_attn_proj: bool = False   # QKV and output projections in fp8 (e4m3 forward, e5m2 dX, bf16 dW); off in BASELINE C4
+    fp8_attn_proj: bool = False   # QKV and output projections in fp8 (e4m3 forward, e5m2 dX, bf16 dW); off in configuration 4 of BASELINE.json
     fp8_attn_dw: bool = False     # with fp8_attn_proj: their weight gradients in fp8 as well (R2_DW8_SET=qkv,proj)
-    fp8_mlp_dw: bool = False      # the MLP's two weight gradients in fp8 as well (R1's DW_ROWS recipe); off in BASELINE C4
+    fp8_mlp_dw: bool = False      # the MLP's two weight gradients in fp8 as well (R1's DW_ROWS recipe); off in configuration 4 of BASELINE.json
     fuse_residual: bool = True    # residual adds in the projections' stores, fp8 operand casts in the norms (same values)
 
     @property
