@@ -202,6 +202,18 @@ def test_relu2_rope_resmix_embedding_bit_exact(ops, dev):
     ops.embedding_bwd(idx2.int().to(dev), dy2.to(dev), dw)
     want.index_add_(0, idx2, dy2.float())
     assert rel_l2(dw, want) < 1e-6
+    # the plain atomic entry point gives the same sums; every row on one token and every row on its own token
+    dwa = ops.fill_f32_(torch.empty(1000, 768, device=dev), 0.0)
+    ops.embedding_bwd(idx.to(dev), dy.to(dev), dwa, grouped=False)
+    ops.embedding_bwd(idx2.to(dev), dy2.to(dev), dwa, grouped=False)
+    assert rel_l2(dwa, want) < 1e-6
+    for ids in (torch.full((512,), 3, dtype=torch.long), torch.randperm(1000, generator=g)[:512]):
+        dy3 = torch.randn(512, 768, generator=g).bfloat16()
+        w3 = torch.zeros(1000, 768).index_add_(0, ids, dy3.float())
+        for grouped in (True, False):
+            d3 = ops.fill_f32_(torch.empty(1000, 768, device=dev), 0.0)
+            ops.embedding_bwd(ids.to(dev), dy3.to(dev), d3, grouped=grouped)
+            assert rel_l2(d3, w3) < 1e-6
 
 
 def test_adamw(ops, dev):

@@ -482,13 +482,15 @@ def attn_bwd(q, k, v, o, do, lse, scale, layout="bhtd", dq=None, dk=None, dv=Non
     delta = torch.empty(2, B, H, T, dtype=torch.float32, device=q.device)
     cos, sin = rope if rope is not None else (None, None)
     _chk(cos), _chk(sin)
-    args = (_p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o), _bht(o, "bthd"), _p(do),
+    ptrs = (_p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o), _bht(o, "bthd"), _p(do),
             _bht(do, "bthd"), _p(dq), _bht(dq, out_layout), _p(dk), _bht(dk, out_layout), _p(dv), _bht(dv, out_layout), _p(lse),
-            _p(delta), _p(cos), _p(sin), B, H, T, D, float(scale))
+            _p(delta))
     if band:
-        _lib.call("tfb_attn_bwd_band", *args, int(band), _stream())
+        _lib.call("tfb_attn_bwd_band", *ptrs, _p(cos), _p(sin), B, H, T, D, float(scale), int(band), _stream())
+    elif rope is not None:
+        _lib.call("tfb_attn_bwd_rope", *ptrs, _p(cos), _p(sin), B, H, T, D, float(scale), _stream())
     else:
-        _lib.call("tfb_attn_bwd_rope", *args, _stream())     # cos = sin = NULL: no rotation (what tfb_attn_bwd forwards to)
+        _lib.call("tfb_attn_bwd", *ptrs, B, H, T, D, float(scale), _stream())
     return dq, dk, dv
 
 
@@ -582,11 +584,15 @@ def embedding_fwd(idx, weight):
     return out
 
 
-def embedding_bwd(idx, dy, dw):
-    """dw (fp32 [V, C]) += scatter of dy rows by idx."""
+def embedding_bwd(idx, dy, dw, grouped=True):
+    """dw (fp32 [V, C]) += scatter of dy rows by idx. grouped: rows sorted by token on the device and summed per token
+    (deterministic order inside a token's run); False: one fp32 atomic add per element (the plain entry point)."""
     _chk(dy), _chk(dw, torch.float32)
     idx = idx.contiguous()
     n, V = idx.numel(), dw.shape[0]
+    if not grouped:
+        _lib.call("tfb_embedding_bwd", _p(idx), int(idx.dtype == torch.int64), _p(dy), _p(dw), n, dy.shape[-1], _stream())
+        return dw
     scr = _scratch(dw.device, _lib.lib().tfb_embedding_bwd_scratch_ints(n, V))  # 4-byte elements, used as int32
     _lib.call("tfb_embedding_bwd_grouped", _p(idx), int(idx.dtype == torch.int64), _p(dy), _p(dw), n, dy.shape[-1], V,
               _p(scr), _stream())
