@@ -62,6 +62,7 @@ class RMSNormPassFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, eps, y8_scale=None):
         x = x.contiguous()
+        ctx.set_materialize_grads(False)      # no zero tensor for the byte output's (or an unused output's) gradient
         if y8_scale is None:
             _, y, inv = ops.rmsnorm_fwd(x, weight, eps)
             outs = (x, y)
