@@ -4,9 +4,9 @@
 // Operand tiles (128 bytes of k per row: 64 bf16 or 128 fp8) go from global memory straight into LDS with
 // global_load_lds_dwordx4 (no staging registers, no VALU work): one instruction moves 1 KB, lane l filling bytes
 // 16 l .. 16 l + 15, so the LDS layout is chosen by which 16-byte global chunk each lane fetches:
-//   K_CONTIG  [rows][K]:  LDS row = 128 bytes of k, chunk c of row r at slot c ^ ((r + r / 8) & 7). The 128-bit
-//             fragment reads of 16 consecutive rows then fall on 16 different 16-byte bank groups (LDS here has
-//             64 banks of 4 bytes, measured 256 B/clk for ds_read_b128).
+//   K_CONTIG  [rows][K]:  LDS row = 128 bytes of k, chunk c of row r at slot c ^ (4 ((r >> 1) & 1) | ((r >> 2) & 3))
+//             (tfb_kc_swz): the 128-bit fragment reads of a wavefront (32 rows x 2 chunks) then count no bank
+//             conflicts (LDS here has 64 banks of 4 bytes).
 //   K_STRIDED [K][rows]:  LDS row = one k with the tile's rows contiguous. bf16: 16-byte chunk c of k-row k at slot
 //             c ^ (4 (k & 3)); fragments are fetched with ds_read_b64_tr_b16, whose 16-lane transpose hands lane i
 //             four consecutive k of row i when lane j points at (k0 + j / 4, row0 + 4 (j % 4)). fp8 (128-row tiles):
@@ -30,6 +30,9 @@
 
 #include "common.hpp"
 
+// slot swizzle of the K_CONTIG layout: chunk c of row r sits at slot c ^ tfb_kc_swz(r). With this map the 128-bit fragment
+// reads count no bank conflicts (SQ_LDS_BANK_CONFLICT 0); the earlier map (r + r / 8) & 7 cost every such read 4 cycles.
+__device__ __forceinline__ int tfb_kc_swz(int r) { return (4 * ((r >> 1) & 1)) | ((r >> 2) & 3); }
 #define TFB_K_CONTIG 0
 #define TFB_K_STRIDED 1
 
@@ -107,8 +110,9 @@ struct TileDma<ROWS, NW, TFB_K_CONTIG, ES> {
     step = 8L * NW * o.ld;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-      // rows 8 g .. 8 g + 7 with g = i * NW + wave; slot (lane & 7) of row r holds chunk slot ^ ((r + g) & 7)
-      const int ch = (lane & 7) ^ ((lrow + v * NW + wave) & 7);
+      // rows 8 g .. 8 g + 7 with g = i * NW + wave; slot (lane & 7) of row r holds chunk slot ^ tfb_kc_swz(r), which
+      // depends on g through its parity only (NW is even), so NV offsets serve all instructions
+      const int ch = (lane & 7) ^ tfb_kc_swz(lrow + 8 * (v * NW + wave));
       voff[v] = (uint32_t)(lrow * o.ld + ch * 16);
     }
   }
@@ -164,7 +168,7 @@ struct FragReader<ROWS, 2, TFB_K_CONTIG> {
   __device__ __forceinline__ void init(int wave_row0, int lane) { row = wave_row0 + (lane & 31); lh = lane >> 5; }
   __device__ __forceinline__ frag_t read(const uint8_t* lds, int i, int s) const {
     const int r = row + 32 * i;
-    return *(const bf16x8*)(lds + r * 128 + ((((2 * s + lh) ^ (r + (r >> 3))) & 7) << 4));
+    return *(const bf16x8*)(lds + r * 128 + ((((2 * s + lh) ^ tfb_kc_swz(r)) & 7) << 4));
   }
 };
 template <int ROWS>
@@ -174,7 +178,7 @@ struct FragReader<ROWS, 1, TFB_K_CONTIG> {
   int row, lh;
   __device__ __forceinline__ void init(int wave_row0, int lane) { row = wave_row0 + (lane & 31); lh = lane >> 5; }
   __device__ __forceinline__ frag_t read(const uint8_t* lds, int i, int s) const {
-    const int r = row + 32 * i, f = r + (r >> 3);
+    const int r = row + 32 * i, f = tfb_kc_swz(r);
     const i32x4 a = *(const i32x4*)(lds + r * 128 + ((((4 * s + 2 * lh) ^ f) & 7) << 4));
     const i32x4 b = *(const i32x4*)(lds + r * 128 + ((((4 * s + 2 * lh + 1) ^ f) & 7) << 4));
     return i32x8{a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
