@@ -106,12 +106,14 @@ int tfb_resmix_bwd_blocks(long n);
 int tfb_resmix_bwd(const void* g, const void* x, const void* x0, const void* ab, void* dx, void* dx0, void* part, void* dab,
                    long n, void* stream);
 
-/* out[i] = w[idx[i]] rows; idx int64 (idx64=1) or int32. Replaces embedding_fwd (round1/source/train.py:8407). */
-int tfb_embedding_fwd(const void* idx, int idx64, const void* w, void* out, long n, int C, void* stream);
-/* dw_f32[idx[i]] += dy[i] (fp32 atomics). Replaces _emb_bwd_kernel (round1/source/train.py:8303). */
-int tfb_embedding_bwd(const void* idx, int idx64, const void* dy, void* dw_f32, long n, int C, void* stream);
+/* out[i] = w[idx[i]] rows, w [V][C]; idx int64 (idx64=1) or int32. An id outside [0, V) is never used as an address: its
+ * output row is zeros, and the backward calls below give it no gradient. Replaces embedding_fwd
+ * (round1/source/train.py:8407). */
+int tfb_embedding_fwd(const void* idx, int idx64, const void* w, void* out, long n, int C, int V, void* stream);
+/* dw_f32[idx[i]] += dy[i] (fp32 atomics), dw_f32 [V][C]. Replaces _emb_bwd_kernel (round1/source/train.py:8303). */
+int tfb_embedding_bwd(const void* idx, int idx64, const void* dy, void* dw_f32, long n, int C, int V, void* stream);
 /* The same sum with the rows grouped by token first (counting sort on the device, then a segmented sum), so that the
- * frequent tokens of a Zipf batch do not serialize on atomics; idx values must lie in [0, V). scratch: int32
+ * frequent tokens of a Zipf batch do not serialize on atomics; ids outside [0, V) are dropped. scratch: int32
  * [tfb_embedding_bwd_scratch_ints(n, V)]. Replaces _emb_bwd_kernel (round1/source/train.py:8303). */
 long tfb_embedding_bwd_scratch_ints(long n, int V);
 int tfb_embedding_bwd_grouped(const void* idx, int idx64, const void* dy, void* dw_f32, long n, int C, int V, void* scratch,
@@ -271,7 +273,8 @@ int tfb_attn_bwd_band(const void* q, const long* q_strides, const void* k, const
 
 /* ---- loss head ------------------------------------------------------------------------------------------------------
  * loss[row] = row_w[row] * (lse - s_target), lse[row] = log sum exp(s), s = softcap tanh(x / softcap) (softcap <= 0:
- * s = x); target < 0 = ignored row (loss 0). logits bf16 [rows][V]; targets int64 (idx64) or int32.
+ * s = x); a target outside [0, V) (the reference's ignore_index -1, or any id beyond the vocabulary) = ignored row:
+ * loss 0, gradient 0, never an address. logits bf16 [rows][V]; targets int64 (idx64) or int32.
  * Replaces _loss_fwd_kernel behind fused_loss (round1/source/train.py:4543, 4691) and _lh_fwd_kernel
  * (round2/source/train.py:5238; host chunked_loss_mean 6364). */
 int tfb_loss_fwd(const void* logits, const void* targets, int idx64, const void* row_w, void* loss, void* lse, long rows,

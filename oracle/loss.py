@@ -24,12 +24,13 @@ def softcap_logits(x, softcap):
 
 
 def loss_rows(logits2, targets, softcap=15.0):
-    """(rows fp32 [N], lse fp32 [N]); rows with target < 0 give 0."""
+    """(rows fp32 [N], lse fp32 [N]); rows whose target lies outside [0, V) (the reference's ignore_index -1; an id
+    beyond the vocabulary is treated the same way) give 0."""
     s = softcap_logits(logits2, softcap)
     lse = torch.logsumexp(s, dim=-1)
     t = targets.reshape(-1).long()
-    valid = t >= 0
-    picked = s.gather(1, t.clamp_min(0)[:, None]).squeeze(1)
+    valid = (t >= 0) & (t < s.shape[-1])
+    picked = s.gather(1, t.clamp(0, s.shape[-1] - 1)[:, None]).squeeze(1)
     return torch.where(valid, lse - picked, torch.zeros_like(lse)), lse
 
 
@@ -51,8 +52,8 @@ def loss_backward(logits2, targets, lse, grow, softcap=15.0):
     """dlogits in logits' dtype; grow [N] fp32 (upstream gradient times row weight)."""
     xf = logits2.float()
     t = targets.reshape(-1).long()
-    valid = (t >= 0).float()
-    onehot = F.one_hot(t.clamp_min(0), xf.shape[-1]).float()
+    valid = ((t >= 0) & (t < xf.shape[-1])).float()
+    onehot = F.one_hot(t.clamp(0, xf.shape[-1] - 1), xf.shape[-1]).float()
     if softcap:
         th = torch.tanh(xf / softcap)
         p = torch.exp(softcap * th - lse[:, None])

@@ -214,6 +214,19 @@ def test_relu2_rope_resmix_embedding_bit_exact(ops, dev):
             d3 = ops.fill_f32_(torch.empty(1000, 768, device=dev), 0.0)
             ops.embedding_bwd(ids.to(dev), dy3.to(dev), d3, grouped=grouped)
             assert rel_l2(d3, w3) < 1e-6
+    # ids outside [0, V) are never addresses: zero rows forward, no gradient backward, every other row unchanged
+    bad = idx2.clone()
+    bad[::7] = 1000
+    bad[3::11] = -5
+    bad[5::13] = 1 << 40
+    ok = (bad >= 0) & (bad < 1000)
+    e = ops.embedding_fwd(bad.to(dev), w.to(dev)).cpu()
+    assert torch.equal(e[ok], w[bad[ok]]) and not e[~ok].any()
+    wantb = torch.zeros(1000, 768).index_add_(0, bad[ok], dy2.float()[ok])
+    for grouped in (True, False):
+        d4 = ops.fill_f32_(torch.empty(1000, 768, device=dev), 0.0)
+        ops.embedding_bwd(bad.to(dev), dy2.to(dev), d4, grouped=grouped)
+        assert rel_l2(d4, wantb) < 1e-6
 
 
 def test_adamw(ops, dev):
@@ -230,6 +243,18 @@ def test_adamw(ops, dev):
         O.adamw_step(p, gr, m, v, step, 3e-4, 0.9, 0.95, 1e-8, 0.1)
     assert (pd.cpu() - p).abs().max().item() < 5e-7 and rel_l2(md, m) < 1e-6 and rel_l2(vd, v) < 1e-6
     assert torch.equal(p16.cpu(), pd.cpu().bfloat16())
+    # sizes that are not a multiple of four (one-element gains, odd vectors): the kernel's element-wise tail
+    for n in (1, 3, 1027):
+        p = torch.randn(n, generator=g)
+        m, v = torch.zeros(n), torch.zeros(n)
+        pd, md, vd = p.to(dev), m.to(dev), v.to(dev)
+        p16 = torch.empty(n, dtype=torch.bfloat16, device=dev)
+        for step in (1, 2):
+            gr = torch.randn(n, generator=g)
+            ops.adamw_(pd, gr.to(dev), md, vd, step, 3e-4, 0.9, 0.95, 1e-8, 0.1, p16)
+            O.adamw_step(p, gr, m, v, step, 3e-4, 0.9, 0.95, 1e-8, 0.1)
+        assert (pd.cpu() - p).abs().max().item() < 5e-7 and (md.cpu() - m).abs().max().item() < 1e-6
+        assert (vd.cpu() - v).abs().max().item() < 1e-6 and torch.equal(p16.cpu(), pd.cpu().bfloat16())
 
 
 # ------------------------------------------------------------------------------------------ fp8 MLP
@@ -524,17 +549,22 @@ def test_loss_fwd_bwd(ops, dev, cap):
     x = (3 * torch.randn(N, V, generator=g)).bfloat16()
     t = torch.randint(0, V, (N,), generator=g)
     t[5] = -1
+    t[9] = V                                                                   # beyond the vocabulary: ignored too, never an address
+    t[11] = 1 << 40
     w = O.row_weights(t, "mean")
     rows, lse = ops.loss_fwd(x.to(dev), t.to(dev), cap, w.to(dev))
+    assert float(rows[9]) == 0.0 and float(rows[11]) == 0.0
     ro, lo = O.loss_rows(x, t, cap)
     assert rel_l2(rows, ro * w) < 1e-5 and rel_l2(lse, lo) < 1e-6
     assert abs(rows.sum().item() - O.fused_loss(x, t, "mean", cap).item()) < 1e-3 * O.fused_loss(x, t, "mean", cap).item()
-    rows32, _ = ops.loss_fwd(x.to(dev), t.int().to(dev), cap, w.to(dev))
+    t32 = t.clamp(max=V).int()
+    rows32, _ = ops.loss_fwd(x.to(dev), t32.to(dev), cap, w.to(dev))
     assert torch.equal(rows32, rows)
     grow = torch.rand(N, generator=g) / N
     d = ops.loss_bwd(x.to(dev), t.to(dev), lse, grow.to(dev), cap)
     assert rel_l2(d, O.loss_backward(x, t, lo, grow, cap)) < BF16_TOL
     assert float(d[5].float().abs().max()) == 0.0                              # the ignored row gets no gradient
+    assert float(d[9].float().abs().max()) == 0.0 and float(d[11].float().abs().max()) == 0.0
 
 
 def test_lmhead_config1(ops, dev):

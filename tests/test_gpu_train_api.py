@@ -311,7 +311,8 @@ def test_head2_and_adamw_fused_step(api, dev):
     o2 = ON.block_head(xt.reshape(-1, 256), x0.reshape(-1, 256), l1[0], l2[0], xt.reshape(-1, 256), l3[0])
     assert none is None and torch.equal(x_new2.cpu().reshape(-1, 256), o2[0])
     # AdamW: three steps against torch.optim.AdamW on the same parameters and gradients
-    ps = [torch.randn(300, 64, generator=g), torch.randn(1000, generator=g)]
+    ps = [torch.randn(300, 64, generator=g), torch.randn(1000, generator=g), torch.randn(1, generator=g),
+          torch.randn(3, generator=g)]                                         # one-element gains and odd sizes step too
     ref = [p.clone().requires_grad_(True) for p in ps]
     mine = [p.clone().to(dev).requires_grad_(True) for p in ps]
     kw = dict(lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
@@ -321,7 +322,9 @@ def test_head2_and_adamw_fused_step(api, dev):
             gr = torch.randn(a.shape, generator=g)
             a.grad, b.grad = gr.clone(), gr.to(dev)
         o_ref.step()
+        versions = [b._version for b in mine]
         assert api.adamw_fused_step(o_mine) is True
+        assert all(b._version > v for b, v in zip(mine, versions))            # the raw kernel write is visible to autograd's counters
     for a, b in zip(ref, mine):
         assert rel_l2(b, a) < 1e-6
         assert rel_l2(o_mine.state[b]["exp_avg_sq"], o_ref.state[a]["exp_avg_sq"]) < 1e-6

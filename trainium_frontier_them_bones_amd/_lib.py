@@ -58,8 +58,8 @@ SIGNATURES = {
     "tfb_rope_norm_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _i, _l, _l, _l, _vp],
     "tfb_resmix_bwd_blocks": [_l],
     "tfb_resmix_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _vp],
-    "tfb_embedding_fwd": [_vp, _i, _vp, _vp, _l, _i, _vp],
-    "tfb_embedding_bwd": [_vp, _i, _vp, _vp, _l, _i, _vp],
+    "tfb_embedding_fwd": [_vp, _i, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_embedding_bwd": [_vp, _i, _vp, _vp, _l, _i, _i, _vp],
     "tfb_embedding_bwd_scratch_ints": [_l, _i],
     "tfb_embedding_bwd_grouped": [_vp, _i, _vp, _vp, _l, _i, _i, _vp, _vp],
     "tfb_adamw": [_vp, _vp, _i, _vp, _vp, _vp, _l, _f, _f, _f, _f, _f, _f, _f, _vp],

@@ -247,27 +247,31 @@ __global__ void sum_pairs_kernel(const float* __restrict__ part, int nblocks, fl
 
 template <typename IDX>
 __global__ __launch_bounds__(256) void embedding_fwd_kernel(const IDX* __restrict__ idx, const bf16_t* __restrict__ w,
-                                                           bf16_t* __restrict__ out, long n, int C) {
+                                                           bf16_t* __restrict__ out, long n, int C, int V) {
   const int cpr = C / 8;
   const long total = n * cpr;
   for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
     long row = i / cpr;
     int c = (int)(i % cpr) * 8;
     long tok = (long)idx[row];
-    *(u32x4*)(out + row * C + c) = *(const u32x4*)(w + tok * C + c);
+    // an id outside [0, V) never becomes an address: its row is zeros (and takes no gradient in the backward)
+    u32x4 val = {0u, 0u, 0u, 0u};
+    if ((unsigned long)tok < (unsigned long)V) val = *(const u32x4*)(w + tok * C + c);
+    *(u32x4*)(out + row * C + c) = val;
   }
 }
 
 // dW[idx[row]] += dY[row] in fp32 with atomics (dW fp32, zeroed or accumulated into by the caller).
 template <typename IDX>
 __global__ __launch_bounds__(256) void embedding_bwd_kernel(const IDX* __restrict__ idx, const bf16_t* __restrict__ dy,
-                                                           float* __restrict__ dw, long n, int C) {
+                                                           float* __restrict__ dw, long n, int C, int V) {
   const int cpr = C / 8;
   const long total = n * cpr;
   for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
     long row = i / cpr;
     int c = (int)(i % cpr) * 8;
     long tok = (long)idx[row];
+    if ((unsigned long)tok >= (unsigned long)V) continue;  // out-of-range id: no gradient row
     u32x4 u = *(const u32x4*)(dy + row * C + c);
     float* d = dw + tok * C + c;
 #pragma unroll
@@ -284,9 +288,14 @@ __global__ __launch_bounds__(256) void emb_zero_kernel(int* __restrict__ p, long
   if (i < n) p[i] = 0;
 }
 template <typename IDX>
-__global__ __launch_bounds__(256) void emb_count_kernel(const IDX* __restrict__ idx, int* __restrict__ count, long n) {
+__device__ __forceinline__ int emb_bucket(IDX t, int V) {
+  // ids outside [0, V) share the extra bucket V, which the sum skips
+  return (unsigned long)(long)t < (unsigned long)V ? (int)t : V;
+}
+template <typename IDX>
+__global__ __launch_bounds__(256) void emb_count_kernel(const IDX* __restrict__ idx, int* __restrict__ count, long n, int V) {
   long i = (long)blockIdx.x * 256 + threadIdx.x;
-  if (i < n) atomicAdd(count + (long)idx[i], 1);
+  if (i < n) atomicAdd(count + emb_bucket(idx[i], V), 1);
 }
 // One workgroup: cursor[v] = exclusive prefix sum of count[v] (count is left untouched).
 __global__ __launch_bounds__(1024) void emb_scan_kernel(const int* __restrict__ count, int* __restrict__ cursor, int V) {
@@ -316,9 +325,9 @@ __global__ __launch_bounds__(1024) void emb_scan_kernel(const int* __restrict__ 
 }
 template <typename IDX>
 __global__ __launch_bounds__(256) void emb_place_kernel(const IDX* __restrict__ idx, int* __restrict__ cursor,
-                                                       int* __restrict__ order, long n) {
+                                                       int* __restrict__ order, long n, int V) {
   long i = (long)blockIdx.x * 256 + threadIdx.x;
-  if (i < n) order[atomicAdd(cursor + (long)idx[i], 1)] = (int)i;
+  if (i < n) order[atomicAdd(cursor + emb_bucket(idx[i], V), 1)] = (int)i;
 }
 // A workgroup sums EMB_SEG consecutive rows of the token-grouped order, thread t owning columns 8t .. 8t+7. A run of
 // equal tokens that lies inside the segment has a single owner and is added with plain loads/stores; the first and the
@@ -326,7 +335,8 @@ __global__ __launch_bounds__(256) void emb_place_kernel(const IDX* __restrict__ 
 constexpr int EMB_SEG = 32;
 template <typename IDX>
 __global__ __launch_bounds__(128) void emb_reduce_kernel(const IDX* __restrict__ idx, const int* __restrict__ order,
-                                                        const bf16_t* __restrict__ dy, float* __restrict__ dw, long n, int C) {
+                                                        const bf16_t* __restrict__ dy, float* __restrict__ dw, long n, int C,
+                                                        int V) {
   __shared__ int rows[EMB_SEG];
   __shared__ int toks[EMB_SEG];
   const long pos0 = (long)blockIdx.x * EMB_SEG;
@@ -334,7 +344,7 @@ __global__ __launch_bounds__(128) void emb_reduce_kernel(const IDX* __restrict__
   if (threadIdx.x < cnt) {
     const int r = order[pos0 + threadIdx.x];
     rows[threadIdx.x] = r;
-    toks[threadIdx.x] = (int)idx[r];
+    toks[threadIdx.x] = emb_bucket(idx[r], V);
   }
   __syncthreads();
   const int c = (blockIdx.y * 128 + threadIdx.x) * 8;
@@ -350,7 +360,9 @@ __global__ __launch_bounds__(128) void emb_reduce_kernel(const IDX* __restrict__
     }
     if (i + 1 == cnt || toks[i + 1] != toks[i]) {
       float* d = dw + (long)toks[i] * C + c;
-      if (run_start == 0 || i + 1 == cnt) {
+      if (toks[i] == V) {
+        // the bucket of out-of-range ids: dropped
+      } else if (run_start == 0 || i + 1 == cnt) {
 #pragma unroll
         for (int k = 0; k < 8; ++k) atomicAdd(d + k, acc[k]);
       } else {
@@ -375,11 +387,21 @@ __device__ __forceinline__ float lerp_torch(float a, float b, float w) {
   return w < 0.5f ? fmaf(w, d, a) : fmaf(-d, 1.0f - w, b);  // torch's lerp contracts to one fma
 }
 
-// p (fp32 master) updated in place; optional bf16 copy written; g is fp32 (GF32) or bf16.
+__device__ __forceinline__ void adamw_one(float& pk, float& mk, float& vk, float gk, const AdamScalars& s) {
+  if (s.wd > 0.f) pk = pk * (1.0f - s.lr * s.wd);
+  mk = lerp_torch(mk, gk, s.omb1);
+  vk = lerp_torch(vk, gk * gk, s.omb2);
+  const float upd = mk / s.bias1 / (sqrtf(vk / s.bias2) + s.eps);
+  pk = pk - upd * s.lr;
+}
+
+// p (fp32 master) updated in place; optional bf16 copy written; g is fp32 (GF32) or bf16. Groups of four elements
+// take 128-bit accesses; the last n % 4 elements (one-element gains, odd-sized vectors) are finished one by one.
 template <bool GF32>
 __global__ __launch_bounds__(256) void adamw_kernel(float* __restrict__ p, const void* __restrict__ g, float* __restrict__ m,
                                                    float* __restrict__ v, bf16_t* __restrict__ p16, long n, AdamScalars s) {
-  for (long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4; i < n; i += (long)gridDim.x * 256 * 4) {
+  const long n4 = n & ~3L;
+  for (long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4; i < n4; i += (long)gridDim.x * 256 * 4) {
     f32x4 pp = *(const f32x4*)(p + i), mm = *(const f32x4*)(m + i), vv = *(const f32x4*)(v + i), gg;
     if (GF32) {
       gg = *(const f32x4*)((const float*)g + i);
@@ -389,12 +411,8 @@ __global__ __launch_bounds__(256) void adamw_kernel(float* __restrict__ p, const
     }
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      float pk = pp[k];
-      if (s.wd > 0.f) pk = pk * (1.0f - s.lr * s.wd);
-      float mk = lerp_torch(mm[k], gg[k], s.omb1);
-      float vk = lerp_torch(vv[k], gg[k] * gg[k], s.omb2);
-      float upd = mk / s.bias1 / (sqrtf(vk / s.bias2) + s.eps);
-      pk = pk - upd * s.lr;
+      float pk = pp[k], mk = mm[k], vk = vv[k];
+      adamw_one(pk, mk, vk, gg[k], s);
       pp[k] = pk;
       mm[k] = mk;
       vv[k] = vk;
@@ -406,6 +424,16 @@ __global__ __launch_bounds__(256) void adamw_kernel(float* __restrict__ p, const
       u32x2 o = {pack2bf(pp[0], pp[1]), pack2bf(pp[2], pp[3])};
       *(u32x2*)(p16 + i) = o;
     }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < (int)(n - n4)) {
+    const long i = n4 + threadIdx.x;
+    float pk = p[i], mk = m[i], vk = v[i];
+    const float gk = GF32 ? ((const float*)g)[i] : bf2f(((const bf16_t*)g)[i]);
+    adamw_one(pk, mk, vk, gk, s);
+    p[i] = pk;
+    m[i] = mk;
+    v[i] = vk;
+    if (p16) p16[i] = f2bf(pk);
   }
 }
 
@@ -492,30 +520,30 @@ extern "C" int tfb_resmix_bwd(const void* g, const void* x, const void* x0, cons
   return TFB_OK;
 }
 
-extern "C" int tfb_embedding_fwd(const void* idx, int idx64, const void* w, void* out, long n, int C, void* stream) {
+extern "C" int tfb_embedding_fwd(const void* idx, int idx64, const void* w, void* out, long n, int C, int V, void* stream) {
   if (!idx || !w || !out) return TFB_ERR_ARG;
-  if (n <= 0 || C <= 0 || C % 8) return TFB_ERR_SHAPE;
+  if (n <= 0 || C <= 0 || C % 8 || V <= 0) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   int nb = blocks_for(n * (C / 8));
-  if (idx64) hipLaunchKernelGGL(embedding_fwd_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, (const bf16_t*)w, (bf16_t*)out, n, C);
-  else hipLaunchKernelGGL(embedding_fwd_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, (const bf16_t*)w, (bf16_t*)out, n, C);
+  if (idx64) hipLaunchKernelGGL(embedding_fwd_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, (const bf16_t*)w, (bf16_t*)out, n, C, V);
+  else hipLaunchKernelGGL(embedding_fwd_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, (const bf16_t*)w, (bf16_t*)out, n, C, V);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
 
-extern "C" int tfb_embedding_bwd(const void* idx, int idx64, const void* dy, void* dw_f32, long n, int C, void* stream) {
+extern "C" int tfb_embedding_bwd(const void* idx, int idx64, const void* dy, void* dw_f32, long n, int C, int V, void* stream) {
   if (!idx || !dy || !dw_f32) return TFB_ERR_ARG;
-  if (n <= 0 || C <= 0 || C % 8) return TFB_ERR_SHAPE;
+  if (n <= 0 || C <= 0 || C % 8 || V <= 0) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   int nb = blocks_for(n * (C / 8));
-  if (idx64) hipLaunchKernelGGL(embedding_bwd_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, (const bf16_t*)dy, (float*)dw_f32, n, C);
-  else hipLaunchKernelGGL(embedding_bwd_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, (const bf16_t*)dy, (float*)dw_f32, n, C);
+  if (idx64) hipLaunchKernelGGL(embedding_bwd_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, (const bf16_t*)dy, (float*)dw_f32, n, C, V);
+  else hipLaunchKernelGGL(embedding_bwd_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, (const bf16_t*)dy, (float*)dw_f32, n, C, V);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
 
 // Scratch (int32 elements) of tfb_embedding_bwd_grouped.
-extern "C" long tfb_embedding_bwd_scratch_ints(long n, int V) { return 2L * V + n; }
+extern "C" long tfb_embedding_bwd_scratch_ints(long n, int V) { return 2L * (V + 1) + n; }
 
 // The same sum as tfb_embedding_bwd, rows grouped by token first: hot tokens (a Zipf batch) no longer serialize on atomics.
 extern "C" int tfb_embedding_bwd_grouped(const void* idx, int idx64, const void* dy, void* dw_f32, long n, int C, int V,
@@ -524,18 +552,18 @@ extern "C" int tfb_embedding_bwd_grouped(const void* idx, int idx64, const void*
   if (n <= 0 || n > 0x7fffffffL || C <= 0 || C % 8 || V <= 0) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   int* count = (int*)scratch;
-  int* cursor = count + V;
-  int* order = cursor + V;
+  int* cursor = count + (V + 1);  // bucket V collects the ids outside [0, V)
+  int* order = cursor + (V + 1);
   const unsigned nb = (unsigned)((n + 255) / 256);
-  hipLaunchKernelGGL(emb_zero_kernel, dim3((unsigned)((V + 255) / 256)), dim3(256), 0, s, count, (long)V);
-  if (idx64) hipLaunchKernelGGL(emb_count_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, count, n);
-  else hipLaunchKernelGGL(emb_count_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, count, n);
-  hipLaunchKernelGGL(emb_scan_kernel, dim3(1), dim3(1024), 0, s, count, cursor, V);
-  if (idx64) hipLaunchKernelGGL(emb_place_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, cursor, order, n);
-  else hipLaunchKernelGGL(emb_place_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, cursor, order, n);
+  hipLaunchKernelGGL(emb_zero_kernel, dim3((unsigned)((V + 256) / 256)), dim3(256), 0, s, count, (long)V + 1);
+  if (idx64) hipLaunchKernelGGL(emb_count_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, count, n, V);
+  else hipLaunchKernelGGL(emb_count_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, count, n, V);
+  hipLaunchKernelGGL(emb_scan_kernel, dim3(1), dim3(1024), 0, s, count, cursor, V + 1);
+  if (idx64) hipLaunchKernelGGL(emb_place_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, cursor, order, n, V);
+  else hipLaunchKernelGGL(emb_place_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, cursor, order, n, V);
   dim3 grid((unsigned)((n + EMB_SEG - 1) / EMB_SEG), (unsigned)((C / 8 + 127) / 128));
-  if (idx64) hipLaunchKernelGGL(emb_reduce_kernel<long>, grid, dim3(128), 0, s, (const long*)idx, order, (const bf16_t*)dy, (float*)dw_f32, n, C);
-  else hipLaunchKernelGGL(emb_reduce_kernel<int>, grid, dim3(128), 0, s, (const int*)idx, order, (const bf16_t*)dy, (float*)dw_f32, n, C);
+  if (idx64) hipLaunchKernelGGL(emb_reduce_kernel<long>, grid, dim3(128), 0, s, (const long*)idx, order, (const bf16_t*)dy, (float*)dw_f32, n, C, V);
+  else hipLaunchKernelGGL(emb_reduce_kernel<int>, grid, dim3(128), 0, s, (const int*)idx, order, (const bf16_t*)dy, (float*)dw_f32, n, C, V);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
@@ -544,10 +572,13 @@ extern "C" int tfb_embedding_bwd_grouped(const void* idx, int idx64, const void*
 extern "C" int tfb_adamw(void* p, const void* g, int g_f32, void* m, void* v, void* p_bf16, long n, float lr, float wd,
                          float one_minus_beta1, float one_minus_beta2, float eps, float bias1, float bias2, void* stream) {
   if (!p || !g || !m || !v) return TFB_ERR_ARG;
-  if (n <= 0 || n % 4) return TFB_ERR_SHAPE;
+  if (n <= 0) return TFB_ERR_SHAPE;
+  // the groups of four are 128-bit accesses (64-bit for bf16 tensors)
+  if ((((uintptr_t)p | (uintptr_t)m | (uintptr_t)v) & 15) || ((uintptr_t)g & (g_f32 ? 15 : 7)) || ((uintptr_t)p_bf16 & 7))
+    return TFB_ERR_ARG;
   AdamScalars sc{lr, wd, one_minus_beta1, one_minus_beta2, eps, bias1, bias2};
   hipStream_t s = (hipStream_t)stream;
-  int nb = blocks_for(n / 4);
+  int nb = blocks_for((n + 3) / 4);
   if (g_f32) hipLaunchKernelGGL(adamw_kernel<true>, dim3(nb), dim3(256), 0, s, (float*)p, g, (float*)m, (float*)v, (bf16_t*)p_bf16, n, sc);
   else hipLaunchKernelGGL(adamw_kernel<false>, dim3(nb), dim3(256), 0, s, (float*)p, g, (float*)m, (float*)v, (bf16_t*)p_bf16, n, sc);
   TFB_LAUNCH_CHECK();

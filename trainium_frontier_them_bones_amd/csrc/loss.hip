@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void loss_fwd_kernel(const bf16_t* __restrict_
     lse[row] = l;
     long tt = (long)tg[row];
     float out = 0.f;
-    if (tt >= 0) {
+    if ((unsigned long)tt < (unsigned long)V) {  // a target outside [0, V) is an ignored row, never an address
       float xt = bf2f(xr[tt]);
       float st = cap > 0.f ? cap * tanh_fast(xt * icap) : xt;
       out = (l - st) * (row_w ? row_w[row] : 1.0f);
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(256) void loss_bwd_kernel(const bf16_t* __restrict_
   const bf16_t* xr = x + row * V;
   bf16_t* dr = dx + row * V;
   const long tt = (long)tg[row];
-  const float g = tt >= 0 ? grow[row] : 0.f;
+  const float g = (unsigned long)tt < (unsigned long)V ? grow[row] : 0.f;  // out of range = ignored
   const float l = lse[row];
   const float icap = cap > 0.f ? 1.0f / cap : 0.f;
   for (int i = threadIdx.x * 8; i < V; i += 256 * 8) {
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(256) void loss_multi_fwd_kernel(const bf16_t* __res
     float out = 0.f;
     for (int k = 0; k < K; ++k) {
       const long tt = (long)tg[(long)k * rows + row];
-      if (tt < 0) continue;
+      if ((unsigned long)tt >= (unsigned long)V) continue;  // negative or beyond the vocabulary: weight 0
       const float xt = bf2f(xr[tt]);
       const float st = cap > 0.f ? cap * tanh_fast(xt * icap) : xt;
       out += rw[(long)k * rows + row] * (l - (1.0f - eps) * st - eps * mean_s);
@@ -233,7 +233,7 @@ __global__ __launch_bounds__(256) void loss_multi_bwd_kernel(const bf16_t* __res
     wk[k] = 0.f;
     if (k < K) {
       tk[k] = (long)tg[(long)k * rows + row];
-      if (tk[k] >= 0) {
+      if ((unsigned long)tk[k] < (unsigned long)V) {
         wk[k] = rw[(long)k * rows + row];
         W += wk[k];
       }
@@ -350,7 +350,7 @@ __global__ __launch_bounds__(256) void lmhead_finish_kernel(const float* __restr
     lse[row] = l;
     long tt = (long)tg[row];
     float out = 0.f;
-    if (tt >= 0) {
+    if ((unsigned long)tt < (unsigned long)V) {  // a target outside [0, V) is an ignored row, never an address
       float xt = bf2f(logits[row * V + tt]);
       float st = cap > 0.f ? cap * tanh_fast(xt / cap) : xt;
       out = (l - st) * (row_w ? row_w[row] : 1.0f);

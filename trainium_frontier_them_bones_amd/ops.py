@@ -574,13 +574,15 @@ def resmix_bwd(g, x, x0, ab):
 
 
 def embedding_fwd(idx, weight):
+    """weight rows gathered by idx; an id outside [0, V) gives a zero row (and receives no gradient in embedding_bwd)."""
     _chk(weight)
     if idx.dtype not in (torch.int64, torch.int32) or not idx.is_cuda:
         raise TypeError("idx must be an int32/int64 device tensor")
     idx = idx.contiguous()
     C = weight.shape[1]
     out = torch.empty(*idx.shape, C, dtype=bf16, device=weight.device)
-    _lib.call("tfb_embedding_fwd", _p(idx), int(idx.dtype == torch.int64), _p(weight), _p(out), idx.numel(), C, _stream())
+    _lib.call("tfb_embedding_fwd", _p(idx), int(idx.dtype == torch.int64), _p(weight), _p(out), idx.numel(), C,
+              weight.shape[0], _stream())
     return out
 
 
@@ -591,7 +593,8 @@ def embedding_bwd(idx, dy, dw, grouped=True):
     idx = idx.contiguous()
     n, V = idx.numel(), dw.shape[0]
     if not grouped:
-        _lib.call("tfb_embedding_bwd", _p(idx), int(idx.dtype == torch.int64), _p(dy), _p(dw), n, dy.shape[-1], _stream())
+        _lib.call("tfb_embedding_bwd", _p(idx), int(idx.dtype == torch.int64), _p(dy), _p(dw), n, dy.shape[-1], V,
+                  _stream())
         return dw
     scr = _scratch(dw.device, _lib.lib().tfb_embedding_bwd_scratch_ints(n, V))  # 4-byte elements, used as int32
     _lib.call("tfb_embedding_bwd_grouped", _p(idx), int(idx.dtype == torch.int64), _p(dy), _p(dw), n, dy.shape[-1], V,

@@ -382,9 +382,17 @@ def adamw_fused_step(opt) -> bool:
                 continue
             gr = p.grad
             if (not p.is_cuda or p.dtype != torch.float32 or not p.is_contiguous() or not gr.is_contiguous()
-                    or gr.shape != p.shape or gr.dtype not in (torch.float32, bf16)):
+                    or gr.shape != p.shape or gr.dtype not in (torch.float32, bf16) or p.numel() == 0
+                    or p.data_ptr() % 16 or gr.data_ptr() % (16 if gr.dtype == torch.float32 else 8)):
                 return False
+            st = opt.state.get(p, {})
+            for key in ("exp_avg", "exp_avg_sq"):
+                t = st.get(key)
+                if t is not None and (t.dtype != torch.float32 or t.device != p.device or t.shape != p.shape
+                                      or not t.is_contiguous() or t.data_ptr() % 16):
+                    return False
             todo.append((g, p))
+    # every (group, parameter) has passed: nothing below can refuse, so the optimizer is never left half-stepped
     for g, p in todo:
         st = opt.state[p]
         if len(st) == 0:
@@ -394,6 +402,9 @@ def adamw_fused_step(opt) -> bool:
         n = int(st["step"]) + 1
         b1, b2 = g["betas"]
         ops.adamw_(p, p.grad, st["exp_avg"], st["exp_avg_sq"], n, float(g["lr"]), b1, b2, g["eps"], g["weight_decay"])
+        # the kernel wrote p behind autograd's back: bump its version as the reference does after its raw kernel write
+        # (R1 optk_adamw_fused_step), so caches keyed on p._version (the per-step fp8 weight cache) see the update
+        torch.autograd.graph.increment_version(p)
         if torch.is_tensor(st["step"]):
             st["step"] += 1
         else:
