@@ -5,7 +5,8 @@
  *   - every pointer is a DEVICE pointer unless the comment says "host"; bf16 tensors are raw 16-bit words,
  *     fp8 tensors raw bytes (OCP e4m3fn / e5m2), row-major, contiguous unless strides are passed;
  *   - `stream` is a hipStream_t; kernels are launched on it and the call returns without synchronising;
- *   - no entry point allocates, frees or synchronises; scratch and workspaces are caller-owned;
+ *   - no entry point allocates, frees or synchronises; scratch and workspaces are caller-owned (one exception:
+ *     tfb_attn_bwd_static keeps its scratch in a static device array of the library);
  *   - return value: 0 ok, 1 unsupported shape (the reference wrappers' "shapes_apply() is false": the caller runs
  *     its own fallback or raises), 2 bad argument, 3 launch failed, 4 workspace too small.
  *
@@ -249,6 +250,17 @@ int tfb_attn_bwd(const void* q, const long* q_strides, const void* k, const long
                  const long* v_strides, const void* o, const long* o_strides, const void* d_o, const long* do_strides,
                  void* dq, const long* dq_strides, void* dk, const long* dk_strides, void* dv, const long* dv_strides,
                  const void* lse, void* delta, int B, int H, int T, int D, float scale, void* stream);
+/* tfb_attn_bwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the same kernels and results, with the delta scratch taken from a static device
+ * array inside the library (8 MiB per GPU, held until the process ends) instead of from the caller. It allocates and
+ * frees nothing. B * H * T <= tfb_attn_bwd_static_max_rows() (1,048,576), otherwise status 4 and the caller uses
+ * tfb_attn_bwd. All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams) race.
+ * Has no counterpart in the reference (its kernels allocate their own outputs and scratch through the NKI runtime). */
+long tfb_attn_bwd_static_max_rows(void);
+int tfb_attn_bwd_static(const void* q, const long* q_strides, const void* k, const long* k_strides, const void* v,
+                        const long* v_strides, const void* o, const long* o_strides, const void* d_o, const long* do_strides,
+                        void* dq, const long* dq_strides, void* dk, const long* dk_strides, void* dv, const long* dv_strides,
+                        const void* lse, int B, int H, int T, int D, float scale, void* stream);
 /* The same, with the inverse RoPE rotation (cos_t, sin_t bf16 [T][D/2]) applied to dq and dk on their way out: the
  * backward half of attention over a rotated fused projection. D == 64; TFB_ERR_SHAPE otherwise (caller runs tfb_rope).
  * Replaces NkiRopeAttnFn.backward / s2attn::rope_attn_bwd (round1/source/train.py:8135; round2/source/train.py:5040). */

@@ -17,7 +17,7 @@ def _declared():
     src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
     decls = {}
     for m in re.finditer(r"\b(int|long)\s+(tfb_\w+)\s*\(([^;]*?)\)\s*;", src, flags=re.S):
-        args = [a.strip() for a in m.group(3).split(",") if a.strip()]
+        args = [a.strip() for a in m.group(3).split(",") if a.strip() and a.strip() != "void"]
         decls[m.group(2)] = (m.group(1), args)
     return decls
 

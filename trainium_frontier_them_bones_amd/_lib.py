@@ -46,6 +46,9 @@ SIGNATURES = {
                           _i, _i, _i, _i, _f, _i, _vp],
     "tfb_attn_bwd": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _vp, _i, _i, _i, _i,
                      _f, _vp],
+    "tfb_attn_bwd_static": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _i, _i, _i, _i,
+                            _f, _vp],
+    "tfb_attn_bwd_static_max_rows": [],
     "tfb_attn_bwd_rope": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _vp, _vp, _vp,
                           _i, _i, _i, _i, _f, _vp],
     "tfb_qkv_rope_fwd": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
@@ -88,7 +91,7 @@ SIGNATURES = {
     "tfb_mlp_dw_proj": [_vp, _vp, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
 }
 
-_LONG_RESULT = {"tfb_mlp8_scale_scratch_floats", "tfb_moe_max_rows", "tfb_embedding_bwd_scratch_ints", "tfb_ns5_workspace_bytes"}
+_LONG_RESULT = {"tfb_attn_bwd_static_max_rows", "tfb_mlp8_scale_scratch_floats", "tfb_moe_max_rows", "tfb_embedding_bwd_scratch_ints", "tfb_ns5_workspace_bytes"}
 
 STATUS = {0: "ok", 1: "unsupported shape", 2: "bad argument", 3: "kernel launch failed", 4: "workspace too small"}
 

@@ -716,3 +716,44 @@ extern "C" int tfb_attn_bwd(const void* q, const long* qs, const void* k, const 
   return tfb_attn_bwd_rope(q, qs, k, ks, v, vs, o, os, go, gos, dq, dqs, dk, dks, dv, dvs, lse, delta, nullptr, nullptr, B, H, T,
                            D, scale, stream);
 }
+
+// ---- attention backward for callers that cannot allocate --------------------------------------------------------------
+// tfb_attn_bwd needs fp32 [2][B*H][T] of device scratch (the row statistics its pre-pass leaves for the two gradient
+// kernels) and takes it from the caller. Code under HIP graph capture, tight serving loops and harnesses that forbid
+// hipMalloc cannot provide one, so this variant keeps that scratch in the library's own image: a file-scope device
+// array of TFB_ATTN_STATIC_ROWS * 2 floats (8 MiB, held by every GPU the library runs on until the process ends).
+// In host code the array's name is only a stand-in for the symbol: its per-device address comes from
+// hipGetSymbolAddress, once per device, and that pointer - never the name - is what the kernels receive.
+// Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams) race on it. The pre-pass
+// writes every element the gradient kernels read, so nothing has to be cleared between calls.
+#define TFB_ATTN_STATIC_ROWS (1L << 20)
+#define TFB_MAX_DEVICES 64
+static __device__ __align__(256) float scratch[2 * TFB_ATTN_STATIC_ROWS];
+static float* volatile scratch_ptr[TFB_MAX_DEVICES];
+
+static int attn_static_scratch(float** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= TFB_MAX_DEVICES) return TFB_ERR_ARG;
+  float* p = scratch_ptr[dev];
+  if (!p) {
+    // (two threads racing here both ask for the same address: the second store is the first one again)
+    if (hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return TFB_ERR_LAUNCH;
+    scratch_ptr[dev] = p;
+  }
+  *out = p;
+  return TFB_OK;
+}
+
+extern "C" long tfb_attn_bwd_static_max_rows(void) { return TFB_ATTN_STATIC_ROWS; }
+
+extern "C" int tfb_attn_bwd_static(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
+                                   const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs,
+                                   void* dk, const long* dks, void* dv, const long* dvs, const void* lse, int B, int H, int T,
+                                   int D, float scale, void* stream) {
+  if (B <= 0 || H <= 0 || T <= 0) return TFB_ERR_SHAPE;
+  if ((long)B * H * T > TFB_ATTN_STATIC_ROWS) return TFB_ERR_WORKSPACE;  // beyond the static scratch: use tfb_attn_bwd
+  float* delta = nullptr;
+  const int st = attn_static_scratch(&delta);
+  if (st != TFB_OK) return st;
+  return tfb_attn_bwd(q, qs, k, ks, v, vs, o, os, go, gos, dq, dqs, dk, dks, dv, dvs, lse, delta, B, H, T, D, scale, stream);
+}

@@ -494,6 +494,27 @@ def attn_bwd(q, k, v, o, do, lse, scale, layout="bhtd", dq=None, dk=None, dv=Non
     return dq, dk, dv
 
 
+def attn_bwd_static_max_rows():
+    """The largest B * H * T attn_bwd_static takes (the size of the library's static scratch array)."""
+    return int(_lib.lib().tfb_attn_bwd_static_max_rows())
+
+
+def attn_bwd_static(q, k, v, o, do, lse, scale, dq, dk, dv, layout="bhtd", out_layout="bhtd"):
+    """attn_bwd into caller-provided dq, dk, dv through the entry point that allocates nothing: its row-statistic scratch
+    is a static device array inside the library (B * H * T <= tfb_attn_bwd_static_max_rows(); TfbError status 4 beyond).
+    Calls that overlap on one GPU share that array and race; this wrapper creates no tensor either."""
+    for t in (q, k, v, o, do, dq, dk, dv):
+        _attn_chk(t)
+    if layout == "bhtd":
+        B, H, T, D = q.shape
+    else:
+        B, T, H, D = q.shape
+    _lib.call("tfb_attn_bwd_static", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o),
+              _bht(o, "bthd"), _p(do), _bht(do, "bthd"), _p(dq), _bht(dq, out_layout), _p(dk), _bht(dk, out_layout), _p(dv),
+              _bht(dv, out_layout), _p(lse), B, H, T, D, float(scale), _stream())
+    return dq, dk, dv
+
+
 # ------------------------------------------------------------------------------------------ elementwise
 def relu2(x):
     _chk(x)
