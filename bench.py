@@ -38,20 +38,106 @@ def flops_per_token(cfg):
     return 6 * mm + 12 * L * cfg.n_head * cfg.head_dim * (cfg.seq_len // 2)
 
 
-def cpu_baseline(cfg, init_values):
-    """The oracle model's step on the host cores, on ONE sequence of the same 16 x 2048 batch."""
+def cpu_baseline_and_parity(cfg, dev):
+    """The oracle model's step on the host cores, on ONE sequence of the benchmark's first batch, timed; and the parity
+    gate in the same pass: a fresh HIP model with the same initial weights takes the same two steps on the same
+    sequence and the losses are compared (step 1 = the oracle's untimed warm-up repetition, step 2 = the timed one)."""
     import torch
     from oracle.model import OracleGPT
-    from trainium_frontier_them_bones_amd.model import zipf_tokens
-    cores = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(cores)
-    o = OracleGPT(cfg, init_values)
+    from trainium_frontier_them_bones_amd.model import GPT, zipf_tokens
+    host = os.cpu_count() or 1
+    threads = min(host, 16)            # the GPU box gives one GPU's job 16 cores, whatever os.cpu_count() shows
+    torch.set_num_threads(threads)
+    m = GPT(cfg, dev, seed=0)
+    o = OracleGPT(cfg, m.init_values)
     idx, tg = zipf_tokens(16, cfg.seq_len, cfg.vocab, seed=0)
+    idx, tg = idx[:1], tg[:1]
+    gpu = [m.train_step(idx.to(dev), tg.to(dev)).item() for _ in range(2)]
+    cpu = [o.train_step(idx, tg).item()]                     # untimed warm-up repetition
     t0 = time.perf_counter()
-    o.train_step(idx[:1], tg[:1])
+    cpu.append(o.train_step(idx, tg).item())
     dt = time.perf_counter() - t0
-    return {"value": round(cfg.seq_len / dt, 2), "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": "1 of the 16 sequences (2048 tokens) through the full 12-layer model, fwd+bwd+AdamW, 1 repetition"}
+    rel = [abs(a - b) / abs(b) for a, b in zip(gpu, cpu)]
+    base = {"value": round(cfg.seq_len / dt, 2), "unit": "tokens/s", "cores": threads, "host_cpus": host, "kind": "port",
+            "sample": "1 of the 16 sequences (2048 tokens) through the full 12-layer model, fwd+bwd+AdamW; 1 untimed "
+                      "warm-up step, then 1 timed step (%.1f s)" % dt}
+    parity = {"loss_rel": round(max(rel), 6), "tolerance": 1e-3, "gpu_loss": [round(v, 5) for v in gpu],
+              "oracle_loss": [round(v, 5) for v in cpu],
+              "what": "HIP model vs CPU oracle, same initial weights, same 2048-token sequence, steps 1 and 2"}
+    return base, parity
+
+
+# ---- per-kernel roofline table: algorithmic work of one call of an entry point, from the arguments of the call --------
+PEAK_FP8_TFLOPS = 5000.0
+PEAK_HBM_GBS = 8000.0
+
+
+def _work(name, a):
+    """(label, bound, work) for one call: flop for "mfma" rows (against the bf16 or fp8 peak), bytes for "hbm" rows."""
+    if name == "tfb_attn_bwd_rope":          # ..., B, H, T, D, scale, stream
+        B, H, T, D = a[-6:-2]
+        return "attention backward", "mfma", 5.0 * B * H * T * T * D
+    if name == "tfb_attn_fwd":
+        B, H, T, D = a[-6:-2]
+        return "attention forward", "mfma", 2.0 * B * H * T * T * D
+    if name == "tfb_qkv_rope_fwd":           # x, w, cos, sin, out, M, N, K, T, rot, stream
+        M, N, K = a[5:8]
+        return "QKV projection + RoPE %dx%dx%d" % (M, N, K), "mfma", 2.0 * M * N * K
+    if name == "tfb_gemm_bf16":              # A, B, C, M, N, K, ta, tb, ...
+        M, N, K, ta, tb = a[3:8]
+        return "bf16 GEMM %dx%dx%d %s%s" % (M, N, K, "T" if ta else "N", "T" if tb else "N"), "mfma", 2.0 * M * N * K
+    if name == "tfb_gemm_bf16_res":          # A, B, res, C, M, N, K, tb, stream
+        M, N, K = a[4:7]
+        return "bf16 GEMM + residual %dx%dx%d" % (M, N, K), "mfma", 2.0 * M * N * K
+    if name in ("tfb_mlp8_fwd", "tfb_mlp8_fwd_res", "tfb_mlp8_bwd", "tfb_mlp8_bwd_q"):
+        M, d, F = a[-4:-1]
+        return {"tfb_mlp8_fwd": "fp8 MLP forward", "tfb_mlp8_fwd_res": "fp8 MLP forward (+ residual)",
+                "tfb_mlp8_bwd": "fp8 MLP backward", "tfb_mlp8_bwd_q": "fp8 MLP backward (+ e4m3 h)"}[name], "mfma8", 4.0 * M * d * F
+    if name == "tfb_mlp8_dw8":               # ..., M, d, F, out_f32, accumulate, ws, ws_bytes, stream
+        M, d, F = a[8:11]
+        return "fp8 MLP weight gradients", "mfma8", 4.0 * M * d * F
+    if name == "tfb_mlp_dw_proj":            # dy, r, dw, M, d, F, ...
+        M, d, F = a[3:6]
+        return "bf16 dW_proj (h = r^2 in the loader)", "mfma", 2.0 * M * d * F
+    if name == "tfb_lmhead_fwd":             # ..., rows, d, V, softcap, stream
+        N, d, V = a[-5:-2]
+        return "LM head forward + lse", "mfma", 2.0 * N * d * V
+    if name == "tfb_loss_bwd":               # ..., rows, V, softcap, stream
+        N, V = a[-4:-2]
+        return "loss backward (dlogits in place)", "hbm", 2.0 * N * V * 2
+    if name in ("tfb_rmsnorm_fwd", "tfb_rmsnorm_fwd_q"):
+        rows, C = a[-4:-2]
+        return "RMSNorm forward", "hbm", rows * C * (2 * 2 + (1 if name.endswith("_q") else 0)) + 4.0 * rows
+    if name == "tfb_rmsnorm_bwd":
+        rows, C = a[-3:-1]
+        return "RMSNorm backward", "hbm", rows * C * 2 * (4 if a[1] else 3)
+    if name == "tfb_adamw":                  # p, g, g_f32, m, v, p16, n, ...
+        n, gf32 = a[6], a[2]
+        return "AdamW", "hbm", n * (24.0 if gf32 else 22.0)
+    return name, None, 0.0
+
+
+def per_kernel_table(rec, steps, top=8):
+    """rec: (start, end, name, args) of every entry-point call over `steps` steps -> the `top` rows by time per step."""
+    rows = {}
+    for s, e, name, a in rec:
+        label, bound, work = _work(name, a)
+        r = rows.setdefault(label, {"kernel": label, "bound": bound, "ms": 0.0, "work": 0.0, "calls": 0})
+        r["ms"] += s.elapsed_time(e)
+        r["work"] += work
+        r["calls"] += 1
+    out = []
+    total = sum(r["ms"] for r in rows.values())
+    for r in sorted(rows.values(), key=lambda r: -r["ms"])[:top]:
+        peak = {"mfma": PEAK_BF16_TFLOPS * 1e12, "mfma8": PEAK_FP8_TFLOPS * 1e12, "hbm": PEAK_HBM_GBS * 1e9}.get(r["bound"])
+        row = {"kernel": r["kernel"], "bound": {"mfma8": "mfma"}.get(r["bound"], r["bound"]),
+               "ms_per_step": round(r["ms"] / steps, 3), "calls_per_step": r["calls"] // steps,
+               "share_of_timed": round(r["ms"] / total, 3)}
+        if peak and r["ms"] > 0:
+            row["frac"] = round(r["work"] / (r["ms"] * 1e-3) / peak, 4)
+            row["peak"] = "fp8 5.0 PFLOP/s" if r["bound"] == "mfma8" else ("bf16 2.5 PFLOP/s" if r["bound"] == "mfma" else "HBM 8 TB/s")
+        out.append(row)
+    return out
 
 
 def traffic_probe():
@@ -187,8 +273,8 @@ def config_probe(which):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true")
     ap.add_argument("--ns-probe", action="store_true")
@@ -210,6 +296,8 @@ def main():
         config_probe(args.config_probe)
         return
 
+    import statistics
+
     import torch
     from trainium_frontier_them_bones_amd import _lib
     from trainium_frontier_them_bones_amd.model import GPT, GPTConfig, zipf_tokens
@@ -221,30 +309,44 @@ def main():
     cfg.fuse_residual = not args.unfused_residual
     model = GPT(cfg, dev, seed=0)
     B = 16
-    idx, tg = zipf_tokens(B, cfg.seq_len, cfg.vocab, seed=0)
-    idx, tg = idx.to(dev), tg.to(dev)
-    for _ in range(args.warmup):
-        model.train_step(idx, tg)
+    # four distinct Zipf batches, resident in HBM, taken in turn: no step sees the buffers of the step before it
+    batches = [tuple(t.to(dev) for t in zipf_tokens(B, cfg.seq_len, cfg.vocab, seed=s)) for s in range(4)]
+    for i in range(args.warmup):
+        model.train_step(*batches[i % 4])
     torch.cuda.synchronize()
 
     rec = []
     _lib.TIMED["tfb_attn_bwd_rope"] = rec
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        loss = model.train_step(idx, tg)
+    marks[0].record()
+    for i in range(args.steps):
+        loss = model.train_step(*batches[i % 4])
+        marks[i + 1].record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     del _lib.TIMED["tfb_attn_bwd_rope"]
     tokens = B * cfg.seq_len
     ms = dt / args.steps * 1e3
+    ms_median = statistics.median(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
 
     # dominant entry point: attention backward (three launches: D = sum dO*O, dK/dV, dQ), timed with events on its stream
     if not rec:
         raise RuntimeError("the timed entry point was never called: roofline.achieved would be meaningless")
-    k_ms = sum(s.elapsed_time(e) for s, e in rec) / len(rec)
+    k_ms = sum(r[0].elapsed_time(r[1]) for r in rec) / len(rec)
     H, D, T = cfg.n_head, cfg.head_dim, cfg.seq_len
     k_flops = 5 * B * H * T * T * D   # causal-halved: 5 matmuls x 2 flop x 1/2
     achieved = k_flops / (k_ms * 1e-3) / 1e12 if k_ms > 0 else 0.0
+
+    # every entry point of the step, timed with events in three further (untimed) steps: the per-kernel table
+    allrec = []
+    _lib.TIMED["*"] = allrec
+    for i in range(3):
+        model.train_step(*batches[i % 4])
+    torch.cuda.synchronize()
+    del _lib.TIMED["*"]
+    table = per_kernel_table(allrec, 3)
+
     out = {
         "metric": "train tokens/s, 12L d768 T2048 fwd+bwd step; per-kernel % MFMA/HBM peak",
         "value": round(tokens / (dt / args.steps), 1),
@@ -253,11 +355,12 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms, 3),
+        "ms_per_step_median": round(ms_median, 3),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16 (fp8 e4m3/e5m2 MLP GEMMs)",
-        "data": "synthetic: Zipf(1.1) token ids, N(0, 0.02) random-init weights",
+        "data": "synthetic: 4 distinct batches of Zipf(1.1) token ids taken in turn, N(0, 0.02) random-init weights",
         "config": {"workload": "C4 full step: 12 layers, d_model 768, 12 heads x 64, MLP 3072 squared-ReLU fp8, RMSNorm "
                                "pre-norm, RoPE, untied head, vocab 32768; batch 16 x 2048 tokens; fwd+bwd+AdamW"
                                + ("; MLP weight gradients in fp8 too (--fp8-dw)" if args.fp8_dw else "")
@@ -270,10 +373,14 @@ def main():
         "roofline": {"kernel": "attention backward (tfb_attn_bwd_rope: attn64_delta + attn64_dkdv + attn64_dq), B16 H12 T2048 D64", "bound": "mfma",
                      "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": ATTN_BWD_TRAFFIC_BYTES,
-                     "launch_ms": round(k_ms, 4), "launches_timed": len(rec)},
+                     "traffic_source": "constant from profiles/attn_c2_hbm_traffic.md (rocprofv3 --pmc), not measured in this run",
+                     "launch_ms": round(k_ms, 4), "launches_timed": len(rec),
+                     "per_kernel": table},
     }
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(cfg, model.init_values)
+        del model
+        torch.cuda.empty_cache()
+        out["cpu_baseline"], out["parity"] = cpu_baseline_and_parity(cfg, dev)
     print(json.dumps(out))
 
 

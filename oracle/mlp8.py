@@ -89,9 +89,10 @@ def forward_scales(w_fc, w_proj, e4m3_limit=E4M3_LIMIT_REF, x_scale=X_SCALE):
                         amax_a, amax_b])
 
 
-def backward_scales(dy2, row):
-    """The backward call's row: the forward row with s_dy, dq_dh2, s_dp, dq_dx filled from this call's dy."""
-    amax = dy2.detach().abs().amax().float()
+def backward_scales(dy2, row, amax=None):
+    """The backward call's row: the forward row with s_dy, dq_dh2, s_dp, dq_dx filled from this call's dy (from a given
+    amax instead when the caller holds only part of the rows the scales are taken over)."""
+    amax = dy2.detach().abs().amax().float() if amax is None else torch.as_tensor(amax, dtype=torch.float32)
     s_dy, i_dy = pow2_floor_scale(amax, E5M2_LIMIT / DY_HEADROOM, *EXP_G)
     bound = torch.sqrt(row[COL["rho2"]] * row[COL["kappa2"]]) * amax * (DP_BOUND * dy2.shape[1])
     s_dp, i_dp = pow2_floor_scale(bound, E5M2_LIMIT, *EXP_G)

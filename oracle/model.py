@@ -125,25 +125,33 @@ class OracleGPT:
             y = F.linear(torch.relu(F.linear(h2, w_fc)).square(), w_proj)
         return y.view(h.shape)
 
+    def block(self, i, x):
+        """One pre-norm block on the residual stream x [B, T, d]: x + attention(norm1(x)), then + MLP(norm2(.))."""
+        return self.mlp_half(i, self.attention_half(i, x))
+
+    def mlp_half(self, i, x):
+        h = _RMSNorm.apply(x, self.p["norm2.%d" % i], self.cfg.norm_eps)
+        return x + self.mlp(h, i)
+
+    def attention_half(self, i, x):
+        cfg, p = self.cfg, self.p
+        B, T, _ = x.shape
+        H, D = cfg.n_head, cfg.head_dim
+        cos, sin = self.cos[:T], self.sin[:T]
+        h = _RMSNorm.apply(x, p["norm1.%d" % i], cfg.norm_eps)
+        qkv = F.linear(h, p["w_qkv.%d" % i])
+        q, k, v = (t.reshape(B, T, H, D) for t in qkv.split(cfg.d_model, dim=-1))
+        q, k = _Rope.apply(q, cos, sin), _Rope.apply(k, cos, sin)
+        o = _Attention.apply(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), 1.0 / math.sqrt(D))
+        att = F.linear(o.reshape(B, T, cfg.d_model), p["w_o.%d" % i])
+        return x + att
+
     def forward(self, idx, targets):
         cfg, p = self.cfg, self.p
-        B, T = idx.shape
-        H, D = cfg.n_head, cfg.head_dim
-        scale = 1.0 / math.sqrt(D)
-        cos, sin = self.cos[:T], self.sin[:T]
         x = F.embedding(idx, p["wte"])
-        h = _RMSNorm.apply(x, p["norm1.0"], cfg.norm_eps)
         for i in range(cfg.n_layer):
-            qkv = F.linear(h, p["w_qkv.%d" % i])
-            q, k, v = (t.reshape(B, T, H, D) for t in qkv.split(cfg.d_model, dim=-1))
-            q, k = _Rope.apply(q, cos, sin), _Rope.apply(k, cos, sin)
-            o = _Attention.apply(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), scale)
-            att = F.linear(o.reshape(B, T, cfg.d_model), p["w_o.%d" % i])
-            x = x + att
-            h = _RMSNorm.apply(x, p["norm2.%d" % i], cfg.norm_eps)
-            x = x + self.mlp(h, i)
-            nw = p["norm1.%d" % (i + 1)] if i + 1 < cfg.n_layer else p["norm_f"]
-            h = _RMSNorm.apply(x, nw, cfg.norm_eps)
+            x = self.block(i, x)
+        h = _RMSNorm.apply(x, p["norm_f"], cfg.norm_eps)
         logits = F.linear(h, p["lm_head"])
         return _Loss.apply(logits.reshape(-1, cfg.vocab), targets.reshape(-1), cfg.softcap or None)
 

@@ -25,15 +25,23 @@ def route(h2, router, topk, bias=None):
     if bias is not None:
         logits = logits + bias.float()
     p = torch.softmax(logits, dim=-1)
+    idx, gate = select(p, topk)
+    return p, idx, gate, logits
+
+
+def select(p, topk):
+    """(idx [N, k] int64, gate [N, k] fp32) from probabilities p [N, E]: the reference's tournament
+    (round2/source/train.py:10505 moe_tournament: the largest value wins, exact ties go to the LOWER expert index),
+    the second choice the same over the rest, gates renormalised over the two (the probability itself at k = 1)."""
     i1 = torch.argmax(p, dim=-1)                      # first maximum: ties go to the lower index
     v1 = p.gather(1, i1[:, None]).squeeze(1)
     if topk == 1:
-        return p, i1[:, None], v1[:, None], logits
+        return i1[:, None], v1[:, None]
     masked = p.masked_fill(F.one_hot(i1, p.shape[1]).bool(), -1.0)
     i2 = torch.argmax(masked, dim=-1)
     v2 = p.gather(1, i2[:, None]).squeeze(1)
     den = v1 + v2
-    return p, torch.stack([i1, i2], 1), torch.stack([v1 / den, v2 / den], 1), logits
+    return torch.stack([i1, i2], 1), torch.stack([v1 / den, v2 / den], 1)
 
 
 def tables(idx, E):
@@ -57,22 +65,27 @@ def tables(idx, E):
 
 class _ExpertMlp8(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x2, w_fc, w_proj, row, x_scale):
+    def forward(ctx, x2, w_fc, w_proj, row, x_scale, dy_amax=None):
         y, r = omlp.forward(x2, w_fc, w_proj, row, x_scale)
         ctx.save_for_backward(x2, r, w_fc, w_proj, row)
+        ctx.dy_amax = dy_amax
         return y
 
     @staticmethod
     def backward(ctx, dy):
         x2, r, w_fc, w_proj, row = ctx.saved_tensors
         dy = dy.contiguous()
-        dx, h, dpre = omlp.backward(dy, r, w_fc, w_proj, omlp.backward_scales(dy, row))
+        # the expert's backward scales come from the amax of ITS rows of dy; a caller that runs only a slice of those
+        # rows passes the amax over all of them (dy_amax), so the slice is rounded exactly as inside the whole layer
+        dx, h, dpre = omlp.backward(dy, r, w_fc, w_proj, omlp.backward_scales(dy, row, ctx.dy_amax))
         dw_fc, dw_proj = omlp.weight_grads(dy, x2, h, dpre)
-        return dx, dw_fc, dw_proj, None, None
+        return dx, dw_fc, dw_proj, None, None, None
 
 
-def moe_forward(h, router, w_fc, w_proj, topk, bias=None, fp8=True, e4m3_limit=240.0, x_scale=4.0):
-    """h [.., d] bf16; router [E, d]; w_fc [E, F, d]; w_proj [E, d, F]. Differentiable (autograd) in h, router, weights."""
+def moe_forward(h, router, w_fc, w_proj, topk, bias=None, fp8=True, e4m3_limit=240.0, x_scale=4.0, dys_amax=None):
+    """h [.., d] bf16; router [E, d]; w_fc [E, F, d]; w_proj [E, d, F]. Differentiable (autograd) in h, router, weights.
+    dys_amax (optional, fp32 [E]): per-expert amax of the expert outputs' gradients to take the backward scales from,
+    for a call that holds only some of the layer's tokens."""
     d = h.shape[-1]
     h2 = h.reshape(-1, d)
     E = w_fc.shape[0]
@@ -87,7 +100,8 @@ def moe_forward(h, router, w_fc, w_proj, topk, bias=None, fp8=True, e4m3_limit=2
             continue
         if fp8:
             row = omlp.forward_scales(w_fc[e].detach(), w_proj[e].detach(), e4m3_limit, x_scale)
-            outs.append(_ExpertMlp8.apply(xe, w_fc[e], w_proj[e], row, x_scale))
+            outs.append(_ExpertMlp8.apply(xe, w_fc[e], w_proj[e], row, x_scale,
+                                          None if dys_amax is None else dys_amax[e]))
         else:
             outs.append(F.linear(torch.relu(F.linear(xe, w_fc[e])).square(), w_proj[e]))
     ys = torch.cat(outs, 0)

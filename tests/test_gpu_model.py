@@ -19,18 +19,66 @@ def test_small_model_losses_and_gradients_track_oracle(dev):
     lo = o.forward(idx, tg)
     lo.backward()
     assert abs(loss.item() - lo.item()) < 1e-3 * lo.item()
-    # end-to-end gradients compound bf16 / fp8 rounding differences through the layers; the per-kernel tests hold the
-    # tight tolerances, here the last layers must agree closely and the first ones within a few percent
+    # the head's gradients: its operand is the stream after every fp8 block, so the fp8 path's bar; the blocks themselves
+    # are held, one by one and without compounding, by test_each_block_against_the_oracle_on_the_blocks_own_inputs
     assert rel_l2(m.p["lm_head"].grad_buf, o.p["lm_head"].grad) < 2e-2
     assert rel_l2(m.p["norm_f"].grad_buf, o.p["norm_f"].grad) < 2e-2
-    for name in ("w_qkv.0", "w_fc.0", "wte"):
-        assert rel_l2(m.p[name].grad_buf, o.p[name].grad) < 8e-2, name
     m2, o2 = GPT(cfg, dev, seed=1), OracleGPT(cfg, m.init_values)
     for _ in range(4):
         a = m2.train_step(idx.to(dev), tg.to(dev)).item()
         b = o2.train_step(idx, tg).item()
         assert abs(a - b) < 1e-3 * b
     assert a < 6.5                                                  # it learns
+
+
+def test_each_half_block_against_the_oracle_on_its_own_inputs(dev):
+    """No compounding: each half of every block of the HIP model (attention with its norm and projections; the fp8 MLP
+    with its norm) is compared with the oracle's half fed the HIP half's OWN input stream and the HIP model's OWN gradient
+    of its output stream. The attention half is a bf16 path: output, input gradient and the gradients of norm1, w_qkv, w_o
+    within 5e-3. The MLP half is the fp8 path: output, input gradient and the gradients of norm2, w_fc, w_proj within 2e-2."""
+    from oracle.model import OracleGPT
+    from trainium_frontier_them_bones_amd.model import GPT, GPTConfig, zipf_tokens
+    cfg = GPTConfig(n_layer=3, d_model=256, n_head=4, d_ff=1024, vocab=1024, seq_len=256)
+    m = GPT(cfg, dev, seed=1)
+    o = OracleGPT(cfg, m.init_values)
+    idx, tg = zipf_tokens(2, 256, cfg.vocab, seed=3)
+    m.trace = []
+    m.zero_grad()
+    m.backward(m.forward(idx.to(dev), tg.to(dev)))
+    assert len(m.trace) == 2 * cfg.n_layer + 1
+    halves = (("attention", o.attention_half, ("norm1", "w_qkv", "w_o"), 5e-3), ("mlp", o.mlp_half, ("norm2", "w_fc", "w_proj"), 2e-2))
+    for i in range(cfg.n_layer):
+        for j, (what, fn, names, tol) in enumerate(halves):
+            print("block %d %s half" % (i, what), flush=True)
+            t_in, t_out = m.trace[2 * i + j], m.trace[2 * i + j + 1]
+            for t in o.p.values():
+                t.grad = None
+            x_in = t_in.detach().cpu().clone().requires_grad_(True)
+            x_out = fn(i, x_in)
+            assert rel_l2(t_out, x_out) < tol, (i, what)
+            x_out.backward(t_out.grad.cpu())
+            assert rel_l2(t_in.grad, x_in.grad) < tol, (i, what)
+            for name in names:
+                key = "%s.%d" % (name, i)
+                assert rel_l2(m.p[key].grad_buf, o.p[key].grad) < tol, key
+
+
+def test_full_size_model_on_one_sequence_against_the_oracle(dev):
+    """Configuration 4 of BASELINE.json at its real model size (12 layers, d 768, 12 heads, MLP 3072, vocab 32768) on ONE
+    sequence of 2048 tokens: the loss of the first step and, after one AdamW update of every parameter, of the second,
+    against the oracle model on the same tokens, within 1e-3 relative."""
+    from oracle.model import OracleGPT
+    from trainium_frontier_them_bones_amd.model import GPT, GPTConfig, zipf_tokens
+    cfg = GPTConfig()
+    m = GPT(cfg, dev, seed=0)
+    o = OracleGPT(cfg, m.init_values)
+    idx, tg = zipf_tokens(16, cfg.seq_len, cfg.vocab, seed=0)
+    idx, tg = idx[:1], tg[:1]
+    for step in range(2):
+        print("full-size model, one sequence, step %d" % step, flush=True)
+        a = m.train_step(idx.to(dev), tg.to(dev)).item()
+        b = o.train_step(idx, tg).item()
+        assert abs(a - b) < 1e-3 * b, (step, a, b)
 
 
 @pytest.mark.parametrize("fp8_attn", [False, True])

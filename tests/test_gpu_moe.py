@@ -28,7 +28,12 @@ def test_routing_tables_bit_exact(dev, topk, skew):
     po, io, go, lo = O.route(h, router, topk, bias)
     assert rel_l2(logits, lo) < 1e-5 and rel_l2(p, po) < 1e-5 and rel_l2(gate, go) < 1e-5
     agree = (idx.cpu().long() == io).all(1)
-    assert agree.float().mean().item() > 0.999           # only exact near-ties may pick differently
+    assert agree.float().mean().item() > 0.999           # against torch's own logits a near-tie may pick differently ...
+    # ... but the selection is index work: on the kernel's OWN probabilities the reference's rule (largest value, ties
+    # to the lower index, gates renormalised over the two) must give the kernel's picks and gates bit for bit
+    isel, gsel = O.select(p.cpu(), topk)
+    assert torch.equal(idx.cpu().long(), isel) and torch.equal(gate.cpu(), gsel)
+    assert rel_l2(p, torch.softmax(logits.cpu(), dim=-1)) < 1e-6
     tab = ops.moe_tables(idx, 8)
     slot, tok, seg = O.tables(idx.cpu().long(), 8)       # oracle tables from the kernel's own selections
     assert torch.equal(tab["seg"].cpu().long(), seg)
@@ -39,6 +44,34 @@ def test_routing_tables_bit_exact(dev, topk, skew):
     for e in range(8):
         assert bool((te[int(seg[e]) // 128:int(seg[e + 1]) // 128] == e).all())
     assert bool((te[R // 128:] == -1).all())
+
+
+@pytest.mark.parametrize("topk", [2, 1])
+def test_routing_exact_ties_go_to_the_lower_index(dev, topk):
+    """Router rows 1 and 4 are equal, and so are rows 2 and 6: their logits and probabilities tie exactly on every token.
+    The reference's tournament (round2/source/train.py:10505) gives a tie to the lower index, for the first choice and
+    for the second."""
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import ops
+    h, router, _, _, _ = _layer(9, 1024, 256, 512, 8)
+    router[4] = router[1]
+    router[6] = router[2]
+    p, idx, gate, logits = ops.moe_route(h.to(dev), router.to(dev), topk, None, want_logits=True)
+    pc, ic = p.cpu(), idx.cpu().long()
+    assert torch.equal(pc[:, 1], pc[:, 4]) and torch.equal(pc[:, 2], pc[:, 6])
+    isel, gsel = O.select(pc, topk)
+    assert torch.equal(ic, isel) and torch.equal(gate.cpu(), gsel)
+    first = ic[:, 0]
+    assert not bool(((first == 4) | (first == 6)).any())                  # the upper twin never wins the first place
+    assert int(((first == 1) | (first == 2)).sum()) > 100                 # and the tie does decide many tokens
+    if topk == 2:
+        # where the lower twin won, its equal upper twin is the runner-up (nothing is larger than the maximum)
+        assert bool((ic[first == 1, 1] == 4).all()) and bool((ic[first == 2, 1] == 6).all())
+        # where the twins tie for second place, the lower one takes it
+        assert not bool((((ic[:, 1] == 4) & (first != 1)) | ((ic[:, 1] == 6) & (first != 2))).any())
+    # and against torch's argmax on torch's own logits (exact ties are exact there too)
+    _, io, _, _ = O.route(h, router, topk)
+    assert (ic == io).all(1).float().mean().item() > 0.999
 
 
 @pytest.mark.parametrize("shape,topk,skew", [((1024, 256, 512, 8), 2, 0.0), ((1024, 256, 512, 4), 1, 0.0),
@@ -151,3 +184,66 @@ def test_moe_auxiliary_router_terms(dev):
     assert rel_l2(rd.grad, ro.grad) < 1e-2
     assert rel_l2(hd.grad, ho.grad) < 2e-2                              # one bf16 rounding of dh
     assert float(wfd.grad.abs().max()) == 0.0                           # no gradient reaches the experts through aux
+
+
+@pytest.mark.parametrize("skew", [0.0, 2.0])
+def test_moe_config5_full_size_backward(dev, skew):
+    """Configuration 5 at full size, forward AND backward (16384 tokens, d 1024, 8 experts top-2, FFN 2816; balanced and
+    with +2.0 on two experts' logits), against the oracle on parts it finishes in seconds: (1) one expert's whole row
+    segment (its activations, input gradient and BOTH weight gradients: the ragged token-contraction GEMMs over
+    thousands of rows), (2) the input gradient of 512 tokens routed to the most frequent expert pair, through autograd
+    of the oracle layer on those tokens with the backward scales taken from the full layer's per-expert amax."""
+    from oracle import mlp8 as O8
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import autograd as A
+    from trainium_frontier_them_bones_amd import ops
+    N, d, Fd, E = 16384, 1024, 2816, 8
+    h, router, wf, wp, bias = _layer(5, N, d, Fd, E, skew)
+    dout = torch.randn(N, d, generator=torch.Generator().manual_seed(6)).bfloat16()
+    hd, rd, wfd, wpd = (t.to(dev).requires_grad_(True) for t in (h, router, wf, wp))
+    st = A.Moe8State()
+    st.refresh(wfd, wpd)
+    b = bias.to(dev) if skew else None
+    print("config 5 full size fwd+bwd, skew %.1f" % skew, flush=True)
+    out = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, st, 2, b)
+    out.backward(dout.to(dev))
+    for t in (out, hd.grad, rd.grad, wfd.grad, wpd.grad):
+        assert bool(torch.isfinite(t.float()).all())
+    # the kernel's own routing (bit-checked against the reference's rule in the tests above) defines the segments
+    p, idx, gate, _ = ops.moe_route(hd.detach(), rd.detach(), 2, b)
+    idx, gate = idx.cpu().long(), gate.cpu()
+    slot, tok, seg = O.tables(idx, E)
+    ksel = torch.zeros_like(tok)
+    for j in range(2):
+        ksel[slot[:, j]] = j
+    rows_all = torch.nonzero(tok >= 0).flatten()
+    gate_rows = torch.zeros(tok.shape[0])
+    gate_rows[rows_all] = gate[tok[rows_all], ksel[rows_all]]
+    dys = (gate_rows.bfloat16()[:, None] * dout[tok.clamp_min(0)]) * (tok >= 0)[:, None]     # bf16(gate) * dout, bf16
+    amax = torch.stack([dys[seg[e]:seg[e + 1]].float().abs().amax() for e in range(E)])
+    # (1) the busiest expert's whole segment
+    cnt = seg[1:] - seg[:-1]
+    e = int(torch.argmax(cnt))
+    rows = torch.arange(int(seg[e]), int(seg[e + 1]))
+    rows = rows[tok[rows] >= 0]
+    xe, ge = h[tok[rows]], dys[rows]
+    row = O8.forward_scales(wf[e], wp[e])
+    ye, re = O8.forward(xe, wf[e], wp[e], row)
+    dxe, he, dpe = O8.backward(ge, re, wf[e], wp[e], O8.backward_scales(ge, row, amax[e]))
+    dwf, dwp = O8.weight_grads(ge, xe, he, dpe)
+    assert rel_l2(wfd.grad[e], dwf) < 2e-2 and rel_l2(wpd.grad[e], dwp) < 2e-2
+    assert rows.numel() > (3000 if not skew else 5000)                    # thousands of rows: the ragged long contraction
+    # (2) 512 tokens of the most frequent (unordered) expert pair, input gradient through the whole layer's backward
+    pair = torch.sort(idx, dim=1).values
+    key = pair[:, 0] * E + pair[:, 1]
+    best = int(torch.mode(key).values)
+    _, io, _, _ = O.route(h, router, 2, bias if skew else None)
+    same = (io == idx).all(1)                                             # (a near-tie on torch's own logits may differ)
+    S = torch.nonzero((key == best) & same).flatten()[:512]
+    assert S.numel() == 512
+    ho, ro = h[S].clone().requires_grad_(True), router.clone().requires_grad_(True)
+    oo, info = O.moe_forward(ho, ro, wf, wp, 2, bias if skew else None, dys_amax=amax)
+    assert torch.equal(info["idx"], idx[S])                               # (torch's logits pick the same experts here)
+    oo.backward(dout[S])
+    assert rel_l2(out[S], oo) < 2e-2
+    assert rel_l2(hd.grad[S], ho.grad) < 2e-2

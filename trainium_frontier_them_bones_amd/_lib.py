@@ -121,12 +121,17 @@ def lib():
 
 
 # name -> list: when an entry point is listed here every call is bracketed by events on torch's current stream
-# (the stream the kernels are launched on) and the (start, end) pair appended; used by the benchmark only.
+# (the stream the kernels are launched on) and (start, end, name, args) appended; the key "*" takes every entry point
+# not listed by name. Used by the benchmark only.
 TIMED = {}
 
 
 def call(name, *args):
-    rec = TIMED.get(name) if TIMED else None
+    rec = None
+    if TIMED:
+        rec = TIMED.get(name)
+        if rec is None:
+            rec = TIMED.get("*")
     if rec is None:
         st = getattr(lib(), name)(*args)
     else:
@@ -135,6 +140,6 @@ def call(name, *args):
         s.record()
         st = getattr(lib(), name)(*args)
         e.record()
-        rec.append((s, e))
+        rec.append((s, e, name, args))
     if st != 0:
         raise TfbError(name, st)

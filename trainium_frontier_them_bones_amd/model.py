@@ -121,6 +121,10 @@ class GPT:
         self.norm_grads = self.others.grad[o0:o0 + len(self.norm_names) * d].view(len(self.norm_names), d)
         self.norm_parts, self.norm_rows, self.norm_fresh = None, 0, True
         self.step_count = 0
+        # a list here makes the fused forward keep the residual stream after the embedding and after every residual add
+        # (with its gradient after the backward pass): [x0, x0 + attention, block 0's output, ...]; tests compare the
+        # two halves of every block on their own inputs
+        self.trace = None
         self.init_weights(seed)
 
     def init_weights(self, seed):
@@ -210,6 +214,12 @@ class GPT:
         elementwise passes per layer fewer."""
         cfg, p = self.cfg, self.p
         q8 = cfg.x_scale if cfg.fp8_attn_proj else None
+
+        def keep(t):
+            if self.trace is not None:
+                t.retain_grad()
+                self.trace.append(t)
+        keep(x)
         x, h, *h8 = A.RMSNormPassFn.apply(x, p["norm1.0"], cfg.norm_eps, q8)
         for i in range(cfg.n_layer):
             if cfg.fp8_attn_proj:
@@ -223,8 +233,10 @@ class GPT:
                     qkv = A.LinearFn.apply(h, p["w_qkv.%d" % i])
                     att = A.RopeAttentionFn.apply(qkv, self.cos[:T], self.sin[:T], cfg.n_head, scale)
                 x = A.LinearFn.apply(att, p["w_o.%d" % i], x)
+            keep(x)
             x, h, h8m = A.RMSNormPassFn.apply(x, p["norm2.%d" % i], cfg.norm_eps, cfg.x_scale)
             x = A.Mlp8Fn.apply(h, p["w_fc.%d" % i], p["w_proj.%d" % i], self.mlp_state[i], h8m, x)
+            keep(x)
             nw = p["norm1.%d" % (i + 1)] if i + 1 < cfg.n_layer else p["norm_f"]
             x, h, *h8 = A.RMSNormPassFn.apply(x, nw, cfg.norm_eps, q8 if i + 1 < cfg.n_layer else None)
         return A.LmHeadLossFn.apply(h, p["lm_head"], targets, cfg.softcap, "mean")
