@@ -1,9 +1,10 @@
 """Benchmark: train tokens/s of the 12-layer d768 T2048 step (fwd + bwd + AdamW) on one MI355X, entirely on the
 HIP kernels, with the roofline position of the dominant kernel and the CPU oracle timed beside it.
 
-python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--fp8-dw] [--unfused-residual]
-Prints ONE JSON line. --fp8-dw (not the default, not the headline configuration) also runs the MLP's two weight-gradient
-GEMMs in fp8, as the recipe of the reference's round1 sources does; the line's config then says so. --unfused-residual runs the same
+python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--bf16-dw] [--unfused-residual]
+Prints ONE JSON line. All six GEMMs of the MLP run in fp8 (e4m3 forward, e5m2 gradients; the weight gradients from the
+bytes the other GEMMs multiplied, as the reference's final recipe does); --bf16-dw keeps the MLP's two weight-gradient
+GEMMs in bf16 for comparison and the line's config then says so. --unfused-residual runs the same
 arithmetic with the residual adds and the MLP's fp8 operand cast as passes of their own (for comparison; same values).
 
 python bench.py --ns-probe        (Muon's Newton-Schulz call on the benchmark model's four stacks of 12 hidden matrices:
@@ -279,8 +280,9 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true")
     ap.add_argument("--ns-probe", action="store_true")
     ap.add_argument("--config-probe", choices=("c1", "c2", "c3", "c5", "all"))
-    ap.add_argument("--fp8-dw", action="store_true")
+    ap.add_argument("--bf16-dw", action="store_true")
     ap.add_argument("--unfused-residual", action="store_true")
+    ap.add_argument("--all-kernels", action="store_true", help="roofline.per_kernel lists every entry point, not the top 8")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -305,7 +307,7 @@ def main():
     _lib.lib()
     dev = torch.device("cuda:0")
     cfg = GPTConfig()
-    cfg.fp8_mlp_dw = bool(args.fp8_dw)
+    cfg.fp8_mlp_dw = not args.bf16_dw
     cfg.fuse_residual = not args.unfused_residual
     model = GPT(cfg, dev, seed=0)
     B = 16
@@ -345,7 +347,7 @@ def main():
         model.train_step(*batches[i % 4])
     torch.cuda.synchronize()
     del _lib.TIMED["*"]
-    table = per_kernel_table(allrec, 3)
+    table = per_kernel_table(allrec, 3, top=1000 if args.all_kernels else 8)
 
     out = {
         "metric": "train tokens/s, 12L d768 T2048 fwd+bwd step; per-kernel % MFMA/HBM peak",
@@ -363,7 +365,7 @@ def main():
         "data": "synthetic: 4 distinct batches of Zipf(1.1) token ids taken in turn, N(0, 0.02) random-init weights",
         "config": {"workload": "C4 full step: 12 layers, d_model 768, 12 heads x 64, MLP 3072 squared-ReLU fp8, RMSNorm "
                                "pre-norm, RoPE, untied head, vocab 32768; batch 16 x 2048 tokens; fwd+bwd+AdamW"
-                               + ("; MLP weight gradients in fp8 too (--fp8-dw)" if args.fp8_dw else "")
+                               + ("; MLP weight gradients in bf16 (--bf16-dw)" if args.bf16_dw else "; all six MLP GEMMs in fp8")
                                + ("; residual adds and fp8 casts as separate passes (--unfused-residual)"
                                   if args.unfused_residual else ""),
                    "global_batch": B, "seq_len": cfg.seq_len, "params": model.num_params(),

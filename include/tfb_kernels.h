@@ -193,7 +193,8 @@ int tfb_gemm_fp8_tn(const void* g8, int fmt_g, const void* a8, int fmt_a, const 
                     long M, int O, int D, int out_f32, int accumulate, void* workspace, long workspace_bytes, void* stream);
 
 /* tfb_mlp8_bwd that also writes hq8 [M][F] = e4m3(min(bf16(r^2) * s_h, hq_limit)) (NULL to skip): the g-side operand of
- * the fp8 weight gradient of w_proj (format E4M3C of nki_dw8.py:312-320; round2/source/train.py:8226). */
+ * the fp8 weight gradient of w_proj (format E4M3C of nki_dw8.py:312-320; round2/source/train.py:8226). dpre may be NULL
+ * here: with both weight gradients in fp8 (tfb_mlp8_dw8) nothing reads the bf16 dpre, only its bytes dp8. */
 int tfb_mlp8_bwd_q(const void* dy8, const void* r, const void* w8, const void* row, void* dx, void* h, void* dpre, void* dp8,
                    void* hq8, float hq_limit, long M, int d, int F, void* stream);
 

@@ -28,18 +28,23 @@ bf16 = torch.bfloat16
 
 class _Mlp8(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x2, w_fc, w_proj, row, x_scale):
+    def forward(ctx, x2, w_fc, w_proj, row, x_scale, dw_fp8_limit=None):
         y, r = omlp.forward(x2, w_fc, w_proj, row, x_scale)
         ctx.save_for_backward(x2, r, w_fc, w_proj, row)
+        ctx.x_scale, ctx.dw_fp8_limit = x_scale, dw_fp8_limit
         return y
 
     @staticmethod
     def backward(ctx, dy):
         x2, r, w_fc, w_proj, row = ctx.saved_tensors
         dy = dy.contiguous()
-        dx, h, dpre = omlp.backward(dy, r, w_fc, w_proj, omlp.backward_scales(dy, row))
-        dw_fc, dw_proj = omlp.weight_grads(dy, x2, h, dpre)
-        return dx, dw_fc, dw_proj, None, None
+        rowb = omlp.backward_scales(dy, row)
+        dx, h, dpre = omlp.backward(dy, r, w_fc, w_proj, rowb)
+        if ctx.dw_fp8_limit is None:
+            dw_fc, dw_proj = omlp.weight_grads(dy, x2, h, dpre)
+        else:   # both weight gradients in fp8 too (round2/source/train.py:8209 under its fp8 weight-gradient switch)
+            dw_fc, dw_proj = omlp.weight_grads_fp8(x2, dy, h, dpre, rowb, ctx.x_scale, ctx.dw_fp8_limit)
+        return dx, dw_fc, dw_proj, None, None, None
 
 
 class _Attention(torch.autograd.Function):
@@ -120,7 +125,8 @@ class OracleGPT:
         w_fc, w_proj = self.p["w_fc.%d" % i], self.p["w_proj.%d" % i]
         h2 = h.reshape(-1, h.shape[-1])
         if self.fp8:
-            y = _Mlp8.apply(h2, w_fc, w_proj, self.rows[i], self.cfg.x_scale)
+            y = _Mlp8.apply(h2, w_fc, w_proj, self.rows[i], self.cfg.x_scale,
+                            self.cfg.e4m3_limit if getattr(self.cfg, "fp8_mlp_dw", False) else None)
         else:
             y = F.linear(torch.relu(F.linear(h2, w_fc)).square(), w_proj)
         return y.view(h.shape)

@@ -425,7 +425,7 @@ class Mlp8Fn(torch.autograd.Function):
         g2 = gy.reshape(-1, gy.shape[-1]).contiguous()
         rowb = ops.mlp8_backward_scales(g2, st.row)
         if st.dw_fp8:
-            dx, _, dp8, hq8, dy8 = ops.mlp8_bwd_q(g2, r, st.w8, rowb, st.e4m3_limit)
+            dx, _, dp8, hq8, dy8 = ops.mlp8_bwd_q(g2, r, st.w8, rowb, st.e4m3_limit, want_dpre=False)
             (bf, af), (bp, ap) = _accumulate_into(w_fc), _accumulate_into(w_proj)
             if (bf is None) != (bp is None) or af != ap:
                 raise RuntimeError("the fp8 weight gradients write both MLP weights' gradient buffers in one call")
@@ -471,7 +471,7 @@ class NrMlpFn(torch.autograd.Function):
         g = g.contiguous()
         rowb = ops.mlp8_backward_scales(g, st.row)
         if st.dw_fp8:
-            dxn, _, dp8, hq8, dy8 = ops.mlp8_bwd_q(g, r, st.w8, rowb, st.e4m3_limit)
+            dxn, _, dp8, hq8, dy8 = ops.mlp8_bwd_q(g, r, st.w8, rowb, st.e4m3_limit, want_dpre=False)
             dw_fc, dw_proj = ops.mlp8_dw8(xa, dp8, hq8, dy8, rowb, st.x_scale)
         else:
             dxn, _, dpre = ops.mlp8_bwd(g, r, st.w8, rowb, want_h=False)

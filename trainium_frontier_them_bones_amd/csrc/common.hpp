@@ -26,14 +26,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float bf2f(bf16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
 
-// fp32 -> bf16, round to nearest even (torch's .to(torch.bfloat16)); NaN stays NaN.
-__device__ __forceinline__ bf16_t f2bf(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
-}
-
 // Two fp32 -> packed bf16 pair (lo in bits 0..15), round to nearest even. Written as a vector conversion so that the
 // compiler selects gfx950's v_cvt_pk_bf16_f32 itself: as inline assembly the instruction is opaque to the hazard
 // recognizer, and a conversion scheduled right behind the MFMA / transcendental that feeds it read stale lanes.
@@ -46,6 +38,11 @@ __device__ __forceinline__ uint32_t pack2bf(float lo, float hi) {
 __device__ __forceinline__ float bflo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bfhi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 
+// fp32 -> bf16, round to nearest even (torch's .to(torch.bfloat16)); NaN stays NaN. One hardware conversion: the
+// integer form of this rounding (add 0x7fff + lsb, shift, a NaN test) costs seven vector instructions per value, and
+// epilogues that round every element twice spent more cycles on it than their GEMM's k-loop on MFMAs.
+__device__ __forceinline__ bf16_t f2bf(float f) { return (bf16_t)pack2bf(f, 0.f); }
+
 // acc + lo + hi of a packed bf16 pair in one instruction (v_dot2c_f32_bf16 against the pair (1, 1)).
 __device__ __forceinline__ float sum2bf(uint32_t w, float acc) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), acc,
@@ -54,7 +51,14 @@ __device__ __forceinline__ float sum2bf(uint32_t w, float acc) {
 
 // Round an fp32 value to the nearest bf16 and return it as fp32 (a rounding point of the
 // reference arithmetic that stays in registers).
-__device__ __forceinline__ float round_bf(float f) { return bf2f(f2bf(f)); }
+__device__ __forceinline__ float round_bf(float f) { return bflo(pack2bf(f, 0.f)); }
+// The same for a pair, in place (one conversion for the two): returns the packed bf16 pair as well.
+__device__ __forceinline__ uint32_t round2_bf(float& a, float& b) {
+  const uint32_t w = pack2bf(a, b);
+  a = bflo(w);
+  b = bfhi(w);
+  return w;
+}
 
 // 8 fp32 values <-> 8 bf16 in four 32-bit words (one 128-bit access)
 __device__ __forceinline__ u32x4 pack8bf(const float (&v)[8]) {
@@ -78,13 +82,16 @@ __device__ __forceinline__ void unpack8bf(u32x4 u, float (&v)[8]) {
 #define TFB_FMT_E4M3 0
 #define TFB_FMT_E5M2 1
 
-template <int FMT>
+// CLAMP = false: for values the caller has already bounded inside the format's range.
+template <int FMT, bool CLAMP = true>
 __device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, float d) {
-  const float mx = FMT == TFB_FMT_E4M3 ? TFB_E4M3_MAX : TFB_E5M2_MAX;
-  a = fminf(fmaxf(a, -mx), mx);
-  b = fminf(fmaxf(b, -mx), mx);
-  c = fminf(fmaxf(c, -mx), mx);
-  d = fminf(fmaxf(d, -mx), mx);
+  if (CLAMP) {
+    const float mx = FMT == TFB_FMT_E4M3 ? TFB_E4M3_MAX : TFB_E5M2_MAX;
+    a = fminf(fmaxf(a, -mx), mx);
+    b = fminf(fmaxf(b, -mx), mx);
+    c = fminf(fmaxf(c, -mx), mx);
+    d = fminf(fmaxf(d, -mx), mx);
+  }
   int w = 0;
   if (FMT == TFB_FMT_E4M3) {
     w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);

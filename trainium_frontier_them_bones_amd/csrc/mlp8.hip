@@ -328,16 +328,22 @@ struct EpiUp {  // pre = x8 @ wf8^T: r, h8
   }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
     const float dq = sc[SC_DQ_FC], c = sc[SC_C_H];
-    float rr[8], hh[8];
+    float hh[8];
+    u32x4 rbits;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      rr[i] = round_bf(fmaxf(v[i] * dq, 0.f));
-      float rc = round_bf(fminf(rr[i] * c, H_CLAMP));
-      hh[i] = rc * rc;
+    for (int i = 0; i < 8; i += 2) {
+      float a = fmaxf(v[i] * dq, 0.f), b = fmaxf(v[i + 1] * dq, 0.f);
+      rbits[i >> 1] = round2_bf(a, b);                       // r = bf16(max(acc dq, 0)): saved before the clamp
+      float ca = fminf(a * c, H_CLAMP), cb = fminf(b * c, H_CLAMP);
+      round2_bf(ca, cb);                                     // rc = bf16(min(r c_h, 15.375))
+      hh[i] = ca * ca;
+      hh[i + 1] = cb * cb;
     }
     const long off = (long)q * F + p;
-    *(u32x4*)(r + off) = pack8bf(rr);
-    u32x2 o = {cvt4_fp8<TFB_FMT_E4M3>(hh[0], hh[1], hh[2], hh[3]), cvt4_fp8<TFB_FMT_E4M3>(hh[4], hh[5], hh[6], hh[7])};
+    *(u32x4*)(r + off) = rbits;
+    // 0 <= rc^2 <= 15.375^2 < 240: inside the e4m3 range, no saturation clamp needed
+    u32x2 o = {cvt4_fp8<TFB_FMT_E4M3, false>(hh[0], hh[1], hh[2], hh[3]),
+               cvt4_fp8<TFB_FMT_E4M3, false>(hh[4], hh[5], hh[6], hh[7])};
     *(u32x2*)(h8 + off) = o;
   }
 };
@@ -416,7 +422,7 @@ struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*
                 // hq8 = e4m3(min(h*s_h, limit)) (the fp8 weight gradient's operand)
   const float* sc;
   const bf16_t* r;  // [M][F]
-  bf16_t* dpre;     // [M][F]
+  bf16_t* dpre;     // [M][F] or null (the fp8 weight gradients read dp8, not dpre)
   uint8_t* dp8;     // [M][F]
   bf16_t* h;        // [M][F] or null
   uint8_t* hq8;     // [M][F] or null
@@ -434,21 +440,32 @@ struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*
     const long off = (long)q * F + p;
     float rr[8], dp[8];
     unpack8bf(rv, rr);
+    u32x4 dbits;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) dp[i] = round_bf((v[i] * dq) * rr[i]);
-    *(u32x4*)(dpre + off) = pack8bf(dp);
+    for (int i = 0; i < 8; i += 2) {
+      dp[i] = (v[i] * dq) * rr[i];
+      dp[i + 1] = (v[i + 1] * dq) * rr[i + 1];
+      dbits[i >> 1] = round2_bf(dp[i], dp[i + 1]);           // dpre = bf16((acc dq_dh2) r)
+    }
+    if (dpre) *(u32x4*)(dpre + off) = dbits;
     u32x2 o = {cvt4_fp8<TFB_FMT_E5M2>(dp[0] * sdp, dp[1] * sdp, dp[2] * sdp, dp[3] * sdp),
                cvt4_fp8<TFB_FMT_E5M2>(dp[4] * sdp, dp[5] * sdp, dp[6] * sdp, dp[7] * sdp)};
     *(u32x2*)(dp8 + off) = o;
     if (h || hq8) {
+      u32x4 hbits;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) rr[i] = round_bf(rr[i] * rr[i]);
-      if (h) *(u32x4*)(h + off) = pack8bf(rr);
+      for (int i = 0; i < 8; i += 2) {
+        rr[i] = rr[i] * rr[i];
+        rr[i + 1] = rr[i + 1] * rr[i + 1];
+        hbits[i >> 1] = round2_bf(rr[i], rr[i + 1]);         // h = bf16(r^2)
+      }
+      if (h) *(u32x4*)(h + off) = hbits;
       if (hq8) {
-        const float sh = sc[SC_S_H];
+        const float sh = sc[SC_S_H], lim = fminf(hq_limit, TFB_E4M3_MAX);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) rr[i] = fminf(rr[i] * sh, hq_limit);
-        u32x2 q = {cvt4_fp8<TFB_FMT_E4M3>(rr[0], rr[1], rr[2], rr[3]), cvt4_fp8<TFB_FMT_E4M3>(rr[4], rr[5], rr[6], rr[7])};
+        for (int i = 0; i < 8; ++i) rr[i] = fminf(rr[i] * sh, lim);   // 0 <= . <= lim: in range, no further clamp
+        u32x2 q = {cvt4_fp8<TFB_FMT_E4M3, false>(rr[0], rr[1], rr[2], rr[3]),
+                   cvt4_fp8<TFB_FMT_E4M3, false>(rr[4], rr[5], rr[6], rr[7])};
         *(u32x2*)(hq8 + off) = q;
       }
     }
@@ -717,7 +734,7 @@ extern "C" int tfb_mlp8_fwd_res(const void* x8, const void* w8, const void* row,
 // gradient of w_proj (K/nki_dw8.py:323 with format E4M3C, round2/source/train.py:8226).
 extern "C" int tfb_mlp8_bwd_q(const void* dy8, const void* r, const void* w8, const void* row, void* dx, void* h, void* dpre,
                               void* dp8, void* hq8, float hq_limit, long M, int d, int F, void* stream) {
-  if (!dy8 || !r || !w8 || !row || !dx || !dpre || !dp8) return TFB_ERR_ARG;
+  if (!dy8 || !r || !w8 || !row || !dx || !dp8) return TFB_ERR_ARG;  // dpre may be NULL: only dp8 is then written
   if (!shapes8(M, d, F)) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   const uint8_t* b = (const uint8_t*)w8;

@@ -34,7 +34,7 @@ class GPTConfig:
     x_scale: float = 4.0          # constant activation scale of the fp8 MLP input (a unit-RMS norm output)
     fp8_attn_proj: bool = False   # QKV and output projections in fp8 (e4m3 forward, e5m2 dX, bf16 dW); off in configuration 4 of BASELINE.json
     fp8_attn_dw: bool = False     # with fp8_attn_proj: their weight gradients in fp8 as well (R2_DW8_SET=qkv,proj)
-    fp8_mlp_dw: bool = False      # the MLP's two weight gradients in fp8 as well (R1's DW_ROWS recipe); off in configuration 4 of BASELINE.json
+    fp8_mlp_dw: bool = True       # the MLP's two weight gradients in fp8 as well: all six MLP GEMMs in fp8, as the reference's final recipe (round1/source/train.py:2226-2233 DW_ROWS '5,6'; round2/source/train.py:8209)
     fuse_residual: bool = True    # residual adds in the projections' stores, fp8 operand casts in the norms (same values)
 
     @property

@@ -365,15 +365,16 @@ def mlp8_bwd(dy2, r, w8, row, want_h=True):
     return dx, h, dpre
 
 
-def mlp8_bwd_q(dy2, r, w8, row, e4m3_limit=240.0):
-    """The fp8 backward keeping the byte tensors of the fp8 weight gradients: (dx [M,d], dpre [M,F], dp8 [M,F] e5m2 bytes,
-    hq8 [M,F] = e4m3(min(bf16(r^2) s_h, e4m3_limit)) bytes, dy8 [M,d] e5m2 bytes)."""
+def mlp8_bwd_q(dy2, r, w8, row, e4m3_limit=240.0, want_dpre=True):
+    """The fp8 backward keeping the byte tensors of the fp8 weight gradients: (dx [M,d], dpre [M,F] (None without
+    want_dpre: the fp8 weight gradients read only its bytes), dp8 [M,F] e5m2 bytes, hq8 [M,F] = e4m3(min(bf16(r^2) s_h,
+    e4m3_limit)) bytes, dy8 [M,d] e5m2 bytes)."""
     _chk(dy2), _chk(r), _chk(w8, torch.uint8), _chk(row, torch.float32)
     M, d = dy2.shape
     F = r.shape[1]
     dy8 = quant_fp8(dy2, row[5:6], FMT_E5M2)
     dx = torch.empty(M, d, dtype=bf16, device=dy2.device)
-    dpre = torch.empty(M, F, dtype=bf16, device=dy2.device)
+    dpre = torch.empty(M, F, dtype=bf16, device=dy2.device) if want_dpre else None
     dp8 = torch.empty(M, F, dtype=torch.uint8, device=dy2.device)
     hq8 = torch.empty(M, F, dtype=torch.uint8, device=dy2.device)
     _lib.call("tfb_mlp8_bwd_q", _p(dy8), _p(r), _p(w8), _p(row), _p(dx), None, _p(dpre), _p(dp8), _p(hq8), float(e4m3_limit),
