@@ -265,6 +265,20 @@ __device__ __forceinline__ Epi epi_for_group(const Epi& e, int g) {
   else return e;
 }
 
+// An epilogue that reads device scalars (scale rows) provides  Epi prepare() const, called once before the k-loop: it
+// returns the functor with those values held in registers. Read inside operator() they would be re-loaded after every
+// store (the stores may alias them), and each re-load's wait also waits for every store still in flight: an epilogue of
+// eight chunks then costs eight store round trips (measured: twice its GEMM's k-loop).
+template <class T, class = void>
+struct has_prepare : std::false_type {};
+template <class T>
+struct has_prepare<T, std::void_t<decltype(std::declval<const T&>().prepare())>> : std::true_type {};
+template <class Epi>
+__device__ __forceinline__ Epi epi_prepare(const Epi& e) {
+  if constexpr (has_prepare<Epi>::value) return e.prepare();
+  else return e;
+}
+
 // A staged epilogue with the static member kPartner32 also receives the 8 values 32 output columns away (p ^ 32: the
 // other half of a 64-wide head, for rotary embeddings): operator()(p, q, v, v_partner, split). Needs a wavefront slice
 // of exactly 64 staged columns.
@@ -383,7 +397,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
     kt0 = k0 * ES / 128;
     a.nkt = (int)((k1 - k0) * ES / 128);  // may be 0: the accumulators stay zero and are still written
   }
-  const Epi epi = epi_for_group(epi_in, group);
+  const Epi epi = epi_prepare(epi_for_group(epi_in, group));
   const int nkt = a.nkt;
 
   TileDma<BP, NW, Cfg::LAYP, ES> dp;

@@ -321,13 +321,19 @@ struct EpiUp {  // pre = x8 @ wf8^T: r, h8
   bf16_t* r;     // [M][F]
   uint8_t* h8;   // [M][F]
   long F;
+  float dq = 0.f, c = 0.f;  // sc[SC_DQ_FC], sc[SC_C_H], read once by prepare()
   __device__ __forceinline__ EpiUp for_group(int g) const {
     EpiUp e = *this;
     e.sc = sc + g * NSC;
     return e;
   }
+  __device__ __forceinline__ EpiUp prepare() const {
+    EpiUp e = *this;
+    e.dq = sc[SC_DQ_FC];
+    e.c = sc[SC_C_H];
+    return e;
+  }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
-    const float dq = sc[SC_DQ_FC], c = sc[SC_C_H];
     float hh[8];
     u32x4 rbits;
 #pragma unroll
@@ -353,13 +359,18 @@ struct EpiScaleStore {  // out = bf16(acc * sc[col])
   int col;
   bf16_t* out;
   long ld;
+  float dq = 0.f;  // sc[col], read once by prepare()
   __device__ __forceinline__ EpiScaleStore for_group(int g) const {
     EpiScaleStore e = *this;
     e.sc = sc + g * NSC;
     return e;
   }
+  __device__ __forceinline__ EpiScaleStore prepare() const {
+    EpiScaleStore e = *this;
+    e.dq = sc[col];
+    return e;
+  }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
-    const float dq = sc[col];
     float r[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) r[i] = v[i] * dq;
@@ -379,17 +390,21 @@ struct EpiDescaleRes {
   const bf16_t* res;
   bf16_t* out;
   long ld;
+  float dq = 0.f;  // the descale factor, read once by prepare()
   using pre_t = u32x4;
+  __device__ __forceinline__ EpiDescaleRes prepare() const {
+    EpiDescaleRes e = *this;
+    if (sc) {
+      e.dq = sc[col];
+    } else {
+      e.dq = dq_imm;
+      if (dq_a) e.dq *= *dq_a;
+      if (dq_b) e.dq *= *dq_b;
+    }
+    return e;
+  }
   __device__ __forceinline__ pre_t prefetch(int p, int q) const { return *(const u32x4*)(res + (long)q * ld + p); }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const pre_t& rv, int) const {
-    float dq;
-    if (sc) {
-      dq = sc[col];
-    } else {
-      dq = dq_imm;
-      if (dq_a) dq *= *dq_a;
-      if (dq_b) dq *= *dq_b;
-    }
     float r[8], a[8], b[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) r[i] = v[i] * dq;
@@ -407,10 +422,15 @@ struct EpiDescale {  // out = bf16(acc * dq), dq = dq_imm * *dq_a * *dq_b (absen
   float dq_imm;
   bf16_t* out;
   long ld;
+  float dq = 0.f;  // dq_imm * *dq_a * *dq_b, read once by prepare()
+  __device__ __forceinline__ EpiDescale prepare() const {
+    EpiDescale e = *this;
+    e.dq = dq_imm;
+    if (dq_a) e.dq *= *dq_a;
+    if (dq_b) e.dq *= *dq_b;
+    return e;
+  }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
-    float dq = dq_imm;
-    if (dq_a) dq *= *dq_a;
-    if (dq_b) dq *= *dq_b;
     float r[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) r[i] = v[i] * dq;
@@ -428,15 +448,22 @@ struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*
   uint8_t* hq8;     // [M][F] or null
   float hq_limit;
   long F;
+  float dq = 0.f, sdp = 0.f, sh = 0.f;  // sc[SC_DQ_DH2], sc[SC_S_DP], sc[SC_S_H], read once by prepare()
   __device__ __forceinline__ EpiDh for_group(int g) const {
     EpiDh e = *this;
     e.sc = sc + g * NSC;
     return e;
   }
+  __device__ __forceinline__ EpiDh prepare() const {
+    EpiDh e = *this;
+    e.dq = sc[SC_DQ_DH2];
+    e.sdp = sc[SC_S_DP];
+    e.sh = sc[SC_S_H];
+    return e;
+  }
   typedef u32x4 pre_t;  // the 8 values of r this chunk needs, requested before the k-loop
   __device__ __forceinline__ pre_t prefetch(int p, int q) const { return *(const u32x4*)(r + (long)q * F + p); }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const pre_t& rv, int) const {
-    const float dq = sc[SC_DQ_DH2], sdp = sc[SC_S_DP];
     const long off = (long)q * F + p;
     float rr[8], dp[8];
     unpack8bf(rv, rr);
@@ -461,7 +488,7 @@ struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*
       }
       if (h) *(u32x4*)(h + off) = hbits;
       if (hq8) {
-        const float sh = sc[SC_S_H], lim = fminf(hq_limit, TFB_E4M3_MAX);
+        const float lim = fminf(hq_limit, TFB_E4M3_MAX);
 #pragma unroll
         for (int i = 0; i < 8; ++i) rr[i] = fminf(rr[i] * sh, lim);   // 0 <= . <= lim: in range, no further clamp
         u32x2 q = {cvt4_fp8<TFB_FMT_E4M3, false>(rr[0], rr[1], rr[2], rr[3]),

@@ -62,6 +62,30 @@ struct Row {
   }
 };
 
+// A row as loaded (bf16 pairs in 32-bit words), to be widened later: the kernels below request the NEXT row of a
+// wavefront before they store the current one. A wait for loaded data also waits for every older memory operation, stores
+// included (one counter orders both), so a loop that loads after its stores pays a full store round trip per row.
+template <int NCH>
+struct RawRow {
+  u32x4 u[NCH];
+  __device__ __forceinline__ void load(const bf16_t* p, int C, int lane) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = (lane + 64 * i) * 8;
+      u[i] = c < C ? *(const u32x4*)(p + c) : u32x4{0u, 0u, 0u, 0u};
+    }
+  }
+  __device__ __forceinline__ void widen(Row<NCH>& r) const {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        r.v[i][2 * k] = bflo(u[i][k]);
+        r.v[i][2 * k + 1] = bfhi(u[i][k]);
+      }
+  }
+};
+
 template <int NCH>
 __device__ __forceinline__ float row_dot(const Row<NCH>& a, const Row<NCH>& b) {
   float s = 0.f;
@@ -81,12 +105,23 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16_t* __restri
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   Row<NCH> wr;
   if (w) wr.load(w, C, lane);
-  for (long row = (long)blockIdx.x * ROWS_PER_BLOCK + wave; row < nrows; row += (long)gridDim.x * ROWS_PER_BLOCK) {
+  const long step = (long)gridDim.x * ROWS_PER_BLOCK;
+  long row = (long)blockIdx.x * ROWS_PER_BLOCK + wave;
+  RawRow<NCH> xa, xr;
+  if (row < nrows) {
+    xa.load(x + row * C, C, lane);
+    if (res) xr.load(res + row * C, C, lane);
+  }
+  for (; row < nrows; row += step) {
     Row<NCH> a;
-    a.load(x + row * C, C, lane);
+    xa.widen(a);
+    Row<NCH> r;
+    if (res) xr.widen(r);
+    if (row + step < nrows) {  // the next row's loads go out before this row's stores
+      xa.load(x + (row + step) * C, C, lane);
+      if (res) xr.load(res + (row + step) * C, C, lane);
+    }
     if (res) {
-      Row<NCH> r;
-      r.load(res + row * C, C, lane);
 #pragma unroll
       for (int i = 0; i < NCH; ++i)
 #pragma unroll
@@ -129,13 +164,28 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16_t* __restri
   Row<NCH> wr, dwacc;
   if (w) wr.load(w, C, lane);
   dwacc.zero();
-  for (long row = (long)blockIdx.x * ROWS_PER_BLOCK + wave; row < nrows; row += (long)gridDim.x * ROWS_PER_BLOCK) {
-    Row<NCH> g, a;
-    g.load(gy + row * C, C, lane);
-    a.load(s + row * C, C, lane);
-    Row<NCH> r;
-    if (gs) r.load(gs + row * C, C, lane);   // issued with the other two loads
-    const float rs = inv[row];
+  const long step = (long)gridDim.x * ROWS_PER_BLOCK;
+  long row = (long)blockIdx.x * ROWS_PER_BLOCK + wave;
+  RawRow<NCH> xg, xa, xr;
+  float rs_next = 0.f;
+  if (row < nrows) {
+    xg.load(gy + row * C, C, lane);
+    xa.load(s + row * C, C, lane);
+    if (gs) xr.load(gs + row * C, C, lane);
+    rs_next = inv[row];
+  }
+  for (; row < nrows; row += step) {
+    Row<NCH> g, a, r;
+    xg.widen(g);
+    xa.widen(a);
+    if (gs) xr.widen(r);
+    const float rs = rs_next;
+    if (row + step < nrows) {  // the next row's loads go out before this row's store
+      xg.load(gy + (row + step) * C, C, lane);
+      xa.load(s + (row + step) * C, C, lane);
+      if (gs) xr.load(gs + (row + step) * C, C, lane);
+      rs_next = inv[row + step];
+    }
     if (w) {
 #pragma unroll
       for (int i = 0; i < NCH; ++i)
