@@ -401,27 +401,38 @@ template <bool GF32>
 __global__ __launch_bounds__(256) void adamw_kernel(float* __restrict__ p, const void* __restrict__ g, float* __restrict__ m,
                                                    float* __restrict__ v, bf16_t* __restrict__ p16, long n, AdamScalars s) {
   const long n4 = n & ~3L;
-  for (long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4; i < n4; i += (long)gridDim.x * 256 * 4) {
-    f32x4 pp = *(const f32x4*)(p + i), mm = *(const f32x4*)(m + i), vv = *(const f32x4*)(v + i), gg;
-    if (GF32) {
-      gg = *(const f32x4*)((const float*)g + i);
-    } else {
-      u32x2 u = *(const u32x2*)((const bf16_t*)g + i);
-      gg = f32x4{bflo(u.x), bfhi(u.x), bflo(u.y), bfhi(u.y)};
-    }
+  const long step = (long)gridDim.x * 256 * 4;
+  long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+  // the next group's four loads go out before this group's stores: a wait for loaded data also waits for every older
+  // store (one counter orders both), so loading after the stores would cost a store round trip per group
+  f32x4 pp, mm, vv, gg;
+  u32x2 gb;
+  auto fetch = [&](long j) {
+    pp = *(const f32x4*)(p + j);
+    mm = *(const f32x4*)(m + j);
+    vv = *(const f32x4*)(v + j);
+    if (GF32) gg = *(const f32x4*)((const float*)g + j);
+    else gb = *(const u32x2*)((const bf16_t*)g + j);
+  };
+  if (i < n4) fetch(i);
+  for (; i < n4; i += step) {
+    f32x4 cp = pp, cm = mm, cv = vv, cg;
+    if (GF32) cg = gg;
+    else cg = f32x4{bflo(gb.x), bfhi(gb.x), bflo(gb.y), bfhi(gb.y)};
+    if (i + step < n4) fetch(i + step);
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      float pk = pp[k], mk = mm[k], vk = vv[k];
-      adamw_one(pk, mk, vk, gg[k], s);
-      pp[k] = pk;
-      mm[k] = mk;
-      vv[k] = vk;
+      float pk = cp[k], mk = cm[k], vk = cv[k];
+      adamw_one(pk, mk, vk, cg[k], s);
+      cp[k] = pk;
+      cm[k] = mk;
+      cv[k] = vk;
     }
-    *(f32x4*)(p + i) = pp;
-    *(f32x4*)(m + i) = mm;
-    *(f32x4*)(v + i) = vv;
+    *(f32x4*)(p + i) = cp;
+    *(f32x4*)(m + i) = cm;
+    *(f32x4*)(v + i) = cv;
     if (p16) {
-      u32x2 o = {pack2bf(pp[0], pp[1]), pack2bf(pp[2], pp[3])};
+      u32x2 o = {pack2bf(cp[0], cp[1]), pack2bf(cp[2], cp[3])};
       *(u32x2*)(p16 + i) = o;
     }
   }

@@ -113,8 +113,12 @@ __global__ __launch_bounds__(256) void loss_bwd_kernel(const bf16_t* __restrict_
   const float g = (unsigned long)tt < (unsigned long)V ? grow[row] : 0.f;  // out of range = ignored
   const float l = lse[row];
   const float icap = cap > 0.f ? 1.0f / cap : 0.f;
+  // (the next chunk is requested before this chunk's store: a wait for loaded data also waits for every older store)
+  u32x4 unext = {0u, 0u, 0u, 0u};
+  if ((int)threadIdx.x * 8 < V) unext = *(const u32x4*)(xr + threadIdx.x * 8);
   for (int i = threadIdx.x * 8; i < V; i += 256 * 8) {
-    u32x4 u = *(const u32x4*)(xr + i);
+    const u32x4 u = unext;
+    if (i + 256 * 8 < V) unext = *(const u32x4*)(xr + i + 256 * 8);
     float v[8], d[8];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
