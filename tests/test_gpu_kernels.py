@@ -276,6 +276,11 @@ def test_fp8_casts_exhaustive_against_format_tables(ops, dev):
             assert bool((sat == lim).all())                               # beyond the range: saturates
         s = torch.tensor([0.5], device=dev)
         assert torch.equal(ops.quant_fp8(allb.to(dev), s, fmt).cpu(), ops.quant_fp8(allb.to(dev), 0.5, fmt).cpu())
+        # a NaN stays a NaN through the cast (as torch's), it is not turned into the format's largest value
+        nan = torch.full((16,), float("nan"), dtype=torch.bfloat16)
+        nan[::2] = 1.0
+        qn = ops.quant_fp8(nan.to(dev), 1.0, fmt).cpu().view(torch.float8_e5m2 if fmt else torch.float8_e4m3fn).float()
+        assert bool(torch.isnan(qn[1::2]).all()) and bool((qn[::2] == 1.0).all())
 
 
 @pytest.mark.parametrize("shape", [(256, 256, 512), (1024, 768, 3072), (384, 1024, 2816 - 2816 % 256)])
@@ -700,3 +705,26 @@ def test_newton_schulz_full_size_properties(ops, dev):
     assert rel_l2(y[:1], yo) < NS_TOL
     with pytest.raises(TfbError):
         ops.ns5(gd[:, :100].contiguous(), dd)                                         # rows % 128 != 0
+
+
+def test_autograd_nodes_do_not_corrupt_what_autograd_cannot_see(ops, dev):
+    """RopeAttentionFn leaves its input qkv untouched (the rotation goes into a buffer of its own); LmHeadLossFn, whose
+    backward overwrites the saved logits with their gradient, refuses a second backward instead of returning garbage."""
+    from trainium_frontier_them_bones_amd import autograd as A
+    from oracle import attention as OA
+    g = _g(31)
+    B, T, H, D = 2, 256, 4, 64
+    qkv = torch.randn(B, T, 3 * H * D, generator=g).bfloat16().to(dev).requires_grad_(True)
+    before = qkv.detach().clone()
+    cos, sin = OA.rope_tables(T, D)
+    out = A.RopeAttentionFn.apply(qkv, cos.to(dev), sin.to(dev), H, 0.125)
+    assert torch.equal(qkv.detach(), before)
+    out.sum().backward()
+    assert torch.equal(qkv.detach(), before) and bool(torch.isfinite(qkv.grad.float()).all())
+    x = torch.randn(256, 256, generator=g).bfloat16().to(dev).requires_grad_(True)
+    W = (0.05 * torch.randn(1024, 256, generator=g)).bfloat16().to(dev).requires_grad_(True)
+    t = torch.randint(0, 1024, (256,), generator=g).to(dev)
+    loss = A.LmHeadLossFn.apply(x, W, t, 0.0, "mean")
+    loss.backward(retain_graph=True)
+    with pytest.raises(RuntimeError):
+        loss.backward()

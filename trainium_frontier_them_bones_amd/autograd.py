@@ -105,9 +105,9 @@ class AddRMSNormFn(torch.autograd.Function):
         if part is not None and gy is not None:
             dx = ops.rmsnorm_bwd(gy.contiguous(), s, inv, weight, None if gs is None else gs.contiguous(), part=part)[0]
             return dx, dx, None, None
-        buf, acc = (None, False) if weight is None else _accumulate_into(weight)
         if gy is None:
             return gs, gs, None, None
+        buf, acc = (None, False) if weight is None else _accumulate_into(weight)   # (only once the buffer is surely written)
         dx, dw = ops.rmsnorm_bwd(gy.contiguous(), s, inv, weight, None if gs is None else gs.contiguous(), buf, acc)
         gw = dw.to(weight.dtype) if (weight is not None and buf is None) else None
         return dx, dx, gw, None
@@ -185,9 +185,10 @@ class CausalAttentionFn(torch.autograd.Function):
 
 
 class RopeAttentionFn(torch.autograd.Function):
-    """Attention straight from the fused projection output qkv [B, T, 3C]: RoPE on the q and k thirds (in place, the
-    buffer has no other reader), causal attention reading the thirds through strides, one dqkv [B, T, 3C] back
-    (the call shape of nki_rope_attention, round1/source/train.py:8197, without its QK-norm)."""
+    """Attention straight from the fused projection output qkv [B, T, 3C]: RoPE of the q and k thirds into a buffer of its
+    own (the input is left untouched: whoever produced or saved it still holds the values it made), causal attention
+    reading q, k from that buffer and v from qkv through strides, one dqkv [B, T, 3C] back (the call shape of
+    nki_rope_attention, round1/source/train.py:8197, without its QK-norm)."""
 
     @staticmethod
     def forward(ctx, qkv, cos, sin, n_head, scale):
@@ -195,21 +196,24 @@ class RopeAttentionFn(torch.autograd.Function):
         C = C3 // 3
         D = C // n_head
         qkv = qkv.contiguous()
-        ops.rope_(qkv.view(B * T, C3), cos, sin, T, 2 * n_head, D)
-        q, k, v = (t.view(B, T, n_head, D) for t in qkv.split(C, dim=-1))
+        rot = torch.empty(B, T, 2 * C, dtype=qkv.dtype, device=qkv.device)
+        ops.rope_(qkv.view(B * T, C3), cos, sin, T, 2 * n_head, D, out=rot.view(B * T, 2 * C))
+        q, k = (t.view(B, T, n_head, D) for t in rot.split(C, dim=-1))
+        v = qkv[..., 2 * C:].view(B, T, n_head, D)
         o, lse = ops.attn_fwd(q, k, v, scale, "bthd")
-        ctx.save_for_backward(qkv, o, lse, cos, sin)
+        ctx.save_for_backward(qkv, rot, o, lse, cos, sin)
         ctx.n_head, ctx.scale = n_head, scale
         return o.view(B, T, C)
 
     @staticmethod
     def backward(ctx, go):
-        qkv, o, lse, cos, sin = ctx.saved_tensors
+        qkv, rot, o, lse, cos, sin = ctx.saved_tensors
         B, T, C3 = qkv.shape
         C = C3 // 3
         H = ctx.n_head
         D = C // H
-        q, k, v = (t.view(B, T, H, D) for t in qkv.split(C, dim=-1))
+        q, k = (t.view(B, T, H, D) for t in rot.split(C, dim=-1))
+        v = qkv[..., 2 * C:].view(B, T, H, D)
         dqkv = torch.empty_like(qkv)
         dq, dk, dv = (t.view(B, T, H, D) for t in dqkv.split(C, dim=-1))
         if D == 64:  # the inverse rotation of dq, dk rides the backward kernels' stores
@@ -500,6 +504,10 @@ class LmHeadLossFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g):
         x2, W, tg, logits, lse, w = ctx.saved_tensors
+        if getattr(ctx, "logits_consumed", False):
+            raise RuntimeError("LmHeadLossFn: second backward through the same node (retain_graph): the saved logits "
+                               "were overwritten by their gradient in the first one")
+        ctx.logits_consumed = True
         grow = (w * g.to(torch.float32)).contiguous()
         dl = ops.loss_bwd(logits, tg, lse, grow, ctx.softcap, inplace=True)
         dx = ops.matmul(dl, W).view(ctx.xshape)
@@ -645,9 +653,14 @@ class MoeMlp8Fn(torch.autograd.Function):
         dys, dgate = ops.moe_combine_bwd(g2, ys, tab, gate)
         rows_b = ops.moe_backward_scales(dys, st.rows, tab)
         dxs, dpre = ops.moe_mlp8_bwd(dys, r, st.w8, rows_b, tab)
-        bf, accf = _accumulate_into(w_fc)
-        bp, accp = _accumulate_into(w_proj)
-        if bf is not None and bp is not None:
+        # one grouped launch writes both gradients: both weights carry a gradient buffer (in the same state) or neither
+        # does; the "fresh" flags are only touched on the branch that really writes the buffers
+        if (getattr(w_fc, "grad_buf", None) is None) != (getattr(w_proj, "grad_buf", None) is None):
+            raise RuntimeError("MoeMlp8Fn: give both expert weights a grad_buf, or neither")
+        if getattr(w_fc, "grad_buf", None) is not None:
+            (bf, accf), (bp, accp) = _accumulate_into(w_fc), _accumulate_into(w_proj)
+            if accf != accp:
+                raise RuntimeError("MoeMlp8Fn: the two expert weights' gradient buffers are in different states")
             ops.moe_dw(dpre, xs, dys, r, tab, E, bf, bp, accumulate=accf)
             dw_fc = dw_proj = None
         else:

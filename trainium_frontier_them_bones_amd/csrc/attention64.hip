@@ -111,8 +111,8 @@ __device__ __forceinline__ int swz(int t) { return (((t >> 1) & 1) << 2) | ((t >
 #ifndef TFB_ATTN_STAGGER
 #define TFB_ATTN_STAGGER 1
 #endif
-__device__ __forceinline__ void stagger_start() {
-  if (TFB_ATTN_STAGGER > 0 && blockIdx.x + gridDim.x * blockIdx.y < 512) {
+__device__ __forceinline__ void stagger_start(int slots) {  // slots: workgroups resident at once (the first round)
+  if (TFB_ATTN_STAGGER > 0 && (int)(blockIdx.x + gridDim.x * blockIdx.y) < slots) {
     if (__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 4) & 1)  // getreg(size 4, offset 0, HW_REG_HW_ID)
       for (int i = 0; i < TFB_ATTN_STAGGER; ++i) __builtin_amdgcn_s_sleep(127);
   }
@@ -193,12 +193,12 @@ __device__ __forceinline__ void store_grad_row(const f32x16 (&acc)[2], float sca
 
 // =========================================================================================== forward
 __global__ __launch_bounds__(256, TFB_FWD64_WPE) void attn64_fwd_kernel(AttnT q, AttnT k, AttnT v, AttnT o, float* __restrict__ lse,
-                                                            int T, int H, float sl2, int nw) {
+                                                            int T, int H, float sl2, int nw, int slots) {
   __shared__ __attribute__((aligned(1024))) uint8_t st0[2 * TILE];
   __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  stagger_start();
+  stagger_start(slots);
   int bx, bh;
   xcd_block(gridDim.x, gridDim.y, bx, bh);
   const int b = bh / H, h = bh % H;
@@ -439,7 +439,7 @@ __global__ __launch_bounds__(256) void attn64_delta_kernel(AttnT o, AttnT go, co
 __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dk, AttnT dv,
                                                              const float* __restrict__ stats, long rows, int T, int H,
                                                              float scale, float sl2, const bf16_t* __restrict__ cs,
-                                                             const bf16_t* __restrict__ sn, int nw) {
+                                                             const bf16_t* __restrict__ sn, int nw, int slots) {
   constexpr int QT = TFB_DKDV64_QT;       // 64-query tiles per LDS stage (one barrier per stage)
   constexpr int R = 64 * QT, RT = R * 128;  // rows and bytes of a staged Q (dO) tile
   constexpr int STAGE = 2 * RT + 8 * R;    // Q tile, dO tile, R x (-lse / scale), R x (-delta)
@@ -447,7 +447,7 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
   __shared__ __attribute__((aligned(1024))) uint8_t st1[STAGE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  stagger_start();
+  stagger_start(slots);
   int bx, bh;
   xcd_block(gridDim.x, gridDim.y, bx, bh);
   const int b = bh / H, h = bh % H;
@@ -598,12 +598,12 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
 __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dq,
                                                            const float* __restrict__ stats, long rows, int T, int H,
                                                            float scale, float sl2, const bf16_t* __restrict__ cs,
-                                                           const bf16_t* __restrict__ sn, int nw) {
+                                                           const bf16_t* __restrict__ sn, int nw, int slots) {
   __shared__ __attribute__((aligned(1024))) uint8_t st0[2 * TILE];
   __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  stagger_start();
+  stagger_start(slots);
   int bx, bh;
   xcd_block(gridDim.x, gridDim.y, bx, bh);
   const int b = bh / H, h = bh % H;
@@ -766,7 +766,7 @@ AttnT mk(const void* p, const long* s) { return AttnT{(bf16_t*)p, s[0], s[1], s[
 int tfb_attn64_fwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs, void* o,
                         const long* os, float* lse, int B, int H, int T, float scale, int nw, hipStream_t s) {
   hipLaunchKernelGGL(attn64_fwd_kernel, dim3(paired_grid(T / 128), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(o, os), lse,
-                     T, H, scale * LOG2E, nw);
+                     T, H, scale * LOG2E, nw, tfb_resident_slots(2));
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
@@ -782,10 +782,10 @@ int tfb_attn64_bwd_impl(const void* q, const long* qs, const void* k, const long
                      stats, T, H, rows, 1.0f / scale);
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(attn64_dkdv_kernel, dim3(paired_grid(T / 128), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
-                     mk(dk, dks), mk(dv, dvs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t, nw);
+                     mk(dk, dks), mk(dv, dvs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t, nw, tfb_resident_slots(2));
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(attn64_dq_kernel, dim3(paired_grid(T / 128), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
-                     mk(dq, dqs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t, nw);
+                     mk(dq, dqs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t, nw, tfb_resident_slots(2));
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

@@ -75,7 +75,7 @@ __device__ __forceinline__ void unpack8bf(u32x4 u, float (&v)[8]) {
 
 // fp32 -> OCP fp8 bytes (gfx950's v_cvt_pk_*_f32 are OCP e4m3fn / e5m2, round to nearest
 // even). Inputs are clamped to the format's finite range first, so a value beyond it
-// saturates instead of becoming NaN/Inf; inside the range the bytes are torch's
+// saturates instead of becoming NaN/Inf (a NaN input stays NaN, as in torch's cast); inside the range the bytes are torch's
 // .to(float8_e4m3fn) / .to(float8_e5m2).
 #define TFB_E4M3_MAX 448.0f
 #define TFB_E5M2_MAX 57344.0f
@@ -85,12 +85,12 @@ __device__ __forceinline__ void unpack8bf(u32x4 u, float (&v)[8]) {
 // CLAMP = false: for values the caller has already bounded inside the format's range.
 template <int FMT, bool CLAMP = true>
 __device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, float d) {
-  if (CLAMP) {
+  if (CLAMP) {  // saturate the finite values; a NaN stays a NaN (fminf / fmaxf alone would turn it into -max)
     const float mx = FMT == TFB_FMT_E4M3 ? TFB_E4M3_MAX : TFB_E5M2_MAX;
-    a = fminf(fmaxf(a, -mx), mx);
-    b = fminf(fmaxf(b, -mx), mx);
-    c = fminf(fmaxf(c, -mx), mx);
-    d = fminf(fmaxf(d, -mx), mx);
+    a = a != a ? a : fminf(fmaxf(a, -mx), mx);
+    b = b != b ? b : fminf(fmaxf(b, -mx), mx);
+    c = c != c ? c : fminf(fmaxf(c, -mx), mx);
+    d = d != d ? d : fminf(fmaxf(d, -mx), mx);
   }
   int w = 0;
   if (FMT == TFB_FMT_E4M3) {
@@ -112,6 +112,20 @@ __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
   return v;
+}
+
+// Workgroups that are resident at once when `per_cu` of them fit a compute unit: per_cu x the device's CU count (read
+// once per device). Kernels use it for what concerns the FIRST round of workgroups only (the start offset between the
+// workgroups that share a CU, the split-K cost model); 256 CUs are assumed if the query fails.
+static inline int tfb_resident_slots(int per_cu) {
+  static int cus[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return per_cu * 256;
+  if (cus[dev] == 0) {
+    int n = 0;
+    cus[dev] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
+  }
+  return per_cu * cus[dev];
 }
 
 #define TFB_LAUNCH_CHECK()                                  \

@@ -48,6 +48,7 @@ struct GemmArgs {
   int splits;   // k-splits: gridDim.x = output tiles * splits
   int gblock;   // tiles of the smaller operand per traversal block (see the kernel); 0: plain row-major traversal
   int ntp;      // tiles along p
+  int slots;    // workgroups resident at once (2 per CU): the first round of the launch
   // Grouped (ragged) launches, both optional:
   const int* q_group;    // group id of each q tile (-1: the tile is beyond the ragged extent, the workgroup exits);
   long p_group_stride;   //   the P operand of group g starts p_group_stride bytes * g further (per-expert weights)
@@ -331,7 +332,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   // under the other's MFMAs (measured -0.5 to -1.3 ms per training step; delaying both costs +0.65 ms, none is the
   // old behaviour). Only where there is a second round to overlap with and no k-split (long k-loops, small epilogues).
   constexpr int kSleeps = stagger_sleeps<Epi>::value;  // an epilogue may name its own count (static kStaggerSleeps)
-  if (Cfg::OCC == 2 && kSleeps > 0 && (a.splits == 1 || TFB_STAGGER_SPLITK) && blockIdx.x < 512 && gridDim.x >= 1024) {
+  if (Cfg::OCC == 2 && kSleeps > 0 && (a.splits == 1 || TFB_STAGGER_SPLITK) && (int)blockIdx.x < a.slots && (int)gridDim.x >= 2 * a.slots) {
     if (__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 4) & 1)  // getreg(size 4, offset 0, HW_REG_HW_ID): wave_id
       for (int i = 0; i < kSleeps; ++i) __builtin_amdgcn_s_sleep(127);  // 127 x 64 clocks each
   }
@@ -568,6 +569,7 @@ static int gemm_launch_args(GemmArgs a, int groups_y, int splits, PreP prep, Pre
   if (a.P.ld <= 0 || a.Q.ld <= 0 || a.P.ld > (1L << 28) || a.Q.ld > (1L << 28)) return TFB_ERR_SHAPE;
   if (((uintptr_t)a.P.base | (uintptr_t)a.Q.base | (uintptr_t)a.P.ld | (uintptr_t)a.Q.ld) & 15) return TFB_ERR_ARG;
   a.splits = splits;
+  a.slots = tfb_resident_slots(2);
   // traversal blocks: the largest divisor of the smaller operand's tile count whose tiles (all of k) stay under ~1.6 MB;
   // none when the whole smaller operand is that small, or when a single tile of it is already larger
   a.gblock = 0;
@@ -706,21 +708,22 @@ static inline int splitk_reduce(const float* ws, void* out, long n, int splits, 
 
 // How many k-splits a token-contraction GEMM with `tiles` output tiles and `nkt` k-tiles should use.
 // 8 splits (one per XCD: each XCD then fetches only its own k-range of both operands; measured 8-20 % faster than the
-// best other count at equal occupancy) when that fills at least 80 % of whole rounds of the 512 workgroup slots
-// (256 CUs x 2 resident workgroups) or fits one round. Otherwise a cost model in units of one k-tile of one workgroup:
+// best other count at equal occupancy) when that fills at least 80 % of whole rounds of the resident workgroup slots
+// (2 per CU: 512 on the 256 CUs of an MI355X) or fits one round. Otherwise a cost model in units of one k-tile of one workgroup:
 // rounds x (k-tiles per split + 10 for prologue and epilogue) + the fp32 partials' round trip through memory (8 bytes
 // per output element and split at ~4 TB/s, one k-tile ~0.7 us).
 static inline int choose_splits(long tiles, int nkt, long out_elems, long ws_bytes) {
-  if (tiles >= 1024 || nkt < 32) return 1;
+  const long slots = tfb_resident_slots(2);
+  if (tiles >= 2 * slots || nkt < 32) return 1;
   if (nkt >= 8 * 16 && 8 * out_elems * 4 <= ws_bytes) {
-    const long wgs = tiles * 8, rounds = (wgs + 511) / 512;
-    if (rounds == 1 || (double)wgs >= 0.8 * (double)(rounds * 512)) return 8;
+    const long wgs = tiles * 8, rounds = (wgs + slots - 1) / slots;
+    if (rounds == 1 || (double)wgs >= 0.8 * (double)(rounds * slots)) return 8;
   }
   int best = 1;
   double best_cost = 1e30;
   for (int sp = 1; sp <= 32; ++sp) {
     if (sp > 1 && (nkt / sp < 16 || (long)sp * out_elems * 4 > ws_bytes)) break;
-    const long rounds = (tiles * sp + 511) / 512;
+    const long rounds = (tiles * sp + slots - 1) / slots;
     const double cost = (double)rounds * ((double)nkt / sp + 10.0) + (sp > 1 ? sp * (double)out_elems * 2e-6 / 0.7 : 0.0);
     if (cost < best_cost) {
       best_cost = cost;

@@ -34,11 +34,13 @@ _WS = {}
 
 
 def _workspace(device, nbytes=256 << 20):
-    """One fp32 split-K workspace per device, allocated on first use."""
-    ws = _WS.get(device)
+    """One fp32 split-K workspace per (device, stream), allocated on first use: launches on different streams would
+    otherwise race on the same partial sums."""
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    ws = _WS.get(key)
     if ws is None or ws.numel() * 4 < nbytes:
         ws = torch.empty(nbytes // 4, dtype=torch.float32, device=device)
-        _WS[device] = ws
+        _WS[key] = ws
     return ws
 
 
@@ -895,9 +897,10 @@ def ns5(g, d, coeffs=NS_COEFFS):
         raise ValueError("one denominator per matrix")
     _chk(inv, torch.float32)
     need = _lib.lib().tfb_ns5_workspace_bytes(K, M, N)
-    key = (g.device, need)
+    # one workspace per (device, stream), grown to the largest stack seen (never one per shape)
+    key = (g.device, torch.cuda.current_stream(g.device).cuda_stream)
     ws = _NS_WS.get(key)
-    if ws is None:
+    if ws is None or ws.numel() < need:
         ws = _NS_WS[key] = torch.empty(max(need, 256), dtype=torch.uint8, device=g.device)
     y = torch.empty(K, r, c, dtype=bf16, device=g.device)
     v = torch.empty(K, M, dtype=torch.float32, device=g.device)
