@@ -1,7 +1,7 @@
 """AdamW oracle: R1:9670-9677 (_adamw_update) == R2:13756-13766 (adamw_math_body): decay, two lerps, the update
 divided by the two bias corrections separately, one subtraction. Not torch.optim.AdamW's operation order.
 
-Pinned by (tests/test_oracle_misc.py): agreement with torch.optim.AdamW to fp32 rounding over several steps, and the
+Pinned by (tests/test_oracle_norm_loss.py): agreement with torch.optim.AdamW to fp32 rounding over several steps, and the
 closed form of the first step from zero state (update = lr * g / (|g| + eps), independent of beta)."""
 import torch
 

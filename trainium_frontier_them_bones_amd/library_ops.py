@@ -7,8 +7,9 @@ The ops allocate and return fresh outputs and mutate nothing, so they can be tra
 Registered (namespace `tfb`):
   tfb::attn_fwd(q, k, v, scale) -> (o [B,T,H,D], lse [B,H,T])          tfb::attn_bwd(q, k, v, o, do, lse, scale) -> (dq, dk, dv)
   tfb::mlp8_precast(w_fc, w_proj, sc) -> w8 [4, F d]                    (s2mlp8l::precast)
-  tfb::mlp8_fwd(x2, w_fc, w_proj, sc, w8) -> (y [M,d], r [M,F])         (s2mlp8l::fwd; r token-major, the reference's rT^T)
-  tfb::mlp8_bwd(dy2, r, x2, w_fc, w_proj, sc, w8) -> (dx, dw_fc, dw_proj)   (s2mlp8l::bwd)
+  tfb::mlp8_fwd(x2, w_fc, w_proj, sc, w8) -> (y [M,d], rT [F,M])        (s2mlp8l::fwd; rT is the reference's shape, here the
+                                                                         transposed VIEW of the token-major r [M,F] the kernels keep)
+  tfb::mlp8_bwd(dy2, rT, x2, w_fc, w_proj, sc, w8) -> (dx, dw_fc, dw_proj)  (s2mlp8l::bwd)
   tfb::loss_head_fwd(logits, targets, row_w, softcap) -> (loss_rows, lz)    tfb::loss_head_bwd(logits, targets, lz, g, softcap) -> dlogits
 `register()` is idempotent and returns the dict of op callables.
 """
@@ -68,12 +69,13 @@ def register():
     def mlp8_fwd(x2: torch.Tensor, w_fc: torch.Tensor, w_proj: torch.Tensor, sc: torch.Tensor,
                  w8: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
         y, r = ops.mlp8_fwd(x2.contiguous(), w8, sc, w_fc.shape[0])
-        return y, r
+        return y, r.t()   # [F, M] as the reference's op returns it (round2/source/train.py:6858); no copy
 
     @op("tfb::mlp8_bwd", mutates_args=())
-    def mlp8_bwd(dy2: torch.Tensor, r: torch.Tensor, x2: torch.Tensor, w_fc: torch.Tensor, w_proj: torch.Tensor,
+    def mlp8_bwd(dy2: torch.Tensor, rT: torch.Tensor, x2: torch.Tensor, w_fc: torch.Tensor, w_proj: torch.Tensor,
                  sc: torch.Tensor, w8: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
         dy2 = dy2.contiguous()
+        r = rT.t().contiguous()                    # token-major [M, F]: free for the view mlp8_fwd returned
         sc_b = ops.mlp8_backward_scales(dy2, sc)   # this call's dy amax and the dpre bound, on the device
         dx, _, dpre = ops.mlp8_bwd(dy2, r, w8, sc_b, want_h=False)
         return dx, ops.matmul(dpre, x2.contiguous(), trans_a=True), ops.mlp_dw_proj(dy2, r)
@@ -84,22 +86,22 @@ def register():
 
     @torch.library.register_fake("tfb::mlp8_fwd")
     def _(x2, w_fc, w_proj, sc, w8):
-        return torch.empty_like(x2), x2.new_empty(x2.shape[0], w_fc.shape[0])
+        return torch.empty_like(x2), x2.new_empty(x2.shape[0], w_fc.shape[0]).t()
 
     @torch.library.register_fake("tfb::mlp8_bwd")
-    def _(dy2, r, x2, w_fc, w_proj, sc, w8):
+    def _(dy2, rT, x2, w_fc, w_proj, sc, w8):
         return torch.empty_like(dy2), torch.empty_like(w_fc), torch.empty_like(w_proj)
 
     def mlp_setup(ctx, inputs, output):
         x2, w_fc, w_proj, sc, w8 = inputs
-        _y, r = output
-        ctx.save_for_backward(x2, r, w_fc, w_proj, sc, w8)
-        ctx.mark_non_differentiable(r)
+        _y, rT = output
+        ctx.save_for_backward(x2, rT, w_fc, w_proj, sc, w8)
+        ctx.mark_non_differentiable(rT)
         ctx.set_materialize_grads(False)
 
     def mlp_backward(ctx, dy2, _d_r):
-        x2, r, w_fc, w_proj, sc, w8 = ctx.saved_tensors
-        dx, dw_fc, dw_proj = mlp8_bwd(dy2, r, x2, w_fc, w_proj, sc, w8)
+        x2, rT, w_fc, w_proj, sc, w8 = ctx.saved_tensors
+        dx, dw_fc, dw_proj = mlp8_bwd(dy2, rT, x2, w_fc, w_proj, sc, w8)
         return dx, dw_fc, dw_proj, None, None
 
     torch.library.register_autograd("tfb::mlp8_fwd", mlp_backward, setup_context=mlp_setup)

@@ -252,13 +252,25 @@ class _EmbeddingShadowFn(torch.autograd.Function):
 
 
 # ------------------------------------------------------------------------------------------ fp8 fused MLP (R2:6617, 6947)
-def fp8_refresh_weights(mlps, e4m3_limit=240.0, x_scale=4.0, dw_fp8=False):
-    """Once per optimizer step: every MLP's scale row and e4m3 weight bytes (R2:6617 fp8_refresh_weights; the reference
-    keeps them on the module as mlp8_sc / mlp8_w8, here as mlp.tfb_mlp8)."""
+def fp8_refresh_weights(model, quantise_fn=None, *, e4m3_limit=240.0, x_scale=4.0, dw_fp8=False):
+    """Once per optimizer step: every MLP's scale row and e4m3 weight bytes (R2:6617 fp8_refresh_weights(model,
+    quantise_fn=None); the reference keeps them on the module as mlp8_sc / mlp8_w8, here as mlp.tfb_mlp8). `model` is
+    the reference's model (its MLPs are model.transformer.h[i].mlp) or any iterable of modules with c_fc / c_proj.
+    quantise_fn, when given, replaces the library's refresh and is called as the reference calls its own
+    (R2:6638: quantise(c_proj weights, c_fc weights, destinations, destinations)), the destinations being the MLPs'
+    Mlp8State objects."""
+    blocks = getattr(getattr(model, "transformer", None), "h", None)
+    mlps = [blk.mlp for blk in blocks] if blocks is not None else list(model)
+    states = []
     for mlp in mlps:
         st = getattr(mlp, "tfb_mlp8", None)
         if st is None:
             st = mlp.tfb_mlp8 = A.Mlp8State(e4m3_limit, x_scale, dw_fp8)
+        states.append(st)
+    if quantise_fn is not None:
+        quantise_fn([m.c_proj.weight for m in mlps], [m.c_fc.weight for m in mlps], states, states)
+        return
+    for mlp, st in zip(mlps, states):
         st.refresh(mlp.c_fc.weight.detach().to(bf16), mlp.c_proj.weight.detach().to(bf16))
 
 
