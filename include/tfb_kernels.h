@@ -335,6 +335,14 @@ int tfb_moe_route(const void* h, const void* wr, const void* bias, void* logits,
 int tfb_moe_tables(const void* idx, void* cnt, void* seg, void* tile_expert, void* slot, void* tok, void* ksel, void* scratch,
                    long N, int E, int topk, long rmax, void* stream);
 
+/* The slot tables under the reference's per-sequence capacity: the N tokens are N / T sequences of T; of one sequence's
+ * assignments to one expert (both choices, token order) the first cap keep a row, the rest get slot -1 (they read the
+ * reference's zero row and receive no gradient). cnt [E]: kept assignments; cnt_all [E]: all of them (the load-balance
+ * term's shares). scratch: int32 [2 * ceil(N/64) * E]. Status 1 unless T % 64 == 0, N % T == 0, cap >= 1.
+ * Replaces moe_positions + moe_gather_tables with their capacity (round2/source/train.py:10555-10634: pos < cap keeps). */
+int tfb_moe_tables_cap(const void* idx, void* cnt, void* cnt_all, void* seg, void* tile_expert, void* slot, void* tok, void* ksel,
+                       void* scratch, long N, long T, int cap, int E, int topk, long rmax, void* stream);
+
 /* xs bf16 [rmax][d] = h[tok] (zero padding rows) and xs8 = e4m3(xs * scale) (scale_ptr device fp32 or scale_imm).
  * Replaces MoeDispatch2.forward (round2/source/train.py:10652-10660). */
 int tfb_moe_gather(const void* h, const void* tok, const void* scale_ptr, float scale_imm, void* xs, void* xs8, long rmax, int d,

@@ -11,7 +11,8 @@ row (R2:10735-10737). Gradients come from torch.autograd over these expressions 
 
 Pinned by (tests/test_oracle_moe.py): torch.topk for the selections, gates summing to one, a brute-force per-token loop
 with the bf16 expert MLP, permutation equivariance over tokens, and the reference's capacity layout computed with a cumsum
-giving the same output when nothing is dropped.
+giving the same output when nothing is dropped; the capacity's keep rule by a plain loop over each sequence's tokens, and the
+reference's [E][b][cap] buffer with its zero row for skipped assignments giving the same output bit for bit when it drops.
 """
 import torch
 import torch.nn.functional as F
@@ -44,22 +45,34 @@ def select(p, topk):
     return torch.stack([i1, i2], 1), torch.stack([v1 / den, v2 / den], 1)
 
 
-def tables(idx, E):
-    """Dropless ragged layout: expert e's assignments contiguous in token order, segments padded to 128 rows.
-    Returns (slot [N, k] int64, tok [R] int64 (-1 padding), seg [E+1])."""
+def tables(idx, E, seq_len=None, capacity=None):
+    """Ragged layout: expert e's assignments contiguous in token order, segments padded to 128 rows.
+    Returns (slot [N, k] int64, tok [R] int64 (-1 padding), seg [E+1]).
+    With seq_len and capacity, the reference's keep rule (round2/source/train.py:10555 moe_positions, :10600 keep = pos < cap):
+    an assignment's position is the number of assignments to its expert at earlier tokens of the same sequence, both choices
+    counted; positions at or beyond the capacity are skipped (slot -1) and hold no row."""
     N, k = idx.shape
     flat_e = idx.reshape(-1)
-    cnt = torch.bincount(flat_e, minlength=E)
+    onehot = F.one_hot(flat_e, E).reshape(N, k, E).sum(1)             # assignments per token per expert (0/1)
+    if capacity is None:
+        keep = torch.ones(N, k, dtype=torch.bool)
+    else:
+        oh3 = onehot.reshape(N // seq_len, seq_len, E)
+        excl = (torch.cumsum(oh3, 1) - oh3).reshape(N, E)             # earlier tokens of the same sequence
+        keep = excl.gather(1, idx) < capacity
+    kept = torch.zeros(N, E, dtype=torch.long)
+    kept.scatter_add_(1, idx, keep.long())                            # kept assignments per token per expert (0/1)
+    cnt = kept.sum(0)
     pad = (cnt + 127) // 128 * 128
     seg = torch.zeros(E + 1, dtype=torch.long)
     seg[1:] = torch.cumsum(pad, 0)
-    onehot = F.one_hot(flat_e, E).reshape(N, k, E).sum(1)             # assignments per token per expert (0/1)
-    before = torch.cumsum(onehot, 0) - onehot                         # from earlier tokens
+    before = torch.cumsum(kept, 0) - kept                             # kept ones from earlier tokens
     pos = before.gather(1, idx)
-    slot = seg[idx] + pos
+    slot = torch.where(keep, seg[idx] + pos, torch.full_like(pos, -1))
     tok = torch.full((int(seg[-1]),), -1, dtype=torch.long)
     for j in range(k):
-        tok[slot[:, j]] = torch.arange(N)
+        kj = keep[:, j]
+        tok[slot[kj, j]] = torch.arange(N)[kj]
     return slot, tok, seg
 
 
@@ -82,7 +95,8 @@ class _ExpertMlp8(torch.autograd.Function):
         return dx, dw_fc, dw_proj, None, None, None
 
 
-def moe_forward(h, router, w_fc, w_proj, topk, bias=None, fp8=True, e4m3_limit=240.0, x_scale=4.0, dys_amax=None):
+def moe_forward(h, router, w_fc, w_proj, topk, bias=None, fp8=True, e4m3_limit=240.0, x_scale=4.0, dys_amax=None,
+                capacity=None):
     """h [.., d] bf16; router [E, d]; w_fc [E, F, d]; w_proj [E, d, F]. Differentiable (autograd) in h, router, weights.
     dys_amax (optional, fp32 [E]): per-expert amax of the expert outputs' gradients to take the backward scales from,
     for a call that holds only some of the layer's tokens."""
@@ -90,7 +104,7 @@ def moe_forward(h, router, w_fc, w_proj, topk, bias=None, fp8=True, e4m3_limit=2
     h2 = h.reshape(-1, d)
     E = w_fc.shape[0]
     p, idx, gate, _ = route(h2, router, topk, bias)
-    slot, tok, seg = tables(idx, E)
+    slot, tok, seg = tables(idx, E) if capacity is None else tables(idx, E, h.shape[-2], capacity)
     pad = torch.cat([h2, h2.new_zeros(1, d)], 0)
     xs = pad.index_select(0, torch.where(tok >= 0, tok, torch.full_like(tok, h2.shape[0])))
     outs = []
@@ -106,9 +120,11 @@ def moe_forward(h, router, w_fc, w_proj, topk, bias=None, fp8=True, e4m3_limit=2
             outs.append(F.linear(torch.relu(F.linear(xe, w_fc[e])).square(), w_proj[e]))
     ys = torch.cat(outs, 0)
     dt = ys.dtype
-    out = gate[:, 0].to(dt).unsqueeze(-1) * ys.index_select(0, slot[:, 0])
+    ysp = torch.cat([ys, ys.new_zeros(1, ys.shape[1])], 0)            # a skipped assignment reads the zero row
+    sl = torch.where(slot >= 0, slot, torch.full_like(slot, ys.shape[0]))
+    out = gate[:, 0].to(dt).unsqueeze(-1) * ysp.index_select(0, sl[:, 0])
     if topk == 2:
-        out = out + gate[:, 1].to(dt).unsqueeze(-1) * ys.index_select(0, slot[:, 1])
+        out = out + gate[:, 1].to(dt).unsqueeze(-1) * ysp.index_select(0, sl[:, 1])
     return out.reshape(h.shape), {"p": p, "idx": idx, "gate": gate, "slot": slot, "tok": tok, "seg": seg}
 
 

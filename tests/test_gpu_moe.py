@@ -247,3 +247,82 @@ def test_moe_config5_full_size_backward(dev, skew):
     oo.backward(dout[S])
     assert rel_l2(out[S], oo) < 2e-2
     assert rel_l2(hd.grad[S], ho.grad) < 2e-2
+
+
+@pytest.mark.parametrize("topk,skew,cap", [(2, 0.0, 100), (2, 2.0, 64), (1, 2.0, 40), (2, 0.0, 512)])
+def test_capacity_tables_bit_exact(dev, topk, skew, cap):
+    """The reference's per-sequence capacity (round2/source/train.py:10555-10600) is index work: on the kernel's own
+    selections the oracle's keep rule must give the same slots (-1 for a skipped assignment), rows and segments bit for bit;
+    a capacity nobody reaches (the last case) gives the dropless tables."""
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import ops
+    b, t, E = 4, 512, 8
+    h, router, _, _, bias = _layer(21, b * t, 256, 512, E, skew)
+    _, idx, _, _ = ops.moe_route(h.to(dev), router.to(dev), topk, bias.to(dev))
+    tab = ops.moe_tables(idx, E, t, cap)
+    slot, tok, seg = O.tables(idx.cpu().long(), E, t, cap)
+    assert torch.equal(tab["slot"].cpu().long(), slot)
+    assert torch.equal(tab["seg"].cpu().long(), seg)
+    R = int(seg[-1])
+    assert torch.equal(tab["tok"].cpu().long()[:R], tok) and bool((tab["tok"].cpu()[R:] == -1).all())
+    kept = torch.bincount(idx.cpu().long()[slot >= 0], minlength=E)
+    assert torch.equal(tab["cnt"].cpu().long(), kept)
+    assert torch.equal(tab["cnt_all"].cpu().long(), torch.bincount(idx.cpu().long().reshape(-1), minlength=E))
+    te = tab["tile_expert"].cpu()
+    for e in range(E):
+        assert bool((te[int(seg[e]) // 128:int(seg[e + 1]) // 128] == e).all())
+    dropped = int((slot < 0).sum())
+    if cap == 512:
+        free = ops.moe_tables(idx, E)
+        assert dropped == 0 and all(torch.equal(tab[k], free[k]) for k in ("slot", "seg", "tok", "cnt", "tile_expert"))
+        live = free["tok"] >= 0                                                 # (ksel is only defined for rows that hold a token)
+        assert torch.equal(tab["ksel"][live], free["ksel"][live])
+    else:
+        assert dropped > 100                                                    # the case does drop
+
+
+def test_capacity_rejects_a_sequence_that_is_not_whole_wavefronts(dev):
+    from trainium_frontier_them_bones_amd import ops
+    from trainium_frontier_them_bones_amd._lib import TfbError
+    idx = torch.zeros(200, 2, dtype=torch.int32, device=dev)
+    idx[:, 1] = 1
+    with pytest.raises(TfbError):
+        ops.moe_tables(idx, 4, 100, 8)
+
+
+def test_moe_layer_with_capacity_forward_backward(dev):
+    """The whole routed layer with a capacity that drops about a sixth of the assignments, against the oracle's restatement
+    of the reference's keep rule: output, input / router / expert-weight gradients, and the load shares of the auxiliary term
+    (made of EVERY assignment, kept or not: round2/source/train.py:10786 takes them from the masks)."""
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import autograd as A
+    from trainium_frontier_them_bones_amd import ops
+    b, t, d, Fd, E, topk, cap = 4, 512, 256, 512, 8, 2, 96
+    h, router, wf, wp, bias = _layer(22, b * t, d, Fd, E, 2.0)
+    h = h.reshape(b, t, d)
+    hd, rd, wfd, wpd = (x.to(dev).requires_grad_(True) for x in (h, router, wf, wp))
+    st = A.Moe8State()
+    st.refresh(wfd, wpd)
+    out, aux, terms = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, st, topk, bias.to(dev), (0.01, 0.001), cap)
+    g = torch.randn(b, t, d, generator=torch.Generator().manual_seed(3)).bfloat16()
+    (out.float() * g.to(dev).float()).sum().add(aux).backward()
+    ho, ro, wfo, wpo = (x.clone().requires_grad_(True) for x in (h, router, wf, wp))
+    oo, info = O.moe_forward(ho, ro, wfo, wpo, topk, bias, capacity=cap)
+    # the comparison needs the two routers to agree on every pick (a different pick would move every later position of
+    # its sequence); the kernel's picks are held to the reference's rule bit for bit in test_routing_tables_bit_exact
+    _, idx, _, _ = ops.moe_route(hd.detach().reshape(-1, d), rd.detach(), topk, bias.to(dev))
+    assert torch.equal(idx.cpu().long(), info["idx"]), "near-tie between the two routers: pick another seed"
+    frac = float((info["slot"] < 0).float().mean())
+    assert 0.05 < frac < 0.5
+    p_o, logits_o = info["p"], torch.nn.functional.linear(ho.reshape(-1, d).float(), ro.float()) + bias
+    lb, z, f = O.aux_terms(p_o, logits_o, info["idx"], topk)
+    (oo.float() * g.float()).sum().add(0.01 * lb + 0.001 * z).backward()
+    assert rel_l2(out, oo) < 2e-2
+    assert rel_l2(terms[2:], f) < 1e-6 and abs(float(terms[0]) - float(lb.detach())) < 1e-4 * abs(float(lb.detach()))
+    assert rel_l2(hd.grad, ho.grad) < 2e-2
+    assert rel_l2(wfd.grad, wfo.grad) < 2e-2 and rel_l2(wpd.grad, wpo.grad) < 2e-2
+    assert rel_l2(rd.grad, ro.grad) < 2e-2
+    # a skipped assignment adds nothing: tokens whose BOTH picks were skipped come out exactly zero
+    both = (info["slot"] < 0).all(1).reshape(b, t)
+    if bool(both.any()):
+        assert float(out.detach().cpu()[both].abs().max()) == 0.0

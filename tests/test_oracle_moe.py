@@ -92,6 +92,49 @@ def test_reference_capacity_layout_gives_same_output_when_nothing_drops():
     assert torch.equal(out, ref)
 
 
+def test_capacity_keep_rule_against_a_token_loop_and_the_reference_layout():
+    """With a capacity that does drop: (1) the keep decisions equal a plain loop over each sequence's tokens (an assignment's
+    position = assignments to its expert at EARLIER tokens of the sequence, both choices; keep while below cap, R2:10555-10600);
+    (2) kept rows are dense per expert in token order; (3) the reference's [E][b][cap] slot buffer with its zero row for
+    skipped assignments (R2:10600: slot = S) gives the oracle's output bit for bit."""
+    h, router, wf, wp = _layer(6, N=256)
+    b, t, E, cap = 2, 128, 8, 20
+    _, idx, gate, _ = O.route(h, router, 2)
+    slot, tok, seg = O.tables(idx, E, t, cap)
+    keep_loop = torch.zeros(b * t, 2, dtype=torch.bool)
+    for r in range(b):
+        count = [0] * E
+        for i in range(r * t, (r + 1) * t):
+            for j in range(2):
+                keep_loop[i, j] = count[int(idx[i, j])] < cap
+            for j in range(2):
+                count[int(idx[i, j])] += 1
+    assert torch.equal(slot >= 0, keep_loop)
+    assert int((~keep_loop).sum()) > 50 and int(keep_loop.sum()) > 50          # the case does drop, and does keep
+    for e in range(E):
+        want = [(i, j) for i in range(b * t) for j in range(2) if int(idx[i, j]) == e and keep_loop[i, j]]
+        rows = tok[int(seg[e]):int(seg[e]) + len(want)]
+        assert rows.tolist() == [i for i, _ in want]
+        assert all(int(slot[i, j]) == int(seg[e]) + n for n, (i, j) in enumerate(want))
+        assert (tok[int(seg[e]) + len(want):int(seg[e + 1])] == -1).all()
+    # the reference's layout and zero row
+    mall = F.one_hot(idx, E).sum(1).reshape(b, t, E)
+    excl = (torch.cumsum(mall, 1) - mall).reshape(b * t, E)
+    row = torch.arange(b).repeat_interleave(t)
+    pos = excl.gather(1, idx)
+    S = E * b * cap
+    rslot = torch.where(pos < cap, (idx * b + row[:, None]) * cap + pos, torch.full_like(pos, S))
+    xs = torch.zeros(S + 1, h.shape[1], dtype=h.dtype)
+    for j in range(2):
+        xs[rslot[:, j]] = h
+    xs[S] = 0
+    ys = torch.stack([F.linear(torch.relu(F.linear(xs[:S].reshape(E, b * cap, -1)[e], wf[e])).square(), wp[e]) for e in range(E)])
+    ys = torch.cat([ys.reshape(S, -1), ys.new_zeros(1, ys.shape[-1])], 0)
+    out = gate[:, 0].bfloat16()[:, None] * ys[rslot[:, 0]] + gate[:, 1].bfloat16()[:, None] * ys[rslot[:, 1]]
+    ref, _ = O.moe_forward(h.reshape(b, t, -1), router, wf, wp, 2, fp8=False, capacity=cap)
+    assert torch.equal(out, ref.reshape(b * t, -1))
+
+
 def test_backward_is_consistent_with_plain_autograd():
     h, router, wf, wp = _layer(5, N=128)
     hs = [h.clone().requires_grad_(True) for _ in range(2)]

@@ -614,7 +614,7 @@ class MoeMlp8Fn(torch.autograd.Function):
     w_fc [E, F, d], w_proj [E, d, F] bf16; router_bias fp32 [E] or None (added to the logits)."""
 
     @staticmethod
-    def forward(ctx, h, router, w_fc, w_proj, state, topk, router_bias, aux_weights=None):
+    def forward(ctx, h, router, w_fc, w_proj, state, topk, router_bias, aux_weights=None, capacity=None):
         """aux_weights = (alpha, beta): also returns (aux, stats) with aux = alpha lb + beta z, the router's weighted
         load-balance and z terms (round2/source/train.py:10779 moe_aux_terms; differentiable, its gradient joins the
         router's in the backward), and stats fp32 [2 + E] = (lb, z, the experts' load shares f_e)."""
@@ -622,7 +622,9 @@ class MoeMlp8Fn(torch.autograd.Function):
         E, F, d = w_fc.shape
         wr = router.detach().float().contiguous()
         p, idx, gate, logits = ops.moe_route(h2, wr, topk, router_bias, want_logits=aux_weights is not None)
-        tab = ops.moe_tables(idx, E)
+        # capacity: the reference's per-sequence count (round2/source/train.py:10555): each row of h [b, t, d] keeps its first
+        # `capacity` assignments per expert; None keeps everything
+        tab = ops.moe_tables(idx, E) if capacity is None else ops.moe_tables(idx, E, h.shape[-2], capacity)
         xs, xs8 = ops.moe_gather(h2, tab, state.x_scale)
         ys, r = ops.moe_mlp8_fwd(xs8, state.w8, state.rows, tab, F)
         out = ops.moe_combine(ys, tab, gate, h2.shape[0])
@@ -667,4 +669,4 @@ class MoeMlp8Fn(torch.autograd.Function):
             dw_fc, dw_proj = ops.moe_dw(dpre, xs, dys, r, tab, E)
         br, accr = _accumulate_into(router)
         dh, dwr, _ = ops.moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, br, accr, aux=aux)
-        return dh.view(ctx.hshape), (None if br is not None else dwr.to(router.dtype)), dw_fc, dw_proj, None, None, None, None
+        return dh.view(ctx.hshape), (None if br is not None else dwr.to(router.dtype)), dw_fc, dw_proj, None, None, None, None, None

@@ -173,10 +173,34 @@ __global__ __launch_bounds__(256) void moe_scan_kernel(int* __restrict__ wave_cn
   }
 }
 
-// Every assignment's row: seg[e] + (assignments to e from earlier wavefronts) + (from earlier lanes of this one).
+// The reference's per-sequence capacity (round2/source/train.py:10555 moe_positions, :10600 keep = pos < cap): an assignment's
+// position is the number of assignments to its expert at EARLIER tokens of the same sequence (both choices count); the
+// first `cap` of a sequence are kept, the rest are skipped. One thread per (sequence, expert) walks the sequence's
+// wavefronts (a sequence is a whole number of 64-token wavefronts): pre[w][e] = assignments before wavefront w inside its
+// sequence, wave_cnt[w][e] becomes the number KEPT in the wavefront (the earliest lanes), cnt_all[e] every assignment.
+__global__ __launch_bounds__(256) void moe_cap_kernel(int* __restrict__ wave_cnt, int* __restrict__ pre, int* __restrict__ cnt_all,
+                                                     int nseq, int wps, int E, int cap) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= nseq * E) return;
+  const int b = i / E, e = i % E;
+  int prefix = 0;
+  for (int w = b * wps; w < (b + 1) * wps; ++w) {
+    const int raw = wave_cnt[(long)w * E + e];
+    pre[(long)w * E + e] = prefix;
+    const int room = cap - prefix;
+    wave_cnt[(long)w * E + e] = room <= 0 ? 0 : (raw < room ? raw : room);
+    prefix += raw;
+  }
+  atomicAdd(cnt_all + e, prefix);
+}
+
+// Every assignment's row: seg[e] + (assignments to e from earlier wavefronts) + (from earlier lanes of this one). With a
+// capacity (pre != NULL) wave_off counts kept assignments only, and an assignment whose position inside its sequence
+// (pre + earlier lanes) reaches cap gets slot -1 and no row.
 __global__ __launch_bounds__(256) void moe_place_kernel(const int* __restrict__ idx, const int* __restrict__ wave_off,
                                                        const int* __restrict__ seg, int* __restrict__ slot,
-                                                       int* __restrict__ tok, int* __restrict__ ksel, long N, int E, int topk) {
+                                                       int* __restrict__ tok, int* __restrict__ ksel, long N, int E, int topk,
+                                                       const int* __restrict__ pre, int cap) {
   const int lane = threadIdx.x & 63;
   const long w = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   const long n = w * 64 + lane;
@@ -195,15 +219,21 @@ __global__ __launch_bounds__(256) void moe_place_kernel(const int* __restrict__ 
     if (a1 == e) r1 = before;
   }
   if (n < N) {
-    int s0 = seg[a0] + wave_off[w * E + a0] + r0;
+    const bool keep0 = !pre || pre[w * E + a0] + r0 < cap;
+    int s0 = keep0 ? seg[a0] + wave_off[w * E + a0] + r0 : -1;
     slot[n * topk] = s0;
-    tok[s0] = (int)n;
-    ksel[s0] = 0;
+    if (keep0) {
+      tok[s0] = (int)n;
+      ksel[s0] = 0;
+    }
     if (topk == 2) {
-      int s1 = seg[a1] + wave_off[w * E + a1] + r1;
+      const bool keep1 = !pre || pre[w * E + a1] + r1 < cap;
+      int s1 = keep1 ? seg[a1] + wave_off[w * E + a1] + r1 : -1;
       slot[n * 2 + 1] = s1;
-      tok[s1] = (int)n;
-      ksel[s1] = 1;
+      if (keep1) {
+        tok[s1] = (int)n;
+        ksel[s1] = 1;
+      }
     }
   }
 }
@@ -242,14 +272,17 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const bf16_t* __restri
   for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
     long n = i / cpr;
     int c = (int)(i % cpr) * 8;
-    float a[8], r[8];
-    load8(ys + (long)slot[n * topk] * d + c, a);
+    // a skipped assignment (slot -1: over the sequence's capacity) reads the reference's zero row
+    float a[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, r[8];
+    const int s1 = slot[n * topk];
+    if (s1 >= 0) load8(ys + (long)s1 * d + c, a);
     const float g1 = round_bf(gate[n * topk]);
 #pragma unroll
     for (int k = 0; k < 8; ++k) r[k] = round_bf(g1 * a[k]);
     if (topk == 2) {
-      float b[8];
-      load8(ys + (long)slot[n * 2 + 1] * d + c, b);
+      float b[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      const int s2 = slot[n * 2 + 1];
+      if (s2 >= 0) load8(ys + (long)s2 * d + c, b);
       const float g2 = round_bf(gate[n * 2 + 1]);
 #pragma unroll
       for (int k = 0; k < 8; ++k) r[k] += round_bf(g2 * b[k]);
@@ -388,13 +421,17 @@ __global__ __launch_bounds__(256) void moe_dispatch_bwd_kernel(const bf16_t* __r
   for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
     long n = i / cpr;
     int c = (int)(i % cpr) * 8;
-    float r[8];
-    load8(dxs + (long)slot[n * topk] * d + c, r);
+    float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const int s1 = slot[n * topk];
+    if (s1 >= 0) load8(dxs + (long)s1 * d + c, r);
     if (topk == 2) {
-      float b[8];
-      load8(dxs + (long)slot[n * 2 + 1] * d + c, b);
+      const int s2 = slot[n * 2 + 1];
+      if (s2 >= 0) {
+        float b[8];
+        load8(dxs + (long)s2 * d + c, b);
 #pragma unroll
-      for (int k = 0; k < 8; ++k) r[k] += b[k];
+        for (int k = 0; k < 8; ++k) r[k] += b[k];
+      }
     }
     if (dlogits) {
       for (int e = 0; e < E; ++e) {
@@ -597,7 +634,41 @@ extern "C" int tfb_moe_tables(const void* idx, void* cnt, void* seg, void* tile_
                      (int*)tile_expert, (int)(rmax / 128));
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(moe_place_kernel, dim3(nb), dim3(256), 0, s, (const int*)idx, (const int*)scratch, (const int*)seg,
-                     (int*)slot, (int*)tok, (int*)ksel, N, E, topk);
+                     (int*)slot, (int*)tok, (int*)ksel, N, E, topk, (const int*)nullptr, 0);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// tfb_moe_tables with the reference's per-sequence capacity (round2/source/train.py:10555-10600): the tokens are N / T
+// sequences of T; of a sequence's assignments to one expert (both choices, in token order) the first `cap` keep a row, the
+// rest get slot -1 (the reference's zero row: they add nothing to the output and receive no gradient). cnt [E] counts the
+// kept assignments (the segments' extents), cnt_all [E] every assignment (what the load-balance term's f_e is made of).
+// scratch: int32 [2 * ceil(N/64) * E]. T % 64 == 0 (a sequence is a whole number of wavefronts), N % T == 0, cap >= 1.
+extern "C" int tfb_moe_tables_cap(const void* idx, void* cnt, void* cnt_all, void* seg, void* tile_expert, void* slot, void* tok,
+                                  void* ksel, void* scratch, long N, long T, int cap, int E, int topk, long rmax, void* stream) {
+  if (!idx || !cnt || !cnt_all || !seg || !tile_expert || !slot || !tok || !ksel || !scratch) return TFB_ERR_ARG;
+  if (N <= 0 || E < 2 || E > MAXE || (topk != 1 && topk != 2) || rmax % 128 || rmax < tfb_moe_max_rows(N, E, topk))
+    return TFB_ERR_SHAPE;
+  if (T <= 0 || T % 64 || N % T || cap < 1) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const int nwaves = (int)(N / 64);
+  const int nb = (nwaves + 3) / 4;
+  const int nseq = (int)(N / T), wps = (int)(T / 64);
+  int* wave_cnt = (int*)scratch;
+  int* pre = wave_cnt + (long)nwaves * E;
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(nblocks(rmax)), dim3(256), 0, s, (int*)tok, -1, rmax);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(256), 0, s, (int*)cnt_all, 0, (long)E);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_count_kernel, dim3(nb), dim3(256), 0, s, (const int*)idx, wave_cnt, N, E, topk);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_cap_kernel, dim3((nseq * E + 255) / 256), dim3(256), 0, s, wave_cnt, pre, (int*)cnt_all, nseq, wps, E, cap);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(256), 0, s, wave_cnt, nwaves, E, (int*)cnt, (int*)seg, (int*)tile_expert,
+                     (int)(rmax / 128));
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_place_kernel, dim3(nb), dim3(256), 0, s, (const int*)idx, (const int*)wave_cnt, (const int*)seg,
+                     (int*)slot, (int*)tok, (int*)ksel, N, E, topk, (const int*)pre, cap);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
@@ -625,6 +696,7 @@ extern "C" int tfb_moe_combine(const void* ys, const void* slot, const void* gat
 }
 
 // dys bf16 [rmax][d], dgate fp32 [N][topk] from dout bf16 [N][d]. Replaces MoeCombine2.backward (10678-10688).
+// Only the assignments that hold a row are written: with a capacity in use the caller zero-fills dgate first.
 extern "C" int tfb_moe_combine_bwd(const void* dout, const void* ys, const void* tok, const void* ksel, const void* gate,
                                    void* dys, void* dgate, long rmax, int d, int topk, void* stream) {
   if (!dout || !ys || !tok || !ksel || !gate || !dys || !dgate) return TFB_ERR_ARG;

@@ -736,8 +736,10 @@ def moe_route(h2, wr, topk, bias=None, want_logits=False):
     return p, idx, gate, logits
 
 
-def moe_tables(idx, E):
-    """Slot tables for the dropless ragged layout: dict(cnt, seg, tile_expert, slot, tok, ksel, rmax)."""
+def moe_tables(idx, E, seq_len=None, capacity=None):
+    """Slot tables for the ragged layout: dict(cnt, seg, tile_expert, slot, tok, ksel, rmax). Dropless by default; with
+    seq_len and capacity the reference's per-sequence capacity (round2/source/train.py:10555-10634): each sequence keeps its
+    first `capacity` assignments per expert, the rest get slot -1; the dict then also holds cnt_all (every assignment)."""
     _chk(idx, torch.int32)
     N, topk = idx.shape
     dev = idx.device
@@ -745,9 +747,19 @@ def moe_tables(idx, E):
     i32 = dict(dtype=torch.int32, device=dev)
     t = {"cnt": torch.empty(E, **i32), "seg": torch.empty(E + 1, **i32), "tile_expert": torch.empty(rmax // 128, **i32),
          "slot": torch.empty(N, topk, **i32), "tok": torch.empty(rmax, **i32), "ksel": torch.empty(rmax, **i32), "rmax": rmax}
-    scratch = torch.empty(((N + 63) // 64) * E, **i32)
-    _lib.call("tfb_moe_tables", _p(idx), _p(t["cnt"]), _p(t["seg"]), _p(t["tile_expert"]), _p(t["slot"]), _p(t["tok"]),
-              _p(t["ksel"]), _p(scratch), N, E, topk, rmax, _stream())
+    nw = (N + 63) // 64
+    if capacity is None:
+        scratch = torch.empty(nw * E, **i32)
+        _lib.call("tfb_moe_tables", _p(idx), _p(t["cnt"]), _p(t["seg"]), _p(t["tile_expert"]), _p(t["slot"]), _p(t["tok"]),
+                  _p(t["ksel"]), _p(scratch), N, E, topk, rmax, _stream())
+        return t
+    if seq_len is None:
+        raise ValueError("a capacity is counted per sequence: seq_len is needed")
+    t["cnt_all"] = torch.empty(E, **i32)
+    t["capacity"] = int(capacity)
+    scratch = torch.empty(2 * nw * E, **i32)
+    _lib.call("tfb_moe_tables_cap", _p(idx), _p(t["cnt"]), _p(t["cnt_all"]), _p(t["seg"]), _p(t["tile_expert"]), _p(t["slot"]),
+              _p(t["tok"]), _p(t["ksel"]), _p(scratch), N, int(seq_len), int(capacity), E, topk, rmax, _stream())
     return t
 
 
@@ -830,7 +842,8 @@ def moe_combine_bwd(dout, ys, tab, gate):
     _chk(dout), _chk(ys), _chk(gate, torch.float32)
     rmax, d = ys.shape
     dys = torch.empty_like(ys)
-    dgate = torch.empty_like(gate)
+    # the kernel writes the gate gradient of every assignment that holds a row; a skipped one's is zero
+    dgate = torch.zeros_like(gate) if "capacity" in tab else torch.empty_like(gate)
     _lib.call("tfb_moe_combine_bwd", _p(dout), _p(ys), _p(tab["tok"]), _p(tab["ksel"]), _p(gate), _p(dys), _p(dgate), rmax, d,
               gate.shape[1], _stream())
     return dys, dgate
@@ -867,7 +880,7 @@ def moe_aux_fwd(p, logits, tab, topk):
     terms = torch.empty(2 + E, dtype=torch.float32, device=p.device)
     lse = torch.empty(N, dtype=torch.float32, device=p.device)
     scr = torch.empty(64 * 17, dtype=torch.float32, device=p.device)
-    _lib.call("tfb_moe_aux_fwd", _p(p), _p(logits), _p(tab["cnt"]), _p(terms), _p(lse), _p(scr), N, E, topk, _stream())
+    _lib.call("tfb_moe_aux_fwd", _p(p), _p(logits), _p(tab.get("cnt_all", tab["cnt"])), _p(terms), _p(lse), _p(scr), N, E, topk, _stream())
     return terms, lse
 
 
