@@ -15,6 +15,9 @@ one line per configuration; run under rocprofv3 --kernel-trace --stats for the p
 
 python bench.py --traffic-probe   (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: a 256 MiB device copy as the
 counters' calibration, then attention forward + backward at the benchmark shape; prints nothing)
+
+python bench.py --hw-probe        (the load-issue and LDS-interference probes of the library: what a 1 KB vector load costs the
+wavefront that issues it, and what operand streams cost the LDS fragment reads of the same CU)
 """
 import argparse
 import json
@@ -271,6 +274,25 @@ def config_probe(which):
                   6 * 2.0 * (2 * N) * d * Fd)
 
 
+def hw_probe():
+    """The two hardware probes behind the operand paths of the GEMM and attention kernels (tfb_probe_load_issue,
+    tfb_probe_lds_mix): the cost of a 1 KB vector load to the wavefront that issues it, and what operand streams cost the
+    fragment reads of the same CU."""
+    import torch
+    from trainium_frontier_them_bones_amd import ops
+    dev = torch.device("cuda:0")
+    ops.probe_load_issue(dev, True, 4, iters=200)   # warm-up
+    print("1 KB vector loads from an L2-resident 2 MB region (8 rows x 128 B at pitch 1536 per instruction):")
+    for to_lds, name in ((True, "global -> LDS DMA (global_load_lds_dwordx4)"), (False, "global -> VGPR (global_load_dwordx4)")):
+        for waves in (1, 4, 8):
+            per, bpc = ops.probe_load_issue(dev, to_lds, waves)
+            print("  %-45s %d wavefront(s) per CU: %6.1f cycles per instruction per wavefront, %5.1f B/clk/CU" % (name, waves, per, bpc))
+    print("LDS fragment reads (four wavefronts, 16 x ds_read_b128 in flight each) beside four streaming wavefronts:")
+    for mode, name in ((0, "readers alone"), (1, "+ global -> LDS DMA"), (2, "+ global -> VGPR -> ds_write_b128"), (3, "+ global -> VGPR only")):
+        rd, ld = ops.probe_lds_mix(dev, mode)
+        print("  %-36s LDS reads %6.1f B/clk/CU   streamed %5.1f B/clk/CU" % (name, rd, ld))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -279,6 +301,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true")
     ap.add_argument("--ns-probe", action="store_true")
+    ap.add_argument("--hw-probe", action="store_true")
     ap.add_argument("--config-probe", choices=("c1", "c2", "c3", "c5", "all"))
     ap.add_argument("--bf16-dw", action="store_true")
     ap.add_argument("--unfused-residual", action="store_true")
@@ -293,6 +316,9 @@ def main():
         return
     if args.ns_probe:
         ns_probe()
+        return
+    if args.hw_probe:
+        hw_probe()
         return
     if args.config_probe:
         config_probe(args.config_probe)

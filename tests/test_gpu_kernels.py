@@ -728,3 +728,16 @@ def test_autograd_nodes_do_not_corrupt_what_autograd_cannot_see(ops, dev):
     loss.backward(retain_graph=True)
     with pytest.raises(RuntimeError):
         loss.backward()
+
+
+def test_hardware_probes_run_and_report_sane_rates(ops, dev):
+    """tfb_probe_load_issue / tfb_probe_lds_mix (diagnostics): they finish, every CU reports, and the rates are inside what
+    the hardware can do (a CU's vector memory path moves well under 128 B/clk, its LDS under 512 B/clk)."""
+    per, bpc = ops.probe_load_issue(dev, True, 4, iters=300)
+    assert 4.0 < per < 5000.0 and 1.0 < bpc < 128.0
+    per1, bpc1 = ops.probe_load_issue(dev, False, 1, iters=300)
+    assert 4.0 < per1 < 5000.0 and 0.5 < bpc1 < 128.0
+    rd, ld = ops.probe_lds_mix(dev, 1, riters=2000, liters=6000)
+    assert 10.0 < rd < 512.0 and 1.0 < ld < 128.0
+    rd0, ld0 = ops.probe_lds_mix(dev, 0, riters=2000, liters=0)
+    assert 10.0 < rd0 < 512.0 and ld0 == 0.0
