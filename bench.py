@@ -243,7 +243,7 @@ def config_probe(which):
         wf = leaf((0.02 * torch.randn(d, F, generator=g)).to(bf).t().contiguous())
         wp = leaf((0.02 * torch.randn(F, d, generator=g)).to(bf).t().contiguous())
         dy = torch.randn(M, d, generator=g).to(bf).to(dev)
-        st = A.Mlp8State(e4m3_limit=448.0)
+        st = A.Mlp8State(e4m3_limit=448.0, dw_fp8=True)   # all six GEMMs in fp8: e4m3 forward, e5m2 gradients
 
         def c3():
             clear(x, wf, wp)
