@@ -41,6 +41,23 @@ struct GemmOperand {
   long ld;  // bytes between consecutive rows (K_CONTIG) or consecutive k (K_STRIDED)
 };
 
+// n / d for 0 <= n < 2^31 as one 64-bit multiply and a shift: m = ceil(2^(31 + s) / d) with s = ceil(log2 d) (exact for
+// every such n because m d - 2^(31 + s) <= 2^s). The host builds it once per launch; in the kernel a division by a launch
+// parameter would otherwise be ~25 dependent instructions per wavefront (~200 for a 64-bit one) before the first load.
+struct FastDiv {
+  uint32_t m, sh;
+};
+static inline FastDiv fastdiv_make(uint32_t d) {
+  if (d == 0) d = 1;
+  uint32_t s = 0;
+  while ((1ull << s) < d) ++s;
+  FastDiv f;
+  f.m = (uint32_t)(((1ull << (31 + s)) + d - 1) / d);
+  f.sh = 31 + s;
+  return f;
+}
+__device__ __forceinline__ int fastdiv(int n, FastDiv f) { return (int)(((uint64_t)(uint32_t)n * f.m) >> f.sh); }
+
 struct GemmArgs {
   GemmOperand P, Q;
   int np, nq;   // output extent (multiples of BP / BQ)
@@ -48,11 +65,20 @@ struct GemmArgs {
   int splits;   // k-splits: gridDim.x = output tiles * splits
   int gblock;   // tiles of the smaller operand per traversal block (see the kernel); 0: plain row-major traversal
   int ntp;      // tiles along p
-  int slots;    // workgroups resident at once (2 per CU): the first round of the launch
+  int slots;    // workgroups resident at once (2 per CU): the first round of the launch, when it is to be staggered
+                //   (see the kernel; 0: no stagger)
   // Grouped (ragged) launches, both optional:
   const int* q_group;    // group id of each q tile (-1: the tile is beyond the ragged extent, the workgroup exits);
   long p_group_stride;   //   the P operand of group g starts p_group_stride bytes * g further (per-expert weights)
   const int* k_seg;      // [groups + 1] k offsets in elements: group = blockIdx.y contracts over k_seg[g] .. k_seg[g+1]
+  // Filled by gemm_launch_args from the fields above (the workgroup -> tile map, with its divisions prepared):
+  int ntiles;   // output tiles
+  int per;      // ntiles / 8 when ntiles is a multiple of 8 (an XCD's run of tiles), else 0: no re-dealing of ids
+  int nfast;    // tiles of the operand the traversal walks fastest
+  int p_fast;   // that operand is P
+  int rows;     // block traversal: rows of tiles of the other operand in one XCD's run (0: plain traversal)
+  int blk;      // gblock * rows
+  FastDiv d_ntiles, d_per, d_nfast, d_blk, d_gblock, d_splits, d_split8;  // d_split8: by splits / 8
 };
 
 // Operand pre-operation, applied to a fragment (8 bf16 along k of one row) on its way into the MFMA.
@@ -248,13 +274,6 @@ __device__ __forceinline__ f32x16 mfma32(const FA& a, const FB& b, f32x16 c) {
   }
 }
 
-// The workgroup's (tile_p, tile_q): consecutive workgroup ids are dealt round-robin to the
-// 8 XCDs (each with its own L2), so ids are re-dealt so that one XCD gets a contiguous run
-// of tiles; p runs fastest, so a run shares its Q rows through that XCD's L2.
-__device__ __forceinline__ int xcd_remap(int pid, int nb) {
-  return (nb & 7) == 0 ? (pid & 7) * (nb >> 3) + (pid >> 3) : pid;
-}
-
 template <class T, class = void>
 struct has_for_group : std::false_type {};
 template <class T>
@@ -332,30 +351,38 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   // under the other's MFMAs (measured -0.5 to -1.3 ms per training step; delaying both costs +0.65 ms, none is the
   // old behaviour). Only where there is a second round to overlap with and no k-split (long k-loops, small epilogues).
   constexpr int kSleeps = stagger_sleeps<Epi>::value;  // an epilogue may name its own count (static kStaggerSleeps)
-  if (Cfg::OCC == 2 && kSleeps > 0 && (a.splits == 1 || TFB_STAGGER_SPLITK) && (int)blockIdx.x < a.slots && (int)gridDim.x >= 2 * a.slots) {
+  // All launch parameters the tile map and the first loads need are asked for here, in one batch: left to the compiler
+  // they are fetched where first used, four or five dependent round trips to the scalar cache in front of every tile.
+  asm volatile("" ::"s"(a.P.base), "s"(a.P.ld), "s"(a.Q.base), "s"(a.Q.ld), "s"(a.nkt), "s"(a.splits), "s"(a.gblock),
+               "s"(a.slots), "s"(a.q_group), "s"(a.p_group_stride), "s"(a.k_seg), "s"(a.ntiles), "s"(a.per), "s"(a.nfast),
+               "s"(a.p_fast), "s"(a.rows), "s"(a.blk), "s"(a.d_per.m), "s"(a.d_per.sh), "s"(a.d_nfast.m), "s"(a.d_nfast.sh),
+               "s"(a.d_blk.m), "s"(a.d_blk.sh), "s"(a.d_gblock.m), "s"(a.d_gblock.sh), "s"(a.d_splits.m), "s"(a.d_splits.sh));
+  if (Cfg::OCC == 2 && kSleeps > 0 && (int)blockIdx.x < a.slots) {
     if (__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 4) & 1)  // getreg(size 4, offset 0, HW_REG_HW_ID): wave_id
       for (int i = 0; i < kSleeps; ++i) __builtin_amdgcn_s_sleep(127);  // 127 x 64 clocks each
   }
   const int wp = wave % Cfg::WP, wq = wave / Cfg::WP;
   const int lr = lane & 31, lh = lane >> 5;
 
-  const int ntq = a.nq / BQ;
   // Workgroup -> (output tile, k-split). Consecutive workgroup ids sit on consecutive XCDs. With a multiple of 8 splits a
   // split stays on ONE XCD: the k-range of both operands it contracts over is then fetched into that XCD's L2 once and
-  // shared by all its output tiles, instead of every XCD streaming most of both operands.
+  // shared by all its output tiles, instead of every XCD streaming most of both operands. Without splits, ids are
+  // re-dealt so that one XCD gets a contiguous run of tiles. (Everything up to the first operand load below is serial
+  // scalar work in front of every tile: the divisions are multiplications prepared by the host.)
+  auto xcd_run = [&](int pid) { return a.per ? (pid & 7) * a.per + (pid >> 3) : pid; };
   int lid, split;
   {
-    const int ntiles = a.ntp * ntq, L = blockIdx.x;
-    if (a.splits > 1 && (a.splits & 7) == 0) {
-      const int m = a.splits >> 3, j = L >> 3;
-      split = (L & 7) + 8 * (j % m);
-      lid = j / m;
-    } else if (a.splits > 1) {
-      split = L / ntiles;
-      lid = xcd_remap(L % ntiles, ntiles);
-    } else {
+    const int L = blockIdx.x;
+    if (a.splits == 1) {
       split = 0;
-      lid = xcd_remap(L, ntiles);
+      lid = xcd_run(L);
+    } else if ((a.splits & 7) == 0) {
+      const int j = L >> 3;
+      lid = fastdiv(j, a.d_split8);
+      split = (L & 7) + 8 * (j - lid * (a.splits >> 3));
+    } else {
+      split = fastdiv(L, a.d_ntiles);
+      lid = xcd_run(L - split * a.ntiles);
     }
   }
   // An XCD's run of tiles walks the smaller operand's tiles fastest: the run then shares few rows of the larger
@@ -363,29 +390,28 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   // does not fit the L2 beside the streaming larger one (a 3.5 MB weight against a 4 MB L2), the run is walked in
   // blocks of `gblock` of its tiles: block 0 against all of the run's rows of the larger operand, then block 1, ...
   // so the smaller operand is fetched once per XCD instead of once per row of tiles.
-  const bool p_fast = a.np <= a.nq || a.q_group;
   int tile_p, tile_q;
   {
-    const int nfast = p_fast ? a.ntp : ntq;  // tiles of the smaller operand
-    const int per = (a.ntp * ntq) >> 3;      // tiles per XCD when the run mapping is active
     int fast, slow;
-    if (a.gblock > 0 && a.splits == 1 && ((a.ntp * ntq) & 7) == 0 && per % nfast == 0) {
-      const int rows = per / nfast;          // rows of tiles (of the larger operand) in this XCD's run
-      const int xcd = lid / per, idx = lid % per;
-      const int blk = a.gblock * rows;
-      const int b = idx / blk, rem = idx % blk;
-      fast = b * a.gblock + rem % a.gblock;
-      slow = xcd * rows + rem / a.gblock;
+    if (a.rows > 0) {
+      const int xcd = fastdiv(lid, a.d_per), idx = lid - xcd * a.per;
+      const int b = fastdiv(idx, a.d_blk), rem = idx - b * a.blk;
+      const int rg = fastdiv(rem, a.d_gblock);
+      fast = b * a.gblock + rem - rg * a.gblock;
+      slow = xcd * a.rows + rg;
     } else {
-      fast = lid % nfast;
-      slow = lid / nfast;
+      slow = fastdiv(lid, a.d_nfast);
+      fast = lid - slow * a.nfast;
     }
-    tile_p = p_fast ? fast : slow;
-    tile_q = p_fast ? slow : fast;
+    tile_p = a.p_fast ? fast : slow;
+    tile_q = a.p_fast ? slow : fast;
   }
   const long p0 = (long)tile_p * BP, q0 = (long)tile_q * BQ;
-  long kt0 = (long)split * a.nkt / a.splits;
-  a.nkt = (int)((long)(split + 1) * a.nkt / a.splits - kt0);
+  int kt0 = 0;
+  if (a.splits > 1) {
+    kt0 = fastdiv(split * a.nkt, a.d_splits);
+    a.nkt = fastdiv((split + 1) * a.nkt, a.d_splits) - kt0;
+  }
   int group = 0;
   if (a.q_group) {
     group = a.q_group[tile_q];
@@ -394,17 +420,24 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   }
   if (a.k_seg) {
     group = blockIdx.y;
-    const long k0 = a.k_seg[group], k1 = a.k_seg[group + 1];
+    const int k0 = a.k_seg[group], k1 = a.k_seg[group + 1];
     kt0 = k0 * ES / 128;
-    a.nkt = (int)((k1 - k0) * ES / 128);  // may be 0: the accumulators stay zero and are still written
+    a.nkt = (k1 - k0) * ES / 128;  // may be 0: the accumulators stay zero and are still written
   }
-  const Epi epi = epi_prepare(epi_for_group(epi_in, group));
   const int nkt = a.nkt;
 
+  // the first k-tile's loads leave before anything else is set up
   TileDma<BP, NW, Cfg::LAYP, ES> dp;
   TileDma<BQ, NW, Cfg::LAYQ, ES> dq;
-  dp.init(a.P, p0, kt0 * 128, wave, lane);
-  dq.init(a.Q, q0, kt0 * 128, wave, lane);
+  dp.init(a.P, p0, (long)kt0 * 128, wave, lane);
+  dq.init(a.Q, q0, (long)kt0 * 128, wave, lane);
+  auto issue = [&](uint8_t* buf, int t) {
+    dp.issue(buf, t, wave);
+    dq.issue(buf + BP * 128, t, wave);
+  };
+  if (nkt > 0) issue(buf0, 0);
+
+  const Epi epi = epi_prepare(epi_for_group(epi_in, group));
   typedef FragReader<BP, ES, Cfg::LAYP> RP;
   typedef FragReader<BQ, ES, Cfg::LAYQ> RQ;
   RP rp;
@@ -434,10 +467,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
         pre[j][k] = epi.prefetch((int)p0 + wp * (TP * 32) + chunk_col(k), (int)q0 + wq * (TQ * 32) + j * 32 + chunk_row(k));
   }
 
-  auto issue = [&](uint8_t* buf, int t) {
-    dp.issue(buf, t, wave);
-    dq.issue(buf + BP * 128, t, wave);
-  };
   auto compute = [&](const uint8_t* buf) {
     const uint8_t* sp = buf;
     const uint8_t* sq = buf + BP * 128;
@@ -475,7 +504,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   };
 
   {
-    if (nkt > 0) issue(buf0, 0);
     __syncthreads();
     for (int t = 0; t + 2 <= nkt; t += 2) {
       issue(buf1, t + 1);
@@ -568,21 +596,37 @@ static int gemm_launch_args(GemmArgs a, int groups_y, int splits, PreP prep, Pre
   // the per-lane part of a load address is a 32-bit offset: 8 rows (K_CONTIG) or 8 k-rows (K_STRIDED) of the operand
   if (a.P.ld <= 0 || a.Q.ld <= 0 || a.P.ld > (1L << 28) || a.Q.ld > (1L << 28)) return TFB_ERR_SHAPE;
   if (((uintptr_t)a.P.base | (uintptr_t)a.Q.base | (uintptr_t)a.P.ld | (uintptr_t)a.Q.ld) & 15) return TFB_ERR_ARG;
+  if ((long)splits * a.nkt >= (1L << 31)) return TFB_ERR_SHAPE;
   a.splits = splits;
+  const int ntq = a.nq / Cfg::BQ;
+  if ((long)a.ntp * ntq * splits >= (1L << 31)) return TFB_ERR_SHAPE;
+  a.ntiles = a.ntp * ntq;
+  // the stagger of the first round: only where there is a second round to overlap with and no k-split
   a.slots = tfb_resident_slots(2);
+  if (!((splits == 1 || TFB_STAGGER_SPLITK) && (long)a.ntiles * splits >= 2L * a.slots)) a.slots = 0;
+  a.per = (a.ntiles & 7) == 0 ? a.ntiles >> 3 : 0;
+  a.p_fast = a.np <= a.nq || a.q_group;
+  a.nfast = a.p_fast ? a.ntp : ntq;
   // traversal blocks: the largest divisor of the smaller operand's tile count whose tiles (all of k) stay under ~1.6 MB;
   // none when the whole smaller operand is that small, or when a single tile of it is already larger
   a.gblock = 0;
   if (splits == 1 && !a.q_group && !a.k_seg) {
-    const bool p_fast = a.np <= a.nq;
-    const int nfast = p_fast ? a.ntp : a.nq / Cfg::BQ;
-    const long tile_bytes = (long)(p_fast ? Cfg::BP : Cfg::BQ) * a.nkt * 128;
+    const long tile_bytes = (long)(a.p_fast ? Cfg::BP : Cfg::BQ) * a.nkt * 128;
     const long budget = 1600 * 1024;
-    if (tile_bytes * nfast > budget && tile_bytes <= budget) {
-      for (int g = 1; g <= nfast; ++g)
-        if (nfast % g == 0 && tile_bytes * g <= budget) a.gblock = g;
+    if (tile_bytes * a.nfast > budget && tile_bytes <= budget) {
+      for (int g = 1; g <= a.nfast; ++g)
+        if (a.nfast % g == 0 && tile_bytes * g <= budget) a.gblock = g;
     }
   }
+  a.rows = (a.gblock > 0 && a.per > 0 && a.per % a.nfast == 0) ? a.per / a.nfast : 0;
+  a.blk = a.gblock * a.rows;
+  a.d_ntiles = fastdiv_make(a.ntiles);
+  a.d_per = fastdiv_make(a.per);
+  a.d_nfast = fastdiv_make(a.nfast);
+  a.d_blk = fastdiv_make(a.blk);
+  a.d_gblock = fastdiv_make(a.gblock);
+  a.d_splits = fastdiv_make(splits);
+  a.d_split8 = fastdiv_make(splits >> 3);
   dim3 grid(a.ntp * (a.nq / Cfg::BQ) * splits, groups_y, 1);
   hipLaunchKernelGGL((gemm_kernel<Cfg, PreP, PreQ, Epi>), grid, dim3(Cfg::NT), 0, stream, a, prep, preq, epi);
   TFB_LAUNCH_CHECK();
