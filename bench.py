@@ -277,9 +277,9 @@ def config_probe(which):
 
 
 def hw_probe():
-    """The two hardware probes behind the operand paths of the GEMM and attention kernels (tfb_probe_load_issue,
+    """The hardware probes behind the operand paths of the GEMM and attention kernels (tfb_probe_load_issue,
     tfb_probe_lds_mix): the cost of a 1 KB vector load to the wavefront that issues it, and what operand streams cost the
-    fragment reads of the same CU."""
+    fragment reads of the same CU; and where a workgroup of the bf16 GEMM spends its cycles (tfb_probe_gemm_phases)."""
     import torch
     from trainium_frontier_them_bones_amd import ops
     dev = torch.device("cuda:0")
@@ -293,6 +293,18 @@ def hw_probe():
     for mode, name in ((0, "readers alone"), (1, "+ global -> LDS DMA"), (2, "+ global -> VGPR -> ds_write_b128"), (3, "+ global -> VGPR only")):
         rd, ld = ops.probe_lds_mix(dev, mode)
         print("  %-36s LDS reads %6.1f B/clk/CU   streamed %5.1f B/clk/CU" % (name, rd, ld))
+    print("Phases of a workgroup of the bf16 GEMM (128 x 128 tile, two workgroups per CU; mean cycles over all workgroups):")
+    g = torch.Generator(device="cpu").manual_seed(5)
+    for what, M, N, K in (("QKV projection", 32768, 2304, 768), ("output projection", 32768, 768, 768),
+                          ("32768 x 3072 x 768", 32768, 3072, 768), ("8192^3", 8192, 8192, 8192)):
+        a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
+        b = torch.randn(N, K, generator=g).to(torch.bfloat16).to(dev)
+        for _ in range(3):
+            _, cyc = ops.probe_gemm_phases(a, b)
+        torch.cuda.synchronize(dev)
+        m = cyc.double().mean(0).tolist()
+        print("  %-20s %5d workgroups: first load issued after %5.0f, first k-tile there after %5.0f, k-loop %6.0f (%4.0f per k-tile), "
+              "epilogue %5.0f" % (what, cyc.shape[0], m[0], m[1], m[2], m[2] / (K * 2 // 128), m[3]))
 
 
 def main():

@@ -420,6 +420,11 @@ int tfb_probe_load_issue(const void* src, long region, int to_lds, int waves, in
  * CU: mode 0 nothing, 1 global -> LDS DMA, 2 global -> VGPR -> ds_write_b128, 3 global -> VGPR only (liters x 8 loads of 1 KB).
  * cycles: uint64 [CUs][16], entries 0..3 the readers, 4..7 the streaming wavefronts. */
 int tfb_probe_lds_mix(const void* src, long region, int mode, int riters, int liters, void* cycles, void* stream);
+/* Where a workgroup of the bf16 GEMM spends its time: c [M][N] = a [M][K] b[N][K]^T through the library's own kernel,
+ * traversal and launch (M, N multiples of 128, K of 64), with cycles: uint64 [(M/128)(N/128)][4] = wavefront 0's cycle
+ * counts from kernel entry to the first operand load's issue, to the first k-tile's arrival, in the k-loop, in the
+ * epilogue. */
+int tfb_probe_gemm_phases(const void* a, const void* b, void* c, long M, long N, long K, void* cycles, void* stream);
 
 #ifdef __cplusplus
 }

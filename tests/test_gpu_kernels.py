@@ -741,3 +741,16 @@ def test_hardware_probes_run_and_report_sane_rates(ops, dev):
     assert 10.0 < rd < 512.0 and 1.0 < ld < 128.0
     rd0, ld0 = ops.probe_lds_mix(dev, 0, riters=2000, liters=0)
     assert 10.0 < rd0 < 512.0 and ld0 == 0.0
+
+
+def test_gemm_phase_probe_is_the_library_kernel(ops, dev):
+    """tfb_probe_gemm_phases (diagnostic): its product is bit-identical to tfb_gemm_bf16's on the same operands (it runs
+    the same kernel and launch path with a reporting epilogue), every workgroup reports, and the phases are ordered."""
+    g = torch.Generator(device="cpu").manual_seed(11)
+    a = torch.randn(1024, 768, generator=g).to(torch.bfloat16).to(dev)
+    b = torch.randn(384, 768, generator=g).to(torch.bfloat16).to(dev)
+    c, cyc = ops.probe_gemm_phases(a, b)
+    assert torch.equal(c, ops.matmul(a, b, trans_b=True))
+    assert cyc.shape == (8 * 3, 4) and bool((cyc > 0).all())
+    assert bool((cyc[:, 0] < cyc[:, 1]).all())          # the first load is issued before the first k-tile is there
+

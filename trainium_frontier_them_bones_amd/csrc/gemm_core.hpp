@@ -312,6 +312,14 @@ struct has_tile_epilogue : std::false_type {};
 template <class T>
 struct has_tile_epilogue<T, std::void_t<decltype(T::kTileEpilogue)>> : std::true_type {};
 
+// A diagnostic epilogue with the member  unsigned long long* phase_cycles  gets the workgroup's phases written there, four
+// numbers per workgroup (wavefront 0's cycle counter): kernel entry -> first operand load issued, -> first k-tile landed
+// (the first barrier), the k-loop, the epilogue. No product epilogue has the member; the code below is compiled out for them.
+template <class T, class = void>
+struct has_phase_probe : std::false_type {};
+template <class T>
+struct has_phase_probe<T, std::void_t<decltype(std::declval<const T&>().phase_cycles)>> : std::true_type {};
+
 #ifndef TFB_STAGGER_SLEEPS
 #define TFB_STAGGER_SLEEPS 2
 #endif
@@ -345,6 +353,9 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   __shared__ __attribute__((aligned(1024))) uint8_t buf1[Cfg::STAGE_BYTES];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  constexpr bool kProbe = has_phase_probe<Epi>::value;
+  [[maybe_unused]] unsigned long long ph0 = 0, ph_issue = 0, ph_first = 0, ph_loop = 0;
+  if constexpr (kProbe) ph0 = __builtin_readcyclecounter();
   // Two workgroups share a CU. Launched together they run in lockstep: both in the k-loop (each at half the MFMA rate),
   // then both in the epilogue (MFMA idle, memory busy). The one that landed in an odd wavefront slot (HW_ID.wave_id
   // bit 0) therefore starts ~7 us late, once, in the first round of workgroups: from then on one's epilogue runs
@@ -435,6 +446,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
     dp.issue(buf, t, wave);
     dq.issue(buf + BP * 128, t, wave);
   };
+  if constexpr (kProbe) ph_issue = __builtin_readcyclecounter();
   if (nkt > 0) issue(buf0, 0);
 
   const Epi epi = epi_prepare(epi_for_group(epi_in, group));
@@ -505,6 +517,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
 
   {
     __syncthreads();
+    if constexpr (kProbe) ph_first = __builtin_readcyclecounter();
     for (int t = 0; t + 2 <= nkt; t += 2) {
       issue(buf1, t + 1);
       compute(buf0);
@@ -515,6 +528,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
     }
     if (nkt & 1) compute(buf0);
     __syncthreads();
+    if constexpr (kProbe) ph_loop = __builtin_readcyclecounter();
   }
 
   const int pw = wp * (TP * 32), qw = wq * (TQ * 32);  // wavefront's origin inside the tile
@@ -563,6 +577,15 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
         }
         __builtin_amdgcn_wave_barrier();
       }
+    }
+  }
+  if constexpr (kProbe) {
+    if (wave == 0 && lane == 0) {
+      unsigned long long* o = epi.phase_cycles + 4L * blockIdx.x;
+      o[0] = ph_issue - ph0;
+      o[1] = ph_first - ph0;
+      o[2] = ph_loop - ph_first;
+      o[3] = __builtin_readcyclecounter() - ph_loop;
     }
   }
 }

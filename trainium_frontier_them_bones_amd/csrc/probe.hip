@@ -2,10 +2,12 @@
 //   tfb_probe_load_issue  what one 1 KB vector load costs the wavefront that issues it, by destination (registers or LDS)
 //                         and by the number of wavefronts of a CU that issue at once, from an L2-resident region;
 //   tfb_probe_lds_mix     how much the fragment reads of four wavefronts slow down while four others stream operands into
-//                         the same CU by global -> LDS DMA, by global -> VGPR -> ds_write_b128, or into registers only.
+//                         the same CU by global -> LDS DMA, by global -> VGPR -> ds_write_b128, or into registers only;
+//   tfb_probe_gemm_phases where a workgroup of the bf16 GEMM (the library's own kernel and launch, with an epilogue that
+//                         also reports cycle counts) spends its time: start-up, first k-tile, k-loop, epilogue.
 // Each wavefront reports its own cycle count (s_memtime); the host turns them into cycles per instruction and bytes per
-// clock per CU. One workgroup per CU.
-#include "common.hpp"
+// clock per CU. One workgroup per CU in the first two.
+#include "gemm_core.hpp"
 
 namespace {
 
@@ -116,6 +118,11 @@ __global__ __launch_bounds__(512, 1) void lds_mix_kernel(const uint8_t* __restri
   if (acc.x == 0x12345678u && acc.y == 0x9abcdef0u) cycles[blockIdx.x * 16 + 15] = acc.z;
 }
 
+// EpiStore with the phase report switched on (see has_phase_probe)
+struct EpiStoreProbe : EpiStore {
+  unsigned long long* phase_cycles;
+};
+
 }  // namespace
 
 // cycles: uint64 [CUs][16], entry [cu][w] = cycles wavefront w spent issuing iters x 8 loads of 1 KB each (8 rows x 128 bytes
@@ -161,4 +168,21 @@ extern "C" int tfb_probe_lds_mix(const void* src, long region, int mode, int rit
   else hipLaunchKernelGGL(lds_mix_kernel<3>, dim3(cus), dim3(512), 0, s, p, rg, c, riters, liters);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
+}
+
+// c [M][N] bf16 = a [M][K] b[N][K]^T (bf16, M, N multiples of 128, K of 64) through the library's bf16 GEMM kernel, tile
+// traversal and launch path, with the phases of every workgroup written to cycles: uint64 [(M / 128) (N / 128)][4] =
+// cycles from kernel entry to the first operand load's issue, to the first k-tile's arrival, in the k-loop, in the epilogue.
+extern "C" int tfb_probe_gemm_phases(const void* a, const void* b, void* c, long M, long N, long K, void* cycles, void* stream) {
+  if (!a || !b || !c || !cycles) return TFB_ERR_ARG;
+  if (M <= 0 || N <= 0 || K <= 0 || M % 128 || N % 128 || K % 64 || M > (1L << 30) || N > (1L << 30)) return TFB_ERR_SHAPE;
+  using Cfg = GemmCfg<128, 128, 2, 2, 2, TFB_K_CONTIG, TFB_K_CONTIG>;
+  EpiStoreProbe e;
+  e.out = c;
+  e.ld = N;
+  e.f32 = 0;
+  e.accumulate = 0;
+  e.phase_cycles = (unsigned long long*)cycles;
+  return gemm_launch<Cfg>(GemmOperand{(const uint8_t*)b, K * 2}, GemmOperand{(const uint8_t*)a, K * 2}, (int)N, (int)M, K * 2, 1,
+                          LoadIdentity{}, LoadIdentity{}, e, (hipStream_t)stream);
 }

@@ -951,3 +951,17 @@ def probe_lds_mix(dev, mode, riters=20000, liters=60000, region=2 << 20):
     rd = float(cyc[live, :4].double().mean())
     ld = float(cyc[live, 4:8].double().mean())
     return 4.0 * riters * 16384.0 / rd, (4.0 * liters * 8192.0 / ld if ld > 0 else 0.0)
+
+
+def probe_gemm_phases(a, b):
+    """c = a [M,K] @ b [N,K]^T (bf16) through the library's bf16 GEMM kernel with its workgroups' phases reported: returns
+    (c, phases) with phases int64 [tiles, 4] = cycles from kernel entry to the first operand load's issue, to the first
+    k-tile's arrival, in the k-loop, in the epilogue (wavefront 0 of each 128 x 128 tile's workgroup)."""
+    M, K = a.shape
+    N = b.shape[0]
+    assert a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16 and b.shape[1] == K and a.is_contiguous() and b.is_contiguous()
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=a.device)
+    cyc = torch.zeros((M // 128) * (N // 128), 4, dtype=torch.int64, device=a.device)
+    _lib.call("tfb_probe_gemm_phases", _p(a), _p(b), _p(c), M, N, K, _p(cyc), _stream())
+    return c, cyc
+
