@@ -67,6 +67,7 @@ struct GemmArgs {
   int ntp;      // tiles along p
   int slots;    // workgroups resident at once (2 per CU): the first round of the launch, when it is to be staggered
                 //   (see the kernel; 0: no stagger)
+  int sleeps;   // length of that stagger in s_sleep(127) units
   // Grouped (ragged) launches, both optional:
   const int* q_group;    // group id of each q tile (-1: the tile is beyond the ragged extent, the workgroup exits);
   long p_group_stride;   //   the P operand of group g starts p_group_stride bytes * g further (per-expert weights)
@@ -323,6 +324,9 @@ struct has_phase_probe<T, std::void_t<decltype(std::declval<const T&>().phase_cy
 #ifndef TFB_STAGGER_SLEEPS
 #define TFB_STAGGER_SLEEPS 2
 #endif
+#ifndef TFB_STAGGER_SHORT_ROUNDS
+#define TFB_STAGGER_SHORT_ROUNDS 4
+#endif
 #ifndef TFB_STAGGER_SPLITK
 #define TFB_STAGGER_SPLITK 0
 #endif
@@ -367,10 +371,11 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   asm volatile("" ::"s"(a.P.base), "s"(a.P.ld), "s"(a.Q.base), "s"(a.Q.ld), "s"(a.nkt), "s"(a.splits), "s"(a.gblock),
                "s"(a.slots), "s"(a.q_group), "s"(a.p_group_stride), "s"(a.k_seg), "s"(a.ntiles), "s"(a.per), "s"(a.nfast),
                "s"(a.p_fast), "s"(a.rows), "s"(a.blk), "s"(a.d_per.m), "s"(a.d_per.sh), "s"(a.d_nfast.m), "s"(a.d_nfast.sh),
-               "s"(a.d_blk.m), "s"(a.d_blk.sh), "s"(a.d_gblock.m), "s"(a.d_gblock.sh), "s"(a.d_splits.m), "s"(a.d_splits.sh));
+               "s"(a.d_blk.m), "s"(a.d_blk.sh), "s"(a.d_gblock.m), "s"(a.d_gblock.sh), "s"(a.d_splits.m), "s"(a.d_splits.sh),
+               "s"(a.sleeps));
   if (Cfg::OCC == 2 && kSleeps > 0 && (int)blockIdx.x < a.slots) {
     if (__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 4) & 1)  // getreg(size 4, offset 0, HW_REG_HW_ID): wave_id
-      for (int i = 0; i < kSleeps; ++i) __builtin_amdgcn_s_sleep(127);  // 127 x 64 clocks each
+      for (int i = 0; i < a.sleeps; ++i) __builtin_amdgcn_s_sleep(127);  // 127 x 64 clocks each
   }
   const int wp = wave % Cfg::WP, wq = wave / Cfg::WP;
   const int lr = lane & 31, lh = lane >> 5;
@@ -627,6 +632,9 @@ static int gemm_launch_args(GemmArgs a, int groups_y, int splits, PreP prep, Pre
   // the stagger of the first round: only where there is a second round to overlap with and no k-split
   a.slots = tfb_resident_slots(2);
   if (!((splits == 1 || TFB_STAGGER_SPLITK) && (long)a.ntiles * splits >= 2L * a.slots)) a.slots = 0;
+  // a launch of few rounds has less to gain from the offset and pays the same for it (measured on the 1536-tile GEMMs of
+  // the step, three rounds: 0.730 / 0.755 ms per step with one / two units; on the 4608- and 6144-tile ones two is better)
+  a.sleeps = a.slots > 0 && (long)a.ntiles * splits <= TFB_STAGGER_SHORT_ROUNDS * (long)a.slots ? 1 : stagger_sleeps<Epi>::value;
   a.per = (a.ntiles & 7) == 0 ? a.ntiles >> 3 : 0;
   a.p_fast = a.np <= a.nq || a.q_group;
   a.nfast = a.p_fast ? a.ntp : ntq;
