@@ -385,9 +385,22 @@ int tfb_moe_route_bwd_aux(const void* dgate, const void* p, const void* idx, con
 /* The router's auxiliary loss terms: terms fp32 [2 + E] = (lb = E sum_e f_e P_e, z = mean_n logsumexp(logits_n)^2, f_e),
  * f_e = cnt_e / (N topk) the share of the assignments that chose e (cnt: the slot tables' counts; no gradient), P_e the
  * mean router probability; lse fp32 [N] is kept for the backward; scratch fp32 [64 * 17].
- * Replaces moe_aux_terms (round2/source/train.py:10779-10793); its per-sequence variant (R2_MOE_AUX_SEQ) is not built. */
+ * Replaces moe_aux_terms (round2/source/train.py:10779-10788); its per-sequence term (R2_MOE_AUX_SEQ, 10789-10792) is
+ * tfb_moe_aux_seq_fwd. */
 int tfb_moe_aux_fwd(const void* p, const void* logits, const void* cnt, void* terms, void* lse, void* scratch, long N, int E,
                     int topk, void* stream);
+/* The per-sequence balance term of moe_aux_terms (round2/source/train.py:10789-10792): term fp32 [1] = the mean over the
+ * N / T sequences of E sum_e fs[b][e] ps[b][e]; fs fp32 [N / T][E] = each sequence's share of its T topk assignments per
+ * expert (from idx int32 [N][topk], every selection counted whether a capacity later drops its row; no gradient; kept for
+ * the backward), ps the sequence's mean router probability. scratch fp32 [N / T]. N % T == 0. */
+int tfb_moe_aux_seq_fwd(const void* p, const void* idx, void* fs, void* term, void* scratch, long N, long T, int E, int topk,
+                        void* stream);
+/* tfb_moe_route_bwd_aux with that term as well: the weighted sum alpha lb + beta z + gamma seq received the gradient *gaux;
+ * fs as tfb_moe_aux_seq_fwd left it. */
+int tfb_moe_route_bwd_aux_seq(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot,
+                              const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate,
+                              void* scratch, const void* terms, const void* lse, const void* gaux, float alpha, float beta,
+                              const void* fs, float gamma, long T, long N, int d, int E, int topk, void* stream);
 
 /* rows_out fp32 [E][16] = rows_in with the backward columns filled from each expert's amax over its rows of dys
  * (backward_scales per expert, round2/source/kernels/nki_mlp_fused8.py:803-813). amax_scratch: uint32 [E]. */

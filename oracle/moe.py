@@ -11,7 +11,8 @@ row (R2:10735-10737). Gradients come from torch.autograd over these expressions 
 
 Pinned by (tests/test_oracle_moe.py): torch.topk for the selections, gates summing to one, a brute-force per-token loop
 with the bf16 expert MLP, permutation equivariance over tokens, and the reference's capacity layout computed with a cumsum
-giving the same output when nothing is dropped; the capacity's keep rule by a plain loop over each sequence's tokens, and the
+giving the same output when nothing is dropped; the auxiliary terms by their closed forms (uniform router, one-hot router),
+fp64 autograd and, for the per-sequence term, its reduction to the global term on one sequence and a token loop; the capacity's keep rule by a plain loop over each sequence's tokens, and the
 reference's [E][b][cap] buffer with its zero row for skipped assignments giving the same output bit for bit when it drops.
 """
 import torch
@@ -128,14 +129,20 @@ def moe_forward(h, router, w_fc, w_proj, topk, bias=None, fp8=True, e4m3_limit=2
     return out.reshape(h.shape), {"p": p, "idx": idx, "gate": gate, "slot": slot, "tok": tok, "seg": seg}
 
 
-def aux_terms(p, logits, idx, topk):
+def aux_terms(p, logits, idx, topk, seq_len=None):
     """(lb, z, f): the Switch load-balance term E sum_e f_e P_e (f_e the share of the k N assignments that chose e, no
     gradient; P_e the mean router probability) and the router z term mean(logsumexp(logits)^2)
-    (round2/source/train.py:10779-10788 moe_aux_terms without its per-sequence variant)."""
+    (round2/source/train.py:10779-10788 moe_aux_terms). With seq_len (the tokens are whole sequences of that length) a
+    fourth value: the per-sequence balance term, the mean over sequences of E sum_e fs_e ps_e with the shares and mean
+    probabilities taken inside each sequence (10789-10792, the reference's R2_MOE_AUX_SEQ)."""
     N, E = p.shape
     mall = torch.zeros(N, E, dtype=p.dtype)
     mall.scatter_add_(1, idx.long(), torch.ones(idx.shape, dtype=p.dtype))
     f = mall.mean(0) / topk
     lb = E * (f * p.mean(0)).sum()
     z = torch.logsumexp(logits, dim=-1).square().mean()
-    return lb, z, f
+    if seq_len is None:
+        return lb, z, f
+    fs = mall.reshape(N // seq_len, seq_len, E).mean(1) / topk
+    ps = p.reshape(N // seq_len, seq_len, E).mean(1)
+    return lb, z, f, (E * (fs * ps).sum(-1)).mean()

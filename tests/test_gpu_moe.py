@@ -186,6 +186,42 @@ def test_moe_auxiliary_router_terms(dev):
     assert float(wfd.grad.abs().max()) == 0.0                           # no gradient reaches the experts through aux
 
 
+@pytest.mark.parametrize("topk", [1, 2])
+def test_moe_per_sequence_balance_term(dev, topk):
+    """The per-sequence balance term of moe_aux_terms (round2/source/train.py:10789-10792): the kernel's term and the
+    sequences' load shares against the oracle ON THE KERNEL'S OWN selections (shares bit-exact: they are counts over a
+    power-of-two length), and through the autograd node: the weighted sum alpha lb + beta z + gamma seq and its gradient to
+    the router and the input, with the layer's own output gradient zero."""
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import autograd as A, ops
+    B, T, d, Fd, E = 8, 256, 256, 512, 8
+    h, router, wf, wp, bias = _layer(7, B * T, d, Fd, E, 1.5)
+    hd, rd = h.to(dev).view(B, T, d).requires_grad_(True), router.to(dev).requires_grad_(True)
+    wfd, wpd = wf.to(dev).requires_grad_(True), wp.to(dev).requires_grad_(True)
+    p, idx, gate, logits = ops.moe_route(hd.detach().reshape(-1, d), rd.detach().float().contiguous(), topk, bias.to(dev), want_logits=True)
+    term, fs = ops.moe_aux_seq_fwd(p, idx, T, topk)
+    *_, seq_o = O.aux_terms(p.cpu().double(), logits.cpu().double(), idx.cpu(), topk, seq_len=T)
+    mall = torch.zeros(B * T, E, dtype=torch.float64).scatter_add_(1, idx.cpu().long(), torch.ones(B * T, topk, dtype=torch.float64))
+    assert torch.equal(fs.cpu().double(), mall.view(B, T, E).mean(1) / topk)
+    assert abs(term.item() - seq_o.item()) < 1e-5 * abs(seq_o.item())
+    st = A.Moe8State()
+    st.refresh(wfd, wpd)
+    alpha, beta, gamma = 0.01, 0.001, 0.02
+    out, aux, terms = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, st, topk, bias.to(dev), (alpha, beta, gamma))
+    out2, aux2, _ = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, st, topk, bias.to(dev), (alpha, beta))
+    assert torch.equal(out, out2)
+    assert abs((aux - aux2).item() - gamma * term.item()) < 1e-6 * abs(aux.item())
+    (aux * 2.0).backward()
+    ho, ro = h.clone().float().requires_grad_(True), router.clone().float().requires_grad_(True)
+    po, _, _, lo = O.route(ho, ro, topk, bias)
+    lb, z, f, seq = O.aux_terms(po, lo, idx.cpu(), topk, seq_len=T)      # the kernel's selections: a near-tie cannot differ
+    (2.0 * (alpha * lb + beta * z + gamma * seq)).backward()
+    assert rel_l2(rd.grad, ro.grad) < 1e-2
+    assert rel_l2(hd.grad.view(-1, d), ho.grad) < 2e-2                  # one bf16 rounding of dh
+    with pytest.raises(ValueError):
+        ops.moe_aux_seq_fwd(p, idx, 384, topk)                          # 2048 tokens are not whole sequences of 384
+
+
 @pytest.mark.parametrize("skew", [0.0, 2.0])
 def test_moe_config5_full_size_backward(dev, skew):
     """Configuration 5 at full size, forward AND backward (16384 tokens, d 1024, 8 experts top-2, FFN 2816; balanced and

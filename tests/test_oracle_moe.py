@@ -173,3 +173,45 @@ def test_aux_terms_closed_forms_and_gradient():
     dp = 0.3 * E * f / N
     want = pd * (dp - (pd * dp).sum(-1, keepdim=True)) + 0.7 * 2.0 / N * torch.logsumexp(logits.detach(), -1, keepdim=True) * pd
     assert torch.allclose(logits.grad, want, atol=1e-12)
+
+
+def test_per_sequence_balance_term_special_cases_and_a_token_loop():
+    """The per-sequence balance term (round2/source/train.py:10789-10792): with ONE sequence it is the global term lb;
+    with identical sequences it equals each sequence's own lb; a sequence whose tokens all go, with all probability, to
+    one expert contributes E, a uniform one 1, so two such sequences give (E + 1) / 2; and on random inputs it matches a
+    plain loop over sequences, tokens and choices."""
+    from oracle import moe as O
+    g = torch.Generator().manual_seed(4)
+    T, E = 32, 8
+    logits = torch.randn(T, E, generator=g, dtype=torch.float64)
+    p = torch.softmax(logits, -1)
+    idx = torch.topk(p, 2, dim=-1).indices
+    lb, z, f, seq = O.aux_terms(p, logits, idx, 2, seq_len=T)
+    assert abs(seq.item() - lb.item()) < 1e-12                                   # one sequence: the global term
+    lb3, _, _, seq3 = O.aux_terms(p.repeat(3, 1), logits.repeat(3, 1), idx.repeat(3, 1), 2, seq_len=T)
+    assert abs(seq3.item() - lb.item()) < 1e-12 and abs(lb3.item() - lb.item()) < 1e-12
+    hot = torch.full((T, E), -60.0, dtype=torch.float64)
+    hot[:, 5] = 60.0
+    flat = torch.zeros(T, E, dtype=torch.float64)
+    lg = torch.cat([hot, flat])
+    ix = torch.cat([torch.full((T, 1), 5), (torch.arange(T) % E).unsqueeze(1)])
+    _, _, _, seq2 = O.aux_terms(torch.softmax(lg, -1), lg, ix, 1, seq_len=T)
+    assert abs(seq2.item() - (E + 1) / 2) < 1e-9
+    B = 5
+    logits = torch.randn(B * T, E, generator=g, dtype=torch.float64) * 2
+    p = torch.softmax(logits, -1)
+    idx = torch.topk(p, 2, dim=-1).indices
+    want = 0.0
+    for b in range(B):
+        cnt = [0] * E
+        psum = [0.0] * E
+        for t in range(T):
+            n = b * T + t
+            for k in range(2):
+                cnt[int(idx[n, k])] += 1
+            for e in range(E):
+                psum[e] += float(p[n, e])
+        want += E * sum((cnt[e] / (2 * T)) * (psum[e] / T) for e in range(E))
+    _, _, _, seq = O.aux_terms(p, logits, idx, 2, seq_len=T)
+    assert abs(seq.item() - want / B) < 1e-12
+

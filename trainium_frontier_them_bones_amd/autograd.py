@@ -617,7 +617,9 @@ class MoeMlp8Fn(torch.autograd.Function):
     def forward(ctx, h, router, w_fc, w_proj, state, topk, router_bias, aux_weights=None, capacity=None):
         """aux_weights = (alpha, beta): also returns (aux, stats) with aux = alpha lb + beta z, the router's weighted
         load-balance and z terms (round2/source/train.py:10779 moe_aux_terms; differentiable, its gradient joins the
-        router's in the backward), and stats fp32 [2 + E] = (lb, z, the experts' load shares f_e)."""
+        router's in the backward), and stats fp32 [2 + E] = (lb, z, the experts' load shares f_e).
+        aux_weights = (alpha, beta, gamma) adds gamma times the per-sequence balance term (the reference's R2_MOE_AUX_SEQ,
+        10789-10792), the sequences being the rows of h [b, t, d]."""
         h2 = h.reshape(-1, h.shape[-1]).contiguous()
         E, F, d = w_fc.shape
         wr = router.detach().float().contiguous()
@@ -633,8 +635,17 @@ class MoeMlp8Fn(torch.autograd.Function):
             ctx.save_for_backward(h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj)
             return out.view(h.shape)
         terms, lse = ops.moe_aux_fwd(p, logits, tab, topk)
-        ctx.save_for_backward(h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj, terms, lse)
         aux = float(aux_weights[0]) * terms[0] + float(aux_weights[1]) * terms[1]
+        if len(aux_weights) > 2 and float(aux_weights[2]) != 0.0:
+            if h.dim() < 3:
+                raise ValueError("MoeMlp8Fn: the per-sequence balance term needs h [b, t, d]")
+            seq_term, fs = ops.moe_aux_seq_fwd(p, idx, h.shape[-2], topk)
+            aux = aux + float(aux_weights[2]) * seq_term[0]
+            ctx.seq_len = h.shape[-2]
+            ctx.save_for_backward(h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj, terms, lse, fs)
+        else:
+            ctx.seq_len = None
+            ctx.save_for_backward(h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj, terms, lse)
         ctx.mark_non_differentiable(terms)
         return out.view(h.shape), aux, terms
 
@@ -644,9 +655,11 @@ class MoeMlp8Fn(torch.autograd.Function):
             h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj = ctx.saved_tensors
             aux = None
         else:
-            h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj, terms, lse = ctx.saved_tensors
+            h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj, terms, lse = ctx.saved_tensors[:13]
             ga = torch.zeros(1, dtype=torch.float32, device=h2.device) if gaux is None else gaux.reshape(1).float().contiguous()
             aux = (terms, lse, ga, ctx.aux_weights[0], ctx.aux_weights[1])
+            if ctx.seq_len is not None:
+                aux = aux + (ctx.saved_tensors[13], ctx.aux_weights[2], ctx.seq_len)
         tab, st = ctx.tab, ctx.state
         E = w_fc.shape[0]
         if gout is None:

@@ -325,12 +325,15 @@ __global__ __launch_bounds__(256) void moe_combine_bwd_kernel(const bf16_t* __re
 // dlogits[n][e] = p_e (dp_e - sum_j p_j dp_j), dp from the gate gradients through the renormalisation.
 // With the auxiliary router terms (terms != NULL: [0] lb, [1] z, [2..] f_e as left by moe_aux_finish_kernel; lse[n]; g =
 // *gaux, the gradient arriving at the weighted sum alpha lb + beta z): dp_e += g alpha (E / N) f_e (f carries no
-// gradient) and, after the softmax Jacobian, dlogits_e += g beta (2 / N) lse_n p_e.
+// gradient) and, after the softmax Jacobian, dlogits_e += g beta (2 / N) lse_n p_e. With the per-sequence balance term
+// (fs != NULL: fs[b][e] the load shares of sequence b = n / T as left by moe_aux_seq_kernel, weight gamma):
+// dp_e += g gamma (E / N) fs[b][e] (the term is a mean over the N / T sequences of E sum_e fs ps, ps a mean over T tokens).
 __global__ __launch_bounds__(256) void moe_dlogits_kernel(const float* __restrict__ dgate, const float* __restrict__ p,
                                                          const int* __restrict__ idx, float* __restrict__ dlogits, long N,
                                                          int E, int topk, const float* __restrict__ terms,
                                                          const float* __restrict__ lse, const float* __restrict__ gaux,
-                                                         float alpha, float beta) {
+                                                         float alpha, float beta, const float* __restrict__ fs, float gamma,
+                                                         long T) {
   long n = (long)blockIdx.x * 256 + threadIdx.x;
   if (n >= N) return;
   float dp[MAXE];
@@ -353,6 +356,11 @@ __global__ __launch_bounds__(256) void moe_dlogits_kernel(const float* __restric
     const float ca = g * alpha * (float)E / (float)N;
     for (int e = 0; e < E; ++e) dp[e] += ca * terms[2 + e];
     zc = g * beta * 2.0f / (float)N * lse[n];
+    if (fs) {
+      const float cs = g * gamma * (float)E / (float)N;
+      const float* fb = fs + (n / T) * E;
+      for (int e = 0; e < E; ++e) dp[e] += cs * fb[e];
+    }
   }
   float dot = 0.f;
   for (int e = 0; e < E; ++e) dot += p[n * E + e] * dp[e];
@@ -409,6 +417,58 @@ __global__ void moe_aux_finish_kernel(const float* __restrict__ part, int nparts
     }
     terms[0] = (float)E * lb;
     terms[1] = tot[MAXE] / (float)N;
+  }
+}
+
+// The per-sequence form of the balance term (round2/source/train.py:10789-10792): one workgroup per sequence b of T tokens.
+// fs[b][e] = (assignments of the sequence's tokens to e) / (T topk), from ALL selections (idx), dropped or not;
+// part[b] = E sum_e fs[b][e] ps[b][e] with ps[b][e] the mean of p over the sequence's tokens.
+__global__ __launch_bounds__(256) void moe_aux_seq_kernel(const float* __restrict__ p, const int* __restrict__ idx,
+                                                         float* __restrict__ fs, float* __restrict__ part, long T, int E,
+                                                         int topk) {
+  __shared__ float red[4][2 * MAXE];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long n0 = (long)blockIdx.x * T;
+  float ps[MAXE], cn[MAXE];
+#pragma unroll
+  for (int e = 0; e < MAXE; ++e) ps[e] = cn[e] = 0.f;
+  for (long i = threadIdx.x; i < T; i += 256) {
+    const long n = n0 + i;
+    const int i1 = idx[n * topk], i2 = topk == 2 ? idx[n * 2 + 1] : -1;
+#pragma unroll
+    for (int e = 0; e < MAXE; ++e)
+      if (e < E) {
+        ps[e] += p[n * E + e];
+        cn[e] += (float)((e == i1) + (e == i2));   // whole numbers below 2^24: exact whatever the order
+      }
+  }
+#pragma unroll
+  for (int e = 0; e < MAXE; ++e) {
+    const float a = wave_sum(ps[e]), c = wave_sum(cn[e]);
+    if (lane == 0) {
+      red[wave][e] = a;
+      red[wave][MAXE + e] = c;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float acc = 0.f;
+    for (int e = 0; e < E; ++e) {
+      const float psum = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
+      const float cnt = (red[0][MAXE + e] + red[1][MAXE + e]) + (red[2][MAXE + e] + red[3][MAXE + e]);
+      const float f = cnt / ((float)T * (float)topk);
+      fs[(long)blockIdx.x * E + e] = f;
+      acc += f * (psum / (float)T);
+    }
+    part[blockIdx.x] = (float)E * acc;
+  }
+}
+// term = the mean of part over the nseq sequences, summed in sequence order
+__global__ void moe_aux_seq_finish_kernel(const float* __restrict__ part, long nseq, float* __restrict__ term) {
+  if (threadIdx.x == 0) {
+    float s = 0.f;
+    for (long b = 0; b < nseq; ++b) s += part[b];
+    *term = s / (float)nseq;
   }
 }
 
@@ -713,13 +773,13 @@ extern "C" int tfb_moe_combine_bwd(const void* dout, const void* ys, const void*
 static int moe_route_bwd_impl(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot,
                               const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate,
                               void* scratch, long N, int d, int E, int topk, const void* terms, const void* lse,
-                              const void* gaux, float alpha, float beta, void* stream) {
+                              const void* gaux, float alpha, float beta, const void* fs, float gamma, long T, void* stream) {
   if (!dgate || !p || !idx || !dxs || !slot || !h || !wr || !dlogits || !dh || !dwr || !scratch) return TFB_ERR_ARG;
   if (N <= 0 || d <= 0 || d % 64 || E < 2 || E > MAXE || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(moe_dlogits_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, (const float*)dgate,
                      (const float*)p, (const int*)idx, (float*)dlogits, N, E, topk, (const float*)terms, (const float*)lse,
-                     (const float*)gaux, alpha, beta);
+                     (const float*)gaux, alpha, beta, (const float*)fs, gamma, T > 0 ? T : N);
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(moe_dispatch_bwd_kernel, dim3(nblocks(N * (d / 8))), dim3(256), 0, s, (const bf16_t*)dxs, (const int*)slot,
                      (const float*)dlogits, (const float*)wr, (bf16_t*)dh, N, d, E, topk);
@@ -739,7 +799,7 @@ extern "C" int tfb_moe_route_bwd(const void* dgate, const void* p, const void* i
                                  const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate,
                                  void* scratch, long N, int d, int E, int topk, void* stream) {
   return moe_route_bwd_impl(dgate, p, idx, dxs, slot, h, wr, dlogits, dh, dwr, dwr_accumulate, scratch, N, d, E, topk, nullptr,
-                            nullptr, nullptr, 0.f, 0.f, stream);
+                            nullptr, nullptr, 0.f, 0.f, nullptr, 0.f, 0, stream);
 }
 // tfb_moe_route_bwd with the gradient of the auxiliary router terms folded into dlogits: the weighted sum
 // alpha lb + beta z of tfb_moe_aux_fwd received the gradient *gaux (device fp32 scalar); terms and lse as that call left them.
@@ -749,13 +809,25 @@ extern "C" int tfb_moe_route_bwd_aux(const void* dgate, const void* p, const voi
                                      float beta, long N, int d, int E, int topk, void* stream) {
   if (!terms || !lse || !gaux) return TFB_ERR_ARG;
   return moe_route_bwd_impl(dgate, p, idx, dxs, slot, h, wr, dlogits, dh, dwr, dwr_accumulate, scratch, N, d, E, topk, terms,
-                            lse, gaux, alpha, beta, stream);
+                            lse, gaux, alpha, beta, nullptr, 0.f, 0, stream);
+}
+// tfb_moe_route_bwd_aux with the per-sequence balance term as well: the weighted sum alpha lb + beta z + gamma seq received
+// the gradient *gaux; fs fp32 [N / T][E] as tfb_moe_aux_seq_fwd left it, T the sequence length (N % T == 0).
+extern "C" int tfb_moe_route_bwd_aux_seq(const void* dgate, const void* p, const void* idx, const void* dxs, const void* slot,
+                                         const void* h, const void* wr, void* dlogits, void* dh, void* dwr, int dwr_accumulate,
+                                         void* scratch, const void* terms, const void* lse, const void* gaux, float alpha,
+                                         float beta, const void* fs, float gamma, long T, long N, int d, int E, int topk,
+                                         void* stream) {
+  if (!terms || !lse || !gaux || !fs) return TFB_ERR_ARG;
+  if (T <= 0 || N % T) return TFB_ERR_SHAPE;
+  return moe_route_bwd_impl(dgate, p, idx, dxs, slot, h, wr, dlogits, dh, dwr, dwr_accumulate, scratch, N, d, E, topk, terms,
+                            lse, gaux, alpha, beta, fs, gamma, T, stream);
 }
 
 // The router's auxiliary terms: terms fp32 [2 + E] = (lb = E sum_e f_e P_e, z = mean_n logsumexp(logits_n)^2, f_e) with
 // f_e = cnt_e / (N topk) the share of the assignments that chose e (from the slot tables' counts) and P_e the mean
 // router probability; lse fp32 [N] (kept for the backward); scratch: fp32 [64][17].
-// Replaces moe_aux_terms (round2/source/train.py:10779-10793; its per-sequence variant is not built).
+// Replaces moe_aux_terms (round2/source/train.py:10779-10788; its per-sequence term is tfb_moe_aux_seq_fwd).
 extern "C" int tfb_moe_aux_fwd(const void* p, const void* logits, const void* cnt, void* terms, void* lse, void* scratch, long N,
                                int E, int topk, void* stream) {
   if (!p || !logits || !cnt || !terms || !lse || !scratch) return TFB_ERR_ARG;
@@ -767,6 +839,25 @@ extern "C" int tfb_moe_aux_fwd(const void* p, const void* logits, const void* cn
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(moe_aux_finish_kernel, dim3(1), dim3(64), 0, s, (const float*)scratch, nb, (const int*)cnt, (float*)terms, N,
                      E, topk);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// The per-sequence balance term of moe_aux_terms (round2/source/train.py:10789-10792, the reference's R2_MOE_AUX_SEQ):
+// term fp32 [1] = mean over the N / T sequences of E sum_e fs[b][e] ps[b][e], fs fp32 [N / T][E] the sequences' load shares
+// (kept for the backward; no gradient), ps the sequences' mean router probabilities. idx int32 [N][topk] the selections
+// (all of them: a capacity drops rows, not assignments, from this count); scratch fp32 [N / T].
+extern "C" int tfb_moe_aux_seq_fwd(const void* p, const void* idx, void* fs, void* term, void* scratch, long N, long T, int E,
+                                   int topk, void* stream) {
+  if (!p || !idx || !fs || !term || !scratch) return TFB_ERR_ARG;
+  if (N <= 0 || T <= 0 || N % T || T >= (1L << 23) || E < 2 || E > MAXE || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const long nseq = N / T;
+  if (nseq > (1L << 30)) return TFB_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_aux_seq_kernel, dim3((unsigned)nseq), dim3(256), 0, s, (const float*)p, (const int*)idx, (float*)fs,
+                     (float*)scratch, T, E, topk);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_aux_seq_finish_kernel, dim3(1), dim3(64), 0, s, (const float*)scratch, nseq, (float*)term);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

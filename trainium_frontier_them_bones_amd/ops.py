@@ -851,7 +851,8 @@ def moe_combine_bwd(dout, ys, tab, gate):
 
 def moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, dwr=None, accumulate=False, aux=None):
     """(dh bf16 [N,d], dwr fp32 [E,d], dlogits fp32 [N,E]). aux = (terms, lse, gaux, alpha, beta): the gradient gaux
-    (1-element fp32 device tensor) of the weighted auxiliary terms alpha lb + beta z of moe_aux_fwd is folded into dlogits."""
+    (1-element fp32 device tensor) of the weighted auxiliary terms alpha lb + beta z of moe_aux_fwd is folded into dlogits;
+    aux = (terms, lse, gaux, alpha, beta, fs, gamma, seq_len) adds the per-sequence term gamma seq of moe_aux_seq_fwd."""
     N, d = h2.shape
     E = wr.shape[0]
     dlogits = torch.empty(N, E, dtype=torch.float32, device=h2.device)
@@ -863,6 +864,14 @@ def moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, dwr=None, accumulate=False, a
     if aux is None:
         _lib.call("tfb_moe_route_bwd", _p(dgate), _p(p), _p(idx), _p(dxs), _p(tab["slot"]), _p(h2), _p(wr), _p(dlogits), _p(dh),
                   _p(dwr), int(accumulate), _p(scr), N, d, E, idx.shape[1], _stream())
+    elif len(aux) == 8:
+        terms, lse, gaux, alpha, beta, fs, gamma, seq_len = aux
+        _chk(terms, torch.float32), _chk(lse, torch.float32), _chk(gaux, torch.float32), _chk(fs, torch.float32)
+        if N % int(seq_len) or tuple(fs.shape) != (N // int(seq_len), E):
+            raise ValueError("moe_route_bwd: fs must be [N / seq_len, E]")
+        _lib.call("tfb_moe_route_bwd_aux_seq", _p(dgate), _p(p), _p(idx), _p(dxs), _p(tab["slot"]), _p(h2), _p(wr), _p(dlogits),
+                  _p(dh), _p(dwr), int(accumulate), _p(scr), _p(terms), _p(lse), _p(gaux), float(alpha), float(beta), _p(fs),
+                  float(gamma), int(seq_len), N, d, E, idx.shape[1], _stream())
     else:
         terms, lse, gaux, alpha, beta = aux
         _chk(terms, torch.float32), _chk(lse, torch.float32), _chk(gaux, torch.float32)
@@ -882,6 +891,21 @@ def moe_aux_fwd(p, logits, tab, topk):
     scr = torch.empty(64 * 17, dtype=torch.float32, device=p.device)
     _lib.call("tfb_moe_aux_fwd", _p(p), _p(logits), _p(tab.get("cnt_all", tab["cnt"])), _p(terms), _p(lse), _p(scr), N, E, topk, _stream())
     return terms, lse
+
+
+def moe_aux_seq_fwd(p, idx, seq_len, topk):
+    """(term fp32 [1], fs fp32 [N / seq_len, E]): the per-sequence balance term of moe_aux_terms
+    (round2/source/train.py:10789-10792) = mean over sequences of E sum_e fs ps, and the sequences' load shares."""
+    _chk(p, torch.float32), _chk(idx, torch.int32)
+    N, E = p.shape
+    T = int(seq_len)
+    if T <= 0 or N % T:
+        raise ValueError("moe_aux_seq_fwd: %d tokens are not whole sequences of %d" % (N, T))
+    fs = torch.empty(N // T, E, dtype=torch.float32, device=p.device)
+    term = torch.empty(1, dtype=torch.float32, device=p.device)
+    scr = torch.empty(N // T, dtype=torch.float32, device=p.device)
+    _lib.call("tfb_moe_aux_seq_fwd", _p(p), _p(idx), _p(fs), _p(term), _p(scr), N, T, E, topk, _stream())
+    return term, fs
 
 
 # ------------------------------------------------------------------------------------------ Muon Newton-Schulz
