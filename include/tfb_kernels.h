@@ -343,8 +343,8 @@ int tfb_moe_tables(const void* idx, void* cnt, void* seg, void* tile_expert, voi
 int tfb_moe_tables_cap(const void* idx, void* cnt, void* cnt_all, void* seg, void* tile_expert, void* slot, void* tok, void* ksel,
                        void* scratch, long N, long T, int cap, int E, int topk, long rmax, void* stream);
 
-/* xs bf16 [rmax][d] = h[tok] (zero padding rows) and xs8 = e4m3(xs * scale) (scale_ptr device fp32 or scale_imm).
- * Replaces MoeDispatch2.forward (round2/source/train.py:10652-10660). */
+/* xs bf16 [rmax][d] = h[tok] (zero padding rows) and xs8 = e4m3(xs * scale) (scale_ptr device fp32 or scale_imm; xs8 may
+ * be NULL: bf16 experts take no fp8 copy). Replaces MoeDispatch2.forward (round2/source/train.py:10652-10660). */
 int tfb_moe_gather(const void* h, const void* tok, const void* scale_ptr, float scale_imm, void* xs, void* xs8, long rmax, int d,
                    void* stream);
 
@@ -360,6 +360,17 @@ int tfb_moe_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void*
  * Replaces the per-expert weight_grads (round2/source/kernels/nki_mlp_fused8.py:706-711). */
 int tfb_moe_dw(const void* dpre, const void* xs, const void* dys, const void* r, const void* seg, void* dw_fc, void* dw_proj,
                int E, int d, int F, int out_f32, int accumulate, void* stream);
+/* The routed experts in bf16 (every expert on this GPU) on the grouped buffers: each expert applies
+ * F.linear(relu(F.linear(x, w_fc[e])).square(), w_proj[e]) to its rows with the bf16 roundings of those four operations.
+ * xs bf16 [rmax][d], w_fc bf16 [E][F][d], w_proj bf16 [E][d][F], tile_expert int32 [rmax/128] -> ys bf16 [rmax][d],
+ * r bf16 [rmax][F] = relu(pre), h bf16 [rmax][F] = r^2 (both kept for the backward). d, F multiples of 128.
+ * Replaces moe_experts_local / the kit's expression of moe_expert_mlp (round2/source/train.py:10716-10727, 10711). */
+int tfb_moe_mlp_fwd(const void* xs, const void* w_fc, const void* w_proj, const void* tile_expert, void* ys, void* r, void* h,
+                    long rmax, int d, int F, void* stream);
+/* Its backward: dpre bf16 [rmax][F] = bf16(bf16(dys w_proj[e]) 2 r), dxs bf16 [rmax][d] = dpre w_fc[e] (autograd through the
+ * same expression); the weight gradients are tfb_moe_dw(dpre, xs, dys, r, ...). */
+int tfb_moe_mlp_bwd(const void* dys, const void* r, const void* w_fc, const void* w_proj, const void* tile_expert, void* dxs,
+                    void* dpre, long rmax, int d, int F, void* stream);
 
 /* out bf16 [N][d] = sum_k bf16(gate_k) ys[slot_k] (the eager bf16 expression's roundings).
  * Replaces MoeCombine2.forward + the gated sum (round2/source/train.py:10672-10676, 10990-10992). */

@@ -97,14 +97,22 @@ class _ExpertMlp8(torch.autograd.Function):
 
 
 def moe_forward(h, router, w_fc, w_proj, topk, bias=None, fp8=True, e4m3_limit=240.0, x_scale=4.0, dys_amax=None,
-                capacity=None):
+                capacity=None, idx=None):
     """h [.., d] bf16; router [E, d]; w_fc [E, F, d]; w_proj [E, d, F]. Differentiable (autograd) in h, router, weights.
+    fp8 False: the experts in bf16, the kit's expression per expert (round2/source/train.py:10716 moe_experts_local).
     dys_amax (optional, fp32 [E]): per-expert amax of the expert outputs' gradients to take the backward scales from,
-    for a call that holds only some of the layer's tokens."""
+    for a call that holds only some of the layer's tokens. idx (optional, [N, k]): selections to use instead of the
+    oracle's own (a checker passes the kernel's, so that a near-tie cannot route a token differently); the gates are
+    still this function's, from its own probabilities at those experts."""
     d = h.shape[-1]
     h2 = h.reshape(-1, d)
     E = w_fc.shape[0]
-    p, idx, gate, _ = route(h2, router, topk, bias)
+    p, idx_own, gate, _ = route(h2, router, topk, bias)
+    if idx is None:
+        idx = idx_own
+    else:
+        v = p.gather(1, idx)
+        gate = v / v.sum(1, keepdim=True) if topk == 2 else v
     slot, tok, seg = tables(idx, E) if capacity is None else tables(idx, E, h.shape[-2], capacity)
     pad = torch.cat([h2, h2.new_zeros(1, d)], 0)
     xs = pad.index_select(0, torch.where(tok >= 0, tok, torch.full_like(tok, h2.shape[0])))

@@ -186,6 +186,46 @@ def test_moe_auxiliary_router_terms(dev):
     assert float(wfd.grad.abs().max()) == 0.0                           # no gradient reaches the experts through aux
 
 
+@pytest.mark.parametrize("shape,topk,skew", [((1024, 256, 512, 8), 2, 0.0), ((1024, 256, 512, 4), 1, 0.0),
+                                              ((2048, 512, 768, 8), 2, 2.0)])
+def test_moe_layer_with_bf16_experts_forward_backward(dev, shape, topk, skew):
+    """The experts in bf16 (MoeMLP.forward with moe_experts_local, round2/source/train.py:10716: the kit's expression per
+    expert): layer output and every gradient against the oracle's bf16 layer fed the KERNEL'S selections (so that a near-tie
+    of the router cannot move a token), to the bf16 bar 5e-3; the grouped expert MLP alone, on the kernel's own gathered
+    rows, against the same expression expert by expert."""
+    import torch.nn.functional as F
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import autograd as A, ops
+    N, d, Fd, E = shape
+    h, router, wf, wp, bias = _layer(2, N, d, Fd, E, skew)
+    hd, rd = h.to(dev).requires_grad_(True), router.to(dev).requires_grad_(True)
+    wfd, wpd = wf.to(dev).requires_grad_(True), wp.to(dev).requires_grad_(True)
+    b = bias.to(dev) if skew else None
+    out = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, None, topk, b)
+    g = torch.randn(N, d, generator=torch.Generator().manual_seed(3)).bfloat16()
+    out.backward(g.to(dev))
+    # the grouped MLP by itself: every expert's segment of the gathered rows through the eager bf16 expression
+    p, idx, gate, _ = ops.moe_route(hd.detach(), rd.detach().float().contiguous(), topk, b, want_logits=True)
+    tab = ops.moe_tables(idx, E)
+    xs, none8 = ops.moe_gather(hd.detach(), tab, None)
+    assert none8 is None
+    ys, r, hh = ops.moe_mlp_fwd(xs, wfd.detach(), wpd.detach(), tab)
+    seg = tab["seg"].cpu().tolist()
+    for e in range(E):
+        xe = xs[seg[e]:seg[e + 1]].cpu()
+        pre = F.linear(xe, wf[e])
+        assert torch.equal(r[seg[e]:seg[e + 1]].cpu(), torch.relu(pre)) or rel_l2(r[seg[e]:seg[e + 1]], torch.relu(pre)) < 3e-3
+        assert rel_l2(ys[seg[e]:seg[e + 1]], F.linear(torch.relu(pre).square(), wp[e])) < 5e-3
+    assert torch.equal(hh[:seg[-1]], (r * r)[:seg[-1]])                   # h = bf16(r^2) exactly (rows past the last segment are not written)
+    ho, ro, wfo, wpo = (t.clone().requires_grad_(True) for t in (h, router, wf, wp))
+    oo, _ = O.moe_forward(ho, ro, wfo, wpo, topk, bias if skew else None, fp8=False, idx=idx.cpu().long())
+    oo.backward(g)
+    assert rel_l2(out, oo) < 5e-3
+    assert rel_l2(hd.grad, ho.grad) < 5e-3
+    assert rel_l2(wfd.grad, wfo.grad) < 5e-3 and rel_l2(wpd.grad, wpo.grad) < 5e-3
+    assert rel_l2(rd.grad, ro.grad) < 1e-2
+
+
 @pytest.mark.parametrize("topk", [1, 2])
 def test_moe_per_sequence_balance_term(dev, topk):
     """The per-sequence balance term of moe_aux_terms (round2/source/train.py:10789-10792): the kernel's term and the

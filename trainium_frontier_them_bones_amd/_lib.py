@@ -88,6 +88,8 @@ SIGNATURES = {
     "tfb_moe_route_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _l, _i, _i, _i, _vp],
     "tfb_moe_route_bwd_aux": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _f, _f, _l, _i, _i, _i, _vp],
     "tfb_moe_aux_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_moe_mlp_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_moe_mlp_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_moe_aux_seq_fwd": [_vp, _vp, _vp, _vp, _vp, _l, _l, _i, _i, _vp],
     "tfb_moe_route_bwd_aux_seq": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _f, _f, _vp, _f, _l, _l, _i, _i, _i, _vp],
     "tfb_moe_backward_scales": [_vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],

@@ -611,7 +611,9 @@ class Moe8State:
 class MoeMlp8Fn(torch.autograd.Function):
     """The routed half of MoeMLP.forward_e8 (round2/source/train.py:11003-11067) with every expert on this GPU:
     router -> top-k -> dropless dispatch -> grouped fp8 expert MLPs -> gated combine. h [.., d] bf16, router fp32 [E, d],
-    w_fc [E, F, d], w_proj [E, d, F] bf16; router_bias fp32 [E] or None (added to the logits)."""
+    w_fc [E, F, d], w_proj [E, d, F] bf16; router_bias fp32 [E] or None (added to the logits).
+    state None: the experts run in bf16 (MoeMLP.forward with moe_experts_local, round2/source/train.py:10941-11001, 10716:
+    the kit's expression per expert, d and F multiples of 128)."""
 
     @staticmethod
     def forward(ctx, h, router, w_fc, w_proj, state, topk, router_bias, aux_weights=None, capacity=None):
@@ -627,8 +629,12 @@ class MoeMlp8Fn(torch.autograd.Function):
         # capacity: the reference's per-sequence count (round2/source/train.py:10555): each row of h [b, t, d] keeps its first
         # `capacity` assignments per expert; None keeps everything
         tab = ops.moe_tables(idx, E) if capacity is None else ops.moe_tables(idx, E, h.shape[-2], capacity)
-        xs, xs8 = ops.moe_gather(h2, tab, state.x_scale)
-        ys, r = ops.moe_mlp8_fwd(xs8, state.w8, state.rows, tab, F)
+        if state is not None:
+            xs, xs8 = ops.moe_gather(h2, tab, state.x_scale)
+            ys, r = ops.moe_mlp8_fwd(xs8, state.w8, state.rows, tab, F)
+        else:
+            xs, _ = ops.moe_gather(h2, tab, None)
+            ys, r, _h = ops.moe_mlp_fwd(xs, w_fc.detach().to(bf16).contiguous(), w_proj.detach().to(bf16).contiguous(), tab)
         out = ops.moe_combine(ys, tab, gate, h2.shape[0])
         ctx.tab, ctx.state, ctx.hshape, ctx.aux_weights = tab, state, h.shape, aux_weights
         if aux_weights is None:
@@ -666,8 +672,11 @@ class MoeMlp8Fn(torch.autograd.Function):
             gout = torch.zeros(ctx.hshape, dtype=h2.dtype, device=h2.device)
         g2 = gout.reshape(-1, gout.shape[-1]).contiguous()
         dys, dgate = ops.moe_combine_bwd(g2, ys, tab, gate)
-        rows_b = ops.moe_backward_scales(dys, st.rows, tab)
-        dxs, dpre = ops.moe_mlp8_bwd(dys, r, st.w8, rows_b, tab)
+        if st is not None:
+            rows_b = ops.moe_backward_scales(dys, st.rows, tab)
+            dxs, dpre = ops.moe_mlp8_bwd(dys, r, st.w8, rows_b, tab)
+        else:
+            dxs, dpre = ops.moe_mlp_bwd(dys, r, w_fc.detach().to(bf16).contiguous(), w_proj.detach().to(bf16).contiguous(), tab)
         # one grouped launch writes both gradients: both weights carry a gradient buffer (in the same state) or neither
         # does; the "fresh" flags are only touched on the branch that really writes the buffers
         if (getattr(w_fc, "grad_buf", None) is None) != (getattr(w_proj, "grad_buf", None) is None):

@@ -905,3 +905,93 @@ extern "C" int tfb_moe_dw(const void* dpre, const void* xs, const void* dys, con
   using CfgSq = GemmCfg<128, 128, 4, 1, 2, TFB_K_STRIDED, TFB_K_STRIDED>;
   return gemm_launch_args<CfgSq>(a, E, 1, LoadSquare{}, LoadIdentity{}, e2, s);
 }
+
+// ---- bf16 experts ------------------------------------------------------------------------------------------------
+// The routed experts in bf16, every expert on this GPU, on the grouped buffers of the slot tables: each expert e applies
+// F.linear(relu(F.linear(x, w_fc[e])).square(), w_proj[e]) to its rows, with the bf16 roundings of those four operations
+// (pre, r = relu(pre), h = r^2, y). Replaces moe_experts_local / the kit's expression of moe_expert_mlp
+// (round2/source/train.py:10716-10727, 10711) and its autograd backward.
+namespace {
+struct EpiRelu2 {  // pre = bf16(acc); r = max(pre, 0); h = bf16(r r)
+  bf16_t* r;
+  bf16_t* h;
+  long F;
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
+    u32x4 rb, hb;
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      float a = v[i], b = v[i + 1];
+      round2_bf(a, b);
+      a = fmaxf(a, 0.f);
+      b = fmaxf(b, 0.f);
+      rb[i >> 1] = pack2bf(a, b);  // exact: a and b are bf16 values
+      a *= a;
+      b *= b;
+      hb[i >> 1] = round2_bf(a, b);
+    }
+    const long off = (long)q * F + p;
+    *(u32x4*)(r + off) = rb;
+    *(u32x4*)(h + off) = hb;
+  }
+};
+struct EpiDpre {  // dpre = bf16(bf16(acc) (2 r)): the gradient through h = r^2 and the ReLU (r = 0 where it was off)
+  const bf16_t* r;
+  bf16_t* dpre;
+  long F;
+  typedef u32x4 pre_t;
+  __device__ __forceinline__ pre_t prefetch(int p, int q) const { return *(const u32x4*)(r + (long)q * F + p); }
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const pre_t& rv, int) const {
+    float rr[8];
+    unpack8bf(rv, rr);
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      float a = v[i], b = v[i + 1];
+      round2_bf(a, b);
+      a *= 2.f * rr[i];
+      b *= 2.f * rr[i + 1];
+      o[i >> 1] = round2_bf(a, b);
+    }
+    *(u32x4*)(dpre + (long)q * F + p) = o;
+  }
+};
+inline bool shapes16(long rmax, int d, int F) { return rmax > 0 && rmax % 128 == 0 && d > 0 && d % 128 == 0 && F > 0 && F % 128 == 0; }
+using CfgNT = GemmCfg<128, 128, 2, 2, 2, TFB_K_CONTIG, TFB_K_CONTIG>;
+using CfgNN = GemmCfg<128, 128, 2, 2, 2, TFB_K_STRIDED, TFB_K_CONTIG>;
+}  // namespace
+
+// xs bf16 [rmax][d] (the gathered rows, padding rows zero), w_fc bf16 [E][F][d], w_proj bf16 [E][d][F], tile_expert int32
+// [rmax / 128] -> ys bf16 [rmax][d], r bf16 [rmax][F] = relu(pre) and h bf16 [rmax][F] = r^2 (both kept for the backward).
+extern "C" int tfb_moe_mlp_fwd(const void* xs, const void* w_fc, const void* w_proj, const void* tile_expert, void* ys, void* r,
+                               void* h, long rmax, int d, int F, void* stream) {
+  if (!xs || !w_fc || !w_proj || !tile_expert || !ys || !r || !h) return TFB_ERR_ARG;
+  if (!shapes16(rmax, d, F)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const long n = (long)F * d;
+  EpiRelu2 e1{(bf16_t*)r, (bf16_t*)h, (long)F};
+  int st = grouped_launch<CfgNT>((const uint8_t*)w_fc, d * 2L, n * 2, (const uint8_t*)xs, d * 2L, F, rmax, d * 2L,
+                                 (const int*)tile_expert, e1, s);
+  if (st != TFB_OK) return st;
+  EpiStore e2{ys, (long)d, 0, 0};
+  return grouped_launch<CfgNT>((const uint8_t*)w_proj, F * 2L, n * 2, (const uint8_t*)h, F * 2L, d, rmax, F * 2L,
+                               (const int*)tile_expert, e2, s);
+}
+
+// dys bf16 [rmax][d], r as the forward left it -> dpre bf16 [rmax][F] = bf16(bf16(dys w_proj[e]) 2 r), dxs bf16 [rmax][d] =
+// dpre w_fc[e]. The weight gradients are tfb_moe_dw(dpre, xs, dys, r, ...): dw_proj contracts dys with bf16(r^2) = h.
+extern "C" int tfb_moe_mlp_bwd(const void* dys, const void* r, const void* w_fc, const void* w_proj, const void* tile_expert,
+                               void* dxs, void* dpre, long rmax, int d, int F, void* stream) {
+  if (!dys || !r || !w_fc || !w_proj || !tile_expert || !dxs || !dpre) return TFB_ERR_ARG;
+  if (!shapes16(rmax, d, F)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const long n = (long)F * d;
+  // dh[row][f] = sum_j dys[row][j] w_proj[e][j][f]: the weight is the k-strided operand (k = j, contiguous in f)
+  EpiDpre e1{(const bf16_t*)r, (bf16_t*)dpre, (long)F};
+  int st = grouped_launch<CfgNN>((const uint8_t*)w_proj, F * 2L, n * 2, (const uint8_t*)dys, d * 2L, F, rmax, d * 2L,
+                                 (const int*)tile_expert, e1, s);
+  if (st != TFB_OK) return st;
+  // dxs[row][j] = sum_f dpre[row][f] w_fc[e][f][j]
+  EpiStore e2{dxs, (long)d, 0, 0};
+  return grouped_launch<CfgNN>((const uint8_t*)w_fc, d * 2L, n * 2, (const uint8_t*)dpre, F * 2L, d, rmax, F * 2L,
+                               (const int*)tile_expert, e2, s);
+}

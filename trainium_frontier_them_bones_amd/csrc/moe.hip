@@ -257,9 +257,11 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const bf16_t* __restric
     float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     if (t >= 0) load8(h + (long)t * d + c, v);
     store8(xs + row * d + c, v);
-    u32x2 o = {cvt4_fp8<TFB_FMT_E4M3>(v[0] * sc, v[1] * sc, v[2] * sc, v[3] * sc),
-               cvt4_fp8<TFB_FMT_E4M3>(v[4] * sc, v[5] * sc, v[6] * sc, v[7] * sc)};
-    *(u32x2*)(xs8 + row * d + c) = o;
+    if (xs8) {
+      u32x2 o = {cvt4_fp8<TFB_FMT_E4M3>(v[0] * sc, v[1] * sc, v[2] * sc, v[3] * sc),
+                 cvt4_fp8<TFB_FMT_E4M3>(v[4] * sc, v[5] * sc, v[6] * sc, v[7] * sc)};
+      *(u32x2*)(xs8 + row * d + c) = o;
+    }
   }
 }
 
@@ -736,7 +738,7 @@ extern "C" int tfb_moe_tables_cap(const void* idx, void* cnt, void* cnt_all, voi
 // xs bf16 [rmax][d] = h[tok] (zero padding rows), xs8 = e4m3(xs * scale). Replaces MoeDispatch2.forward (10652-10660).
 extern "C" int tfb_moe_gather(const void* h, const void* tok, const void* scale_ptr, float scale_imm, void* xs, void* xs8,
                               long rmax, int d, void* stream) {
-  if (!h || !tok || !xs || !xs8) return TFB_ERR_ARG;
+  if (!h || !tok || !xs) return TFB_ERR_ARG;   // xs8 may be null: bf16 experts take no fp8 copy
   if (rmax <= 0 || d <= 0 || d % 8) return TFB_ERR_SHAPE;
   hipLaunchKernelGGL(moe_gather_kernel, dim3(nblocks(rmax * (d / 8))), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)h,
                      (const int*)tok, (const float*)scale_ptr, scale_imm, (bf16_t*)xs, (uint8_t*)xs8, rmax, d);

@@ -764,11 +764,14 @@ def moe_tables(idx, E, seq_len=None, capacity=None):
 
 
 def moe_gather(h2, tab, x_scale=4.0):
-    """(xs bf16 [rmax,d], xs8 uint8 [rmax,d])."""
+    """(xs bf16 [rmax,d], xs8 uint8 [rmax,d]); x_scale None: no fp8 copy (xs8 is None)."""
     _chk(h2)
     d = h2.shape[1]
     rmax = tab["rmax"]
     xs = torch.empty(rmax, d, dtype=bf16, device=h2.device)
+    if x_scale is None:
+        _lib.call("tfb_moe_gather", _p(h2), _p(tab["tok"]), None, 1.0, _p(xs), None, rmax, d, _stream())
+        return xs, None
     xs8 = torch.empty(rmax, d, dtype=torch.uint8, device=h2.device)
     if isinstance(x_scale, torch.Tensor):
         _lib.call("tfb_moe_gather", _p(h2), _p(tab["tok"]), _p(x_scale), 0.0, _p(xs), _p(xs8), rmax, d, _stream())
@@ -786,6 +789,32 @@ def moe_mlp8_fwd(xs8, w8, rows, tab, F):
     h8 = torch.empty(rmax, F, dtype=torch.uint8, device=xs8.device)
     _lib.call("tfb_moe_mlp8_fwd", _p(xs8), _p(w8), _p(rows), _p(tab["tile_expert"]), _p(ys), _p(r), _p(h8), rmax, d, F, _stream())
     return ys, r
+
+
+def moe_mlp_fwd(xs, w_fc, w_proj, tab):
+    """Grouped bf16 expert MLP forward: (ys bf16 [rmax,d], r bf16 [rmax,F] = relu(pre), h bf16 [rmax,F] = r^2).
+    w_fc bf16 [E,F,d], w_proj bf16 [E,d,F]."""
+    _chk(xs), _chk(w_fc), _chk(w_proj)
+    rmax, d = xs.shape
+    E, F, _ = w_fc.shape
+    if tuple(w_fc.shape) != (E, F, d) or tuple(w_proj.shape) != (E, d, F):
+        raise ValueError("moe_mlp_fwd: w_fc [E,F,d] and w_proj [E,d,F] expected")
+    ys = torch.empty(rmax, d, dtype=bf16, device=xs.device)
+    r = torch.empty(rmax, F, dtype=bf16, device=xs.device)
+    h = torch.empty(rmax, F, dtype=bf16, device=xs.device)
+    _lib.call("tfb_moe_mlp_fwd", _p(xs), _p(w_fc), _p(w_proj), _p(tab["tile_expert"]), _p(ys), _p(r), _p(h), rmax, d, F, _stream())
+    return ys, r, h
+
+
+def moe_mlp_bwd(dys, r, w_fc, w_proj, tab):
+    """Grouped bf16 expert MLP backward: (dxs bf16 [rmax,d], dpre bf16 [rmax,F])."""
+    _chk(dys), _chk(r), _chk(w_fc), _chk(w_proj)
+    rmax, d = dys.shape
+    F = r.shape[1]
+    dxs = torch.empty(rmax, d, dtype=bf16, device=dys.device)
+    dpre = torch.empty(rmax, F, dtype=bf16, device=dys.device)
+    _lib.call("tfb_moe_mlp_bwd", _p(dys), _p(r), _p(w_fc), _p(w_proj), _p(tab["tile_expert"]), _p(dxs), _p(dpre), rmax, d, F, _stream())
+    return dxs, dpre
 
 
 def moe_backward_scales(dys, rows, tab):
