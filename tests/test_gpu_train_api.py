@@ -406,3 +406,66 @@ def test_band_attention_through_the_reference_calls(api, dev):
     a = api.nki_causal_attention(q64, q64, q64, nw=4)
     b = api.nki_causal_attention(q64, q64, q64)
     assert torch.equal(a, b)                                                     # a band as wide as the sequence
+
+
+class _Lin:
+    def __init__(self, w):
+        self.weight = w
+
+
+class _SharedMlp:
+    def __init__(self, wf, wp):
+        self.c_fc, self.c_proj = _Lin(wf), _Lin(wp)
+
+
+class _MoeModule:
+    """The attributes of the reference's MoeMLP (round2/source/train.py:10818-10875) that moe_mlp reads."""
+
+    def __init__(self, router, w_fc, w_proj, topk, cap, e8, shared):
+        self.router, self.w_fc, self.w_proj, self.topk, self.cap, self.e8, self.shared = router, w_fc, w_proj, topk, cap, e8, shared
+
+
+@pytest.mark.parametrize("e8", [True, False])
+def test_moe_mlp_module_mirror(api, dev, e8):
+    """train_api.moe_mlp as MoeMLP.forward / forward_e8 (round2/source/train.py:10941-11067): the routed output against the
+    oracle layer with the same per-sequence capacity on the kernel's selections (fp8 experts 2e-2, bf16 experts 5e-3), the
+    shared half added to it, the statistics vector (kept share, lb, z, load shares) against the oracle's tables and terms,
+    and gradients reaching the router, the experts and the shared half."""
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import ops
+    B, T, d, H, E, topk, cap = 4, 256, 256, 512, 8, 2, 48
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(B, T, d, generator=g).bfloat16()
+    router = torch.randn(E, d, generator=g) * 0.5
+    wf = (torch.randn(E, H, d, generator=g) * 0.05).bfloat16()
+    wp = (torch.randn(E, d, H, generator=g) * 0.05).bfloat16()
+    sf = (torch.randn(2 * H, d, generator=g) * 0.05).bfloat16()
+    sp = (torch.randn(d, 2 * H, generator=g) * 0.05).bfloat16()
+    xd = x.to(dev).requires_grad_(True)
+    rd, wfd, wpd = (t.to(dev).requires_grad_(True) for t in (router, wf, wp))
+    sfd, spd = sf.to(dev).requires_grad_(True), sp.to(dev).requires_grad_(True)
+    alpha, beta, gamma = 0.01, 0.001, 0.02
+    bare = _MoeModule(rd, wfd, wpd, topk, cap, e8, None)
+    full = _MoeModule(rd, wfd, wpd, topk, cap, e8, _SharedMlp(sfd, spd))
+    routed = api.moe_mlp(bare, xd)
+    out, aux, stats = api.moe_mlp(full, xd, want_stats=True, aux_weights=(alpha, beta, gamma))
+    # the kernel's selections, then the oracle's layer on them
+    p, idx, _, logits = ops.moe_route(x.to(dev).reshape(-1, d), router.to(dev).contiguous(), topk, None, want_logits=True)
+    ic = idx.cpu().long()
+    xo, ro, wfo, wpo = (t.clone().requires_grad_(True) for t in (x, router, wf, wp))
+    oo, _ = O.moe_forward(xo, ro, wfo, wpo, topk, None, fp8=e8, capacity=cap, idx=ic)
+    tol = 2e-2 if e8 else 5e-3
+    assert rel_l2(routed, oo) < tol
+    shared_out = api.mlp_fused8(full.shared, xd) if e8 else api.relu_squared(xd.detach() @ sfd.detach().t()) @ spd.detach().t()
+    assert rel_l2(out, routed.detach().float() + shared_out.detach().float()) < 5e-3
+    slot, _, _ = O.tables(ic, E, T, cap)
+    lb, z, f, seq = O.aux_terms(p.cpu().double(), logits.cpu().double(), ic, topk, seq_len=T)
+    assert stats.shape == (3 + E,)
+    assert abs(stats[0].item() - float((slot >= 0).sum()) / (B * T * topk)) < 1e-6 and stats[0].item() < 1.0   # it does drop
+    assert abs(stats[1].item() - lb.item()) < 1e-4 * lb.item() and abs(stats[2].item() - z.item()) < 1e-4 * z.item()
+    assert rel_l2(stats[3:], f) < 1e-6
+    assert abs(aux.item() - (alpha * lb + beta * z + gamma * seq).item()) < 1e-4 * abs(aux.item())
+    (out.float().square().mean() + aux).backward()
+    for t in (xd, rd, wfd, wpd, sfd, spd):
+        assert t.grad is not None and bool(torch.isfinite(t.grad.float()).all()) and float(t.grad.float().abs().max()) > 0
+

@@ -616,12 +616,14 @@ class MoeMlp8Fn(torch.autograd.Function):
     the kit's expression per expert, d and F multiples of 128)."""
 
     @staticmethod
-    def forward(ctx, h, router, w_fc, w_proj, state, topk, router_bias, aux_weights=None, capacity=None):
+    def forward(ctx, h, router, w_fc, w_proj, state, topk, router_bias, aux_weights=None, capacity=None, info=None):
         """aux_weights = (alpha, beta): also returns (aux, stats) with aux = alpha lb + beta z, the router's weighted
         load-balance and z terms (round2/source/train.py:10779 moe_aux_terms; differentiable, its gradient joins the
         router's in the backward), and stats fp32 [2 + E] = (lb, z, the experts' load shares f_e).
         aux_weights = (alpha, beta, gamma) adds gamma times the per-sequence balance term (the reference's R2_MOE_AUX_SEQ,
-        10789-10792), the sequences being the rows of h [b, t, d]."""
+        10789-10792), the sequences being the rows of h [b, t, d].
+        info: a dict that receives "kept" = the share of the assignments that hold a row (1 without a capacity), the first
+        entry of the reference layer's statistics vector."""
         h2 = h.reshape(-1, h.shape[-1]).contiguous()
         E, F, d = w_fc.shape
         wr = router.detach().float().contiguous()
@@ -636,6 +638,8 @@ class MoeMlp8Fn(torch.autograd.Function):
             xs, _ = ops.moe_gather(h2, tab, None)
             ys, r, _h = ops.moe_mlp_fwd(xs, w_fc.detach().to(bf16).contiguous(), w_proj.detach().to(bf16).contiguous(), tab)
         out = ops.moe_combine(ys, tab, gate, h2.shape[0])
+        if info is not None:
+            info["kept"] = tab["cnt"].sum().float() / float(h2.shape[0] * topk)
         ctx.tab, ctx.state, ctx.hshape, ctx.aux_weights = tab, state, h.shape, aux_weights
         if aux_weights is None:
             ctx.save_for_backward(h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj)
@@ -691,4 +695,5 @@ class MoeMlp8Fn(torch.autograd.Function):
             dw_fc, dw_proj = ops.moe_dw(dpre, xs, dys, r, tab, E)
         br, accr = _accumulate_into(router)
         dh, dwr, _ = ops.moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, br, accr, aux=aux)
-        return dh.view(ctx.hshape), (None if br is not None else dwr.to(router.dtype)), dw_fc, dw_proj, None, None, None, None, None
+        return (dh.view(ctx.hshape), (None if br is not None else dwr.to(router.dtype)), dw_fc, dw_proj, None, None, None, None,
+                None, None)

@@ -294,6 +294,53 @@ def mlp_fused8(mlp, x):
     return y.reshape(b, t, c)
 
 
+def moe_refresh_weights(moe, *, e4m3_limit=240.0, x_scale=4.0):
+    """Once per optimizer step for a MoE block with fp8 experts: every expert's scale row and e4m3 weight bytes (what
+    fp8_refresh_weights writes into MoeMLP.exp8_sc, R2:10862-10872), kept as moe.tfb_moe8."""
+    st = getattr(moe, "tfb_moe8", None)
+    if st is None:
+        st = moe.tfb_moe8 = A.Moe8State(e4m3_limit, x_scale)
+    st.refresh(moe.w_fc.detach().to(bf16), moe.w_proj.detach().to(bf16))
+    return st
+
+
+def moe_mlp(moe, x, want_stats=False, aux_weights=(0.0, 0.0, 0.0)):
+    """MoeMLP.forward / forward_e8 (R2:10941-11067) with every expert on this GPU: x [b, t, d] bf16 -> the block's MLP output
+    (routed experts, plus the shared half when the module has one); with want_stats also the weighted auxiliary sum
+    aux_weights = (R2_MOE_AUX, R2_MOE_ZLOSS, R2_MOE_AUX_SEQ) . (lb, z, seq) and the statistics vector [3 + E] = (kept share
+    of the assignments, lb, z, the experts' load shares), as the reference returns them. `moe` is the reference's module:
+    router [E, d], w_fc [E, H, d], w_proj [E, d, H], topk, cap (per-sequence capacity; None or absent: dropless), e8 (fp8
+    experts; their scales come from moe_refresh_weights, made here on first use), shared (a module with c_fc / c_proj, or
+    None: run as mlp_fused8 when the experts are fp8, else as c_proj(relu_squared(c_fc(x))))."""
+    if x.dim() != 3:
+        raise ValueError("moe_mlp takes x [b, t, d]")
+    e8 = bool(getattr(moe, "e8", False))
+    st = None
+    if e8:
+        st = getattr(moe, "tfb_moe8", None)
+        if st is None or st.rows is None:
+            st = moe_refresh_weights(moe)
+    cap = getattr(moe, "cap", None)
+    info = {}
+    args = (x, moe.router, moe.w_fc, moe.w_proj, st, int(moe.topk), None)
+    if want_stats:
+        out, aux, terms = A.MoeMlp8Fn.apply(*args, tuple(float(w) for w in aux_weights), cap, info)
+    else:
+        out = A.MoeMlp8Fn.apply(*args, None, cap, info)
+    shared = getattr(moe, "shared", None)
+    if shared is not None:
+        if e8:
+            out = out + mlp_fused8(shared, x)
+        else:
+            wf, wp = shared.c_fc.weight, shared.c_proj.weight
+            out = out + A.LinearFn.apply(relu_squared(A.LinearFn.apply(x, wf if wf.dtype == bf16 else wf.to(bf16))),
+                                         wp if wp.dtype == bf16 else wp.to(bf16))
+    if not want_stats:
+        return out
+    stats = torch.cat([info["kept"].reshape(1), terms]).detach()
+    return out, aux, stats
+
+
 def nr_mlp(mlp, x1):
     """x1 + MLP(rms_norm(x1)) on [b, t, n_embd] with the norm and the residual add folded into the fp8 MLP's two calls
     (R2:9202 nr_mlp / 9168 NrMlp; kernels K/nki_mlp_nr8.py:1032): the norm's pass also writes the e4m3 operand, the add
