@@ -266,7 +266,7 @@ def config_probe(which):
             bias = torch.zeros(E)
             bias[:2] = skew
             b = bias.to(dev) if skew else None
-            st = A.Moe8State()
+            st = A.Moe8State(dw_fp8=True)
 
             def c5():
                 clear(h, router, wf, wp)

@@ -355,6 +355,17 @@ int tfb_moe_mlp8_fwd(const void* x8, const void* w8, const void* rows, const voi
                      long rmax, int d, int F, void* stream);
 int tfb_moe_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* rows, const void* tile_expert, void* dx,
                      void* dpre, void* dp8, long rmax, int d, int F, void* stream);
+/* tfb_moe_mlp8_bwd for the fp8 weight gradients: dpre may be NULL (they read dp8), and with hq8 non-NULL also
+ * hq8 [rmax][F] = e4m3(min(bf16(r^2) s_h, hq_limit)) at each expert's own s_h (tfb_mlp8_bwd_q, grouped). */
+int tfb_moe_mlp8_bwd_q(const void* dy8, const void* r, const void* w8, const void* rows, const void* tile_expert, void* dx,
+                       void* dpre, void* dp8, void* hq8, float hq_limit, long rmax, int d, int F, void* stream);
+/* The experts' two weight gradients in fp8 over each expert's row segment [seg[e], seg[e+1]) of the grouped byte buffers:
+ * dw_fc [E][F][d] (+)= bf16((dp8_e^T @ xs8_e) / (s_dp[e] x_scale)), dw_proj [E][d][F] (+)= bf16((dy8_e^T @ hq8_e) /
+ * (s_dy[e] s_h[e])); rows fp32 [E][16] = the backward call's rows; bf16 or fp32 outputs, optionally accumulated into.
+ * Replaces mlp8_weight_grads under its fp8 weight-gradient switch (round2/source/train.py:8209-8229) inside the experts'
+ * backward (moe_expert8_mlp, round2/source/train.py:10731), expert by expert. */
+int tfb_moe_dw8(const void* xs8, const void* dp8, const void* hq8, const void* dy8, const void* rows, float x_scale,
+                const void* seg, void* dw_fc, void* dw_proj, int E, int d, int F, int out_f32, int accumulate, void* stream);
 
 /* dw_fc [E][F][d] (+)= dpre_e^T xs_e, dw_proj [E][d][F] (+)= dys_e^T bf16(r_e^2) over each expert's row segment.
  * Replaces the per-expert weight_grads (round2/source/kernels/nki_mlp_fused8.py:706-711). */

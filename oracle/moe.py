@@ -79,10 +79,10 @@ def tables(idx, E, seq_len=None, capacity=None):
 
 class _ExpertMlp8(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x2, w_fc, w_proj, row, x_scale, dy_amax=None):
+    def forward(ctx, x2, w_fc, w_proj, row, x_scale, dy_amax=None, dw_fp8=False, e4m3_limit=240.0):
         y, r = omlp.forward(x2, w_fc, w_proj, row, x_scale)
         ctx.save_for_backward(x2, r, w_fc, w_proj, row)
-        ctx.dy_amax = dy_amax
+        ctx.dy_amax, ctx.dw_fp8, ctx.x_scale, ctx.e4m3_limit = dy_amax, dw_fp8, x_scale, e4m3_limit
         return y
 
     @staticmethod
@@ -91,13 +91,17 @@ class _ExpertMlp8(torch.autograd.Function):
         dy = dy.contiguous()
         # the expert's backward scales come from the amax of ITS rows of dy; a caller that runs only a slice of those
         # rows passes the amax over all of them (dy_amax), so the slice is rounded exactly as inside the whole layer
-        dx, h, dpre = omlp.backward(dy, r, w_fc, w_proj, omlp.backward_scales(dy, row, ctx.dy_amax))
-        dw_fc, dw_proj = omlp.weight_grads(dy, x2, h, dpre)
-        return dx, dw_fc, dw_proj, None, None, None
+        row_b = omlp.backward_scales(dy, row, ctx.dy_amax)
+        dx, h, dpre = omlp.backward(dy, r, w_fc, w_proj, row_b)
+        if ctx.dw_fp8:   # the fp8 weight-gradient switch (round2/source/train.py:8209-8229) inside the expert's backward
+            dw_fc, dw_proj = omlp.weight_grads_fp8(x2, dy, h, dpre, row_b, ctx.x_scale, ctx.e4m3_limit)
+        else:
+            dw_fc, dw_proj = omlp.weight_grads(dy, x2, h, dpre)
+        return dx, dw_fc, dw_proj, None, None, None, None, None
 
 
 def moe_forward(h, router, w_fc, w_proj, topk, bias=None, fp8=True, e4m3_limit=240.0, x_scale=4.0, dys_amax=None,
-                capacity=None, idx=None):
+                capacity=None, idx=None, dw_fp8=False):
     """h [.., d] bf16; router [E, d]; w_fc [E, F, d]; w_proj [E, d, F]. Differentiable (autograd) in h, router, weights.
     fp8 False: the experts in bf16, the kit's expression per expert (round2/source/train.py:10716 moe_experts_local).
     dys_amax (optional, fp32 [E]): per-expert amax of the expert outputs' gradients to take the backward scales from,
@@ -124,7 +128,7 @@ def moe_forward(h, router, w_fc, w_proj, topk, bias=None, fp8=True, e4m3_limit=2
         if fp8:
             row = omlp.forward_scales(w_fc[e].detach(), w_proj[e].detach(), e4m3_limit, x_scale)
             outs.append(_ExpertMlp8.apply(xe, w_fc[e], w_proj[e], row, x_scale,
-                                          None if dys_amax is None else dys_amax[e]))
+                                          None if dys_amax is None else dys_amax[e], dw_fp8, e4m3_limit))
         else:
             outs.append(F.linear(torch.relu(F.linear(xe, w_fc[e])).square(), w_proj[e]))
     ys = torch.cat(outs, 0)

@@ -226,6 +226,37 @@ def test_moe_layer_with_bf16_experts_forward_backward(dev, shape, topk, skew):
     assert rel_l2(rd.grad, ro.grad) < 1e-2
 
 
+@pytest.mark.parametrize("shape,topk,skew", [((1024, 256, 512, 8), 2, 0.0), ((2048, 512, 768, 8), 2, 2.0)])
+def test_moe_layer_with_fp8_weight_gradients(dev, shape, topk, skew):
+    """The experts' weight gradients in fp8 as well (round2/source/train.py:8209-8229 inside each expert's backward): same
+    output and input / router gradients as with bf16 weight gradients (those GEMMs are untouched: bit-equal), the weight
+    gradients against the oracle's fp8 form on the kernel's selections within the fp8 bar, and close to the bf16 ones."""
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import autograd as A, ops
+    N, d, Fd, E = shape
+    h, router, wf, wp, bias = _layer(2, N, d, Fd, E, skew)
+    b = bias.to(dev) if skew else None
+    g = torch.randn(N, d, generator=torch.Generator().manual_seed(3)).bfloat16()
+    res = {}
+    for dw8 in (False, True):
+        hd, rd = h.to(dev).requires_grad_(True), router.to(dev).requires_grad_(True)
+        wfd, wpd = wf.to(dev).requires_grad_(True), wp.to(dev).requires_grad_(True)
+        st = A.Moe8State(dw_fp8=dw8)
+        st.refresh(wfd, wpd)
+        out = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, st, topk, b)
+        out.backward(g.to(dev))
+        res[dw8] = (out.detach(), hd.grad, rd.grad, wfd.grad, wpd.grad)
+    assert torch.equal(res[True][0], res[False][0]) and torch.equal(res[True][1], res[False][1])
+    assert torch.equal(res[True][2], res[False][2])
+    assert rel_l2(res[True][3], res[False][3]) < 6e-2 and rel_l2(res[True][4], res[False][4]) < 6e-2
+    assert not torch.equal(res[True][3], res[False][3])                  # it is another arithmetic
+    _, idx, _, _ = ops.moe_route(h.to(dev), router.to(dev).contiguous(), topk, b, want_logits=True)
+    ho, ro, wfo, wpo = (t.clone().requires_grad_(True) for t in (h, router, wf, wp))
+    oo, _ = O.moe_forward(ho, ro, wfo, wpo, topk, bias if skew else None, idx=idx.cpu().long(), dw_fp8=True)
+    oo.backward(g)
+    assert rel_l2(res[True][3], wfo.grad) < 2e-2 and rel_l2(res[True][4], wpo.grad) < 2e-2
+
+
 @pytest.mark.parametrize("topk", [1, 2])
 def test_moe_per_sequence_balance_term(dev, topk):
     """The per-sequence balance term of moe_aux_terms (round2/source/train.py:10789-10792): the kernel's term and the

@@ -88,6 +88,8 @@ SIGNATURES = {
     "tfb_moe_route_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _l, _i, _i, _i, _vp],
     "tfb_moe_route_bwd_aux": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _f, _f, _l, _i, _i, _i, _vp],
     "tfb_moe_aux_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_moe_mlp8_bwd_q": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _l, _i, _i, _vp],
+    "tfb_moe_dw8": [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "tfb_moe_mlp_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_moe_mlp_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_moe_aux_seq_fwd": [_vp, _vp, _vp, _vp, _vp, _l, _l, _i, _i, _vp],

@@ -592,8 +592,10 @@ class Moe8State:
     """Per-layer fp8 state of the experts, refreshed once per optimizer step: a scale row and an e4m3 weight pack per
     expert (the reference's exp8_sc [E,128,16] / exp8_w8 buffers, round2/source/train.py:10900-10935)."""
 
-    def __init__(self, e4m3_limit=240.0, x_scale=4.0):
-        self.e4m3_limit, self.x_scale = e4m3_limit, x_scale
+    def __init__(self, e4m3_limit=240.0, x_scale=4.0, dw_fp8=False):
+        """dw_fp8: the experts' weight gradients in fp8 as well, from the bytes the other four GEMMs multiplied (the
+        reference's fp8 weight-gradient switch, round2/source/train.py:8209-8229, inside each expert's backward)."""
+        self.e4m3_limit, self.x_scale, self.dw_fp8 = e4m3_limit, x_scale, dw_fp8
         self.rows = None
         self.w8 = None
 
@@ -641,6 +643,7 @@ class MoeMlp8Fn(torch.autograd.Function):
         if info is not None:
             info["kept"] = tab["cnt"].sum().float() / float(h2.shape[0] * topk)
         ctx.tab, ctx.state, ctx.hshape, ctx.aux_weights = tab, state, h.shape, aux_weights
+        ctx.xs8 = xs8 if state is not None and state.dw_fp8 else None    # the fp8 weight gradient's operand (not an input of any op)
         if aux_weights is None:
             ctx.save_for_backward(h2, wr, p, idx, gate, xs, ys, r, router, w_fc, w_proj)
             return out.view(h.shape)
@@ -676,7 +679,11 @@ class MoeMlp8Fn(torch.autograd.Function):
             gout = torch.zeros(ctx.hshape, dtype=h2.dtype, device=h2.device)
         g2 = gout.reshape(-1, gout.shape[-1]).contiguous()
         dys, dgate = ops.moe_combine_bwd(g2, ys, tab, gate)
-        if st is not None:
+        dw8 = st is not None and st.dw_fp8
+        if dw8:
+            rows_b = ops.moe_backward_scales(dys, st.rows, tab)
+            dxs, dp8, hq8, dy8 = ops.moe_mlp8_bwd_q(dys, r, st.w8, rows_b, tab, st.e4m3_limit)
+        elif st is not None:
             rows_b = ops.moe_backward_scales(dys, st.rows, tab)
             dxs, dpre = ops.moe_mlp8_bwd(dys, r, st.w8, rows_b, tab)
         else:
@@ -689,8 +696,13 @@ class MoeMlp8Fn(torch.autograd.Function):
             (bf, accf), (bp, accp) = _accumulate_into(w_fc), _accumulate_into(w_proj)
             if accf != accp:
                 raise RuntimeError("MoeMlp8Fn: the two expert weights' gradient buffers are in different states")
-            ops.moe_dw(dpre, xs, dys, r, tab, E, bf, bp, accumulate=accf)
+            if dw8:
+                ops.moe_dw8(ctx.xs8, dp8, hq8, dy8, rows_b, st.x_scale, tab, E, bf, bp, accumulate=accf)
+            else:
+                ops.moe_dw(dpre, xs, dys, r, tab, E, bf, bp, accumulate=accf)
             dw_fc = dw_proj = None
+        elif dw8:
+            dw_fc, dw_proj = ops.moe_dw8(ctx.xs8, dp8, hq8, dy8, rows_b, st.x_scale, tab, E)
         else:
             dw_fc, dw_proj = ops.moe_dw(dpre, xs, dys, r, tab, E)
         br, accr = _accumulate_into(router)

@@ -859,18 +859,95 @@ extern "C" int tfb_moe_mlp8_fwd(const void* x8, const void* w8, const void* rows
   return grouped_launch<Cfg8>(b + 2 * n, F, 4 * n, (const uint8_t*)h8, F, d, rmax, F, (const int*)tile_expert, e2, s);
 }
 
-extern "C" int tfb_moe_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* rows, const void* tile_expert,
-                                void* dx, void* dpre, void* dp8, long rmax, int d, int F, void* stream) {
-  if (!dy8 || !r || !w8 || !rows || !tile_expert || !dx || !dpre || !dp8) return TFB_ERR_ARG;
-  if (!shapes8(rmax, d, F)) return TFB_ERR_SHAPE;
+// dpre may be null (the fp8 weight gradients read dp8, not dpre); hq8 non-null: also hq8 [rmax][F] = e4m3(min(bf16(r^2) s_h,
+// hq_limit)), the activation operand of the fp8 dW_proj (each expert at its own s_h).
+extern "C" int tfb_moe_mlp8_bwd_q(const void* dy8, const void* r, const void* w8, const void* rows, const void* tile_expert,
+                                  void* dx, void* dpre, void* dp8, void* hq8, float hq_limit, long rmax, int d, int F,
+                                  void* stream) {
+  if (!dy8 || !r || !w8 || !rows || !tile_expert || !dx || !dp8) return TFB_ERR_ARG;
+  if (!shapes8(rmax, d, F) || (hq8 && !(hq_limit > 0.f))) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   const uint8_t* b = (const uint8_t*)w8;
   const long n = (long)F * d;
-  EpiDh e1{(const float*)rows, (const bf16_t*)r, (bf16_t*)dpre, (uint8_t*)dp8, nullptr, nullptr, 0.f, (long)F};
+  EpiDh e1{(const float*)rows, (const bf16_t*)r, (bf16_t*)dpre, (uint8_t*)dp8, nullptr, (uint8_t*)hq8, hq_limit, (long)F};
   int st = grouped_launch<Cfg8g>(b + 3 * n, d, 4 * n, (const uint8_t*)dy8, d, F, rmax, d, (const int*)tile_expert, e1, s);
   if (st != TFB_OK) return st;
   EpiScaleStore e2{(const float*)rows, SC_DQ_DX, (bf16_t*)dx, (long)d};
   return grouped_launch<Cfg8g>(b + n, F, 4 * n, (const uint8_t*)dp8, F, d, rmax, F, (const int*)tile_expert, e2, s);
+}
+extern "C" int tfb_moe_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* rows, const void* tile_expert,
+                                void* dx, void* dpre, void* dp8, long rmax, int d, int F, void* stream) {
+  if (!dpre) return TFB_ERR_ARG;
+  return tfb_moe_mlp8_bwd_q(dy8, r, w8, rows, tile_expert, dx, dpre, dp8, nullptr, 0.f, rmax, d, F, stream);
+}
+
+namespace {
+// out[g] (+)= acc imm / (rows[g][ca] rows[g][cb]): a grouped fp8 weight gradient leaves the accumulators at its expert's
+// power-of-two scales (cb < 0: one scale)
+struct EpiDescaleGrouped {
+  EpiStore base;
+  long slab;  // elements per group
+  const float* rows;
+  int ca, cb;
+  float imm;
+  float mul = 0.f;
+  __device__ __forceinline__ EpiDescaleGrouped for_group(int g) const {
+    EpiDescaleGrouped e = *this;
+    e.base.out = base.f32 ? (void*)((float*)base.out + (long)g * slab) : (void*)((bf16_t*)base.out + (long)g * slab);
+    e.rows = rows + (long)g * NSC;
+    return e;
+  }
+  __device__ __forceinline__ EpiDescaleGrouped prepare() const {
+    EpiDescaleGrouped e = *this;
+    float dsc = rows[ca];
+    if (cb >= 0) dsc *= rows[cb];
+    e.mul = imm / dsc;
+    return e;
+  }
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int s) const {
+    float w[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = v[i] * mul;
+    base(p, q, w, s);
+  }
+};
+}  // namespace
+
+// The experts' two weight gradients in fp8 over each expert's row segment [seg[e], seg[e+1]) of the grouped byte buffers
+// (every segment a multiple of 128 rows): dw_fc [E][F][d] (+)= bf16((dp8_e^T @ xs8_e) / (s_dp[e] x_scale)), dw_proj [E][d][F]
+// (+)= bf16((dy8_e^T @ hq8_e) / (s_dy[e] s_h[e])), with the scales of rows fp32 [E][16] (the backward call's rows).
+// xs8 e4m3 (the gather's), dp8 e5m2 and hq8 e4m3 (tfb_moe_mlp8_bwd_q's), dy8 e5m2 (the backward's input bytes).
+// Replaces mlp8_weight_grads under its fp8 weight-gradient switch (round2/source/train.py:8209-8229) inside
+// moe_expert8_mlp's backward, expert by expert.
+extern "C" int tfb_moe_dw8(const void* xs8, const void* dp8, const void* hq8, const void* dy8, const void* rows, float x_scale,
+                           const void* seg, void* dw_fc, void* dw_proj, int E, int d, int F, int out_f32, int accumulate,
+                           void* stream) {
+  if (!xs8 || !dp8 || !hq8 || !dy8 || !rows || !seg || !dw_fc || !dw_proj) return TFB_ERR_ARG;
+  if (E <= 0 || d <= 0 || F <= 0 || d % 128 || F % 128 || !(x_scale > 0.f)) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  using Cfg = GemmCfg<128, 128, 2, 2, 1, TFB_K_STRIDED, TFB_K_STRIDED, TFB_FMT_E4M3, TFB_FMT_E5M2>;
+  GemmArgs a;
+  a.q_group = nullptr;
+  a.p_group_stride = 0;
+  a.k_seg = (const int*)seg;
+  a.nkt = 0;
+  // dw_fc[e][f][j] = sum_m dp8[m][f] xs8[m][j]: output contiguous in j -> P = xs8 (e4m3), Q = dp8 (e5m2)
+  a.P = GemmOperand{(const uint8_t*)xs8, (long)d};
+  a.Q = GemmOperand{(const uint8_t*)dp8, (long)F};
+  a.np = d;
+  a.nq = F;
+  a.ntp = d / 128;
+  EpiDescaleGrouped e1{EpiStore{dw_fc, (long)d, out_f32, accumulate}, (long)F * d, (const float*)rows, SC_S_DP, -1, 1.0f / x_scale};
+  int st = gemm_launch_args<Cfg>(a, E, 1, LoadIdentity{}, LoadIdentity{}, e1, s);
+  if (st != TFB_OK) return st;
+  // dw_proj[e][j][f] = sum_m dy8[m][j] hq8[m][f]: output contiguous in f -> P = hq8 (e4m3), Q = dy8 (e5m2)
+  a.P = GemmOperand{(const uint8_t*)hq8, (long)F};
+  a.Q = GemmOperand{(const uint8_t*)dy8, (long)d};
+  a.np = F;
+  a.nq = d;
+  a.ntp = F / 128;
+  EpiDescaleGrouped e2{EpiStore{dw_proj, (long)F, out_f32, accumulate}, (long)F * d, (const float*)rows, SC_S_DY, SC_S_H, 1.0f};
+  return gemm_launch_args<Cfg>(a, E, 1, LoadIdentity{}, LoadIdentity{}, e2, s);
 }
 
 // Per-expert weight gradients over the expert's row segment [seg[e], seg[e+1]) of the grouped buffers:

@@ -848,6 +848,33 @@ def moe_mlp8_bwd(dys, r, w8, rows_bwd, tab):
     return dxs, dpre
 
 
+def moe_mlp8_bwd_q(dys, r, w8, rows_bwd, tab, hq_limit):
+    """The grouped fp8 backward for the fp8 weight gradients: (dxs bf16 [rmax,d], dp8 e5m2 [rmax,F], hq8 e4m3 [rmax,F],
+    dy8 e5m2 [rmax,d]); no bf16 dpre is written."""
+    _chk(dys), _chk(r)
+    rmax, d = dys.shape
+    F = r.shape[1]
+    dy8 = moe_quant(dys, rows_bwd, 5, FMT_E5M2, tab)
+    dxs = torch.empty(rmax, d, dtype=bf16, device=dys.device)
+    dp8 = torch.empty(rmax, F, dtype=torch.uint8, device=dys.device)
+    hq8 = torch.empty(rmax, F, dtype=torch.uint8, device=dys.device)
+    _lib.call("tfb_moe_mlp8_bwd_q", _p(dy8), _p(r), _p(w8), _p(rows_bwd), _p(tab["tile_expert"]), _p(dxs), None, _p(dp8), _p(hq8),
+              float(hq_limit), rmax, d, F, _stream())
+    return dxs, dp8, hq8, dy8
+
+
+def moe_dw8(xs8, dp8, hq8, dy8, rows_bwd, x_scale, tab, E, dw_fc=None, dw_proj=None, accumulate=False, out_dtype=bf16):
+    """(dw_fc [E,F,d], dw_proj [E,d,F]) in fp8 over each expert's row segment, from the bytes the other GEMMs multiplied."""
+    _chk(xs8, torch.uint8), _chk(dp8, torch.uint8), _chk(hq8, torch.uint8), _chk(dy8, torch.uint8), _chk(rows_bwd, torch.float32)
+    d, F = xs8.shape[1], dp8.shape[1]
+    if dw_fc is None:
+        dw_fc = torch.empty(E, F, d, dtype=out_dtype, device=xs8.device)
+        dw_proj = torch.empty(E, d, F, dtype=out_dtype, device=xs8.device)
+    _lib.call("tfb_moe_dw8", _p(xs8), _p(dp8), _p(hq8), _p(dy8), _p(rows_bwd), float(x_scale), _p(tab["seg"]), _p(dw_fc), _p(dw_proj),
+              E, d, F, int(dw_fc.dtype == torch.float32), int(accumulate), _stream())
+    return dw_fc, dw_proj
+
+
 def moe_dw(dpre, xs, dys, r, tab, E, dw_fc=None, dw_proj=None, accumulate=False, out_dtype=bf16):
     """(dw_fc [E,F,d], dw_proj [E,d,F]) over each expert's row segment."""
     d, F = xs.shape[1], r.shape[1]
