@@ -32,75 +32,145 @@ __device__ __forceinline__ void store8(bf16_t* p, const float (&v)[8]) {
 
 // ------------------------------------------------------------------------------------------------ router
 // One wavefront per token: logits = h . Wr[e] (+ bias) in fp32, softmax, first-maximum top-k, gates.
+// The EP (8 or 16) per-lane partial sums are reduced over the wavefront together: at each of the first log2(EP) butterfly
+// steps a lane keeps half of its values and hands the other half to its partner, so the whole reduction is EP - 1 + 6 -
+// log2(EP) shuffles instead of 6 EP, with the same additions in the same order as a butterfly sum of every value
+// (a + b is b + a bit for bit), so two experts with equal weights still get equal logits.
+template <int EP>
+__device__ __forceinline__ float route_reduce(const float (&acc)[EP], int lane) {
+  float v[EP];
+#pragma unroll
+  for (int e = 0; e < EP; ++e) v[e] = acc[e];
+  int n = EP, off = 32;
+#pragma unroll
+  for (int lvl = 0; lvl < (EP == 16 ? 4 : 3); ++lvl) {
+    const bool hi = (lane & off) != 0;
+    n >>= 1;
+#pragma unroll
+    for (int j = 0; j < EP / 2; ++j) {
+      if (j < n) {
+        const float keep = hi ? v[n + j] : v[j], send = hi ? v[j] : v[n + j];
+        v[j] = keep + __shfl_xor(send, off, 64);
+      }
+    }
+    off >>= 1;
+  }
+  float r = v[0];
+#pragma unroll
+  for (int o = (EP == 16 ? 2 : 4); o > 0; o >>= 1) r += __shfl_xor(r, o, 64);
+  return r;  // the total of expert (lane >> (EP == 16 ? 2 : 3)) with its index bits in the order the steps split them
+}
+// the lane whose route_reduce result is expert e's total: step k (offset 32 >> k) split on bit (log2(EP) - 1 - k) of e
+template <int EP>
+__device__ __forceinline__ int route_lane_of(int e) {
+  return EP == 16 ? (e << 2) : (e << 3);
+}
+
+// TPW tokens per wavefront at a time (sharing one fetch of the router's weights) was measured at 2 and 4: slower than 1
+// (41 and 49 us against 36 for 16384 tokens of d = 1024), as was staging the weights in LDS under one round of workgroups.
+template <int EP, int TPW>
 __global__ __launch_bounds__(256) void moe_route_kernel(const bf16_t* __restrict__ h, const float* __restrict__ wr,
                                                        const float* __restrict__ bias, float* __restrict__ logits_out,
                                                        float* __restrict__ p_out, int* __restrict__ idx_out,
                                                        float* __restrict__ gate_out, long N, int d, int E, int topk) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (long n = (long)blockIdx.x * 4 + wave; n < N; n += (long)gridDim.x * 4) {
-    float acc[MAXE];
+  for (long n0 = ((long)blockIdx.x * 4 + wave) * TPW; n0 < N; n0 += (long)gridDim.x * 4 * TPW) {
+    float acc[TPW][EP];
 #pragma unroll
-    for (int e = 0; e < MAXE; ++e) acc[e] = 0.f;
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+      for (int e = 0; e < EP; ++e) acc[t][e] = 0.f;
     for (int c = lane * 8; c < d; c += 512) {
-      float x[8];
-      load8(h + n * d + c, x);
+      float x[TPW][8];
 #pragma unroll
-      for (int e = 0; e < MAXE; ++e) {
-        if (e < E) {
-          const float* w = wr + (long)e * d + c;
-          f32x4 w0 = *(const f32x4*)w, w1 = *(const f32x4*)(w + 4);
-          acc[e] += x[0] * w0[0] + x[1] * w0[1] + x[2] * w0[2] + x[3] * w0[3] + x[4] * w1[0] + x[5] * w1[1] + x[6] * w1[2] +
-                    x[7] * w1[3];
+      for (int t = 0; t < TPW; ++t) load8(h + (n0 + t < N ? n0 + t : N - 1) * d + c, x[t]);  // (a group's tail re-reads the last token)
+      if constexpr (EP <= 8) {
+        // no branch on e < E here: behind one, each expert's two loads wait for the previous expert's (2 E dependent round
+        // trips to the L2 per chunk: 42 -> 36 us); an expert beyond E re-reads the last one's weights, its sum is never used
+        f32x4 w0[EP], w1[EP];
+#pragma unroll
+        for (int e = 0; e < EP; ++e) {
+          const float* w = wr + (long)(e < E ? e : E - 1) * d + c;
+          w0[e] = *(const f32x4*)w;
+          w1[e] = *(const f32x4*)(w + 4);
         }
-      }
-    }
-    float mx = -INFINITY;
 #pragma unroll
-    for (int e = 0; e < MAXE; ++e) {
-      if (e < E) {
-        acc[e] = wave_sum(acc[e]) + (bias ? bias[e] : 0.f);
-        mx = fmaxf(mx, acc[e]);
-      }
-    }
-    float p[MAXE], den = 0.f;
+        for (int t = 0; t < TPW; ++t)
 #pragma unroll
-    for (int e = 0; e < MAXE; ++e) {
-      p[e] = e < E ? expf(acc[e] - mx) : 0.f;
-      den += p[e];
-    }
-    int i1 = 0, i2 = 0;
-    float v1 = -1.f, v2 = -1.f;
-#pragma unroll
-    for (int e = 0; e < MAXE; ++e) {
-      if (e < E) {
-        p[e] = p[e] / den;
-        if (p[e] > v1) {
-          v1 = p[e];
-          i1 = e;
-        }
-      }
-    }
-#pragma unroll
-    for (int e = 0; e < MAXE; ++e) {
-      if (e < E && e != i1 && p[e] > v2) {
-        v2 = p[e];
-        i2 = e;
-      }
-    }
-    if (lane == 0) {
-      for (int e = 0; e < E; ++e) {
-        p_out[n * E + e] = p[e];
-        if (logits_out) logits_out[n * E + e] = acc[e];
-      }
-      if (topk == 2) {
-        const float s = v1 + v2;
-        idx_out[n * 2] = i1;
-        idx_out[n * 2 + 1] = i2;
-        gate_out[n * 2] = v1 / s;
-        gate_out[n * 2 + 1] = v2 / s;
+          for (int e = 0; e < EP; ++e)
+            acc[t][e] += x[t][0] * w0[e][0] + x[t][1] * w0[e][1] + x[t][2] * w0[e][2] + x[t][3] * w0[e][3] + x[t][4] * w1[e][0] +
+                         x[t][5] * w1[e][1] + x[t][6] * w1[e][2] + x[t][7] * w1[e][3];
       } else {
-        idx_out[n] = i1;
-        gate_out[n] = v1;
+        // sixteen experts' weights of a chunk would be 128 registers: one expert at a time (102 us against 135 at d = 2048)
+#pragma unroll
+        for (int e = 0; e < EP; ++e) {
+          if (e < E) {
+            const float* w = wr + (long)e * d + c;
+            const f32x4 w0 = *(const f32x4*)w, w1 = *(const f32x4*)(w + 4);
+#pragma unroll
+            for (int t = 0; t < TPW; ++t)
+              acc[t][e] += x[t][0] * w0[0] + x[t][1] * w0[1] + x[t][2] * w0[2] + x[t][3] * w0[3] + x[t][4] * w1[0] +
+                           x[t][5] * w1[1] + x[t][6] * w1[2] + x[t][7] * w1[3];
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) {
+      const long n = n0 + t;
+      float lg[EP];
+      float mx = -INFINITY;
+      if constexpr (EP <= 8) {
+        const float mine = route_reduce<EP>(acc[t], lane);
+#pragma unroll
+        for (int e = 0; e < EP; ++e) lg[e] = e < E ? __shfl(mine, route_lane_of<EP>(e), 64) + (bias ? bias[e] : 0.f) : 0.f;
+      } else {  // (the joint reduction of sixteen values measured slower than sixteen butterflies: 114 against 102 us)
+#pragma unroll
+        for (int e = 0; e < EP; ++e) lg[e] = e < E ? wave_sum(acc[t][e]) + (bias ? bias[e] : 0.f) : 0.f;
+      }
+#pragma unroll
+      for (int e = 0; e < EP; ++e)
+        if (e < E) mx = fmaxf(mx, lg[e]);
+      float p[EP], den = 0.f;
+#pragma unroll
+      for (int e = 0; e < EP; ++e) {
+        p[e] = e < E ? expf(lg[e] - mx) : 0.f;
+        den += p[e];
+      }
+      int i1 = 0, i2 = 0;
+      float v1 = -1.f, v2 = -1.f;
+#pragma unroll
+      for (int e = 0; e < EP; ++e) {
+        if (e < E) {
+          p[e] = p[e] / den;
+          if (p[e] > v1) {
+            v1 = p[e];
+            i1 = e;
+          }
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < EP; ++e) {
+        if (e < E && e != i1 && p[e] > v2) {
+          v2 = p[e];
+          i2 = e;
+        }
+      }
+      if (lane == 0 && n < N) {
+        for (int e = 0; e < E; ++e) {
+          p_out[n * E + e] = p[e];
+          if (logits_out) logits_out[n * E + e] = lg[e];
+        }
+        if (topk == 2) {
+          const float s = v1 + v2;
+          idx_out[n * 2] = i1;
+          idx_out[n * 2 + 1] = i2;
+          gate_out[n * 2] = v1 / s;
+          gate_out[n * 2 + 1] = v2 / s;
+        } else {
+          idx_out[n] = i1;
+          gate_out[n] = v1;
+        }
       }
     }
   }
@@ -671,8 +741,12 @@ extern "C" int tfb_moe_route(const void* h, const void* wr, const void* bias, vo
                              int d, int E, int topk, void* stream) {
   if (!h || !wr || !p || !idx || !gate) return TFB_ERR_ARG;
   if (N <= 0 || d <= 0 || d % 8 || E < 2 || E > MAXE || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
-  hipLaunchKernelGGL(moe_route_kernel, dim3(nblocks(N * 64)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)h,
-                     (const float*)wr, (const float*)bias, (float*)logits, (float*)p, (int*)idx, (float*)gate, N, d, E, topk);
+  if (E <= 8)
+    hipLaunchKernelGGL((moe_route_kernel<8, 1>), dim3(nblocks(N * 64)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)h,
+                       (const float*)wr, (const float*)bias, (float*)logits, (float*)p, (int*)idx, (float*)gate, N, d, E, topk);
+  else
+    hipLaunchKernelGGL((moe_route_kernel<16, 1>), dim3(nblocks(N * 64)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)h,
+                       (const float*)wr, (const float*)bias, (float*)logits, (float*)p, (int*)idx, (float*)gate, N, d, E, topk);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
