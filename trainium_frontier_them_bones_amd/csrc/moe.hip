@@ -545,14 +545,27 @@ __global__ void moe_aux_seq_finish_kernel(const float* __restrict__ part, long n
 }
 
 // dh[n] = dxs[slot1] + dxs[slot2] + sum_e dlogits[n][e] Wr[e] (fp32 sum, one rounding).
+// A thread keeps ONE 8-column chunk for all the tokens it visits (the launch makes the thread count a multiple of the chunks
+// per row), so its slice of every expert's router weights stays in registers: fetched per token from the L2 they were 16
+// times the bytes of the output (537 MB for 16384 tokens of d = 1024) and what the kernel waited for.
+template <int EP>
 __global__ __launch_bounds__(256) void moe_dispatch_bwd_kernel(const bf16_t* __restrict__ dxs, const int* __restrict__ slot,
                                                               const float* __restrict__ dlogits, const float* __restrict__ wr,
                                                               bf16_t* __restrict__ dh, long N, int d, int E, int topk) {
   const int cpr = d / 8;
-  const long total = N * cpr;
-  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
-    long n = i / cpr;
-    int c = (int)(i % cpr) * 8;
+  const long tid = (long)blockIdx.x * 256 + threadIdx.x, nthreads = (long)gridDim.x * 256;
+  const int c = (int)(tid % cpr) * 8;
+  const long nstep = nthreads / cpr;
+  f32x4 w0[EP], w1[EP];
+  if (dlogits) {
+#pragma unroll
+    for (int e = 0; e < EP; ++e) {
+      const float* w = wr + (long)(e < E ? e : E - 1) * d + c;   // (an expert beyond E: the last one's, with a zero gradient)
+      w0[e] = *(const f32x4*)w;
+      w1[e] = *(const f32x4*)(w + 4);
+    }
+  }
+  for (long n = tid / cpr; n < N; n += nstep) {
     float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const int s1 = slot[n * topk];
     if (s1 >= 0) load8(dxs + (long)s1 * d + c, r);
@@ -566,14 +579,13 @@ __global__ __launch_bounds__(256) void moe_dispatch_bwd_kernel(const bf16_t* __r
       }
     }
     if (dlogits) {
-      for (int e = 0; e < E; ++e) {
-        const float g = dlogits[n * E + e];
-        const float* w = wr + (long)e * d + c;
-        f32x4 w0 = *(const f32x4*)w, w1 = *(const f32x4*)(w + 4);
+#pragma unroll
+      for (int e = 0; e < EP; ++e) {
+        const float g = e < E ? dlogits[n * E + e] : 0.f;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-          r[k] += g * w0[k];
-          r[4 + k] += g * w1[k];
+          r[k] += g * w0[e][k];
+          r[4 + k] += g * w1[e][k];
         }
       }
     }
@@ -857,8 +869,25 @@ static int moe_route_bwd_impl(const void* dgate, const void* p, const void* idx,
                      (const float*)p, (const int*)idx, (float*)dlogits, N, E, topk, (const float*)terms, (const float*)lse,
                      (const float*)gaux, alpha, beta, (const float*)fs, gamma, T > 0 ? T : N);
   TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(moe_dispatch_bwd_kernel, dim3(nblocks(N * (d / 8))), dim3(256), 0, s, (const bf16_t*)dxs, (const int*)slot,
-                     (const float*)dlogits, (const float*)wr, (bf16_t*)dh, N, d, E, topk);
+  {
+    // a thread count that is a multiple of the 8-column chunks per row: every thread then stays on one chunk
+    const int cpr = d / 8;
+    int g = cpr, b = 256;
+    while (b) {
+      const int t = g % b;
+      g = b;
+      b = t;
+    }
+    const int m = cpr / g;   // blocks per whole number of rows
+    int blocks = nblocks(N * cpr, 2048);
+    blocks = blocks < m ? m : blocks / m * m;
+    if (E <= 8)
+      hipLaunchKernelGGL(moe_dispatch_bwd_kernel<8>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)dxs, (const int*)slot,
+                         (const float*)dlogits, (const float*)wr, (bf16_t*)dh, N, d, E, topk);
+    else
+      hipLaunchKernelGGL(moe_dispatch_bwd_kernel<16>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)dxs, (const int*)slot,
+                         (const float*)dlogits, (const float*)wr, (bf16_t*)dh, N, d, E, topk);
+  }
   TFB_LAUNCH_CHECK();
   const long chunk = ((N + DWR_CHUNKS - 1) / DWR_CHUNKS + 31) / 32 * 32;
   const int chunks = (int)((N + chunk - 1) / chunk);
