@@ -367,28 +367,41 @@ __global__ __launch_bounds__(256) void emb_rank_kernel(const IDX* __restrict__ i
     if (i < n) rank[i] = hist[tok[k]] + lr[k];
   }
 }
-// Exclusive prefix sum of count[0 .. V) into cursor, one workgroup: each thread sums a contiguous slice, one scan over the
-// 1024 slice totals, each thread writes its slice.
-__global__ __launch_bounds__(1024) void emb_scan_slices_kernel(const int* __restrict__ count, int* __restrict__ cursor, int V) {
+// Exclusive prefix sum of count[0 .. V) into cursor, one workgroup per tile of 1024 counters and no dependency between
+// workgroups: each first adds up everything before its tile (at most 128 KB, loads eight tiles at a time), then scans its own.
+__global__ __launch_bounds__(1024) void emb_scan_tiles_kernel(const int* __restrict__ count, int* __restrict__ cursor, int V) {
   __shared__ int wsum[16];
+  __shared__ int wtot[16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int per = (V + 1023) / 1024, lo = tid * per, hi = min(V, lo + per);
-  int tot = 0;
-  for (int v = lo; v < hi; ++v) tot += count[v];
-  int x = tot;
+  const int lo = blockIdx.x * 1024;
+  int s = 0;
+  for (int base = 0; base < lo; base += 8 * 1024) {
+    int v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = base + j * 1024 + tid;
+      v[j] = i < lo ? count[i] : 0;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s += v[j];
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+  const int i = lo + tid;
+  const int c = i < V ? count[i] : 0;
+  int x = c;
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) {
     int y = __shfl_up(x, o, 64);
     if (lane >= o) x += y;
   }
   if (lane == 63) wsum[wave] = x;
+  if (lane == 0) wtot[wave] = s;
   __syncthreads();
-  int before = x - tot;
+  int before = 0;
+  for (int w = 0; w < 16; ++w) before += wtot[w];
   for (int w = 0; w < wave; ++w) before += wsum[w];
-  for (int v = lo; v < hi; ++v) {
-    cursor[v] = before;
-    before += count[v];
-  }
+  if (i < V) cursor[i] = before + x - c;
 }
 template <typename IDX>
 __global__ __launch_bounds__(256) void emb_scatter_kernel(const IDX* __restrict__ idx, const int* __restrict__ cursor,
@@ -646,7 +659,7 @@ extern "C" int tfb_embedding_bwd_grouped(const void* idx, int idx64, const void*
       return TFB_ERR_LAUNCH;
     if (idx64) hipLaunchKernelGGL(emb_rank_kernel<long>, dim3(nw), dim3(256), hist_bytes, s, (const long*)idx, count, rank, n, V);
     else hipLaunchKernelGGL(emb_rank_kernel<int>, dim3(nw), dim3(256), hist_bytes, s, (const int*)idx, count, rank, n, V);
-    hipLaunchKernelGGL(emb_scan_slices_kernel, dim3(1), dim3(1024), 0, s, count, cursor, V + 1);
+    hipLaunchKernelGGL(emb_scan_tiles_kernel, dim3((unsigned)((V + 1 + 1023) / 1024)), dim3(1024), 0, s, count, cursor, V + 1);
     if (idx64) hipLaunchKernelGGL(emb_scatter_kernel<long>, dim3(nb), dim3(256), 0, s, (const long*)idx, cursor, rank, order, n, V);
     else hipLaunchKernelGGL(emb_scatter_kernel<int>, dim3(nb), dim3(256), 0, s, (const int*)idx, cursor, rank, order, n, V);
   } else {
