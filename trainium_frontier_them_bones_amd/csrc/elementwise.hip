@@ -413,19 +413,27 @@ __global__ __launch_bounds__(256) void emb_scatter_kernel(const IDX* __restrict_
 // A workgroup sums EMB_SEG consecutive rows of the token-grouped order, thread t owning columns 8t .. 8t+7. A run of
 // equal tokens that lies inside the segment has a single owner and is added with plain loads/stores; the first and the
 // last run may continue in the neighbouring segments and use atomics.
-constexpr int EMB_SEG = 32;
+#ifndef TFB_EMB_SEG
+#define TFB_EMB_SEG 32
+#endif
+constexpr int EMB_SEG = TFB_EMB_SEG;
 template <typename IDX>
 __global__ __launch_bounds__(128) void emb_reduce_kernel(const IDX* __restrict__ idx, const int* __restrict__ order,
                                                         const bf16_t* __restrict__ dy, float* __restrict__ dw, long n, int C,
                                                         int V) {
   __shared__ int rows[EMB_SEG];
   __shared__ int toks[EMB_SEG];
+  __shared__ int edge[2];  // the tokens of the rows just before and just after this segment (-1: none)
   const long pos0 = (long)blockIdx.x * EMB_SEG;
   const int cnt = (int)min((long)EMB_SEG, n - pos0);
   if (threadIdx.x < cnt) {
     const int r = order[pos0 + threadIdx.x];
     rows[threadIdx.x] = r;
     toks[threadIdx.x] = emb_bucket(idx[r], V);
+  } else if (threadIdx.x == EMB_SEG) {
+    edge[0] = pos0 > 0 ? emb_bucket(idx[order[pos0 - 1]], V) : -1;
+  } else if (threadIdx.x == EMB_SEG + 1) {
+    edge[1] = pos0 + cnt < n ? emb_bucket(idx[order[pos0 + cnt]], V) : -1;
   }
   __syncthreads();
   const int c = (blockIdx.y * 128 + threadIdx.x) * 8;
@@ -443,7 +451,8 @@ __global__ __launch_bounds__(128) void emb_reduce_kernel(const IDX* __restrict__
       float* d = dw + (long)toks[i] * C + c;
       if (toks[i] == V) {
         // the bucket of out-of-range ids: dropped
-      } else if (run_start == 0 || i + 1 == cnt) {
+      } else if ((run_start == 0 && edge[0] == toks[i]) || (i + 1 == cnt && edge[1] == toks[i])) {
+        // the token's run goes on in a neighbouring segment: another workgroup adds to the same row
 #pragma unroll
         for (int k = 0; k < 8; ++k) atomicAdd(d + k, acc[k]);
       } else {
