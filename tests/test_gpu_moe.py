@@ -99,9 +99,11 @@ def test_moe_layer_forward_backward(dev, shape, topk, skew):
     assert rel_l2(rd.grad, ro.grad) < 2e-2
 
 
-def test_moe_starved_expert_and_ragged_token_count(dev):
+@pytest.mark.parametrize("experts", ["fp8", "fp8 weight gradients too", "bf16"])
+def test_moe_starved_expert_and_ragged_token_count(dev, experts):
     """One expert's router bias keeps every token away from it (empty segment, zero weight gradient, finite scales) and the
-    token count is not a multiple of the 64-token counting groups."""
+    token count is not a multiple of the 64-token counting groups; with the experts in fp8, with their weight gradients in
+    fp8 as well, and in bf16."""
     from oracle import moe as O
     from trainium_frontier_them_bones_amd import autograd as A
     from trainium_frontier_them_bones_amd import ops
@@ -109,8 +111,10 @@ def test_moe_starved_expert_and_ragged_token_count(dev):
     h, router, wf, wp, bias = _layer(11, N, d, Fd, E)
     bias[2] = -1e4
     hd, rd, wfd, wpd = (t.to(dev).requires_grad_(True) for t in (h, router, wf, wp))
-    st = A.Moe8State()
-    st.refresh(wfd, wpd)
+    st = None
+    if experts != "bf16":
+        st = A.Moe8State(dw_fp8=experts != "fp8")
+        st.refresh(wfd, wpd)
     out = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, st, 2, bias.to(dev))
     g = torch.randn(N, d, generator=torch.Generator().manual_seed(5)).bfloat16()
     out.backward(g.to(dev))
@@ -119,7 +123,7 @@ def test_moe_starved_expert_and_ragged_token_count(dev):
     assert int(tab["cnt"][2]) == 0 and int(tab["cnt"].sum()) == 2 * N
     assert int(tab["seg"][3]) == int(tab["seg"][2])                              # an empty segment takes no rows
     ho, ro, wfo, wpo = (t.clone().requires_grad_(True) for t in (h, router, wf, wp))
-    oo, _ = O.moe_forward(ho, ro, wfo, wpo, 2, bias)
+    oo, _ = O.moe_forward(ho, ro, wfo, wpo, 2, bias, fp8=experts != "bf16", dw_fp8=experts == "fp8 weight gradients too")
     oo.backward(g)
     assert rel_l2(out, oo) < 2e-2 and rel_l2(hd.grad, ho.grad) < 2e-2 and rel_l2(rd.grad, ro.grad) < 2e-2
     assert float(wfd.grad[2].float().abs().max()) == 0.0 and float(wpd.grad[2].float().abs().max()) == 0.0
@@ -397,8 +401,9 @@ def test_capacity_rejects_a_sequence_that_is_not_whole_wavefronts(dev):
         ops.moe_tables(idx, 4, 100, 8)
 
 
-def test_moe_layer_with_capacity_forward_backward(dev):
-    """The whole routed layer with a capacity that drops about a sixth of the assignments, against the oracle's restatement
+@pytest.mark.parametrize("experts", ["fp8", "fp8 weight gradients too", "bf16"])
+def test_moe_layer_with_capacity_forward_backward(dev, experts):
+    """The whole routed layer (experts in fp8, with fp8 weight gradients, in bf16) with a capacity that drops about a sixth of the assignments, against the oracle's restatement
     of the reference's keep rule: output, input / router / expert-weight gradients, and the load shares of the auxiliary term
     (made of EVERY assignment, kept or not: round2/source/train.py:10786 takes them from the masks)."""
     from oracle import moe as O
@@ -408,13 +413,16 @@ def test_moe_layer_with_capacity_forward_backward(dev):
     h, router, wf, wp, bias = _layer(22, b * t, d, Fd, E, 2.0)
     h = h.reshape(b, t, d)
     hd, rd, wfd, wpd = (x.to(dev).requires_grad_(True) for x in (h, router, wf, wp))
-    st = A.Moe8State()
-    st.refresh(wfd, wpd)
+    st = None
+    if experts != "bf16":
+        st = A.Moe8State(dw_fp8=experts != "fp8")
+        st.refresh(wfd, wpd)
     out, aux, terms = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, st, topk, bias.to(dev), (0.01, 0.001), cap)
     g = torch.randn(b, t, d, generator=torch.Generator().manual_seed(3)).bfloat16()
     (out.float() * g.to(dev).float()).sum().add(aux).backward()
     ho, ro, wfo, wpo = (x.clone().requires_grad_(True) for x in (h, router, wf, wp))
-    oo, info = O.moe_forward(ho, ro, wfo, wpo, topk, bias, capacity=cap)
+    oo, info = O.moe_forward(ho, ro, wfo, wpo, topk, bias, capacity=cap, fp8=experts != "bf16",
+                             dw_fp8=experts == "fp8 weight gradients too")
     # the comparison needs the two routers to agree on every pick (a different pick would move every later position of
     # its sequence); the kernel's picks are held to the reference's rule bit for bit in test_routing_tables_bit_exact
     _, idx, _, _ = ops.moe_route(hd.detach().reshape(-1, d), rd.detach(), topk, bias.to(dev))
