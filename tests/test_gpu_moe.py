@@ -297,12 +297,12 @@ def test_moe_per_sequence_balance_term(dev, topk):
         ops.moe_aux_seq_fwd(p, idx, 384, topk)                          # 2048 tokens are not whole sequences of 384
 
 
-@pytest.mark.parametrize("skew", [0.0, 2.0])
-def test_moe_config5_full_size_backward(dev, skew):
+@pytest.mark.parametrize("skew,dw_fp8", [(0.0, False), (2.0, False), (2.0, True)])
+def test_moe_config5_full_size_backward(dev, skew, dw_fp8):
     """Configuration 5 at full size, forward AND backward (16384 tokens, d 1024, 8 experts top-2, FFN 2816; balanced and
     with +2.0 on two experts' logits), against the oracle on parts it finishes in seconds: (1) one expert's whole row
     segment (its activations, input gradient and BOTH weight gradients: the ragged token-contraction GEMMs over
-    thousands of rows), (2) the input gradient of 512 tokens routed to the most frequent expert pair, through autograd
+    thousands of rows, in bf16 and, dw_fp8, in fp8 from the bytes the other GEMMs multiplied), (2) the input gradient of 512 tokens routed to the most frequent expert pair, through autograd
     of the oracle layer on those tokens with the backward scales taken from the full layer's per-expert amax."""
     from oracle import mlp8 as O8
     from oracle import moe as O
@@ -312,10 +312,10 @@ def test_moe_config5_full_size_backward(dev, skew):
     h, router, wf, wp, bias = _layer(5, N, d, Fd, E, skew)
     dout = torch.randn(N, d, generator=torch.Generator().manual_seed(6)).bfloat16()
     hd, rd, wfd, wpd = (t.to(dev).requires_grad_(True) for t in (h, router, wf, wp))
-    st = A.Moe8State()
+    st = A.Moe8State(dw_fp8=dw_fp8)
     st.refresh(wfd, wpd)
     b = bias.to(dev) if skew else None
-    print("config 5 full size fwd+bwd, skew %.1f" % skew, flush=True)
+    print("config 5 full size fwd+bwd, skew %.1f, fp8 weight gradients %s" % (skew, dw_fp8), flush=True)
     out = A.MoeMlp8Fn.apply(hd, rd, wfd, wpd, st, 2, b)
     out.backward(dout.to(dev))
     for t in (out, hd.grad, rd.grad, wfd.grad, wpd.grad):
@@ -340,8 +340,9 @@ def test_moe_config5_full_size_backward(dev, skew):
     xe, ge = h[tok[rows]], dys[rows]
     row = O8.forward_scales(wf[e], wp[e])
     ye, re = O8.forward(xe, wf[e], wp[e], row)
-    dxe, he, dpe = O8.backward(ge, re, wf[e], wp[e], O8.backward_scales(ge, row, amax[e]))
-    dwf, dwp = O8.weight_grads(ge, xe, he, dpe)
+    row_b = O8.backward_scales(ge, row, amax[e])
+    dxe, he, dpe = O8.backward(ge, re, wf[e], wp[e], row_b)
+    dwf, dwp = O8.weight_grads_fp8(xe, ge, he, dpe, row_b) if dw_fp8 else O8.weight_grads(ge, xe, he, dpe)
     assert rel_l2(wfd.grad[e], dwf) < 2e-2 and rel_l2(wpd.grad[e], dwp) < 2e-2
     assert rows.numel() > (3000 if not skew else 5000)                    # thousands of rows: the ragged long contraction
     # (2) 512 tokens of the most frequent (unordered) expert pair, input gradient through the whole layer's backward
