@@ -476,13 +476,19 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   auto chunk_row = [&](int k) { return 2 * (((lane >> 3) + k * 8) / (EPI_CPR / 4)) + ((lane >> 2) & 1); };
   auto chunk_col = [&](int k) { return (4 * (((lane >> 3) + k * 8) % (EPI_CPR / 4)) + (lane & 3)) * 8; };
   [[maybe_unused]] typename prefetch_type<Epi>::type pre[TQ][EPI_NK];
-  if constexpr (kPrefetch) {
+  auto prefetch_epilogue = [&]() {
+    if constexpr (kPrefetch) {
 #pragma unroll
-    for (int j = 0; j < TQ; ++j)
+      for (int j = 0; j < TQ; ++j)
 #pragma unroll
-      for (int k = 0; k < EPI_NK; ++k)
-        pre[j][k] = epi.prefetch((int)p0 + wp * (TP * 32) + chunk_col(k), (int)q0 + wq * (TQ * 32) + j * 32 + chunk_row(k));
-  }
+        for (int k = 0; k < EPI_NK; ++k)
+          pre[j][k] = epi.prefetch((int)p0 + wp * (TP * 32) + chunk_col(k), (int)q0 + wq * (TQ * 32) + j * 32 + chunk_row(k));
+    }
+  };
+#ifndef TFB_PREFETCH_AFTER_FIRST
+#define TFB_PREFETCH_AFTER_FIRST 1
+#endif
+  if (!TFB_PREFETCH_AFTER_FIRST) prefetch_epilogue();
 
   auto compute = [&](const uint8_t* buf) {
     const uint8_t* sp = buf;
@@ -523,6 +529,9 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   {
     __syncthreads();
     if constexpr (kProbe) ph_first = __builtin_readcyclecounter();
+    // The epilogue's operands are requested here, behind the first k-tile's barrier: vector loads return in order, so
+    // asked for before it they made that barrier wait for a stream from HBM; now they fly under the first k-tile's MFMAs.
+    if (TFB_PREFETCH_AFTER_FIRST) prefetch_epilogue();
     for (int t = 0; t + 2 <= nkt; t += 2) {
       issue(buf1, t + 1);
       compute(buf0);
