@@ -754,3 +754,28 @@ def test_gemm_phase_probe_is_the_library_kernel(ops, dev):
     assert cyc.shape == (8 * 3, 4) and bool((cyc > 0).all())
     assert bool((cyc[:, 0] < cyc[:, 1]).all())          # the first load is issued before the first k-tile is there
 
+
+@pytest.mark.parametrize("V", [32768, 50304])
+def test_embedding_backward_at_full_size_on_a_zipf_batch(ops, dev, V):
+    """The grouped embedding backward at the benchmark's size (32768 rows of 768, Zipf(1.1) ids): with the vocabulary's
+    counters in LDS (V = 32768: per-workgroup histogram, placement without atomics) and on the per-row path a larger
+    vocabulary takes (V = 50304: its counters do not fit), both against index_add_ in fp32 and against the plain atomic
+    entry point; int64 and int32 ids, ids outside [0, V) dropped."""
+    from trainium_frontier_them_bones_amd.model import zipf_tokens
+    idx, _ = zipf_tokens(16, 2048, V, seed=9)
+    idx = idx.reshape(-1).clone()
+    idx[5::97] = V + 3
+    idx[11::89] = -1
+    ok = (idx >= 0) & (idx < V)
+    g = torch.Generator().manual_seed(2)
+    dy = torch.randn(idx.numel(), 768, generator=g).bfloat16()
+    want = torch.zeros(V, 768).index_add_(0, idx[ok], dy.float()[ok])
+    for ids in (idx, idx.int()):
+        dw = ops.fill_f32_(torch.empty(V, 768, device=dev), 0.0)
+        ops.embedding_bwd(ids.to(dev), dy.to(dev), dw)
+        assert rel_l2(dw, want) < 1e-6
+    dwa = ops.fill_f32_(torch.empty(V, 768, device=dev), 0.0)
+    ops.embedding_bwd(idx.to(dev), dy.to(dev), dwa, grouped=False)
+    assert rel_l2(dwa, want) < 1e-6
+    assert int((want.abs().sum(1) > 0).sum()) > 3000 and int(torch.bincount(idx[ok]).max()) > 1000   # many tokens, one very hot
+
