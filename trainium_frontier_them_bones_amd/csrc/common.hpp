@@ -103,6 +103,20 @@ __device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, float d)
   return (uint32_t)w;
 }
 
+// Streaming accesses: a tensor written now and read again much later (or read once) goes past the L2's retention with the
+// non-temporal hint, so that it does not push out the tiles other workgroups re-read. Only for accesses that cover whole
+// 128-byte lines between the lanes of one instruction: on partial lines the hint bypasses the L2's write merging.
+// Each use is switched by a macro (default on) so that it can be measured alone.
+template <class T>
+__device__ __forceinline__ void tfb_store_nt(T* p, T v, bool on = true) {
+  if (on) __builtin_nontemporal_store(v, p);
+  else *p = v;
+}
+template <class T>
+__device__ __forceinline__ T tfb_load_nt(const T* p, bool on = true) {
+  return on ? __builtin_nontemporal_load(p) : *p;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
