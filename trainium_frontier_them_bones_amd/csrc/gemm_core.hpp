@@ -321,6 +321,10 @@ struct has_phase_probe : std::false_type {};
 template <class T>
 struct has_phase_probe<T, std::void_t<decltype(std::declval<const T&>().phase_cycles)>> : std::true_type {};
 
+// the residual a projection's store adds is read once by that kernel (output projection with the hint: 0.72 -> 0.70 ms per step)
+#ifndef TFB_NT_RES
+#define TFB_NT_RES 1
+#endif
 #ifndef TFB_STAGGER_SLEEPS
 #define TFB_STAGGER_SLEEPS 2
 #endif
@@ -681,7 +685,7 @@ struct EpiStoreRes {
   const bf16_t* res;
   long ld;  // elements, of both
   using pre_t = u32x4;
-  __device__ __forceinline__ pre_t prefetch(int p, int q) const { return *(const u32x4*)(res + (long)q * ld + p); }
+  __device__ __forceinline__ pre_t prefetch(int p, int q) const { return tfb_load_nt((const u32x4*)(res + (long)q * ld + p), TFB_NT_RES); }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const pre_t& r, int) const {
     float a[8], b[8];
     unpack8bf(pack8bf(v), a);

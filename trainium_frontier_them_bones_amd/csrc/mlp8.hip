@@ -406,7 +406,7 @@ struct EpiDescaleRes {
     }
     return e;
   }
-  __device__ __forceinline__ pre_t prefetch(int p, int q) const { return *(const u32x4*)(res + (long)q * ld + p); }
+  __device__ __forceinline__ pre_t prefetch(int p, int q) const { return tfb_load_nt((const u32x4*)(res + (long)q * ld + p), TFB_NT_RES); }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const pre_t& rv, int) const {
     float r[8], a[8], b[8];
 #pragma unroll
