@@ -1012,7 +1012,7 @@ struct EpiRelu2 {  // pre = bf16(acc); r = max(pre, 0); h = bf16(r r)
       hb[i >> 1] = round2_bf(a, b);
     }
     const long off = (long)q * F + p;
-    *(u32x4*)(r + off) = rb;
+    __builtin_nontemporal_store(rb, (u32x4*)(r + off));   // (kept for the backward only, as the fp8 experts' r)
     *(u32x4*)(h + off) = hb;
   }
 };
@@ -1021,7 +1021,7 @@ struct EpiDpre {  // dpre = bf16(bf16(acc) (2 r)): the gradient through h = r^2 
   bf16_t* dpre;
   long F;
   typedef u32x4 pre_t;
-  __device__ __forceinline__ pre_t prefetch(int p, int q) const { return *(const u32x4*)(r + (long)q * F + p); }
+  __device__ __forceinline__ pre_t prefetch(int p, int q) const { return __builtin_nontemporal_load((const u32x4*)(r + (long)q * F + p)); }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const pre_t& rv, int) const {
     float rr[8];
     unpack8bf(rv, rr);
