@@ -392,6 +392,13 @@ int tfb_moe_combine(const void* ys, const void* slot, const void* gate, void* ou
 int tfb_moe_combine_bwd(const void* dout, const void* ys, const void* tok, const void* ksel, const void* gate, void* dys,
                         void* dgate, long rmax, int d, int topk, void* stream);
 
+/* tfb_moe_combine_bwd that also leaves rowmax fp32 [rmax] = max |dys[row]| of the rounded values (0 for a padding row), so
+ * that the experts' backward scales (tfb_moe_backward_scales_rowmax) need no pass of their own over dys.
+ * Replaces MoeCombine2.backward (round2/source/train.py:10678-10688) + the amax(dy) of backward_scales
+ * (round2/source/kernels/nki_mlp_fused8.py:803). */
+int tfb_moe_combine_bwd_rowmax(const void* dout, const void* ys, const void* tok, const void* ksel, const void* gate, void* dys,
+                               void* dgate, void* rowmax, long rmax, int d, int topk, void* stream);
+
 /* dlogits fp32 [N][E] from dgate through the renormalisation and the softmax; dh bf16 [N][d] = dxs[slot_1] + dxs[slot_2] +
  * dlogits Wr; dwr fp32 [E][d] (+)= dlogits^T h, summed over 64 token chunks in a fixed order through scratch fp32 [64][E][d].
  * Replaces MoeDispatch2.backward (round2/source/train.py:10662-10666) and autograd through moe_route / the router matmul. */
@@ -428,6 +435,12 @@ int tfb_moe_route_bwd_aux_seq(const void* dgate, const void* p, const void* idx,
  * (backward_scales per expert, round2/source/kernels/nki_mlp_fused8.py:803-813). amax_scratch: uint32 [E]. */
 int tfb_moe_backward_scales(const void* dys, const void* tile_expert, const void* rows_in, void* rows_out, void* amax_scratch,
                             long rmax, int d, int E, void* stream);
+
+/* The same rows from rowmax fp32 [rmax] (tfb_moe_combine_bwd_rowmax) and seg int32 [E + 1] (tfb_moe_tables): expert e's amax
+ * is the maximum over rows seg[e] .. seg[e + 1]; bit-equal to tfb_moe_backward_scales on the same dys; d as there.
+ * Replaces backward_scales per expert (round2/source/kernels/nki_mlp_fused8.py:803-813). */
+int tfb_moe_backward_scales_rowmax(const void* rowmax, const void* seg, const void* rows_in, void* rows_out, int d, int E,
+                                   void* stream);
 
 /* out8 = fp8(x * rows[expert of the row's tile][col]); fmt 0 e4m3, 1 e5m2; padding tiles give zero bytes. */
 int tfb_moe_quant(const void* x, const void* tile_expert, const void* rows, int col, int fmt, void* out8, long rmax, int d,

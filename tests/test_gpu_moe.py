@@ -74,6 +74,54 @@ def test_routing_exact_ties_go_to_the_lower_index(dev, topk):
     assert (ic == io).all(1).float().mean().item() > 0.999
 
 
+@pytest.mark.parametrize("N,d,E", [(1003, 768, 5), (7, 64, 2), (4096, 1024, 8), (1000, 520, 11)])
+@pytest.mark.parametrize("topk", [2, 1])
+def test_routing_ragged_shapes(dev, N, d, E, topk):
+    """Token counts that are not whole groups of eight, widths that leave lanes without columns (768, 520, 64) and expert
+    counts below eight (and above, which take the one-token kernel): logits against the oracle, selections and gates by the
+    reference's rule on the kernel's own probabilities, bit for bit."""
+    from oracle import moe as O
+    from trainium_frontier_them_bones_amd import ops
+    h, router, _, _, _ = _layer(21, N, d, 64, E)
+    bias = 0.1 * torch.randn(E, generator=torch.Generator().manual_seed(3))
+    p, idx, gate, logits = ops.moe_route(h.to(dev), router.to(dev), topk, bias.to(dev), want_logits=True)
+    po, _, _, lo = O.route(h, router, topk, bias)
+    assert rel_l2(logits, lo) < 1e-5 and rel_l2(p, po) < 1e-5
+    isel, gsel = O.select(p.cpu(), topk)
+    assert torch.equal(idx.cpu().long(), isel) and torch.equal(gate.cpu(), gsel)
+    assert rel_l2(p, torch.softmax(logits.cpu(), dim=-1)) < 1e-6
+    p2, idx2, gate2, _ = ops.moe_route(h.to(dev), router.to(dev), topk, bias.to(dev))          # without the logits output
+    assert torch.equal(p2, p) and torch.equal(idx2, idx) and torch.equal(gate2, gate)
+
+
+@pytest.mark.parametrize("skew", [0.0, 2.0])
+def test_backward_scales_from_the_combine_backward_row_maxima(dev, skew):
+    """The experts' amax(dys) taken inside the combine backward (row maxima, then one maximum per segment) gives the scale
+    rows of the separate pass over dys bit for bit, with a starved expert and padding rows in the buffer."""
+    from trainium_frontier_them_bones_amd import autograd as A
+    from trainium_frontier_them_bones_amd import ops
+    N, d, Fd, E = 1000, 256, 512, 8
+    h, router, wf, wp, bias = _layer(31, N, d, Fd, E, skew)
+    bias[5] = -1e4
+    hd, rd = h.to(dev), router.to(dev)
+    st = A.Moe8State()
+    st.refresh(wf.to(dev), wp.to(dev))
+    _, idx, gate, _ = ops.moe_route(hd, rd, 2, bias.to(dev))
+    tab = ops.moe_tables(idx, E)
+    rmax = tab["tok"].shape[0]
+    g = torch.Generator().manual_seed(7)
+    ys = torch.randn(rmax, d, generator=g).bfloat16().to(dev)
+    dout = (torch.randn(N, d, generator=g) * torch.logspace(-3, 2, N)[:, None]).bfloat16().to(dev)
+    dys, dgate = ops.moe_combine_bwd(dout, ys, tab, gate)
+    dys2, dgate2, rowmax = ops.moe_combine_bwd(dout, ys, tab, gate, want_rowmax=True)
+    assert torch.equal(dys, dys2) and torch.equal(dgate, dgate2)
+    assert torch.equal(rowmax, dys.float().abs().amax(1))
+    rows_a = ops.moe_backward_scales(dys, st.rows, tab)
+    rows_b = ops.moe_backward_scales_rowmax(rowmax, st.rows, tab, d)
+    assert torch.equal(rows_a, rows_b)
+    assert bool(torch.isfinite(rows_b).all()) and int(tab["cnt"][5]) == 0
+
+
 @pytest.mark.parametrize("shape,topk,skew", [((1024, 256, 512, 8), 2, 0.0), ((1024, 256, 512, 4), 1, 0.0),
                                               ((2048, 512, 768, 8), 2, 2.0)])
 def test_moe_layer_forward_backward(dev, shape, topk, skew):

@@ -85,6 +85,7 @@ SIGNATURES = {
     "tfb_moe_dw": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "tfb_moe_combine": [_vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_moe_combine_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_moe_combine_bwd_rowmax": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_moe_route_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _l, _i, _i, _i, _vp],
     "tfb_moe_route_bwd_aux": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _f, _f, _l, _i, _i, _i, _vp],
     "tfb_moe_aux_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
@@ -95,6 +96,7 @@ SIGNATURES = {
     "tfb_moe_aux_seq_fwd": [_vp, _vp, _vp, _vp, _vp, _l, _l, _i, _i, _vp],
     "tfb_moe_route_bwd_aux_seq": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _f, _f, _vp, _f, _l, _l, _i, _i, _i, _vp],
     "tfb_moe_backward_scales": [_vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_moe_backward_scales_rowmax": [_vp, _vp, _vp, _vp, _i, _i, _vp],
     "tfb_moe_quant": [_vp, _vp, _vp, _i, _i, _vp, _l, _i, _vp],
     "tfb_ns5_workspace_bytes": [_i, _i, _i],
     "tfb_ns5": [_vp, _vp, _fp, _vp, _vp, _i, _i, _i, _i, _vp, _l, _vp],

@@ -678,13 +678,15 @@ class MoeMlp8Fn(torch.autograd.Function):
         if gout is None:
             gout = torch.zeros(ctx.hshape, dtype=h2.dtype, device=h2.device)
         g2 = gout.reshape(-1, gout.shape[-1]).contiguous()
-        dys, dgate = ops.moe_combine_bwd(g2, ys, tab, gate)
         dw8 = st is not None and st.dw_fp8
+        if st is not None:   # the experts' amax(dys) rides the kernel that writes dys
+            dys, dgate, rowmax = ops.moe_combine_bwd(g2, ys, tab, gate, want_rowmax=True)
+            rows_b = ops.moe_backward_scales_rowmax(rowmax, st.rows, tab, dys.shape[1])
+        else:
+            dys, dgate = ops.moe_combine_bwd(g2, ys, tab, gate)
         if dw8:
-            rows_b = ops.moe_backward_scales(dys, st.rows, tab)
             dxs, dp8, hq8, dy8 = ops.moe_mlp8_bwd_q(dys, r, st.w8, rows_b, tab, st.e4m3_limit)
         elif st is not None:
-            rows_b = ops.moe_backward_scales(dys, st.rows, tab)
             dxs, dpre = ops.moe_mlp8_bwd(dys, r, st.w8, rows_b, tab)
         else:
             dxs, dpre = ops.moe_mlp_bwd(dys, r, w_fc.detach().to(bf16).contiguous(), w_proj.detach().to(bf16).contiguous(), tab)

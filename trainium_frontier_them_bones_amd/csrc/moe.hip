@@ -16,6 +16,11 @@
 namespace {
 
 constexpr int MAXE = 16;
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+#ifndef TFB_ROUTE_RESIDENT
+#define TFB_ROUTE_RESIDENT 1
+#endif
 
 __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
   u32x4 u = *(const u32x4*)p;
@@ -64,6 +69,73 @@ __device__ __forceinline__ float route_reduce(const float (&acc)[EP], int lane) 
 template <int EP>
 __device__ __forceinline__ int route_lane_of(int e) {
   return EP == 16 ? (e << 2) : (e << 3);
+}
+
+// One token's logits from the lanes' partial sums, then softmax, the first-maximum top-k and the gates; lane 0 stores.
+template <int EP>
+__device__ __forceinline__ void route_finish(const float (&acc)[EP], int lane, long n, long N, int E, int topk,
+                                             const float* __restrict__ bias, float* __restrict__ logits_out,
+                                             float* __restrict__ p_out, int* __restrict__ idx_out,
+                                             float* __restrict__ gate_out) {
+  float lg[EP];
+  float mx = -INFINITY;
+  if constexpr (EP <= 8) {
+    const float mine = route_reduce<EP>(acc, lane);
+#pragma unroll
+    for (int e = 0; e < EP; ++e) lg[e] = e < E ? __shfl(mine, route_lane_of<EP>(e), 64) + (bias ? bias[e] : 0.f) : 0.f;
+  } else {  // (the joint reduction of sixteen values measured slower than sixteen butterflies: 114 against 102 us)
+#pragma unroll
+    for (int e = 0; e < EP; ++e) lg[e] = e < E ? wave_sum(acc[e]) + (bias ? bias[e] : 0.f) : 0.f;
+  }
+#pragma unroll
+  for (int e = 0; e < EP; ++e)
+    if (e < E) mx = fmaxf(mx, lg[e]);
+  float p[EP], den = 0.f;
+#pragma unroll
+  for (int e = 0; e < EP; ++e) {
+    p[e] = e < E ? expf(lg[e] - mx) : 0.f;
+    den += p[e];
+  }
+  int i1 = 0, i2 = 0;
+  float v1 = -1.f, v2 = -1.f;
+#pragma unroll
+  for (int e = 0; e < EP; ++e) {
+    if (e < E) {
+      p[e] = p[e] / den;
+      if (p[e] > v1) {
+        v1 = p[e];
+        i1 = e;
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < EP; ++e) {
+    if (e < E && e != i1 && p[e] > v2) {
+      v2 = p[e];
+      i2 = e;
+    }
+  }
+  if (n >= N) return;
+  if (lane < E) {   // lane e stores expert e's probability and logit: one store instruction each instead of E
+    float pe = p[0], le = lg[0];
+#pragma unroll
+    for (int e = 1; e < EP; ++e) {
+      pe = lane == e ? p[e] : pe;
+      le = lane == e ? lg[e] : le;
+    }
+    p_out[n * E + lane] = pe;
+    if (logits_out) logits_out[n * E + lane] = le;
+  }
+  if (lane == 0) {
+    if (topk == 2) {
+      const float s = v1 + v2;
+      *(i32x2*)(idx_out + n * 2) = i32x2{i1, i2};
+      *(f32x2*)(gate_out + n * 2) = f32x2{v1 / s, v2 / s};
+    } else {
+      idx_out[n] = i1;
+      gate_out[n] = v1;
+    }
+  }
 }
 
 // TPW tokens per wavefront at a time (sharing one fetch of the router's weights) was measured at 2 and 4: slower than 1
@@ -118,60 +190,114 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const bf16_t* __restrict
 #pragma unroll
     for (int t = 0; t < TPW; ++t) {
       const long n = n0 + t;
-      float lg[EP];
-      float mx = -INFINITY;
-      if constexpr (EP <= 8) {
-        const float mine = route_reduce<EP>(acc[t], lane);
+      route_finish<EP>(acc[t], lane, n, N, E, topk, bias, logits_out, p_out, idx_out, gate_out);
+    }
+  }
+}
+
+// Eight tokens per wavefront, finished one (token, expert) pair per lane. The 64 per-lane partial sums (8 tokens x 8
+// experts) go through ONE joint butterfly (63 shuffles for eight tokens; value t * 8 + e ends up complete in lane t * 8 + e,
+// added in the order of a butterfly sum, so a token's logits are the bits the one-token kernel above gives), and the
+// softmax, the first-maximum top-k and the gates then run once over the wavefront with a token's eight experts in eight
+// neighbouring lanes, instead of once per token with every lane repeating the same arithmetic. A chunk of the router's
+// weights is fetched once per eight tokens. 16384 tokens of d = 1024: 36 -> 15 us. E <= 8.
+template <int HALF>
+__device__ __forceinline__ void route_fold(float (&v)[64], int lane) {   // a lane keeps HALF of its 2 HALF values, its partner (lane ^ HALF) the others
+  const bool hi = (lane & HALF) != 0;
 #pragma unroll
-        for (int e = 0; e < EP; ++e) lg[e] = e < E ? __shfl(mine, route_lane_of<EP>(e), 64) + (bias ? bias[e] : 0.f) : 0.f;
-      } else {  // (the joint reduction of sixteen values measured slower than sixteen butterflies: 114 against 102 us)
+  for (int j = 0; j < HALF; ++j) {
+    const float keep = hi ? v[HALF + j] : v[j], send = hi ? v[j] : v[HALF + j];
+    v[j] = keep + __shfl_xor(send, HALF, 64);
+  }
+}
+__device__ __forceinline__ float route_reduce64(float (&v)[64], int lane) {
+  route_fold<32>(v, lane);
+  route_fold<16>(v, lane);
+  route_fold<8>(v, lane);
+  route_fold<4>(v, lane);
+  route_fold<2>(v, lane);
+  route_fold<1>(v, lane);
+  return v[0];
+}
+
+__global__ __launch_bounds__(256) void moe_route8_kernel(const bf16_t* __restrict__ h, const float* __restrict__ wr,
+                                                        const float* __restrict__ bias, float* __restrict__ logits_out,
+                                                        float* __restrict__ p_out, int* __restrict__ idx_out,
+                                                        float* __restrict__ gate_out, long N, int d, int E, int topk) {
+  const int lane = threadIdx.x & 63;
+  const long n0 = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 8;
+  if (n0 >= N) return;
+  float acc[64];
 #pragma unroll
-        for (int e = 0; e < EP; ++e) lg[e] = e < E ? wave_sum(acc[t][e]) + (bias ? bias[e] : 0.f) : 0.f;
+  for (int i = 0; i < 64; ++i) acc[i] = 0.f;
+  for (int c = lane * 8; c < d; c += 512) {
+    u32x4 raw[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) raw[t] = *(const u32x4*)(h + (n0 + t < N ? n0 + t : N - 1) * d + c);  // (a tail re-reads the last token)
+    f32x4 w0[8], w1[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {   // an expert beyond E re-reads the last one's weights; its sums are never used
+      const float* w = wr + (long)(e < E ? e : E - 1) * d + c;
+      w0[e] = *(const f32x4*)w;
+      w1[e] = *(const f32x4*)(w + 4);
+    }
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      float x[8];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        x[2 * k] = bflo(raw[t][k]);
+        x[2 * k + 1] = bfhi(raw[t][k]);
       }
 #pragma unroll
-      for (int e = 0; e < EP; ++e)
-        if (e < E) mx = fmaxf(mx, lg[e]);
-      float p[EP], den = 0.f;
+      for (int e = 0; e < 8; ++e)
+        acc[t * 8 + e] += x[0] * w0[e][0] + x[1] * w0[e][1] + x[2] * w0[e][2] + x[3] * w0[e][3] + x[4] * w1[e][0] +
+                          x[5] * w1[e][1] + x[6] * w1[e][2] + x[7] * w1[e][3];
+    }
+  }
+  const int e = lane & 7;
+  const long n = n0 + (lane >> 3);
+  const bool live = e < E;
+  const float lg = route_reduce64(acc, lane) + (bias && live ? bias[e] : 0.f);
+  float mx = live ? lg : -INFINITY;
 #pragma unroll
-      for (int e = 0; e < EP; ++e) {
-        p[e] = e < E ? expf(lg[e] - mx) : 0.f;
-        den += p[e];
-      }
-      int i1 = 0, i2 = 0;
-      float v1 = -1.f, v2 = -1.f;
+  for (int o = 1; o < 8; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  float p = live ? expf(lg - mx) : 0.f;
+  float den = p;
 #pragma unroll
-      for (int e = 0; e < EP; ++e) {
-        if (e < E) {
-          p[e] = p[e] / den;
-          if (p[e] > v1) {
-            v1 = p[e];
-            i1 = e;
-          }
-        }
-      }
+  for (int o = 1; o < 8; o <<= 1) den += __shfl_xor(den, o, 64);
+  p = p / den;
+  // first maximum over the token's eight lanes: the larger value wins, equal values go to the lower expert
+  auto best_of = [&](float v, int i, float& bv, int& bi) {
+    bv = v;
+    bi = i;
 #pragma unroll
-      for (int e = 0; e < EP; ++e) {
-        if (e < E && e != i1 && p[e] > v2) {
-          v2 = p[e];
-          i2 = e;
-        }
+    for (int o = 1; o < 8; o <<= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
       }
-      if (lane == 0 && n < N) {
-        for (int e = 0; e < E; ++e) {
-          p_out[n * E + e] = p[e];
-          if (logits_out) logits_out[n * E + e] = lg[e];
-        }
-        if (topk == 2) {
-          const float s = v1 + v2;
-          idx_out[n * 2] = i1;
-          idx_out[n * 2 + 1] = i2;
-          gate_out[n * 2] = v1 / s;
-          gate_out[n * 2 + 1] = v2 / s;
-        } else {
-          idx_out[n] = i1;
-          gate_out[n] = v1;
-        }
-      }
+    }
+  };
+  float v1, v2;
+  int i1, i2;
+  best_of(live ? p : -1.f, e, v1, i1);
+  best_of(live && e != i1 ? p : -1.f, e, v2, i2);
+  if (n >= N) return;
+  if (live) {
+    p_out[n * E + e] = p;
+    if (logits_out) logits_out[n * E + e] = lg;
+  }
+  if (e == 0) {
+    if (topk == 2) {
+      const float s = v1 + v2;
+      *(i32x2*)(idx_out + n * 2) = i32x2{i1, i2};
+      *(f32x2*)(gate_out + n * 2) = f32x2{v1 / s, v2 / s};
+    } else {
+      idx_out[n] = i1;
+      gate_out[n] = v1;
     }
   }
 }
@@ -364,33 +490,45 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const bf16_t* __restri
 }
 
 // One wavefront per slot row: dys[row] = bf16(bf16(g_k) dout[tok]); dgate[tok][k] = bf16(sum_d dout[tok] ys[row]).
+// ROWMAX: rowmax[row] = max |dys[row]| of the rounded values (0 for a padding row), from which the experts' backward scales
+// are taken without another pass over dys.
+template <bool ROWMAX>
 __global__ __launch_bounds__(256) void moe_combine_bwd_kernel(const bf16_t* __restrict__ dout, const bf16_t* __restrict__ ys,
                                                              const int* __restrict__ tok, const int* __restrict__ ksel,
                                                              const float* __restrict__ gate, bf16_t* __restrict__ dys,
-                                                             float* __restrict__ dgate, long rmax, int d, int topk) {
+                                                             float* __restrict__ dgate, float* __restrict__ rowmax, long rmax,
+                                                             int d, int topk) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (long row = (long)blockIdx.x * 4 + wave; row < rmax; row += (long)gridDim.x * 4) {
     const int t = tok[row];
     if (t < 0) {
       for (int c = lane * 8; c < d; c += 512) *(u32x4*)(dys + row * d + c) = u32x4{0, 0, 0, 0};
+      if (ROWMAX && lane == 0) rowmax[row] = 0.f;
       continue;
     }
     const int k = ksel[row];
     const float g = round_bf(gate[(long)t * topk + k]);
-    float dot = 0.f;
+    float dot = 0.f, m = 0.f;
     for (int c = lane * 8; c < d; c += 512) {
-      float go[8], y[8], r[8];
+      float go[8], y[8];
       load8(dout + (long)t * d + c, go);
       load8(ys + row * d + c, y);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        r[j] = g * go[j];
-        dot += go[j] * y[j];
+      for (int j = 0; j < 8; ++j) dot += go[j] * y[j];
+      const u32x4 u = {pack2bf(g * go[0], g * go[1]), pack2bf(g * go[2], g * go[3]), pack2bf(g * go[4], g * go[5]),
+                       pack2bf(g * go[6], g * go[7])};
+      *(u32x4*)(dys + row * d + c) = u;
+      if (ROWMAX) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) m = fmaxf(m, fmaxf(fabsf(bflo(u[j])), fabsf(bfhi(u[j]))));
       }
-      store8(dys + row * d + c, r);
     }
     dot = wave_sum(dot);
-    if (lane == 0) dgate[(long)t * topk + k] = round_bf(dot);
+    if (ROWMAX) m = wave_max(m);
+    if (lane == 0) {
+      dgate[(long)t * topk + k] = round_bf(dot);
+      if (ROWMAX) rowmax[row] = m;
+    }
   }
 }
 
@@ -597,9 +735,13 @@ __global__ __launch_bounds__(256) void moe_dispatch_bwd_kernel(const bf16_t* __r
 // and the y-th chunk of the tokens (32 row lanes stride over it) and leaves its sums in part[y][e][c]; the finish adds the
 // chunks in order. DWR_CHUNKS chunks at most: part is fp32 [DWR_CHUNKS][E][d].
 constexpr int DWR_CHUNKS = 64;
+#ifndef DWR_WANT
+#define DWR_WANT 0
+#endif
 __global__ __launch_bounds__(256) void moe_dwr_partial_kernel(const float* __restrict__ dlogits, const bf16_t* __restrict__ h,
                                                              float* __restrict__ part, long N, long chunk, int d, int E) {
-  __shared__ float red[32][8][9];
+  __shared__ __align__(16) float red[4][8][64];
+  __shared__ __align__(16) float gs[256][8];
   const int cl = threadIdx.x & 7, rl = threadIdx.x >> 3;
   const int c = blockIdx.x * 64 + cl * 8;
   const long n0 = blockIdx.y * chunk, n1 = n0 + chunk < N ? n0 + chunk : N;
@@ -609,28 +751,66 @@ __global__ __launch_bounds__(256) void moe_dwr_partial_kernel(const float* __res
     for (int e = 0; e < 8; ++e)
 #pragma unroll
       for (int k = 0; k < 8; ++k) acc[e][k] = 0.f;
-    for (long n = n0 + rl; n < n1; n += 32) {
-      float x[8];
-      load8(h + n * d + c, x);
+    // 256 tokens at a time: their dlogits go to LDS (so no registers wait for them) while all eight of a row lane's rows of
+    // h are in flight together; 16384 tokens are one such round per workgroup (one row at a time it was eight dependent
+    // round trips to memory, 28 us for 16384 x 1024)
+    for (long nb = n0; nb < n1; nb += 256) {
+      __syncthreads();   // (the previous round's dlogits have been read)
+      {
+        const long n = nb + threadIdx.x;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        if (e0 + e < E) {
-          const float g = dlogits[n * E + e0 + e];
+        for (int e = 0; e < 8; ++e) gs[threadIdx.x][e] = n < n1 && e0 + e < E ? dlogits[n * E + e0 + e] : 0.f;
+      }
+      u32x4 raw[8];
 #pragma unroll
-          for (int k = 0; k < 8; ++k) acc[e][k] += g * x[k];
+      for (int j = 0; j < 8; ++j) {
+        const long nj = nb + rl + 32 * j;
+        raw[j] = *(const u32x4*)(h + (nj < n1 ? nj : n1 - 1) * d + c);
+      }
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (nb + rl + 32 * j < n1) {
+          const f32x4 g0 = *(const f32x4*)&gs[rl + 32 * j][0], g1 = *(const f32x4*)&gs[rl + 32 * j][4];
+          const float g[8] = {g0[0], g0[1], g0[2], g0[3], g1[0], g1[1], g1[2], g1[3]};
+          float x[8];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            x[2 * k] = bflo(raw[j][k]);
+            x[2 * k + 1] = bfhi(raw[j][k]);
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+#pragma unroll
+            for (int k = 0; k < 8; ++k) acc[e][k] += g[e] * x[k];
         }
       }
     }
+    // the wavefront's eight row lanes first, by the joint butterfly over lane bits 3..5 (56 shuffles; the lane of row-lane
+    // index e is left with expert e's eight columns), then the four wavefronts through LDS: one barrier instead of sixteen
+    float v[64];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      __syncthreads();
+    for (int e = 0; e < 8; ++e)
 #pragma unroll
-      for (int k = 0; k < 8; ++k) red[rl][cl][k] = acc[e][k];
-      __syncthreads();
-      if (rl < 8 && e0 + e < E) {   // row lane rl adds column k = rl of this thread's eight
-        float s = 0.f;
-        for (int r = 0; r < 32; ++r) s += red[r][cl][rl];
-        part[((long)blockIdx.y * E + e0 + e) * d + c + rl] = s;
+      for (int k = 0; k < 8; ++k) v[e * 8 + k] = acc[e][k];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    route_fold<32>(v, lane);
+    route_fold<16>(v, lane);
+    route_fold<8>(v, lane);
+    __syncthreads();   // (the previous group of experts has been read)
+    {
+      const int e = (lane >> 3) & 7;
+      *(f32x4*)&red[wave][e][cl * 8] = f32x4{v[0], v[1], v[2], v[3]};
+      *(f32x4*)&red[wave][e][cl * 8 + 4] = f32x4{v[4], v[5], v[6], v[7]};
+    }
+    __syncthreads();
+    {
+      const int e = threadIdx.x >> 5, col = (threadIdx.x & 31) * 2;
+      if (e0 + e < E) {
+        f32x2 s2 = *(const f32x2*)&red[0][e][col];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) s2 += *(const f32x2*)&red[w][e][col];
+        *(f32x2*)(part + ((long)blockIdx.y * E + e0 + e) * d + blockIdx.x * 64 + col) = s2;
       }
     }
   }
@@ -695,14 +875,8 @@ __device__ void pow2_le_moe(float v, float limit, int e_lo, int e_hi, float* s_o
 
 // rows_out[e] = rows_in[e] with the four backward columns filled from the expert's amax(dy)
 // (round2/source/kernels/nki_mlp_fused8.py:803-813, once per expert).
-__global__ void moe_backward_scales_kernel(const unsigned* __restrict__ amax_bits, const float* __restrict__ rows_in,
-                                           float* __restrict__ rows_out, int E, float dp_factor) {
-  int e = threadIdx.x;
-  if (e >= E) return;
-  const float* in = rows_in + e * 16;
-  float* out = rows_out + e * 16;
+__device__ void moe_backward_scale_row(const float* in, float* out, float amax_dy, float dp_factor) {
   for (int i = 0; i < 16; ++i) out[i] = in[i];
-  const float amax_dy = __uint_as_float(amax_bits[e]);
   float s_dy, i_dy, s_dp, i_dp;
   pow2_le_moe(amax_dy, TFB_E5M2_MAX / 2.0f, -40, 60, &s_dy, &i_dy);
   float bound = sqrtf(in[9] * in[10]) * amax_dy * dp_factor;
@@ -711,6 +885,34 @@ __global__ void moe_backward_scales_kernel(const unsigned* __restrict__ amax_bit
   out[6] = i_dy * in[12] * 2.0f;
   out[7] = s_dp;
   out[8] = i_dp * in[11];
+}
+__global__ void moe_backward_scales_kernel(const unsigned* __restrict__ amax_bits, const float* __restrict__ rows_in,
+                                           float* __restrict__ rows_out, int E, float dp_factor) {
+  int e = threadIdx.x;
+  if (e >= E) return;
+  moe_backward_scale_row(rows_in + e * 16, rows_out + e * 16, __uint_as_float(amax_bits[e]), dp_factor);
+}
+// The same from the row maxima the combine backward left: workgroup e takes the maximum over expert e's rows
+// seg[e] .. seg[e + 1] (a maximum does not depend on the order, so the scales are those of the kernel above bit for bit).
+__global__ __launch_bounds__(256) void moe_backward_scales_rowmax_kernel(const float* __restrict__ rowmax, const int* __restrict__ seg,
+                                                                        const float* __restrict__ rows_in,
+                                                                        float* __restrict__ rows_out, float dp_factor) {
+  __shared__ float red[4];
+  const int e = blockIdx.x;
+  float m = 0.f;
+  const int end = seg[e + 1];
+  for (int r = seg[e] + threadIdx.x; r < end; r += 256 * 8) {   // eight loads in flight per thread
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = r + 256 * j < end ? rowmax[r + 256 * j] : 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) m = fmaxf(m, v[j]);
+  }
+  m = wave_max(m);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0)
+    moe_backward_scale_row(rows_in + e * 16, rows_out + e * 16, fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])), dp_factor);
 }
 
 // out8[row] = fp8(x[row] * rows[expert of row][col]) for the rows of live tiles; padding tiles are zero-filled.
@@ -753,7 +955,10 @@ extern "C" int tfb_moe_route(const void* h, const void* wr, const void* bias, vo
                              int d, int E, int topk, void* stream) {
   if (!h || !wr || !p || !idx || !gate) return TFB_ERR_ARG;
   if (N <= 0 || d <= 0 || d % 8 || E < 2 || E > MAXE || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
-  if (E <= 8)
+  if (E <= 8 && TFB_ROUTE_RESIDENT)
+    hipLaunchKernelGGL(moe_route8_kernel, dim3((unsigned)((N + 31) / 32)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)h,
+                       (const float*)wr, (const float*)bias, (float*)logits, (float*)p, (int*)idx, (float*)gate, N, d, E, topk);
+  else if (E <= 8)
     hipLaunchKernelGGL((moe_route_kernel<8, 1>), dim3(nblocks(N * 64)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)h,
                        (const float*)wr, (const float*)bias, (float*)logits, (float*)p, (int*)idx, (float*)gate, N, d, E, topk);
   else
@@ -849,9 +1054,21 @@ extern "C" int tfb_moe_combine_bwd(const void* dout, const void* ys, const void*
                                    void* dys, void* dgate, long rmax, int d, int topk, void* stream) {
   if (!dout || !ys || !tok || !ksel || !gate || !dys || !dgate) return TFB_ERR_ARG;
   if (rmax <= 0 || d <= 0 || d % 8 || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
-  hipLaunchKernelGGL(moe_combine_bwd_kernel, dim3(nblocks(rmax * 64)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)dout,
-                     (const bf16_t*)ys, (const int*)tok, (const int*)ksel, (const float*)gate, (bf16_t*)dys, (float*)dgate, rmax,
-                     d, topk);
+  hipLaunchKernelGGL(moe_combine_bwd_kernel<false>, dim3(nblocks(rmax * 64)), dim3(256), 0, (hipStream_t)stream,
+                     (const bf16_t*)dout, (const bf16_t*)ys, (const int*)tok, (const int*)ksel, (const float*)gate, (bf16_t*)dys,
+                     (float*)dgate, (float*)nullptr, rmax, d, topk);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+// tfb_moe_combine_bwd that also leaves rowmax fp32 [rmax] = max |dys[row]| (0 for a padding row) for
+// tfb_moe_backward_scales_rowmax: the experts' backward scales then cost no pass of their own over dys.
+extern "C" int tfb_moe_combine_bwd_rowmax(const void* dout, const void* ys, const void* tok, const void* ksel, const void* gate,
+                                          void* dys, void* dgate, void* rowmax, long rmax, int d, int topk, void* stream) {
+  if (!dout || !ys || !tok || !ksel || !gate || !dys || !dgate || !rowmax) return TFB_ERR_ARG;
+  if (rmax <= 0 || d <= 0 || d % 8 || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_combine_bwd_kernel<true>, dim3(nblocks(rmax * 64)), dim3(256), 0, (hipStream_t)stream,
+                     (const bf16_t*)dout, (const bf16_t*)ys, (const int*)tok, (const int*)ksel, (const float*)gate, (bf16_t*)dys,
+                     (float*)dgate, (float*)rowmax, rmax, d, topk);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
@@ -889,7 +1106,10 @@ static int moe_route_bwd_impl(const void* dgate, const void* p, const void* idx,
                          (const float*)dlogits, (const float*)wr, (bf16_t*)dh, N, d, E, topk);
   }
   TFB_LAUNCH_CHECK();
-  const long chunk = ((N + DWR_CHUNKS - 1) / DWR_CHUNKS + 31) / 32 * 32;
+  // as many token chunks as give one round of resident workgroups (three per CU at this kernel's registers), DWR_CHUNKS at most
+  const int resident = tfb_resident_slots(3) / (d / 64);
+  const int want = DWR_WANT ? DWR_WANT : (resident < 1 ? 1 : (resident < DWR_CHUNKS ? resident : DWR_CHUNKS));
+  const long chunk = ((N + want - 1) / want + 31) / 32 * 32;
   const int chunks = (int)((N + chunk - 1) / chunk);
   hipLaunchKernelGGL(moe_dwr_partial_kernel, dim3(d / 64, chunks), dim3(256), 0, s, (const float*)dlogits, (const bf16_t*)h,
                      (float*)scratch, N, chunk, d, E);
@@ -980,6 +1200,18 @@ extern "C" int tfb_moe_backward_scales(const void* dys, const void* tile_expert,
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(moe_backward_scales_kernel, dim3(1), dim3(64), 0, s, (const unsigned*)amax_scratch, (const float*)rows_in,
                      (float*)rows_out, E, (float)(36.16 * (double)d));
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// tfb_moe_backward_scales from rowmax fp32 [rmax] (tfb_moe_combine_bwd_rowmax) and the segment offsets seg int32 [E + 1]
+// (tfb_moe_tables): the same rows, one small launch. d is the experts' model width (it sets the bound of dpre).
+extern "C" int tfb_moe_backward_scales_rowmax(const void* rowmax, const void* seg, const void* rows_in, void* rows_out, int d, int E,
+                                              void* stream) {
+  if (!rowmax || !seg || !rows_in || !rows_out) return TFB_ERR_ARG;
+  if (d <= 0 || d % 8 || E < 1 || E > MAXE) return TFB_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_backward_scales_rowmax_kernel, dim3(E), dim3(256), 0, (hipStream_t)stream, (const float*)rowmax,
+                     (const int*)seg, (const float*)rows_in, (float*)rows_out, (float)(36.16 * (double)d));
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

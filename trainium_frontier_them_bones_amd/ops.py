@@ -827,6 +827,15 @@ def moe_backward_scales(dys, rows, tab):
     return out
 
 
+def moe_backward_scales_rowmax(rowmax, rows, tab, d):
+    """moe_backward_scales from the row maxima moe_combine_bwd(..., want_rowmax=True) left: the same rows, no pass over dys."""
+    _chk(rowmax, torch.float32), _chk(rows, torch.float32)
+    E = rows.shape[0]
+    out = torch.empty_like(rows)
+    _lib.call("tfb_moe_backward_scales_rowmax", _p(rowmax), _p(tab["seg"]), _p(rows), _p(out), d, E, _stream())
+    return out
+
+
 def moe_quant(x, rows, col, fmt, tab):
     _chk(x), _chk(rows, torch.float32)
     out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
@@ -894,12 +903,18 @@ def moe_combine(ys, tab, gate, N):
     return out
 
 
-def moe_combine_bwd(dout, ys, tab, gate):
+def moe_combine_bwd(dout, ys, tab, gate, want_rowmax=False):
+    """(dys, dgate), and with want_rowmax the fp32 [rmax] maxima of |dys| per row for moe_backward_scales_rowmax."""
     _chk(dout), _chk(ys), _chk(gate, torch.float32)
     rmax, d = ys.shape
     dys = torch.empty_like(ys)
     # the kernel writes the gate gradient of every assignment that holds a row; a skipped one's is zero
     dgate = torch.zeros_like(gate) if "capacity" in tab else torch.empty_like(gate)
+    if want_rowmax:
+        rowmax = torch.empty(rmax, dtype=torch.float32, device=ys.device)
+        _lib.call("tfb_moe_combine_bwd_rowmax", _p(dout), _p(ys), _p(tab["tok"]), _p(tab["ksel"]), _p(gate), _p(dys), _p(dgate),
+                  _p(rowmax), rmax, d, gate.shape[1], _stream())
+        return dys, dgate, rowmax
     _lib.call("tfb_moe_combine_bwd", _p(dout), _p(ys), _p(tab["tok"]), _p(tab["ksel"]), _p(gate), _p(dys), _p(dgate), rmax, d,
               gate.shape[1], _stream())
     return dys, dgate
