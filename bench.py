@@ -11,7 +11,8 @@ python bench.py --ns-probe        (Muon's Newton-Schulz call on the benchmark mo
 one line per stack with its time and flop rate; not part of the AdamW step the headline line times)
 
 python bench.py --config-probe c1|c2|c3|c5|all   (the standalone configurations beside the full step, fwd + bwd each:
-one line per configuration; run under rocprofv3 --kernel-trace --stats for the per-kernel durations)
+one line per configuration; run under rocprofv3 --kernel-trace --stats for the per-kernel durations; with --graphs a
+second line per configuration: the same repetition recorded once as a HIP graph and replayed, without the host's launch work)
 
 python bench.py --traffic-probe   (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: a 256 MiB device copy as the
 counters' calibration, then attention forward + backward at the benchmark shape; prints nothing)
@@ -185,7 +186,7 @@ def ns_probe():
         print("ns5 K=%d %dx%d: %.3f ms, %.0f TFLOP/s" % (K, r, c, dt * 1e3, flop / dt / 1e12), flush=True)
 
 
-def config_probe(which):
+def config_probe(which, graphs=False):
     """The standalone configurations beside the full step, each fwd + bwd through the autograd layer, 3 untimed and 5 timed
     repetitions: c1 RMSNorm -> LM head -> cross-entropy on 8192 tokens; c2 causal attention 16 x 12 x 2048 x 64; c3 the
     fp8 MLP on 16384 tokens with a per-tensor amax activation scale; c5 the 8-expert top-2 fp8 layer on 16384 tokens,
@@ -206,6 +207,30 @@ def config_probe(which):
         torch.cuda.synchronize()
         dt = (time.perf_counter() - t0) / 5
         print("%s: %.3f ms per fwd+bwd, %.0f TFLOP/s of algorithmic work" % (name, dt * 1e3, flop / dt / 1e12), flush=True)
+        if not graphs:
+            return
+        # the same repetition recorded once as a HIP graph and replayed: what is left when the host's launch work (some
+        # twenty Python calls per repetition) is out of the way. Warm-up on a side stream first, as torch's capture asks.
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fn()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            graph.replay()
+        torch.cuda.synchronize()
+        dg = (time.perf_counter() - t0) / 5
+        print("%s, replayed as a HIP graph: %.3f ms per fwd+bwd, %.0f TFLOP/s of algorithmic work"
+              % (name, dg * 1e3, flop / dg / 1e12), flush=True)
 
     def leaf(t):
         return t.to(dev).requires_grad_(True)
@@ -249,7 +274,7 @@ def config_probe(which):
 
         def c3():
             clear(x, wf, wp)
-            st.x_scale = float(ops.amax_scale(x.detach(), 448.0, -20, 20)[0].item())   # power of two under amax
+            st.x_scale = ops.amax_scale(x.detach(), 448.0, -20, 20)[0:1]   # power of two under amax, left on the device
             st.refresh(wf, wp)
             A.Mlp8Fn.apply(x, wf, wp, st).backward(dy)
         timed("c3 fp8 MLP, 16384 tokens (scales and weight packs refreshed inside)", c3, 6 * 2.0 * M * d * F)
@@ -317,6 +342,7 @@ def main():
     ap.add_argument("--ns-probe", action="store_true")
     ap.add_argument("--hw-probe", action="store_true")
     ap.add_argument("--config-probe", choices=("c1", "c2", "c3", "c5", "all"))
+    ap.add_argument("--graphs", action="store_true", help="with --config-probe: also time each repetition replayed as a HIP graph")
     ap.add_argument("--bf16-dw", action="store_true")
     ap.add_argument("--unfused-residual", action="store_true")
     ap.add_argument("--all-kernels", action="store_true", help="roofline.per_kernel lists every entry point, not the top 8")
@@ -335,7 +361,7 @@ def main():
         hw_probe()
         return
     if args.config_probe:
-        config_probe(args.config_probe)
+        config_probe(args.config_probe, args.graphs)
         return
 
     import statistics

@@ -136,9 +136,11 @@ long tfb_mlp8_scale_scratch_floats(int F);
 /* row_out fp32 [16] = the layer's scale row from w_fc [F][d], w_proj [d][F] (bf16): columns s_wfc, dq_fc, c_h, s_wproj,
  * dq_proj, s_dy, dq_dh2, s_dp, dq_dx, rho2, kappa2, i_wfc, i_wproj, s_h, amax_wfc, amax_wproj.
  * Replaces forward_scales (round2/source/kernels/nki_mlp_fused8.py:782-800) and the statistics kernels of
- * round2/source/kernels/nki_scstat.py. e4m3_limit 240 gives the reference's rows. */
+ * round2/source/kernels/nki_scstat.py. e4m3_limit 240 gives the reference's rows. x_scale: the activation scale the
+ * forward casts x at (the reference's constant 4), or x_scale_dev (not NULL: a device fp32 scalar, e.g. tfb_amax_scale's
+ * output, read by the kernel so that a per-tensor amax scale costs no host synchronisation; x_scale is then ignored). */
 int tfb_mlp8_forward_scales(const void* w_fc, const void* w_proj, void* row_out, void* scratch, int F, int d,
-                            float e4m3_limit, float x_scale, void* stream);
+                            float e4m3_limit, float x_scale, const void* x_scale_dev, void* stream);
 
 /* row_out = row_in with s_dy, dq_dh2, s_dp, dq_dx filled from amax(dy); scratch fp32 [1024].
  * Replaces backward_scales (nki_mlp_fused8.py:803-813). */
@@ -202,12 +204,13 @@ int tfb_mlp8_bwd_q(const void* dy8, const void* r, const void* w8, const void* r
  * dw_fc [F][d] = ((dp8^T @ x8) / (s_dp * x_scale)), dp8 = e5m2(dpre s_dp) from tfb_mlp8_bwd, x8 = e4m3(x x_scale);
  * dw_proj [d][F] = ((dy8^T @ hq8) / (s_dy * s_h)), dy8 = e5m2(dy s_dy), hq8 from tfb_mlp8_bwd_q. row = the backward row.
  * Outputs bf16 (out_f32 = 0) or fp32, optionally accumulated into (one rounding); fp32 accumulation over all tokens;
- * workspace >= splits * d * F * 4 bytes (256 MB always suffices). Shapes as tfb_mlp8_fwd.
+ * workspace >= splits * d * F * 4 bytes (256 MB always suffices). Shapes as tfb_mlp8_fwd. x_scale_dev (not NULL): the
+ * activation scale as a device fp32 scalar instead of x_scale, as in tfb_mlp8_forward_scales.
  * Replaces mlp8_weight_grads under the fp8 weight-gradient switch (round2/source/train.py:8209-8229: dw8_grad twice,
  * nki_dw8.py:323 emulate_dw / _dw8_kernel) and R1's fp8 dW rows (round1/source/train.py:3182 run_tn_fp8). */
 int tfb_mlp8_dw8(const void* x8, const void* dp8, const void* hq8, const void* dy8, const void* row, float x_scale, void* dw_fc,
                  void* dw_proj, long M, int d, int F, int out_f32, int accumulate, void* workspace, long workspace_bytes,
-                 void* stream);
+                 const void* x_scale_dev, void* stream);
 
 /* ---- fp8 projections (attention QKV / output projection in fp8) -----------------------------------------------------
  * out8 [R][C], outT8 [C][R] = e4m3(w [R][C] * *scale_ptr): a weight pre-cast once per optimizer step in both byte layouts.

@@ -369,6 +369,76 @@ def test_mlp8_fp8_weight_grads(ops, dev, shape, limit):
     assert rel_l2(a_fc, ref_fc + acc_fc) < 1e-4 and rel_l2(a_pj, ref_pj + acc_pj) < 1e-4
 
 
+def test_mlp8_activation_scale_from_the_device(ops, dev):
+    """The activation scale as a device scalar (the per-tensor amax scale, never read back by the host) gives the layer
+    the host-float path's outputs and gradients bit for bit: scale row, forward, backward and both fp8 weight gradients."""
+    from trainium_frontier_them_bones_amd import autograd as A
+    M, d, F = 1024, 256, 512
+    g = _g(4242)
+    x = (3.0 * torch.randn(M, d, generator=g)).bfloat16().to(dev)
+    wf = (0.02 * torch.randn(F, d, generator=g)).bfloat16().to(dev)
+    wp = (0.02 * torch.randn(d, F, generator=g)).bfloat16().to(dev)
+    dy = torch.randn(M, d, generator=g).bfloat16().to(dev)
+    sc = ops.amax_scale(x, 448.0, -20, 20)
+    host = float(sc[0].item())
+    assert host > 0 and host == 2.0 ** round(torch.log2(torch.tensor(host)).item())      # a power of two
+    outs = []
+    for x_scale in (host, sc[0:1]):
+        xl, wfl, wpl = (t.clone().requires_grad_(True) for t in (x, wf, wp))
+        st = A.Mlp8State(e4m3_limit=448.0, x_scale=x_scale, dw_fp8=True)
+        st.refresh(wfl, wpl)
+        y = A.Mlp8Fn.apply(xl, wfl, wpl, st)
+        y.backward(dy)
+        outs.append((st.row, y.detach(), xl.grad, wfl.grad, wpl.grad))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    with pytest.raises(ValueError):
+        ops.mlp8_forward_scales(wf, wp, 448.0, sc)                                       # three elements: not a scalar
+
+
+def test_mlp8_layer_replayed_as_a_hip_graph(ops, dev):
+    """The fp8 MLP layer with everything per-step inside (amax activation scale on the device, scale row, weight packs,
+    forward, backward, fp8 weight gradients) recorded once as a HIP graph: three replays on new inputs, with eager runs
+    of the same layer and synchronisations between them, each equal to the eager result bit for bit."""
+    from trainium_frontier_them_bones_amd import autograd as A
+    M, d, F = 1024, 256, 512
+    g = _g(77)
+
+    def fresh():
+        return ((2.0 * torch.randn(M, d, generator=g)).bfloat16().to(dev), (0.02 * torch.randn(F, d, generator=g)).bfloat16().to(dev),
+                (0.02 * torch.randn(d, F, generator=g)).bfloat16().to(dev), torch.randn(M, d, generator=g).bfloat16().to(dev))
+
+    def layer(x, wf, wp, dy):
+        xl, wfl, wpl = (t.detach().requires_grad_(True) for t in (x, wf, wp))
+        st = A.Mlp8State(e4m3_limit=448.0, x_scale=ops.amax_scale(xl.detach(), 448.0, -20, 20)[0:1], dw_fp8=True)
+        st.refresh(wfl, wpl)
+        y = A.Mlp8Fn.apply(xl, wfl, wpl, st)
+        y.backward(dy)
+        return y.detach(), xl.grad, wfl.grad, wpl.grad
+
+    static = fresh()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            layer(*static)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = layer(*static)
+    for _ in range(3):
+        new = fresh()
+        want = [t.clone() for t in layer(*new)]          # eager work between the replays
+        torch.cuda.synchronize()
+        for s_, n_ in zip(static, new):
+            s_.copy_(n_)
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(outs, want):
+            assert torch.equal(a, b)
+
+
 def test_mlp8_refresh_of_all_layers_equals_per_layer_calls(ops, dev):
     g = _g(31)
     L, d, F = 3, 256, 512

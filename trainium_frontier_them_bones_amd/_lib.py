@@ -28,7 +28,7 @@ SIGNATURES = {
     "tfb_block_head_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_block_head_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _vp],
     "tfb_mlp8_scale_scratch_floats": [_i],
-    "tfb_mlp8_forward_scales": [_vp, _vp, _vp, _vp, _i, _i, _f, _f, _vp],
+    "tfb_mlp8_forward_scales": [_vp, _vp, _vp, _vp, _i, _i, _f, _f, _vp, _vp],
     "tfb_mlp8_backward_scales": [_vp, _vp, _vp, _vp, _l, _i, _vp],
     "tfb_amax_scale": [_vp, _l, _f, _i, _i, _vp, _vp, _vp],
     "tfb_quant_fp8": [_vp, _vp, _f, _i, _vp, _l, _vp],
@@ -39,7 +39,7 @@ SIGNATURES = {
     "tfb_mlp8_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_mlp8_bwd_q": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _l, _i, _i, _vp],
     "tfb_gemm_fp8_tn": [_vp, _i, _vp, _i, _vp, _vp, _f, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
-    "tfb_mlp8_dw8": [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
+    "tfb_mlp8_dw8": [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp, _vp],
     "tfb_attn_fwd": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _i, _i, _i, _i, _f, _vp],
     "tfb_attn_fwd_band": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _i, _i, _i, _i, _f, _i, _vp],
     "tfb_attn_bwd_band": [_vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _lp, _vp, _vp, _vp, _vp,

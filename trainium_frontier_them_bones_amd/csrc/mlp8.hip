@@ -196,7 +196,7 @@ __device__ float reduce_max_array(const float* a, int n, float* red) {
 __global__ __launch_bounds__(256) void forward_scales_kernel(const float* rowss, int F, const float* amax_fc_part, int nfc,
                                                             const float* colss, const float* amax_pj_part, int npj,
                                                             float e4m3_limit, float h_bound, float inv_x_scale,
-                                                            float* row_out, long oz) {
+                                                            const float* __restrict__ x_scale_dev, float* row_out, long oz) {
   __shared__ float red[4];
   rowss += blockIdx.z * oz;
   amax_fc_part += blockIdx.z * oz;
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(256) void forward_scales_kernel(const float* rowss,
     pow2_le(amax_pj, e4m3_limit, -24, 40, &s_wpj, &i_wpj);
     pow4_le(rho2 * h_bound, e4m3_limit, -16, 8, &s_h, &i_h, &c_h);
     row_out[SC_S_WFC] = s_wfc;
-    row_out[SC_DQ_FC] = i_wfc * inv_x_scale;
+    row_out[SC_DQ_FC] = i_wfc * (x_scale_dev ? 1.0f / *x_scale_dev : inv_x_scale);   // (a power of two: exact either way)
     row_out[SC_C_H] = c_h;
     row_out[SC_S_WPROJ] = s_wpj;
     row_out[SC_DQ_PROJ] = i_h * i_wpj;
@@ -537,7 +537,7 @@ extern "C" long tfb_mlp8_scale_scratch_floats(int F) { return (2L + COL_SLICES) 
 // The forward scale rows of `layers` MLPs whose weights sit `wz` elements apart (w_fc and w_proj alike): four launches
 // whatever the layer count. scratch: layers x tfb_mlp8_scale_scratch_floats(F) floats; row_out: layers x 16 floats.
 static int launch_forward_scales(const void* w_fc, const void* w_proj, void* row_out, void* scratch, int F, int d,
-                                 float e4m3_limit, float x_scale, int layers, long wz, hipStream_t s) {
+                                 float e4m3_limit, float x_scale, const void* x_scale_dev, int layers, long wz, hipStream_t s) {
   const long oz = tfb_mlp8_scale_scratch_floats(F);
   float* rowss = (float*)scratch;
   float* colss = rowss + F;
@@ -558,17 +558,18 @@ static int launch_forward_scales(const void* w_fc, const void* w_proj, void* row
   TFB_LAUNCH_CHECK();
   const float h_bound = (float)(1.3 * (double)d);
   hipLaunchKernelGGL(forward_scales_kernel, dim3(1, 1, layers), dim3(256), 0, s, rowss, F, pa, nfc, colss, pb, npj * slices,
-                     e4m3_limit, h_bound, (float)(1.0 / (double)x_scale), (float*)row_out, oz);
+                     e4m3_limit, h_bound, x_scale_dev ? 0.f : (float)(1.0 / (double)x_scale), (const float*)x_scale_dev,
+                     (float*)row_out, oz);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
 
 extern "C" int tfb_mlp8_forward_scales(const void* w_fc, const void* w_proj, void* row_out, void* scratch, int F, int d,
-                                       float e4m3_limit, float x_scale, void* stream) {
+                                       float e4m3_limit, float x_scale, const void* x_scale_dev, void* stream) {
   if (!w_fc || !w_proj || !row_out || !scratch) return TFB_ERR_ARG;
-  if (F <= 0 || d <= 0 || F % 8 || d % 8) return TFB_ERR_SHAPE;
+  if (F <= 0 || d <= 0 || F % 8 || d % 8 || (!x_scale_dev && !(x_scale > 0.f))) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
-  return launch_forward_scales(w_fc, w_proj, row_out, scratch, F, d, e4m3_limit, x_scale, 1, 0, s);
+  return launch_forward_scales(w_fc, w_proj, row_out, scratch, F, d, e4m3_limit, x_scale, x_scale_dev, 1, 0, s);
 }
 
 extern "C" int tfb_mlp8_backward_scales(const void* dy, const void* row_in, void* row_out, void* scratch, long M, int d,
@@ -640,7 +641,7 @@ extern "C" int tfb_mlp8_refresh_layers(const void* w_fc, const void* w_proj, lon
       !(x_scale > 0.f))
     return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
-  int st = launch_forward_scales(w_fc, w_proj, rows, scratch, F, d, e4m3_limit, x_scale, layers, layer_stride, s);
+  int st = launch_forward_scales(w_fc, w_proj, rows, scratch, F, d, e4m3_limit, x_scale, nullptr, layers, layer_stride, s);
   if (st != TFB_OK) return st;
   uint8_t* b = (uint8_t*)w8;
   const long n = (long)F * d;
@@ -791,13 +792,13 @@ extern "C" int tfb_mlp8_bwd(const void* dy8, const void* r, const void* w8, cons
 // Replaces mlp8_weight_grads under switch 9k (round2/source/train.py:8209-8229) = K/nki_dw8.py:323 emulate_dw.
 extern "C" int tfb_mlp8_dw8(const void* x8, const void* dp8, const void* hq8, const void* dy8, const void* row, float x_scale,
                             void* dw_fc, void* dw_proj, long M, int d, int F, int out_f32, int accumulate, void* workspace,
-                            long workspace_bytes, void* stream) {
+                            long workspace_bytes, const void* x_scale_dev, void* stream) {
   if (!x8 || !dp8 || !hq8 || !dy8 || !row || !dw_fc || !dw_proj || !workspace) return TFB_ERR_ARG;
-  if (!shapes8(M, d, F) || !(x_scale > 0.f)) return TFB_ERR_SHAPE;
+  if (!shapes8(M, d, F) || (!x_scale_dev && !(x_scale > 0.f))) return TFB_ERR_SHAPE;
   const float* sc = (const float*)row;
-  // dw_fc[f][dd] = sum_m dp8[m][f] x8[m][dd]: g = dp8 (e5m2), a = x8 (e4m3)
-  int st = tfb_gemm_fp8_tn(dp8, TFB_FMT_E5M2, x8, TFB_FMT_E4M3, sc + SC_S_DP, nullptr, 1.0f / x_scale, dw_fc, M, F, d, out_f32,
-                           accumulate, workspace, workspace_bytes, stream);
+  // dw_fc[f][dd] = sum_m dp8[m][f] x8[m][dd]: g = dp8 (e5m2), a = x8 (e4m3); x8's scale from the device when it lives there
+  int st = tfb_gemm_fp8_tn(dp8, TFB_FMT_E5M2, x8, TFB_FMT_E4M3, sc + SC_S_DP, x_scale_dev, x_scale_dev ? 1.0f : 1.0f / x_scale,
+                           dw_fc, M, F, d, out_f32, accumulate, workspace, workspace_bytes, stream);
   if (st != TFB_OK) return st;
   // dw_proj[dd][f] = sum_m dy8[m][dd] hq8[m][f]: g = dy8 (e5m2), a = hq8 (e4m3)
   return tfb_gemm_fp8_tn(dy8, TFB_FMT_E5M2, hq8, TFB_FMT_E4M3, sc + SC_S_DY, sc + SC_S_H, 1.0f, dw_proj, M, d, F, out_f32,

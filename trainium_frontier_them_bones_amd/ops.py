@@ -199,16 +199,27 @@ def _scratch(device, nfloats):
     return torch.empty(nfloats, dtype=torch.float32, device=device)
 
 
+def _scale_arg(x_scale):
+    """(float, device pointer) for an activation scale given as a python float or as a 1-element fp32 device tensor."""
+    if isinstance(x_scale, torch.Tensor):
+        _chk(x_scale, torch.float32)
+        if x_scale.numel() != 1:
+            raise ValueError("a device activation scale is one fp32 element")
+        return 0.0, _p(x_scale)
+    return float(x_scale), None
+
+
 def mlp8_forward_scales(w_fc, w_proj, e4m3_limit=240.0, x_scale=4.0):
-    """The layer's fp32 [16] scale row, computed on the device from the bf16 weights (w_fc [F,d], w_proj [d,F])."""
+    """The layer's fp32 [16] scale row, computed on the device from the bf16 weights (w_fc [F,d], w_proj [d,F]).
+    x_scale: python float (the reference's constant 4) or a 1-element fp32 device tensor (no host synchronisation)."""
     _chk(w_fc), _chk(w_proj)
     F, d = w_fc.shape
     if tuple(w_proj.shape) != (d, F):
         raise ValueError("w_proj must be [d, F]")
     row = torch.empty(NSC, dtype=torch.float32, device=w_fc.device)
     scr = _scratch(w_fc.device, _lib.lib().tfb_mlp8_scale_scratch_floats(F))
-    _lib.call("tfb_mlp8_forward_scales", _p(w_fc), _p(w_proj), _p(row), _p(scr), F, d, float(e4m3_limit), float(x_scale),
-              _stream())
+    xf, xd = _scale_arg(x_scale)
+    _lib.call("tfb_mlp8_forward_scales", _p(w_fc), _p(w_proj), _p(row), _p(scr), F, d, float(e4m3_limit), xf, xd, _stream())
     return row
 
 
@@ -408,8 +419,9 @@ def mlp8_dw8(x8, dp8, hq8, dy8, row, x_scale=4.0, dw_fc=None, dw_proj=None, accu
         if tuple(dw_fc.shape) != (F, d) or tuple(dw_proj.shape) != (d, F):
             raise ValueError("bad output shapes")
     ws = _workspace(x8.device)
-    _lib.call("tfb_mlp8_dw8", _p(x8), _p(dp8), _p(hq8), _p(dy8), _p(row), float(x_scale), _p(dw_fc), _p(dw_proj), M, d, F,
-              int(dw_fc.dtype == torch.float32), int(accumulate), _p(ws), ws.numel() * 4, _stream())
+    xf, xd = _scale_arg(x_scale)
+    _lib.call("tfb_mlp8_dw8", _p(x8), _p(dp8), _p(hq8), _p(dy8), _p(row), xf, _p(dw_fc), _p(dw_proj), M, d, F,
+              int(dw_fc.dtype == torch.float32), int(accumulate), _p(ws), ws.numel() * 4, xd, _stream())
     return dw_fc, dw_proj
 
 
