@@ -316,7 +316,7 @@ int tfb_loss_multi_bwd(const void* logits, const void* targets, int idx64, const
                        const void* g, void* dlogits, long rows, int V, float softcap, void* stream);
 
 /* logits = x @ W^T (x [rows][d], W [V][d]) with the row log-sum-exp reduced in the GEMM epilogue, then loss / lse as
- * tfb_loss_fwd. part: fp32 [rows][V/64][2] scratch. rows, V multiples of 128, d of 64.
+ * tfb_loss_fwd. part: fp32 scratch of rows * (V / 64) * 2 elements. rows, V multiples of 128, d of 64.
  * Replaces the lm_head matmul + loss forward pair (round1/source/train.py:8668, 9191-9212). */
 int tfb_lmhead_fwd(const void* x, const void* W, const void* targets, int idx64, const void* row_w, void* logits, void* part,
                    void* loss, void* lse, long rows, int d, int V, float softcap, void* stream);

@@ -276,8 +276,8 @@ __global__ __launch_bounds__(256) void loss_multi_bwd_kernel(const bf16_t* __res
 struct EpiLmHead {
   static constexpr bool kTileEpilogue = true;
   bf16_t* logits;  // [rows][V]
-  float* part;     // [rows][V/64][2] (max, sum)
-  long V;
+  float* part;     // [V/64][rows][2] (max, sum): slab-major, so that a wavefront's 32 rows of one slab are one 256-byte store
+  long V, rows;
   int nchunk;      // V / 64
   float cap;
   template <int TP, int TQ>
@@ -321,35 +321,38 @@ struct EpiLmHead {
         a.m = mx;
         a.s = t;
       }
-      if (lh == 0) {
-        float* pp = part + (row * nchunk + (pw >> 6)) * 2;
-        pp[0] = a.m;
-        pp[1] = a.s;
-      }
+      if (lh == 0) *(f32x2_t*)(part + ((long)(pw >> 6) * rows + row) * 2) = f32x2_t{a.m, a.s};
     }
   }
 };
 
-// One wavefront per row: merge the row's partial pairs, read the target logit, write lse and the row loss.
+// A workgroup per 64 rows, a lane per row: each wavefront merges a quarter of the row's slab pairs (eight coalesced 512-byte
+// loads in flight), the four quarters meet in LDS, then the target logit is read and lse and the row loss are written.
 template <typename IDX>
 __global__ __launch_bounds__(256) void lmhead_finish_kernel(const float* __restrict__ part, const bf16_t* __restrict__ logits,
                                                            const IDX* __restrict__ tg, const float* __restrict__ row_w,
                                                            float* __restrict__ loss, float* __restrict__ lse, long rows, long V,
                                                            int nchunk, float cap) {
+  __shared__ float rm[4][64], rs[4][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const long row = (long)blockIdx.x * 4 + wave;
-  if (row >= rows) return;
+  const long row = (long)blockIdx.x * 64 + lane;
+  const long rr = row < rows ? row : rows - 1;
+  const int q = (nchunk + 3) / 4, c0 = wave * q, c1 = c0 + q < nchunk ? c0 + q : nchunk;
   MS a{-1e30f, 0.f};
-  for (int c = lane; c < nchunk; c += 64) {
-    const float* pp = part + (row * nchunk + c) * 2;
-    a = ms_merge(a, MS{pp[0], pp[1]});
-  }
+  for (int c = c0; c < c1; c += 8) {
+    f32x2_t v[8];
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    MS b{__shfl_xor(a.m, o, 64), __shfl_xor(a.s, o, 64)};
-    a = ms_merge(a, b);
+    for (int j = 0; j < 8; ++j)
+      v[j] = c + j < c1 ? *(const f32x2_t*)(part + ((long)(c + j) * rows + rr) * 2) : f32x2_t{-1e30f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) a = ms_merge(a, MS{v[j][0], v[j][1]});
   }
-  if (lane == 0) {
+  rm[wave][lane] = a.m;
+  rs[wave][lane] = a.s;
+  __syncthreads();
+  if (wave == 0 && row < rows) {
+#pragma unroll
+    for (int w = 1; w < 4; ++w) a = ms_merge(a, MS{rm[w][lane], rs[w][lane]});
     float l = a.m + logf(a.s);
     lse[row] = l;
     long tt = (long)tg[row];
@@ -445,10 +448,10 @@ extern "C" int tfb_lmhead_fwd(const void* x, const void* W, const void* targets,
   // workgroup and nothing to hide its epilogue behind); a wavefront spans 64 vocabulary columns.
   using Cfg = GemmCfg<128, 128, 2, 2, 2, TFB_K_CONTIG, TFB_K_CONTIG>;
   GemmOperand P{(const uint8_t*)W, (long)d * 2}, Q{(const uint8_t*)x, (long)d * 2};
-  EpiLmHead e{(bf16_t*)logits, (float*)part, (long)V, V / 64, softcap};
+  EpiLmHead e{(bf16_t*)logits, (float*)part, (long)V, rows, V / 64, softcap};
   int st = gemm_launch<Cfg>(P, Q, V, (int)rows, (long)d * 2, 1, LoadIdentity{}, LoadIdentity{}, e, s);
   if (st != TFB_OK) return st;
-  unsigned nb = (unsigned)((rows + 3) / 4);
+  unsigned nb = (unsigned)((rows + 63) / 64);
   if (idx64)
     hipLaunchKernelGGL(lmhead_finish_kernel<long>, dim3(nb), dim3(256), 0, s, (const float*)part, (const bf16_t*)logits,
                        (const long*)targets, (const float*)row_w, (float*)loss, (float*)lse, rows, (long)V, V / 64, softcap);
