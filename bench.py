@@ -90,7 +90,7 @@ def _work(name, a):
     if name == "tfb_qkv_rope_fwd":           # x, w, cos, sin, out, M, N, K, T, rot, stream
         M, N, K = a[5:8]
         return "QKV projection + RoPE %dx%dx%d" % (M, N, K), "mfma", 2.0 * M * N * K
-    if name == "tfb_gemm_bf16":              # A, B, C, M, N, K, ta, tb, ...
+    if name in ("tfb_gemm_bf16", "tfb_gemm_bf16_scaled"):   # A, B, C, M, N, K, ta, tb, ...
         M, N, K, ta, tb = a[3:8]
         return "bf16 GEMM %dx%dx%d %s%s" % (M, N, K, "T" if ta else "N", "T" if tb else "N"), "mfma", 2.0 * M * N * K
     if name == "tfb_gemm_bf16_res":          # A, B, res, C, M, N, K, tb, stream
@@ -109,6 +109,9 @@ def _work(name, a):
     if name == "tfb_lmhead_fwd":             # ..., rows, d, V, softcap, stream
         N, d, V = a[-5:-2]
         return "LM head forward + lse", "mfma", 2.0 * N * d * V
+    if name == "tfb_loss_fwd_bwd":           # ..., rows, V, softcap, stream
+        N, V = a[-4:-2]
+        return "loss forward + backward (one pass, dlogits in place)", "hbm", 2.0 * N * V * 2
     if name == "tfb_loss_bwd":               # ..., rows, V, softcap, stream
         N, V = a[-4:-2]
         return "loss backward (dlogits in place)", "hbm", 2.0 * N * V * 2

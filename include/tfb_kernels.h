@@ -27,6 +27,11 @@ extern "C" {
  * weight-gradient accumulate of round1/source/train.py:8463-8509. */
 int tfb_gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int trans_a, int trans_b, int out_f32,
                   int accumulate, void* workspace, long workspace_bytes, void* stream);
+/* tfb_gemm_bf16 with the product multiplied by the device fp32 scalar *alpha (NULL = 1) before its one rounding:
+ * C (+)= alpha op(A) @ op(B). The gradient GEMMs of the LM head take the loss's upstream gradient this way
+ * (autograd's grad_output of round1/source/train.py:9191-9212's loss, which the reference multiplies into dlogits). */
+int tfb_gemm_bf16_scaled(const void* A, const void* B, void* C, int M, int N, int K, int trans_a, int trans_b, int out_f32,
+                         int accumulate, void* workspace, long workspace_bytes, const void* alpha, void* stream);
 /* C [M,N] = bf16(res + bf16(A [M,K] @ op(B))), res [M,N] bf16: a projection with the residual add that follows it made in
  * the GEMM's store; equal to tfb_gemm_bf16 followed by a bf16 add, bit for bit. B is [K,N] (trans_b=0) or [N,K].
  * The bf16 form of _proj8_fwd_ra_kernel (round2/source/kernels/nki_attn_nr8.py:1003: out = bf16(res + bf16(acc dq))). */
@@ -314,6 +319,13 @@ int tfb_loss_multi_fwd(const void* logits, const void* targets, int idx64, const
  * (round2/source/train.py:5767). */
 int tfb_loss_multi_bwd(const void* logits, const void* targets, int idx64, const void* row_w, int K, float eps, const void* lse,
                        const void* g, void* dlogits, long rows, int V, float softcap, void* stream);
+
+/* tfb_loss_fwd followed by tfb_loss_bwd with grow = row_w (an upstream gradient of one), in place and in ONE pass over the
+ * logits (a row is held in a workgroup's registers, V <= 65536; TFB_ERR_SHAPE beyond): loss and lse as tfb_loss_fwd writes
+ * them, logits overwritten by d logits = row_w (softmax - onehot) (1 - tanh^2), all three bit-equal to the two calls.
+ * Replaces _loss_fwd_kernel + _loss_bwd_kernel (round1/source/train.py:4543, 4584) when the loss is differentiated. */
+int tfb_loss_fwd_bwd(void* logits, const void* targets, int idx64, const void* row_w, void* loss, void* lse, long rows, int V,
+                     float softcap, void* stream);
 
 /* logits = x @ W^T (x [rows][d], W [V][d]) with the row log-sum-exp reduced in the GEMM epilogue, then loss / lse as
  * tfb_loss_fwd. part: fp32 scratch of rows * (V / 64) * 2 elements. rows, V multiples of 128, d of 64.

@@ -663,6 +663,64 @@ def test_lmhead_config1(ops, dev):
     assert rel_l2(xd.grad, dx) < BF16_TOL and rel_l2(Wd.grad, dW) < BF16_TOL and rel_l2(nd.grad, dnw) < BF16_TOL
 
 
+@pytest.mark.parametrize("V", [1024, 32768, 50304, 65536])
+@pytest.mark.parametrize("cap,idx", [(0.0, torch.int64), (15.0, torch.int32)])
+def test_loss_forward_and_backward_in_one_pass_equal_the_two_kernels(ops, dev, V, cap, idx):
+    """tfb_loss_fwd_bwd against tfb_loss_fwd + tfb_loss_bwd with grow = the row weights: row losses, lse and the gradient
+    written in place of the logits, bit for bit; ignored rows (target < 0 or >= V) give zero loss and a zero gradient row."""
+    g = _g(900 + V)
+    N = 192
+    x = (3.0 * torch.randn(N, V, generator=g)).bfloat16().to(dev)
+    t = torch.randint(0, V, (N,), generator=g).to(idx)
+    t[3], t[100] = -1, V + 7
+    t = t.to(dev)
+    w = torch.rand(N, generator=g).to(dev)
+    rows0, lse0 = ops.loss_fwd(x, t, cap, w)
+    d0 = ops.loss_bwd(x, t, lse0, w, cap)
+    y = x.clone()
+    rows1, lse1 = ops.loss_fwd_bwd(y, t, w, cap)
+    assert torch.equal(rows0, rows1) and torch.equal(lse0, lse1) and torch.equal(d0, y)
+    assert float(rows1[3]) == 0.0 and float(y[3].float().abs().max()) == 0.0 and float(y[100].float().abs().max()) == 0.0
+    y2 = x.clone()
+    rows2, _ = ops.loss_fwd_bwd(y2, t, None, cap)                                   # no row weights: weight one
+    assert torch.equal(y2, ops.loss_bwd(x, t, lse0, torch.ones_like(w), cap))
+
+
+def test_lmhead_loss_node_with_an_upstream_gradient(ops, dev):
+    """LmHeadLossFn under an upstream gradient of one equals, bit for bit, the composition of the separate calls (GEMM, loss rows and
+    lse, dlogits in place, two gradient GEMMs); under another upstream gradient (a scaled loss) the gradients follow the oracle's."""
+    from oracle import loss as O
+    from trainium_frontier_them_bones_amd import autograd as A
+    g = _g(41)
+    N, d, V = 1024, 256, 8192
+    x = torch.randn(N, d, generator=g).bfloat16()
+    W = (0.05 * torch.randn(V, d, generator=g)).bfloat16()
+    t = torch.randint(0, V, (N,), generator=g)
+    t[17] = -1
+    xd, Wd, td = x.to(dev).requires_grad_(True), W.to(dev).requires_grad_(True), t.to(dev)
+    loss = A.LmHeadLossFn.apply(xd, Wd, td, 15.0, "mean")
+    loss.backward()
+    valid = (td >= 0).float()
+    w = valid / valid.sum()
+    logits = ops.matmul(xd.detach(), Wd.detach(), trans_b=True)
+    rows, lse = ops.loss_fwd(logits, td, 15.0, w)
+    dl = ops.loss_bwd(logits, td, lse, w, 15.0, inplace=True)
+    assert torch.equal(loss.detach(), rows.sum())
+    assert torch.equal(xd.grad, ops.matmul(dl, Wd.detach())) and torch.equal(Wd.grad, ops.matmul(dl, xd.detach(), trans_a=True))
+    gx, gw = xd.grad.clone(), Wd.grad.clone()
+    xd.grad = Wd.grad = None
+    (0.37 * A.LmHeadLossFn.apply(xd, Wd, td, 15.0, "mean")).backward()
+    assert rel_l2(xd.grad, 0.37 * gx.float()) < BF16_TOL and rel_l2(Wd.grad, 0.37 * gw.float()) < BF16_TOL
+    _, lse_o = O.loss_rows(F_linear(x, W), t, 15.0)
+    grow = 0.37 * O.row_weights(t, "mean")
+    dlo = O.loss_backward(F_linear(x, W), t, lse_o, grow, 15.0)
+    assert rel_l2(xd.grad, dlo.float() @ W.float()) < BF16_TOL and rel_l2(Wd.grad, dlo.float().t() @ x.float()) < BF16_TOL
+
+
+def F_linear(x, W):
+    return (x.float() @ W.float().t()).bfloat16()
+
+
 def test_lmhead_softcap_matches_materialised_path(ops, dev):
     g = _g(22)
     N, d, V = 1024, 768, 32768
@@ -778,7 +836,7 @@ def test_newton_schulz_full_size_properties(ops, dev):
 
 
 def test_autograd_nodes_do_not_corrupt_what_autograd_cannot_see(ops, dev):
-    """RopeAttentionFn leaves its input qkv untouched (the rotation goes into a buffer of its own); LmHeadLossFn, whose
+    """RopeAttentionFn leaves its input qkv untouched (the rotation goes into a buffer of its own); LmHeadLossFn, where its
     backward overwrites the saved logits with their gradient, refuses a second backward instead of returning garbage."""
     from trainium_frontier_them_bones_amd import autograd as A
     from oracle import attention as OA
@@ -791,13 +849,25 @@ def test_autograd_nodes_do_not_corrupt_what_autograd_cannot_see(ops, dev):
     assert torch.equal(qkv.detach(), before)
     out.sum().backward()
     assert torch.equal(qkv.detach(), before) and bool(torch.isfinite(qkv.grad.float()).all())
+    # beyond the one-pass loss kernel's vocabulary limit the node saves the logits and overwrites them in its backward
+    V = 65536 + 128
+    x = torch.randn(128, 128, generator=g).bfloat16().to(dev).requires_grad_(True)
+    W = (0.05 * torch.randn(V, 128, generator=g)).bfloat16().to(dev).requires_grad_(True)
+    t = torch.randint(0, V, (128,), generator=g).to(dev)
+    loss = A.LmHeadLossFn.apply(x, W, t, 0.0, "mean")
+    loss.backward(retain_graph=True)
+    with pytest.raises(RuntimeError):
+        loss.backward()
+    # within it the saved tensor is the gradient itself, and a second backward accumulates the same gradients again
     x = torch.randn(256, 256, generator=g).bfloat16().to(dev).requires_grad_(True)
     W = (0.05 * torch.randn(1024, 256, generator=g)).bfloat16().to(dev).requires_grad_(True)
     t = torch.randint(0, 1024, (256,), generator=g).to(dev)
     loss = A.LmHeadLossFn.apply(x, W, t, 0.0, "mean")
     loss.backward(retain_graph=True)
-    with pytest.raises(RuntimeError):
-        loss.backward()
+    gx, gw = x.grad.clone(), W.grad.clone()
+    x.grad = W.grad = None
+    loss.backward()
+    assert torch.equal(x.grad, gx) and torch.equal(W.grad, gw)
 
 
 def test_hardware_probes_run_and_report_sane_rates(ops, dev):

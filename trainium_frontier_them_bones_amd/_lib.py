@@ -19,6 +19,7 @@ _fp = ctypes.POINTER(ctypes.c_float)   # a HOST array of floats (tfb_ns5's coeff
 # name -> argtypes (restype is always int status unless listed in _RESTYPE)
 SIGNATURES = {
     "tfb_gemm_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _vp],
+    "tfb_gemm_bf16_scaled": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _vp, _vp],
     "tfb_gemm_bf16_res": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "tfb_norm_bwd_blocks": [_l],
     "tfb_rmsnorm_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _f, _vp],
@@ -68,6 +69,7 @@ SIGNATURES = {
     "tfb_adamw": [_vp, _vp, _i, _vp, _vp, _vp, _l, _f, _f, _f, _f, _f, _f, _f, _vp],
     "tfb_fill_f32": [_vp, _f, _l, _vp],
     "tfb_loss_fwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
+    "tfb_loss_fwd_bwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_loss_bwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_loss_multi_fwd": [_vp, _vp, _i, _vp, _i, _f, _vp, _vp, _l, _i, _f, _vp],
     "tfb_loss_multi_bwd": [_vp, _vp, _i, _vp, _i, _f, _vp, _vp, _vp, _l, _i, _f, _vp],

@@ -485,9 +485,16 @@ class NrMlpFn(torch.autograd.Function):
         return gx, dw_fc, dw_proj, None, None
 
 
+LM_HEAD_ONE_PASS = True   # False: LmHeadLossFn always takes the GEMM with the lse epilogue and the separate loss backward
+
+
 class LmHeadLossFn(torch.autograd.Function):
-    """loss = reduce(CE(softcap(x @ W^T), targets)): the LM-head GEMM with the log-sum-exp in its epilogue, then (in
-    the backward) dlogits written in place over the logits and the two gradient GEMMs."""
+    """loss = reduce(CE(softcap(x @ W^T), targets)). When a gradient is wanted the forward is the plain LM-head GEMM followed
+    by ONE pass over the logits that writes lse and the row losses and leaves, in place of the logits, their gradient for an
+    upstream gradient of one; the backward is the two gradient GEMMs, each multiplying its product by the upstream scalar
+    (a device value) before its rounding. The logits thus make one trip to HBM each way, and nothing recomputes an
+    exponential. Without a gradient (or beyond the one-pass kernel's vocabulary limit) the GEMM with the log-sum-exp in its
+    epilogue runs instead, and a backward from there writes dlogits in place of the logits first."""
 
     @staticmethod
     def forward(ctx, x, W, targets, softcap, reduction):
@@ -495,27 +502,39 @@ class LmHeadLossFn(torch.autograd.Function):
         tg = targets.reshape(-1)
         valid = (tg >= 0).to(torch.float32)
         w = valid / valid.sum().clamp_min(1.0) if reduction == "mean" else valid
-        logits, rows, lse = ops.lmhead_fwd(x2, W, tg, softcap, w)
-        ctx.save_for_backward(x2, W, tg, logits, lse, w)
         ctx.softcap = softcap
         ctx.xshape = x.shape
+        ctx.one_pass = (LM_HEAD_ONE_PASS and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
+                        and W.shape[0] <= ops.LOSS_FWD_BWD_MAX_V)
+        if ctx.one_pass:
+            dl = ops.matmul(x2, W, trans_b=True)
+            rows, _ = ops.loss_fwd_bwd(dl, tg, w, softcap)
+            ctx.save_for_backward(x2, W, dl)
+            return rows.sum()
+        logits, rows, lse = ops.lmhead_fwd(x2, W, tg, softcap, w)
+        ctx.save_for_backward(x2, W, tg, logits, lse, w)
         return rows.sum()
 
     @staticmethod
     def backward(ctx, g):
-        x2, W, tg, logits, lse, w = ctx.saved_tensors
-        if getattr(ctx, "logits_consumed", False):
-            raise RuntimeError("LmHeadLossFn: second backward through the same node (retain_graph): the saved logits "
-                               "were overwritten by their gradient in the first one")
-        ctx.logits_consumed = True
-        grow = (w * g.to(torch.float32)).contiguous()
-        dl = ops.loss_bwd(logits, tg, lse, grow, ctx.softcap, inplace=True)
-        dx = ops.matmul(dl, W).view(ctx.xshape)
+        if ctx.one_pass:
+            x2, W, dl = ctx.saved_tensors
+            alpha = g.detach().to(torch.float32).reshape(1)
+        else:
+            x2, W, tg, logits, lse, w = ctx.saved_tensors
+            if getattr(ctx, "logits_consumed", False):
+                raise RuntimeError("LmHeadLossFn: second backward through the same node (retain_graph): the saved logits "
+                                   "were overwritten by their gradient in the first one")
+            ctx.logits_consumed = True
+            grow = (w * g.to(torch.float32)).contiguous()
+            dl = ops.loss_bwd(logits, tg, lse, grow, ctx.softcap, inplace=True)
+            alpha = None
+        dx = ops.matmul(dl, W, alpha=alpha).view(ctx.xshape)
         buf, acc = _accumulate_into(W)
         if buf is not None:
-            ops.matmul(dl, x2, trans_a=True, out=buf, accumulate=acc)
+            ops.matmul(dl, x2, trans_a=True, out=buf, accumulate=acc, alpha=alpha)
             return dx, None, None, None, None
-        return dx, ops.matmul(dl, x2, trans_a=True), None, None, None
+        return dx, ops.matmul(dl, x2, trans_a=True, alpha=alpha), None, None, None
 
 
 class FusedLossFn(torch.autograd.Function):

@@ -9,18 +9,18 @@ namespace {
 
 template <int LAYP, int LAYQ>
 int run(GemmOperand P, GemmOperand Q, int N, int M, int K, void* C, int out_f32, int accumulate, float* ws, long ws_bytes,
-        hipStream_t stream) {
+        const float* alpha, hipStream_t stream) {
   using Cfg = GemmCfg<128, 128, 2, 2, 2, LAYP, LAYQ>;
   const long tiles = (long)(N / 128) * (M / 128);
   const int splits = ws ? choose_splits(tiles, K / 64, (long)M * N, ws_bytes) : 1;
   if (splits == 1) {
-    EpiStore e{C, (long)N, out_f32, accumulate};
+    EpiStore e{C, (long)N, out_f32, accumulate, alpha};
     return gemm_launch<Cfg>(P, Q, N, M, (long)K * 2, 1, LoadIdentity{}, LoadIdentity{}, e, stream);
   }
   EpiSplit e{ws, (long)N, (long)M * N};
   int st = gemm_launch<Cfg>(P, Q, N, M, (long)K * 2, splits, LoadIdentity{}, LoadIdentity{}, e, stream);
   if (st != TFB_OK) return st;
-  return splitk_reduce(ws, C, (long)M * N, splits, out_f32, accumulate, stream);
+  return splitk_reduce(ws, C, (long)M * N, splits, out_f32, accumulate, stream, nullptr, nullptr, 1.0f, alpha);
 }
 
 // out [q][ld] = bf16(D) with the rotary embedding applied to the first rot_cols columns (heads of 64: y1 = x1 c + x2 s,
@@ -66,8 +66,11 @@ struct EpiStoreRope {
 
 }  // namespace
 
-extern "C" int tfb_gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int trans_a, int trans_b,
-                             int out_f32, int accumulate, void* workspace, long workspace_bytes, void* stream) {
+// tfb_gemm_bf16 with the product multiplied by the device fp32 scalar *alpha (NULL = 1) before its one rounding:
+// C (+)= alpha op(A) @ op(B). For gradient GEMMs whose upstream scalar lives on the device.
+extern "C" int tfb_gemm_bf16_scaled(const void* A, const void* B, void* C, int M, int N, int K, int trans_a, int trans_b,
+                                    int out_f32, int accumulate, void* workspace, long workspace_bytes, const void* alpha,
+                                    void* stream) {
   if (!A || !B || !C) return TFB_ERR_ARG;
   if (M <= 0 || N <= 0 || K <= 0 || M % 128 || N % 128 || K % 64) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
@@ -78,10 +81,16 @@ extern "C" int tfb_gemm_bf16(const void* A, const void* B, void* C, int M, int N
   P.ld = trans_b ? (long)K * 2 : (long)N * 2;
   Q.ld = trans_a ? (long)M * 2 : (long)K * 2;
   float* ws = (float*)workspace;
-  if (trans_b && !trans_a) return run<TFB_K_CONTIG, TFB_K_CONTIG>(P, Q, N, M, K, C, out_f32, accumulate, ws, workspace_bytes, s);
-  if (!trans_b && !trans_a) return run<TFB_K_STRIDED, TFB_K_CONTIG>(P, Q, N, M, K, C, out_f32, accumulate, ws, workspace_bytes, s);
-  if (!trans_b && trans_a) return run<TFB_K_STRIDED, TFB_K_STRIDED>(P, Q, N, M, K, C, out_f32, accumulate, ws, workspace_bytes, s);
-  return run<TFB_K_CONTIG, TFB_K_STRIDED>(P, Q, N, M, K, C, out_f32, accumulate, ws, workspace_bytes, s);
+  const float* al = (const float*)alpha;
+  if (trans_b && !trans_a) return run<TFB_K_CONTIG, TFB_K_CONTIG>(P, Q, N, M, K, C, out_f32, accumulate, ws, workspace_bytes, al, s);
+  if (!trans_b && !trans_a) return run<TFB_K_STRIDED, TFB_K_CONTIG>(P, Q, N, M, K, C, out_f32, accumulate, ws, workspace_bytes, al, s);
+  if (!trans_b && trans_a) return run<TFB_K_STRIDED, TFB_K_STRIDED>(P, Q, N, M, K, C, out_f32, accumulate, ws, workspace_bytes, al, s);
+  return run<TFB_K_CONTIG, TFB_K_STRIDED>(P, Q, N, M, K, C, out_f32, accumulate, ws, workspace_bytes, al, s);
+}
+
+extern "C" int tfb_gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int trans_a, int trans_b,
+                             int out_f32, int accumulate, void* workspace, long workspace_bytes, void* stream) {
+  return tfb_gemm_bf16_scaled(A, B, C, M, N, K, trans_a, trans_b, out_f32, accumulate, workspace, workspace_bytes, nullptr, stream);
 }
 
 // C [M][N] = bf16(res + bf16(A [M][K] @ op(B))), B [N][K] (trans_b) or [K][N]: a projection with the residual add that

@@ -702,10 +702,12 @@ struct EpiStore {
   long ld;  // elements
   int f32;
   int accumulate;
+  const float* alpha = nullptr;  // optional device scalar the product is multiplied by before the (one) rounding
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
     float r[8];
+    const float a = alpha ? *alpha : 1.0f;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) r[k] = v[k];
+    for (int k = 0; k < 8; ++k) r[k] = v[k] * a;
     if (f32) {
       float* o = (float*)out + (long)q * ld + p;
       if (accumulate) {
@@ -755,9 +757,10 @@ struct EpiSplit {
 };
 
 // out (+)= scale * (sum over splits of ws), rounded once; scale = imm / (*sa * *sb) (absent factors are 1: the fp8
-// GEMMs' power-of-two descale, exact)
+// GEMMs' power-of-two descale, exact), times *alpha when given
 static __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* out, long n, int splits, int f32,
-                                            int accumulate, const float* sa, const float* sb, float imm) {
+                                            int accumulate, const float* sa, const float* sb, float imm,
+                                            const float* alpha) {
   long i = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (i >= n) return;
   f32x4 s = *(const f32x4*)(ws + i);
@@ -768,6 +771,7 @@ static __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* 
     if (sb) d *= *sb;
     s *= imm / d;
   }
+  if (alpha) s *= *alpha;
   if (f32) {
     float* o = (float*)out + i;
     if (accumulate) s += *(const f32x4*)o;
@@ -787,9 +791,10 @@ static __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* 
 }
 
 static inline int splitk_reduce(const float* ws, void* out, long n, int splits, int f32, int accumulate, hipStream_t s,
-                                const float* sa = nullptr, const float* sb = nullptr, float imm = 1.0f) {
+                                const float* sa = nullptr, const float* sb = nullptr, float imm = 1.0f,
+                                const float* alpha = nullptr) {
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, s, ws, out, n, splits, f32,
-                     accumulate, sa, sb, imm);
+                     accumulate, sa, sb, imm, alpha);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

@@ -141,6 +141,107 @@ __global__ __launch_bounds__(256) void loss_bwd_kernel(const bf16_t* __restrict_
   }
 }
 
+// loss_fwd_kernel and loss_bwd_kernel for grow = row_w in ONE pass over the logits: a workgroup keeps its row in registers
+// (NCH chunks of eight values per thread, V <= 2048 NCH), reduces it to lse in the order of loss_fwd_kernel, writes lse and
+// the weighted row loss, and overwrites the row with d x_v = w (softmax_v - [v = t]) (1 - tanh^2): the gradient for an
+// upstream gradient of one, which the caller's two gradient GEMMs scale by the real one. The logits are read once and
+// written once where the two kernels read them twice; values equal theirs bit for bit.
+template <typename IDX, int NCH>
+__global__ __launch_bounds__(256) void loss_fwd_bwd_kernel(bf16_t* x, const IDX* __restrict__ tg, const float* __restrict__ row_w,
+                                                          float* __restrict__ loss, float* __restrict__ lse, int V, float cap) {
+  __shared__ float rm[4], rs[4], lsh;
+  const long row = blockIdx.x;
+  bf16_t* xr = x + row * V;
+  const float icap = cap > 0.f ? 1.0f / cap : 0.f;
+  u32x4 u[NCH];
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    const int i = threadIdx.x * 8 + j * 2048;
+    u[j] = i < V ? *(const u32x4*)(xr + i) : u32x4{0u, 0u, 0u, 0u};
+  }
+  MS a{-1e30f, 0.f};
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    if (threadIdx.x * 8 + j * 2048 < V) {
+      float v[8];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        v[2 * k] = bflo(u[j][k]);
+        v[2 * k + 1] = bfhi(u[j][k]);
+      }
+      if (cap > 0.f) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) a.s += fexp(cap * tanh_fast(v[k] * icap) - cap);
+        a.m = cap;
+      } else {
+        float mx = a.m;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) mx = fmaxf(mx, v[k]);
+        float sc = fexp(a.m - mx), t = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) t += fexp(v[k] - mx);
+        a.s = a.s * sc + t;
+        a.m = mx;
+      }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    MS b{__shfl_xor(a.m, o, 64), __shfl_xor(a.s, o, 64)};
+    a = ms_merge(a, b);
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    rm[wave] = a.m;
+    rs[wave] = a.s;
+  }
+  __syncthreads();
+  const long tt = (long)tg[row];
+  const bool valid = (unsigned long)tt < (unsigned long)V;  // a target outside [0, V) is an ignored row, never an address
+  const float w = valid ? (row_w ? row_w[row] : 1.0f) : 0.f;
+  if (threadIdx.x == 0) {
+    MS t{rm[0], rs[0]};
+    for (int i = 1; i < 4; ++i) t = ms_merge(t, MS{rm[i], rs[i]});
+    const float l = t.m + logf(t.s);
+    lse[row] = l;
+    float out = 0.f;
+    if (valid) {
+      const float xt = bf2f(xr[tt]);   // (read before any thread overwrites the row: the barrier below)
+      const float st = cap > 0.f ? cap * tanh_fast(xt * icap) : xt;
+      out = (l - st) * w;
+    }
+    loss[row] = out;
+    lsh = l;
+  }
+  __syncthreads();
+  const float l = lsh;
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    const int i = threadIdx.x * 8 + j * 2048;
+    if (i < V) {
+      float v[8], d[8];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        v[2 * k] = bflo(u[j][k]);
+        v[2 * k + 1] = bfhi(u[j][k]);
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const float hot = (i + k == tt) ? 1.0f : 0.0f;
+        if (cap > 0.f) {
+          const float t = tanh_fast(v[k] * icap);
+          const float p = fexp(cap * t - l);
+          d[k] = w * (p - hot) * (1.0f - t * t);
+        } else {
+          d[k] = w * (fexp(v[k] - l) - hot);
+        }
+      }
+      u32x4 o = {pack2bf(d[0], d[1]), pack2bf(d[2], d[3]), pack2bf(d[4], d[5]), pack2bf(d[6], d[7])};
+      *(u32x4*)(xr + i) = o;
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------ several targets / label smoothing
 // loss_row = sum_k rw_k (lse - (1 - eps) s_{t_k} - (eps / V) sum_v s_v), targets tg [K][rows] and weights rw [K][rows]
 // (a target < 0 counts with weight 0). K > 1 is the multi-token-prediction loss (round1/source/train.py:4725), eps > 0
@@ -381,6 +482,29 @@ extern "C" int tfb_loss_fwd(const void* logits, const void* targets, int idx64, 
   else
     hipLaunchKernelGGL(loss_fwd_kernel<int>, dim3((unsigned)rows), dim3(256), 0, s, (const bf16_t*)logits, (const int*)targets,
                        (const float*)row_w, (float*)loss, (float*)lse, V, softcap);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// tfb_loss_fwd followed by tfb_loss_bwd with grow = row_w (an upstream gradient of one), in place and in one pass over the
+// logits: loss and lse as tfb_loss_fwd writes them, and logits overwritten by that gradient, bit for bit what the two calls
+// give. V <= 65536 (a row is held in one workgroup's registers); status TFB_ERR_SHAPE beyond, for the caller to take the two calls.
+extern "C" int tfb_loss_fwd_bwd(void* logits, const void* targets, int idx64, const void* row_w, void* loss, void* lse, long rows,
+                                int V, float softcap, void* stream) {
+  if (!logits || !targets || !loss || !lse) return TFB_ERR_ARG;
+  if (rows <= 0 || V <= 0 || V % 8 || V > 65536) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+#define TFB_LFB(IDX, NCH)                                                                                                  \
+  hipLaunchKernelGGL((loss_fwd_bwd_kernel<IDX, NCH>), dim3((unsigned)rows), dim3(256), 0, s, (bf16_t*)logits,             \
+                     (const IDX*)targets, (const float*)row_w, (float*)loss, (float*)lse, V, softcap)
+  if (V <= 16384) {
+    if (idx64) TFB_LFB(long, 8); else TFB_LFB(int, 8);
+  } else if (V <= 32768) {
+    if (idx64) TFB_LFB(long, 16); else TFB_LFB(int, 16);
+  } else {
+    if (idx64) TFB_LFB(long, 32); else TFB_LFB(int, 32);
+  }
+#undef TFB_LFB
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

@@ -44,10 +44,13 @@ def _workspace(device, nbytes=256 << 20):
     return ws
 
 
-def matmul(a, b, trans_a=False, trans_b=False, out=None, accumulate=False, out_dtype=bf16):
+def matmul(a, b, trans_a=False, trans_b=False, out=None, accumulate=False, out_dtype=bf16, alpha=None):
     """op(a) @ op(b) with fp32 accumulation. a is [M,K] (or [K,M] with trans_a), b is [K,N] (or [N,K] with
-    trans_b). `out` (bf16 or fp32) may be given; accumulate=True adds into it (one rounding)."""
-    _chk(a), _chk(b)
+    trans_b). `out` (bf16 or fp32) may be given; accumulate=True adds into it (one rounding). alpha: a 1-element fp32
+    device tensor the product is multiplied by before that rounding (no host read-back)."""
+    _chk(a), _chk(b), _chk(alpha, torch.float32)
+    if alpha is not None and alpha.numel() != 1:
+        raise ValueError("alpha is one fp32 element")
     M, K = (a.shape[1], a.shape[0]) if trans_a else (a.shape[0], a.shape[1])
     Kb, N = (b.shape[1], b.shape[0]) if trans_b else (b.shape[0], b.shape[1])
     if K != Kb:
@@ -61,8 +64,8 @@ def matmul(a, b, trans_a=False, trans_b=False, out=None, accumulate=False, out_d
         if out.dtype not in (bf16, torch.float32) or tuple(out.shape) != (M, N):
             raise ValueError("bad out")
     ws = _workspace(a.device)
-    _lib.call("tfb_gemm_bf16", _p(a), _p(b), _p(out), M, N, K, int(trans_a), int(trans_b),
-              int(out.dtype == torch.float32), int(accumulate), _p(ws), ws.numel() * 4, _stream())
+    _lib.call("tfb_gemm_bf16_scaled", _p(a), _p(b), _p(out), M, N, K, int(trans_a), int(trans_b),
+              int(out.dtype == torch.float32), int(accumulate), _p(ws), ws.numel() * 4, _p(alpha), _stream())
     return out
 
 
@@ -683,6 +686,22 @@ def loss_bwd(logits2, targets, lse, grow, softcap=15.0, inplace=False):
     _lib.call("tfb_loss_bwd", _p(logits2), _p(tg), int(tg.dtype == torch.int64), _p(lse), _p(grow), _p(out), N, V,
               float(softcap or 0.0), _stream())
     return out
+
+
+LOSS_FWD_BWD_MAX_V = 65536
+
+
+def loss_fwd_bwd(logits2, targets, row_w=None, softcap=15.0):
+    """(loss rows fp32 [N], lse fp32 [N]) as loss_fwd gives them, and logits2 OVERWRITTEN by the gradient of sum(rows):
+    row_w (softmax - onehot) (1 - tanh^2), what loss_bwd gives for grow = row_w. One pass over the logits; V <= 65536."""
+    _chk(logits2), _chk(row_w, torch.float32)
+    tg = _tg(targets)
+    N, V = logits2.shape
+    loss = torch.empty(N, dtype=torch.float32, device=logits2.device)
+    lse = torch.empty(N, dtype=torch.float32, device=logits2.device)
+    _lib.call("tfb_loss_fwd_bwd", _p(logits2), _p(tg), int(tg.dtype == torch.int64), _p(row_w), _p(loss), _p(lse), N, V,
+              float(softcap or 0.0), _stream())
+    return loss, lse
 
 
 def loss_multi_fwd(logits2, targets, row_w, softcap=15.0, eps=0.0):
