@@ -21,6 +21,12 @@
 // contiguous, so q/k/v may be thirds of a fused qkv [B,T,3C] buffer and o / dO are [B,T,H,D].
 #include "common.hpp"
 
+#ifndef TFB_ATTN128_XCD
+#define TFB_ATTN128_XCD 1  // re-deal workgroups so that a (batch, head) pair's blocks share an XCD's L2
+#endif
+#ifndef TFB_FWD128_WPE
+#define TFB_FWD128_WPE 2  // D = 128 forward: 262 registers at one wavefront per SIMD, 70 KB of LDS: two workgroups fit a CU at 256
+#endif
 #ifndef TFB_FWD_WPE
 #define TFB_FWD_WPE 3  // wavefronts per SIMD the forward kernel is compiled for (register budget 512 / WPE)
 #endif
@@ -93,6 +99,21 @@ __device__ __forceinline__ void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0x
 
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
+// Workgroup -> (block along the sequence, batch*head): consecutive workgroup ids go round-robin to the 8 XCDs, each with
+// its own L2, so the ids are re-dealt to keep all sequence blocks of one (batch, head) - which stream the same K / V (or
+// Q / dO) tiles - on one XCD (the D = 64 kernels do the same). nx = blocks per (batch, head), nbh = batch*head count.
+__device__ __forceinline__ void xcd_block128(int nx, int nbh, int& bx, int& bh) {
+  const int lin = blockIdx.y * nx + blockIdx.x;
+  if (TFB_ATTN128_XCD && nbh % 8 == 0) {
+    const int xcd = lin & 7, idx = lin >> 3;
+    bh = xcd + 8 * (idx / nx);
+    bx = idx % nx;
+  } else {
+    bh = blockIdx.y;
+    bx = blockIdx.x;
+  }
+}
+
 // LDS row of a transposed tile: 64 tokens + 8 bytes of pad. With 32 banks and 64-bit accesses resolved per 16 lanes,
 // a 136-byte stride puts the 16 rows a half-wavefront's fragment read touches on 16 different bank pairs, and the
 // transposing writes (16 consecutive lanes along the tokens of one row) are conflict-free as well.
@@ -102,7 +123,7 @@ constexpr int TROW = 64 * 2 + 8;
 // QG = query groups of 32 per wavefront. With QG = 2 every K / V^T fragment read from LDS feeds two MFMAs (half the LDS
 // traffic per flop) and the two groups' softmax arithmetic and MFMAs are independent instruction streams that co-execute.
 template <int D, int QG>
-__global__ __launch_bounds__(256, (D == 64 && QG == 1) ? TFB_FWD_WPE : 1) void attn_fwd_kernel(AttnT q, AttnT k, AttnT v, AttnT o, float* __restrict__ lse, int T,
+__global__ __launch_bounds__(256, (D == 64 && QG == 1) ? TFB_FWD_WPE : (QG == 1 ? TFB_FWD128_WPE : 1)) void attn_fwd_kernel(AttnT q, AttnT k, AttnT v, AttnT o, float* __restrict__ lse, int T,
                                                       int H, float sl2, int nw) {
   constexpr int DS = D / 16, DT = D / 32, NV = D / 64;
   constexpr int KROW = D * 2 + 16;
@@ -110,8 +131,10 @@ __global__ __launch_bounds__(256, (D == 64 && QG == 1) ? TFB_FWD_WPE : 1) void a
   constexpr int QB = 128 * QG, QW = 32 * QG;  // queries per workgroup / per wavefront
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
-  const int qb = gridDim.x - 1 - blockIdx.x;  // longest rows first
-  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  int bx, bh;
+  xcd_block128(gridDim.x, gridDim.y, bx, bh);
+  const int qb = gridDim.x - 1 - bx;  // longest rows first
+  const int b = bh / H, h = bh % H;
   const bf16_t* qp = q.p + b * q.sb + h * q.sh;
   const bf16_t* kp = k.p + b * k.sb + h * k.sh;
   const bf16_t* vp = v.p + b * v.sb + h * v.sh;
@@ -317,8 +340,9 @@ __global__ __launch_bounds__(256, D == 64 ? TFB_DKDV_WPE : 1) void attn_bwd_dkdv
   constexpr int OFF_L = 2 * NBYTES + 2 * TBYTES, BUF = OFF_L + 512;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
-  const int kb = blockIdx.x;  // low key blocks see the most query tiles: already longest first
-  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  int kb, bh;  // low key blocks see the most query tiles: already longest first
+  xcd_block128(gridDim.x, gridDim.y, kb, bh);
+  const int b = bh / H, h = bh % H;
   const bf16_t* qp = q.p + b * q.sb + h * q.sh;
   const bf16_t* kp = k.p + b * k.sb + h * k.sh;
   const bf16_t* vp = v.p + b * v.sb + h * v.sh;
@@ -464,8 +488,10 @@ __global__ __launch_bounds__(256, D == 64 ? TFB_DQ_WPE : 1) void attn_bwd_dq_ker
   constexpr int OFF_KN = 0, OFF_VN = NBYTES, OFF_KT = 2 * NBYTES, BUF = 2 * NBYTES + TBYTES;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
-  const int qb = gridDim.x - 1 - blockIdx.x;
-  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  int bx, bh;
+  xcd_block128(gridDim.x, gridDim.y, bx, bh);
+  const int qb = gridDim.x - 1 - bx;
+  const int b = bh / H, h = bh % H;
   const bf16_t* qp = q.p + b * q.sb + h * q.sh;
   const bf16_t* kp = k.p + b * k.sb + h * k.sh;
   const bf16_t* vp = v.p + b * v.sb + h * v.sh;
