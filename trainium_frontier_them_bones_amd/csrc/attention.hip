@@ -30,6 +30,9 @@
 #ifndef TFB_FWD_WPE
 #define TFB_FWD_WPE 3  // wavefronts per SIMD the forward kernel is compiled for (register budget 512 / WPE)
 #endif
+#ifndef TFB_DKDV128_WPE
+#define TFB_DKDV128_WPE 1  // D = 128 dK/dV: 326 registers; at two wavefronts per SIMD it spills 36 and runs 0.90 vs 0.80 ms
+#endif
 #ifndef TFB_DKDV_WPE
 #define TFB_DKDV_WPE 2
 #endif
@@ -330,7 +333,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(AttnT o, AttnT go, floa
 
 // =========================================================================================== dK / dV
 template <int D>
-__global__ __launch_bounds__(256, D == 64 ? TFB_DKDV_WPE : 1) void attn_bwd_dkdv_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dk, AttnT dv,
+__global__ __launch_bounds__(256, D == 64 ? TFB_DKDV_WPE : TFB_DKDV128_WPE) void attn_bwd_dkdv_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dk, AttnT dv,
                                                            const float* __restrict__ lse, const float* __restrict__ delta,
                                                            int T, int H, float scale, float sl2, int nw) {
   constexpr int DS = D / 16, DT = D / 32, NV = D / 64;
