@@ -358,8 +358,9 @@ int tfb_moe_tables(const void* idx, void* cnt, void* seg, void* tile_expert, voi
 int tfb_moe_tables_cap(const void* idx, void* cnt, void* cnt_all, void* seg, void* tile_expert, void* slot, void* tok, void* ksel,
                        void* scratch, long N, long T, int cap, int E, int topk, long rmax, void* stream);
 
-/* xs bf16 [rmax][d] = h[tok] (zero padding rows) and xs8 = e4m3(xs * scale) (scale_ptr device fp32 or scale_imm; xs8 may
- * be NULL: bf16 experts take no fp8 copy). Replaces MoeDispatch2.forward (round2/source/train.py:10652-10660). */
+/* xs bf16 [rmax][d] = h[tok] (zero padding rows) and xs8 = e4m3(xs * scale) (scale_ptr device fp32 or scale_imm; either
+ * output may be NULL: bf16 experts take no fp8 copy, fp8 experts with fp8 weight gradients no bf16 one).
+ * Replaces MoeDispatch2.forward (round2/source/train.py:10652-10660). */
 int tfb_moe_gather(const void* h, const void* tok, const void* scale_ptr, float scale_imm, void* xs, void* xs8, long rmax, int d,
                    void* stream);
 

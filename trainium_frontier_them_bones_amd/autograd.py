@@ -653,7 +653,7 @@ class MoeMlp8Fn(torch.autograd.Function):
         # `capacity` assignments per expert; None keeps everything
         tab = ops.moe_tables(idx, E) if capacity is None else ops.moe_tables(idx, E, h.shape[-2], capacity)
         if state is not None:
-            xs, xs8 = ops.moe_gather(h2, tab, state.x_scale)
+            xs, xs8 = ops.moe_gather(h2, tab, state.x_scale, want_xs=not state.dw_fp8)
             ys, r = ops.moe_mlp8_fwd(xs8, state.w8, state.rows, tab, F)
         else:
             xs, _ = ops.moe_gather(h2, tab, None)

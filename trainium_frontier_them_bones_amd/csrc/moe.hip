@@ -439,7 +439,7 @@ __global__ void fill_i32_kernel(int* __restrict__ p, int val, long n) {
 }
 
 // ------------------------------------------------------------------------------------------------ dispatch / combine
-// xs[row] = h[tok[row]] (zero rows for padding), and its e4m3 cast at `scale`.
+// xs[row] = h[tok[row]] (zero rows for padding), and / or its e4m3 cast at `scale`.
 __global__ __launch_bounds__(256) void moe_gather_kernel(const bf16_t* __restrict__ h, const int* __restrict__ tok,
                                                         const float* __restrict__ scale_ptr, float scale_imm,
                                                         bf16_t* __restrict__ xs, uint8_t* __restrict__ xs8, long rmax, int d) {
@@ -452,7 +452,7 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const bf16_t* __restric
     int t = tok[row];
     float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     if (t >= 0) load8(h + (long)t * d + c, v);
-    store8(xs + row * d + c, v);
+    if (xs) store8(xs + row * d + c, v);
     if (xs8) {
       u32x2 o = {cvt4_fp8<TFB_FMT_E4M3>(v[0] * sc, v[1] * sc, v[2] * sc, v[3] * sc),
                  cvt4_fp8<TFB_FMT_E4M3>(v[4] * sc, v[5] * sc, v[6] * sc, v[7] * sc)};
@@ -1029,7 +1029,8 @@ extern "C" int tfb_moe_tables_cap(const void* idx, void* cnt, void* cnt_all, voi
 // xs bf16 [rmax][d] = h[tok] (zero padding rows), xs8 = e4m3(xs * scale). Replaces MoeDispatch2.forward (10652-10660).
 extern "C" int tfb_moe_gather(const void* h, const void* tok, const void* scale_ptr, float scale_imm, void* xs, void* xs8,
                               long rmax, int d, void* stream) {
-  if (!h || !tok || !xs) return TFB_ERR_ARG;   // xs8 may be null: bf16 experts take no fp8 copy
+  if (!h || !tok || (!xs && !xs8)) return TFB_ERR_ARG;   // either copy may be left out (bf16 experts take no fp8 rows; fp8 experts
+                                                        // with fp8 weight gradients no bf16 ones)
   if (rmax <= 0 || d <= 0 || d % 8) return TFB_ERR_SHAPE;
   hipLaunchKernelGGL(moe_gather_kernel, dim3(nblocks(rmax * (d / 8))), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)h,
                      (const int*)tok, (const float*)scale_ptr, scale_imm, (bf16_t*)xs, (uint8_t*)xs8, rmax, d);

@@ -794,12 +794,13 @@ def moe_tables(idx, E, seq_len=None, capacity=None):
     return t
 
 
-def moe_gather(h2, tab, x_scale=4.0):
-    """(xs bf16 [rmax,d], xs8 uint8 [rmax,d]); x_scale None: no fp8 copy (xs8 is None)."""
+def moe_gather(h2, tab, x_scale=4.0, want_xs=True):
+    """(xs bf16 [rmax,d], xs8 uint8 [rmax,d]); x_scale None: no fp8 copy (xs8 is None); want_xs False: no bf16 copy (xs is
+    None: fp8 experts whose weight gradients are in fp8 too never read it)."""
     _chk(h2)
     d = h2.shape[1]
     rmax = tab["rmax"]
-    xs = torch.empty(rmax, d, dtype=bf16, device=h2.device)
+    xs = torch.empty(rmax, d, dtype=bf16, device=h2.device) if want_xs or x_scale is None else None
     if x_scale is None:
         _lib.call("tfb_moe_gather", _p(h2), _p(tab["tok"]), None, 1.0, _p(xs), None, rmax, d, _stream())
         return xs, None
