@@ -50,7 +50,8 @@ int tfb_rmsnorm_fwd(const void* x, const void* res, const void* w, void* s_out, 
 /* tfb_rmsnorm_fwd that also writes y8 [nrows][C] = e4m3(bf16(y) * y8_scale): the operand cast of the fp8 GEMM that
  * consumes y (tfb_mlp8_fwd's x8 at the constant scale 4, tfb_gemm_fp8's a8), made in the norm's pass instead of one of
  * its own. Replaces the norm prologue of _mlp8_fwd_nr_kernel (round2/source/kernels/nki_mlp_nr8.py:1032: xn, rs and the
- * casts at X_SCALE) and of _proj8_fwd_nm_kernel (round2/source/kernels/nki_attn_nr8.py:929). */
+ * casts at X_SCALE) and of _proj8_fwd_nm_kernel (round2/source/kernels/nki_attn_nr8.py:929). y may be NULL here: with the
+ * weight gradients in fp8 too nothing reads the bf16 rows, and they are then not written. */
 int tfb_rmsnorm_fwd_q(const void* x, const void* res, const void* w, void* s_out, void* y, void* inv, void* y8,
                       float y8_scale, long nrows, int C, float eps, void* stream);
 

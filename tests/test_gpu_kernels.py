@@ -396,6 +396,34 @@ def test_mlp8_activation_scale_from_the_device(ops, dev):
         ops.mlp8_forward_scales(wf, wp, 448.0, sc)                                       # three elements: not a scalar
 
 
+def test_norm_that_writes_only_the_bytes_the_mlp_reads(ops, dev):
+    """RMSNormPassFn(bytes_only) -> Mlp8Fn with fp8 weight gradients: the norm's bf16 rows are not written (the tensor handed
+    on is a storage-less NaN placeholder) and outputs and gradients equal the path that writes them, bit for bit."""
+    from trainium_frontier_them_bones_amd import autograd as A
+    M, d, F = 1024, 256, 512
+    g = _g(515)
+    x = torch.randn(4, M // 4, d, generator=g).bfloat16().to(dev)
+    nw = (1 + 0.1 * torch.randn(d, generator=g)).bfloat16().to(dev)
+    wf = (0.02 * torch.randn(F, d, generator=g)).bfloat16().to(dev)
+    wp = (0.02 * torch.randn(d, F, generator=g)).bfloat16().to(dev)
+    dy = torch.randn(4, M // 4, d, generator=g).bfloat16().to(dev)
+    outs = []
+    for bytes_only in (False, True):
+        xl, nl, wfl, wpl = (t.clone().requires_grad_(True) for t in (x, nw, wf, wp))
+        st = A.Mlp8State(dw_fp8=True)
+        st.refresh(wfl, wpl)
+        s, h, h8 = A.RMSNormPassFn.apply(xl, nl, 1e-6, st.x_scale, bytes_only)
+        if bytes_only:
+            assert h.shape == x.shape and h.stride() == (0, 0, 0) and bool(torch.isnan(h).all())
+        y = A.Mlp8Fn.apply(h, wfl, wpl, st, h8, s)
+        y.backward(dy)
+        outs.append((y.detach(), xl.grad, nl.grad, wfl.grad, wpl.grad))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    with pytest.raises(ValueError):
+        A.RMSNormPassFn.apply(x, nw, 1e-6, None, True)
+
+
 def test_mlp8_layer_replayed_as_a_hip_graph(ops, dev):
     """The fp8 MLP layer with everything per-step inside (amax activation scale on the device, scale row, weight packs,
     forward, backward, fp8 weight gradients) recorded once as a HIP graph: three replays on new inputs, with eager runs

@@ -60,14 +60,21 @@ class RMSNormPassFn(torch.autograd.Function):
     and nki_attn_nr8.py:929)."""
 
     @staticmethod
-    def forward(ctx, x, weight, eps, y8_scale=None):
+    def forward(ctx, x, weight, eps, y8_scale=None, bytes_only=False):
+        """bytes_only (with y8_scale): the consumer reads y8 alone (Mlp8Fn with its weight gradients in fp8 too), so the bf16
+        rows of y are not written; the y handed back is then a placeholder of y's shape without storage of its own (one NaN
+        element, expanded), there only to carry the gradient edge: whoever reads it gets NaN, not stale memory."""
         x = x.contiguous()
         ctx.set_materialize_grads(False)      # no zero tensor for the byte output's (or an unused output's) gradient
         if y8_scale is None:
+            if bytes_only:
+                raise ValueError("bytes_only needs y8_scale")
             _, y, inv = ops.rmsnorm_fwd(x, weight, eps)
             outs = (x, y)
         else:
-            _, y, inv, y8 = ops.rmsnorm_fwd_q(x, weight, eps, None, float(y8_scale))
+            _, y, inv, y8 = ops.rmsnorm_fwd_q(x, weight, eps, None, float(y8_scale), want_y=not bytes_only)
+            if y is None:
+                y = torch.full((1,), float("nan"), dtype=x.dtype, device=x.device).expand(x.shape)
             ctx.mark_non_differentiable(y8)
             outs = (x, y, y8)
         ctx.save_for_backward(x, inv, weight)
@@ -78,14 +85,14 @@ class RMSNormPassFn(torch.autograd.Function):
         x, inv, weight = ctx.saved_tensors
         gs = None if gs is None else gs.contiguous()
         if gy is None:
-            return gs, None, None, None
+            return gs, None, None, None, None
         part = getattr(weight, "dw_part", None)
         if part is not None:
-            return ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, gs, part=part)[0], None, None, None
+            return ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, gs, part=part)[0], None, None, None, None
         buf, acc = (None, False) if weight is None else _accumulate_into(weight)
         dx, dw = ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, gs, buf, acc)
         gw = dw.to(weight.dtype) if (weight is not None and buf is None) else None
-        return dx, gw, None, None
+        return dx, gw, None, None, None
 
 
 class AddRMSNormFn(torch.autograd.Function):
@@ -409,9 +416,11 @@ class Mlp8Fn(torch.autograd.Function):
     def forward(ctx, x, w_fc, w_proj, state, x8=None, res=None):
         """x8: the bytes e4m3(x * state.x_scale) when the norm that made x already cast them (RMSNormPassFn); res: the
         block's residual, added in the second GEMM's store: y = bf16(res + bf16(MLP(x))) (nki_mlp_nr8.py:1032)."""
-        x2 = x.reshape(-1, x.shape[-1]).contiguous()
-        x8 = None if x8 is None else x8.reshape(x2.shape)
-        r2 = None if res is None else res.reshape(x2.shape).contiguous()
+        rows2 = (x.numel() // x.shape[-1], x.shape[-1])
+        x8 = None if x8 is None else x8.reshape(rows2)
+        r2 = None if res is None else res.reshape(rows2).contiguous()
+        # with the bytes given and the weight gradients in fp8 nothing reads x itself (it may be a storage-less placeholder)
+        x2 = None if (x8 is not None and state.dw_fp8) else x.reshape(rows2).contiguous()
         if state.dw_fp8:
             y, r, x8 = ops.mlp8_fwd(x2, state.w8, state.row, w_fc.shape[0], state.x_scale, want_x8=True, x8=x8, res=r2)
             ctx.save_for_backward(x8, r, w_fc, w_proj)

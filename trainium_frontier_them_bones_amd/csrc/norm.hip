@@ -134,7 +134,7 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16_t* __restri
     for (int i = 0; i < NCH; ++i)
 #pragma unroll
       for (int k = 0; k < 8; ++k) a.v[i][k] = w ? a.v[i][k] * rs * wr.v[i][k] : a.v[i][k] * rs;
-    a.store(y + row * C, C, lane);
+    if (y) a.store(y + row * C, C, lane);
     if (y8) {  // e4m3(bf16(y) * scale): the cast the fp8 GEMM that consumes y would otherwise make in a pass of its own
       a.round();
 #pragma unroll
@@ -386,7 +386,7 @@ extern "C" int tfb_norm_bwd_blocks(long nrows) { return grid_for(nrows, 1024); }
 // instead of in a pass of its own.
 static int rmsnorm_fwd_impl(const void* x, const void* res, const void* w, void* s_out, void* y, void* inv, void* y8,
                             float y8_scale, long nrows, int C, float eps, void* stream) {
-  if (!x || !y) return TFB_ERR_ARG;
+  if (!x || (!y && !y8)) return TFB_ERR_ARG;   // y may be left out when only its fp8 cast is read (both MLP GEMM kinds in fp8)
   if (res && !s_out) return TFB_ERR_ARG;
   if (!norm_shape_ok(nrows, C)) return TFB_ERR_SHAPE;
   int grid = grid_for(nrows, 8192);

@@ -234,7 +234,8 @@ class GPT:
                     att = A.RopeAttentionFn.apply(qkv, self.cos[:T], self.sin[:T], cfg.n_head, scale)
                 x = A.LinearFn.apply(att, p["w_o.%d" % i], x)
             keep(x)
-            x, h, h8m = A.RMSNormPassFn.apply(x, p["norm2.%d" % i], cfg.norm_eps, cfg.x_scale)
+            # (with the weight gradients in fp8 too the MLP reads only the norm's bytes: its bf16 rows are not written)
+            x, h, h8m = A.RMSNormPassFn.apply(x, p["norm2.%d" % i], cfg.norm_eps, cfg.x_scale, self.mlp_state[i].dw_fp8)
             x = A.Mlp8Fn.apply(h, p["w_fc.%d" % i], p["w_proj.%d" % i], self.mlp_state[i], h8m, x)
             keep(x)
             nw = p["norm1.%d" % (i + 1)] if i + 1 < cfg.n_layer else p["norm_f"]

@@ -107,13 +107,14 @@ def rmsnorm_fwd(x, weight=None, eps=2.0 ** -23, res=None):
     return s, y, inv
 
 
-def rmsnorm_fwd_q(x, weight=None, eps=2.0 ** -23, res=None, y8_scale=4.0):
+def rmsnorm_fwd_q(x, weight=None, eps=2.0 ** -23, res=None, y8_scale=4.0, want_y=True):
     """rmsnorm_fwd that also returns y8 = e4m3(bf16(y) * y8_scale) bytes, the operand cast of the fp8 GEMM that consumes y
-    (equal to quant_fp8(y, y8_scale), bit for bit). Returns (s, y, inv, y8)."""
+    (equal to quant_fp8(y, y8_scale), bit for bit). Returns (s, y, inv, y8); want_y False: the bf16 rows are not written and
+    y is None (for a consumer that reads only the bytes)."""
     _chk(x), _chk(res), _chk(weight)
     C = x.shape[-1]
     rows = x.numel() // C
-    y = torch.empty_like(x)
+    y = torch.empty_like(x) if want_y else None
     s = torch.empty_like(x) if res is not None else x
     inv = torch.empty(rows, dtype=torch.float32, device=x.device)
     y8 = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
@@ -350,14 +351,17 @@ def mlp8_fwd(x2, w8, row, F, x_scale=4.0, want_x8=False, x8=None, res=None):
     rmsnorm_fwd_q) is used instead of casting x2; with res [M,d], y = bf16(res + bf16(MLP(x))) (the block's residual add
     made in the second GEMM's store)."""
     _chk(x2), _chk(w8, torch.uint8), _chk(row, torch.float32), _chk(x8, torch.uint8), _chk(res)
-    M, d = x2.shape
+    if x2 is None and x8 is None:
+        raise ValueError("give x2 or its bytes x8")
+    M, d = x2.shape if x2 is not None else x8.shape      # x2 may be left out when its bytes are given
+    dev = w8.device
     if x8 is None:
         x8 = quant_fp8(x2, x_scale, FMT_E4M3)
     elif tuple(x8.shape) != (M, d):
         raise ValueError("x8 shape")
-    y = torch.empty(M, d, dtype=bf16, device=x2.device)
-    r = torch.empty(M, F, dtype=bf16, device=x2.device)
-    h8 = torch.empty(M, F, dtype=torch.uint8, device=x2.device)
+    y = torch.empty(M, d, dtype=bf16, device=dev)
+    r = torch.empty(M, F, dtype=bf16, device=dev)
+    h8 = torch.empty(M, F, dtype=torch.uint8, device=dev)
     if res is None:
         _lib.call("tfb_mlp8_fwd", _p(x8), _p(w8), _p(row), _p(y), _p(r), _p(h8), M, d, F, _stream())
     else:
