@@ -187,7 +187,10 @@ class CausalAttentionFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, go):
         q, k, v, o, lse = ctx.saved_tensors
-        dq, dk, dv = ops.attn_bwd(q, k, v, o, go.contiguous(), lse, ctx.scale, "bhtd", band=ctx.band)
+        # gradients in the inputs' own (contiguous [B, H, T, D]) layout: autograd then keeps them as they are instead of
+        # copying a permuted dv into that layout (34 us of the 0.72 ms that B16 H12 T2048 D64 takes forward + backward)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        ops.attn_bwd(q, k, v, o, go.contiguous(), lse, ctx.scale, "bhtd", dq, dk, dv, "bhtd", band=ctx.band)
         return dq, dk, dv, None, None
 
 
