@@ -62,6 +62,12 @@ int tfb_rmsnorm_fwd_q(const void* x, const void* res, const void* w, void* s_out
 int tfb_rmsnorm_bwd(const void* gy, const void* gs, const void* s, const void* w, const void* inv, void* dx, void* dw_part,
                     void* dw, int dw_accumulate, long nrows, int C, void* stream);
 
+/* tfb_rmsnorm_bwd that also leaves amax_part fp32 [tfb_norm_bwd_blocks(nrows)]: per workgroup, the largest |dx| it wrote
+ * (of the rounded values), for the fp8 MLP whose backward receives this dx as its dy (tfb_mlp8_backward_scales_part).
+ * Has no counterpart in the reference, whose backward_scales reads dy for its amax (nki_mlp_fused8.py:803). */
+int tfb_rmsnorm_bwd_amax(const void* gy, const void* gs, const void* s, const void* w, const void* inv, void* dx, void* dw_part,
+                         void* dw, int dw_accumulate, void* amax_part, long nrows, int C, void* stream);
+
 /* tfb_rmsnorm_bwd with dw = NULL leaves the weight gradient as per-workgroup partial sums in dw_part; this call finishes
  * `count` of them in one launch: dw[i][c] (+)= sum_r dw_part[i][r][c], i < count, r < tfb_norm_bwd_blocks(nrows)
  * (part_stride, dw_stride: floats between consecutive i). The sums are taken in a fixed order (bit-reproducible).
@@ -151,6 +157,9 @@ int tfb_mlp8_forward_scales(const void* w_fc, const void* w_proj, void* row_out,
 /* row_out = row_in with s_dy, dq_dh2, s_dp, dq_dx filled from amax(dy); scratch fp32 [1024].
  * Replaces backward_scales (nki_mlp_fused8.py:803-813). */
 int tfb_mlp8_backward_scales(const void* dy, const void* row_in, void* row_out, void* scratch, long M, int d, void* stream);
+/* The same row from npart amax partials whose maximum is amax(dy) (as tfb_rmsnorm_bwd_amax leaves them): no pass over dy.
+ * Replaces backward_scales (nki_mlp_fused8.py:803-813). */
+int tfb_mlp8_backward_scales_part(const void* amax_part, int npart, const void* row_in, void* row_out, int d, void* stream);
 
 /* out fp32 [3] = (s, 1/s, amax): s = 2^e the largest with amax(x) s <= limit, e in [e_lo, e_hi]; scratch fp32 [1024].
  * The reference's _pow2_le (nki_mlp_fused8.py:742) applied to a tensor's amax. */

@@ -424,6 +424,59 @@ def test_norm_that_writes_only_the_bytes_the_mlp_reads(ops, dev):
         A.RMSNormPassFn.apply(x, nw, 1e-6, None, True)
 
 
+def test_norm_backward_hands_its_amax_to_the_mlp_backward(ops, dev):
+    """rmsnorm_bwd(want_amax): the partials' maximum is amax of the dx it wrote, bit for bit, and the scale row taken from
+    them equals the one taken from a pass over dx. Through autograd (two norm + fp8 MLP blocks in a row, so that the first
+    block's MLP receives the second block's norm gradient): gradients with the hand-over equal those without it."""
+    from trainium_frontier_them_bones_amd import autograd as A
+    M, d, F = 1024, 256, 512
+    g = _g(616)
+    x = torch.randn(M, d, generator=g).bfloat16().to(dev)
+    gy = torch.randn(M, d, generator=g).bfloat16().to(dev)
+    gs = (torch.randn(M, d, generator=g) * torch.logspace(-2, 1, M)[:, None]).bfloat16().to(dev)
+    nw = (1 + 0.1 * torch.randn(d, generator=g)).bfloat16().to(dev)
+    _, _, inv = ops.rmsnorm_fwd(x, nw, 1e-6)
+    dx0, dw0 = ops.rmsnorm_bwd(gy, x, inv, nw, gs)
+    dx1, dw1, am = ops.rmsnorm_bwd(gy, x, inv, nw, gs, want_amax=True)
+    assert torch.equal(dx0, dx1) and torch.equal(dw0, dw1)
+    assert float(am.max()) == float(dx1.float().abs().max()) and am.numel() == ops.norm_bwd_blocks(M)
+    wf = (0.02 * torch.randn(F, d, generator=g)).bfloat16().to(dev)
+    wp = (0.02 * torch.randn(d, F, generator=g)).bfloat16().to(dev)
+    row = ops.mlp8_forward_scales(wf, wp)
+    assert torch.equal(ops.mlp8_backward_scales(dx1, row), ops.mlp8_backward_scales(dx1, row, am))
+
+    def two_blocks(hint):
+        old = A.USE_AMAX_HINT
+        A.USE_AMAX_HINT = hint
+        try:
+            xl = x.clone().requires_grad_(True)
+            ps = [t.clone().requires_grad_(True) for t in (nw, wf, wp, nw, wf, wp)]
+            h = xl
+            for b in range(2):
+                n_, f_, p_ = ps[3 * b:3 * b + 3]
+                st = A.Mlp8State(dw_fp8=True)
+                st.refresh(f_, p_)
+                s_, y_, y8_ = A.RMSNormPassFn.apply(h, n_, 1e-6, st.x_scale, True)
+                h = A.Mlp8Fn.apply(y_, f_, p_, st, y8_, s_)
+            h.backward(gy)
+            return [xl.grad] + [t.grad for t in ps]
+        finally:
+            A.USE_AMAX_HINT = old
+
+    seen = []
+    real = ops.mlp8_backward_scales
+    ops.mlp8_backward_scales = lambda dy2, row_, amax_part=None: (seen.append(amax_part is not None), real(dy2, row_, amax_part))[1]
+    try:
+        with_hint = two_blocks(True)
+        assert seen == [False, True]           # the last block's dy comes from outside, the first block's from the norm backward
+        without = two_blocks(False)
+        assert seen == [False, True, False, False]
+    finally:
+        ops.mlp8_backward_scales = real
+    for a, b in zip(with_hint, without):
+        assert torch.equal(a, b)
+
+
 def test_mlp8_layer_replayed_as_a_hip_graph(ops, dev):
     """The fp8 MLP layer with everything per-step inside (amax activation scale on the device, scale row, weight packs,
     forward, backward, fp8 weight gradients) recorded once as a HIP graph: three replays on new inputs, with eager runs

@@ -25,12 +25,14 @@ SIGNATURES = {
     "tfb_rmsnorm_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_rmsnorm_fwd_q": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _l, _i, _f, _vp],
     "tfb_rmsnorm_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _l, _i, _vp],
+    "tfb_rmsnorm_bwd_amax": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _l, _i, _vp],
     "tfb_norm_dw_finish": [_vp, _vp, _i, _l, _l, _i, _l, _i, _vp],
     "tfb_block_head_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_block_head_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _vp],
     "tfb_mlp8_scale_scratch_floats": [_i],
     "tfb_mlp8_forward_scales": [_vp, _vp, _vp, _vp, _i, _i, _f, _f, _vp, _vp],
     "tfb_mlp8_backward_scales": [_vp, _vp, _vp, _vp, _l, _i, _vp],
+    "tfb_mlp8_backward_scales_part": [_vp, _i, _vp, _vp, _i, _vp],
     "tfb_amax_scale": [_vp, _l, _f, _i, _i, _vp, _vp, _vp],
     "tfb_quant_fp8": [_vp, _vp, _f, _i, _vp, _l, _vp],
     "tfb_mlp8_precast": [_vp, _vp, _vp, _vp, _i, _i, _vp],

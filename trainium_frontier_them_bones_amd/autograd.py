@@ -52,6 +52,16 @@ class RMSNormFn(torch.autograd.Function):
         return dx, dw.to(weight.dtype), None
 
 
+AMAX_HINT = "_tfb_amax_part"   # attribute on a gradient tensor: fp32 partials whose maximum is the tensor's amax
+USE_AMAX_HINT = True           # False: consumers ignore the attribute and read the tensor for its amax
+
+
+def _amax_hint(g, g2):
+    """The amax partials the producer of gradient g attached to it, when g2 (the rows the caller will use) is g's own memory."""
+    am = getattr(g, AMAX_HINT, None) if USE_AMAX_HINT else None
+    return am if (am is not None and g2.data_ptr() == g.data_ptr() and g2.numel() == g.numel()) else None
+
+
 class RMSNormPassFn(torch.autograd.Function):
     """(x, y[, y8]) = (x, RMSNorm(x) * weight[, e4m3(y * y8_scale)]) for a residual stream whose adds are made in the
     stores of the projections (LinearFn / Linear8Fn / Mlp8Fn with `res`): x is handed through so that the stream's
@@ -86,11 +96,16 @@ class RMSNormPassFn(torch.autograd.Function):
         gs = None if gs is None else gs.contiguous()
         if gy is None:
             return gs, None, None, None, None
+        # the gradient handed upstream carries its amax partials (attribute AMAX_HINT): an fp8 MLP whose backward receives
+        # this very tensor as its dy takes its scales from them instead of reading it once more
         part = getattr(weight, "dw_part", None)
         if part is not None:
-            return ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, gs, part=part)[0], None, None, None, None
+            dx, _, am = ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, gs, part=part, want_amax=True)
+            setattr(dx, AMAX_HINT, am)
+            return dx, None, None, None, None
         buf, acc = (None, False) if weight is None else _accumulate_into(weight)
-        dx, dw = ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, gs, buf, acc)
+        dx, dw, am = ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, gs, buf, acc, want_amax=True)
+        setattr(dx, AMAX_HINT, am)
         gw = dw.to(weight.dtype) if (weight is not None and buf is None) else None
         return dx, gw, None, None, None
 
@@ -439,7 +454,7 @@ class Mlp8Fn(torch.autograd.Function):
         x2, r, w_fc, w_proj = ctx.saved_tensors
         st = ctx.state
         g2 = gy.reshape(-1, gy.shape[-1]).contiguous()
-        rowb = ops.mlp8_backward_scales(g2, st.row)
+        rowb = ops.mlp8_backward_scales(g2, st.row, _amax_hint(gy, g2))
         if st.dw_fp8:
             dx, _, dp8, hq8, dy8 = ops.mlp8_bwd_q(g2, r, st.w8, rowb, st.e4m3_limit, want_dpre=False)
             (bf, af), (bp, ap) = _accumulate_into(w_fc), _accumulate_into(w_proj)

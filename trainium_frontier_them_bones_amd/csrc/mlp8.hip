@@ -588,6 +588,18 @@ extern "C" int tfb_mlp8_backward_scales(const void* dy, const void* row_in, void
   return TFB_OK;
 }
 
+// tfb_mlp8_backward_scales from amax partials that the producer of dy left (tfb_rmsnorm_bwd_amax: npart values whose
+// maximum is amax(dy)): the same row, without the pass over dy. d = dy's row length.
+extern "C" int tfb_mlp8_backward_scales_part(const void* amax_part, int npart, const void* row_in, void* row_out, int d,
+                                             void* stream) {
+  if (!amax_part || !row_in || !row_out) return TFB_ERR_ARG;
+  if (npart <= 0 || d <= 0) return TFB_ERR_SHAPE;
+  hipLaunchKernelGGL(backward_scales_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const float*)amax_part, npart,
+                     (const float*)row_in, (float)(36.16 * (double)d), (float*)row_out);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
 // out: fp32 [3] device = {s, 1/s, amax}: per-tensor power-of-two scale from the exact amax.
 extern "C" int tfb_amax_scale(const void* x, long n, float limit, int e_lo, int e_hi, void* out, void* scratch,
                               void* stream) {

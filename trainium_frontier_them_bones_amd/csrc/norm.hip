@@ -158,9 +158,12 @@ template <int NCH>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16_t* __restrict__ gy, const bf16_t* __restrict__ gs,
                                                          const bf16_t* __restrict__ s, const bf16_t* __restrict__ w,
                                                          const float* __restrict__ inv, bf16_t* __restrict__ dx,
-                                                         float* __restrict__ dw_part, long nrows, int C) {
+                                                         float* __restrict__ dw_part, float* __restrict__ amax_part, long nrows,
+                                                         int C) {
   __shared__ float red[ROWS_PER_BLOCK][NCH * 512];
+  __shared__ float amred[ROWS_PER_BLOCK];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float am = 0.f;   // amax of the rounded dx this wavefront wrote (amax_part: one value per workgroup)
   Row<NCH> wr, dwacc;
   if (w) wr.load(w, C, lane);
   dwacc.zero();
@@ -207,7 +210,27 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16_t* __restri
 #pragma unroll
         for (int k = 0; k < 8; ++k) g.v[i][k] += r.v[i][k];
     }
+    if (amax_part) {
+      g.round();
+#pragma unroll
+      for (int i = 0; i < NCH; ++i)
+        if ((lane + 64 * i) * 8 < C) {
+#pragma unroll
+          for (int k = 0; k < 8; ++k) am = fmaxf(am, fabsf(g.v[i][k]));
+        }
+    }
     g.store(dx + row * C, C, lane);
+  }
+  if (amax_part) {
+    am = wave_max(am);
+    if (lane == 0) amred[wave] = am;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float t = amred[0];
+#pragma unroll
+      for (int r = 1; r < ROWS_PER_BLOCK; ++r) t = fmaxf(t, amred[r]);
+      amax_part[blockIdx.x] = t;
+    }
   }
   if (w && dw_part) {
 #pragma unroll
@@ -410,8 +433,8 @@ extern "C" int tfb_rmsnorm_fwd_q(const void* x, const void* res, const void* w, 
 }
 
 // dw_part: fp32 [tfb_norm_bwd_blocks(nrows)][C] scratch (only when w != NULL); dw: fp32 [C].
-extern "C" int tfb_rmsnorm_bwd(const void* gy, const void* gs, const void* s, const void* w, const void* inv, void* dx,
-                               void* dw_part, void* dw, int dw_accumulate, long nrows, int C, void* stream) {
+static int rmsnorm_bwd_impl(const void* gy, const void* gs, const void* s, const void* w, const void* inv, void* dx,
+                            void* dw_part, void* dw, int dw_accumulate, void* amax_part, long nrows, int C, void* stream) {
   if (!gy || !s || !inv || !dx) return TFB_ERR_ARG;
   if (w && !dw_part) return TFB_ERR_ARG;
   if (!norm_shape_ok(nrows, C)) return TFB_ERR_SHAPE;
@@ -419,7 +442,7 @@ extern "C" int tfb_rmsnorm_bwd(const void* gy, const void* gs, const void* s, co
 #define CALL(N)                                                                                                        \
   hipLaunchKernelGGL(rmsnorm_bwd_kernel<N>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)gy,          \
                      (const bf16_t*)gs, (const bf16_t*)s, (const bf16_t*)w, (const float*)inv, (bf16_t*)dx,            \
-                     (float*)dw_part, nrows, C)
+                     (float*)dw_part, (float*)amax_part, nrows, C)
   DISPATCH_NCH(C, CALL);
 #undef CALL
   TFB_LAUNCH_CHECK();
@@ -429,6 +452,20 @@ extern "C" int tfb_rmsnorm_bwd(const void* gy, const void* gs, const void* s, co
     TFB_LAUNCH_CHECK();
   }
   return TFB_OK;
+}
+
+extern "C" int tfb_rmsnorm_bwd(const void* gy, const void* gs, const void* s, const void* w, const void* inv, void* dx,
+                               void* dw_part, void* dw, int dw_accumulate, long nrows, int C, void* stream) {
+  return rmsnorm_bwd_impl(gy, gs, s, w, inv, dx, dw_part, dw, dw_accumulate, nullptr, nrows, C, stream);
+}
+// tfb_rmsnorm_bwd that also leaves amax_part fp32 [tfb_norm_bwd_blocks(nrows)]: per workgroup, the largest |dx| it wrote
+// (of the rounded values). The fp8 MLP whose backward receives this dx as its dy takes its scales from these
+// (tfb_mlp8_backward_scales_part) instead of reading dy once more for its amax.
+extern "C" int tfb_rmsnorm_bwd_amax(const void* gy, const void* gs, const void* s, const void* w, const void* inv, void* dx,
+                                    void* dw_part, void* dw, int dw_accumulate, void* amax_part, long nrows, int C,
+                                    void* stream) {
+  if (!amax_part) return TFB_ERR_ARG;
+  return rmsnorm_bwd_impl(gy, gs, s, w, inv, dx, dw_part, dw, dw_accumulate, amax_part, nrows, C, stream);
 }
 
 // Finish `count` weight gradients at once: dw[i][c] (+)= sum_r part[i][r][c], part = count blocks of

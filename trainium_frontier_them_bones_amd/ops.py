@@ -123,19 +123,30 @@ def rmsnorm_fwd_q(x, weight=None, eps=2.0 ** -23, res=None, y8_scale=4.0, want_y
     return s, y, inv, y8
 
 
-def rmsnorm_bwd(gy, s, inv, weight=None, gs=None, dw=None, accumulate=False, part=None):
+def rmsnorm_bwd(gy, s, inv, weight=None, gs=None, dw=None, accumulate=False, part=None, want_amax=False):
     """dx = gs + J^T(gy) for y = RMSNorm(s) * weight. Returns (dx, dw fp32 [C] or None); a given dw is written, or
     added into with accumulate=True. With `part` (fp32 [tfb_norm_bwd_blocks(rows), C]) the weight gradient is left there
-    as partial sums for norm_dw_finish and None is returned for it."""
+    as partial sums for norm_dw_finish and None is returned for it. want_amax: a third value, fp32 [tfb_norm_bwd_blocks(rows)]
+    whose maximum is amax(dx) (per-workgroup partials, for mlp8_backward_scales(..., amax_part=))."""
     _chk(gy), _chk(s), _chk(weight), _chk(gs), _chk(inv, torch.float32)
     C = s.shape[-1]
     rows = s.numel() // C
     dx = torch.empty_like(s)
     acc = 0
+    am = torch.empty(_lib.lib().tfb_norm_bwd_blocks(rows), dtype=torch.float32, device=s.device) if want_amax else None
+
+    def call(part_, dw_, acc_):
+        if want_amax:
+            _lib.call("tfb_rmsnorm_bwd_amax", _p(gy), _p(gs), _p(s), _p(weight), _p(inv), _p(dx), _p(part_), _p(dw_), acc_, _p(am),
+                      rows, C, _stream())
+        else:
+            _lib.call("tfb_rmsnorm_bwd", _p(gy), _p(gs), _p(s), _p(weight), _p(inv), _p(dx), _p(part_), _p(dw_), acc_, rows, C,
+                      _stream())
+
     if weight is not None and part is not None:
         _chk(part, torch.float32)
-        _lib.call("tfb_rmsnorm_bwd", _p(gy), _p(gs), _p(s), _p(weight), _p(inv), _p(dx), _p(part), None, 0, rows, C, _stream())
-        return dx, None
+        call(part, None, 0)
+        return (dx, None, am) if want_amax else (dx, None)
     if weight is not None:
         nb = _lib.lib().tfb_norm_bwd_blocks(rows)
         part = torch.empty(nb, C, dtype=torch.float32, device=s.device)
@@ -144,9 +155,8 @@ def rmsnorm_bwd(gy, s, inv, weight=None, gs=None, dw=None, accumulate=False, par
         else:
             _chk(dw, torch.float32)
             acc = int(accumulate)
-    _lib.call("tfb_rmsnorm_bwd", _p(gy), _p(gs), _p(s), _p(weight), _p(inv), _p(dx), _p(part), _p(dw), acc, rows, C,
-              _stream())
-    return dx, dw
+    call(part, dw, acc)
+    return (dx, dw, am) if want_amax else (dx, dw)
 
 
 def norm_bwd_blocks(rows):
@@ -247,10 +257,15 @@ def mlp8_refresh_layers(w_fc0, w_proj0, layer_stride, layers, e4m3_limit=240.0, 
     return rows, w8
 
 
-def mlp8_backward_scales(dy2, row):
-    _chk(dy2), _chk(row, torch.float32)
+def mlp8_backward_scales(dy2, row, amax_part=None):
+    """The backward call's scale row from amax(dy2), or from amax_part (fp32 partials whose maximum is that amax, as
+    rmsnorm_bwd(want_amax=True) leaves them for the dx it wrote) without reading dy2."""
+    _chk(dy2), _chk(row, torch.float32), _chk(amax_part, torch.float32)
     M, d = dy2.shape
     out = torch.empty(NSC, dtype=torch.float32, device=dy2.device)
+    if amax_part is not None:
+        _lib.call("tfb_mlp8_backward_scales_part", _p(amax_part), amax_part.numel(), _p(row), _p(out), d, _stream())
+        return out
     scr = _scratch(dy2.device, 4096)
     _lib.call("tfb_mlp8_backward_scales", _p(dy2), _p(row), _p(out), _p(scr), M, d, _stream())
     return out
