@@ -118,7 +118,7 @@ def _work(name, a):
     if name in ("tfb_rmsnorm_fwd", "tfb_rmsnorm_fwd_q"):
         rows, C = a[-4:-2]
         return "RMSNorm forward", "hbm", rows * C * (2 * 2 + (1 if name.endswith("_q") else 0)) + 4.0 * rows
-    if name == "tfb_rmsnorm_bwd":
+    if name in ("tfb_rmsnorm_bwd", "tfb_rmsnorm_bwd_amax"):   # ..., nrows, C, stream
         rows, C = a[-3:-1]
         return "RMSNorm backward", "hbm", rows * C * 2 * (4 if a[1] else 3)
     if name == "tfb_adamw":                  # p, g, g_f32, m, v, p16, n, ...
