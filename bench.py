@@ -31,7 +31,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0
-# HBM-side bytes one tfb_attn_bwd_rope call moves at B16 H12 T2048 D64 (delta + dkdv + dq kernels), from the FETCH_SIZE and
+# HBM-side bytes one tfb_attn_bwd_rope call moves at B16 H12 T2048 D64 (dq + dkdv kernels), from the FETCH_SIZE and
 # WRITE_SIZE counters scaled by a 256 MiB copy (profiles/attn_c2_hbm_traffic.md): 570 MB fetched + 154 MB written.
 ATTN_BWD_TRAFFIC_BYTES = 7.241e8
 
@@ -441,7 +441,7 @@ def main():
                    "step_tflops": round(flops_per_token(cfg) * tokens / 1e12, 2),
                    "model_tflops_per_s": round(flops_per_token(cfg) * tokens / (dt / args.steps) / 1e12, 1),
                    "final_loss": round(float(loss.item()), 4)},
-        "roofline": {"kernel": "attention backward (tfb_attn_bwd_rope: attn64_delta + attn64_dkdv + attn64_dq), B16 H12 T2048 D64", "bound": "mfma",
+        "roofline": {"kernel": "attention backward (tfb_attn_bwd_rope: attn64_dq, which also makes the row statistics, + attn64_dkdv), B16 H12 T2048 D64", "bound": "mfma",
                      "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": ATTN_BWD_TRAFFIC_BYTES,
                      "traffic_source": "constant from profiles/attn_c2_hbm_traffic.md (rocprofv3 --pmc), not measured in this run",

@@ -747,14 +747,14 @@ extern "C" int tfb_attn_bwd(const void* q, const long* qs, const void* k, const 
 }
 
 // ---- attention backward for callers that cannot allocate --------------------------------------------------------------
-// tfb_attn_bwd needs fp32 [2][B*H][T] of device scratch (the row statistics its pre-pass leaves for the two gradient
-// kernels) and takes it from the caller. Code under HIP graph capture, tight serving loops and harnesses that forbid
+// tfb_attn_bwd needs fp32 [2][B*H][T] of device scratch (the row statistics its first kernel leaves for the second:
+// a pre-pass's for D = 128, the dQ kernel's for D = 64) and takes it from the caller. Code under HIP graph capture, tight serving loops and harnesses that forbid
 // hipMalloc cannot provide one, so this variant keeps that scratch in the library's own image: a file-scope device
 // array of TFB_ATTN_STATIC_ROWS * 2 floats (8 MiB, held by every GPU the library runs on until the process ends).
 // In host code the array's name is only a stand-in for the symbol: its per-device address comes from
 // hipGetSymbolAddress, once per device, and that pointer - never the name - is what the kernels receive.
-// Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams) race on it. The pre-pass
-// writes every element the gradient kernels read, so nothing has to be cleared between calls.
+// Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams) race on it. The first
+// kernel writes every element the later ones read, so nothing has to be cleared between calls.
 #define TFB_ATTN_STATIC_ROWS (1L << 20)
 #define TFB_MAX_DEVICES 64
 static __device__ __align__(256) float scratch[2 * TFB_ATTN_STATIC_ROWS];

@@ -44,6 +44,9 @@
 #ifndef TFB_FWD64_WPE
 #define TFB_FWD64_WPE 2
 #endif
+#ifndef TFB_ATTN_DELTA_IN_DQ
+#define TFB_ATTN_DELTA_IN_DQ 1  // the dQ kernel makes the rows' -delta and -lse / scale itself (0: the separate pre-pass)
+#endif
 
 namespace {
 
@@ -596,9 +599,10 @@ __global__ __launch_bounds__(256, 2) void attn64_dkdv_kernel(AttnT q, AttnT k, A
 
 // =========================================================================================== dQ
 __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dq,
-                                                           const float* __restrict__ stats, long rows, int T, int H,
+                                                           float* __restrict__ stats, long rows, int T, int H,
                                                            float scale, float sl2, const bf16_t* __restrict__ cs,
-                                                           const bf16_t* __restrict__ sn, int nw, int slots) {
+                                                           const bf16_t* __restrict__ sn, int nw, int slots, AttnT o,
+                                                           const float* __restrict__ lse) {
   __shared__ __attribute__((aligned(1024))) uint8_t st0[2 * TILE];
   __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
@@ -623,8 +627,30 @@ __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, A
     qf[s] = *(const bf16x8*)(qp + (long)myq * q.st + 16 * s + 8 * lh);
     gf[s] = *(const bf16x8*)(gp + (long)myq * go.st + 16 * s + 8 * lh);
   }
-  const float myD = stats[(long)bh * T + myq];
-  const float myL = stats[rows + (long)bh * T + myq];
+  float myD, myL;
+  if (TFB_ATTN_DELTA_IN_DQ) {
+    // the row statistics of this wavefront's queries, made here (this kernel runs first) from the dO fragments it holds
+    // anyway and the same elements of O, and left in `stats` for the dK/dV kernel: -sum_d dO O and -lse / scale
+    const bf16_t* orow = o.p + b * o.sb + h * o.sh + (long)myq * o.st;
+    float dot = 0.f;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const u32x4 ov = *(const u32x4*)(orow + 16 * s + 8 * lh);
+      const u32x4 gv = __builtin_bit_cast(u32x4, gf[s]);
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        dot += bflo(ov[w]) * bflo(gv[w]);
+        dot += bfhi(ov[w]) * bfhi(gv[w]);
+      }
+    }
+    dot += __shfl_xor(dot, 32, 64);
+    myD = -dot;
+    myL = -lse[(long)bh * T + myq] * (1.0f / scale);   // (stored with the block's dQ at the end: a store here would sit in
+                                                       // front of the first tile's wait for its loads)
+  } else {
+    myD = stats[(long)bh * T + myq];
+    myL = stats[rows + (long)bh * T + myq];
+  }
 
   TileLoad<2> lk, lv;
   lk.init(kst, wave, lane);
@@ -754,6 +780,10 @@ __global__ __launch_bounds__(256, TFB_DQ64_WPE) void attn64_dq_kernel(AttnT q, A
 
   bf16_t* dqp = dq.p + b * dq.sb + h * dq.sh + (long)myq * dq.st;
   store_grad_row(dqa, scale, dqp, cs, sn, myq, lh);
+  if (TFB_ATTN_DELTA_IN_DQ && lh == 0) {
+    stats[(long)bh * T + myq] = myD;
+    stats[rows + (long)bh * T + myq] = myL;
+  }
   __syncthreads();  // the stages are free for the partner block
   }
 }
@@ -778,14 +808,19 @@ int tfb_attn64_bwd_impl(const void* q, const long* qs, const void* k, const long
                         const long* dks, void* dv, const long* dvs, const float* lse, float* stats, int B, int H, int T,
                         float scale, const void* cos_t, const void* sin_t, int nw, hipStream_t s) {
   const long rows = (long)B * H * T;
-  hipLaunchKernelGGL(attn64_delta_kernel, dim3((unsigned)((rows * 4 + 255) / 256)), dim3(256), 0, s, mk(o, os), mk(go, gos), lse,
-                     stats, T, H, rows, 1.0f / scale);
+  // dQ first: it makes the row statistics of its own queries on the way (from fragments it loads anyway) and leaves them
+  // for dK/dV, so no pass of its own reads O and dO for them (the separate pre-pass took 16.6 us at B16 H12 T2048)
+  if (!TFB_ATTN_DELTA_IN_DQ) {
+    hipLaunchKernelGGL(attn64_delta_kernel, dim3((unsigned)((rows * 4 + 255) / 256)), dim3(256), 0, s, mk(o, os), mk(go, gos), lse,
+                       stats, T, H, rows, 1.0f / scale);
+    TFB_LAUNCH_CHECK();
+  }
+  hipLaunchKernelGGL(attn64_dq_kernel, dim3(paired_grid(T / 128), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
+                     mk(dq, dqs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t, nw,
+                     tfb_resident_slots(2), mk(o, os), lse);
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(attn64_dkdv_kernel, dim3(paired_grid(T / 128), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
                      mk(dk, dks), mk(dv, dvs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t, nw, tfb_resident_slots(2));
-  TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(attn64_dq_kernel, dim3(paired_grid(T / 128), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs), mk(go, gos),
-                     mk(dq, dqs), stats, rows, T, H, scale, scale * LOG2E, (const bf16_t*)cos_t, (const bf16_t*)sin_t, nw, tfb_resident_slots(2));
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
