@@ -62,6 +62,17 @@ def _amax_hint(g, g2):
     return am if (am is not None and g2.data_ptr() == g.data_ptr() and g2.numel() == g.numel()) else None
 
 
+_NAN = {}
+
+
+def _nan_placeholder(like):
+    """A tensor of like's shape and dtype without storage of its own: one NaN element (made once per device and dtype), expanded."""
+    key = (like.device, like.dtype)
+    if key not in _NAN:
+        _NAN[key] = torch.full((1,), float("nan"), dtype=like.dtype, device=like.device)
+    return _NAN[key].expand(like.shape)
+
+
 class RMSNormPassFn(torch.autograd.Function):
     """(x, y[, y8]) = (x, RMSNorm(x) * weight[, e4m3(y * y8_scale)]) for a residual stream whose adds are made in the
     stores of the projections (LinearFn / Linear8Fn / Mlp8Fn with `res`): x is handed through so that the stream's
@@ -84,7 +95,7 @@ class RMSNormPassFn(torch.autograd.Function):
         else:
             _, y, inv, y8 = ops.rmsnorm_fwd_q(x, weight, eps, None, float(y8_scale), want_y=not bytes_only)
             if y is None:
-                y = torch.full((1,), float("nan"), dtype=x.dtype, device=x.device).expand(x.shape)
+                y = _nan_placeholder(x)
             ctx.mark_non_differentiable(y8)
             outs = (x, y, y8)
         ctx.save_for_backward(x, inv, weight)
