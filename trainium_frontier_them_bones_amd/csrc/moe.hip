@@ -18,8 +18,8 @@ namespace {
 constexpr int MAXE = 16;
 typedef int i32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
-#ifndef TFB_ROUTE_RESIDENT
-#define TFB_ROUTE_RESIDENT 1
+#ifndef TFB_ROUTE_EIGHT
+#define TFB_ROUTE_EIGHT 1  // E <= 8: the eight-tokens-per-wavefront router (0: one token per wavefront)
 #endif
 
 __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
@@ -955,7 +955,7 @@ extern "C" int tfb_moe_route(const void* h, const void* wr, const void* bias, vo
                              int d, int E, int topk, void* stream) {
   if (!h || !wr || !p || !idx || !gate) return TFB_ERR_ARG;
   if (N <= 0 || d <= 0 || d % 8 || E < 2 || E > MAXE || (topk != 1 && topk != 2)) return TFB_ERR_SHAPE;
-  if (E <= 8 && TFB_ROUTE_RESIDENT)
+  if (E <= 8 && TFB_ROUTE_EIGHT)
     hipLaunchKernelGGL(moe_route8_kernel, dim3((unsigned)((N + 31) / 32)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)h,
                        (const float*)wr, (const float*)bias, (float*)logits, (float*)p, (int*)idx, (float*)gate, N, d, E, topk);
   else if (E <= 8)
