@@ -422,6 +422,23 @@ def test_norm_that_writes_only_the_bytes_the_mlp_reads(ops, dev):
         assert torch.equal(a, b)
     with pytest.raises(ValueError):
         A.RMSNormPassFn.apply(x, nw, 1e-6, None, True)
+    # the one-node form (parameter-free norm, x + MLP(norm(x))) with fp8 weight gradients writes no bf16 rows either and
+    # equals the two-node composition that does
+    eps = 2.0 ** -23
+    res = []
+    for fused in (True, False):
+        xl, wfl, wpl = (t.clone().requires_grad_(True) for t in (x.reshape(M, d), wf, wp))
+        st = A.Mlp8State(dw_fp8=True)
+        st.refresh(wfl, wpl)
+        if fused:
+            y = A.NrMlpFn.apply(xl, wfl, wpl, st, eps)
+        else:
+            s, h, h8 = A.RMSNormPassFn.apply(xl, None, eps, st.x_scale, False)
+            y = A.Mlp8Fn.apply(h, wfl, wpl, st, h8, s)
+        y.backward(dy.reshape(M, d))
+        res.append((y.detach(), xl.grad, wfl.grad, wpl.grad))
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
 
 
 def test_norm_backward_hands_its_amax_to_the_mlp_backward(ops, dev):

@@ -500,7 +500,8 @@ class NrMlpFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x2, w_fc, w_proj, state, eps=2.0 ** -23):
         x2 = x2.contiguous()
-        _, xn, inv, x8 = ops.rmsnorm_fwd_q(x2, None, eps, None, state.x_scale)
+        # (with the weight gradients in fp8 too nothing reads the norm's bf16 rows: only its e4m3 bytes are written)
+        _, xn, inv, x8 = ops.rmsnorm_fwd_q(x2, None, eps, None, state.x_scale, want_y=not state.dw_fp8)
         xo, r = ops.mlp8_fwd(xn, state.w8, state.row, w_fc.shape[0], state.x_scale, x8=x8, res=x2)
         ctx.save_for_backward(x2, x8 if state.dw_fp8 else xn, inv, r, w_fc, w_proj)
         ctx.state = state
