@@ -511,8 +511,8 @@ class NrMlpFn(torch.autograd.Function):
     def backward(ctx, g):
         x2, xa, inv, r, w_fc, w_proj = ctx.saved_tensors
         st = ctx.state
-        g = g.contiguous()
-        rowb = ops.mlp8_backward_scales(g, st.row)
+        g_in, g = g, g.contiguous()
+        rowb = ops.mlp8_backward_scales(g, st.row, _amax_hint(g_in, g))
         if st.dw_fp8:
             dxn, _, dp8, hq8, dy8 = ops.mlp8_bwd_q(g, r, st.w8, rowb, st.e4m3_limit, want_dpre=False)
             dw_fc, dw_proj = ops.mlp8_dw8(xa, dp8, hq8, dy8, rowb, st.x_scale)
@@ -520,7 +520,8 @@ class NrMlpFn(torch.autograd.Function):
             dxn, _, dpre = ops.mlp8_bwd(g, r, st.w8, rowb, want_h=False)
             dw_fc = ops.matmul(dpre, xa, trans_a=True)
             dw_proj = ops.mlp_dw_proj(g, r)
-        gx = ops.rmsnorm_bwd(dxn, x2, inv, None, g)[0]
+        gx, _, am = ops.rmsnorm_bwd(dxn, x2, inv, None, g, want_amax=True)
+        setattr(gx, AMAX_HINT, am)      # for the block before this one, whose backward receives gx as its dy
         return gx, dw_fc, dw_proj, None, None
 
 
