@@ -703,31 +703,57 @@ __global__ __launch_bounds__(256) void moe_dispatch_bwd_kernel(const bf16_t* __r
       w1[e] = *(const f32x4*)(w + 4);
     }
   }
-  for (long n = tid / cpr; n < N; n += nstep) {
-    float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    const int s1 = slot[n * topk];
-    if (s1 >= 0) load8(dxs + (long)s1 * d + c, r);
+  // Software-pipelined over the thread's tokens: a token's slots and router gradients are requested one token ahead, and
+  // its two rows of dxs are loaded without a branch between them (a skipped assignment reads row 0 and is zeroed by a
+  // select), so a token costs one round trip to memory instead of three dependent ones (36 -> 28 us for 16384 x 1024).
+  auto fetch_meta = [&](long n, int& s1, int& s2, float (&g)[EP]) {
     if (topk == 2) {
-      const int s2 = slot[n * 2 + 1];
-      if (s2 >= 0) {
-        float b[8];
-        load8(dxs + (long)s2 * d + c, b);
+      const i32x2 sv = *(const i32x2*)(slot + n * 2);
+      s1 = sv.x;
+      s2 = sv.y;
+    } else {
+      s1 = slot[n];
+      s2 = -1;
+    }
+    if (dlogits) {
 #pragma unroll
-        for (int k = 0; k < 8; ++k) r[k] += b[k];
-      }
+      for (int e = 0; e < EP; ++e) g[e] = dlogits[n * E + (e < E ? e : E - 1)];
+    }
+  };
+  long n = tid / cpr;
+  int s1 = -1, s2 = -1, t1 = -1, t2 = -1;
+  float g[EP], gn[EP];
+#pragma unroll
+  for (int e = 0; e < EP; ++e) g[e] = gn[e] = 0.f;
+  if (n < N) fetch_meta(n, s1, s2, g);
+  for (; n < N; n += nstep) {
+    const u32x4 ra = *(const u32x4*)(dxs + (long)(s1 >= 0 ? s1 : 0) * d + c);
+    const u32x4 rb = *(const u32x4*)(dxs + (long)(s2 >= 0 ? s2 : 0) * d + c);
+    if (n + nstep < N) fetch_meta(n + nstep, t1, t2, gn);
+    float r[8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float a0 = s1 >= 0 ? bflo(ra[k]) : 0.f, a1 = s1 >= 0 ? bfhi(ra[k]) : 0.f;
+      const float b0 = s2 >= 0 ? bflo(rb[k]) : 0.f, b1 = s2 >= 0 ? bfhi(rb[k]) : 0.f;
+      r[2 * k] = a0 + b0;
+      r[2 * k + 1] = a1 + b1;
     }
     if (dlogits) {
 #pragma unroll
       for (int e = 0; e < EP; ++e) {
-        const float g = e < E ? dlogits[n * E + e] : 0.f;
+        const float ge = e < E ? g[e] : 0.f;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-          r[k] += g * w0[e][k];
-          r[4 + k] += g * w1[e][k];
+          r[k] += ge * w0[e][k];
+          r[4 + k] += ge * w1[e][k];
         }
       }
     }
     store8(dh + n * d + c, r);
+    s1 = t1;
+    s2 = t2;
+#pragma unroll
+    for (int e = 0; e < EP; ++e) g[e] = gn[e];
   }
 }
 
