@@ -99,3 +99,24 @@ def test_every_entry_point_is_reached_from_the_host_layer():
     tests = "".join(open(f).read() for f in glob.glob(os.path.join(root, "tests", "test_gpu_*.py")))
     for name in _lib.SIGNATURES:
         assert ('"%s"' % name) in host or ("." + name + "(") in host or name in tests, name
+
+
+def test_amax_hint_is_void_after_an_in_place_update():
+    """The amax partials a producer hangs on a gradient tensor are used only while the tensor still holds what they were
+    taken from: the same memory, and no in-place write since (autograd may accumulate a second gradient into it)."""
+    import torch
+    from trainium_frontier_them_bones_amd import autograd as A
+    t = torch.randn(8, 4)
+    am = torch.tensor([float(t.abs().max())])
+    A._attach_amax(t, am)
+    assert A._amax_hint(t, t.reshape(8, 4)) is am
+    assert A._amax_hint(t, t.clone()) is None                 # a copy is other memory
+    old = A.USE_AMAX_HINT
+    A.USE_AMAX_HINT = False
+    try:
+        assert A._amax_hint(t, t) is None
+    finally:
+        A.USE_AMAX_HINT = old
+    t.add_(1.0)
+    assert A._amax_hint(t, t) is None                         # written to since: the partials are void
+    assert A._amax_hint(torch.randn(3), torch.randn(3)) is None

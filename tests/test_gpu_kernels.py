@@ -462,19 +462,23 @@ def test_norm_backward_hands_its_amax_to_the_mlp_backward(ops, dev):
     row = ops.mlp8_forward_scales(wf, wp)
     assert torch.equal(ops.mlp8_backward_scales(dx1, row), ops.mlp8_backward_scales(dx1, row, am))
 
-    def two_blocks(hint):
+    def two_blocks(hint, skip=False):
         old = A.USE_AMAX_HINT
         A.USE_AMAX_HINT = hint
         try:
             xl = x.clone().requires_grad_(True)
             ps = [t.clone().requires_grad_(True) for t in (nw, wf, wp, nw, wf, wp)]
             h = xl
+            mids = []
             for b in range(2):
                 n_, f_, p_ = ps[3 * b:3 * b + 3]
                 st = A.Mlp8State(dw_fp8=True)
                 st.refresh(f_, p_)
                 s_, y_, y8_ = A.RMSNormPassFn.apply(h, n_, 1e-6, st.x_scale, True)
                 h = A.Mlp8Fn.apply(y_, f_, p_, st, y8_, s_)
+                mids.append(h)
+            if skip:                           # the first block's output has a second reader: its gradient is a sum
+                h = h + 0.5 * mids[0]
             h.backward(gy)
             return [xl.grad] + [t.grad for t in ps]
         finally:
@@ -491,6 +495,10 @@ def test_norm_backward_hands_its_amax_to_the_mlp_backward(ops, dev):
     finally:
         ops.mlp8_backward_scales = real
     for a, b in zip(with_hint, without):
+        assert torch.equal(a, b)
+    # with a second reader of the first block's output, autograd sums two gradients for it and may do so in place in the
+    # tensor the norm backward wrote: partials taken before the sum must not be used for it
+    for a, b in zip(two_blocks(True, skip=True), two_blocks(False, skip=True)):
         assert torch.equal(a, b)
 
 

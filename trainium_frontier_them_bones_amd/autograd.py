@@ -56,10 +56,21 @@ AMAX_HINT = "_tfb_amax_part"   # attribute on a gradient tensor: fp32 partials w
 USE_AMAX_HINT = True           # False: consumers ignore the attribute and read the tensor for its amax
 
 
+def _attach_amax(t, am):
+    """Hang the amax partials of t's present contents on t, with t's version counter: an in-place update of t afterwards
+    (autograd may add a second incoming gradient into it) makes the partials void."""
+    setattr(t, AMAX_HINT, (am, t._version))
+    return t
+
+
 def _amax_hint(g, g2):
-    """The amax partials the producer of gradient g attached to it, when g2 (the rows the caller will use) is g's own memory."""
-    am = getattr(g, AMAX_HINT, None) if USE_AMAX_HINT else None
-    return am if (am is not None and g2.data_ptr() == g.data_ptr() and g2.numel() == g.numel()) else None
+    """The amax partials the producer of gradient g attached to it, when g2 (the rows the caller will use) is g's own memory
+    and g has not been written to since."""
+    hint = getattr(g, AMAX_HINT, None) if USE_AMAX_HINT else None
+    if hint is None:
+        return None
+    am, version = hint
+    return am if (g._version == version and g2.data_ptr() == g.data_ptr() and g2.numel() == g.numel()) else None
 
 
 _NAN = {}
@@ -112,11 +123,11 @@ class RMSNormPassFn(torch.autograd.Function):
         part = getattr(weight, "dw_part", None)
         if part is not None:
             dx, _, am = ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, gs, part=part, want_amax=True)
-            setattr(dx, AMAX_HINT, am)
+            _attach_amax(dx, am)
             return dx, None, None, None, None
         buf, acc = (None, False) if weight is None else _accumulate_into(weight)
         dx, dw, am = ops.rmsnorm_bwd(gy.contiguous(), x, inv, weight, gs, buf, acc, want_amax=True)
-        setattr(dx, AMAX_HINT, am)
+        _attach_amax(dx, am)
         gw = dw.to(weight.dtype) if (weight is not None and buf is None) else None
         return dx, gw, None, None, None
 
@@ -521,7 +532,7 @@ class NrMlpFn(torch.autograd.Function):
             dw_fc = ops.matmul(dpre, xa, trans_a=True)
             dw_proj = ops.mlp_dw_proj(g, r)
         gx, _, am = ops.rmsnorm_bwd(dxn, x2, inv, None, g, want_amax=True)
-        setattr(gx, AMAX_HINT, am)      # for the block before this one, whose backward receives gx as its dy
+        _attach_amax(gx, am)      # for the block before this one, whose backward receives gx as its dy
         return gx, dw_fc, dw_proj, None, None
 
 
