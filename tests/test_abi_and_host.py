@@ -120,3 +120,30 @@ def test_amax_hint_is_void_after_an_in_place_update():
     t.add_(1.0)
     assert A._amax_hint(t, t) is None                         # written to since: the partials are void
     assert A._amax_hint(torch.randn(3), torch.randn(3)) is None
+
+
+def test_every_entry_point_rejects_null_pointers_and_empty_shapes_on_the_host():
+    """Argument checks come before any device work: with every pointer NULL an entry point answers "bad argument" (or
+    "unsupported shape" where the sizes are looked at first), and with dummy non-null pointers and all sizes zero it answers
+    with one of the two as well; no call reaches a kernel launch (status 3), so this runs without a GPU."""
+    import ctypes
+    from trainium_frontier_them_bones_amd import _lib
+    L = _lib.lib()
+    plain = _lib._LONG_RESULT | {"tfb_norm_bwd_blocks", "tfb_resmix_bwd_blocks"}      # size queries: no status to check
+    for name, sig in _lib.SIGNATURES.items():
+        if name in plain:
+            continue
+        for null in (True, False):
+            args = []
+            for t in sig:
+                if t is _lib._vp:
+                    args.append(None if null else 0x1000)          # never dereferenced on the host
+                elif t is _lib._lp:
+                    args.append(None if null else (ctypes.c_long * 4)())
+                elif t is _lib._fp:
+                    args.append(None if null else (ctypes.c_float * 16)())
+                elif t is _lib._f:
+                    args.append(0.0)
+                else:
+                    args.append(0)
+            assert getattr(L, name)(*args) in (1, 2), (name, null)
