@@ -106,16 +106,12 @@ __global__ __launch_bounds__(256) void amax_partial_kernel(const bf16_t* __restr
 
 // One wavefront per row of w [rows][cols]: sum of squares per row; amax partial per workgroup.
 // blockIdx.z = layer of a batched refresh: w advances by wz elements, the outputs by their per-layer sizes (oz floats).
-__global__ __launch_bounds__(256) void row_stats_kernel(const bf16_t* __restrict__ w, int rows, int cols,
-                                                       float* __restrict__ rowss, float* __restrict__ amax_part, long wz,
-                                                       long oz) {
-  __shared__ float red[4];
+// (bx of gx workgroups; the job of weight_stats_kernel's first gx workgroups)
+__device__ __forceinline__ void row_stats_job(const bf16_t* __restrict__ w, int rows, int cols, float* __restrict__ rowss,
+                                              float* __restrict__ amax_part, int bx, int gx, float* red) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  w += blockIdx.z * wz;
-  rowss += blockIdx.z * oz;
-  amax_part += blockIdx.z * oz;
   float m = 0.f;
-  for (int r = blockIdx.x * 4 + wave; r < rows; r += gridDim.x * 4) {
+  for (int r = bx * 4 + wave; r < rows; r += gx * 4) {
     float ss = 0.f;
     for (int c = lane * 8; c < cols; c += 512) {
       u32x4 u = *(const u32x4*)(w + (long)r * cols + c);
@@ -131,25 +127,20 @@ __global__ __launch_bounds__(256) void row_stats_kernel(const bf16_t* __restrict
     if (lane == 0) rowss[r] = ss;
   }
   m = block_max(m, red);
-  if (threadIdx.x == 0) amax_part[blockIdx.x] = m;
+  if (threadIdx.x == 0) amax_part[bx] = m;
 }
 
 // Column sums of squares of w [rows][cols]: a workgroup owns 512 columns (64 lanes x 8) of one slice of the rows
 // (blockIdx.y of COL_SLICES), its 4 wavefronts take interleaved rows; the slices' partial sums go to
 // colss_part [COL_SLICES][cols] and are added in slice order by the scale kernel; amax partial per workgroup.
 constexpr int COL_SLICES = 32;
-__global__ __launch_bounds__(256) void col_stats_kernel(const bf16_t* __restrict__ w, int rows, int cols,
-                                                       float* __restrict__ colss_part, float* __restrict__ amax_part, long wz,
-                                                       long oz) {
-  __shared__ float red[4];
-  __shared__ float acc[4][512];
+__device__ __forceinline__ void col_stats_job(const bf16_t* __restrict__ w, int rows, int cols, float* __restrict__ colss_part,
+                                              float* __restrict__ amax_part, int bx, int by, int gx, int gy, float* red,
+                                              float (*acc)[512]) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  w += blockIdx.z * wz;
-  colss_part += blockIdx.z * oz;
-  amax_part += blockIdx.z * oz;
-  const int c = blockIdx.x * 512 + lane * 8;
-  const int per = (rows + gridDim.y - 1) / gridDim.y;
-  const int r0 = blockIdx.y * per, r1 = min(rows, r0 + per);
+  const int c = bx * 512 + lane * 8;
+  const int per = (rows + gy - 1) / gy;
+  const int r0 = by * per, r1 = min(rows, r0 + per);
   float ss[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   float m = 0.f;
   if (c < cols) {
@@ -168,13 +159,32 @@ __global__ __launch_bounds__(256) void col_stats_kernel(const bf16_t* __restrict
   for (int k = 0; k < 8; ++k) acc[wave][lane * 8 + k] = ss[k];
   m = block_max(m, red);  // contains the barriers that publish acc
   for (int i = threadIdx.x; i < 512; i += 256) {
-    int cc = blockIdx.x * 512 + i;
-    if (cc < cols) colss_part[(long)blockIdx.y * cols + cc] = acc[0][i] + acc[1][i] + acc[2][i] + acc[3][i];
+    int cc = bx * 512 + i;
+    if (cc < cols) colss_part[(long)by * cols + cc] = acc[0][i] + acc[1][i] + acc[2][i] + acc[3][i];
   }
-  if (threadIdx.x == 0) amax_part[blockIdx.y * gridDim.x + blockIdx.x] = m;
+  if (threadIdx.x == 0) amax_part[by * gx + bx] = m;
 }
 
-// colss[c] = sum over the row slices, in slice order
+// Both weights' statistics in one launch: workgroups [0, nfc) take the rows of w_fc [F][d], the other npj x slices the
+// column slices of w_proj [d][F] (the two jobs share nothing, so one launch instead of two costs neither anything).
+__global__ __launch_bounds__(256) void weight_stats_kernel(const bf16_t* __restrict__ w_fc, const bf16_t* __restrict__ w_proj,
+                                                          int F, int d, float* __restrict__ rowss,
+                                                          float* __restrict__ amax_fc_part, float* __restrict__ colss_part,
+                                                          float* __restrict__ amax_pj_part, int nfc, int npj, int slices,
+                                                          long wz, long oz) {
+  __shared__ float red[4];
+  __shared__ float acc[4][512];
+  const long wo = blockIdx.z * wz, oo = blockIdx.z * oz;
+  const int b = blockIdx.x;
+  if (b < nfc) {
+    row_stats_job(w_fc + wo, F, d, rowss + oo, amax_fc_part + oo, b, nfc, red);
+  } else {
+    const int bb = b - nfc;
+    col_stats_job(w_proj + wo, d, F, colss_part + oo, amax_pj_part + oo, bb % npj, bb / npj, npj, slices, red, acc);
+  }
+}
+
+// colss[c] = sum over the row slices, in slice order (eight loads in flight, the additions in that order all the same)
 __global__ __launch_bounds__(256) void col_finish_kernel(const float* __restrict__ part, int n, int slices,
                                                         float* __restrict__ colss, long oz) {
   const int i = blockIdx.x * 256 + threadIdx.x;
@@ -182,7 +192,15 @@ __global__ __launch_bounds__(256) void col_finish_kernel(const float* __restrict
   part += blockIdx.z * oz;
   colss += blockIdx.z * oz;
   float t = 0.f;
-  for (int sl = 0; sl < slices; ++sl) t += part[(long)sl * n + i];
+  int sl = 0;
+  for (; sl + 8 <= slices; sl += 8) {
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = part[(long)(sl + k) * n + i];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) t += v[k];
+  }
+  for (; sl < slices; ++sl) t += part[(long)sl * n + i];
   colss[i] = t;
 }
 
@@ -197,17 +215,39 @@ __global__ __launch_bounds__(256) void forward_scales_kernel(const float* rowss,
                                                             const float* colss, const float* amax_pj_part, int npj,
                                                             float e4m3_limit, float h_bound, float inv_x_scale,
                                                             const float* __restrict__ x_scale_dev, float* row_out, long oz) {
-  __shared__ float red[4];
   rowss += blockIdx.z * oz;
   amax_fc_part += blockIdx.z * oz;
   colss += blockIdx.z * oz;
   amax_pj_part += blockIdx.z * oz;
   row_out += blockIdx.z * NSC;
-  float rho2 = reduce_max_array(rowss, F, red);
-  float kappa2 = reduce_max_array(colss, F, red);
-  float amax_fc = reduce_max_array(amax_fc_part, nfc, red);
-  float amax_pj = reduce_max_array(amax_pj_part, npj, red);
+  // the four maxima: a thread's loads of all four arrays are in flight together, then ONE reduction over the workgroup
+  // (a maximum does not depend on the order, so the values equal four reduce_max_array calls')
+  __shared__ float red4[4][4];
+  float mx[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int i = threadIdx.x; i < F; i += 1024) {
+    float a[4], b[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int j = i + 256 * k;
+      a[k] = j < F ? rowss[j] : 0.f;
+      b[k] = j < F ? colss[j] : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) mx[0] = fmaxf(mx[0], a[k]), mx[1] = fmaxf(mx[1], b[k]);
+  }
+  for (int i = threadIdx.x; i < nfc; i += 256) mx[2] = fmaxf(mx[2], amax_fc_part[i]);
+  for (int i = threadIdx.x; i < npj; i += 256) mx[3] = fmaxf(mx[3], amax_pj_part[i]);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) mx[k] = wave_max(mx[k]);
+  if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) red4[threadIdx.x >> 6][k] = mx[k];
+  }
+  __syncthreads();
   if (threadIdx.x == 0) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) mx[k] = fmaxf(fmaxf(red4[0][k], red4[1][k]), fmaxf(red4[2][k], red4[3][k]));
+    const float rho2 = mx[0], kappa2 = mx[1], amax_fc = mx[2], amax_pj = mx[3];
     float s_wfc, i_wfc, s_wpj, i_wpj, s_h, i_h, c_h;
     pow2_le(amax_fc, e4m3_limit, -24, 40, &s_wfc, &i_wfc);
     pow2_le(amax_pj, e4m3_limit, -24, 40, &s_wpj, &i_wpj);
@@ -534,7 +574,7 @@ constexpr int AMAX_BLOCKS = 1024;
 extern "C" long tfb_mlp8_scale_scratch_floats(int F) { return (2L + COL_SLICES) * F + 4L * AMAX_BLOCKS; }
 
 // row_out: fp32 [16] device. e4m3_limit: 240 reproduces the reference's rows; 448 is the OCP maximum.
-// The forward scale rows of `layers` MLPs whose weights sit `wz` elements apart (w_fc and w_proj alike): four launches
+// The forward scale rows of `layers` MLPs whose weights sit `wz` elements apart (w_fc and w_proj alike): three launches
 // whatever the layer count. scratch: layers x tfb_mlp8_scale_scratch_floats(F) floats; row_out: layers x 16 floats.
 static int launch_forward_scales(const void* w_fc, const void* w_proj, void* row_out, void* scratch, int F, int d,
                                  float e4m3_limit, float x_scale, const void* x_scale_dev, int layers, long wz, hipStream_t s) {
@@ -547,12 +587,10 @@ static int launch_forward_scales(const void* w_fc, const void* w_proj, void* row
   int nfc = (F + 3) / 4;
   if (nfc > AMAX_BLOCKS) nfc = AMAX_BLOCKS;
   int npj = (F + 511) / 512;
-  hipLaunchKernelGGL(row_stats_kernel, dim3(nfc, 1, layers), dim3(256), 0, s, (const bf16_t*)w_fc, F, d, rowss, pa, wz, oz);
-  TFB_LAUNCH_CHECK();
   int slices = AMAX_BLOCKS / npj < COL_SLICES ? AMAX_BLOCKS / npj : COL_SLICES;
   if (slices < 1) return TFB_ERR_SHAPE;
-  hipLaunchKernelGGL(col_stats_kernel, dim3(npj, slices, layers), dim3(256), 0, s, (const bf16_t*)w_proj, d, F, colpart, pb, wz,
-                     oz);
+  hipLaunchKernelGGL(weight_stats_kernel, dim3(nfc + npj * slices, 1, layers), dim3(256), 0, s, (const bf16_t*)w_fc,
+                     (const bf16_t*)w_proj, F, d, rowss, pa, colpart, pb, nfc, npj, slices, wz, oz);
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(col_finish_kernel, dim3((F + 255) / 256, 1, layers), dim3(256), 0, s, colpart, F, slices, colss, oz);
   TFB_LAUNCH_CHECK();
@@ -642,7 +680,7 @@ extern "C" int tfb_mlp8_precast(const void* w_fc, const void* w_proj, const void
   return TFB_OK;
 }
 
-// The per-optimizer-step refresh of `layers` MLPs in six launches: scale rows [layers][16] and e4m3 packs [layers][4 F d]
+// The per-optimizer-step refresh of `layers` MLPs in five launches: scale rows [layers][16] and e4m3 packs [layers][4 F d]
 // (layouts as tfb_mlp8_forward_scales / tfb_mlp8_precast) from weights laid out with one stride: layer i's w_fc at
 // w_fc + i * layer_stride elements, its w_proj at w_proj + i * layer_stride. scratch: layers x
 // tfb_mlp8_scale_scratch_floats(F) floats. The per-layer calls cost ~45 us of small launches each.
