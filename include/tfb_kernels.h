@@ -173,7 +173,7 @@ int tfb_quant_fp8(const void* x, const void* scale_ptr, float scale_imm, int fmt
  * Replaces _precast8_kernel / precast_ref (round2/source/kernels/nki_mlp_l4t.py:392, 948-970). */
 int tfb_mlp8_precast(const void* w_fc, const void* w_proj, const void* row, void* w8, int F, int d, void* stream);
 
-/* tfb_mlp8_forward_scales + tfb_mlp8_precast for `layers` MLPs in five launches: rows fp32 [layers][16], w8 uint8
+/* tfb_mlp8_forward_scales + tfb_mlp8_precast for `layers` MLPs in four launches: rows fp32 [layers][16], w8 uint8
  * [layers][4][F*d], from weights laid out with one stride (layer i's w_fc at w_fc + i * layer_stride elements, its
  * w_proj at w_proj + i * layer_stride). scratch: layers * tfb_mlp8_scale_scratch_floats(F) floats. F, d multiples of 64.
  * Replaces the loop over layers of fp8_refresh_weights (round2/source/train.py:6617: mlp8_scales_into 7003 +

@@ -672,7 +672,7 @@ class Moe8State:
     def refresh(self, w_fc, w_proj):
         E, F, d = w_fc.shape
         wf, wp = w_fc.detach(), w_proj.detach()
-        if wf.is_contiguous() and wp.is_contiguous():      # the experts as E layers of one flat buffer: five launches
+        if wf.is_contiguous() and wp.is_contiguous():      # the experts as E layers of one flat buffer: four launches
             self.rows, self.w8 = ops.mlp8_refresh_layers(wf[0], wp[0], F * d, E, self.e4m3_limit, self.x_scale)
             return
         rows = [ops.mlp8_forward_scales(wf[e], wp[e], self.e4m3_limit, self.x_scale) for e in range(E)]

@@ -319,16 +319,8 @@ __global__ __launch_bounds__(256) void quant_kernel(const bf16_t* __restrict__ x
 }
 
 // w [R][C] bf16 -> out [R][C] e4m3 and outT [C][R] e4m3, 64 x 64 tiles through LDS.
-__global__ __launch_bounds__(256) void precast_kernel(const bf16_t* __restrict__ w, const float* __restrict__ scale_ptr,
-                                                     uint8_t* __restrict__ out, uint8_t* __restrict__ outT, int R, int C,
-                                                     long wz, long sz, long bz) {
-  __shared__ uint8_t t[64][80];
-  w += blockIdx.z * wz;
-  scale_ptr += blockIdx.z * sz;
-  out += blockIdx.z * bz;
-  outT += blockIdx.z * bz;
-  const float s = *scale_ptr;
-  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+__device__ __forceinline__ void precast_tile(const bf16_t* __restrict__ w, const float s, uint8_t* __restrict__ out,
+                                             uint8_t* __restrict__ outT, int R, int C, int r0, int c0, uint8_t (*t)[80]) {
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     int ch = threadIdx.x + i * 256;  // 512 chunks of 8 elements
@@ -349,6 +341,36 @@ __global__ __launch_bounds__(256) void precast_kernel(const bf16_t* __restrict__
     int c = threadIdx.x >> 2, j = (threadIdx.x & 3) * 16;
     u32x4 v = *(const u32x4*)(&t[c][j]);
     *(u32x4*)(outT + (long)(c0 + c) * R + r0 + j) = v;
+  }
+}
+
+__global__ __launch_bounds__(256) void precast_kernel(const bf16_t* __restrict__ w, const float* __restrict__ scale_ptr,
+                                                     uint8_t* __restrict__ out, uint8_t* __restrict__ outT, int R, int C,
+                                                     long wz, long sz, long bz) {
+  __shared__ uint8_t t[64][80];
+  const long z = blockIdx.z;
+  precast_tile(w + z * wz, scale_ptr[z * sz], out + z * bz, outT + z * bz, R, C, blockIdx.y * 64, blockIdx.x * 64, t);
+}
+
+// An MLP's two weights in one launch: workgroups [0, T) take the tiles of w_fc [F][d], [T, 2T) those of w_proj [d][F],
+// T = (F / 64)(d / 64); the pack b8 [4][F d] gets w_fc8, its transpose, w_proj8, its transpose. row: the layer's scale row.
+__global__ __launch_bounds__(256) void precast_mlp_kernel(const bf16_t* __restrict__ w_fc, const bf16_t* __restrict__ w_proj,
+                                                         const float* __restrict__ row, uint8_t* __restrict__ b8, int F, int d,
+                                                         long wz, long sz, long bz) {
+  __shared__ uint8_t t[64][80];
+  const long z = blockIdx.z;
+  const long n = (long)F * d;
+  const int T = (F >> 6) * (d >> 6);
+  row += z * sz;
+  b8 += z * bz;
+  int b = blockIdx.x;
+  if (b < T) {
+    const int nc = d >> 6;
+    precast_tile(w_fc + z * wz, row[SC_S_WFC], b8, b8 + n, F, d, (b / nc) * 64, (b % nc) * 64, t);
+  } else {
+    b -= T;
+    const int nc = F >> 6;
+    precast_tile(w_proj + z * wz, row[SC_S_WPROJ], b8 + 2 * n, b8 + 3 * n, d, F, (b / nc) * 64, (b % nc) * 64, t);
   }
 }
 
@@ -670,17 +692,13 @@ extern "C" int tfb_mlp8_precast(const void* w_fc, const void* w_proj, const void
   if (F <= 0 || d <= 0 || F % 64 || d % 64) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   uint8_t* b = (uint8_t*)w8;
-  const long n = (long)F * d;
-  hipLaunchKernelGGL(precast_kernel, dim3(d / 64, F / 64, 1), dim3(256), 0, s, (const bf16_t*)w_fc,
-                     (const float*)row + SC_S_WFC, b, b + n, F, d, 0L, 0L, 0L);
-  TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(precast_kernel, dim3(F / 64, d / 64, 1), dim3(256), 0, s, (const bf16_t*)w_proj,
-                     (const float*)row + SC_S_WPROJ, b + 2 * n, b + 3 * n, d, F, 0L, 0L, 0L);
+  hipLaunchKernelGGL(precast_mlp_kernel, dim3(2 * (F / 64) * (d / 64), 1, 1), dim3(256), 0, s, (const bf16_t*)w_fc,
+                     (const bf16_t*)w_proj, (const float*)row, b, F, d, 0L, 0L, 0L);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
 
-// The per-optimizer-step refresh of `layers` MLPs in five launches: scale rows [layers][16] and e4m3 packs [layers][4 F d]
+// The per-optimizer-step refresh of `layers` MLPs in four launches: scale rows [layers][16] and e4m3 packs [layers][4 F d]
 // (layouts as tfb_mlp8_forward_scales / tfb_mlp8_precast) from weights laid out with one stride: layer i's w_fc at
 // w_fc + i * layer_stride elements, its w_proj at w_proj + i * layer_stride. scratch: layers x
 // tfb_mlp8_scale_scratch_floats(F) floats. The per-layer calls cost ~45 us of small launches each.
@@ -695,11 +713,8 @@ extern "C" int tfb_mlp8_refresh_layers(const void* w_fc, const void* w_proj, lon
   if (st != TFB_OK) return st;
   uint8_t* b = (uint8_t*)w8;
   const long n = (long)F * d;
-  hipLaunchKernelGGL(precast_kernel, dim3(d / 64, F / 64, layers), dim3(256), 0, s, (const bf16_t*)w_fc,
-                     (const float*)rows + SC_S_WFC, b, b + n, F, d, layer_stride, (long)NSC, 4 * n);
-  TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL(precast_kernel, dim3(F / 64, d / 64, layers), dim3(256), 0, s, (const bf16_t*)w_proj,
-                     (const float*)rows + SC_S_WPROJ, b + 2 * n, b + 3 * n, d, F, layer_stride, (long)NSC, 4 * n);
+  hipLaunchKernelGGL(precast_mlp_kernel, dim3(2 * (F / 64) * (d / 64), 1, layers), dim3(256), 0, s, (const bf16_t*)w_fc,
+                     (const bf16_t*)w_proj, (const float*)rows, b, F, d, layer_stride, (long)NSC, 4 * n);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

@@ -151,7 +151,7 @@ class GPT:
         o_pj = [self.mats.offsets["w_proj.%d" % i][0] for i in range(L)]
         stride = o_fc[1] - o_fc[0] if L > 1 else 0
         if all(o_fc[i] - o_fc[0] == i * stride and o_pj[i] - o_pj[0] == i * stride for i in range(L)):
-            # the layers' weights sit one stride apart in the flat buffer: one batched refresh (five launches)
+            # the layers' weights sit one stride apart in the flat buffer: one batched refresh (four launches)
             st0 = self.mlp_state[0]
             self._mlp_rows, self._mlp_w8 = ops.mlp8_refresh_layers(
                 self.p["w_fc.0"].detach(), self.p["w_proj.0"].detach(), stride, L, st0.e4m3_limit, st0.x_scale,
