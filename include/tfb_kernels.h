@@ -330,6 +330,11 @@ int tfb_loss_multi_fwd(const void* logits, const void* targets, int idx64, const
 int tfb_loss_multi_bwd(const void* logits, const void* targets, int idx64, const void* row_w, int K, float eps, const void* lse,
                        const void* g, void* dlogits, long rows, int V, float softcap, void* stream);
 
+/* w fp32 [rows] = each row's weight in the reduced loss: (t >= 0) / max(1, #{t >= 0}) when mean != 0 (the mean over the
+ * rows whose target counts, targets < 0 ignored), (t >= 0) otherwise. One launch for the compare / sum / clamp / divide the
+ * caller of fused_loss(reduction=) makes on the host side (round1/source/train.py:4703-4707 scales the row losses there). */
+int tfb_loss_row_weights(const void* targets, int idx64, void* w, long rows, int mean, void* stream);
+
 /* tfb_loss_fwd followed by tfb_loss_bwd with grow = row_w (an upstream gradient of one), in place and in ONE pass over the
  * logits (a row is held in a workgroup's registers, V <= 65536; TFB_ERR_SHAPE beyond): loss and lse as tfb_loss_fwd writes
  * them, logits overwritten by d logits = row_w (softmax - onehot) (1 - tanh^2), all three bit-equal to the two calls.

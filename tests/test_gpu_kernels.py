@@ -1025,3 +1025,19 @@ def test_embedding_backward_at_full_size_on_a_zipf_batch(ops, dev, V):
     assert rel_l2(dwa, want) < 1e-6
     assert int((want.abs().sum(1) > 0).sum()) > 3000 and int(torch.bincount(idx[ok]).max()) > 1000   # many tokens, one very hot
 
+
+
+def test_loss_row_weights_equal_the_host_expression(ops, dev):
+    """tfb_loss_row_weights: (t >= 0) / max(1, count) for the mean, (t >= 0) for the sum, bit for bit what the compare /
+    cast / sum / clamp / divide chain gives; int64 and int32 targets, lengths off every stride of the kernel, no row valid."""
+    g = _g(4242)
+    for n in (1, 63, 1024, 4097, 32768, 100003):
+        for dt in (torch.int64, torch.int32):
+            t = torch.randint(0, 1000, (n,), generator=g).to(dt)
+            t[torch.rand(n, generator=g) < 0.3] = -1
+            t = t.to(dev)
+            valid = (t >= 0).to(torch.float32)
+            assert torch.equal(ops.loss_row_weights(t, "mean"), valid / valid.sum().clamp_min(1.0))
+            assert torch.equal(ops.loss_row_weights(t, "sum"), valid)
+    none = torch.full((777,), -1, dtype=torch.int64, device=dev)
+    assert torch.equal(ops.loss_row_weights(none, "mean"), torch.zeros(777, device=dev))

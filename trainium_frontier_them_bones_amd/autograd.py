@@ -551,8 +551,7 @@ class LmHeadLossFn(torch.autograd.Function):
     def forward(ctx, x, W, targets, softcap, reduction):
         x2 = x.reshape(-1, x.shape[-1]).contiguous()
         tg = targets.reshape(-1)
-        valid = (tg >= 0).to(torch.float32)
-        w = valid / valid.sum().clamp_min(1.0) if reduction == "mean" else valid
+        w = ops.loss_row_weights(tg, reduction)
         ctx.softcap = softcap
         ctx.xshape = x.shape
         ctx.one_pass = (LM_HEAD_ONE_PASS and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1])

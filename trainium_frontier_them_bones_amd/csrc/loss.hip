@@ -39,6 +39,34 @@ __device__ __forceinline__ MS ms_merge(MS a, MS b) {
   return r;
 }
 
+// ------------------------------------------------------------------------------------ row weights
+// One workgroup: w[i] = (t_i >= 0) / max(1, #{t >= 0}) for the mean over the rows that count (mean != 0), else (t_i >= 0).
+template <typename IDX>
+__global__ __launch_bounds__(1024) void loss_row_weights_kernel(const IDX* __restrict__ tg, float* __restrict__ w, long rows,
+                                                               int mean) {
+  __shared__ int cnt[16];
+  float each = 1.0f;
+  if (mean) {
+    int c = 0;
+    for (long i = threadIdx.x; i < rows; i += 4096) {
+      IDX t[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) t[k] = i + 1024 * k < rows ? tg[i + 1024 * k] : (IDX)-1;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) c += t[k] >= 0;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
+    if ((threadIdx.x & 63) == 0) cnt[threadIdx.x >> 6] = c;
+    __syncthreads();
+    int n = 0;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) n += cnt[k];
+    each = 1.0f / (float)(n > 1 ? n : 1);
+  }
+  for (long i = threadIdx.x; i < rows; i += 1024) w[i] = tg[i] >= 0 ? each : 0.f;
+}
+
 // ------------------------------------------------------------------------------------ loss on logits
 // One workgroup per row. loss_row = w * (lse - s_t) with w = row_w[row] (or 1), 0 for target < 0.
 template <typename IDX>
@@ -482,6 +510,21 @@ extern "C" int tfb_loss_fwd(const void* logits, const void* targets, int idx64, 
   else
     hipLaunchKernelGGL(loss_fwd_kernel<int>, dim3((unsigned)rows), dim3(256), 0, s, (const bf16_t*)logits, (const int*)targets,
                        (const float*)row_w, (float*)loss, (float*)lse, V, softcap);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// w fp32 [rows]: the weight of each row's loss in the reduction, (t >= 0) / max(1, number of rows with t >= 0) for the
+// mean over the rows that count (mean != 0: F.cross_entropy(ignore_index < 0) semantics), (t >= 0) for the sum. One small
+// launch in place of a compare, a cast, a sum, a clamp and a division.
+extern "C" int tfb_loss_row_weights(const void* targets, int idx64, void* w, long rows, int mean, void* stream) {
+  if (!targets || !w) return TFB_ERR_ARG;
+  if (rows <= 0) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  if (idx64)
+    hipLaunchKernelGGL(loss_row_weights_kernel<long>, dim3(1), dim3(1024), 0, s, (const long*)targets, (float*)w, rows, mean);
+  else
+    hipLaunchKernelGGL(loss_row_weights_kernel<int>, dim3(1), dim3(1024), 0, s, (const int*)targets, (float*)w, rows, mean);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

@@ -707,6 +707,15 @@ def loss_bwd(logits2, targets, lse, grow, softcap=15.0, inplace=False):
     return out
 
 
+def loss_row_weights(targets, reduction="mean"):
+    """fp32 [N] weights of the row losses in the reduced loss: (t >= 0) / max(1, count of t >= 0) for "mean", (t >= 0) for
+    "sum" (targets < 0 are ignored rows)."""
+    tg = _tg(targets)
+    w = torch.empty(tg.numel(), dtype=torch.float32, device=tg.device)
+    _lib.call("tfb_loss_row_weights", _p(tg), int(tg.dtype == torch.int64), _p(w), tg.numel(), int(reduction == "mean"), _stream())
+    return w
+
+
 LOSS_FWD_BWD_MAX_V = 65536
 
 

@@ -114,8 +114,7 @@ def chunked_loss_mean(logits, targets, smooth=False, tok_w=None, eps=0.0):
     b, t, v = logits.shape
     n = b * t
     y = targets.reshape(n)
-    valid = y >= 0
-    w = valid.to(torch.float32) / valid.sum().clamp_min(1).to(torch.float32)
+    w = ops.loss_row_weights(y, "mean")
     if tok_w is not None:
         w = w * tok_w.reshape(n).to(torch.float32)
     x2 = logits.reshape(n, v).contiguous()
