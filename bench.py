@@ -32,8 +32,8 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0
 # HBM-side bytes one tfb_attn_bwd_rope call moves at B16 H12 T2048 D64 (dq + dkdv kernels), from the FETCH_SIZE and
-# WRITE_SIZE counters scaled by a 256 MiB copy (profiles/attn_c2_hbm_traffic.md): 512 MB fetched + 154 MB written.
-ATTN_BWD_TRAFFIC_BYTES = 6.659e8
+# WRITE_SIZE counters scaled by a 256 MiB copy (profiles/attn_c2_hbm_traffic.md): 513.5 MB fetched + 154.2 MB written.
+ATTN_BWD_TRAFFIC_BYTES = 6.677e8
 
 
 def flops_per_token(cfg):
