@@ -16,9 +16,6 @@ second line per configuration: the same repetition recorded once as a HIP graph 
 
 python bench.py --traffic-probe   (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: a 256 MiB device copy as the
 counters' calibration, then attention forward + backward at the benchmark shape; prints nothing)
-
-python bench.py --hw-probe        (the load-issue and LDS-interference probes of the library: what a 1 KB vector load costs the
-wavefront that issues it, and what operand streams cost the LDS fragment reads of the same CU)
 """
 import argparse
 import json
@@ -304,37 +301,6 @@ def config_probe(which, graphs=False):
                   6 * 2.0 * (2 * N) * d * Fd)
 
 
-def hw_probe():
-    """The hardware probes behind the operand paths of the GEMM and attention kernels (tfb_probe_load_issue,
-    tfb_probe_lds_mix): the cost of a 1 KB vector load to the wavefront that issues it, and what operand streams cost the
-    fragment reads of the same CU; and where a workgroup of the bf16 GEMM spends its cycles (tfb_probe_gemm_phases)."""
-    import torch
-    from trainium_frontier_them_bones_amd import ops
-    dev = torch.device("cuda:0")
-    ops.probe_load_issue(dev, True, 4, iters=200)   # warm-up
-    print("1 KB vector loads from an L2-resident 2 MB region (8 rows x 128 B at pitch 1536 per instruction):")
-    for to_lds, name in ((True, "global -> LDS DMA (global_load_lds_dwordx4)"), (False, "global -> VGPR (global_load_dwordx4)")):
-        for waves in (1, 4, 8):
-            per, bpc = ops.probe_load_issue(dev, to_lds, waves)
-            print("  %-45s %d wavefront(s) per CU: %6.1f cycles per instruction per wavefront, %5.1f B/clk/CU" % (name, waves, per, bpc))
-    print("LDS fragment reads (four wavefronts, 16 x ds_read_b128 in flight each) beside four streaming wavefronts:")
-    for mode, name in ((0, "readers alone"), (1, "+ global -> LDS DMA"), (2, "+ global -> VGPR -> ds_write_b128"), (3, "+ global -> VGPR only")):
-        rd, ld = ops.probe_lds_mix(dev, mode)
-        print("  %-36s LDS reads %6.1f B/clk/CU   streamed %5.1f B/clk/CU" % (name, rd, ld))
-    print("Phases of a workgroup of the bf16 GEMM (128 x 128 tile, two workgroups per CU; mean cycles over all workgroups):")
-    g = torch.Generator(device="cpu").manual_seed(5)
-    for what, M, N, K in (("QKV projection", 32768, 2304, 768), ("output projection", 32768, 768, 768),
-                          ("32768 x 3072 x 768", 32768, 3072, 768), ("8192^3", 8192, 8192, 8192)):
-        a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
-        b = torch.randn(N, K, generator=g).to(torch.bfloat16).to(dev)
-        for _ in range(3):
-            _, cyc = ops.probe_gemm_phases(a, b)
-        torch.cuda.synchronize(dev)
-        m = cyc.double().mean(0).tolist()
-        print("  %-20s %5d workgroups: first load issued after %5.0f, first k-tile there after %5.0f, k-loop %6.0f (%4.0f per k-tile), "
-              "epilogue %5.0f" % (what, cyc.shape[0], m[0], m[1], m[2], m[2] / (K * 2 // 128), m[3]))
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -343,7 +309,6 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true")
     ap.add_argument("--ns-probe", action="store_true")
-    ap.add_argument("--hw-probe", action="store_true")
     ap.add_argument("--config-probe", choices=("c1", "c2", "c3", "c5", "all"))
     ap.add_argument("--graphs", action="store_true", help="with --config-probe: also time each repetition replayed as a HIP graph")
     ap.add_argument("--bf16-dw", action="store_true")
@@ -359,9 +324,6 @@ def main():
         return
     if args.ns_probe:
         ns_probe()
-        return
-    if args.hw_probe:
-        hw_probe()
         return
     if args.config_probe:
         config_probe(args.config_probe, args.graphs)

@@ -489,22 +489,6 @@ long tfb_ns5_workspace_bytes(int K, int M, int N);
 int tfb_ns5(const void* g, const void* inv_d, const float* coeffs, void* y, void* v, int K, int M, int N, int wide,
             void* workspace, long workspace_bytes, void* stream);
 
-/* ---- hardware probes (diagnostics; no counterpart in the reference, nothing on the training path calls them) ------------
- * What a 1 KB vector load costs the wavefront that issues it: `waves` (1, 4 or 8) wavefronts on every CU each issue
- * iters x 8 loads of 8 rows x 128 bytes (pitch 1536) from the first `region` bytes of src (keep it L2-resident: 2 MB), into
- * LDS by global -> LDS DMA (to_lds 1) or into registers (0). cycles: uint64 [CUs][16] device, zero-filled by the caller;
- * [cu][w] = cycles of wavefront w. These figures decide how the GEMM and attention kernels move their operands. */
-int tfb_probe_load_issue(const void* src, long region, int to_lds, int waves, int iters, void* cycles, void* stream);
-/* Four wavefronts of every CU read LDS fragments (riters x 16 ds_read_b128) while four others stream operands into the same
- * CU: mode 0 nothing, 1 global -> LDS DMA, 2 global -> VGPR -> ds_write_b128, 3 global -> VGPR only (liters x 8 loads of 1 KB).
- * cycles: uint64 [CUs][16], entries 0..3 the readers, 4..7 the streaming wavefronts. */
-int tfb_probe_lds_mix(const void* src, long region, int mode, int riters, int liters, void* cycles, void* stream);
-/* Where a workgroup of the bf16 GEMM spends its time: c [M][N] = a [M][K] b[N][K]^T through the library's own kernel,
- * traversal and launch (M, N multiples of 128, K of 64), with cycles: uint64 [(M/128)(N/128)][4] = wavefront 0's cycle
- * counts from kernel entry to the first operand load's issue, to the first k-tile's arrival, in the k-loop, in the
- * epilogue. */
-int tfb_probe_gemm_phases(const void* a, const void* b, void* c, long M, long N, long K, void* cycles, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -976,31 +976,6 @@ def test_autograd_nodes_do_not_corrupt_what_autograd_cannot_see(ops, dev):
     assert torch.equal(x.grad, gx) and torch.equal(W.grad, gw)
 
 
-def test_hardware_probes_run_and_report_sane_rates(ops, dev):
-    """tfb_probe_load_issue / tfb_probe_lds_mix (diagnostics): they finish, every CU reports, and the rates are inside what
-    the hardware can do (a CU's vector memory path moves well under 128 B/clk, its LDS under 512 B/clk)."""
-    per, bpc = ops.probe_load_issue(dev, True, 4, iters=300)
-    assert 4.0 < per < 5000.0 and 1.0 < bpc < 128.0
-    per1, bpc1 = ops.probe_load_issue(dev, False, 1, iters=300)
-    assert 4.0 < per1 < 5000.0 and 0.5 < bpc1 < 128.0
-    rd, ld = ops.probe_lds_mix(dev, 1, riters=2000, liters=6000)
-    assert 10.0 < rd < 512.0 and 1.0 < ld < 128.0
-    rd0, ld0 = ops.probe_lds_mix(dev, 0, riters=2000, liters=0)
-    assert 10.0 < rd0 < 512.0 and ld0 == 0.0
-
-
-def test_gemm_phase_probe_is_the_library_kernel(ops, dev):
-    """tfb_probe_gemm_phases (diagnostic): its product is bit-identical to tfb_gemm_bf16's on the same operands (it runs
-    the same kernel and launch path with a reporting epilogue), every workgroup reports, and the phases are ordered."""
-    g = torch.Generator(device="cpu").manual_seed(11)
-    a = torch.randn(1024, 768, generator=g).to(torch.bfloat16).to(dev)
-    b = torch.randn(384, 768, generator=g).to(torch.bfloat16).to(dev)
-    c, cyc = ops.probe_gemm_phases(a, b)
-    assert torch.equal(c, ops.matmul(a, b, trans_b=True))
-    assert cyc.shape == (8 * 3, 4) and bool((cyc > 0).all())
-    assert bool((cyc[:, 0] < cyc[:, 1]).all())          # the first load is issued before the first k-tile is there
-
-
 @pytest.mark.parametrize("V", [32768, 50304])
 def test_embedding_backward_at_full_size_on_a_zipf_batch(ops, dev, V):
     """The grouped embedding backward at the benchmark's size (32768 rows of 768, Zipf(1.1) ids): with the vocabulary's

@@ -80,9 +80,6 @@ SIGNATURES = {
     "tfb_moe_max_rows": [_l, _i, _i],
     "tfb_moe_route": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _i, _vp],
     "tfb_moe_tables": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _l, _vp],
-    "tfb_probe_load_issue": [_vp, _l, _i, _i, _i, _vp, _vp],
-    "tfb_probe_lds_mix": [_vp, _l, _i, _i, _i, _vp, _vp],
-    "tfb_probe_gemm_phases": [_vp, _vp, _vp, _l, _l, _l, _vp, _vp],
     "tfb_moe_tables_cap": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _l, _i, _i, _i, _l, _vp],
     "tfb_moe_gather": [_vp, _vp, _vp, _f, _vp, _vp, _l, _i, _vp],
     "tfb_moe_mlp8_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],

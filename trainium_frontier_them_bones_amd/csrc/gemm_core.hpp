@@ -313,14 +313,6 @@ struct has_tile_epilogue : std::false_type {};
 template <class T>
 struct has_tile_epilogue<T, std::void_t<decltype(T::kTileEpilogue)>> : std::true_type {};
 
-// A diagnostic epilogue with the member  unsigned long long* phase_cycles  gets the workgroup's phases written there, four
-// numbers per workgroup (wavefront 0's cycle counter): kernel entry -> first operand load issued, -> first k-tile landed
-// (the first barrier), the k-loop, the epilogue. No product epilogue has the member; the code below is compiled out for them.
-template <class T, class = void>
-struct has_phase_probe : std::false_type {};
-template <class T>
-struct has_phase_probe<T, std::void_t<decltype(std::declval<const T&>().phase_cycles)>> : std::true_type {};
-
 // the residual a projection's store adds is read once by that kernel (output projection with the hint: 0.72 -> 0.70 ms per step)
 #ifndef TFB_NT_RES
 #define TFB_NT_RES 1
@@ -361,9 +353,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
   __shared__ __attribute__((aligned(1024))) uint8_t buf1[Cfg::STAGE_BYTES];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-  constexpr bool kProbe = has_phase_probe<Epi>::value;
-  [[maybe_unused]] unsigned long long ph0 = 0, ph_issue = 0, ph_first = 0, ph_loop = 0;
-  if constexpr (kProbe) ph0 = __builtin_readcyclecounter();
   // Two workgroups share a CU. Launched together they run in lockstep: both in the k-loop (each at half the MFMA rate),
   // then both in the epilogue (MFMA idle, memory busy). The one that landed in an odd wavefront slot (HW_ID.wave_id
   // bit 0) therefore starts ~7 us late, once, in the first round of workgroups: from then on one's epilogue runs
@@ -455,7 +444,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
     dp.issue(buf, t, wave);
     dq.issue(buf + BP * 128, t, wave);
   };
-  if constexpr (kProbe) ph_issue = __builtin_readcyclecounter();
   if (nkt > 0) issue(buf0, 0);
 
   const Epi epi = epi_prepare(epi_for_group(epi_in, group));
@@ -532,7 +520,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
 
   {
     __syncthreads();
-    if constexpr (kProbe) ph_first = __builtin_readcyclecounter();
     // The epilogue's operands are requested here, behind the first k-tile's barrier: vector loads return in order, so
     // asked for before it they made that barrier wait for a stream from HBM; now they fly under the first k-tile's MFMAs.
     if (TFB_PREFETCH_AFTER_FIRST) prefetch_epilogue();
@@ -546,7 +533,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
     }
     if (nkt & 1) compute(buf0);
     __syncthreads();
-    if constexpr (kProbe) ph_loop = __builtin_readcyclecounter();
   }
 
   const int pw = wp * (TP * 32), qw = wq * (TQ * 32);  // wavefront's origin inside the tile
@@ -595,15 +581,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::OCC) void gemm_kernel(GemmArgs a, Pre
         }
         __builtin_amdgcn_wave_barrier();
       }
-    }
-  }
-  if constexpr (kProbe) {
-    if (wave == 0 && lane == 0) {
-      unsigned long long* o = epi.phase_cycles + 4L * blockIdx.x;
-      o[0] = ph_issue - ph0;
-      o[1] = ph_first - ph0;
-      o[2] = ph_loop - ph_first;
-      o[3] = __builtin_readcyclecounter() - ph_loop;
     }
   }
 }

@@ -64,8 +64,12 @@ def matmul(a, b, trans_a=False, trans_b=False, out=None, accumulate=False, out_d
         if out.dtype not in (bf16, torch.float32) or tuple(out.shape) != (M, N):
             raise ValueError("bad out")
     ws = _workspace(a.device)
-    _lib.call("tfb_gemm_bf16_scaled", _p(a), _p(b), _p(out), M, N, K, int(trans_a), int(trans_b),
-              int(out.dtype == torch.float32), int(accumulate), _p(ws), ws.numel() * 4, _p(alpha), _stream())
+    if alpha is None:
+        _lib.call("tfb_gemm_bf16", _p(a), _p(b), _p(out), M, N, K, int(trans_a), int(trans_b),
+                  int(out.dtype == torch.float32), int(accumulate), _p(ws), ws.numel() * 4, _stream())
+    else:
+        _lib.call("tfb_gemm_bf16_scaled", _p(a), _p(b), _p(out), M, N, K, int(trans_a), int(trans_b),
+                  int(out.dtype == torch.float32), int(accumulate), _p(ws), ws.numel() * 4, _p(alpha), _stream())
     return out
 
 
@@ -1075,48 +1079,4 @@ def ns5(g, d, coeffs=NS_COEFFS):
     co = (ctypes.c_float * 15)(*[float(x) for t in coeffs for x in t])
     _lib.call("tfb_ns5", _p(g), _p(inv), co, _p(y), _p(v), K, M, N, int(wide), _p(ws), ws.numel(), _stream())
     return y, v
-
-
-# ------------------------------------------------------------------------------------------ hardware probes (diagnostics)
-def _probe_region(dev, region):
-    return torch.ones(region + 4096, dtype=torch.uint8, device=dev)
-
-
-def probe_load_issue(dev, to_lds, waves, iters=4000, region=2 << 20):
-    """What a 1 KB vector load costs its wavefront: (cycles per instruction per wavefront, bytes per clock per CU) with
-    `waves` wavefronts of every CU issuing, into LDS (to_lds) or into registers, from an L2-resident region."""
-    src = _probe_region(dev, region)
-    cyc = torch.zeros(4096, 16, dtype=torch.int64, device=dev)
-    _lib.call("tfb_probe_load_issue", _p(src), region, int(bool(to_lds)), waves, iters, _p(cyc), _stream())
-    torch.cuda.synchronize(dev)
-    c = cyc[:, :waves].double()
-    c = c[c.sum(1) > 0]
-    per = float(c.mean())
-    return per / (iters * 8.0), waves * iters * 8.0 * 1024.0 / per
-
-
-def probe_lds_mix(dev, mode, riters=20000, liters=60000, region=2 << 20):
-    """Fragment reads of four wavefronts beside four streaming ones (mode 0 none, 1 DMA, 2 through registers and
-    ds_write_b128, 3 into registers only): (LDS bytes read per clock per CU, bytes streamed per clock per CU)."""
-    src = _probe_region(dev, region)
-    cyc = torch.zeros(4096, 16, dtype=torch.int64, device=dev)
-    _lib.call("tfb_probe_lds_mix", _p(src), region, mode, riters, liters, _p(cyc), _stream())
-    torch.cuda.synchronize(dev)
-    live = cyc[:, :4].sum(1) > 0
-    rd = float(cyc[live, :4].double().mean())
-    ld = float(cyc[live, 4:8].double().mean())
-    return 4.0 * riters * 16384.0 / rd, (4.0 * liters * 8192.0 / ld if ld > 0 else 0.0)
-
-
-def probe_gemm_phases(a, b):
-    """c = a [M,K] @ b [N,K]^T (bf16) through the library's bf16 GEMM kernel with its workgroups' phases reported: returns
-    (c, phases) with phases int64 [tiles, 4] = cycles from kernel entry to the first operand load's issue, to the first
-    k-tile's arrival, in the k-loop, in the epilogue (wavefront 0 of each 128 x 128 tile's workgroup)."""
-    M, K = a.shape
-    N = b.shape[0]
-    assert a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16 and b.shape[1] == K and a.is_contiguous() and b.is_contiguous()
-    c = torch.empty(M, N, dtype=torch.bfloat16, device=a.device)
-    cyc = torch.zeros((M // 128) * (N // 128), 4, dtype=torch.int64, device=a.device)
-    _lib.call("tfb_probe_gemm_phases", _p(a), _p(b), _p(c), M, N, K, _p(cyc), _stream())
-    return c, cyc
 
