@@ -3,7 +3,7 @@
 // sum) and split-K through an fp32 workspace for small outputs with a long contraction.
 // Replaces the reference's nki_matmul(a, b, trans_a, trans_b) (round1/source/train.py:1137)
 // and the torch matmuls its Linear glue issues (round1/source/train.py:8419-8711).
-#include "gemm_core.hpp"
+#include "gemm_pp.hpp"
 
 namespace {
 
@@ -15,6 +15,9 @@ int run(GemmOperand P, GemmOperand Q, int N, int M, int K, void* C, int out_f32,
   const int splits = ws ? choose_splits(tiles, K / 64, (long)M * N, ws_bytes) : 1;
   if (splits == 1) {
     EpiStore e{C, (long)N, out_f32, accumulate, alpha};
+    // large outputs with both operands k-contiguous: the persistent 256 x 256 kernel (same sums in the same order)
+    if (LAYP == TFB_K_CONTIG && LAYQ == TFB_K_CONTIG && !out_f32 && !accumulate && gemm_pp_applies(N, M, (long)K * 2))
+      return gemm_pp_launch<2, 0, 0>(P, Q, N, M, (long)K * 2, e, stream);
     return gemm_launch<Cfg>(P, Q, N, M, (long)K * 2, 1, LoadIdentity{}, LoadIdentity{}, e, stream);
   }
   EpiSplit e{ws, (long)N, (long)M * N};
@@ -49,6 +52,24 @@ struct EpiStoreRope {
     u32x4 x = pack8bf(v);
     if (p < rot_cols) {
       const u32x4 y = pack8bf(vp);
+      const bool low = (p & 32) == 0;
+      const u32x4 c = tab.c, s = tab.s;
+      u32x4 o;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float x0 = bflo(x[k]), x1 = bfhi(x[k]), y0 = bflo(y[k]), y1 = bfhi(y[k]);
+        const float c0 = bflo(c[k]), c1 = bfhi(c[k]), s0 = bflo(s[k]), s1 = bfhi(s[k]);
+        o[k] = low ? pack2bf(x0 * c0 + y0 * s0, x1 * c1 + y1 * s1) : pack2bf(x0 * c0 - y0 * s0, x1 * c1 - y1 * s1);
+      }
+      x = o;
+    }
+    *(u32x4*)(out + (long)q * ld + p) = x;
+  }
+  // the 256 x 256 kernel's protocol: the same from the rounded products
+  __device__ __forceinline__ float pre(float x) const { return x; }
+  __device__ __forceinline__ void chunk(int p, int q, const u32x4& xin, const u32x4& y, const pre_t& tab) const {
+    u32x4 x = xin;
+    if (p < rot_cols) {
       const bool low = (p & 32) == 0;
       const u32x4 c = tab.c, s = tab.s;
       u32x4 o;
@@ -102,6 +123,7 @@ extern "C" int tfb_gemm_bf16_res(const void* A, const void* B, const void* res, 
   if (M <= 0 || N <= 0 || K <= 0 || M % 128 || N % 128 || K % 64) return TFB_ERR_SHAPE;
   GemmOperand P{(const uint8_t*)B, trans_b ? (long)K * 2 : (long)N * 2}, Q{(const uint8_t*)A, (long)K * 2};
   EpiStoreRes e{(bf16_t*)C, (const bf16_t*)res, (long)N};
+  if (trans_b && gemm_pp_applies(N, M, (long)K * 2)) return gemm_pp_launch<2, 0, 0>(P, Q, N, M, (long)K * 2, e, (hipStream_t)stream);
   if (trans_b)
     return gemm_launch<GemmCfg<128, 128, 2, 2, 2, TFB_K_CONTIG, TFB_K_CONTIG>>(P, Q, N, M, (long)K * 2, 1, LoadIdentity{},
                                                                                LoadIdentity{}, e, (hipStream_t)stream);
@@ -120,5 +142,6 @@ extern "C" int tfb_qkv_rope_fwd(const void* x, const void* w, const void* cos_t,
   using Cfg = GemmCfg<128, 128, 2, 2, 2, TFB_K_CONTIG, TFB_K_CONTIG>;
   GemmOperand P{(const uint8_t*)w, (long)K * 2}, Q{(const uint8_t*)x, (long)K * 2};
   EpiStoreRope e{(bf16_t*)out, (long)N, (const bf16_t*)cos_t, (const bf16_t*)sin_t, T, rot_cols};
+  if (gemm_pp_applies(N, M, (long)K * 2)) return gemm_pp_launch<2, 0, 0>(P, Q, N, M, (long)K * 2, e, (hipStream_t)stream);
   return gemm_launch<Cfg>(P, Q, N, M, (long)K * 2, 1, LoadIdentity{}, LoadIdentity{}, e, (hipStream_t)stream);
 }

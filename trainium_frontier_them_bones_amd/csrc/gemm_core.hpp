@@ -671,6 +671,16 @@ struct EpiStoreRes {
     for (int k = 0; k < 8; ++k) a[k] += b[k];
     *(u32x4*)(out + (long)q * ld + p) = pack8bf(a);
   }
+  // the same from the rounded product (the 256 x 256 kernel's epilogue protocol: pre() before the rounding, chunk() after)
+  __device__ __forceinline__ float pre(float x) const { return x; }
+  __device__ __forceinline__ void chunk(int p, int q, const u32x4& v, const pre_t& r) const {
+    float a[8], b[8];
+    unpack8bf(v, a);
+    unpack8bf(r, b);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) a[k] += b[k];
+    *(u32x4*)(out + (long)q * ld + p) = pack8bf(a);
+  }
 };
 
 // out (bf16 or fp32) [nq][ld] (+)= D
@@ -680,9 +690,17 @@ struct EpiStore {
   int f32;
   int accumulate;
   const float* alpha = nullptr;  // optional device scalar the product is multiplied by before the (one) rounding
+  float a = 1.0f;                // *alpha, read once by prepare()
+  __device__ __forceinline__ EpiStore prepare() const {
+    EpiStore e = *this;
+    e.a = alpha ? *alpha : 1.0f;
+    return e;
+  }
+  // the 256 x 256 kernel's protocol, for a plain bf16 output (no accumulation)
+  __device__ __forceinline__ float pre(float x) const { return x * a; }
+  __device__ __forceinline__ void chunk(int p, int q, const u32x4& v) const { *(u32x4*)((bf16_t*)out + (long)q * ld + p) = v; }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int) const {
     float r[8];
-    const float a = alpha ? *alpha : 1.0f;
 #pragma unroll
     for (int k = 0; k < 8; ++k) r[k] = v[k] * a;
     if (f32) {

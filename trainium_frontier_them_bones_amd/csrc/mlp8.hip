@@ -14,7 +14,7 @@
 //   x8 = e4m3(x * s_x); r = bf16(max(acc * dq_fc, 0)); rc = bf16(min(r * c_h, 15.375));
 //   h8 = e4m3(rc^2); y = bf16(acc * dq_proj); dy8 = e5m2(dy * s_dy);
 //   dpre = bf16((acc * dq_dh2) * r); dp8 = e5m2(dpre * s_dp); dx = bf16(acc * dq_dx).
-#include "gemm_core.hpp"
+#include "gemm_pp.hpp"
 
 // scale-row columns (nki_mlp_fused8.py:111-114)
 #define SC_S_WFC 0
@@ -417,6 +417,24 @@ struct EpiUp {  // pre = x8 @ wf8^T: r, h8
                cvt4_fp8<TFB_FMT_E4M3, false>(hh[4], hh[5], hh[6], hh[7])};
     *(u32x2*)(h8 + off) = o;   // (read by the next GEMM: a non-temporal store here costs 0.2 ms per step)
   }
+  // the 256 x 256 kernel's protocol (pre() before the rounding to bf16, chunk() on the 8 rounded values): the same values
+  __device__ __forceinline__ float pre(float x) const { return fmaxf(x * dq, 0.f); }
+  __device__ __forceinline__ void chunk(int p, int q, const u32x4& rbits) const {
+    float a[8], hh[8];
+    unpack8bf(rbits, a);
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      float ca = fminf(a[i] * c, H_CLAMP), cb = fminf(a[i + 1] * c, H_CLAMP);
+      round2_bf(ca, cb);
+      hh[i] = ca * ca;
+      hh[i + 1] = cb * cb;
+    }
+    const long off = (long)q * F + p;
+    __builtin_nontemporal_store(rbits, (u32x4*)(r + off));
+    u32x2 o = {cvt4_fp8<TFB_FMT_E4M3, false>(hh[0], hh[1], hh[2], hh[3]),
+               cvt4_fp8<TFB_FMT_E4M3, false>(hh[4], hh[5], hh[6], hh[7])};
+    *(u32x2*)(h8 + off) = o;
+  }
 };
 
 struct EpiScaleStore {  // out = bf16(acc * sc[col])
@@ -441,6 +459,8 @@ struct EpiScaleStore {  // out = bf16(acc * sc[col])
     for (int i = 0; i < 8; ++i) r[i] = v[i] * dq;
     *(u32x4*)(out + (long)q * ld + p) = pack8bf(r);
   }
+  __device__ __forceinline__ float pre(float x) const { return x * dq; }
+  __device__ __forceinline__ void chunk(int p, int q, const u32x4& v) const { *(u32x4*)(out + (long)q * ld + p) = v; }
 };
 
 // out = bf16(res + bf16(acc * dq)): EpiScaleStore / EpiDescale with the residual add that follows the projection made in
@@ -479,6 +499,15 @@ struct EpiDescaleRes {
     for (int i = 0; i < 8; ++i) a[i] += b[i];
     *(u32x4*)(out + (long)q * ld + p) = pack8bf(a);
   }
+  __device__ __forceinline__ float pre(float x) const { return x * dq; }
+  __device__ __forceinline__ void chunk(int p, int q, const u32x4& v, const pre_t& rv) const {
+    float a[8], b[8];
+    unpack8bf(v, a);
+    unpack8bf(rv, b);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a[i] += b[i];
+    *(u32x4*)(out + (long)q * ld + p) = pack8bf(a);
+  }
 };
 
 struct EpiDescale {  // out = bf16(acc * dq), dq = dq_imm * *dq_a * *dq_b (absent factors are 1)
@@ -501,6 +530,8 @@ struct EpiDescale {  // out = bf16(acc * dq), dq = dq_imm * *dq_a * *dq_b (absen
     for (int i = 0; i < 8; ++i) r[i] = v[i] * dq;
     *(u32x4*)(out + (long)q * ld + p) = pack8bf(r);
   }
+  __device__ __forceinline__ float pre(float x) const { return x * dq; }
+  __device__ __forceinline__ void chunk(int p, int q, const u32x4& v) const { *(u32x4*)(out + (long)q * ld + p) = v; }
 };
 
 struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*s_dp), optional h = bf16(r^2) and
@@ -733,6 +764,14 @@ extern "C" int tfb_precast8(const void* w, const void* scale_ptr, void* out8, vo
 using Cfg8 = GemmCfg<128, 128, 2, 2, 1, TFB_K_CONTIG, TFB_K_CONTIG, TFB_FMT_E4M3, TFB_FMT_E4M3>;
 using Cfg8g = GemmCfg<128, 128, 2, 2, 1, TFB_K_CONTIG, TFB_K_CONTIG, TFB_FMT_E4M3, TFB_FMT_E5M2>;
 
+// A dense fp8 GEMM with both operands k-contiguous: the persistent 256 x 256 kernel where the shape allows it (the same
+// sums in the same order, the epilogue's values bit for bit), else the 128 x 128 kernel.
+template <class Cfg, class Epi>
+static int launch8(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes, Epi e, hipStream_t s) {
+  if (gemm_pp_applies(np, nq, kbytes)) return gemm_pp_launch<1, Cfg::FMTP, Cfg::FMTQ>(P, Q, np, nq, kbytes, e, s);
+  return gemm_launch<Cfg>(P, Q, np, nq, kbytes, 1, LoadIdentity{}, LoadIdentity{}, e, s);
+}
+
 // out [M][N] bf16 = bf16((a8 [M][K] @ b8 [N][K]^T) * dq): the fp8 projection GEMM. a8 is e4m3 (fmt_a 0: forward
 // activations) or e5m2 (fmt_a 1: gradients); b8 is e4m3 (a pre-cast weight layout). dq = dq_imm * *dq_a * *dq_b, the
 // pointers being device fp32 scalars (inverse power-of-two scales) or null.
@@ -744,8 +783,8 @@ extern "C" int tfb_gemm_fp8(const void* a8, int fmt_a, const void* b8, const voi
   GemmOperand P{(const uint8_t*)b8, (long)K}, Q{(const uint8_t*)a8, (long)K};
   EpiDescale e{(const float*)dq_a, (const float*)dq_b, dq_imm, (bf16_t*)out, (long)N};
   if (fmt_a == TFB_FMT_E4M3)
-    return gemm_launch<Cfg8>(P, Q, N, (int)M, (long)K, 1, LoadIdentity{}, LoadIdentity{}, e, (hipStream_t)stream);
-  return gemm_launch<Cfg8g>(P, Q, N, (int)M, (long)K, 1, LoadIdentity{}, LoadIdentity{}, e, (hipStream_t)stream);
+    return launch8<Cfg8>(P, Q, N, (int)M, (long)K, e, (hipStream_t)stream);
+  return launch8<Cfg8g>(P, Q, N, (int)M, (long)K, e, (hipStream_t)stream);
 }
 
 // tfb_gemm_fp8 with the residual add in the store: out = bf16(res + bf16((a8 @ b8^T) * dq)), res [M][N] bf16; e4m3
@@ -757,7 +796,7 @@ extern "C" int tfb_gemm_fp8_res(const void* a8, const void* b8, const void* dq_a
   if (M <= 0 || N <= 0 || K <= 0 || M % 128 || N % 128 || K % 128 || M > 0x7fffffffL) return TFB_ERR_SHAPE;
   GemmOperand P{(const uint8_t*)b8, (long)K}, Q{(const uint8_t*)a8, (long)K};
   EpiDescaleRes e{nullptr, 0, (const float*)dq_a, (const float*)dq_b, dq_imm, (const bf16_t*)res, (bf16_t*)out, (long)N};
-  return gemm_launch<Cfg8>(P, Q, N, (int)M, (long)K, 1, LoadIdentity{}, LoadIdentity{}, e, (hipStream_t)stream);
+  return launch8<Cfg8>(P, Q, N, (int)M, (long)K, e, (hipStream_t)stream);
 }
 
 // out [O][D] (+)= ((g8 [M][O]^T @ a8 [M][D]) * imm / (*s_g * *s_a)): the fp8 weight gradient of a projection, contraction
@@ -799,11 +838,11 @@ extern "C" int tfb_mlp8_fwd(const void* x8, const void* w8, const void* row, voi
   const long n = (long)F * d;
   GemmOperand Pw{b, (long)d}, Qx{(const uint8_t*)x8, (long)d};
   EpiUp e1{(const float*)row, (bf16_t*)r, (uint8_t*)h8, (long)F};
-  int st = gemm_launch<Cfg8>(Pw, Qx, F, (int)M, (long)d, 1, LoadIdentity{}, LoadIdentity{}, e1, s);
+  int st = launch8<Cfg8>(Pw, Qx, F, (int)M, (long)d, e1, s);
   if (st != TFB_OK) return st;
   GemmOperand Pp{b + 2 * n, (long)F}, Qh{(const uint8_t*)h8, (long)F};
   EpiScaleStore e2{(const float*)row, SC_DQ_PROJ, (bf16_t*)y, (long)d};
-  return gemm_launch<Cfg8>(Pp, Qh, d, (int)M, (long)F, 1, LoadIdentity{}, LoadIdentity{}, e2, s);
+  return launch8<Cfg8>(Pp, Qh, d, (int)M, (long)F, e2, s);
 }
 
 // tfb_mlp8_fwd with the block's residual add in the second GEMM's store: y = bf16(res + bf16(MLP(x))), res [M][d] bf16 (the
@@ -819,11 +858,11 @@ extern "C" int tfb_mlp8_fwd_res(const void* x8, const void* w8, const void* row,
   const long n = (long)F * d;
   GemmOperand Pw{b, (long)d}, Qx{(const uint8_t*)x8, (long)d};
   EpiUp e1{(const float*)row, (bf16_t*)r, (uint8_t*)h8, (long)F};
-  int st = gemm_launch<Cfg8>(Pw, Qx, F, (int)M, (long)d, 1, LoadIdentity{}, LoadIdentity{}, e1, s);
+  int st = launch8<Cfg8>(Pw, Qx, F, (int)M, (long)d, e1, s);
   if (st != TFB_OK) return st;
   GemmOperand Pp{b + 2 * n, (long)F}, Qh{(const uint8_t*)h8, (long)F};
   EpiDescaleRes e2{(const float*)row, SC_DQ_PROJ, nullptr, nullptr, 1.0f, (const bf16_t*)res, (bf16_t*)y, (long)d};
-  return gemm_launch<Cfg8>(Pp, Qh, d, (int)M, (long)F, 1, LoadIdentity{}, LoadIdentity{}, e2, s);
+  return launch8<Cfg8>(Pp, Qh, d, (int)M, (long)F, e2, s);
 }
 
 // Backward: dy8 [M][d] e5m2 (cast at the row's s_dy), r [M][F] -> dx [M][d], dpre [M][F] bf16, h [M][F] bf16 (optional,
@@ -843,7 +882,7 @@ extern "C" int tfb_mlp8_bwd_q(const void* dy8, const void* r, const void* w8, co
   if (st != TFB_OK) return st;
   GemmOperand Pf{b + n, (long)F}, Qd{(const uint8_t*)dp8, (long)F};  // wf8T [d][F]
   EpiScaleStore e2{(const float*)row, SC_DQ_DX, (bf16_t*)dx, (long)d};
-  return gemm_launch<Cfg8g>(Pf, Qd, d, (int)M, (long)F, 1, LoadIdentity{}, LoadIdentity{}, e2, s);
+  return launch8<Cfg8g>(Pf, Qd, d, (int)M, (long)F, e2, s);
 }
 extern "C" int tfb_mlp8_bwd(const void* dy8, const void* r, const void* w8, const void* row, void* dx, void* h, void* dpre,
                             void* dp8, long M, int d, int F, void* stream) {
