@@ -274,6 +274,8 @@ int tfb_attn_bwd(const void* q, const long* q_strides, const void* k, const long
  * array inside the library (8 MiB per GPU, held until the process ends) instead of from the caller. It allocates and
  * frees nothing. B * H * T <= tfb_attn_bwd_static_max_rows() (1,048,576), otherwise status 4 and the caller uses
  * tfb_attn_bwd. All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams) race.
+ * The first call on a device looks up the array's address (hipGetSymbolAddress) and sets the kernels' LDS size
+ * attribute: make one call eagerly on each device (same head dimension) before capturing a call into a HIP graph.
  * Has no counterpart in the reference (its kernels allocate their own outputs and scratch through the NKI runtime). */
 long tfb_attn_bwd_static_max_rows(void);
 int tfb_attn_bwd_static(const void* q, const long* q_strides, const void* k, const long* k_strides, const void* v,
@@ -330,10 +332,11 @@ int tfb_loss_multi_fwd(const void* logits, const void* targets, int idx64, const
 int tfb_loss_multi_bwd(const void* logits, const void* targets, int idx64, const void* row_w, int K, float eps, const void* lse,
                        const void* g, void* dlogits, long rows, int V, float softcap, void* stream);
 
-/* w fp32 [rows] = each row's weight in the reduced loss: (t >= 0) / max(1, #{t >= 0}) when mean != 0 (the mean over the
- * rows whose target counts, targets < 0 ignored), (t >= 0) otherwise. One launch for the compare / sum / clamp / divide the
- * caller of fused_loss(reduction=) makes on the host side (round1/source/train.py:4703-4707 scales the row losses there). */
-int tfb_loss_row_weights(const void* targets, int idx64, void* w, long rows, int mean, void* stream);
+/* w fp32 [rows] = each row's weight in the reduced loss: valid / max(1, #valid) when mean != 0 (the mean over the rows
+ * whose target counts), valid otherwise; valid = 0 <= t < V, the rows the loss kernels give a loss to (V <= 0: no upper
+ * bound). One launch for the compare / sum / clamp / divide the caller of fused_loss(reduction=) makes on the host side
+ * (round1/source/train.py:4703-4707 scales the row losses there). */
+int tfb_loss_row_weights(const void* targets, int idx64, void* w, long rows, int mean, int V, void* stream);
 
 /* tfb_loss_fwd followed by tfb_loss_bwd with grow = row_w (an upstream gradient of one), in place and in ONE pass over the
  * logits (a row is held in a workgroup's registers, V <= 65536; TFB_ERR_SHAPE beyond): loss and lse as tfb_loss_fwd writes

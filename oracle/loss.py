@@ -34,9 +34,11 @@ def loss_rows(logits2, targets, softcap=15.0):
     return torch.where(valid, lse - picked, torch.zeros_like(lse)), lse
 
 
-def row_weights(targets, reduction="mean"):
-    """valid / sum(valid) for "mean", valid for "sum"."""
-    valid = (targets.reshape(-1) >= 0).float()
+def row_weights(targets, reduction="mean", V=None):
+    """valid / sum(valid) for "mean", valid for "sum"; a row is valid when 0 <= t < V (V None: when t >= 0): the rows
+    loss_rows gives a loss to."""
+    t = targets.reshape(-1)
+    valid = ((t >= 0) if V is None else ((t >= 0) & (t < V))).float()
     return valid / valid.sum().clamp_min(1.0) if reduction == "mean" else valid
 
 
@@ -45,7 +47,7 @@ def fused_loss(logits, targets, reduction="mean", softcap=15.0):
     rows, _ = loss_rows(logits.reshape(-1, V), targets, softcap)
     if reduction == "none":
         return rows.view_as(targets)
-    return (rows * row_weights(targets, reduction)).sum()
+    return (rows * row_weights(targets, reduction, V)).sum()
 
 
 def loss_backward(logits2, targets, lse, grow, softcap=15.0):
@@ -76,7 +78,7 @@ def lmhead_loss_backward(x, norm_w, W, targets, saved, eps=1e-6, softcap=None, g
     from . import norm as _n
     xn, inv, logits = saved
     _, lse = loss_rows(logits, targets, softcap)
-    grow = row_weights(targets, "mean") * gloss
+    grow = row_weights(targets, "mean", logits.shape[-1]) * gloss
     dl = loss_backward(logits, targets, lse, grow, softcap)
     dxn = (dl.float() @ W.float()).to(x.dtype)
     dW = (dl.float().t() @ xn.float()).to(x.dtype)

@@ -92,7 +92,7 @@ class _Loss(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits2, targets, softcap):
         rows, lse = oloss.loss_rows(logits2, targets, softcap)
-        w = oloss.row_weights(targets, "mean")
+        w = oloss.row_weights(targets, "mean", logits2.shape[-1])
         ctx.save_for_backward(logits2, targets, lse, w)
         ctx.softcap = softcap
         return (rows * w).sum()

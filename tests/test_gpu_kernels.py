@@ -586,6 +586,66 @@ def test_mlp8_full_size_properties(ops, dev):
     assert torch.isfinite(dx.float()).all() and torch.isfinite(y.float()).all()
 
 
+@pytest.mark.parametrize("shape", [(512, 256, 512), (16384, 768, 3072)])
+def test_mlp8_as_the_benchmark_times_it(ops, dev, shape):
+    """Configuration 3 of BASELINE.json in the form bench.py times: OCP e4m3 at 448, the activation scale from the tensor's
+    amax (a power of two, left on the device), all six GEMMs in fp8 (weight gradients from the bytes the other GEMMs
+    multiplied), through the autograd wrapper. Against the oracle with the same limit and the same activation scale:
+    y and dx on two 512-row slices (2e-2), both weight gradients over all rows (2e-2)."""
+    from oracle import mlp8 as O
+    from trainium_frontier_them_bones_amd import autograd as A
+    M, d, F = shape
+    g = _g(20263)
+    x = torch.randn(M, d, generator=g).bfloat16()
+    wf = (0.02 * torch.randn(d, F, generator=g)).bfloat16().t().contiguous()      # W_up [d, F] -> [F, d]
+    wp = (0.02 * torch.randn(F, d, generator=g)).bfloat16().t().contiguous()      # W_down [F, d] -> [d, F]
+    dy = torch.randn(M, d, generator=g).bfloat16()
+    xl, wfl, wpl = (t.to(dev).requires_grad_(True) for t in (x, wf, wp))
+    st = A.Mlp8State(e4m3_limit=448.0, dw_fp8=True)
+    sc = ops.amax_scale(xl.detach(), 448.0, -20, 20)
+    st.x_scale = sc[0:1]
+    st.refresh(wfl, wpl)
+    y = A.Mlp8Fn.apply(xl, wfl, wpl, st)
+    y.backward(dy.to(dev))
+    # the oracle's activation scale: the largest power of two s with amax(x) s <= 448
+    xs, _ = O.pow2_floor_scale(x.float().abs().amax(), 448.0, -20, 20)
+    assert float(sc[0].item()) == float(xs)
+    xs = float(xs)
+    row_o = O.forward_scales(wf, wp, 448.0, xs)
+    assert torch.equal(st.row.cpu()[[0, 1, 2, 3, 4]], row_o[[0, 1, 2, 3, 4]])
+    yo, ro = O.forward(x, wf, wp, row_o, xs)
+    rowb_o = O.backward_scales(dy, row_o)
+    dxo, ho, dpo = O.backward(dy, ro, wf, wp, rowb_o)
+    for sl in (slice(0, 512), slice(M - 512, M)):
+        assert rel_l2(y[sl], yo[sl]) < FP8_TOL and rel_l2(xl.grad[sl], dxo[sl]) < FP8_TOL
+    o_fc, o_pj = O.weight_grads_fp8(x, dy, ho, dpo, rowb_o, x_scale=xs, e4m3_limit=448.0)
+    assert rel_l2(wfl.grad, o_fc) < FP8_TOL and rel_l2(wpl.grad, o_pj) < FP8_TOL
+    # and within the fp8 budget of the plain bf16 layer (the reference's off-device expression)
+    b_fc, b_pj = O.weight_grads(dy, x, ho, dpo)
+    assert rel_l2(wfl.grad, b_fc) < 0.08 and rel_l2(wpl.grad, b_pj) < 0.08
+
+
+@pytest.mark.parametrize("shape", [(2048, 1024, 1024, 128), (512, 4096, 1536, 128), (8192, 256, 1984, 128)])
+def test_gemm_256_tile_kernel_equals_the_128_tile_kernel(ops, dev, shape):
+    """A product large enough for the persistent 256 x 256 kernel (both operands k-contiguous, 16 to 31 k-tiles: long enough
+    for that kernel, short enough that no k-split is chosen) equals, bit for bit, the same product assembled from column
+    slices too narrow for it (which run the 128 x 128 kernel): the two kernels add the same terms in the same order. Also
+    against the fp64 product, with the residual add in the store and with the device scalar factor."""
+    M, N, K, w = shape
+    g = _g(M + N + K)
+    a = torch.randn(M, K, generator=g).bfloat16().to(dev)
+    b = torch.randn(N, K, generator=g).bfloat16().to(dev)
+    c = ops.matmul(a, b, trans_b=True)
+    parts = [ops.matmul(a, b[n0:n0 + w].contiguous(), trans_b=True) for n0 in range(0, N, w)]
+    assert torch.equal(c, torch.cat(parts, dim=1))
+    ref = a[:256].double() @ b.double().t()
+    assert rel_l2(c[:256], ref) < BF16_TOL
+    res = torch.randn(M, N, generator=g).bfloat16().to(dev)
+    assert torch.equal(ops.matmul_res(a, b, res, trans_b=True), (c.float() + res.float()).bfloat16())
+    al = torch.tensor([0.37], device=dev)
+    assert rel_l2(ops.matmul(a, b, trans_b=True, alpha=al)[:256], 0.37 * ref) < BF16_TOL
+
+
 # ------------------------------------------------------------------------------------------ attention
 @pytest.mark.parametrize("shape", [(1, 2, 128, 64), (2, 3, 512, 64), (1, 1, 1024, 64), (1, 2, 256, 128), (2, 1, 512, 128)])
 def test_attention_fwd_bwd(ops, dev, shape):
@@ -721,6 +781,34 @@ def test_attention_full_size_properties(ops, dev):
     assert rel_l2(dv1[3, 5, :, 0], p.sum(0)) < BF16_TOL
 
 
+@pytest.mark.parametrize("T,nw", [(2048, 0), (4096, 0), (2048, 4), (4096, 4)])
+def test_attention_head_dim_128_at_the_reference_lengths(ops, dev, T, nw):
+    """Head dimension 128 (the reference's own models) at the sequence lengths the reference runs it on, B2 H6: two
+    (batch, head) pairs against the oracle, forward and backward, the full causal triangle and a band of four tiles."""
+    from oracle import attention as O
+    B, H, D = 2, 6, 128
+    g = _g(T + nw)
+    q, k, v = (torch.randn(B, H, T, D, generator=g).bfloat16() for _ in range(3))
+    do = torch.randn(B, T, H, D, generator=g).bfloat16()
+    scale = 1.0 / math.sqrt(D)
+    qd, kd, vd, dod = q.to(dev), k.to(dev), v.to(dev), do.to(dev)
+    band = nw if nw else None
+    if nw:
+        o, lse = ops.attn_fwd(qd, kd, vd, scale, band=nw)
+        dq, dk, dv = ops.attn_bwd(qd, kd, vd, o, dod, lse, scale, band=nw)
+    else:
+        o, lse = ops.attn_fwd(qd, kd, vd, scale)
+        dq, dk, dv = ops.attn_bwd(qd, kd, vd, o, dod, lse, scale)
+    for (b, h) in ((0, 1), (1, 5)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        oo, lo = O.forward(q[sl], k[sl], v[sl], scale, band_tiles=band)
+        assert rel_l2(o[b:b + 1, :, h:h + 1], oo) < BF16_TOL and rel_l2(lse[sl], lo) < 1e-4
+        dqo, dko, dvo = O.backward(q[sl], k[sl], v[sl], o[b:b + 1, :, h:h + 1].cpu(), do[b:b + 1, :, h:h + 1], lse[sl].cpu(),
+                                   scale, band_tiles=band)
+        assert rel_l2(dq[sl], dqo) < BF16_TOL and rel_l2(dk[sl], dko) < BF16_TOL and rel_l2(dv[sl], dvo) < BF16_TOL
+
+
+
 # ------------------------------------------------------------------------------------------ loss head
 @pytest.mark.parametrize("cap", [15.0, None])
 def test_loss_fwd_bwd(ops, dev, cap):
@@ -732,7 +820,7 @@ def test_loss_fwd_bwd(ops, dev, cap):
     t[5] = -1
     t[9] = V                                                                   # beyond the vocabulary: ignored too, never an address
     t[11] = 1 << 40
-    w = O.row_weights(t, "mean")
+    w = O.row_weights(t, "mean", V)
     rows, lse = ops.loss_fwd(x.to(dev), t.to(dev), cap, w.to(dev))
     assert float(rows[9]) == 0.0 and float(rows[11]) == 0.0
     ro, lo = O.loss_rows(x, t, cap)
@@ -818,7 +906,7 @@ def test_lmhead_loss_node_with_an_upstream_gradient(ops, dev):
     (0.37 * A.LmHeadLossFn.apply(xd, Wd, td, 15.0, "mean")).backward()
     assert rel_l2(xd.grad, 0.37 * gx.float()) < BF16_TOL and rel_l2(Wd.grad, 0.37 * gw.float()) < BF16_TOL
     _, lse_o = O.loss_rows(F_linear(x, W), t, 15.0)
-    grow = 0.37 * O.row_weights(t, "mean")
+    grow = 0.37 * O.row_weights(t, "mean", V)
     dlo = O.loss_backward(F_linear(x, W), t, lse_o, grow, 15.0)
     assert rel_l2(xd.grad, dlo.float() @ W.float()) < BF16_TOL and rel_l2(Wd.grad, dlo.float().t() @ x.float()) < BF16_TOL
 
@@ -1016,3 +1104,52 @@ def test_loss_row_weights_equal_the_host_expression(ops, dev):
             assert torch.equal(ops.loss_row_weights(t, "sum"), valid)
     none = torch.full((777,), -1, dtype=torch.int64, device=dev)
     assert torch.equal(ops.loss_row_weights(none, "mean"), torch.zeros(777, device=dev))
+    # with the vocabulary size given, a target at or beyond it is a row without a loss: it counts neither in the numerator
+    # nor in the mean's denominator (the loss kernels give such a row 0)
+    t = torch.tensor([3, 999, 1000, -1, 5000, 0], dtype=torch.int64, device=dev)
+    want = torch.tensor([1, 1, 0, 0, 0, 1], dtype=torch.float32, device=dev)
+    assert torch.equal(ops.loss_row_weights(t, "mean", 1000), want / 3.0)
+    assert torch.equal(ops.loss_row_weights(t, "sum", 1000), want)
+
+
+def test_lm_head_loss_without_grad_takes_the_forward_only_path(ops, dev):
+    """Under torch.no_grad() the LM-head wrapper runs the GEMM with the log-sum-exp in its epilogue (no dlogits pass) even when
+    its inputs are parameters; the loss equals the training path's."""
+    from trainium_frontier_them_bones_amd import autograd as A
+    g = _g(123)
+    x = torch.randn(256, 128, generator=g).bfloat16().to(dev).requires_grad_(True)
+    W = (0.05 * torch.randn(512, 128, generator=g)).bfloat16().to(dev).requires_grad_(True)
+    t = torch.randint(0, 512, (256,), generator=g).to(dev)
+    calls = []
+    real = ops.loss_fwd_bwd
+    ops.loss_fwd_bwd = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
+    try:
+        train = A.LmHeadLossFn.apply(x, W, t, 0.0, "mean")
+        assert calls == [1]
+        with torch.no_grad():
+            ev = A.LmHeadLossFn.apply(x, W, t, 0.0, "mean")
+        assert calls == [1]
+    finally:
+        ops.loss_fwd_bwd = real
+    assert abs(train.item() - ev.item()) < 1e-5 * abs(train.item())
+
+
+def test_mean_loss_with_a_target_beyond_the_vocabulary(ops, dev):
+    """A target id >= V is a row without a loss: the mean divides by the rows that have one. LM-head wrapper against the
+    oracle's mean and against F.cross_entropy over the rows that count."""
+    from oracle import loss as O
+    from trainium_frontier_them_bones_amd import autograd as A
+    g = _g(99)
+    N, d, V = 256, 128, 512
+    x = torch.randn(N, d, generator=g).bfloat16()
+    W = (0.05 * torch.randn(V, d, generator=g)).bfloat16()
+    t = torch.randint(0, V, (N,), generator=g)
+    t[7] = V + 3
+    t[100] = -1
+    logits = (x.float() @ W.float().t()).bfloat16()
+    want = O.fused_loss(logits, t, "mean", None)
+    keep = (t >= 0) & (t < V)
+    ref = torch.nn.functional.cross_entropy(logits.float()[keep], t[keep])
+    assert abs(want.item() - ref.item()) < 1e-5
+    got = A.LmHeadLossFn.apply(x.to(dev).requires_grad_(True), W.to(dev).requires_grad_(True), t.to(dev), 0.0, "mean")
+    assert abs(got.item() - want.item()) < 1e-3 * want.item()

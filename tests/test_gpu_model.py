@@ -117,6 +117,26 @@ def test_gradient_accumulation_in_place(dev):
         assert rel_l2(p.grad_buf, 2 * once[k].float()) < 1e-2, k
 
 
+def test_full_size_batch_first_loss_against_the_oracle(dev):
+    """Configuration 4 of BASELINE.json at its stated batch (16 sequences of 2048 tokens): the loss of the first forward pass
+    against the mean of the oracle's sixteen per-sequence forward losses (equal lengths, no ignored target: the batch mean),
+    within 1e-3 relative."""
+    from oracle.model import OracleGPT
+    from trainium_frontier_them_bones_amd.model import GPT, GPTConfig, zipf_tokens
+    cfg = GPTConfig()
+    m = GPT(cfg, dev, seed=0)
+    o = OracleGPT(cfg, m.init_values)
+    idx, tg = zipf_tokens(16, cfg.seq_len, cfg.vocab, seed=0)
+    got = m.forward(idx.to(dev), tg.to(dev)).item()
+    per = []
+    with torch.no_grad():
+        for b in range(16):
+            print("oracle forward, sequence %d" % b, flush=True)
+            per.append(o.forward(idx[b:b + 1], tg[b:b + 1]).item())
+    want = sum(per) / len(per)
+    assert abs(got - want) < 1e-3 * want, (got, want)
+
+
 def test_full_size_step_runs_and_loss_is_sane(dev):
     from trainium_frontier_them_bones_amd.model import GPT, GPTConfig, zipf_tokens
     import math

@@ -53,6 +53,61 @@ def test_attn_bwd_static_matches_attn_bwd_on_two_calls_in_a_row(ops, dev):
     _case(ops, dev, 1, 2, 256, 128, 73, fused=False)       # the D = 128 kernels read the same scratch
 
 
+def test_attn_bwd_static_captured_into_a_hip_graph(ops, dev):
+    """After one eager call (which resolves the static array's address and the kernels' LDS attributes), the entry point is
+    captured into a HIP graph: three replays on new inputs, with eager calls and synchronisations between them, each
+    equal to tfb_attn_bwd's gradients bit for bit."""
+    B, H, T, D = 2, 4, 512, 64
+    g = torch.Generator().manual_seed(81)
+
+    def fresh():
+        q, k, v = (torch.randn(B, H, T, D, generator=g).bfloat16().to(dev) for _ in range(3))
+        do = torch.randn(B, T, H, D, generator=g).bfloat16().to(dev)
+        o, lse = ops.attn_fwd(q, k, v, 0.125)
+        return q, k, v, o, do, lse
+
+    static = fresh()
+    outs = tuple(torch.empty(B, H, T, D, dtype=torch.bfloat16, device=dev) for _ in range(3))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.attn_bwd_static(*static, 0.125, *outs)            # the warm-up the capture needs
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.attn_bwd_static(*static, 0.125, *outs)
+    for rep in range(3):
+        print("attn_bwd_static graph replay %d" % rep, flush=True)
+        new = fresh()
+        want = tuple(torch.empty(B, H, T, D, dtype=torch.bfloat16, device=dev) for _ in range(3))
+        ops.attn_bwd(*new, 0.125, dq=want[0], dk=want[1], dv=want[2])   # eager work between the replays
+        torch.cuda.synchronize()
+        for s_, n_ in zip(static, new):
+            s_.copy_(n_)
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(outs, want):
+            assert torch.equal(a, b)
+
+
+def test_attn_bwd_host_checks_reject_mismatched_tensors(ops, dev):
+    q, k, v = (torch.zeros(1, 2, 256, 64, dtype=torch.bfloat16, device=dev) for _ in range(3))
+    o = torch.zeros(1, 256, 2, 64, dtype=torch.bfloat16, device=dev)
+    lse = torch.zeros(1, 2, 256, dtype=torch.float32, device=dev)
+    outs = tuple(torch.zeros(1, 2, 256, 64, dtype=torch.bfloat16, device=dev) for _ in range(3))
+    with pytest.raises(ValueError):
+        ops.attn_bwd_static(q, k, v, o, o, lse[:, :1], 0.125, *outs)               # lse too short
+    with pytest.raises(ValueError):
+        ops.attn_bwd_static(q, k, v, o, o, lse.double(), 0.125, *outs)             # lse not fp32
+    with pytest.raises(ValueError):
+        ops.attn_bwd_static(q, k[:, :1], v, o, o, lse, 0.125, *outs)               # k with fewer heads
+    with pytest.raises(ValueError):
+        ops.attn_bwd(q, k, v, o.permute(0, 2, 1, 3), o, lse, 0.125)                # o not [B, T, H, D]
+    with pytest.raises(ValueError):
+        ops.attn_bwd_static(q, k, v, o, o, lse, 0.125, outs[0], outs[1], outs[2][:, :, :128])   # dv too short
+
+
 def test_attn_bwd_static_refuses_sizes_beyond_its_array(ops, dev):
     from trainium_frontier_them_bones_amd import _lib
     max_rows = ops.attn_bwd_static_max_rows()

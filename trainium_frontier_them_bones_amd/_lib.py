@@ -72,7 +72,7 @@ SIGNATURES = {
     "tfb_fill_f32": [_vp, _f, _l, _vp],
     "tfb_loss_fwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_loss_fwd_bwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
-    "tfb_loss_row_weights": [_vp, _i, _vp, _l, _i, _vp],
+    "tfb_loss_row_weights": [_vp, _i, _vp, _l, _i, _i, _vp],
     "tfb_loss_bwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_loss_multi_fwd": [_vp, _vp, _i, _vp, _i, _f, _vp, _vp, _l, _i, _f, _vp],
     "tfb_loss_multi_bwd": [_vp, _vp, _i, _vp, _i, _f, _vp, _vp, _vp, _l, _i, _f, _vp],

@@ -547,14 +547,24 @@ class LmHeadLossFn(torch.autograd.Function):
     exponential. Without a gradient (or beyond the one-pass kernel's vocabulary limit) the GEMM with the log-sum-exp in its
     epilogue runs instead, and a backward from there writes dlogits in place of the logits first."""
 
+    _caller_grad_mode = True
+
+    @classmethod
+    def apply(cls, *args):
+        # inside forward() the grad mode is always off, and needs_input_grad is True for parameters under torch.no_grad()
+        # as well: the caller's mode is noted here, so that evaluation takes the cheaper forward
+        cls._caller_grad_mode = torch.is_grad_enabled()
+        return super().apply(*args)
+
     @staticmethod
     def forward(ctx, x, W, targets, softcap, reduction):
         x2 = x.reshape(-1, x.shape[-1]).contiguous()
         tg = targets.reshape(-1)
-        w = ops.loss_row_weights(tg, reduction)
+        w = ops.loss_row_weights(tg, reduction, W.shape[0])
         ctx.softcap = softcap
         ctx.xshape = x.shape
-        ctx.one_pass = (LM_HEAD_ONE_PASS and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
+        ctx.one_pass = (LM_HEAD_ONE_PASS and LmHeadLossFn._caller_grad_mode
+                        and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
                         and W.shape[0] <= ops.LOSS_FWD_BWD_MAX_V)
         if ctx.one_pass:
             dl = ops.matmul(x2, W, trans_b=True)

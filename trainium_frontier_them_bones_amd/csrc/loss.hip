@@ -40,10 +40,12 @@ __device__ __forceinline__ MS ms_merge(MS a, MS b) {
 }
 
 // ------------------------------------------------------------------------------------ row weights
-// One workgroup: w[i] = (t_i >= 0) / max(1, #{t >= 0}) for the mean over the rows that count (mean != 0), else (t_i >= 0).
+// One workgroup: w[i] = valid_i / max(1, #valid) for the mean over the rows that count (mean != 0), else valid_i; a row
+// counts when 0 <= t_i < V (V <= 0: when 0 <= t_i): the rows the loss kernels give a loss to.
 template <typename IDX>
 __global__ __launch_bounds__(1024) void loss_row_weights_kernel(const IDX* __restrict__ tg, float* __restrict__ w, long rows,
-                                                               int mean) {
+                                                               int mean, long V) {
+  auto valid = [&](IDX t) { return t >= 0 && (long)t < V; };
   __shared__ int cnt[16];
   float each = 1.0f;
   if (mean) {
@@ -53,7 +55,7 @@ __global__ __launch_bounds__(1024) void loss_row_weights_kernel(const IDX* __res
 #pragma unroll
       for (int k = 0; k < 4; ++k) t[k] = i + 1024 * k < rows ? tg[i + 1024 * k] : (IDX)-1;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) c += t[k] >= 0;
+      for (int k = 0; k < 4; ++k) c += valid(t[k]);
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
@@ -64,7 +66,7 @@ __global__ __launch_bounds__(1024) void loss_row_weights_kernel(const IDX* __res
     for (int k = 0; k < 16; ++k) n += cnt[k];
     each = 1.0f / (float)(n > 1 ? n : 1);
   }
-  for (long i = threadIdx.x; i < rows; i += 1024) w[i] = tg[i] >= 0 ? each : 0.f;
+  for (long i = threadIdx.x; i < rows; i += 1024) w[i] = valid(tg[i]) ? each : 0.f;
 }
 
 // ------------------------------------------------------------------------------------ loss on logits
@@ -514,17 +516,19 @@ extern "C" int tfb_loss_fwd(const void* logits, const void* targets, int idx64, 
   return TFB_OK;
 }
 
-// w fp32 [rows]: the weight of each row's loss in the reduction, (t >= 0) / max(1, number of rows with t >= 0) for the
-// mean over the rows that count (mean != 0: F.cross_entropy(ignore_index < 0) semantics), (t >= 0) for the sum. One small
-// launch in place of a compare, a cast, a sum, a clamp and a division.
-extern "C" int tfb_loss_row_weights(const void* targets, int idx64, void* w, long rows, int mean, void* stream) {
+// w fp32 [rows]: the weight of each row's loss in the reduction, valid / max(1, number of valid rows) for the mean over the
+// rows that count (mean != 0: F.cross_entropy(ignore_index < 0) semantics), valid for the sum; valid = 0 <= t < V, the rows
+// the loss kernels give a loss to (V <= 0: no upper bound). One small launch in place of a compare, a cast, a sum, a clamp
+// and a division.
+extern "C" int tfb_loss_row_weights(const void* targets, int idx64, void* w, long rows, int mean, int V, void* stream) {
   if (!targets || !w) return TFB_ERR_ARG;
   if (rows <= 0) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
+  const long vmax = V > 0 ? (long)V : (1L << 62);
   if (idx64)
-    hipLaunchKernelGGL(loss_row_weights_kernel<long>, dim3(1), dim3(1024), 0, s, (const long*)targets, (float*)w, rows, mean);
+    hipLaunchKernelGGL(loss_row_weights_kernel<long>, dim3(1), dim3(1024), 0, s, (const long*)targets, (float*)w, rows, mean, vmax);
   else
-    hipLaunchKernelGGL(loss_row_weights_kernel<int>, dim3(1), dim3(1024), 0, s, (const int*)targets, (float*)w, rows, mean);
+    hipLaunchKernelGGL(loss_row_weights_kernel<int>, dim3(1), dim3(1024), 0, s, (const int*)targets, (float*)w, rows, mean, vmax);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

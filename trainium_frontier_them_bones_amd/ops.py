@@ -484,6 +484,30 @@ def _attn_chk(t):
         raise TypeError("attention takes bf16 device tensors")
 
 
+def _attn_bwd_chk(q, k, v, o, do, lse, dq, dk, dv, layout, out_layout):
+    """Host checks of an attention backward call: a tensor of the wrong shape, or a log-sum-exp that is not fp32
+    [B, H, T] contiguous, would be an out-of-bounds access on the device (the entry point sees only pointers and strides)."""
+    for t in (q, k, v, o, do, dq, dk, dv):
+        _attn_chk(t)
+        if t.dim() != 4:
+            raise ValueError("attention tensors are 4-D")
+    B, H, T, D = q.shape if layout == "bhtd" else (q.shape[0], q.shape[2], q.shape[1], q.shape[3])
+    if T % 128 or D not in (64, 128):
+        raise ValueError("attention takes T % 128 == 0 and D 64 or 128")
+    inp = (B, H, T, D) if layout == "bhtd" else (B, T, H, D)
+    outp = (B, H, T, D) if out_layout == "bhtd" else (B, T, H, D)
+    if tuple(k.shape) != inp or tuple(v.shape) != inp or tuple(q.shape) != inp:
+        raise ValueError("q, k, v shapes differ")
+    if tuple(o.shape) != (B, T, H, D) or tuple(do.shape) != (B, T, H, D):
+        raise ValueError("o and do are [B, T, H, D]")
+    for t in (dq, dk, dv):
+        if tuple(t.shape) != outp:
+            raise ValueError("dq, dk, dv shapes do not match out_layout")
+    if not lse.is_cuda or lse.dtype != torch.float32 or not lse.is_contiguous() or lse.numel() != B * H * T:
+        raise ValueError("lse is fp32 [B, H, T] contiguous")
+    return B, H, T, D
+
+
 def attn_fwd(q, k, v, scale, layout="bhtd", band=0):
     """q, k, v: 4-D views [B,H,T,D] ("bhtd") or [B,T,H,D] ("bthd"), arbitrary batch/head/token strides.
     Returns o [B,T,H,D] contiguous and lse [B,H,T] fp32. band = nw > 0: the reference's tile band (a query of 128-token
@@ -509,8 +533,9 @@ def attn_bwd(q, k, v, o, do, lse, scale, layout="bhtd", dq=None, dk=None, dv=Non
     """Gradients of attn_fwd. o, do are [B,T,H,D]. dq/dk/dv may be given as (strided) views with `out_layout`;
     otherwise dq, dk are allocated [B,H,T,D] and dv [B,T,H,D] (returned as a [B,H,T,D] view), as the reference returns.
     rope = (cos, sin) (bf16 [T, D/2]): dq and dk come back with the inverse rotation applied (D = 64)."""
-    for t in (q, k, v, o, do):
-        _attn_chk(t)
+    _attn_chk(q)
+    if q.dim() != 4:
+        raise ValueError("attention tensors are 4-D")
     if layout == "bhtd":
         B, H, T, D = q.shape
     else:
@@ -520,6 +545,7 @@ def attn_bwd(q, k, v, o, do, lse, scale, layout="bhtd", dq=None, dk=None, dv=Non
         dk = torch.empty(B, H, T, D, dtype=bf16, device=q.device)
         dv = torch.empty(B, T, H, D, dtype=bf16, device=q.device).permute(0, 2, 1, 3)
         out_layout = "bhtd"
+    _attn_bwd_chk(q, k, v, o, do, lse, dq, dk, dv, layout, out_layout)
     delta = torch.empty(2, B, H, T, dtype=torch.float32, device=q.device)
     cos, sin = rope if rope is not None else (None, None)
     _chk(cos), _chk(sin)
@@ -543,13 +569,10 @@ def attn_bwd_static_max_rows():
 def attn_bwd_static(q, k, v, o, do, lse, scale, dq, dk, dv, layout="bhtd", out_layout="bhtd"):
     """attn_bwd into caller-provided dq, dk, dv through the entry point that allocates nothing: its row-statistic scratch
     is a static device array inside the library (B * H * T <= tfb_attn_bwd_static_max_rows(); TfbError status 4 beyond).
-    Calls that overlap on one GPU share that array and race; this wrapper creates no tensor either."""
-    for t in (q, k, v, o, do, dq, dk, dv):
-        _attn_chk(t)
-    if layout == "bhtd":
-        B, H, T, D = q.shape
-    else:
-        B, T, H, D = q.shape
+    Calls that overlap on one GPU share that array and race; this wrapper creates no tensor either. The FIRST call on a
+    device looks up the array's address and sets the kernels' LDS attributes: make one call (or any attention backward of
+    the same head dimension) eagerly before capturing this one into a HIP graph."""
+    B, H, T, D = _attn_bwd_chk(q, k, v, o, do, lse, dq, dk, dv, layout, out_layout)
     _lib.call("tfb_attn_bwd_static", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o),
               _bht(o, "bthd"), _p(do), _bht(do, "bthd"), _p(dq), _bht(dq, out_layout), _p(dk), _bht(dk, out_layout), _p(dv),
               _bht(dv, out_layout), _p(lse), B, H, T, D, float(scale), _stream())
@@ -711,12 +734,13 @@ def loss_bwd(logits2, targets, lse, grow, softcap=15.0, inplace=False):
     return out
 
 
-def loss_row_weights(targets, reduction="mean"):
-    """fp32 [N] weights of the row losses in the reduced loss: (t >= 0) / max(1, count of t >= 0) for "mean", (t >= 0) for
-    "sum" (targets < 0 are ignored rows)."""
+def loss_row_weights(targets, reduction="mean", V=None):
+    """fp32 [N] weights of the row losses in the reduced loss: valid / max(1, count of valid) for "mean", valid for "sum";
+    a row is valid when 0 <= t < V (the rows the loss kernels give a loss to; V None: when t >= 0)."""
     tg = _tg(targets)
     w = torch.empty(tg.numel(), dtype=torch.float32, device=tg.device)
-    _lib.call("tfb_loss_row_weights", _p(tg), int(tg.dtype == torch.int64), _p(w), tg.numel(), int(reduction == "mean"), _stream())
+    _lib.call("tfb_loss_row_weights", _p(tg), int(tg.dtype == torch.int64), _p(w), tg.numel(), int(reduction == "mean"),
+              int(V or 0), _stream())
     return w
 
 

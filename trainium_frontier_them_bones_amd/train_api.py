@@ -91,7 +91,7 @@ def fused_loss(logits, targets, reduction="mean", softcap=LOGIT_SOFTCAP):
         return rows.sum()
     if reduction != "mean":
         raise ValueError("reduction must be 'mean', 'sum' or 'none'")
-    return rows.sum() / (t >= 0).sum().clamp_min(1).to(rows.dtype)
+    return rows.sum() / ((t >= 0) & (t < V)).sum().clamp_min(1).to(rows.dtype)   # the rows the kernel gives a loss to
 
 
 def fused_loss_multi(logits, tg, rw, softcap=LOGIT_SOFTCAP, ref=None):
@@ -114,7 +114,7 @@ def chunked_loss_mean(logits, targets, smooth=False, tok_w=None, eps=0.0):
     b, t, v = logits.shape
     n = b * t
     y = targets.reshape(n)
-    w = ops.loss_row_weights(y, "mean")
+    w = ops.loss_row_weights(y, "mean", v)
     if tok_w is not None:
         w = w * tok_w.reshape(n).to(torch.float32)
     x2 = logits.reshape(n, v).contiguous()
