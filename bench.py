@@ -14,6 +14,9 @@ python bench.py --config-probe c1|c2|c3|c5|all   (the standalone configurations 
 one line per configuration; run under rocprofv3 --kernel-trace --stats for the per-kernel durations; with --graphs a
 second line per configuration: the same repetition recorded once as a HIP graph and replayed, without the host's launch work)
 
+python bench.py --gemm-probe      (this library's bf16 GEMM beside torch.matmul, i.e. the vendor BLAS, on the step's own GEMM
+shapes and 8192^3, in one process on one box: a yardstick only, the product never calls the vendor library)
+
 python bench.py --traffic-probe   (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: a 256 MiB device copy as the
 counters' calibration, then attention forward + backward at the benchmark shape; prints nothing)
 """
@@ -165,6 +168,51 @@ def traffic_probe():
     torch.cuda.synchronize()
 
 
+def gemm_probe():
+    """This library's bf16 GEMM (tfb_gemm_bf16) beside torch.matmul (the vendor BLAS) on the step's GEMM shapes, 20 timed
+    calls each after 3 warm-up calls, alternating in one process; prints one table row per shape. The vendor library is the
+    yardstick only: nothing in the package calls it."""
+    import torch
+    from trainium_frontier_them_bones_amd import ops
+    dev = torch.device("cuda:0")
+
+    def t(f, n=20):
+        for _ in range(3):
+            f()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(n):
+            f()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / n * 1e3
+
+    M = 32768
+    shapes = [("QKV projection (NT)", M, 2304, 768, False, True), ("output projection (NT)", M, 768, 768, False, True),
+              ("32768 x 3072 x 768 (NT)", M, 3072, 768, False, True), ("QKV dX (NN)", M, 768, 2304, False, False),
+              ("output projection dX (NN)", M, 768, 768, False, False), ("QKV dW (TN)", 2304, 768, M, True, False),
+              ("MLP-shaped dW (TN)", 3072, 768, M, True, False), ("LM head logits (NT)", M, 32768, 768, False, True),
+              ("LM head dX (NN)", M, 768, 32768, False, False), ("LM head dW (TN)", 32768, 768, M, True, False),
+              ("8192^3 (NT)", 8192, 8192, 8192, False, True)]
+    print("| shape | m | n | k | vendor BLAS us | TFLOP/s | this library us | TFLOP/s | ratio | rel-L2 between them |")
+    print("|---|---|---|---|---|---|---|---|---|---|")
+    torch.manual_seed(0)
+    for name, m, n, k, ta, tb in shapes:
+        a = torch.randn((k, m) if ta else (m, k), device=dev).bfloat16()
+        b = torch.randn((n, k) if tb else (k, n), device=dev).bfloat16()
+        av, bv = (a.t() if ta else a), (b.t() if tb else b)
+        out = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
+        tv = t(lambda: torch.matmul(av, bv, out=out))
+        ref = out.float().clone()
+        tl = t(lambda: ops.matmul(a, b, trans_a=ta, trans_b=tb, out=out))
+        err = ((out.float() - ref).norm() / ref.norm()).item()
+        fl = 2.0 * m * n * k
+        print("| %s | %d | %d | %d | %.1f | %.0f | %.1f | %.0f | %.2f | %.1e |"
+              % (name, m, n, k, tv, fl / tv / 1e6, tl, fl / tl / 1e6, tv / tl, err), flush=True)
+        del a, b, out, ref
+
+
 def ns_probe():
     import torch
     from trainium_frontier_them_bones_amd import ops
@@ -309,6 +357,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true")
     ap.add_argument("--ns-probe", action="store_true")
+    ap.add_argument("--gemm-probe", action="store_true")
     ap.add_argument("--config-probe", choices=("c1", "c2", "c3", "c5", "all"))
     ap.add_argument("--graphs", action="store_true", help="with --config-probe: also time each repetition replayed as a HIP graph")
     ap.add_argument("--bf16-dw", action="store_true")
@@ -324,6 +373,9 @@ def main():
         return
     if args.ns_probe:
         ns_probe()
+        return
+    if args.gemm_probe:
+        gemm_probe()
         return
     if args.config_probe:
         config_probe(args.config_probe, args.graphs)
