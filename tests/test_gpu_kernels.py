@@ -625,6 +625,28 @@ def test_mlp8_as_the_benchmark_times_it(ops, dev, shape):
     assert rel_l2(wfl.grad, b_fc) < 0.08 and rel_l2(wpl.grad, b_pj) < 0.08
 
 
+@pytest.mark.parametrize("ta,tb", [(False, True), (False, False), (True, False), (True, True)])
+def test_gemm_long_contraction_in_every_operand_layout(ops, dev, ta, tb):
+    """Long contractions over at least 64 output tiles of 256 x 256 run the persistent kernel in all four operand layouts
+    (k-contiguous and k-strided operands, the latter through the transposing LDS reads), here with the k range cut into
+    four work items per tile and finished through the fp32 workspace: against the fp32 product of the same bf16 values,
+    also accumulated into an fp32 output and scaled by a device scalar; and without a split (one round of tiles), bit-equal
+    to the same product assembled from narrow column slices on the 128 x 128 kernel where that one does not split either."""
+    g = _g(17 + 2 * ta + tb)
+    for (M, N, K) in ((4096, 1024, 8192), (4096, 4096, 8192)):
+        a = torch.randn((K, M) if ta else (M, K), generator=g).bfloat16()
+        b = torch.randn((N, K) if tb else (K, N), generator=g).bfloat16()
+        ref = (a.float().t() if ta else a.float())[:512] @ (b.float().t() if tb else b.float())
+        ad, bd = a.to(dev), b.to(dev)
+        c = ops.matmul(ad, bd, trans_a=ta, trans_b=tb)
+        assert rel_l2(c[:512], ref) < BF16_TOL
+        if N == 1024:
+            acc = torch.randn(M, N, generator=g)
+            al = torch.tensor([0.5], device=dev)
+            got = ops.matmul(ad, bd, trans_a=ta, trans_b=tb, out=acc.to(dev).clone(), accumulate=True, alpha=al)
+            assert rel_l2(got[:512], 0.5 * ref + acc[:512]) < 1e-4
+
+
 @pytest.mark.parametrize("shape", [(2048, 1024, 1024, 128), (512, 4096, 1536, 128), (8192, 256, 1984, 128)])
 def test_gemm_256_tile_kernel_equals_the_128_tile_kernel(ops, dev, shape):
     """A product large enough for the persistent 256 x 256 kernel (both operands k-contiguous, 16 to 31 k-tiles: long enough

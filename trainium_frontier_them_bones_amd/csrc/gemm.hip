@@ -11,6 +11,32 @@ template <int LAYP, int LAYQ>
 int run(GemmOperand P, GemmOperand Q, int N, int M, int K, void* C, int out_f32, int accumulate, float* ws, long ws_bytes,
         const float* alpha, hipStream_t stream) {
   using Cfg = GemmCfg<128, 128, 2, 2, 2, LAYP, LAYQ>;
+  // Long contractions (at least 128 k-tiles) over at least 64 output tiles of 256 x 256, in any operand layout: the
+  // persistent 256 x 256 kernel, the k range cut into the fewest equal parts that fill whole rounds of the CUs to 90 %
+  // (the LM head's two gradient GEMMs: 384 tiles x 2 = 3 per CU), partial tiles through the fp32 workspace.
+#ifndef TFB_PP_LONGK
+#define TFB_PP_LONGK 1
+#endif
+  if (TFB_PP && TFB_PP_LONGK && N % 256 == 0 && M % 256 == 0 && K % 64 == 0 && K / 64 >= 128 && (long)(N / 256) * (M / 256) >= 64) {
+    const long t256 = (long)(N / 256) * (M / 256), nkt = K / 64, cus = tfb_resident_slots(1);
+    int sp = 0;
+    for (int c = 1; c <= 8 && !sp; ++c) {
+      if (nkt % c || nkt / c < 32) continue;
+      if (c > 1 && (!ws || (long)c * M * N * 4 > ws_bytes)) continue;
+      const long items = t256 * c, rounds = (items + cus - 1) / cus;
+      if ((double)items >= 0.9 * (double)(rounds * cus)) sp = c;
+    }
+    if (sp == 1 && !out_f32 && !accumulate) {
+      EpiStore e{C, (long)N, out_f32, accumulate, alpha};
+      return gemm_pp_launch_lay<2, 0, 0, LAYP, LAYQ>(P, Q, N, M, (long)K * 2, 1, e, stream);
+    }
+    if (sp > 1) {
+      EpiSplit e{ws, (long)N, (long)M * N};
+      int st = gemm_pp_launch_lay<2, 0, 0, LAYP, LAYQ>(P, Q, N, M, (long)K * 2, sp, e, stream);
+      if (st != TFB_OK) return st;
+      return splitk_reduce(ws, C, (long)M * N, sp, out_f32, accumulate, stream, nullptr, nullptr, 1.0f, alpha);
+    }
+  }
   const long tiles = (long)(N / 128) * (M / 128);
   const int splits = ws ? choose_splits(tiles, K / 64, (long)M * N, ws_bytes) : 1;
   if (splits == 1) {

@@ -742,6 +742,7 @@ struct EpiStoreGrouped {
 
 // fp32 partial of one k-split: ws [splits][nq][ld]
 struct EpiSplit {
+  static constexpr bool kSplitF32 = true;  // (the 256 x 256 kernel hands this epilogue the raw fp32 accumulators)
   float* ws;
   long ld, slab;  // slab = nq * ld
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], int split) const {

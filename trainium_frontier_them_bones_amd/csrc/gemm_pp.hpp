@@ -17,8 +17,15 @@
 // Fragment reads are inline assembly (ds_read_b128 with immediate offsets) with explicit s_waitcnt: left to the compiler,
 // every LDS read beside global -> LDS loads in flight would wait for vmcnt(0).
 //
-// LDS map (bytes): stage S at S * 65536: P half 0, P half 1, Q half 0, Q half 1 (16 KB each); row r of a half at r * 128,
-// 16-byte chunk c at slot c ^ tfb_kc_swz(r) (no bank conflicts for the 128-bit fragment reads).
+// LDS map (bytes): stage S at S * 65536: P half 0, P half 1, Q half 0, Q half 1 (16 KB each). A k-contiguous operand
+// ([rows][K]) keeps row r of a half at r * 128, 16-byte chunk c at slot c ^ tfb_kc_swz(r) (no bank conflicts for the 128-bit
+// fragment reads). A k-strided bf16 operand ([K][rows], the token-contraction GEMMs) keeps one k per 256-byte LDS row,
+// chunk c of k-row k at slot c ^ (4 (k & 3)), and its fragments come through ds_read_b64_tr_b16 (two per fragment), the
+// layout and lane map of the 128 x 128 kernel's K_STRIDED reader.
+//
+// Long contractions with few output tiles (the LM head's gradients: 384 tiles of 512 k-tiles) are split along k into
+// work items of equal length; each leaves its fp32 partial tile in a workspace (epilogues with kSplitF32, staged as
+// fp32) and splitk_reduce_kernel finishes them.
 #pragma once
 #include "gemm_core.hpp"
 
@@ -41,8 +48,11 @@ __device__ __forceinline__ T tfb_lds_read128(uint32_t addr) {
 
 struct PpArgs {
   GemmOperand P, Q;
-  int nkt;      // k-tiles per output tile (>= 2)
-  int ntiles;   // output tiles
+  int nkt;      // k-tiles per work item (>= 2): all of k, or one of `splits` equal parts
+  int ntiles;   // work items = output tiles * splits (item w: split w / nout, output tile w % nout)
+  int nout;     // output tiles
+  int splits;
+  FastDiv d_nout;
   int nwg;      // workgroups launched (a multiple of 8 when rect)
   int p_fast;   // the fast-walking operand is P
   int nfast;    // tiles of that operand
@@ -70,9 +80,27 @@ struct EpiStoreBf16 {
 #ifdef PP_DBG
 __device__ unsigned long long pp_dbg[256 * 4];
 #endif
-// ES: element size (2: bf16, 1: OCP fp8 with FMTP / FMTQ = 0 e4m3, 1 e5m2 per side)
-template <int ES, int FMTP, int FMTQ, class Epi>
+typedef short tfb_s16x8 __attribute__((ext_vector_type(8)));
+template <int OFF>
+__device__ __forceinline__ tfb_s16x4 tfb_lds_read_tr64(uint32_t addr) {
+  tfb_s16x4 v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+
+// An epilogue with the static member kSplitF32 receives the raw fp32 accumulators, operator()(p, q, v[8], split): the
+// partial tile of a k-split.
+template <class T, class = void>
+struct has_split_f32 : std::false_type {};
+template <class T>
+struct has_split_f32<T, std::void_t<decltype(T::kSplitF32)>> : std::true_type {};
+
+// ES: element size (2: bf16, 1: OCP fp8 with FMTP / FMTQ = 0 e4m3, 1 e5m2 per side); LAYP / LAYQ: TFB_K_CONTIG or (bf16
+// only) TFB_K_STRIDED
+template <int ES, int FMTP, int FMTQ, int LAYP, int LAYQ, class Epi>
 __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
+  static_assert(ES == 2 || (LAYP == TFB_K_CONTIG && LAYQ == TFB_K_CONTIG), "k-strided operands are bf16");
+  constexpr bool kF32 = has_split_f32<Epi>::value;
 #ifdef PP_DBG
   const unsigned long long c_start = __builtin_readcyclecounter();
   unsigned long long c_epi = 0, c_loop = 0;
@@ -87,8 +115,47 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
   const int nkt = a.nkt;
   uint8_t* stg = stg_all + wave * 4096;
 
-  // work item -> output tile origin (rows of P, rows of Q)
-  auto tile_of = [&](int w, long& p0, long& q0) {
+  // ---- operand loads. A quarter is 16 instructions of 1 KB, two per wavefront (g = wave and wave + 8):
+  //   k-contiguous: instruction g = rows 8 g .. 8 g + 7 x 128 bytes of k, lane l -> row l / 8, chunk (l % 8) ^ swizzle;
+  //   k-strided:    instruction g = k-rows 4 g .. 4 g + 3 x 128 rows (256 bytes), lane l -> k-row l / 16, chunk (l % 16) ^ 4 (k & 3).
+  // Per operand: v = the lane's byte offset, istep = from instruction g to g + 8, hstep = from half 0 to half 1,
+  // kstep = from one k-tile to the next, and the byte origin of output tile row-block r0.
+  struct Side {
+    const uint8_t* base;  // operand base + this wavefront's first instruction
+    uint32_t v;
+    long istep, hstep, kstep, tstep;  // tstep: bytes per row of the output tile origin
+  };
+  auto make_side = [&](const GemmOperand& o, int lay) {
+    Side sd;
+    if (lay == TFB_K_CONTIG) {
+      const int lrow = lane >> 3;
+      const int dch = (lane & 7) ^ tfb_kc_swz(lrow + 8 * wave);
+      sd.base = o.base + 8L * wave * o.ld;
+      sd.v = (uint32_t)(lrow * o.ld + dch * 16);
+      sd.istep = 64 * o.ld;
+      sd.hstep = 128 * o.ld;
+      sd.kstep = 128;
+      sd.tstep = o.ld;
+    } else {
+      const int kl = lane >> 4, slot = lane & 15;
+      sd.base = o.base + 4L * wave * o.ld;
+      sd.v = (uint32_t)(kl * o.ld + ((slot ^ (4 * kl)) << 4));
+      sd.istep = 32 * o.ld;
+      sd.hstep = 256;
+      sd.kstep = 64 * o.ld;
+      sd.tstep = 2;
+    }
+    return sd;
+  };
+  const Side sp = make_side(a.P, LAYP), sq = make_side(a.Q, LAYQ);
+
+  // work item -> operand addresses of its first k-tile (P side, Q side), output tile origin and split
+  auto tile_of = [&](int w, long& p0, long& q0, int& split) {
+    split = 0;
+    if (a.splits > 1) {
+      split = fastdiv(w, a.d_nout);
+      w -= split * a.nout;
+    }
     int fast, slow;
     if (a.rect) {
       const int x = w & 7, j = w >> 3;
@@ -106,23 +173,16 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
     p0 = (long)(a.p_fast ? fast : slow) * 256;
     q0 = (long)(a.p_fast ? slow : fast) * 256;
   };
+  auto origin = [&](const Side& sd, long r0, int split) { return sd.base + r0 * sd.tstep + (long)split * nkt * sd.kstep; };
 
-  // ---- operand loads: a quarter = 16 instructions of 8 rows x 128 B; this wavefront issues rows 8 wave + {0, 64} + lane / 8
-  const int lrow = lane >> 3;
-  const int dch = (lane & 7) ^ tfb_kc_swz(lrow + 8 * wave);
-  const uint32_t vp = (uint32_t)(lrow * a.P.ld + dch * 16), vq = (uint32_t)(lrow * a.Q.ld + dch * 16);
-  const long p64 = 64 * a.P.ld, q64 = 64 * a.Q.ld;
-  const uint8_t* bp = a.P.base + 8L * wave * a.P.ld;
-  const uint8_t* bq = a.Q.base + 8L * wave * a.Q.ld;
-  // quarter (X: 0 P, 1 Q; half h) of stage S <- 128 bytes of k at g (the operand's row-0 address of the tile + k offset)
+  // quarter (X: 0 P, 1 Q; half h) of stage S <- the k-tile at g (the side's address of that k-tile of the output tile)
   auto dma = [&](int S, int X, int h, const uint8_t* g) {
-    const long r64 = X ? q64 : p64;
-    const uint32_t v = X ? vq : vp;
+    const Side& sd = X ? sq : sp;
     uint8_t* d = lds + S * 65536 + X * 32768 + h * 16384 + wave * 1024;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
-      __builtin_amdgcn_global_load_lds((tfb_glb_void_t*)(g + (2 * h + i) * r64 + (size_t)v), (tfb_lds_void_t*)(d + i * 8192),
-                                       16, 0, 0);
+      __builtin_amdgcn_global_load_lds((tfb_glb_void_t*)(g + h * sd.hstep + i * sd.istep + (size_t)sd.v),
+                                       (tfb_lds_void_t*)(d + i * 8192), 16, 0, 0);
   };
 
   // ---- fragment addresses (stage 0; the stage bit is toggled after every k-tile)
@@ -130,31 +190,71 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
   {
     const uint32_t lbase = (uint32_t)(size_t)(tfb_lds_u8*)lds;
     const int rp = wr * 64 + lr, rq = wc * 32 + lr;
-    // bf16: k-step s (16 k) of a row is chunk 2 s + lh; fp8: k-step s (64 k) is chunks 4 s + 2 lh, + 1: entry 2 s + u
+    // k-contiguous, one address per k-step. bf16: k-step s (16 k) of a row is chunk 2 s + lh; fp8: k-step s (64 k) is
+    // chunks 4 s + 2 lh, + 1: entry 2 s + u
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int c = ES == 2 ? 2 * s + lh : 4 * (s >> 1) + 2 * lh + (s & 1);
       ap[s] = lbase + rp * 128 + (((c ^ tfb_kc_swz(rp)) & 7) << 4);
       aq[s] = lbase + 32768 + rq * 128 + (((c ^ tfb_kc_swz(rq)) & 7) << 4);
     }
+    // k-strided: 16-lane group g4 reads rows 16 (g4 & 1) .. + 15 of an MFMA tile, k-group g4 >> 1; lane j of the group
+    // points at k-row j / 4 (of four consecutive k), rows 4 (j % 4) .. + 3. One address per 32-row tile (ap[0], ap[1]:
+    // the second tile's chunk index differs in bit 2, which the swizzle also touches, so it is not an immediate offset);
+    // k-step s is 16 k-rows further (an immediate), the fragment's upper four k another 4 k-rows.
+    const int g4 = lane >> 4, j = lane & 15, kq = j >> 2;
+    auto tr_addr = [&](int row0) {
+      const int p = row0 + 16 * (g4 & 1) + 4 * (j & 3);
+      return (uint32_t)((8 * (g4 >> 1) + kq) * 256 + ((((p >> 3) ^ (4 * kq)) << 4) | ((p & 4) << 1)));
+    };
+    if (LAYP == TFB_K_STRIDED) {
+      ap[0] = lbase + tr_addr(wr * 64);
+      ap[1] = lbase + tr_addr(wr * 64 + 32);
+    }
+    if (LAYQ == TFB_K_STRIDED) aq[0] = lbase + 32768 + tr_addr(wc * 32);
   }
+  constexpr int NAP = LAYP == TFB_K_STRIDED ? 2 : 4, NAQ = LAYQ == TFB_K_STRIDED ? 1 : 4;  // addresses in use
 
   f32x16 acc[2][2][2];  // [P half][i][Q half]
   // fragments: bf16 four k-steps of 16 (one 128-bit read each), fp8 two k-steps of 64 (two 128-bit reads each)
   typedef std::conditional_t<ES == 2, bf16x8, i32x4> r128_t;
   r128_t fa[2][4], fb0[4], fb1[4];
-  auto readA = [&](auto H) {
+  auto tr_frag = [&](auto OFF, uint32_t addr) {
+    constexpr int off = decltype(OFF)::value;
+    const tfb_s16x4 lo = tfb_lds_read_tr64<off>(addr), hi = tfb_lds_read_tr64<off + 1024>(addr);
+    const tfb_s16x8 v = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    return __builtin_bit_cast(r128_t, v);
+  };
+  auto readA = [&](auto H) __attribute__((always_inline)) {
     constexpr int h = decltype(H)::value;
+    if constexpr (LAYP == TFB_K_CONTIG) {
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      fa[0][s] = tfb_lds_read128<h * 16384, r128_t>(ap[s]);
-      fa[1][s] = tfb_lds_read128<h * 16384 + 4096, r128_t>(ap[s]);
+      for (int s = 0; s < 4; ++s) {
+        fa[0][s] = tfb_lds_read128<h * 16384, r128_t>(ap[s]);
+        fa[1][s] = tfb_lds_read128<h * 16384 + 4096, r128_t>(ap[s]);
+      }
+    } else {
+      fa[0][0] = tr_frag(std::integral_constant<int, h * 16384>{}, ap[0]);
+      fa[1][0] = tr_frag(std::integral_constant<int, h * 16384>{}, ap[1]);
+      fa[0][1] = tr_frag(std::integral_constant<int, h * 16384 + 4096>{}, ap[0]);
+      fa[1][1] = tr_frag(std::integral_constant<int, h * 16384 + 4096>{}, ap[1]);
+      fa[0][2] = tr_frag(std::integral_constant<int, h * 16384 + 8192>{}, ap[0]);
+      fa[1][2] = tr_frag(std::integral_constant<int, h * 16384 + 8192>{}, ap[1]);
+      fa[0][3] = tr_frag(std::integral_constant<int, h * 16384 + 12288>{}, ap[0]);
+      fa[1][3] = tr_frag(std::integral_constant<int, h * 16384 + 12288>{}, ap[1]);
     }
   };
-  auto readB = [&](auto H, r128_t(&fb)[4]) {
+  auto readB = [&](auto H, r128_t(&fb)[4]) __attribute__((always_inline)) {
     constexpr int h = decltype(H)::value;
+    if constexpr (LAYQ == TFB_K_CONTIG) {
 #pragma unroll
-    for (int s = 0; s < 4; ++s) fb[s] = tfb_lds_read128<h * 16384, r128_t>(aq[s]);
+      for (int s = 0; s < 4; ++s) fb[s] = tfb_lds_read128<h * 16384, r128_t>(aq[s]);
+    } else {
+      fb[0] = tr_frag(std::integral_constant<int, h * 16384>{}, aq[0]);
+      fb[1] = tr_frag(std::integral_constant<int, h * 16384 + 4096>{}, aq[0]);
+      fb[2] = tr_frag(std::integral_constant<int, h * 16384 + 8192>{}, aq[0]);
+      fb[3] = tr_frag(std::integral_constant<int, h * 16384 + 12288>{}, aq[0]);
+    }
   };
   // the fragments pass through the wait as in/out operands, so that no MFMA that reads them is scheduled ahead of it
   auto waitA = [&]() {
@@ -208,22 +308,20 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
   const Epi epi = epi_prepare(epi_in);
   int w = blockIdx.x;
   if (w >= a.ntiles) return;  // (whole workgroup)
-#ifdef PP_STAG
-  for (int i = 0; i < (int)((blockIdx.x >> 3) & 3) * PP_STAG; ++i) __builtin_amdgcn_s_sleep(32);
-#endif
   long p0, q0;
-  tile_of(w, p0, q0);
-  const uint8_t* gp = bp + p0 * a.P.ld;  // current tile
-  const uint8_t* gq = bq + q0 * a.Q.ld;
+  int split;
+  tile_of(w, p0, q0, split);
+  const uint8_t* gp = origin(sp, p0, split);  // current work item: the sides' addresses of its first k-tile
+  const uint8_t* gq = origin(sq, q0, split);
 
   // ---- prologue: all of k-tile 0 into stage 0, three quarters of k-tile 1 into stage 1
   dma(0, 1, 0, gq);
   dma(0, 0, 0, gp);
   dma(0, 1, 1, gq);
   dma(0, 0, 1, gp);
-  dma(1, 0, 0, gp + 128);
-  dma(1, 1, 0, gq + 128);
-  dma(1, 1, 1, gq + 128);
+  dma(1, 0, 0, gp + sp.kstep);
+  dma(1, 1, 0, gq + sq.kstep);
+  dma(1, 1, 1, gq + sq.kstep);
   asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
   TFB_SBAR();               // k-tile 0 is there for everybody
   if (wr == 1) TFB_SBAR();  // group 1 runs one cluster behind from here on
@@ -251,9 +349,11 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) {
         const f32x16& c = acc[hp][i][hq];
-        u32x2 v = {pack2bf(epi.pre(c[4 * jj + 0]), epi.pre(c[4 * jj + 1])),
-                   pack2bf(epi.pre(c[4 * jj + 2]), epi.pre(c[4 * jj + 3]))};
-        *(u32x2*)(stg + lr * 128 + (((4 * i + jj) ^ ((lr >> 1) & 7)) << 4) + 8 * lh) = v;
+        if constexpr (!kF32) {
+          u32x2 v = {pack2bf(epi.pre(c[4 * jj + 0]), epi.pre(c[4 * jj + 1])),
+                     pack2bf(epi.pre(c[4 * jj + 2]), epi.pre(c[4 * jj + 3]))};
+          *(u32x2*)(stg + lr * 128 + (((4 * i + jj) ^ ((lr >> 1) & 7)) << 4) + 8 * lh) = v;
+        }
       }
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -270,24 +370,57 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
         else epi.chunk(p, q, v, vp);
       } else if constexpr (kPrefetch) {
         epi.chunk(p, q, v, pre[k]);
-      } else {
+      } else if constexpr (!kF32) {
         epi.chunk(p, q, v);
       }
     }
     __builtin_amdgcn_wave_barrier();
   };
 
+  // The same for the partial tile of a k-split (epilogues with kSplitF32): sixteen output rows at a time pass through the
+  // 4 KB as fp32 (row = 256 bytes, 16-byte chunk c at slot c ^ row), and a lane finishes 8 consecutive fp32 outputs.
+  auto store_block_f32 = [&](auto HP, auto HQ, long tp0, long tq0, int sp_) __attribute__((always_inline)) {
+    constexpr int hp = decltype(HP)::value, hq = decltype(HQ)::value;
+    const int pb = (int)tp0 + hp * 128 + wr * 64, qb = (int)tq0 + hq * 128 + wc * 32;
+    const int ch = lane & 7, r8 = lane >> 3;
+#pragma unroll
+    for (int qh = 0; qh < 2; ++qh) {
+      if ((lr >> 4) == qh) {
+        const int row = lr & 15;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj) {
+            const f32x16& c = acc[hp][i][hq];
+            const f32x4 v = {c[4 * jj + 0], c[4 * jj + 1], c[4 * jj + 2], c[4 * jj + 3]};
+            *(f32x4*)(stg + row * 256 + (((8 * i + 2 * jj + lh) ^ row) << 4)) = v;
+          }
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int row = r8 + 8 * k;
+        const f32x4 lo = *(const f32x4*)(stg + row * 256 + (((2 * ch) ^ row) << 4));
+        const f32x4 hi = *(const f32x4*)(stg + row * 256 + (((2 * ch + 1) ^ row) << 4));
+        const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        if constexpr (kF32) epi(pb + 8 * ch, qb + 16 * qh + row, v, sp_);
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  };
+
   int S = 0;
   bool have_prev = false;  // the previous tile's accumulators are still to be stored
   long pp0 = 0, pq0 = 0;   // its origin
   for (;;) {
-    // the workgroup's next tile (its first k-tiles are requested by this tile's last iterations); past the end: this tile
-    // again (loads nobody reads, from valid memory)
+    // the workgroup's next work item (its first k-tiles are requested by this one's last iterations); past the end: this
+    // one again (loads nobody reads, from valid memory)
     const int wn = w + a.nwg;
     long pn = p0, qn = q0;
-    if (wn < a.ntiles) tile_of(wn, pn, qn);
-    const uint8_t* gpn = bp + pn * a.P.ld;
-    const uint8_t* gqn = bq + qn * a.Q.ld;
+    int splitn = split;
+    if (wn < a.ntiles) tile_of(wn, pn, qn, splitn);
+    const uint8_t* gpn = origin(sp, pn, splitn);
+    const uint8_t* gqn = origin(sq, qn, splitn);
 
     // One k-tile. In a tile's first iteration the MFMAs start from zero, and each accumulator block of the PREVIOUS tile is
     // stored in the memory cluster in front of the MFMA cluster that overwrites it: the stores of one group (4 KB per
@@ -296,15 +429,17 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
       constexpr bool first = decltype(FIRST)::value;
       // k positions one and two ahead in the workgroup's stream of k-tiles
       const bool in1 = kt + 1 < nkt, in2 = kt + 2 < nkt;
-      const long k1 = (long)(in1 ? kt + 1 : 0) * 128, k2 = (long)(in2 ? kt + 2 : kt + 2 - nkt) * 128;
-      const uint8_t* gp1 = (in1 ? gp : gpn) + k1;
-      const uint8_t* gp2 = (in2 ? gp : gpn) + k2;
-      const uint8_t* gq2 = (in2 ? gq : gqn) + k2;
+      const long k1 = in1 ? kt + 1 : 0, k2 = in2 ? kt + 2 : kt + 2 - nkt;
+      const uint8_t* gp1 = (in1 ? gp : gpn) + k1 * sp.kstep;
+      const uint8_t* gp2 = (in2 ? gp : gpn) + k2 * sp.kstep;
+      const uint8_t* gq2 = (in2 ? gq : gqn) + k2 * sq.kstep;
       // c0
       readB(H0{}, fb0);
       readA(H0{});
       dma(S ^ 1, 0, 1, gp1);
-      if (first && have_prev) store_block(H0{}, H0{}, pp0, pq0);
+      if constexpr (!kF32) {
+        if (first && have_prev) store_block(H0{}, H0{}, pp0, pq0);
+      }
       TFB_SBAR();
       // c1
       waitB(fb0);
@@ -314,7 +449,9 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
       // c2
       readB(H1{}, fb1);
       dma(S, 0, 0, gp2);
-      if (first && have_prev) store_block(H0{}, H1{}, pp0, pq0);
+      if constexpr (!kF32) {
+        if (first && have_prev) store_block(H0{}, H1{}, pp0, pq0);
+      }
       TFB_SBAR();
       // c3
       waitB(fb1);
@@ -323,7 +460,9 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
       // c4
       readA(H1{});
       dma(S, 1, 0, gq2);
-      if (first && have_prev) store_block(H1{}, H0{}, pp0, pq0);
+      if constexpr (!kF32) {
+        if (first && have_prev) store_block(H1{}, H0{}, pp0, pq0);
+      }
       TFB_SBAR();
       // c5
       waitA();
@@ -334,8 +473,8 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
       // Completion is reported in issue order, stores included. Everything up to the quarter requested in c0 has to be
       // there: all but the three quarters requested since (6 instructions), and in a first iteration with stores all but
       // those and the 16 stores (c0's four were issued behind its loads).
-      if (first && have_prev) {
-        store_block(H1{}, H1{}, pp0, pq0);
+      if (!kF32 && first && have_prev) {
+        if constexpr (!kF32) store_block(H1{}, H1{}, pp0, pq0);
         asm volatile("s_waitcnt vmcnt(22)" ::: "memory");
       } else {
         asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
@@ -346,10 +485,9 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
       TFB_SBAR();
       S ^= 1;
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        ap[s] ^= 0x10000u;
-        aq[s] ^= 0x10000u;
-      }
+      for (int s = 0; s < NAP; ++s) ap[s] ^= 0x10000u;
+#pragma unroll
+      for (int s = 0; s < NAQ; ++s) aq[s] ^= 0x10000u;
     };
 #ifdef PP_DBG
     const unsigned long long c_l0 = __builtin_readcyclecounter();
@@ -364,21 +502,36 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
     c_loop += __builtin_readcyclecounter() - c_e0;
     ++n_tiles;
 #endif
-    have_prev = true;
-    pp0 = p0;
-    pq0 = q0;
+    if constexpr (kF32) {
+      // a k-split's partial tile: stored here, both groups together (a work item is hundreds of k-tiles long)
+      if (wr == 0) TFB_SBAR();  // group 0 waits for group 1's last cluster
+      store_block_f32(H0{}, H0{}, p0, q0, split);
+      store_block_f32(H0{}, H1{}, p0, q0, split);
+      store_block_f32(H1{}, H0{}, p0, q0, split);
+      store_block_f32(H1{}, H1{}, p0, q0, split);
+    } else {
+      have_prev = true;
+      pp0 = p0;
+      pq0 = q0;
+    }
     w = wn;
     if (w >= a.ntiles) break;
     p0 = pn;
     q0 = qn;
+    split = splitn;
     gp = gpn;
     gq = gqn;
+    if constexpr (kF32) {
+      if (wr == 1) TFB_SBAR();  // group 1 falls one cluster behind again
+    }
   }
-  // the last tile's accumulators
-  store_block(H0{}, H0{}, pp0, pq0);
-  store_block(H0{}, H1{}, pp0, pq0);
-  store_block(H1{}, H0{}, pp0, pq0);
-  store_block(H1{}, H1{}, pp0, pq0);
+  if constexpr (!kF32) {
+    // the last tile's accumulators
+    store_block(H0{}, H0{}, pp0, pq0);
+    store_block(H0{}, H1{}, pp0, pq0);
+    store_block(H1{}, H0{}, pp0, pq0);
+    store_block(H1{}, H1{}, pp0, pq0);
+  }
 #ifdef PP_DBG
   if (tid == 0 && blockIdx.x < 256) {
     pp_dbg[blockIdx.x * 4 + 0] = __builtin_readcyclecounter() - c_start;
@@ -405,30 +558,38 @@ static inline bool gemm_pp_applies(long np, long nq, long kbytes) {
   return TFB_PP == 2 || kbytes / 128 >= 16 || tiles >= 4096;
 }
 
-template <int ES, int FMTP, int FMTQ, class Epi>
-static int gemm_pp_launch(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes, Epi epi, hipStream_t stream) {
-  if (np <= 0 || nq <= 0 || kbytes < 256 || np % 256 || nq % 256 || kbytes % 128) return TFB_ERR_SHAPE;
+// np, nq multiples of 256; kbytes = the contraction in bytes of a k-contiguous row (elements * ES), a multiple of
+// 128 * splits with at least two k-tiles per split. With splits > 1 the epilogue is one with kSplitF32 (EpiSplit).
+template <int ES, int FMTP, int FMTQ, int LAYP, int LAYQ, class Epi>
+static int gemm_pp_launch_lay(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes, int splits, Epi epi, hipStream_t stream) {
+  if (np <= 0 || nq <= 0 || splits <= 0 || np % 256 || nq % 256 || kbytes % (128L * splits) || kbytes / 128 / splits < 2)
+    return TFB_ERR_SHAPE;
   if (P.ld <= 0 || Q.ld <= 0 || P.ld > (1L << 28) || Q.ld > (1L << 28)) return TFB_ERR_SHAPE;
   if (((uintptr_t)P.base | (uintptr_t)Q.base | (uintptr_t)P.ld | (uintptr_t)Q.ld) & 15) return TFB_ERR_ARG;
+  if ((splits > 1) != has_split_f32<Epi>::value) return TFB_ERR_ARG;
   PpArgs a = {};
   a.P = P;
   a.Q = Q;
-  a.nkt = (int)(kbytes / 128);
+  a.splits = splits;
+  a.nkt = (int)(kbytes / 128 / splits);
   const int ntp = np / 256, ntq = nq / 256;
-  if ((long)ntp * ntq >= (1L << 30)) return TFB_ERR_SHAPE;
-  a.ntiles = ntp * ntq;
+  if ((long)ntp * ntq * splits >= (1L << 30)) return TFB_ERR_SHAPE;
+  a.nout = ntp * ntq;
+  a.ntiles = a.nout * splits;
   const int cus = tfb_resident_slots(1);
   a.p_fast = np <= nq;
   a.nfast = a.p_fast ? ntp : ntq;
   const int nslow = a.p_fast ? ntq : ntp;
-  a.rect = (nslow % 8 == 0) && a.ntiles >= 8;
+  a.rect = (nslow % 8 == 0) && a.nout >= 8;
   a.nwg = a.ntiles < cus ? a.ntiles : cus;
   if (a.rect) a.nwg &= ~7;
+  if (a.nwg <= 0) return TFB_ERR_SHAPE;
   a.R = a.rect ? nslow / 8 : 1;
-  // panel width: GW * R ~ the 32 workgroups an XCD runs together, at least 1 and at most all columns
+  // panel width: GW * R ~ the 32 workgroups an XCD runs together; a narrow fast operand (<= 4 tiles) is walked whole, so
+  // that the tiles sharing a row block of the slow operand run together
   int gw = a.R >= 32 ? 1 : (32 + a.R - 1) / a.R;
   if (a.R > 8 && a.R < 32) gw = 32 / a.R > 0 ? 32 / a.R : 1;
-  if (gw > a.nfast) gw = a.nfast;
+  if (gw > a.nfast || a.nfast <= 4) gw = a.nfast;
   a.GW = gw;
   a.panel = a.GW * a.R;
   a.gw_last = a.nfast % a.GW ? a.nfast % a.GW : a.GW;
@@ -436,7 +597,15 @@ static int gemm_pp_launch(GemmOperand P, GemmOperand Q, int np, int nq, long kby
   a.d_panel = fastdiv_make(a.panel);
   a.d_gw = fastdiv_make(a.GW);
   a.d_gw_last = fastdiv_make(a.gw_last);
-  hipLaunchKernelGGL((gemm_pp_kernel<ES, FMTP, FMTQ, Epi>), dim3(a.nwg), dim3(512), 0, stream, a, epi);
+  a.d_nout = fastdiv_make(a.nout);
+  hipLaunchKernelGGL((gemm_pp_kernel<ES, FMTP, FMTQ, LAYP, LAYQ, Epi>), dim3(a.nwg), dim3(512), 0, stream, a, epi);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
+}
+
+// both operands k-contiguous, no k-split
+template <int ES, int FMTP, int FMTQ, class Epi>
+static int gemm_pp_launch(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes, Epi epi, hipStream_t stream) {
+  if (kbytes < 256) return TFB_ERR_SHAPE;
+  return gemm_pp_launch_lay<ES, FMTP, FMTQ, TFB_K_CONTIG, TFB_K_CONTIG>(P, Q, np, nq, kbytes, 1, epi, stream);
 }
