@@ -16,13 +16,17 @@ namespace {
 
 constexpr int ROWS_PER_BLOCK = 4;  // one wavefront per row, 4 wavefronts per workgroup
 
-template <int NCH>
+// A row is held by G lanes (a whole wavefront, or half of one: two rows per wavefront when the row length is a multiple
+// of 256 up to 1024, so that every lane has work in every chunk and a wavefront keeps two rows' loads in flight), each
+// lane NCH chunks of 8 elements: chunk i of lane l covers columns 8 (l + G i) .. + 7. `lane` below is the lane's index
+// inside its group.
+template <int NCH, int G = 64>
 struct Row {
   float v[NCH][8];
   __device__ __forceinline__ void load(const bf16_t* p, int C, int lane) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      int c = (lane + 64 * i) * 8;
+      int c = (lane + G * i) * 8;
       if (c < C) {
         u32x4 u = *(const u32x4*)(p + c);
 #pragma unroll
@@ -39,7 +43,7 @@ struct Row {
   __device__ __forceinline__ void store(bf16_t* p, int C, int lane) const {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      int c = (lane + 64 * i) * 8;
+      int c = (lane + G * i) * 8;
       if (c < C) {
         u32x4 u;
 #pragma unroll
@@ -65,17 +69,17 @@ struct Row {
 // A row as loaded (bf16 pairs in 32-bit words), to be widened later: the kernels below request the NEXT row of a
 // wavefront before they store the current one. A wait for loaded data also waits for every older memory operation, stores
 // included (one counter orders both), so a loop that loads after its stores pays a full store round trip per row.
-template <int NCH>
+template <int NCH, int G = 64>
 struct RawRow {
   u32x4 u[NCH];
   __device__ __forceinline__ void load(const bf16_t* p, int C, int lane) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int c = (lane + 64 * i) * 8;
+      const int c = (lane + G * i) * 8;
       u[i] = c < C ? *(const u32x4*)(p + c) : u32x4{0u, 0u, 0u, 0u};
     }
   }
-  __device__ __forceinline__ void widen(Row<NCH>& r) const {
+  __device__ __forceinline__ void widen(Row<NCH, G>& r) const {
 #pragma unroll
     for (int i = 0; i < NCH; ++i)
 #pragma unroll
@@ -86,36 +90,44 @@ struct RawRow {
   }
 };
 
-template <int NCH>
-__device__ __forceinline__ float row_dot(const Row<NCH>& a, const Row<NCH>& b) {
+// sum / max over the G lanes that hold a row (the butterfly stays inside the group)
+template <int G>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int o = G / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+template <int NCH, int G>
+__device__ __forceinline__ float row_dot(const Row<NCH, G>& a, const Row<NCH, G>& b) {
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < NCH; ++i)
 #pragma unroll
     for (int k = 0; k < 8; ++k) s += a.v[i][k] * b.v[i][k];
-  return wave_sum(s);
+  return group_sum<G>(s);
 }
 
 // ------------------------------------------------------------------------------------------
-template <int NCH>
+template <int NCH, int G>
 __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ res,
                                                          const bf16_t* __restrict__ w, bf16_t* __restrict__ s_out,
                                                          bf16_t* __restrict__ y, float* __restrict__ inv, long nrows,
                                                          int C, float eps, uint8_t* __restrict__ y8, float y8_scale) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  Row<NCH> wr;
+  constexpr int RPW = 64 / G;  // rows per wavefront
+  const int lane = threadIdx.x & (G - 1), sub = (threadIdx.x & 63) / G, wave = threadIdx.x >> 6;
+  Row<NCH, G> wr;
   if (w) wr.load(w, C, lane);
-  const long step = (long)gridDim.x * ROWS_PER_BLOCK;
-  long row = (long)blockIdx.x * ROWS_PER_BLOCK + wave;
-  RawRow<NCH> xa, xr;
+  const long step = (long)gridDim.x * ROWS_PER_BLOCK * RPW;
+  long row = ((long)blockIdx.x * ROWS_PER_BLOCK + wave) * RPW + sub;
+  RawRow<NCH, G> xa, xr;
   if (row < nrows) {
     xa.load(x + row * C, C, lane);
     if (res) xr.load(res + row * C, C, lane);
   }
   for (; row < nrows; row += step) {
-    Row<NCH> a;
+    Row<NCH, G> a;
     xa.widen(a);
-    Row<NCH> r;
+    Row<NCH, G> r;
     if (res) xr.widen(r);
     if (row + step < nrows) {  // the next row's loads go out before this row's stores
       xa.load(x + (row + step) * C, C, lane);
@@ -139,7 +151,7 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16_t* __restri
       a.round();
 #pragma unroll
       for (int i = 0; i < NCH; ++i) {
-        const int c = (lane + 64 * i) * 8;
+        const int c = (lane + G * i) * 8;
         if (c < C) {
           u32x2 o;
           o.x = cvt4_fp8<TFB_FMT_E4M3>(a.v[i][0] * y8_scale, a.v[i][1] * y8_scale, a.v[i][2] * y8_scale, a.v[i][3] * y8_scale);
@@ -154,22 +166,23 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16_t* __restri
 
 // dx = gs + J^T(gy): J^T(gy) = inv * (gh - s * (gh . s) * inv^2 / C), gh = gy * w.
 // dw partial [gridDim.x][C] = sum over the workgroup's rows of gy * s * inv.
-template <int NCH>
+template <int NCH, int G>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16_t* __restrict__ gy, const bf16_t* __restrict__ gs,
                                                          const bf16_t* __restrict__ s, const bf16_t* __restrict__ w,
                                                          const float* __restrict__ inv, bf16_t* __restrict__ dx,
                                                          float* __restrict__ dw_part, float* __restrict__ amax_part, long nrows,
                                                          int C) {
-  __shared__ float red[ROWS_PER_BLOCK][NCH * 512];
+  constexpr int RPW = 64 / G, RPB = ROWS_PER_BLOCK * RPW;  // rows per wavefront, per workgroup
+  __shared__ float red[RPB][NCH * G * 8];
   __shared__ float amred[ROWS_PER_BLOCK];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & (G - 1), sub = (threadIdx.x & 63) / G, wave = threadIdx.x >> 6;
   float am = 0.f;   // amax of the rounded dx this wavefront wrote (amax_part: one value per workgroup)
-  Row<NCH> wr, dwacc;
+  Row<NCH, G> wr, dwacc;
   if (w) wr.load(w, C, lane);
   dwacc.zero();
-  const long step = (long)gridDim.x * ROWS_PER_BLOCK;
-  long row = (long)blockIdx.x * ROWS_PER_BLOCK + wave;
-  RawRow<NCH> xg, xa, xr;
+  const long step = (long)gridDim.x * RPB;
+  long row = ((long)blockIdx.x * ROWS_PER_BLOCK + wave) * RPW + sub;
+  RawRow<NCH, G> xg, xa, xr;
   float rs_next = 0.f;
   if (row < nrows) {
     xg.load(gy + row * C, C, lane);
@@ -178,7 +191,7 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16_t* __restri
     rs_next = inv[row];
   }
   for (; row < nrows; row += step) {
-    Row<NCH> g, a, r;
+    Row<NCH, G> g, a, r;
     xg.widen(g);
     xa.widen(a);
     if (gs) xr.widen(r);
@@ -214,7 +227,7 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16_t* __restri
       g.round();
 #pragma unroll
       for (int i = 0; i < NCH; ++i)
-        if ((lane + 64 * i) * 8 < C) {
+        if ((lane + G * i) * 8 < C) {
 #pragma unroll
           for (int k = 0; k < 8; ++k) am = fmaxf(am, fabsf(g.v[i][k]));
         }
@@ -223,7 +236,7 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16_t* __restri
   }
   if (amax_part) {
     am = wave_max(am);
-    if (lane == 0) amred[wave] = am;
+    if ((threadIdx.x & 63) == 0) amred[wave] = am;
     __syncthreads();
     if (threadIdx.x == 0) {
       float t = amred[0];
@@ -236,12 +249,12 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16_t* __restri
 #pragma unroll
     for (int i = 0; i < NCH; ++i)
 #pragma unroll
-      for (int k = 0; k < 8; ++k) red[wave][(lane + 64 * i) * 8 + k] = dwacc.v[i][k];
+      for (int k = 0; k < 8; ++k) red[wave * RPW + sub][(lane + G * i) * 8 + k] = dwacc.v[i][k];
     __syncthreads();
     for (int c = threadIdx.x; c < C; c += 256) {
       float t = 0.f;
 #pragma unroll
-      for (int r = 0; r < ROWS_PER_BLOCK; ++r) t += red[r][c];
+      for (int r = 0; r < RPB; ++r) t += red[r][c];
       dw_part[(long)blockIdx.x * C + c] = t;
     }
   }
@@ -400,6 +413,21 @@ inline int grid_for(long nrows, int cap) {
     else if ((C) <= 2048) { CALL(4); }   \
     else { CALL(8); }                    \
   } while (0)
+// the RMSNorm pair: rows of 256, 512, 768 or 1024 elements on half a wavefront each (two rows per wavefront), else a
+// wavefront per row
+#define DISPATCH_ROWS(C, CALL)                                   \
+  do {                                                           \
+    if ((C) % 256 == 0 && (C) <= 1024) {                         \
+      if ((C) == 256) { CALL(1, 32); }                           \
+      else if ((C) == 512) { CALL(2, 32); }                      \
+      else if ((C) == 768) { CALL(3, 32); }                      \
+      else { CALL(4, 32); }                                      \
+    } else if ((C) <= 512) { CALL(1, 64); }                      \
+    else if ((C) <= 1024) { CALL(2, 64); }                       \
+    else if ((C) <= 2048) { CALL(4, 64); }                       \
+    else { CALL(8, 64); }                                        \
+  } while (0)
+static inline int norm_rows_per_block(int C) { return (C % 256 == 0 && C <= 1024) ? 2 * ROWS_PER_BLOCK : ROWS_PER_BLOCK; }
 
 static bool norm_shape_ok(long nrows, int C) { return nrows > 0 && C > 0 && C % 8 == 0 && C <= 4096; }
 
@@ -412,12 +440,13 @@ static int rmsnorm_fwd_impl(const void* x, const void* res, const void* w, void*
   if (!x || (!y && !y8)) return TFB_ERR_ARG;   // y may be left out when only its fp8 cast is read (both MLP GEMM kinds in fp8)
   if (res && !s_out) return TFB_ERR_ARG;
   if (!norm_shape_ok(nrows, C)) return TFB_ERR_SHAPE;
-  int grid = grid_for(nrows, 8192);
-#define CALL(N)                                                                                                       \
-  hipLaunchKernelGGL(rmsnorm_fwd_kernel<N>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x,          \
+  const long rpb = norm_rows_per_block(C), nb = (nrows + rpb - 1) / rpb;
+  int grid = (int)(nb < 8192 ? nb : 8192);
+#define CALL(N, G)                                                                                                    \
+  hipLaunchKernelGGL((rmsnorm_fwd_kernel<N, G>), dim3(grid), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x,     \
                      (const bf16_t*)res, (const bf16_t*)w, (bf16_t*)s_out, (bf16_t*)y, (float*)inv, nrows, C, eps,    \
                      (uint8_t*)y8, y8_scale)
-  DISPATCH_NCH(C, CALL);
+  DISPATCH_ROWS(C, CALL);
 #undef CALL
   TFB_LAUNCH_CHECK();
   return TFB_OK;
@@ -438,12 +467,14 @@ static int rmsnorm_bwd_impl(const void* gy, const void* gs, const void* s, const
   if (!gy || !s || !inv || !dx) return TFB_ERR_ARG;
   if (w && !dw_part) return TFB_ERR_ARG;
   if (!norm_shape_ok(nrows, C)) return TFB_ERR_SHAPE;
+  // (the grid is tfb_norm_bwd_blocks(nrows) whatever the rows per workgroup: every partial row of dw_part / amax_part is
+  // written, by a workgroup without rows as zeros)
   int grid = grid_for(nrows, 1024);
-#define CALL(N)                                                                                                        \
-  hipLaunchKernelGGL(rmsnorm_bwd_kernel<N>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)gy,          \
+#define CALL(N, G)                                                                                                     \
+  hipLaunchKernelGGL((rmsnorm_bwd_kernel<N, G>), dim3(grid), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)gy,     \
                      (const bf16_t*)gs, (const bf16_t*)s, (const bf16_t*)w, (const float*)inv, (bf16_t*)dx,            \
                      (float*)dw_part, (float*)amax_part, nrows, C)
-  DISPATCH_NCH(C, CALL);
+  DISPATCH_ROWS(C, CALL);
 #undef CALL
   TFB_LAUNCH_CHECK();
   if (w && dw) {
