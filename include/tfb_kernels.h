@@ -492,6 +492,43 @@ long tfb_ns5_workspace_bytes(int K, int M, int N);
 int tfb_ns5(const void* g, const void* inv_d, const float* coeffs, void* y, void* v, int K, int M, int N, int wide,
             void* workspace, long workspace_bytes, void* stream);
 
+/* ---- dense bf16 fused MLP ---------------------------------------------------------------------------------------------
+ * x bf16 [M][d], w_fc bf16 [F][d], w_proj bf16 [d][F] (nn.Linear layouts) -> y bf16 [M][d] = bf16(h @ w_proj^T) with
+ * r = bf16(relu(x @ w_fc^T)) (bf16 [M][F], token-major, saved for the backward) and h = bf16(r r) (bf16 [M][F], the second
+ * GEMM's operand). M, d, F multiples of 128.
+ * Replaces _mlp_fwd_kernel(x2, w_fc, w_proj, tb) -> (y, rT) (round2/source/kernels/nki_mlp_fused.py:242; arithmetic
+ * emulate_forward :372); the reference saves r's transpose. */
+int tfb_mlp_fwd(const void* x, const void* w_fc, const void* w_proj, void* y, void* r, void* h, long M, int d, int F,
+                void* stream);
+/* dy bf16 [M][d], r as the forward left it -> dx bf16 [M][d], dpre bf16 [M][F] = bf16(((dy @ w_proj) 2) r) (one rounding),
+ * h bf16 [M][F] = bf16(r r) (optional, may be NULL): dpre and h are what the weight gradients contract (dpre^T x, dy^T h).
+ * Replaces _mlp_bwd_kernel(dy2, rT, w_fc, w_proj, tb, dw_mode) -> (dx, h, dpre) with dw_mode 0
+ * (round2/source/kernels/nki_mlp_fused.py:290; arithmetic emulate_backward :382, weight_grads :394). */
+int tfb_mlp_bwd(const void* dy, const void* r, const void* w_fc, const void* w_proj, void* dx, void* h, void* dpre, long M,
+                int d, int F, void* stream);
+
+/* ---- gradient norm ---------------------------------------------------------------------------------------------------
+ * out fp32 [4] = (sum of squares of g_bf16 [n_bf16], of g_f32 [n_f32], sqrt of their sum, min(clip / (norm + 1e-6), 1) or 1
+ * when clip <= 0), left on the device; either buffer may be absent (NULL, 0). scratch: fp32
+ * [tfb_gradnorm_scratch_floats()]. Two launches, sums in a fixed order.
+ * Replaces _gradnorm_kernel (round1/source/train.py:1480) and the norm / clip-factor arithmetic of reduce_fused (:1634). */
+long tfb_gradnorm_scratch_floats(void);
+int tfb_gradnorm(const void* g_bf16, long n_bf16, const void* g_f32, long n_f32, float clip, void* scratch, void* out,
+                 void* stream);
+
+/* ---- mixer tail ------------------------------------------------------------------------------------------------------
+ * x bf16 [nrows][C] (nrows = sequences of T tokens), lam a device fp32 scalar -> s1 = bf16(x + bf16(lam shift1(x))) where
+ * shift1 hands token t the row of token t - 1 of its sequence (zeros at t = 0), xn2 = RMSNorm(s1) without weight, inv fp32
+ * [nrows]. Replaces mix_tail's forward kernel _mix_fwd_kernel (round1/source/train.py:7097, wrapper :7308). */
+int tfb_mix_tail_fwd(const void* x, const void* lam, void* s1, void* xn2, void* inv, long nrows, int C, int T, float eps,
+                     void* stream);
+/* gy (gradient of xn2), ge (gradient of s1), either may be NULL -> gx bf16 [nrows][C] = bf16(g[t] + bf16(lam g[t + 1])) with
+ * g the tail norm's backward bf16(ge + inv (gy - s1 (gy . s1) inv^2 / C)) (g[t + 1] = 0 at a sequence's last token), and
+ * dlam fp32 [1] = the fp32 sum of the bf16 products bf16(g shift1(x)). part: fp32 [tfb_norm_bwd_blocks(nrows)] scratch.
+ * Replaces _mix_bwd_kernel (round1/source/train.py:7145). */
+int tfb_mix_tail_bwd(const void* s1, const void* gy, const void* ge, const void* inv, const void* x, const void* lam, void* gx,
+                     void* part, void* dlam, long nrows, int C, int T, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

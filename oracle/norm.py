@@ -107,3 +107,41 @@ def resmix_backward(g, x, x0, a, b):
     da = (g * x).float().sum()
     db = (g * x0).float().sum()
     return dx, dx0, da, db
+
+
+def shift1(x):
+    """[B, T, C]: token t reads token t - 1 of its sequence, token 0 zeros (round1/source/train.py:300)."""
+    return torch.cat([torch.zeros_like(x[:, :1]), x[:, :-1]], dim=1)
+
+
+def mix_tail(x, lam, eps=2.0 ** -23):
+    """(s1, xn2, inv) for x [B, T, C] bf16: s1 = bf16(x + bf16(lam shift1(x))), xn2 = RMSNorm(s1) without weight
+    (round1/source/train.py:7098 docstring; the unfused chain :7275-7278)."""
+    dt = x.dtype
+    mix = (float(lam) * shift1(x).float()).to(dt)
+    s1 = (x.float() + mix.float()).to(dt)
+    sf = s1.float()
+    inv = torch.rsqrt((sf * sf).mean(dim=-1) + eps)
+    return s1, (sf * inv[..., None]).to(dt), inv
+
+
+def mix_tail_backward(x, s1, inv, lam, gy, ge):
+    """(gx, dlam fp32): g = bf16(ge + inv (gy - s1 (gy . s1) inv^2 / C)) (the tail norm's backward, one rounding),
+    gx[t] = bf16(g[t] + bf16(lam g[t + 1])) (zero past a sequence's end), dlam = the fp32 sum of the bf16 products
+    bf16(g shift1(x)) (round1/source/train.py:7041 _g_rows, :7146 docstring)."""
+    dt = x.dtype
+    C = x.shape[-1]
+    sf = s1.float()
+    g = torch.zeros_like(sf)
+    if gy is not None:
+        gyf = gy.float()
+        dot = (gyf * sf).sum(dim=-1, keepdim=True)
+        iv = inv[..., None]
+        g = iv * (gyf - sf * (dot * iv * iv * (1.0 / C)))
+    if ge is not None:
+        g = g + ge.float()
+    g = g.to(dt)
+    nxt = torch.cat([g[:, 1:], torch.zeros_like(g[:, :1])], dim=1)
+    gx = (g.float() + (float(lam) * nxt.float()).to(dt).float()).to(dt)
+    dlam = (g.float() * shift1(x).float()).to(dt).float().sum()
+    return gx, dlam

@@ -469,3 +469,98 @@ def test_moe_mlp_module_mirror(api, dev, e8):
     for t in (xd, rd, wfd, wpd, sfd, spd):
         assert t.grad is not None and bool(torch.isfinite(t.grad.float()).all()) and float(t.grad.float().abs().max()) > 0
 
+
+def test_dense_bf16_fused_mlp_kernels_and_wrapper(dev):
+    """mlp_fwd_kernel / mlp_bwd_kernel in the reference's call style ((x2, w_fc, w_proj, tb) -> (y, rT);
+    (dy2, rT, w_fc, w_proj, tb, dw_mode) -> (dx, h, dpre), K/nki_mlp_fused.py:242, 290) against the oracle's restatement of
+    the kernels' arithmetic, and mlp_fused(mlp, x) with its weight gradients against autograd of the kit's expression."""
+    from oracle import mlp8 as O
+    from trainium_frontier_them_bones_amd import train_api as T
+    g = torch.Generator().manual_seed(5)
+    M, d, F = 512, 256, 1024
+    x = torch.randn(M, d, generator=g).bfloat16()
+    wf = (0.05 * torch.randn(F, d, generator=g)).bfloat16()
+    wp = (0.05 * torch.randn(d, F, generator=g)).bfloat16()
+    dy = torch.randn(M, d, generator=g).bfloat16()
+    assert T.mlp_fused_applies(x, F) and not T.mlp_fused_applies(x[:100], F)
+    y, rT = T.mlp_fwd_kernel(x.to(dev), wf.to(dev), wp.to(dev), 512)
+    yo, ro = O.forward_bf16(x, wf, wp)
+    assert tuple(rT.shape) == (F, M)
+    assert rel_l2(rT.t(), ro) < 2e-3 and rel_l2(y, yo) < 5e-3
+    dx, h, dpre = T.mlp_bwd_kernel(dy.to(dev), rT, wf.to(dev), wp.to(dev), 512, 0)
+    dxo, ho, dpo = O.backward_bf16(dy, rT.t().cpu(), wf, wp)
+    assert torch.equal(h.cpu(), ho) and rel_l2(dpre, dpo) < 2e-3 and rel_l2(dx, dxo) < 5e-3
+    dx1, hT, dpT = T.mlp_bwd_kernel(dy.to(dev), rT, wf.to(dev), wp.to(dev), 512, 1)
+    assert torch.equal(dx1, dx) and torch.equal(hT, h.t()) and torch.equal(dpT, dpre.t())
+
+    class M_:                                        # a module with the reference's attribute names
+        pass
+    mlp = M_()
+    mlp.c_fc, mlp.c_proj = M_(), M_()
+    mlp.c_fc.weight = wf.to(dev).requires_grad_(True)
+    mlp.c_proj.weight = wp.to(dev).requires_grad_(True)
+    xl = x.view(2, M // 2, d).to(dev).requires_grad_(True)
+    out = T.mlp_fused(mlp, xl)
+    out.backward(dy.view(2, M // 2, d).to(dev))
+    xr, wfr, wpr = (t.clone().float().requires_grad_(True) for t in (x, wf, wp))
+    ref = torch.nn.functional.linear(torch.relu(torch.nn.functional.linear(xr, wfr)).square(), wpr)
+    ref.backward(dy.float())
+    assert rel_l2(out.reshape(M, d), ref) < 5e-3 and rel_l2(xl.grad.reshape(M, d), xr.grad) < 1e-2
+    assert rel_l2(mlp.c_fc.weight.grad, wfr.grad) < 1e-2 and rel_l2(mlp.c_proj.weight.grad, wpr.grad) < 1e-2
+    with pytest.raises(Exception):
+        T.mlp_fwd_kernel(x[:100].to(dev), wf.to(dev), wp.to(dev))     # 100 rows: not a shape the kernels take
+
+
+def test_fused_gradient_norm_and_clip_factor(dev):
+    """grad_norm_fused over a bf16 and an fp32 gradient buffer (lengths off every vector width): the norm against fp64, the
+    clipping factor clamp(clip / (gnorm + 1e-6), max=1) (R1:1714), each buffer alone, and clip <= 0 giving 1."""
+    from trainium_frontier_them_bones_amd import ops
+    from trainium_frontier_them_bones_amd import train_api as T
+    g = torch.Generator().manual_seed(9)
+    for nb, nf in ((8 * 1000 + 8, 4 * 333 + 4), (1 << 22, 1 << 20), (8 * 77, 4 * 5)):
+        gb = torch.randn(nb, generator=g).bfloat16()
+        gf = torch.randn(nf, generator=g)
+        want = math.sqrt(float(gb.double().pow(2).sum() + gf.double().pow(2).sum()))
+        gn, sc = T.grad_norm_fused(gb.to(dev), gf.to(dev), 1.0)
+        assert abs(gn.item() - want) < 1e-5 * want
+        assert abs(sc.item() - min(1.0 / (want + 1e-6), 1.0)) < 1e-5
+        out = ops.gradnorm(gb.to(dev), gf.to(dev), 0.0).cpu()
+        assert abs(out[0].item() - float(gb.double().pow(2).sum())) < 1e-5 * out[0].item() and out[3].item() == 1.0
+        only_b = ops.gradnorm(gb.to(dev), None, 1e9).cpu()
+        assert abs(only_b[2].item() - math.sqrt(float(gb.double().pow(2).sum()))) < 1e-5 * only_b[2].item() and only_b[3].item() == 1.0
+        only_f = ops.gradnorm(None, gf.to(dev), 0.5).cpu()
+        assert abs(only_f[1].item() - float(gf.double().pow(2).sum())) < 1e-5 * only_f[1].item()
+
+
+@pytest.mark.parametrize("shape", [(2, 128, 256), (4, 256, 768), (1, 512, 1024)])
+def test_mix_tail_forward_and_backward(dev, shape):
+    """mix_tail(x, xn_dead, lam) (R1:7308) against the oracle: s1 bit for bit, xn2 and inv to rounding, and the gradients of
+    both outputs (gx, and dlam rounded to lam's dtype) through autograd; sequence starts read zeros and nothing crosses a
+    sequence boundary (perturbing one sequence leaves the others' outputs and gradients unchanged)."""
+    from oracle import norm as O
+    from trainium_frontier_them_bones_amd import train_api as T
+    B, Tn, C = shape
+    g = torch.Generator().manual_seed(B + Tn + C)
+    x = torch.randn(B, Tn, C, generator=g).bfloat16()
+    lam = torch.tensor(0.37).bfloat16()
+    gy = torch.randn(B, Tn, C, generator=g).bfloat16()
+    ge = torch.randn(B, Tn, C, generator=g).bfloat16()
+    xl = x.to(dev).requires_grad_(True)
+    ll = lam.to(dev).requires_grad_(True)
+    s1, y = T.mix_tail(xl, None, ll)
+    so, yo, invo = O.mix_tail(x, lam.float())
+    assert torch.equal(s1.cpu(), so) and rel_l2(y, yo) < 2e-3
+    torch.autograd.backward([s1, y], [ge.to(dev), gy.to(dev)])
+    gxo, dlo = O.mix_tail_backward(x, so, invo, lam.float(), gy, ge)
+    assert rel_l2(xl.grad, gxo) < 3e-3
+    assert ll.grad.dtype == torch.bfloat16 and abs(ll.grad.float().item() - float(dlo)) <= 2e-2 * abs(float(dlo)) + 0.5
+    # only one of the two gradients given
+    xl2 = x.to(dev).requires_grad_(True)
+    s2, y2 = T.mix_tail(xl2, None, lam.to(dev))
+    y2.backward(gy.to(dev))
+    assert rel_l2(xl2.grad, O.mix_tail_backward(x, so, invo, lam.float(), gy, None)[0]) < 3e-3
+    if B > 1:
+        xp = x.clone()
+        xp[0] += 1.0
+        s3, y3 = T.mix_tail(xp.to(dev), None, lam.to(dev))
+        assert torch.equal(s3[1:], s1[1:].detach()) and torch.equal(y3[1:], y[1:].detach())

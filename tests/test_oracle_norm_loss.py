@@ -187,3 +187,42 @@ def test_multi_target_and_label_smoothed_rows_against_cross_entropy_and_autograd
             _, lse_k = OL.loss_multi_rows(x, tg[:kk], rw[:kk], cap, eps)
             d = OL.loss_multi_backward(x.float(), tg[:kk], rw[:kk], lse_k, gup, cap, eps)
             assert rel_l2(d, xd.grad) < 1e-5
+
+
+def test_mix_tail_is_the_eager_chain_and_its_autograd():
+    """oracle/norm.py mix_tail / mix_tail_backward against the reference's unfused expression lam * shift1(x) -> tail_norm2
+    written with library routines: the forward in bf16 arithmetic (bit for bit), the backward against fp64 autograd of
+    the same chain (bf16 roundings bound the distance), the shift's adjoint identity, and lam = 0 (s1 = x, the norm's
+    own backward)."""
+    g = torch.Generator().manual_seed(11)
+    B, T, C = 3, 16, 256
+    x = torch.randn(B, T, C, generator=g).bfloat16()
+    lam = torch.tensor(0.37).bfloat16()
+    s1, y, inv = ON.mix_tail(x, lam.float())
+    sh = torch.cat([torch.zeros_like(x[:, :1]), x[:, :-1]], dim=1)
+    s_ref = x + lam * sh                                     # the eager bf16 ops: mul rounds, add rounds
+    assert torch.equal(s1, s_ref)
+    assert torch.equal(y, F.rms_norm(s_ref, (C,), None, ON.RMS_EPS))
+    assert float(sh[:, 0].abs().max()) == 0.0 and torch.equal(sh[:, 1:], x[:, :-1])
+    gy = torch.randn(B, T, C, generator=g).bfloat16()
+    ge = torch.randn(B, T, C, generator=g).bfloat16()
+    gx, dlam = ON.mix_tail_backward(x, s1, inv, lam.float(), gy, ge)
+    xd = x.double().requires_grad_(True)
+    ld = lam.double().requires_grad_(True)
+    shd = torch.cat([torch.zeros_like(xd[:, :1]), xd[:, :-1]], dim=1)
+    sd = xd + ld * shd
+    yd = sd * torch.rsqrt(sd.pow(2).mean(-1, keepdim=True) + ON.RMS_EPS)
+    (yd * gy.double()).sum().backward(retain_graph=True)
+    (sd * ge.double()).sum().backward()
+    assert rel_l2(gx, xd.grad) < 6e-3
+    assert abs(float(dlam) - float(ld.grad)) < 2e-2 * abs(float(ld.grad)) + 0.5
+    # the shift's adjoint: <shift1(x), g> = <x, shift1^T(g)>, with shift1^T(g)[t] = g[t + 1]
+    gg = torch.randn(B, T, C, generator=g).double()
+    nxt = torch.cat([gg[:, 1:], torch.zeros_like(gg[:, :1])], dim=1)
+    assert abs(float((ON.shift1(x).double() * gg).sum() - (x.double() * nxt).sum())) < 1e-9
+    # lam = 0: s1 = x and gx is the tail norm's own backward, dlam still the sum of g * shift1(x)
+    s0, _, inv0 = ON.mix_tail(x, 0.0)
+    assert torch.equal(s0, x)
+    gx0, _ = ON.mix_tail_backward(x, s0, inv0, 0.0, gy, None)
+    dx0, _ = ON.rmsnorm_backward(gy.reshape(-1, C), x.reshape(-1, C), inv0.reshape(-1), None)
+    assert rel_l2(gx0.reshape(-1, C), dx0) < 4e-3

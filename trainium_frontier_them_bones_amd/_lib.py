@@ -72,6 +72,12 @@ SIGNATURES = {
     "tfb_fill_f32": [_vp, _f, _l, _vp],
     "tfb_loss_fwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_loss_fwd_bwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
+    "tfb_mlp_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_mlp_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
+    "tfb_gradnorm_scratch_floats": [],
+    "tfb_gradnorm": [_vp, _l, _vp, _l, _f, _vp, _vp, _vp],
+    "tfb_mix_tail_fwd": [_vp, _vp, _vp, _vp, _vp, _l, _i, _i, _f, _vp],
+    "tfb_mix_tail_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _l, _i, _i, _vp],
     "tfb_loss_row_weights": [_vp, _i, _vp, _l, _i, _i, _vp],
     "tfb_loss_bwd": [_vp, _vp, _i, _vp, _vp, _vp, _l, _i, _f, _vp],
     "tfb_loss_multi_fwd": [_vp, _vp, _i, _vp, _i, _f, _vp, _vp, _l, _i, _f, _vp],
@@ -105,7 +111,7 @@ SIGNATURES = {
     "tfb_mlp_dw_proj": [_vp, _vp, _vp, _l, _i, _i, _i, _i, _vp, _l, _vp],
 }
 
-_LONG_RESULT = {"tfb_attn_bwd_static_max_rows", "tfb_mlp8_scale_scratch_floats", "tfb_moe_max_rows", "tfb_embedding_bwd_scratch_ints", "tfb_ns5_workspace_bytes"}
+_LONG_RESULT = {"tfb_gradnorm_scratch_floats", "tfb_attn_bwd_static_max_rows", "tfb_mlp8_scale_scratch_floats", "tfb_moe_max_rows", "tfb_embedding_bwd_scratch_ints", "tfb_ns5_workspace_bytes"}
 
 STATUS = {0: "ok", 1: "unsupported shape", 2: "bad argument", 3: "kernel launch failed", 4: "workspace too small"}
 

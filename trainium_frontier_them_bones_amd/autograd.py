@@ -790,3 +790,56 @@ class MoeMlp8Fn(torch.autograd.Function):
         dh, dwr, _ = ops.moe_route_bwd(dgate, p, idx, dxs, tab, h2, wr, br, accr, aux=aux)
         return (dh.view(ctx.hshape), (None if br is not None else dwr.to(router.dtype)), dw_fc, dw_proj, None, None, None, None,
                 None, None)
+
+
+class MlpFusedFn(torch.autograd.Function):
+    """The dense bf16 fused MLP: y = c_proj(relu(c_fc(x))^2) on [M, d] rows with the fused kernels' rounding points; saves
+    x2 and r only; dW accumulates into the weights' grad_buf when present (round2/source/kernels/nki_mlp_fused.py:408
+    EmulatedFusedMlp; kernels :242, :290)."""
+
+    @staticmethod
+    def forward(ctx, x2, w_fc, w_proj):
+        x2 = x2.contiguous()
+        y, r = ops.mlp_fwd(x2, w_fc, w_proj)
+        ctx.save_for_backward(x2, r, w_fc, w_proj)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2, r, w_fc, w_proj = ctx.saved_tensors
+        dy = dy.contiguous()
+        dx, h, dpre = ops.mlp_bwd(dy, r, w_fc, w_proj)
+        grads = []
+        for w, a, b in ((w_fc, dpre, x2), (w_proj, dy, h)):     # dw_fc = dpre^T x, dw_proj = dy^T h
+            buf, acc = _accumulate_into(w)
+            if buf is not None:
+                ops.matmul(a, b, trans_a=True, out=buf, accumulate=acc)
+                grads.append(None)
+            else:
+                grads.append(ops.matmul(a, b, trans_a=True))
+        return dx, grads[0], grads[1]
+
+
+class MixTailFn(torch.autograd.Function):
+    """(s1, xn2) = (x + lam shift1(x), RMSNorm(s1)) on the [N, C] stream, sequences of T rows; gradients (gx, dlam)
+    (round1/source/train.py:7330 MixTailFn)."""
+
+    @staticmethod
+    def forward(ctx, x2, lam, T):
+        ctx.set_materialize_grads(False)
+        x2 = x2.contiguous()
+        lam32 = lam.detach().reshape(1).to(torch.float32)
+        s1, xn2, inv = ops.mix_tail_fwd(x2, lam32, T)
+        ctx.save_for_backward(x2, s1, inv, lam32)
+        ctx.T, ctx.lam_meta = T, (lam.shape, lam.dtype)
+        return s1, xn2
+
+    @staticmethod
+    def backward(ctx, ge, gy):
+        x2, s1, inv, lam32 = ctx.saved_tensors
+        if ge is None and gy is None:
+            return None, None, None
+        gx, dlam = ops.mix_tail_bwd(s1, inv, x2, lam32, ctx.T, None if gy is None else gy.contiguous(),
+                                    None if ge is None else ge.contiguous())
+        shape, dtype = ctx.lam_meta
+        return gx, dlam.to(dtype).reshape(shape), None

@@ -714,3 +714,96 @@ extern "C" int tfb_fill_f32(void* p, float val, long n, void* stream) {
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }
+
+// ---- gradient norm -------------------------------------------------------------------------------------------------
+// The sums of squares of the step's gradient buffers (a bf16 one: the matrices' flat gradient; an fp32 one: embedding and
+// norm weights) in one pass, and from them the global norm and the clipping factor, all left on the device.
+// Replaces _gradnorm_kernel (round1/source/train.py:1480) and the norm / gate arithmetic of reduce_fused (:1634-1720):
+// gnorm = sqrt(sum of squares), scale = min(clip / (gnorm + 1e-6), 1) for clip > 0, else 1.
+namespace {
+constexpr int GN_BLOCKS = 1024;
+__global__ __launch_bounds__(256) void gradnorm_partial_kernel(const bf16_t* __restrict__ gb, long nb, const float* __restrict__ gf,
+                                                              long nf, float* __restrict__ part) {
+  __shared__ float red[2][4];
+  float sb = 0.f, sf = 0.f;
+  const long t = (long)blockIdx.x * 256 + threadIdx.x, stride = (long)gridDim.x * 256;
+  const long nb8 = nb / 8, nf4 = nf / 4;
+  for (long i = t; i < nb8; i += stride) {
+    const u32x4 u = __builtin_nontemporal_load((const u32x4*)gb + i);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float a = bflo(u[k]), b = bfhi(u[k]);
+      sb += a * a;
+      sb += b * b;
+    }
+  }
+  for (long i = nb8 * 8 + t; i < nb; i += stride) sb += bf2f(gb[i]) * bf2f(gb[i]);
+  for (long i = t; i < nf4; i += stride) {
+    const f32x4 v = __builtin_nontemporal_load((const f32x4*)gf + i);
+    sf += v[0] * v[0];
+    sf += v[1] * v[1];
+    sf += v[2] * v[2];
+    sf += v[3] * v[3];
+  }
+  for (long i = nf4 * 4 + t; i < nf; i += stride) sf += gf[i] * gf[i];
+  sb = wave_sum(sb);
+  sf = wave_sum(sf);
+  if ((threadIdx.x & 63) == 0) {
+    red[0][threadIdx.x >> 6] = sb;
+    red[1][threadIdx.x >> 6] = sf;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    part[2 * blockIdx.x] = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+    part[2 * blockIdx.x + 1] = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+  }
+}
+// out[0], out[1] = the two sums (partials added in a fixed order), out[2] = gnorm, out[3] = the clipping factor
+__global__ __launch_bounds__(256) void gradnorm_finish_kernel(const float* __restrict__ part, int blocks, float clip,
+                                                             float* __restrict__ out) {
+  __shared__ float red[2][4];
+  float sb = 0.f, sf = 0.f;
+  for (int i = threadIdx.x; i < blocks; i += 256) {
+    sb += part[2 * i];
+    sf += part[2 * i + 1];
+  }
+  sb = wave_sum(sb);
+  sf = wave_sum(sf);
+  if ((threadIdx.x & 63) == 0) {
+    red[0][threadIdx.x >> 6] = sb;
+    red[1][threadIdx.x >> 6] = sf;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const float a = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+    const float b = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+    const float gn = sqrtf(a + b);
+    out[0] = a;
+    out[1] = b;
+    out[2] = gn;
+    out[3] = clip > 0.f ? fminf(clip / (gn + 1e-6f), 1.0f) : 1.0f;
+  }
+}
+}  // namespace
+
+extern "C" long tfb_gradnorm_scratch_floats(void) { return 2L * GN_BLOCKS; }
+
+// g_bf16 [n_bf16] (may be NULL with n 0), g_f32 [n_f32] (likewise), both 16-byte aligned; scratch fp32
+// [tfb_gradnorm_scratch_floats()]; out fp32 [4] = (sum of squares of g_bf16, of g_f32, the norm of both together,
+// min(clip / (norm + 1e-6), 1) or 1 when clip <= 0). Two launches, deterministic.
+extern "C" int tfb_gradnorm(const void* g_bf16, long n_bf16, const void* g_f32, long n_f32, float clip, void* scratch, void* out,
+                            void* stream) {
+  if (!scratch || !out || (n_bf16 > 0 && !g_bf16) || (n_f32 > 0 && !g_f32)) return TFB_ERR_ARG;
+  if (n_bf16 < 0 || n_f32 < 0 || n_bf16 + n_f32 <= 0) return TFB_ERR_SHAPE;
+  if (((uintptr_t)g_bf16 | (uintptr_t)g_f32) & 15) return TFB_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const long work = n_bf16 / 8 + n_f32 / 4;
+  int blocks = (int)((work + 255) / 256);
+  blocks = blocks < 1 ? 1 : (blocks > GN_BLOCKS ? GN_BLOCKS : blocks);
+  hipLaunchKernelGGL(gradnorm_partial_kernel, dim3(blocks), dim3(256), 0, s, (const bf16_t*)g_bf16, n_bf16, (const float*)g_f32,
+                     n_f32, (float*)scratch);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(gradnorm_finish_kernel, dim3(1), dim3(256), 0, s, (const float*)scratch, blocks, clip, (float*)out);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}

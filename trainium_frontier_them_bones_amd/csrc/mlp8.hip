@@ -1182,3 +1182,67 @@ extern "C" int tfb_moe_mlp_bwd(const void* dys, const void* r, const void* w_fc,
   return grouped_launch<CfgNN>((const uint8_t*)w_fc, d * 2L, n * 2, (const uint8_t*)dpre, F * 2L, d, rmax, F * 2L,
                                (const int*)tile_expert, e2, s);
 }
+
+// ---- dense bf16 fused MLP ------------------------------------------------------------------------------------------
+// y = bf16(h @ w_proj^T) with r = bf16(relu(x @ w_fc^T)), h = bf16(r r); backward dpre = bf16(((dy @ w_proj) 2) r) (ONE
+// rounding: the fused kernel folds the factors into the product's evacuation), h = bf16(r r), dx = bf16(dpre @ w_fc).
+// Replaces _mlp_fwd_kernel(x2, w_fc, w_proj, tb) -> (y, rT) and _mlp_bwd_kernel(dy2, rT, w_fc, w_proj, tb, dw_mode) ->
+// (dx, h, dpre) (round2/source/kernels/nki_mlp_fused.py:242, 290; arithmetic emulate_forward / emulate_backward :372-392).
+// The saved activation is token-major r [M][F] (the reference keeps its transpose for its SBUF layout).
+namespace {
+struct EpiDpre1 {  // dpre = bf16((acc 2) r); optionally h = bf16(r r)
+  const bf16_t* r;
+  bf16_t* dpre;
+  bf16_t* h;  // or null
+  long F;
+  typedef u32x4 pre_t;
+  __device__ __forceinline__ pre_t prefetch(int p, int q) const { return *(const u32x4*)(r + (long)q * F + p); }
+  __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const pre_t& rv, int) const {
+    float rr[8];
+    unpack8bf(rv, rr);
+    u32x4 o, hb;
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      o[i >> 1] = pack2bf((v[i] * 2.f) * rr[i], (v[i + 1] * 2.f) * rr[i + 1]);
+      hb[i >> 1] = pack2bf(rr[i] * rr[i], rr[i + 1] * rr[i + 1]);
+    }
+    const long off = (long)q * F + p;
+    *(u32x4*)(dpre + off) = o;
+    if (h) *(u32x4*)(h + off) = hb;
+  }
+};
+}  // namespace
+
+// x bf16 [M][d], w_fc bf16 [F][d], w_proj bf16 [d][F] -> y bf16 [M][d], r bf16 [M][F] (saved for the backward), h bf16
+// [M][F] (the second GEMM's operand; scratch for the caller). M, d, F multiples of 128.
+extern "C" int tfb_mlp_fwd(const void* x, const void* w_fc, const void* w_proj, void* y, void* r, void* h, long M, int d, int F,
+                           void* stream) {
+  if (!x || !w_fc || !w_proj || !y || !r || !h) return TFB_ERR_ARG;
+  if (!shapes16(M, d, F) || M > 0x7fffffffL) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  GemmOperand Pw{(const uint8_t*)w_fc, d * 2L}, Qx{(const uint8_t*)x, d * 2L};
+  EpiRelu2 e1{(bf16_t*)r, (bf16_t*)h, (long)F};
+  int st = gemm_launch<CfgNT>(Pw, Qx, F, (int)M, d * 2L, 1, LoadIdentity{}, LoadIdentity{}, e1, s);
+  if (st != TFB_OK) return st;
+  GemmOperand Pp{(const uint8_t*)w_proj, F * 2L}, Qh{(const uint8_t*)h, F * 2L};
+  EpiStore e2{y, (long)d, 0, 0};
+  return gemm_launch<CfgNT>(Pp, Qh, d, (int)M, F * 2L, 1, LoadIdentity{}, LoadIdentity{}, e2, s);
+}
+
+// dy bf16 [M][d], r as the forward left it -> dx bf16 [M][d], dpre bf16 [M][F], h bf16 [M][F] (optional, may be NULL):
+// what the weight gradients dw_fc = dpre^T x and dw_proj = dy^T h contract (weight_grads, :394).
+extern "C" int tfb_mlp_bwd(const void* dy, const void* r, const void* w_fc, const void* w_proj, void* dx, void* h, void* dpre,
+                           long M, int d, int F, void* stream) {
+  if (!dy || !r || !w_fc || !w_proj || !dx || !dpre) return TFB_ERR_ARG;
+  if (!shapes16(M, d, F) || M > 0x7fffffffL) return TFB_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  // dh[m][f] = sum_j dy[m][j] w_proj[j][f]: the weight is the k-strided operand (k = j, contiguous in f)
+  GemmOperand Pp{(const uint8_t*)w_proj, F * 2L}, Qg{(const uint8_t*)dy, d * 2L};
+  EpiDpre1 e1{(const bf16_t*)r, (bf16_t*)dpre, (bf16_t*)h, (long)F};
+  int st = gemm_launch<CfgNN>(Pp, Qg, F, (int)M, d * 2L, 1, LoadIdentity{}, LoadIdentity{}, e1, s);
+  if (st != TFB_OK) return st;
+  // dx[m][j] = sum_f dpre[m][f] w_fc[f][j]
+  GemmOperand Pf{(const uint8_t*)w_fc, d * 2L}, Qd{(const uint8_t*)dpre, F * 2L};
+  EpiStore e2{dx, (long)d, 0, 0};
+  return gemm_launch<CfgNN>(Pf, Qd, d, (int)M, F * 2L, 1, LoadIdentity{}, LoadIdentity{}, e2, s);
+}

@@ -399,6 +399,109 @@ __global__ __launch_bounds__(256) void block_head_bwd_kernel(const bf16_t* __res
   if (threadIdx.x == 3) gain_part[(long)blockIdx.x * 4 + 3] = 0.f;
 }
 
+// ------------------------------------------------------------------------------------------ mixer tail
+// The attention-less block's causal one-token shift in front of the tail norm:
+//   s1 = bf16(x + bf16(lam * shift1(x))), xn2 = RMSNorm(s1), inv saved; shift1 gives token t the row of token t - 1 of its
+//   sequence (zeros at t = 0). One wavefront per row; the previous row is read again (it is the neighbour's row, from L2).
+template <int NCH>
+__global__ __launch_bounds__(256) void mix_tail_fwd_kernel(const bf16_t* __restrict__ x, const float* __restrict__ lam,
+                                                          bf16_t* __restrict__ s1, bf16_t* __restrict__ xn2,
+                                                          float* __restrict__ inv, long nrows, int C, int T, float eps) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float l = lam[0];
+  for (long row = (long)blockIdx.x * ROWS_PER_BLOCK + wave; row < nrows; row += (long)gridDim.x * ROWS_PER_BLOCK) {
+    Row<NCH> a, b;
+    a.load(x + row * C, C, lane);
+    if (row % T) b.load(x + (row - 1) * C, C, lane);
+    else b.zero();
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) a.v[i][k] = round_bf(a.v[i][k] + round_bf(l * b.v[i][k]));
+    a.store(s1 + row * C, C, lane);
+    const float ss = row_dot(a, a);
+    const float rs = 1.0f / sqrtf(ss * (1.0f / C) + eps);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) a.v[i][k] *= rs;
+    a.store(xn2 + row * C, C, lane);
+    if (lane == 0) inv[row] = rs;
+  }
+}
+
+// g = bf16(ge + inv (gy - s (gy . s) inv^2 / C)) (the tail norm's backward, one rounding; ge and/or gy may be absent);
+// gx[t] = bf16(g[t] + bf16(lam g[t + 1])) (g[t + 1] = 0 at a sequence's last token: the shift's adjoint);
+// dlam partial [gridDim.x] = sum over the workgroup's rows of the bf16 products bf16(g[t] x[t - 1]) in fp32.
+// Row t + 1's g is recomputed by the wavefront that owns row t (the chain is per row: the same bits).
+template <int NCH>
+__global__ __launch_bounds__(256) void mix_tail_bwd_kernel(const bf16_t* __restrict__ s, const bf16_t* __restrict__ gy,
+                                                          const bf16_t* __restrict__ ge, const float* __restrict__ inv,
+                                                          const bf16_t* __restrict__ x, const float* __restrict__ lam,
+                                                          bf16_t* __restrict__ gx, float* __restrict__ dlam_part, long nrows,
+                                                          int C, int T) {
+  __shared__ float red[ROWS_PER_BLOCK];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float l = lam[0];
+  float dl = 0.f;
+  auto g_row = [&](long row, Row<NCH>& g) {
+    Row<NCH> a;
+    a.load(s + row * C, C, lane);
+    if (gy) {
+      g.load(gy + row * C, C, lane);
+      const float rs = inv[row];
+      const float coef = row_dot(g, a) * rs * rs * (1.0f / C);
+#pragma unroll
+      for (int i = 0; i < NCH; ++i)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) g.v[i][k] = rs * (g.v[i][k] - a.v[i][k] * coef);
+    } else {
+      g.zero();
+    }
+    if (ge) {
+      Row<NCH> e;
+      e.load(ge + row * C, C, lane);
+#pragma unroll
+      for (int i = 0; i < NCH; ++i)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) g.v[i][k] += e.v[i][k];
+    }
+    g.round();
+  };
+  for (long row = (long)blockIdx.x * ROWS_PER_BLOCK + wave; row < nrows; row += (long)gridDim.x * ROWS_PER_BLOCK) {
+    Row<NCH> g, gn, xp;
+    g_row(row, g);
+    if ((row + 1) % T) g_row(row + 1, gn);
+    else gn.zero();
+    if (row % T) xp.load(x + (row - 1) * C, C, lane);
+    else xp.zero();
+    float part = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        part += round_bf(g.v[i][k] * xp.v[i][k]);
+        g.v[i][k] = g.v[i][k] + round_bf(l * gn.v[i][k]);
+      }
+    dl += wave_sum(part);
+    g.store(gx + row * C, C, lane);
+  }
+  if (lane == 0) red[wave] = dl;
+  __syncthreads();
+  if (threadIdx.x == 0) dlam_part[blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// out[0] = sum of part[0 .. n) in a fixed order (one workgroup)
+__global__ __launch_bounds__(256) void sum_partials_kernel(const float* __restrict__ part, int n, float* __restrict__ out) {
+  __shared__ float red[4];
+  float t = 0.f;
+  for (int i = threadIdx.x; i < n; i += 256) t += part[i];
+  t = wave_sum(t);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = t;
+  __syncthreads();
+  if (threadIdx.x == 0) out[0] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
 inline int grid_for(long nrows, int cap) {
   long b = (nrows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
   return (int)(b < cap ? b : cap);
@@ -546,6 +649,42 @@ extern "C" int tfb_block_head_bwd(const void* g_new, const void* g_norm, const v
   TFB_LAUNCH_CHECK();
   hipLaunchKernelGGL(colsum_kernel, dim3(1), dim3(64, 16), 0, (hipStream_t)stream, (const float*)gain_part, (float*)dgains,
                      grid, 4, 0);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+// ---- mixer tail (round1/source/train.py:7308 mix_tail; kernels _mix_fwd_kernel :7097, _mix_bwd_kernel :7145) -----------------
+// x bf16 [nrows][C] (nrows = sequences x T tokens), lam: device fp32 scalar -> s1 = bf16(x + bf16(lam shift1(x))),
+// xn2 = RMSNorm(s1) (no weight), inv fp32 [nrows].
+extern "C" int tfb_mix_tail_fwd(const void* x, const void* lam, void* s1, void* xn2, void* inv, long nrows, int C, int T,
+                                float eps, void* stream) {
+  if (!x || !lam || !s1 || !xn2 || !inv) return TFB_ERR_ARG;
+  if (!norm_shape_ok(nrows, C) || T <= 0 || nrows % T) return TFB_ERR_SHAPE;
+  int grid = grid_for(nrows, 8192);
+#define CALL(N)                                                                                                          \
+  hipLaunchKernelGGL(mix_tail_fwd_kernel<N>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x,            \
+                     (const float*)lam, (bf16_t*)s1, (bf16_t*)xn2, (float*)inv, nrows, C, T, eps)
+  DISPATCH_NCH(C, CALL);
+#undef CALL
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+// s1, inv as the forward left them; gy (gradient of xn2) and ge (gradient of s1) bf16 [nrows][C], either may be NULL (not
+// both); x the forward's input -> gx bf16 [nrows][C], dlam fp32 [1] = sum over all elements of bf16(g shift1(x)) (the
+// caller rounds it to lam's dtype). part: fp32 [tfb_norm_bwd_blocks(nrows)] scratch.
+extern "C" int tfb_mix_tail_bwd(const void* s1, const void* gy, const void* ge, const void* inv, const void* x, const void* lam,
+                                void* gx, void* part, void* dlam, long nrows, int C, int T, void* stream) {
+  if (!s1 || (!gy && !ge) || !inv || !x || !lam || !gx || !part || !dlam) return TFB_ERR_ARG;
+  if (!norm_shape_ok(nrows, C) || T <= 0 || nrows % T) return TFB_ERR_SHAPE;
+  int grid = grid_for(nrows, 1024);
+#define CALL(N)                                                                                                          \
+  hipLaunchKernelGGL(mix_tail_bwd_kernel<N>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)s1,           \
+                     (const bf16_t*)gy, (const bf16_t*)ge, (const float*)inv, (const bf16_t*)x, (const float*)lam,       \
+                     (bf16_t*)gx, (float*)part, nrows, C, T)
+  DISPATCH_NCH(C, CALL);
+#undef CALL
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sum_partials_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const float*)part, grid, (float*)dlam);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
 }

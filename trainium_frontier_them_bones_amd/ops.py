@@ -1104,3 +1104,74 @@ def ns5(g, d, coeffs=NS_COEFFS):
     _lib.call("tfb_ns5", _p(g), _p(inv), co, _p(y), _p(v), K, M, N, int(wide), _p(ws), ws.numel(), _stream())
     return y, v
 
+
+# ------------------------------------------------------------------------------------------ dense bf16 fused MLP
+def mlp_fwd(x2, w_fc, w_proj):
+    """(y [M,d], r [M,F]) bf16: y = bf16(bf16(r r) @ w_proj^T), r = bf16(relu(x2 @ w_fc^T)); w_fc [F,d], w_proj [d,F]
+    (K/nki_mlp_fused.py:242). r is token-major (the reference's rT is r.t())."""
+    _chk(x2), _chk(w_fc), _chk(w_proj)
+    M, d = x2.shape
+    F = w_fc.shape[0]
+    if tuple(w_fc.shape) != (F, d) or tuple(w_proj.shape) != (d, F):
+        raise ValueError("w_fc is [F, d], w_proj is [d, F]")
+    y = torch.empty(M, d, dtype=bf16, device=x2.device)
+    r = torch.empty(M, F, dtype=bf16, device=x2.device)
+    h = torch.empty(M, F, dtype=bf16, device=x2.device)
+    _lib.call("tfb_mlp_fwd", _p(x2), _p(w_fc), _p(w_proj), _p(y), _p(r), _p(h), M, d, F, _stream())
+    return y, r
+
+
+def mlp_bwd(dy2, r, w_fc, w_proj, want_h=True):
+    """(dx [M,d], h [M,F] or None, dpre [M,F]) bf16: dpre = bf16(((dy2 @ w_proj) 2) r), h = bf16(r r), dx = bf16(dpre @ w_fc)
+    (K/nki_mlp_fused.py:290 with dw_mode 0)."""
+    _chk(dy2), _chk(r), _chk(w_fc), _chk(w_proj)
+    M, d = dy2.shape
+    F = w_fc.shape[0]
+    if tuple(r.shape) != (M, F) or tuple(w_fc.shape) != (F, d) or tuple(w_proj.shape) != (d, F):
+        raise ValueError("shapes differ")
+    dx = torch.empty(M, d, dtype=bf16, device=dy2.device)
+    dpre = torch.empty(M, F, dtype=bf16, device=dy2.device)
+    h = torch.empty(M, F, dtype=bf16, device=dy2.device) if want_h else None
+    _lib.call("tfb_mlp_bwd", _p(dy2), _p(r), _p(w_fc), _p(w_proj), _p(dx), _p(h), _p(dpre), M, d, F, _stream())
+    return dx, h, dpre
+
+
+# ------------------------------------------------------------------------------------------ gradient norm
+def gradnorm(g_bf16=None, g_f32=None, clip=0.0):
+    """fp32 [4] on the device: (sum of squares of g_bf16, of g_f32, the norm of both together, the clipping factor
+    min(clip / (norm + 1e-6), 1), 1 when clip <= 0). Either buffer may be None (R1:1480, 1634)."""
+    _chk(g_bf16), _chk(g_f32, torch.float32)
+    ref = g_bf16 if g_bf16 is not None else g_f32
+    if ref is None:
+        raise ValueError("give at least one gradient buffer")
+    out = torch.empty(4, dtype=torch.float32, device=ref.device)
+    scr = _scratch(ref.device, int(_lib.lib().tfb_gradnorm_scratch_floats()))
+    _lib.call("tfb_gradnorm", _p(g_bf16), 0 if g_bf16 is None else g_bf16.numel(), _p(g_f32),
+              0 if g_f32 is None else g_f32.numel(), float(clip), _p(scr), _p(out), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------ mixer tail
+def mix_tail_fwd(x2, lam, T, eps=2.0 ** -23):
+    """(s1, xn2, inv): s1 = bf16(x2 + bf16(lam shift1(x2))) with shift1 inside sequences of T rows, xn2 = RMSNorm(s1);
+    lam a 1-element fp32 device tensor (R1:7097)."""
+    _chk(x2), _chk(lam, torch.float32)
+    rows, C = x2.shape
+    s1, xn2 = torch.empty_like(x2), torch.empty_like(x2)
+    inv = torch.empty(rows, dtype=torch.float32, device=x2.device)
+    _lib.call("tfb_mix_tail_fwd", _p(x2), _p(lam), _p(s1), _p(xn2), _p(inv), rows, C, int(T), float(eps), _stream())
+    return s1, xn2, inv
+
+
+def mix_tail_bwd(s1, inv, x2, lam, T, gy=None, ge=None):
+    """(gx bf16 [rows,C], dlam fp32 [1]) from the gradients gy of xn2 and ge of s1 (either may be None) (R1:7145)."""
+    _chk(s1), _chk(x2), _chk(gy), _chk(ge), _chk(inv, torch.float32), _chk(lam, torch.float32)
+    if gy is None and ge is None:
+        raise ValueError("give gy or ge")
+    rows, C = s1.shape
+    gx = torch.empty_like(s1)
+    part = _scratch(s1.device, int(_lib.lib().tfb_norm_bwd_blocks(rows)))
+    dlam = torch.empty(1, dtype=torch.float32, device=s1.device)
+    _lib.call("tfb_mix_tail_bwd", _p(s1), _p(gy), _p(ge), _p(inv), _p(x2), _p(lam), _p(gx), _p(part), _p(dlam), rows, C, int(T),
+              _stream())
+    return gx, dlam

@@ -472,3 +472,60 @@ def adamw_fused_step(opt) -> bool:
 
 # ------------------------------------------------------------------------------------------ R1 fp8 MLP rows (R1:1780-4140)
 from .r1_fp8 import nki_gemm_fp8, nki_gemm_fp8_nn  # noqa: E402  (namespaces, as the reference uses its modules)
+
+
+# ------------------------------------------------------------------------------------------ dense bf16 fused MLP (R2:6782; K/nki_mlp_fused.py)
+def mlp_fused_applies(x2, f):
+    """The shapes the dense fused MLP kernels take: token rows, model width and hidden width multiples of 128
+    (K/nki_mlp_fused.py:364 shapes_apply)."""
+    return x2.dim() == 2 and x2.shape[0] > 0 and x2.shape[0] % 128 == 0 and x2.shape[1] % 128 == 0 and f % 128 == 0
+
+
+def mlp_fwd_kernel(x2, w_fc, w_proj, tb=None):
+    """(y [M, d], rT [F, M]) as _mlp_fwd_kernel returns them (K/nki_mlp_fused.py:242); rT is a transposed view of the
+    token-major r the backward reads. `tb` (the reference's token-block size) is accepted and unused."""
+    y, r = ops.mlp_fwd(x2.contiguous(), w_fc.contiguous(), w_proj.contiguous())
+    return y, r.t()
+
+
+def mlp_bwd_kernel(dy2, rT, w_fc, w_proj, tb=None, dw_mode=0):
+    """(dx, h, dpre) as _mlp_bwd_kernel returns them (K/nki_mlp_fused.py:290): token-major [M, F] for dw_mode 0, their
+    transposes [F, M] for dw_mode 1."""
+    r = rT.t()
+    dx, h, dpre = ops.mlp_bwd(dy2.contiguous(), r if r.is_contiguous() else r.contiguous(), w_fc.contiguous(), w_proj.contiguous())
+    if dw_mode == 1:
+        return dx, h.t().contiguous(), dpre.t().contiguous()
+    return dx, h, dpre
+
+
+def mlp_fused(mlp, x):
+    """MLP.forward on [b, t, n_embd] through the dense bf16 fused kernels (R2:6782): `mlp` has c_fc.weight [F, d] and
+    c_proj.weight [d, F]. Raises TfbError for a shape the kernels do not take (the round-2 policy)."""
+    b, t, c = x.shape
+    x2 = x.reshape(b * t, c).contiguous()
+    w_fc = mlp.c_fc.weight.to(dtype=x.dtype)
+    w_proj = mlp.c_proj.weight.to(dtype=x.dtype)
+    return A.MlpFusedFn.apply(x2, w_fc, w_proj).view(b, t, c)
+
+
+# ------------------------------------------------------------------------------------------ gradient norm (R1:1480, 1634)
+def grad_norm_fused(g_bf16=None, g_f32=None, clip=0.0):
+    """(gnorm, scale) as 0-dim device tensors: the global gradient norm over the two flat gradient buffers in one kernel
+    pair, and the clipping factor clamp(clip / (gnorm + 1e-6), max=1) the caller multiplies the gradients by (1 for
+    clip <= 0), as reduce_fused computes them (R1:1634-1720). Nothing is read back by the host."""
+    out = ops.gradnorm(g_bf16, g_f32, clip)
+    return out[2], out[3]
+
+
+# ------------------------------------------------------------------------------------------ mixer tail (R1:7308)
+def shift1(x):
+    """Token t of every sequence reads token t - 1; token 0 reads zeros (R1:300)."""
+    return torch.cat([torch.zeros_like(x[:, :1]), x[:, :-1]], dim=1)
+
+
+def mix_tail(x, xn_dead, lam):
+    """(s1, xn2) = (x + lam * shift1(x), RMSNorm(s1)) for a [B, T, C] stream in one launch each way (R1:7308). xn_dead (the
+    head's unused x_norm) is accepted for the reference's signature and not read."""
+    B, T, C = x.shape
+    s1, y = A.MixTailFn.apply(x.reshape(B * T, C), lam, T)
+    return s1.view(B, T, C), y.view(B, T, C)
