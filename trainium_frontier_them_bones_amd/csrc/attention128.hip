@@ -1,0 +1,586 @@
+// Causal flash attention for head dimension 128 on gfx950 (the reference's own models run D = 128): the kernels the C-ABI
+// entry points in attention.hip run for D = 128. Same arithmetic contract as the other head dimension (stated in
+// attention.hip) and the same data movement as the D = 64 kernels:
+//   * 64-token x D tiles go from global memory straight into LDS with global_load_lds_dwordx4 (no staging registers, no
+//     VALU transposes); a token's row is 2 D bytes and 16-byte chunk c of token t sits at slot c ^ swz(t), a swizzle under
+//     which ONE copy of a tile serves both MFMA operand forms without bank conflicts: token-major fragments (ds_read_b128:
+//     16 consecutive tokens of one chunk on 16 different 16-byte bank groups) and transposed fragments
+//     (ds_read_b64_tr_b16: the four tokens of a 32-lane access on four different 64-byte bank quarters);
+//   * two LDS stages (separate __shared__ objects), one barrier per stage;
+//   * workgroups re-dealt so that all sequence blocks of a (batch, head) pair run on one XCD (its L2 then serves the K/V or
+//     Q/dO tiles those blocks stream repeatedly), and a workgroup does block i and then block nx - 1 - i (equal causal work
+//     per workgroup);
+//   * a wavefront owns 32 queries (forward, dQ) or 32 keys (dK/dV) as the MFMA column index: row statistics are per-lane
+//     scalars and the packed score registers are directly the B operand of the second product;
+//   * the backward accumulators start from the rows' -lse / scale and -delta, which the dQ kernel makes from the dO
+//     fragments it holds anyway and leaves for dK/dV.
+// The tile loops are plain (not software-pipelined): at D = 128 a second set of scores does not fit the registers of two
+// wavefronts per SIMD. Forward and dQ run two wavefronts per SIMD (221 / 256 registers); dK/dV holds K, V fragments and
+// both gradients' accumulators (192 registers before any score) and runs one (at two it spills 100 registers and takes
+// 0.52 instead of 0.38 ms at B16 H6 T2048).
+#include <type_traits>
+#include "common.hpp"
+
+#ifndef TFB_DKDV128_R
+#define TFB_DKDV128_R 64  // queries per LDS stage of the dK/dV kernel (128: 0.39 vs 0.38 ms at B16 H6 T2048)
+#endif
+#ifndef TFB_DKDV128_WPE
+#define TFB_DKDV128_WPE 1  // wavefronts per SIMD the dK/dV kernel is compiled for
+#endif
+
+namespace {
+
+struct AttnT {
+  bf16_t* p;
+  long sb, sh, st;
+};
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef const __attribute__((address_space(1))) void glb_void_t;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4_t;
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+__device__ __forceinline__ f32x16 mfma_bf16(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ bf16x8 frag_from(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  u32x4 v = {a, b, c, d};
+  return __builtin_bit_cast(bf16x8, v);
+}
+__device__ __forceinline__ void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // s_waitcnt vmcnt(0)
+
+template <int D>
+struct Geo {
+  static constexpr int ROWB = 2 * D;        // bytes of a token's row
+  static constexpr int TILE = 64 * ROWB;    // bytes of a 64-token tile
+  static constexpr int NKS = D / 16;        // MFMA k-steps over the head dimension
+  static constexpr int NDT = D / 32;        // 32-element tiles of the head dimension
+  static constexpr int LPT = ROWB / 16;     // lanes (16-byte chunks) per token
+  static constexpr int TPI = 64 / LPT;      // tokens per 1 KB load instruction
+  // slot swizzle: chunk c of token t at slot c ^ swz(t)
+  __device__ static __forceinline__ int swz(int t) {
+    if (D == 64) return (((t >> 1) & 1) << 2) | ((t >> 2) & 3);
+    return ((t & 3) << 2) | ((t >> 2) & 3);
+  }
+};
+
+// Workgroup -> (sequence block slot bx, batch x head index bh). Workgroup ids are dealt round-robin over the 8 XCDs, so
+// id & 7 is the XCD: every (batch, head) pair is given to one XCD. With paired blocks (gridDim.x = nx / 2, equal work per
+// workgroup) a pair's workgroups are consecutive on their XCD; with one block per workgroup (gridDim.x = nx) the order on
+// an XCD is slot-major - the heaviest block of each of its pairs first, then the next heaviest of each - which is
+// longest-first scheduling of the unequal causal work, and the blocks of one pair that run together stream the same
+// K/V (Q/dO) tiles at the same time.
+__device__ __forceinline__ void xcd_block(int nx, int nbh, int& bx, int& bh) {
+  const int gx = gridDim.x, lin = blockIdx.y * gx + blockIdx.x;
+  if (nbh % 8 == 0) {
+    const int xcd = lin & 7, idx = lin >> 3;
+    if (gx == nx) {
+      const int per = nbh >> 3;
+      bx = idx / per;
+      bh = xcd + 8 * (idx % per);
+    } else {
+      bh = xcd + 8 * (idx / gx);
+      bx = idx % gx;
+    }
+  } else {
+    bh = blockIdx.y;
+    bx = blockIdx.x;
+  }
+}
+__device__ __forceinline__ int paired_passes(int nx) { return (int)gridDim.x * 2 == nx ? 2 : 1; }
+__device__ __forceinline__ int paired_block(int nx, int bx, int pass, bool heavy_last) {
+  const int first = heavy_last ? nx - 1 - bx : bx;
+  return pass == 0 ? first : nx - 1 - first;
+}
+// first 64-key tile a 128-token query tile qb sees under a band of nw key tiles; 0 without a band
+__device__ __forceinline__ int band_first_tile(int qb, int nw) { return nw > 0 && qb - nw + 1 > 0 ? 2 * (qb - nw + 1) : 0; }
+// Blocks are paired when the paired grid fills its rounds of resident workgroups to 90 % (or is long enough not to care).
+__host__ inline unsigned paired_grid(int nx, int nbh, int per_cu) {
+  if (nx % 2) return (unsigned)nx;
+  const long wgs = (long)(nx / 2) * nbh, slots = tfb_resident_slots(per_cu), rounds = (wgs + slots - 1) / slots;
+  return (unsigned)(wgs * 10 >= rounds * slots * 9 ? nx / 2 : nx);
+}
+
+// This wavefront's share of a (16 NI TPI / 4 ...)-token tile load: instructions g = wave + 4 i, i < NI, each TPI tokens.
+template <int D, int NI>
+struct TileLoad {
+  typedef Geo<D> G;
+  uint32_t voff;
+  int wave;
+  __device__ __forceinline__ void init(long stride, int wave_, int lane) {
+    wave = wave_;
+    const int lrow = lane / G::LPT;
+    // token = TPI g + lrow with g = wave + 4 i: the swizzle depends on g only through bits that 4 i does not touch
+    const int chunk = (lane % G::LPT) ^ G::swz(G::TPI * wave + lrow);
+    voff = (uint32_t)(lrow * stride + chunk * 16);
+  }
+  __device__ __forceinline__ void issue(const uint8_t* rows, long stride, uint8_t* lds) const {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int g = wave + 4 * i;
+      __builtin_amdgcn_global_load_lds((glb_void_t*)(rows + (long)G::TPI * g * stride + (size_t)voff),
+                                       (lds_void_t*)(lds + g * 1024), 16, 0, 0);
+    }
+  }
+};
+
+// token-major fragment: token = 32 half + (lane & 31), elements 16 s + 8 (lane >> 5) .. + 7
+template <int D>
+__device__ __forceinline__ bf16x8 frag_rows(const uint8_t* tile, int half, int s, int lr, int lh) {
+  const int t = 32 * half + lr;
+  return *(const bf16x8*)(tile + t * Geo<D>::ROWB + (((2 * s + lh) ^ Geo<D>::swz(t)) << 4));
+}
+// transposed fragment: element (MFMA row) 32 dt + (lane & 31); tokens tok0 + 4 lh + {0..3} and tok0 + 8 + 4 lh + {0..3}
+template <int D>
+__device__ __forceinline__ bf16x8 frag_cols(const uint8_t* tile, int dt, int tok0, int lane) {
+  typedef Geo<D> G;
+  const int g4 = lane >> 4, j = lane & 15;
+  const int d = 32 * dt + 16 * (g4 & 1) + 4 * (j & 3);
+  const int t = tok0 + 4 * (g4 >> 1) + (j >> 2);
+  const int off0 = t * G::ROWB + (((d >> 3) ^ G::swz(t)) << 4) + ((d & 4) << 1);
+  const int off1 = (t + 8) * G::ROWB + (((d >> 3) ^ G::swz(t + 8)) << 4) + ((d & 4) << 1);
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(tile + off0));
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(tile + off1));
+  const s16x8 v = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+// One token's gradient row from the NDT accumulators a lane holds (elements 32 dt + 8 j + 4 lh + i), scaled and rounded
+// once to bf16.
+template <int D>
+__device__ __forceinline__ void store_grad_row(const f32x16 (&acc)[Geo<D>::NDT], float scale, bf16_t* row, int lh) {
+#pragma unroll
+  for (int dt = 0; dt < Geo<D>::NDT; ++dt)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      u32x2 w = {pack2bf(acc[dt][4 * j] * scale, acc[dt][4 * j + 1] * scale),
+                 pack2bf(acc[dt][4 * j + 2] * scale, acc[dt][4 * j + 3] * scale)};
+      *(u32x2*)(row + 32 * dt + 8 * j + 4 * lh) = w;
+    }
+}
+
+// =========================================================================================== forward
+template <int D>
+__global__ __launch_bounds__(256, 2) void attnT_fwd_kernel(AttnT q, AttnT k, AttnT v, AttnT o, float* __restrict__ lse, int T,
+                                                           int H, float sl2, int nw) {
+  typedef Geo<D> G;
+  constexpr int TILE = G::TILE, NKS = G::NKS, NDT = G::NDT;
+  __shared__ __attribute__((aligned(1024))) uint8_t st0[2 * TILE];
+  __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
+  const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int bx, bh;
+  xcd_block(T / 128, gridDim.y, bx, bh);
+  const int b = bh / H, h = bh % H;
+  const bf16_t* qp = q.p + b * q.sb + h * q.sh;
+  const uint8_t* kp = (const uint8_t*)(k.p + b * k.sb + h * k.sh);
+  const uint8_t* vp = (const uint8_t*)(v.p + b * v.sb + h * v.sh);
+  bf16_t* op = o.p + b * o.sb + h * o.sh;
+  const int nx = T / 128, npass = paired_passes(nx);
+  const long kst = k.st * 2, vst = v.st * 2;
+  TileLoad<D, 16 / G::TPI> lk, lv;
+  lk.init(kst, wave, lane);
+  lv.init(vst, wave, lane);
+  auto issue = [&](uint8_t* st, int tile) {
+    lk.issue(kp + (long)tile * 64 * kst, kst, st);
+    lv.issue(vp + (long)tile * 64 * vst, vst, st + TILE);
+  };
+  for (int pass = 0; pass < npass; ++pass) {
+    const int qb = paired_block(nx, bx, pass, true);
+    const int q0 = qb * 128, qw0 = q0 + wave * 32;
+    bf16x8 qf[NKS];
+#pragma unroll
+    for (int s = 0; s < NKS; ++s) qf[s] = *(const bf16x8*)(qp + (long)(qw0 + lr) * q.st + 16 * s + 8 * lh);
+    f32x16 oacc[NDT];
+    float m = -1e30f, l = 0.f;  // running maximum of the raw scores, running sum
+#pragma unroll
+    for (int i = 0; i < NDT; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) oacc[i][e] = 0.f;
+
+    // one 64-key tile against the wavefront's 32 queries
+    auto tile_step = [&](const uint8_t* st, int tile) {
+      const int k0 = tile * 64;
+      if (k0 > qw0 + 31) return;  // every key in this wavefront's future
+      f32x16 sc[2];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sc[kt][e] = 0.f;
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) sc[kt] = mfma_bf16(frag_rows<D>(st, kt, s, lr, lh), qf[s], sc[kt]);
+      }
+      if (k0 + 63 > qw0) {  // wavefront-uniform; the per-element masking is branch-free selects
+        const int kbase = k0 + lh * 4 - (qw0 + lr);  // key - q for element (kt, e) is kbase + kt*32 + (e>>2)*8 + (e&3)
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) sc[kt][e] = (kbase + kt * 32 + (e >> 2) * 8 + (e & 3) > 0) ? -INFINITY : sc[kt][e];
+      }
+      float mx = m;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int e = 0; e < 16; e += 2) mx = fmaxf(fmaxf(mx, sc[kt][e]), sc[kt][e + 1]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      // the reference point of the exponentials follows the running maximum only when some row's maximum has grown by more
+      // than 2^8: O and lse do not depend on it
+      if (__builtin_amdgcn_ballot_w64((mx - m) * sl2 > 8.0f)) {
+        const float alpha = fast_exp2((m - mx) * sl2);
+        m = mx;
+        l *= alpha;
+#pragma unroll
+        for (int i = 0; i < NDT; ++i)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) oacc[i][e] *= alpha;
+      }
+      const float negm = -m * sl2;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          uint32_t pw[4];
+#pragma unroll
+          for (int x = 0; x < 4; ++x) {
+            const int e = 8 * hf + 2 * x;
+            const float p0 = fast_exp2(fmaf(sc[kt][e], sl2, negm)), p1 = fast_exp2(fmaf(sc[kt][e + 1], sl2, negm));
+            pw[x] = pack2bf(p0, p1);
+            l = sum2bf(pw[x], l);
+          }
+          const bf16x8 bb = frag_from(pw[0], pw[1], pw[2], pw[3]);
+#pragma unroll
+          for (int dt = 0; dt < NDT; ++dt) oacc[dt] = mfma_bf16(frag_cols<D>(st + TILE, dt, kt * 32 + 16 * hf, lane), bb, oacc[dt]);
+        }
+    };
+
+    const int n = (q0 + 128) / 64;           // even; tiles n - 2 and n - 1 cover the workgroup's own 128 tokens
+    const int t0 = band_first_tile(qb, nw);  // even
+    issue(st0, t0);
+    wait_all_loads();
+    __syncthreads();
+    for (int t = t0; t < n; t += 2) {
+      issue(st1, t + 1);
+      tile_step(st0, t);
+      __syncthreads();
+      if (t + 2 < n) issue(st0, t + 2);
+      tile_step(st1, t + 1);
+      __syncthreads();
+    }
+
+    const int myq = qw0 + lr;
+    const float lt = l + __shfl_xor(l, 32, 64);
+    const float inv = 1.0f / lt;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = dt * 32 + 8 * j + 4 * lh;
+        u32x2 w = {pack2bf(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
+                   pack2bf(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv)};
+        *(u32x2*)(op + (long)myq * o.st + d) = w;
+      }
+    if (lh == 0) lse[(long)bh * T + myq] = (m * sl2 + log2f(lt)) * LN2;  // m is the raw-score maximum
+  }
+}
+
+// =========================================================================================== dQ
+template <int D>
+__global__ __launch_bounds__(256, 2) void attnT_dq_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dq,
+                                                                        float* __restrict__ stats, long rows, int T, int H,
+                                                                        float scale, float sl2, int nw, AttnT o,
+                                                                        const float* __restrict__ lse) {
+  typedef Geo<D> G;
+  constexpr int TILE = G::TILE, NKS = G::NKS, NDT = G::NDT;
+  __shared__ __attribute__((aligned(1024))) uint8_t st0[2 * TILE];
+  __shared__ __attribute__((aligned(1024))) uint8_t st1[2 * TILE];
+  const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int bx, bh;
+  xcd_block(T / 128, gridDim.y, bx, bh);
+  const int b = bh / H, h = bh % H;
+  const bf16_t* qp = q.p + b * q.sb + h * q.sh;
+  const bf16_t* gp = go.p + b * go.sb + h * go.sh;
+  const uint8_t* kp = (const uint8_t*)(k.p + b * k.sb + h * k.sh);
+  const uint8_t* vp = (const uint8_t*)(v.p + b * v.sb + h * v.sh);
+  const int nx = T / 128, npass = paired_passes(nx);
+  const long kst = k.st * 2, vst = v.st * 2;
+  TileLoad<D, 16 / G::TPI> lk, lv;
+  lk.init(kst, wave, lane);
+  lv.init(vst, wave, lane);
+  auto issue = [&](uint8_t* st, int tile) {
+    lk.issue(kp + (long)tile * 64 * kst, kst, st);
+    lv.issue(vp + (long)tile * 64 * vst, vst, st + TILE);
+  };
+  for (int pass = 0; pass < npass; ++pass) {
+    const int qb = paired_block(nx, bx, pass, true);
+    const int q0 = qb * 128, qw0 = q0 + wave * 32, myq = qw0 + lr;
+    bf16x8 qf[NKS], gf[NKS];
+#pragma unroll
+    for (int s = 0; s < NKS; ++s) {
+      qf[s] = *(const bf16x8*)(qp + (long)myq * q.st + 16 * s + 8 * lh);
+      gf[s] = *(const bf16x8*)(gp + (long)myq * go.st + 16 * s + 8 * lh);
+    }
+    // the row statistics of this wavefront's queries, made here (this kernel runs first) and left for dK/dV:
+    // -sum_d dO O and -lse / scale
+    float myD, myL;
+    {
+      const bf16_t* orow = o.p + b * o.sb + h * o.sh + (long)myq * o.st;
+      float dot = 0.f;
+#pragma unroll
+      for (int s = 0; s < NKS; ++s) {
+        const u32x4 ov = *(const u32x4*)(orow + 16 * s + 8 * lh);
+        const u32x4 gv = __builtin_bit_cast(u32x4, gf[s]);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          dot += bflo(ov[w]) * bflo(gv[w]);
+          dot += bfhi(ov[w]) * bfhi(gv[w]);
+        }
+      }
+      dot += __shfl_xor(dot, 32, 64);
+      myD = -dot;
+      myL = -lse[(long)bh * T + myq] * (1.0f / scale);
+    }
+    f32x16 dqa[NDT];
+#pragma unroll
+    for (int i = 0; i < NDT; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) dqa[i][e] = 0.f;
+
+    auto tile_step = [&](const uint8_t* st, int tile) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        const int klo = tile * 64 + kt * 32;
+        if (klo > qw0 + 31) continue;
+        f32x16 S, dP;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          S[e] = myL;
+          dP[e] = myD;
+        }
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) S = mfma_bf16(frag_rows<D>(st, kt, s, lr, lh), qf[s], S);
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) dP = mfma_bf16(frag_rows<D>(st + TILE, kt, s, lr, lh), gf[s], dP);
+        if (klo + 31 > qw0) {
+          const int kbase = klo + lh * 4 - myq;
+#pragma unroll
+          for (int e = 0; e < 16; ++e) S[e] = (kbase + (e >> 2) * 8 + (e & 3) > 0) ? -INFINITY : S[e];
+        }
+        uint32_t dsw[8];
+#pragma unroll
+        for (int e = 0; e < 16; e += 2) {
+          const float p0 = fast_exp2(S[e] * sl2), p1 = fast_exp2(S[e + 1] * sl2);
+          const uint32_t w = pack2bf(p0, p1);  // the reference multiplies dP - delta by the rounded P
+          dsw[e >> 1] = pack2bf(bflo(w) * dP[e], bfhi(w) * dP[e + 1]);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          const bf16x8 db = frag_from(dsw[4 * ks], dsw[4 * ks + 1], dsw[4 * ks + 2], dsw[4 * ks + 3]);
+#pragma unroll
+          for (int dt = 0; dt < NDT; ++dt) dqa[dt] = mfma_bf16(frag_cols<D>(st, dt, kt * 32 + 16 * ks, lane), db, dqa[dt]);
+        }
+      }
+    };
+
+    const int n = (q0 + 128) / 64;
+    const int t0 = band_first_tile(qb, nw);
+    issue(st0, t0);
+    wait_all_loads();
+    __syncthreads();
+    for (int t = t0; t < n; t += 2) {
+      issue(st1, t + 1);
+      tile_step(st0, t);
+      __syncthreads();
+      if (t + 2 < n) issue(st0, t + 2);
+      tile_step(st1, t + 1);
+      __syncthreads();
+    }
+    bf16_t* dqp = dq.p + b * dq.sb + h * dq.sh + (long)myq * dq.st;
+    store_grad_row<D>(dqa, scale, dqp, lh);
+    if (lh == 0) {
+      stats[(long)bh * T + myq] = myD;
+      stats[rows + (long)bh * T + myq] = myL;
+    }
+  }
+}
+
+// =========================================================================================== dK / dV
+template <int D, int R>  // R: queries per LDS stage (64 or 128)
+__global__ __launch_bounds__(256, D == 64 ? 2 : TFB_DKDV128_WPE) void attnT_dkdv_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dk, AttnT dv,
+                                                                          const float* __restrict__ stats, long rows, int T,
+                                                                          int H, float scale, float sl2, int nw) {
+  typedef Geo<D> G;
+  constexpr int NKS = G::NKS, NDT = G::NDT;
+  constexpr int RT = R * G::ROWB;           // bytes of a staged Q (dO) tile
+  constexpr int RPB = 128 / R;              // stages per 128-token query tile
+  constexpr int STAGE = 2 * RT + 8 * R;     // Q tile, dO tile, R x (-lse / scale), R x (-delta)
+  __shared__ __attribute__((aligned(1024))) uint8_t st0[STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t st1[STAGE];
+  const int tid = threadIdx.x, lane = tid & 63, lr = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int bx, bh;
+  xcd_block(T / 128, gridDim.y, bx, bh);
+  const int b = bh / H, h = bh % H;
+  const uint8_t* qp = (const uint8_t*)(q.p + b * q.sb + h * q.sh);
+  const uint8_t* gp = (const uint8_t*)(go.p + b * go.sb + h * go.sh);
+  const bf16_t* kp = k.p + b * k.sb + h * k.sh;
+  const bf16_t* vp = v.p + b * v.sb + h * v.sh;
+  const float* delp = stats + (long)bh * T;
+  const float* nlp = stats + rows + (long)bh * T;
+  const int nx = T / 128, npass = paired_passes(nx);
+  const long qst = q.st * 2, gst = go.st * 2;
+  TileLoad<D, R / 4 / G::TPI> lq, lg;
+  lq.init(qst, wave, lane);
+  lg.init(gst, wave, lane);
+  for (int pass = 0; pass < npass; ++pass) {
+    const int kb = paired_block(nx, bx, pass, false);  // low key blocks see the most query tiles
+    const int kw0 = kb * 128 + wave * 32, mykey = kw0 + lr;
+    bf16x8 kf[NKS], vf[NKS];
+#pragma unroll
+    for (int s = 0; s < NKS; ++s) {
+      kf[s] = *(const bf16x8*)(kp + (long)mykey * k.st + 16 * s + 8 * lh);
+      vf[s] = *(const bf16x8*)(vp + (long)mykey * v.st + 16 * s + 8 * lh);
+    }
+    // with a band the keys of tile kb are seen by the queries of tiles kb .. kb + nw - 1 only
+    const int nall = nx - kb, n = RPB * (nw > 0 && nw < nall ? nw : nall);
+    auto issue = [&](uint8_t* st, int i) {
+      const long r0 = (long)kb * 128 + (long)i * R;
+      lq.issue(qp + r0 * qst, qst, st);
+      lg.issue(gp + r0 * gst, gst, st + RT);
+      // the row statistics: R floats each, 4-byte loads (wavefront 0: -lse / scale, wavefront 1: -delta)
+      if (wave < 2) {
+        const float* src = (wave == 0 ? nlp : delp) + r0;
+#pragma unroll
+        for (int x = 0; x < R / 64; ++x)
+          __builtin_amdgcn_global_load_lds((glb_void_t*)(src + 64 * x + lane), (lds_void_t*)(st + 2 * RT + wave * 4 * R + 256 * x),
+                                           4, 0, 0);
+      }
+    };
+    f32x16 dka[NDT], dva[NDT];
+#pragma unroll
+    for (int i = 0; i < NDT; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        dka[i][e] = 0.f;
+        dva[i][e] = 0.f;
+      }
+
+    auto compute = [&](const uint8_t* st, int i) {
+      const uint8_t* qt_ = st;
+      const uint8_t* gt_ = st + RT;
+      const float* ls = (const float*)(st + 2 * RT);
+      const int qbase = kb * 128 + i * R;
+#pragma unroll
+      for (int qs = 0; qs < R / 32; ++qs) {
+        const int qlo = qbase + qs * 32;
+        if (qlo + 31 < kw0) continue;  // every key of this wavefront is in the future of these queries
+        // the accumulators start from the rows' -lse / scale and -delta
+        f32x16 S, dP;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const f32x4 L = *(const f32x4*)(ls + qs * 32 + 8 * j + 4 * lh);
+          const f32x4 Dl = *(const f32x4*)(ls + R + qs * 32 + 8 * j + 4 * lh);
+#pragma unroll
+          for (int x = 0; x < 4; ++x) {
+            S[4 * j + x] = L[x];
+            dP[4 * j + x] = Dl[x];
+          }
+        }
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) S = mfma_bf16(frag_rows<D>(qt_, qs, s, lr, lh), kf[s], S);
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) dP = mfma_bf16(frag_rows<D>(gt_, qs, s, lr, lh), vf[s], dP);
+        const int kq = mykey - (qlo + 4 * lh);  // key - q for element e is kq - (e>>2)*8 - (e&3)
+        if (kw0 + 31 > qlo) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) S[e] = (kq - 8 * (e >> 2) - (e & 3) > 0) ? -INFINITY : S[e];
+        }
+        uint32_t pw[8], dsw[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float p[4];
+#pragma unroll
+          for (int x = 0; x < 4; ++x) p[x] = fast_exp2(S[4 * j + x] * sl2);
+          const uint32_t w0 = pack2bf(p[0], p[1]), w1 = pack2bf(p[2], p[3]);
+          pw[2 * j] = w0;
+          pw[2 * j + 1] = w1;
+          dsw[2 * j] = pack2bf(bflo(w0) * dP[4 * j], bfhi(w0) * dP[4 * j + 1]);
+          dsw[2 * j + 1] = pack2bf(bflo(w1) * dP[4 * j + 2], bfhi(w1) * dP[4 * j + 3]);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          const bf16x8 pb = frag_from(pw[4 * ks], pw[4 * ks + 1], pw[4 * ks + 2], pw[4 * ks + 3]);
+          const bf16x8 db = frag_from(dsw[4 * ks], dsw[4 * ks + 1], dsw[4 * ks + 2], dsw[4 * ks + 3]);
+#pragma unroll
+          for (int dt = 0; dt < NDT; ++dt) {
+            dva[dt] = mfma_bf16(frag_cols<D>(gt_, dt, qs * 32 + 16 * ks, lane), pb, dva[dt]);
+            dka[dt] = mfma_bf16(frag_cols<D>(qt_, dt, qs * 32 + 16 * ks, lane), db, dka[dt]);
+          }
+        }
+      }
+    };
+
+    issue(st0, 0);
+    wait_all_loads();
+    __syncthreads();
+    for (int t = 0; t + 2 <= n; t += 2) {
+      issue(st1, t + 1);
+      compute(st0, t);
+      __syncthreads();
+      if (t + 2 < n) issue(st0, t + 2);
+      compute(st1, t + 1);
+      __syncthreads();
+    }
+    if (n & 1) compute(st0, n - 1);
+    __syncthreads();  // the stages are free for the partner block
+
+    bf16_t* dkp = dk.p + b * dk.sb + h * dk.sh + (long)mykey * dk.st;
+    bf16_t* dvp = dv.p + b * dv.sb + h * dv.sh + (long)mykey * dv.st;
+    store_grad_row<D>(dka, scale, dkp, lh);
+    store_grad_row<D>(dva, 1.0f, dvp, lh);
+  }
+}
+
+AttnT mk(const void* p, const long* s) { return AttnT{(bf16_t*)p, s[0], s[1], s[2]}; }
+
+template <int D>
+int fwd_launch(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs, void* o,
+               const long* os, float* lse, int B, int H, int T, float scale, int nw, hipStream_t s) {
+  hipLaunchKernelGGL(attnT_fwd_kernel<D>, dim3(paired_grid(T / 128, B * H, 2), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs),
+                     mk(o, os), lse, T, H, scale * LOG2E, nw);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+template <int D>
+int bwd_launch(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs, const void* o,
+               const long* os, const void* go, const long* gos, void* dq, const long* dqs, void* dk, const long* dks, void* dv,
+               const long* dvs, const float* lse, float* stats, int B, int H, int T, float scale, int nw, hipStream_t s) {
+  const long rows = (long)B * H * T;
+  hipLaunchKernelGGL(attnT_dq_kernel<D>, dim3(paired_grid(T / 128, B * H, 2), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs),
+                     mk(go, gos), mk(dq, dqs), stats, rows, T, H, scale, scale * LOG2E, nw, mk(o, os), lse);
+  TFB_LAUNCH_CHECK();
+  hipLaunchKernelGGL((attnT_dkdv_kernel<D, TFB_DKDV128_R>), dim3(paired_grid(T / 128, B * H, D == 64 ? 2 : TFB_DKDV128_WPE), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs),
+                     mk(go, gos), mk(dk, dks), mk(dv, dvs), stats, rows, T, H, scale, scale * LOG2E, nw);
+  TFB_LAUNCH_CHECK();
+  return TFB_OK;
+}
+
+}  // namespace
+
+// Called by tfb_attn_fwd / tfb_attn_bwd for D = 128 (arguments validated there: T % 128 == 0, strides % 8 == 0).
+int tfb_attn128_fwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
+                       void* o, const long* os, float* lse, int B, int H, int T, float scale, int nw, hipStream_t s) {
+  return fwd_launch<128>(q, qs, k, ks, v, vs, o, os, lse, B, H, T, scale, nw, s);
+}
+// stats: fp32 [2][B*H][T] scratch (-delta, then -lse / scale), written by the dQ kernel and read by dK/dV.
+int tfb_attn128_bwd_impl(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs,
+                       const void* o, const long* os, const void* go, const long* gos, void* dq, const long* dqs, void* dk,
+                       const long* dks, void* dv, const long* dvs, const float* lse, float* stats, int B, int H, int T,
+                       float scale, int nw, hipStream_t s) {
+  return bwd_launch<128>(q, qs, k, ks, v, vs, o, os, go, gos, dq, dqs, dk, dks, dv, dvs, lse, stats, B, H, T, scale, nw, s);
+}
