@@ -647,6 +647,29 @@ def test_gemm_long_contraction_in_every_operand_layout(ops, dev, ta, tb):
             assert rel_l2(got[:512], 0.5 * ref + acc[:512]) < 1e-4
 
 
+@pytest.mark.parametrize("shape", [(2304, 768, 8192), (768, 768, 32768), (768, 3072, 16384), (1024, 512, 20480)])
+def test_gemm_long_contraction_over_few_tiles(ops, dev, shape):
+    """Weight-gradient shapes: a token contraction of at least 128 k-tiles over fewer than 64 output tiles of 256 x 256 runs the
+    persistent kernel with one k range per workgroup (27 tiles: 8 ranges; 9 tiles: 24 uneven ranges of 21 or 22 k-tiles; 36
+    tiles: 7 ranges; 8 tiles: 32 ranges of 10 k-tiles are too short, so fewer), the partial tiles summed through the fp32
+    workspace: against the fp32 product of the same bf16 values, fresh, accumulated into an fp32 buffer, and scaled."""
+    M, N, K = shape
+    g = _g(M + 3 * N + K)
+    a = torch.randn(K, M, generator=g).bfloat16()
+    b = torch.randn(K, N, generator=g).bfloat16()
+    ad, bd = a.to(dev), b.to(dev)
+    ref = (ad.float().t() @ bd.float()).cpu()
+    c = ops.matmul(ad, bd, trans_a=True)
+    assert rel_l2(c, ref) < BF16_TOL
+    acc = torch.randn(M, N, generator=g)
+    al = torch.tensor([0.25], device=dev)
+    got = ops.matmul(ad, bd, trans_a=True, out=acc.to(dev).clone(), accumulate=True, alpha=al)
+    assert rel_l2(got, 0.25 * ref + acc) < 1e-4
+    # the other operand order of the same contraction (k-strided P against k-contiguous Q)
+    c2 = ops.matmul(ad, bd.t().contiguous(), trans_a=True, trans_b=True)
+    assert rel_l2(c2, ref) < BF16_TOL
+
+
 @pytest.mark.parametrize("shape", [(2048, 1024, 1024, 128), (512, 4096, 1536, 128), (8192, 256, 1984, 128)])
 def test_gemm_256_tile_kernel_equals_the_128_tile_kernel(ops, dev, shape):
     """A product large enough for the persistent 256 x 256 kernel (both operands k-contiguous, 16 to 31 k-tiles: long enough

@@ -11,20 +11,30 @@ template <int LAYP, int LAYQ>
 int run(GemmOperand P, GemmOperand Q, int N, int M, int K, void* C, int out_f32, int accumulate, float* ws, long ws_bytes,
         const float* alpha, hipStream_t stream) {
   using Cfg = GemmCfg<128, 128, 2, 2, 2, LAYP, LAYQ>;
-  // Long contractions (at least 128 k-tiles) over at least 64 output tiles of 256 x 256, in any operand layout: the
-  // persistent 256 x 256 kernel, the k range cut into the fewest equal parts that fill whole rounds of the CUs to 90 %
-  // (the LM head's two gradient GEMMs: 384 tiles x 2 = 3 per CU), partial tiles through the fp32 workspace.
+  // Long contractions (at least 128 k-tiles) in any operand layout: the persistent 256 x 256 kernel, partial tiles through
+  // the fp32 workspace. With 64 or more output tiles the k range is cut into the fewest parts that fill whole rounds of
+  // the CUs to 90 % (the LM head's two gradient GEMMs: 384 tiles x 2 = 3 per CU). With fewer (the layers' weight
+  // gradients: 9 to 27 tiles of 512 k-tiles) every workgroup gets one work item: as many k ranges per XCD as its 32 CUs
+  // have room for tiles, so that an XCD's workgroups read one k range of the operands together (27 tiles: 8 ranges,
+  // 9 tiles: 24), or, from 33 tiles, the number of ranges that fills the CUs.
 #ifndef TFB_PP_LONGK
 #define TFB_PP_LONGK 1
 #endif
-  if (TFB_PP && TFB_PP_LONGK && N % 256 == 0 && M % 256 == 0 && K % 64 == 0 && K / 64 >= 128 && (long)(N / 256) * (M / 256) >= 64) {
+#ifndef TFB_PP_FEWTILE
+#define TFB_PP_FEWTILE 1
+#endif
+  if (TFB_PP && TFB_PP_LONGK && N % 256 == 0 && M % 256 == 0 && K % 64 == 0 && K / 64 >= 128) {
     const long t256 = (long)(N / 256) * (M / 256), nkt = K / 64, cus = tfb_resident_slots(1);
     int sp = 0;
-    for (int c = 1; c <= 8 && !sp; ++c) {
-      if (nkt % c || nkt / c < 32) continue;
-      if (c > 1 && (!ws || (long)c * M * N * 4 > ws_bytes)) continue;
-      const long items = t256 * c, rounds = (items + cus - 1) / cus;
-      if ((double)items >= 0.9 * (double)(rounds * cus)) sp = c;
+    if (t256 >= 64) {
+      for (int c = 1; c <= 8 && !sp; ++c) {
+        if (nkt / c < 32) continue;
+        if (c > 1 && (!ws || (long)c * M * N * 4 > ws_bytes)) continue;
+        const long items = t256 * c, rounds = (items + cus - 1) / cus;
+        if ((double)items >= 0.9 * (double)(rounds * cus)) sp = c;
+      }
+    } else if (ws && TFB_PP_FEWTILE) {
+      sp = gemm_pp_fewtile_splits(t256, nkt, (long)M * N, ws_bytes);
     }
     if (sp == 1 && !out_f32 && !accumulate) {
       EpiStore e{C, (long)N, out_f32, accumulate, alpha};

@@ -21,7 +21,9 @@
 // ([rows][K]) keeps row r of a half at r * 128, 16-byte chunk c at slot c ^ tfb_kc_swz(r) (no bank conflicts for the 128-bit
 // fragment reads). A k-strided bf16 operand ([K][rows], the token-contraction GEMMs) keeps one k per 256-byte LDS row,
 // chunk c of k-row k at slot c ^ (4 (k & 3)), and its fragments come through ds_read_b64_tr_b16 (two per fragment), the
-// layout and lane map of the 128 x 128 kernel's K_STRIDED reader.
+// layout and lane map of the 128 x 128 kernel's K_STRIDED reader. A k-strided fp8 operand keeps one k per 128-byte LDS row
+// (128 k-rows per quarter), chunk c of k-row k at slot c ^ (2 ((k >> 1) & 3)), fragments through ds_read_b64_tr_b8 (four
+// per 64-k fragment).
 //
 // Long contractions with few output tiles (the LM head's gradients: 384 tiles of 512 k-tiles) are split along k into
 // work items of equal length; each leaves its fp32 partial tile in a workspace (epilogues with kSplitF32, staged as
@@ -48,10 +50,12 @@ __device__ __forceinline__ T tfb_lds_read128(uint32_t addr) {
 
 struct PpArgs {
   GemmOperand P, Q;
-  int nkt;      // k-tiles per work item (>= 2): all of k, or one of `splits` equal parts
+  int nk_total; // k-tiles of the contraction; split s of `splits` takes [s nk / splits, (s + 1) nk / splits), >= 2 each
   int ntiles;   // work items = output tiles * splits (item w: split w / nout, output tile w % nout)
   int nout;     // output tiles
   int splits;
+  int ipx;      // > 0 (few output tiles, one work item per workgroup): XCD x (= workgroup & 7) takes the ipx consecutive
+                // work items from x * ipx, so that an XCD's workgroups share one or two k ranges of the operands in its L2
   FastDiv d_nout;
   int nwg;      // workgroups launched (a multiple of 8 when rect)
   int p_fast;   // the fast-walking operand is P
@@ -87,6 +91,13 @@ __device__ __forceinline__ tfb_s16x4 tfb_lds_read_tr64(uint32_t addr) {
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
   return v;
 }
+typedef int tfb_pp_i32x2 __attribute__((ext_vector_type(2)));
+template <int OFF>
+__device__ __forceinline__ tfb_pp_i32x2 tfb_lds_read_tr64_b8(uint32_t addr) {
+  tfb_pp_i32x2 v;
+  asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
 
 // An epilogue with the static member kSplitF32 receives the raw fp32 accumulators, operator()(p, q, v[8], split): the
 // partial tile of a k-split.
@@ -95,11 +106,10 @@ struct has_split_f32 : std::false_type {};
 template <class T>
 struct has_split_f32<T, std::void_t<decltype(T::kSplitF32)>> : std::true_type {};
 
-// ES: element size (2: bf16, 1: OCP fp8 with FMTP / FMTQ = 0 e4m3, 1 e5m2 per side); LAYP / LAYQ: TFB_K_CONTIG or (bf16
-// only) TFB_K_STRIDED
+// ES: element size (2: bf16, 1: OCP fp8 with FMTP / FMTQ = 0 e4m3, 1 e5m2 per side); LAYP / LAYQ: TFB_K_CONTIG or
+// TFB_K_STRIDED
 template <int ES, int FMTP, int FMTQ, int LAYP, int LAYQ, class Epi>
 __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
-  static_assert(ES == 2 || (LAYP == TFB_K_CONTIG && LAYQ == TFB_K_CONTIG), "k-strided operands are bf16");
   constexpr bool kF32 = has_split_f32<Epi>::value;
 #ifdef PP_DBG
   const unsigned long long c_start = __builtin_readcyclecounter();
@@ -112,12 +122,13 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int wr = wave >> 2, wc = wave & 3;  // wr: the group (wavefronts 0-3 / 4-7 sit on SIMDs 0-3 each)
   const int lr = lane & 31, lh = lane >> 5;
-  const int nkt = a.nkt;
+  int nkt;  // k-tiles of the current work item
   uint8_t* stg = stg_all + wave * 4096;
 
   // ---- operand loads. A quarter is 16 instructions of 1 KB, two per wavefront (g = wave and wave + 8):
   //   k-contiguous: instruction g = rows 8 g .. 8 g + 7 x 128 bytes of k, lane l -> row l / 8, chunk (l % 8) ^ swizzle;
-  //   k-strided:    instruction g = k-rows 4 g .. 4 g + 3 x 128 rows (256 bytes), lane l -> k-row l / 16, chunk (l % 16) ^ 4 (k & 3).
+  //   k-strided:    instruction g = k-rows 4 g .. 4 g + 3 x 128 rows (256 bytes), lane l -> k-row l / 16, chunk (l % 16) ^ 4 (k & 3);
+  //                 fp8: k-rows 8 g .. 8 g + 7 x 128 rows (128 bytes), lane l -> k-row l / 8, chunk (l % 8) ^ 2 ((k >> 1) & 3).
   // Per operand: v = the lane's byte offset, istep = from instruction g to g + 8, hstep = from half 0 to half 1,
   // kstep = from one k-tile to the next, and the byte origin of output tile row-block r0.
   struct Side {
@@ -136,7 +147,7 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
       sd.hstep = 128 * o.ld;
       sd.kstep = 128;
       sd.tstep = o.ld;
-    } else {
+    } else if (ES == 2) {
       const int kl = lane >> 4, slot = lane & 15;
       sd.base = o.base + 4L * wave * o.ld;
       sd.v = (uint32_t)(kl * o.ld + ((slot ^ (4 * kl)) << 4));
@@ -144,6 +155,14 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
       sd.hstep = 256;
       sd.kstep = 64 * o.ld;
       sd.tstep = 2;
+    } else {
+      const int kl = lane >> 3, slot = lane & 7;
+      sd.base = o.base + 8L * wave * o.ld;
+      sd.v = (uint32_t)(kl * o.ld + ((slot ^ (2 * ((kl >> 1) & 3))) << 4));
+      sd.istep = 64 * o.ld;
+      sd.hstep = 128;
+      sd.kstep = 128 * o.ld;
+      sd.tstep = 1;
     }
     return sd;
   };
@@ -173,7 +192,15 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
     p0 = (long)(a.p_fast ? fast : slow) * 256;
     q0 = (long)(a.p_fast ? slow : fast) * 256;
   };
-  auto origin = [&](const Side& sd, long r0, int split) { return sd.base + r0 * sd.tstep + (long)split * nkt * sd.kstep; };
+  auto krange = [&](int split, int& k0, int& n) {
+    k0 = 0;
+    n = a.nk_total;
+    if (a.splits > 1) {
+      k0 = (int)((long)split * a.nk_total / a.splits);
+      n = (int)((long)(split + 1) * a.nk_total / a.splits) - k0;
+    }
+  };
+  auto origin = [&](const Side& sd, long r0, int k0) { return sd.base + r0 * sd.tstep + (long)k0 * sd.kstep; };
 
   // quarter (X: 0 P, 1 Q; half h) of stage S <- the k-tile at g (the side's address of that k-tile of the output tile)
   auto dma = [&](int S, int X, int h, const uint8_t* g) {
@@ -203,9 +230,15 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
     // the second tile's chunk index differs in bit 2, which the swizzle also touches, so it is not an immediate offset);
     // k-step s is 16 k-rows further (an immediate), the fragment's upper four k another 4 k-rows.
     const int g4 = lane >> 4, j = lane & 15, kq = j >> 2;
+    // fp8: lane j of the group points at k-row j / 2 (of eight consecutive k), rows 8 (j % 2) .. + 7; the group's k-half
+    // is 32 k-rows further, a k-step 64, the fragment's next eight k 8 (immediates).
     auto tr_addr = [&](int row0) {
-      const int p = row0 + 16 * (g4 & 1) + 4 * (j & 3);
-      return (uint32_t)((8 * (g4 >> 1) + kq) * 256 + ((((p >> 3) ^ (4 * kq)) << 4) | ((p & 4) << 1)));
+      if (ES == 2) {
+        const int p = row0 + 16 * (g4 & 1) + 4 * (j & 3);
+        return (uint32_t)((8 * (g4 >> 1) + kq) * 256 + ((((p >> 3) ^ (4 * kq)) << 4) | ((p & 4) << 1)));
+      }
+      const int p = row0 + 16 * (g4 & 1) + 8 * (j & 1), k8 = j >> 1;
+      return (uint32_t)((32 * (g4 >> 1) + k8) * 128 + ((((p >> 4) ^ (2 * ((k8 >> 1) & 3))) << 4) | (p & 8)));
     };
     if (LAYP == TFB_K_STRIDED) {
       ap[0] = lbase + tr_addr(wr * 64);
@@ -221,10 +254,17 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
   r128_t fa[2][4], fb0[4], fb1[4];
   auto tr_frag = [&](auto OFF, uint32_t addr) {
     constexpr int off = decltype(OFF)::value;
-    const tfb_s16x4 lo = tfb_lds_read_tr64<off>(addr), hi = tfb_lds_read_tr64<off + 1024>(addr);
-    const tfb_s16x8 v = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    return __builtin_bit_cast(r128_t, v);
+    if constexpr (ES == 2) {  // k-step off / 4096: 16 k-rows of 256 bytes; the upper four k 4 rows further
+      const tfb_s16x4 lo = tfb_lds_read_tr64<off>(addr), hi = tfb_lds_read_tr64<off + 1024>(addr);
+      const tfb_s16x8 v = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      return __builtin_bit_cast(r128_t, v);
+    } else {  // half a 64-k fragment: 16 k of a row, two reads 8 k-rows (1 KB) apart
+      const tfb_pp_i32x2 lo = tfb_lds_read_tr64_b8<off>(addr), hi = tfb_lds_read_tr64_b8<off + 1024>(addr);
+      return r128_t{lo.x, lo.y, hi.x, hi.y};
+    }
   };
+  // fragment entry e (bf16: k-step e of 16 k; fp8: half e & 1 of k-step e >> 1 of 64 k) -> byte offset in a quarter
+  constexpr int TR1 = ES == 2 ? 4096 : 2048, TR2 = 8192, TR3 = ES == 2 ? 12288 : 8192 + 2048;
   auto readA = [&](auto H) __attribute__((always_inline)) {
     constexpr int h = decltype(H)::value;
     if constexpr (LAYP == TFB_K_CONTIG) {
@@ -236,12 +276,12 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
     } else {
       fa[0][0] = tr_frag(std::integral_constant<int, h * 16384>{}, ap[0]);
       fa[1][0] = tr_frag(std::integral_constant<int, h * 16384>{}, ap[1]);
-      fa[0][1] = tr_frag(std::integral_constant<int, h * 16384 + 4096>{}, ap[0]);
-      fa[1][1] = tr_frag(std::integral_constant<int, h * 16384 + 4096>{}, ap[1]);
-      fa[0][2] = tr_frag(std::integral_constant<int, h * 16384 + 8192>{}, ap[0]);
-      fa[1][2] = tr_frag(std::integral_constant<int, h * 16384 + 8192>{}, ap[1]);
-      fa[0][3] = tr_frag(std::integral_constant<int, h * 16384 + 12288>{}, ap[0]);
-      fa[1][3] = tr_frag(std::integral_constant<int, h * 16384 + 12288>{}, ap[1]);
+      fa[0][1] = tr_frag(std::integral_constant<int, h * 16384 + TR1>{}, ap[0]);
+      fa[1][1] = tr_frag(std::integral_constant<int, h * 16384 + TR1>{}, ap[1]);
+      fa[0][2] = tr_frag(std::integral_constant<int, h * 16384 + TR2>{}, ap[0]);
+      fa[1][2] = tr_frag(std::integral_constant<int, h * 16384 + TR2>{}, ap[1]);
+      fa[0][3] = tr_frag(std::integral_constant<int, h * 16384 + TR3>{}, ap[0]);
+      fa[1][3] = tr_frag(std::integral_constant<int, h * 16384 + TR3>{}, ap[1]);
     }
   };
   auto readB = [&](auto H, r128_t(&fb)[4]) __attribute__((always_inline)) {
@@ -251,9 +291,9 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
       for (int s = 0; s < 4; ++s) fb[s] = tfb_lds_read128<h * 16384, r128_t>(aq[s]);
     } else {
       fb[0] = tr_frag(std::integral_constant<int, h * 16384>{}, aq[0]);
-      fb[1] = tr_frag(std::integral_constant<int, h * 16384 + 4096>{}, aq[0]);
-      fb[2] = tr_frag(std::integral_constant<int, h * 16384 + 8192>{}, aq[0]);
-      fb[3] = tr_frag(std::integral_constant<int, h * 16384 + 12288>{}, aq[0]);
+      fb[1] = tr_frag(std::integral_constant<int, h * 16384 + TR1>{}, aq[0]);
+      fb[2] = tr_frag(std::integral_constant<int, h * 16384 + TR2>{}, aq[0]);
+      fb[3] = tr_frag(std::integral_constant<int, h * 16384 + TR3>{}, aq[0]);
     }
   };
   // the fragments pass through the wait as in/out operands, so that no MFMA that reads them is scheduled ahead of it
@@ -307,12 +347,17 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
 
   const Epi epi = epi_prepare(epi_in);
   int w = blockIdx.x;
+  if (a.ipx > 0) {
+    if ((w >> 3) >= a.ipx) return;
+    w = (w & 7) * a.ipx + (w >> 3);
+  }
   if (w >= a.ntiles) return;  // (whole workgroup)
   long p0, q0;
-  int split;
+  int split, k0;
   tile_of(w, p0, q0, split);
-  const uint8_t* gp = origin(sp, p0, split);  // current work item: the sides' addresses of its first k-tile
-  const uint8_t* gq = origin(sq, q0, split);
+  krange(split, k0, nkt);
+  const uint8_t* gp = origin(sp, p0, k0);  // current work item: the sides' addresses of its first k-tile
+  const uint8_t* gq = origin(sq, q0, k0);
 
   // ---- prologue: all of k-tile 0 into stage 0, three quarters of k-tile 1 into stage 1
   dma(0, 1, 0, gq);
@@ -415,12 +460,15 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
   for (;;) {
     // the workgroup's next work item (its first k-tiles are requested by this one's last iterations); past the end: this
     // one again (loads nobody reads, from valid memory)
-    const int wn = w + a.nwg;
+    const int wn = a.ipx > 0 ? a.ntiles : w + a.nwg;
     long pn = p0, qn = q0;
-    int splitn = split;
-    if (wn < a.ntiles) tile_of(wn, pn, qn, splitn);
-    const uint8_t* gpn = origin(sp, pn, splitn);
-    const uint8_t* gqn = origin(sq, qn, splitn);
+    int splitn = split, k0n = k0, nktn = nkt;
+    if (wn < a.ntiles) {
+      tile_of(wn, pn, qn, splitn);
+      krange(splitn, k0n, nktn);
+    }
+    const uint8_t* gpn = origin(sp, pn, k0n);
+    const uint8_t* gqn = origin(sq, qn, k0n);
 
     // One k-tile. In a tile's first iteration the MFMAs start from zero, and each accumulator block of the PREVIOUS tile is
     // stored in the memory cluster in front of the MFMA cluster that overwrites it: the stores of one group (4 KB per
@@ -519,6 +567,8 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
     p0 = pn;
     q0 = qn;
     split = splitn;
+    k0 = k0n;
+    nkt = nktn;
     gp = gpn;
     gq = gqn;
     if constexpr (kF32) {
@@ -558,11 +608,12 @@ static inline bool gemm_pp_applies(long np, long nq, long kbytes) {
   return TFB_PP == 2 || kbytes / 128 >= 16 || tiles >= 4096;
 }
 
-// np, nq multiples of 256; kbytes = the contraction in bytes of a k-contiguous row (elements * ES), a multiple of
-// 128 * splits with at least two k-tiles per split. With splits > 1 the epilogue is one with kSplitF32 (EpiSplit).
+// np, nq multiples of 256; kbytes = the contraction in bytes of a k-contiguous row (elements * ES), a multiple of 128
+// with at least two k-tiles per split. With splits > 1 the epilogue is one with kSplitF32 (EpiSplit); when all work items
+// fit one round of the CUs they are dealt to the XCDs in consecutive runs (PpArgs::ipx).
 template <int ES, int FMTP, int FMTQ, int LAYP, int LAYQ, class Epi>
 static int gemm_pp_launch_lay(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes, int splits, Epi epi, hipStream_t stream) {
-  if (np <= 0 || nq <= 0 || splits <= 0 || np % 256 || nq % 256 || kbytes % (128L * splits) || kbytes / 128 / splits < 2)
+  if (np <= 0 || nq <= 0 || splits <= 0 || np % 256 || nq % 256 || kbytes % 128 || kbytes / 128 / splits < 2)
     return TFB_ERR_SHAPE;
   if (P.ld <= 0 || Q.ld <= 0 || P.ld > (1L << 28) || Q.ld > (1L << 28)) return TFB_ERR_SHAPE;
   if (((uintptr_t)P.base | (uintptr_t)Q.base | (uintptr_t)P.ld | (uintptr_t)Q.ld) & 15) return TFB_ERR_ARG;
@@ -571,7 +622,7 @@ static int gemm_pp_launch_lay(GemmOperand P, GemmOperand Q, int np, int nq, long
   a.P = P;
   a.Q = Q;
   a.splits = splits;
-  a.nkt = (int)(kbytes / 128 / splits);
+  a.nk_total = (int)(kbytes / 128);
   const int ntp = np / 256, ntq = nq / 256;
   if ((long)ntp * ntq * splits >= (1L << 30)) return TFB_ERR_SHAPE;
   a.nout = ntp * ntq;
@@ -582,6 +633,11 @@ static int gemm_pp_launch_lay(GemmOperand P, GemmOperand Q, int np, int nq, long
   const int nslow = a.p_fast ? ntq : ntp;
   a.rect = (nslow % 8 == 0) && a.nout >= 8;
   a.nwg = a.ntiles < cus ? a.ntiles : cus;
+  if (splits > 1 && a.ntiles <= cus) {
+    a.rect = 0;
+    a.ipx = (a.ntiles + 7) / 8;
+    a.nwg = 8 * a.ipx;
+  }
   if (a.rect) a.nwg &= ~7;
   if (a.nwg <= 0) return TFB_ERR_SHAPE;
   a.R = a.rect ? nslow / 8 : 1;
@@ -601,6 +657,18 @@ static int gemm_pp_launch_lay(GemmOperand P, GemmOperand Q, int np, int nq, long
   hipLaunchKernelGGL((gemm_pp_kernel<ES, FMTP, FMTQ, LAYP, LAYQ, Epi>), dim3(a.nwg), dim3(512), 0, stream, a, epi);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
+}
+
+// k ranges for a long contraction (nkt k-tiles) over fewer than 64 output tiles of 256 x 256, one work item per workgroup:
+// up to 32 tiles, as many ranges per XCD as its CUs have room for tiles (an XCD's workgroups then read one k range of the
+// operands together: 27 tiles -> 8 ranges, 9 tiles -> 24); beyond, the count that fills the CUs. 0: not worth it (less
+// than 80 % of the CUs busy, fewer than 16 k-tiles per item, or the partial tiles do not fit the workspace).
+static inline int gemm_pp_fewtile_splits(long t256, long nkt, long out_elems, long ws_bytes) {
+  const long cus = tfb_resident_slots(1);
+  if (t256 <= 0 || t256 >= 64) return 0;
+  int c = t256 * 8 <= cus ? 8 * (int)(cus / 8 / t256) : (int)(cus / t256);
+  while (c > 1 && (nkt / c < 16 || (long)c * out_elems * 4 > ws_bytes)) --c;
+  return (c > 1 && (double)(t256 * c) >= 0.8 * (double)cus) ? c : 0;
 }
 
 // both operands k-contiguous, no k-split

@@ -814,6 +814,22 @@ extern "C" int tfb_gemm_fp8_tn(const void* g8, int fmt_g, const void* a8, int fm
   if (M <= 0 || O <= 0 || D <= 0 || M % 128 || O % 128 || D % 128) return TFB_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   const long n = (long)O * D;
+  // a long contraction over few 256 x 256 tiles (the MLP's weight gradients: 36 tiles of 256 k-tiles): the persistent kernel,
+  // one k range per workgroup
+#ifndef TFB_PP_DW8
+#define TFB_PP_DW8 1
+#endif
+  if (TFB_PP && TFB_PP_DW8 && O % 256 == 0 && D % 256 == 0 && M / 128 >= 128) {
+    const int sp = gemm_pp_fewtile_splits((long)(O / 256) * (D / 256), M / 128, n, workspace_bytes);
+    if (sp > 1) {
+      GemmOperand P{(const uint8_t*)a8, (long)D}, Q{(const uint8_t*)g8, (long)O};
+      EpiSplit e{(float*)workspace, (long)D, n};
+      int st = ga ? gemm_pp_launch_lay<1, TFB_FMT_E4M3, TFB_FMT_E5M2, TFB_K_STRIDED, TFB_K_STRIDED>(P, Q, D, O, M, sp, e, s)
+                  : gemm_pp_launch_lay<1, TFB_FMT_E5M2, TFB_FMT_E4M3, TFB_K_STRIDED, TFB_K_STRIDED>(P, Q, D, O, M, sp, e, s);
+      if (st != TFB_OK) return st;
+      return splitk_reduce((const float*)workspace, out, n, sp, out_f32, accumulate, s, (const float*)s_g, (const float*)s_a, imm);
+    }
+  }
   const int splits = choose_splits(n / (128 * 128), (int)(M / 128), n, workspace_bytes);
   if ((long)splits * n * 4 > workspace_bytes) return TFB_ERR_SHAPE;
   float* ws = (float*)workspace;
