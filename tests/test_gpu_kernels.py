@@ -685,6 +685,11 @@ def test_gemm_256_tile_kernel_equals_the_128_tile_kernel(ops, dev, shape):
     assert torch.equal(c, torch.cat(parts, dim=1))
     ref = a[:256].double() @ b.double().t()
     assert rel_l2(c[:256], ref) < BF16_TOL
+    # the same product with either operand stored k-strided (the transposing LDS reads feed the same sums)
+    at, bt = a.t().contiguous(), b.t().contiguous()
+    assert torch.equal(ops.matmul(at, b, trans_a=True, trans_b=True), c)
+    assert torch.equal(ops.matmul(a, bt), c)
+    assert torch.equal(ops.matmul(at, bt, trans_a=True), c)
     res = torch.randn(M, N, generator=g).bfloat16().to(dev)
     assert torch.equal(ops.matmul_res(a, b, res, trans_b=True), (c.float() + res.float()).bfloat16())
     al = torch.tensor([0.37], device=dev)

@@ -51,9 +51,10 @@ int run(GemmOperand P, GemmOperand Q, int N, int M, int K, void* C, int out_f32,
   const int splits = ws ? choose_splits(tiles, K / 64, (long)M * N, ws_bytes) : 1;
   if (splits == 1) {
     EpiStore e{C, (long)N, out_f32, accumulate, alpha};
-    // large outputs with both operands k-contiguous: the persistent 256 x 256 kernel (same sums in the same order)
-    if (LAYP == TFB_K_CONTIG && LAYQ == TFB_K_CONTIG && !out_f32 && !accumulate && gemm_pp_applies(N, M, (long)K * 2))
-      return gemm_pp_launch<2, 0, 0>(P, Q, N, M, (long)K * 2, e, stream);
+    // large outputs: the persistent 256 x 256 kernel (same sums in the same order), in any operand layout (the input
+    // gradient of the QKV projection, whose weight is read k-strided: 123.6 -> 117.7 us inside the step)
+    if (!out_f32 && !accumulate && gemm_pp_applies(N, M, (long)K * 2))
+      return gemm_pp_launch_lay<2, 0, 0, LAYP, LAYQ>(P, Q, N, M, (long)K * 2, 1, e, stream);
     return gemm_launch<Cfg>(P, Q, N, M, (long)K * 2, 1, LoadIdentity{}, LoadIdentity{}, e, stream);
   }
   EpiSplit e{ws, (long)N, (long)M * N};
