@@ -10,7 +10,7 @@ arithmetic with the residual adds and the MLP's fp8 operand cast as passes of th
 python bench.py --ns-probe        (Muon's Newton-Schulz call on the benchmark model's four stacks of 12 hidden matrices:
 one line per stack with its time and flop rate; not part of the AdamW step the headline line times)
 
-python bench.py --config-probe c1|c2|c3|c5|all   (the standalone configurations beside the full step, fwd + bwd each:
+python bench.py --config-probe c1|c2|c2d128|c3|c5|all   (the standalone configurations beside the full step, fwd + bwd each:
 one line per configuration; run under rocprofv3 --kernel-trace --stats for the per-kernel durations; with --graphs a
 second line per configuration: the same repetition recorded once as a HIP graph and replayed, without the host's launch work)
 
@@ -236,7 +236,8 @@ def ns_probe():
 
 def config_probe(which, graphs=False):
     """The standalone configurations beside the full step, each fwd + bwd through the autograd layer, 3 untimed and 5 timed
-    repetitions: c1 RMSNorm -> LM head -> cross-entropy on 8192 tokens; c2 causal attention 16 x 12 x 2048 x 64; c3 the
+    repetitions: c1 RMSNorm -> LM head -> cross-entropy on 8192 tokens; c2 causal attention 16 x 12 x 2048 x 64 (c2d128: 16 x 6 x
+    2048 x 128); c3 the
     fp8 MLP on 16384 tokens with a per-tensor amax activation scale; c5 the 8-expert top-2 fp8 layer on 16384 tokens,
     balanced and with +2.0 on two experts' router logits. Prints one line per configuration with its time per repetition."""
     import torch
@@ -311,6 +312,18 @@ def config_probe(which, graphs=False):
             A.CausalAttentionFn.apply(q, k, v, 0.125).backward(do)
         timed("c2 causal attention 16x12x2048x64", c2, 7.0 * B * H * T * T * D)
         del q, k, v, do
+    if which in ("c2d128", "all"):
+        # the same model width with the reference's own head dimension: 6 heads of 128
+        g = torch.Generator().manual_seed(20266)
+        B, H, T, D = 16, 6, 2048, 128
+        q, k, v = (leaf(torch.randn(B, H, T, D, generator=g).to(bf)) for _ in range(3))
+        do = torch.randn(B, T, H, D, generator=g).to(bf).to(dev)
+
+        def c2d():
+            clear(q, k, v)
+            A.CausalAttentionFn.apply(q, k, v, D ** -0.5).backward(do)
+        timed("c2d128 causal attention 16x6x2048x128", c2d, 7.0 * B * H * T * T * D)
+        del q, k, v, do
     if which in ("c3", "all"):
         g = torch.Generator().manual_seed(20263)
         M, d, F = 16384, 768, 3072
@@ -358,7 +371,7 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true")
     ap.add_argument("--ns-probe", action="store_true")
     ap.add_argument("--gemm-probe", action="store_true")
-    ap.add_argument("--config-probe", choices=("c1", "c2", "c3", "c5", "all"))
+    ap.add_argument("--config-probe", choices=("c1", "c2", "c2d128", "c3", "c5", "all"))
     ap.add_argument("--graphs", action="store_true", help="with --config-probe: also time each repetition replayed as a HIP graph")
     ap.add_argument("--bf16-dw", action="store_true")
     ap.add_argument("--unfused-residual", action="store_true")

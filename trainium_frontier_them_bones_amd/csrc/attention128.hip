@@ -166,7 +166,7 @@ __device__ __forceinline__ void store_grad_row(const f32x16 (&acc)[Geo<D>::NDT],
 
 // =========================================================================================== forward
 template <int D>
-__global__ __launch_bounds__(256, 2) void attnT_fwd_kernel(AttnT q, AttnT k, AttnT v, AttnT o, float* __restrict__ lse, int T,
+__global__ __launch_bounds__(256, 2) void attnD_fwd_kernel(AttnT q, AttnT k, AttnT v, AttnT o, float* __restrict__ lse, int T,
                                                            int H, float sl2, int nw) {
   typedef Geo<D> G;
   constexpr int TILE = G::TILE, NKS = G::NKS, NDT = G::NDT;
@@ -290,7 +290,7 @@ __global__ __launch_bounds__(256, 2) void attnT_fwd_kernel(AttnT q, AttnT k, Att
 
 // =========================================================================================== dQ
 template <int D>
-__global__ __launch_bounds__(256, 2) void attnT_dq_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dq,
+__global__ __launch_bounds__(256, 2) void attnD_dq_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dq,
                                                                         float* __restrict__ stats, long rows, int T, int H,
                                                                         float scale, float sl2, int nw, AttnT o,
                                                                         const float* __restrict__ lse) {
@@ -411,7 +411,7 @@ __global__ __launch_bounds__(256, 2) void attnT_dq_kernel(AttnT q, AttnT k, Attn
 
 // =========================================================================================== dK / dV
 template <int D, int R>  // R: queries per LDS stage (64 or 128)
-__global__ __launch_bounds__(256, D == 64 ? 2 : TFB_DKDV128_WPE) void attnT_dkdv_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dk, AttnT dv,
+__global__ __launch_bounds__(256, D == 64 ? 2 : TFB_DKDV128_WPE) void attnD_dkdv_kernel(AttnT q, AttnT k, AttnT v, AttnT go, AttnT dk, AttnT dv,
                                                                           const float* __restrict__ stats, long rows, int T,
                                                                           int H, float scale, float sl2, int nw) {
   typedef Geo<D> G;
@@ -551,7 +551,7 @@ AttnT mk(const void* p, const long* s) { return AttnT{(bf16_t*)p, s[0], s[1], s[
 template <int D>
 int fwd_launch(const void* q, const long* qs, const void* k, const long* ks, const void* v, const long* vs, void* o,
                const long* os, float* lse, int B, int H, int T, float scale, int nw, hipStream_t s) {
-  hipLaunchKernelGGL(attnT_fwd_kernel<D>, dim3(paired_grid(T / 128, B * H, 2), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs),
+  hipLaunchKernelGGL(attnD_fwd_kernel<D>, dim3(paired_grid(T / 128, B * H, 2), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs),
                      mk(o, os), lse, T, H, scale * LOG2E, nw);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
@@ -561,10 +561,10 @@ int bwd_launch(const void* q, const long* qs, const void* k, const long* ks, con
                const long* os, const void* go, const long* gos, void* dq, const long* dqs, void* dk, const long* dks, void* dv,
                const long* dvs, const float* lse, float* stats, int B, int H, int T, float scale, int nw, hipStream_t s) {
   const long rows = (long)B * H * T;
-  hipLaunchKernelGGL(attnT_dq_kernel<D>, dim3(paired_grid(T / 128, B * H, 2), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs),
+  hipLaunchKernelGGL(attnD_dq_kernel<D>, dim3(paired_grid(T / 128, B * H, 2), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs),
                      mk(go, gos), mk(dq, dqs), stats, rows, T, H, scale, scale * LOG2E, nw, mk(o, os), lse);
   TFB_LAUNCH_CHECK();
-  hipLaunchKernelGGL((attnT_dkdv_kernel<D, TFB_DKDV128_R>), dim3(paired_grid(T / 128, B * H, D == 64 ? 2 : TFB_DKDV128_WPE), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs),
+  hipLaunchKernelGGL((attnD_dkdv_kernel<D, TFB_DKDV128_R>), dim3(paired_grid(T / 128, B * H, D == 64 ? 2 : TFB_DKDV128_WPE), B * H), dim3(256), 0, s, mk(q, qs), mk(k, ks), mk(v, vs),
                      mk(go, gos), mk(dk, dks), mk(dv, dvs), stats, rows, T, H, scale, scale * LOG2E, nw);
   TFB_LAUNCH_CHECK();
   return TFB_OK;
