@@ -31,6 +31,10 @@
 #pragma once
 #include "gemm_core.hpp"
 
+#ifndef TFB_PP_EARLYB
+#define TFB_PP_EARLYB 1  // a k-tile's first Q fragments requested in the previous k-tile's last MFMA cluster
+#endif
+
 typedef __attribute__((address_space(3))) uint8_t tfb_lds_u8;
 typedef unsigned tfb_u32x2 __attribute__((ext_vector_type(2)));
 
@@ -284,16 +288,17 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
       fa[1][3] = tr_frag(std::integral_constant<int, h * 16384 + TR3>{}, ap[1]);
     }
   };
-  auto readB = [&](auto H, r128_t(&fb)[4]) __attribute__((always_inline)) {
+  // flip = 0x10000: the fragments of the OTHER stage (the next k-tile)
+  auto readB = [&](auto H, r128_t(&fb)[4], uint32_t flip = 0) __attribute__((always_inline)) {
     constexpr int h = decltype(H)::value;
     if constexpr (LAYQ == TFB_K_CONTIG) {
 #pragma unroll
-      for (int s = 0; s < 4; ++s) fb[s] = tfb_lds_read128<h * 16384, r128_t>(aq[s]);
+      for (int s = 0; s < 4; ++s) fb[s] = tfb_lds_read128<h * 16384, r128_t>(aq[s] ^ flip);
     } else {
-      fb[0] = tr_frag(std::integral_constant<int, h * 16384>{}, aq[0]);
-      fb[1] = tr_frag(std::integral_constant<int, h * 16384 + TR1>{}, aq[0]);
-      fb[2] = tr_frag(std::integral_constant<int, h * 16384 + TR2>{}, aq[0]);
-      fb[3] = tr_frag(std::integral_constant<int, h * 16384 + TR3>{}, aq[0]);
+      fb[0] = tr_frag(std::integral_constant<int, h * 16384>{}, aq[0] ^ flip);
+      fb[1] = tr_frag(std::integral_constant<int, h * 16384 + TR1>{}, aq[0] ^ flip);
+      fb[2] = tr_frag(std::integral_constant<int, h * 16384 + TR2>{}, aq[0] ^ flip);
+      fb[3] = tr_frag(std::integral_constant<int, h * 16384 + TR3>{}, aq[0] ^ flip);
     }
   };
   // the fragments pass through the wait as in/out operands, so that no MFMA that reads them is scheduled ahead of it
@@ -455,6 +460,7 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
   };
 
   int S = 0;
+  if (TFB_PP_EARLYB) readB(H0{}, fb0);
   bool have_prev = false;  // the previous tile's accumulators are still to be stored
   long pp0 = 0, pq0 = 0;   // its origin
   for (;;) {
@@ -481,8 +487,8 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
       const uint8_t* gp1 = (in1 ? gp : gpn) + k1 * sp.kstep;
       const uint8_t* gp2 = (in2 ? gp : gpn) + k2 * sp.kstep;
       const uint8_t* gq2 = (in2 ? gq : gqn) + k2 * sq.kstep;
-      // c0
-      readB(H0{}, fb0);
+      // c0 (the Q fragments of half 0 were requested in the previous k-tile's c7)
+      if (!TFB_PP_EARLYB) readB(H0{}, fb0);
       readA(H0{});
       dma(S ^ 1, 0, 1, gp1);
       if constexpr (!kF32) {
@@ -515,20 +521,26 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(PpArgs a, Epi epi_in) {
       // c5
       waitA();
       mma(FIRST, H1{}, H0{}, fb0);
+      if (TFB_PP_EARLYB) {
+        // Completion is reported in issue order, stores included. Everything up to the quarter requested in c0 has to be
+        // there one cluster before the other group's matching wait: all but the two quarters requested since (4
+        // instructions), and in a first iteration with stores all but those and the 12 stores (c0's four were issued
+        // behind its loads). After the barrier that ends c6 both groups have waited, so the next k-tile is complete.
+        if (!kF32 && first && have_prev) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      }
       TFB_SBAR();
       // c6
       dma(S, 1, 1, gq2);
-      // Completion is reported in issue order, stores included. Everything up to the quarter requested in c0 has to be
-      // there: all but the three quarters requested since (6 instructions), and in a first iteration with stores all but
-      // those and the 16 stores (c0's four were issued behind its loads).
       if (!kF32 && first && have_prev) {
         if constexpr (!kF32) store_block(H1{}, H1{}, pp0, pq0);
-        asm volatile("s_waitcnt vmcnt(22)" ::: "memory");
+        if (!TFB_PP_EARLYB) asm volatile("s_waitcnt vmcnt(22)" ::: "memory");
       } else {
-        asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+        if (!TFB_PP_EARLYB) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
       }
       TFB_SBAR();
-      // c7
+      // c7: the next k-tile's first Q fragments are requested under this cluster's MFMAs (fb0 was last read in c5)
+      if (TFB_PP_EARLYB) readB(H0{}, fb0, 0x10000u);
       mma(FIRST, H1{}, H1{}, fb1);
       TFB_SBAR();
       S ^= 1;
