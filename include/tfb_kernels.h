@@ -256,14 +256,15 @@ int tfb_qkv_rope_fwd(const void* x, const void* w, const void* cos_t, const void
 /* ---- attention ----------------------------------------------------------------------------------------------------
  * Causal flash attention, bf16. Every tensor comes with host long[3] element strides (batch, head, token); head dim
  * contiguous; so q/k/v can be [B,H,T,D], [B,T,H,D] or thirds of a fused [B,T,3C] projection. lse fp32 [B*H][T].
- * T % 128 == 0, D == 64.
+ * T % 128 == 0, D == 64 or 128.
  * Replaces _attn_fwd_kernel behind nki_causal_attention (round1/source/train.py:7536, 8069;
  * round2/source/kernels/nki_attn_bandpro.py:1850); op s2attn::*_fwd (round2/source/train.py:4988). */
 int tfb_attn_fwd(const void* q, const long* q_strides, const void* k, const long* k_strides, const void* v,
                  const long* v_strides, void* o, const long* o_strides, void* lse, int B, int H, int T, int D, float scale,
                  void* stream);
 
-/* dq, dk, dv from (q, k, v, o, do, lse); delta fp32 [2][B*H][T] scratch.
+/* dq, dk, dv from (q, k, v, o, do, lse); delta fp32 [2][B*H][T] scratch (the rows' -sum(dO O) and -lse / scale, which the
+ * first kernel, dQ, leaves for the second).
  * Replaces _attn_bwd_kernel / NkiAttnFn.backward (round1/source/train.py:7591, 8036). */
 int tfb_attn_bwd(const void* q, const long* q_strides, const void* k, const long* k_strides, const void* v,
                  const long* v_strides, const void* o, const long* o_strides, const void* d_o, const long* do_strides,
@@ -274,8 +275,8 @@ int tfb_attn_bwd(const void* q, const long* q_strides, const void* k, const long
  * array inside the library (8 MiB per GPU, held until the process ends) instead of from the caller. It allocates and
  * frees nothing. B * H * T <= tfb_attn_bwd_static_max_rows() (1,048,576), otherwise status 4 and the caller uses
  * tfb_attn_bwd. All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams) race.
- * The first call on a device looks up the array's address (hipGetSymbolAddress) and sets the kernels' LDS size
- * attribute: make one call eagerly on each device (same head dimension) before capturing a call into a HIP graph.
+ * The first call on a device looks up the array's address (hipGetSymbolAddress): make one call eagerly on each device
+ * before capturing a call into a HIP graph.
  * Has no counterpart in the reference (its kernels allocate their own outputs and scratch through the NKI runtime). */
 long tfb_attn_bwd_static_max_rows(void);
 int tfb_attn_bwd_static(const void* q, const long* q_strides, const void* k, const long* k_strides, const void* v,

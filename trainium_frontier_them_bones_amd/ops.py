@@ -570,8 +570,7 @@ def attn_bwd_static(q, k, v, o, do, lse, scale, dq, dk, dv, layout="bhtd", out_l
     """attn_bwd into caller-provided dq, dk, dv through the entry point that allocates nothing: its row-statistic scratch
     is a static device array inside the library (B * H * T <= tfb_attn_bwd_static_max_rows(); TfbError status 4 beyond).
     Calls that overlap on one GPU share that array and race; this wrapper creates no tensor either. The FIRST call on a
-    device looks up the array's address and sets the kernels' LDS attributes: make one call (or any attention backward of
-    the same head dimension) eagerly before capturing this one into a HIP graph."""
+    device looks up the array's address: make one call eagerly before capturing this one into a HIP graph."""
     B, H, T, D = _attn_bwd_chk(q, k, v, o, do, lse, dq, dk, dv, layout, out_layout)
     _lib.call("tfb_attn_bwd_static", _p(q), _bht(q, layout), _p(k), _bht(k, layout), _p(v), _bht(v, layout), _p(o),
               _bht(o, "bthd"), _p(do), _bht(do, "bthd"), _p(dq), _bht(dq, out_layout), _p(dk), _bht(dk, out_layout), _p(dv),
