@@ -17,6 +17,9 @@ second line per configuration: the same repetition recorded once as a HIP graph 
 python bench.py --gemm-probe      (this library's bf16 GEMM beside torch.matmul, i.e. the vendor BLAS, on the step's own GEMM
 shapes and 8192^3, in one process on one box: a yardstick only, the product never calls the vendor library)
 
+python bench.py --power-probe     (the step's largest kernels timed on N(0, 1) operands and on all-zero operands, alternating:
+identical instruction streams, so the difference is the clock the GPU sustains under its power limit)
+
 python bench.py --traffic-probe   (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: a 256 MiB device copy as the
 counters' calibration, then attention forward + backward at the benchmark shape; prints nothing)
 """
@@ -213,6 +216,63 @@ def gemm_probe():
         del a, b, out, ref
 
 
+def power_probe():
+    """The same launches timed on N(0, 1) operands and on all-zero operands, alternating (random, zeros, random, zeros):
+    a GEMM's instruction stream does not depend on its data and the attention kernels' hardly does (no row maximum grows
+    by 2^8 in either case), so what differs between the columns is the clock the GPU sustains under its power limit.
+    20 timed calls after 5 warm-up calls per cell; one table row per kernel."""
+    import torch
+    from trainium_frontier_them_bones_amd import ops
+    dev = torch.device("cuda:0")
+
+    def t(f, n=20):
+        for _ in range(5):
+            f()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(n):
+            f()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / n * 1e3
+
+    def rnd(*shape):
+        return torch.randn(*shape, device=dev).bfloat16()
+
+    def zer(*shape):
+        return torch.zeros(*shape, device=dev, dtype=torch.bfloat16)
+
+    def gemm(m, n, k):
+        def make(mk):
+            a, b, out = mk(m, k), mk(n, k), torch.empty(m, n, device=dev, dtype=torch.bfloat16)
+            return lambda: ops.matmul(a, b, trans_b=True, out=out)
+        return make
+
+    def attn(bwd):
+        B, H, T, D = 16, 12, 2048, 64
+
+        def make(mk):
+            q, k, v, do = mk(B, H, T, D), mk(B, H, T, D), mk(B, H, T, D), mk(B, T, H, D)
+            o, lse = ops.attn_fwd(q, k, v, 0.125)
+            if bwd:
+                return lambda: ops.attn_bwd(q, k, v, o, do, lse, 0.125)
+            return lambda: ops.attn_fwd(q, k, v, 0.125)
+        return make
+
+    rows = [("bf16 GEMM 8192^3 (NT)", gemm(8192, 8192, 8192)), ("QKV projection 32768 x 2304 x 768", gemm(32768, 2304, 768)),
+            ("LM head logits 32768 x 32768 x 768", gemm(32768, 32768, 768)),
+            ("attention forward 16 x 12 x 2048 x 64", attn(False)), ("attention backward 16 x 12 x 2048 x 64", attn(True))]
+    print("| kernel | random us | zeros us | random us | zeros us | zeros / random |")
+    print("|---|---|---|---|---|---|")
+    torch.manual_seed(0)
+    for name, make in rows:
+        fr, fz = make(rnd), make(zer)
+        ts = [t(fr), t(fz), t(fr), t(fz)]
+        print("| %s | %.1f | %.1f | %.1f | %.1f | %.2f |" % (name, *ts, (ts[1] + ts[3]) / (ts[0] + ts[2])), flush=True)
+        del fr, fz
+
+
 def ns_probe():
     import torch
     from trainium_frontier_them_bones_amd import ops
@@ -371,6 +431,7 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true")
     ap.add_argument("--ns-probe", action="store_true")
     ap.add_argument("--gemm-probe", action="store_true")
+    ap.add_argument("--power-probe", action="store_true")
     ap.add_argument("--config-probe", choices=("c1", "c2", "c2d128", "c3", "c5", "all"))
     ap.add_argument("--graphs", action="store_true", help="with --config-probe: also time each repetition replayed as a HIP graph")
     ap.add_argument("--bf16-dw", action="store_true")
@@ -389,6 +450,9 @@ def main():
         return
     if args.gemm_probe:
         gemm_probe()
+        return
+    if args.power_probe:
+        power_probe()
         return
     if args.config_probe:
         config_probe(args.config_probe, args.graphs)
