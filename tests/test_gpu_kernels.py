@@ -586,6 +586,33 @@ def test_mlp8_full_size_properties(ops, dev):
     assert torch.isfinite(dx.float()).all() and torch.isfinite(y.float()).all()
 
 
+@pytest.mark.parametrize("M,Ms,F", [(2048, 1920, 3072), (8192, 8064, 768), (5632, 5504, 1280)])
+def test_mlp8_weight_stationary_kernel_equals_the_tiled_kernel(ops, dev, M, Ms, F):
+    """With d_model = 768 the up-projection and the dH GEMM of a batch of a multiple of 512 tokens run the weight-stationary
+    kernel (weights in registers, tokens streamed), any other batch the 128 x 128 tiled kernel. Tokens are independent, so
+    the rows the two batches share must come out bit for bit the same: r, y, dx, dpre, h, and the fp8 bytes handed to the
+    weight gradients. M is a multiple of 512 (weight-stationary), Ms = M - 128 is not (tiled); the shapes give runs of equal
+    and of unequal length per workgroup, with and without panel borders inside a run."""
+    d = 768
+    g = _g(768 + F)
+    x = torch.randn(M, d, generator=g).bfloat16().to(dev)
+    wf = (0.02 * torch.randn(F, d, generator=g)).bfloat16().to(dev)
+    wp = (0.02 * torch.randn(d, F, generator=g)).bfloat16().to(dev)
+    dy = torch.randn(M, d, generator=g).bfloat16().to(dev)
+    row = ops.mlp8_forward_scales(wf, wp, 448.0)
+    w8 = ops.mlp8_precast(wf, wp, row)
+    y, r = ops.mlp8_fwd(x, w8, row, F)
+    ys, rs = ops.mlp8_fwd(x[:Ms].contiguous(), w8, row, F)
+    assert torch.equal(r[:Ms], rs) and torch.equal(y[:Ms], ys)
+    rowb = ops.mlp8_backward_scales(dy, row)
+    dx, h, dpre = ops.mlp8_bwd(dy, r, w8, rowb)
+    dxs, hs, dps = ops.mlp8_bwd(dy[:Ms].contiguous(), rs, w8, rowb)
+    assert torch.equal(dpre[:Ms], dps) and torch.equal(h[:Ms], hs) and torch.equal(dx[:Ms], dxs)
+    dxq, _, dp8, hq8, _ = ops.mlp8_bwd_q(dy, r, w8, rowb, 448.0, want_dpre=False)
+    dxqs, _, dp8s, hq8s, _ = ops.mlp8_bwd_q(dy[:Ms].contiguous(), rs, w8, rowb, 448.0, want_dpre=False)
+    assert torch.equal(dp8[:Ms], dp8s) and torch.equal(hq8[:Ms], hq8s) and torch.equal(dxq[:Ms], dxqs) and torch.equal(dxq, dx)
+
+
 @pytest.mark.parametrize("shape", [(512, 256, 512), (16384, 768, 3072)])
 def test_mlp8_as_the_benchmark_times_it(ops, dev, shape):
     """Configuration 3 of BASELINE.json in the form bench.py times: OCP e4m3 at 448, the activation scale from the tensor's

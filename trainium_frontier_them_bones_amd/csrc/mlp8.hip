@@ -14,7 +14,7 @@
 //   x8 = e4m3(x * s_x); r = bf16(max(acc * dq_fc, 0)); rc = bf16(min(r * c_h, 15.375));
 //   h8 = e4m3(rc^2); y = bf16(acc * dq_proj); dy8 = e5m2(dy * s_dy);
 //   dpre = bf16((acc * dq_dh2) * r); dp8 = e5m2(dpre * s_dp); dx = bf16(acc * dq_dx).
-#include "gemm_pp.hpp"
+#include "gemm_ws8.hpp"
 
 // scale-row columns (nki_mlp_fused8.py:111-114)
 #define SC_S_WFC 0
@@ -772,6 +772,15 @@ static int launch8(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes, Ep
   return gemm_launch<Cfg>(P, Q, np, nq, kbytes, 1, LoadIdentity{}, LoadIdentity{}, e, s);
 }
 
+// The MLP's two GEMMs that contract over d_model with a heavy epilogue (up-projection, dH): with d_model = 768 the
+// weight-stationary kernel (the weights in registers, only the tokens stream), else the 128 x 128 kernel. The same sums in
+// the same order, the same epilogue code.
+template <class Cfg, class Epi>
+static int launch_k768(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes, Epi e, hipStream_t s) {
+  if (gemm_ws8_applies(np, nq, kbytes)) return gemm_ws8_launch<Cfg::FMTP, Cfg::FMTQ>(P, Q, np, nq, kbytes, e, s);
+  return gemm_launch<Cfg>(P, Q, np, nq, kbytes, 1, LoadIdentity{}, LoadIdentity{}, e, s);
+}
+
 // out [M][N] bf16 = bf16((a8 [M][K] @ b8 [N][K]^T) * dq): the fp8 projection GEMM. a8 is e4m3 (fmt_a 0: forward
 // activations) or e5m2 (fmt_a 1: gradients); b8 is e4m3 (a pre-cast weight layout). dq = dq_imm * *dq_a * *dq_b, the
 // pointers being device fp32 scalars (inverse power-of-two scales) or null.
@@ -854,7 +863,7 @@ extern "C" int tfb_mlp8_fwd(const void* x8, const void* w8, const void* row, voi
   const long n = (long)F * d;
   GemmOperand Pw{b, (long)d}, Qx{(const uint8_t*)x8, (long)d};
   EpiUp e1{(const float*)row, (bf16_t*)r, (uint8_t*)h8, (long)F};
-  int st = launch8<Cfg8>(Pw, Qx, F, (int)M, (long)d, e1, s);
+  int st = launch_k768<Cfg8>(Pw, Qx, F, (int)M, (long)d, e1, s);
   if (st != TFB_OK) return st;
   GemmOperand Pp{b + 2 * n, (long)F}, Qh{(const uint8_t*)h8, (long)F};
   EpiScaleStore e2{(const float*)row, SC_DQ_PROJ, (bf16_t*)y, (long)d};
@@ -874,7 +883,7 @@ extern "C" int tfb_mlp8_fwd_res(const void* x8, const void* w8, const void* row,
   const long n = (long)F * d;
   GemmOperand Pw{b, (long)d}, Qx{(const uint8_t*)x8, (long)d};
   EpiUp e1{(const float*)row, (bf16_t*)r, (uint8_t*)h8, (long)F};
-  int st = launch8<Cfg8>(Pw, Qx, F, (int)M, (long)d, e1, s);
+  int st = launch_k768<Cfg8>(Pw, Qx, F, (int)M, (long)d, e1, s);
   if (st != TFB_OK) return st;
   GemmOperand Pp{b + 2 * n, (long)F}, Qh{(const uint8_t*)h8, (long)F};
   EpiDescaleRes e2{(const float*)row, SC_DQ_PROJ, nullptr, nullptr, 1.0f, (const bf16_t*)res, (bf16_t*)y, (long)d};
@@ -894,7 +903,7 @@ extern "C" int tfb_mlp8_bwd_q(const void* dy8, const void* r, const void* w8, co
   const long n = (long)F * d;
   GemmOperand Pw{b + 3 * n, (long)d}, Qg{(const uint8_t*)dy8, (long)d};  // wp8T [F][d]
   EpiDh e1{(const float*)row, (const bf16_t*)r, (bf16_t*)dpre, (uint8_t*)dp8, (bf16_t*)h, (uint8_t*)hq8, hq_limit, (long)F};
-  int st = gemm_launch<Cfg8g>(Pw, Qg, F, (int)M, (long)d, 1, LoadIdentity{}, LoadIdentity{}, e1, s);
+  int st = launch_k768<Cfg8g>(Pw, Qg, F, (int)M, (long)d, e1, s);
   if (st != TFB_OK) return st;
   GemmOperand Pf{b + n, (long)F}, Qd{(const uint8_t*)dp8, (long)F};  // wf8T [d][F]
   EpiScaleStore e2{(const float*)row, SC_DQ_DX, (bf16_t*)dx, (long)d};
