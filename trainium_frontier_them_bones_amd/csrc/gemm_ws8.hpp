@@ -34,6 +34,9 @@ struct Ws8Args {
 #ifndef TFB_WS8
 #define TFB_WS8 1  // 0: these GEMMs stay on the tiled kernels
 #endif
+#ifndef TFB_WS8_DEPTH
+#define TFB_WS8_DEPTH 1  // k-steps the B fragment reads run ahead of the MFMAs (1 or 2)
+#endif
 
 template <int FMTP, int FMTQ, class Epi>
 __global__ __launch_bounds__(512, 2) void gemm_ws8_kernel(Ws8Args a, Epi epi_in) {
@@ -137,10 +140,11 @@ __global__ __launch_bounds__(512, 2) void gemm_ws8_kernel(Ws8Args a, Epi epi_in)
       b[2] = tfb_lds_read128<off + 4096, i32x4>(ab[2 * u] + so);
       b[3] = tfb_lds_read128<off + 4096, i32x4>(ab[2 * u + 1] + so);
     };
-    auto mm = [&](auto KS, i32x4(&b)[4], bool more) __attribute__((always_inline)) {
-      constexpr int ks = decltype(KS)::value;
-      // the four reads of the next k-step were issued behind these: all but those four have to be there
-      if (more) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+    auto mm = [&](auto KS, i32x4(&b)[4], auto NEWER) __attribute__((always_inline)) {
+      constexpr int ks = decltype(KS)::value, newer = decltype(NEWER)::value;
+      // `newer` reads were issued behind this k-step's four: all but those have to be there
+      if (newer == 8) asm volatile("s_waitcnt lgkmcnt(8)" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+      else if (newer == 4) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
       else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
       const i32x8 bv0 = {b[0].x, b[0].y, b[0].z, b[0].w, b[1].x, b[1].y, b[1].z, b[1].w};
       const i32x8 bv1 = {b[2].x, b[2].y, b[2].z, b[2].w, b[3].x, b[3].y, b[3].z, b[3].w};
@@ -151,19 +155,38 @@ __global__ __launch_bounds__(512, 2) void gemm_ws8_kernel(Ws8Args a, Epi epi_in)
     };
 #define TFB_WS_KS(n) std::integral_constant<int, n> {}
     __builtin_amdgcn_s_setprio(1);
+#if TFB_WS8_DEPTH == 2
+    // fragments two k-steps ahead of the MFMAs (three register sets)
+    i32x4 b2[4];
     rd(TFB_WS_KS(0), b0);
-    rd(TFB_WS_KS(1), b1);  mm(TFB_WS_KS(0), b0, true);
-    rd(TFB_WS_KS(2), b0);  mm(TFB_WS_KS(1), b1, true);
-    rd(TFB_WS_KS(3), b1);  mm(TFB_WS_KS(2), b0, true);
-    rd(TFB_WS_KS(4), b0);  mm(TFB_WS_KS(3), b1, true);
-    rd(TFB_WS_KS(5), b1);  mm(TFB_WS_KS(4), b0, true);
-    rd(TFB_WS_KS(6), b0);  mm(TFB_WS_KS(5), b1, true);
-    rd(TFB_WS_KS(7), b1);  mm(TFB_WS_KS(6), b0, true);
-    rd(TFB_WS_KS(8), b0);  mm(TFB_WS_KS(7), b1, true);
-    rd(TFB_WS_KS(9), b1);  mm(TFB_WS_KS(8), b0, true);
-    rd(TFB_WS_KS(10), b0); mm(TFB_WS_KS(9), b1, true);
-    rd(TFB_WS_KS(11), b1); mm(TFB_WS_KS(10), b0, true);
-    mm(TFB_WS_KS(11), b1, false);
+    rd(TFB_WS_KS(1), b1);
+    rd(TFB_WS_KS(2), b2);  mm(TFB_WS_KS(0), b0, TFB_WS_KS(8));
+    rd(TFB_WS_KS(3), b0);  mm(TFB_WS_KS(1), b1, TFB_WS_KS(8));
+    rd(TFB_WS_KS(4), b1);  mm(TFB_WS_KS(2), b2, TFB_WS_KS(8));
+    rd(TFB_WS_KS(5), b2);  mm(TFB_WS_KS(3), b0, TFB_WS_KS(8));
+    rd(TFB_WS_KS(6), b0);  mm(TFB_WS_KS(4), b1, TFB_WS_KS(8));
+    rd(TFB_WS_KS(7), b1);  mm(TFB_WS_KS(5), b2, TFB_WS_KS(8));
+    rd(TFB_WS_KS(8), b2);  mm(TFB_WS_KS(6), b0, TFB_WS_KS(8));
+    rd(TFB_WS_KS(9), b0);  mm(TFB_WS_KS(7), b1, TFB_WS_KS(8));
+    rd(TFB_WS_KS(10), b1); mm(TFB_WS_KS(8), b2, TFB_WS_KS(8));
+    rd(TFB_WS_KS(11), b2); mm(TFB_WS_KS(9), b0, TFB_WS_KS(8));
+    mm(TFB_WS_KS(10), b1, TFB_WS_KS(4));
+    mm(TFB_WS_KS(11), b2, TFB_WS_KS(0));
+#else
+    rd(TFB_WS_KS(0), b0);
+    rd(TFB_WS_KS(1), b1);  mm(TFB_WS_KS(0), b0, TFB_WS_KS(4));
+    rd(TFB_WS_KS(2), b0);  mm(TFB_WS_KS(1), b1, TFB_WS_KS(4));
+    rd(TFB_WS_KS(3), b1);  mm(TFB_WS_KS(2), b0, TFB_WS_KS(4));
+    rd(TFB_WS_KS(4), b0);  mm(TFB_WS_KS(3), b1, TFB_WS_KS(4));
+    rd(TFB_WS_KS(5), b1);  mm(TFB_WS_KS(4), b0, TFB_WS_KS(4));
+    rd(TFB_WS_KS(6), b0);  mm(TFB_WS_KS(5), b1, TFB_WS_KS(4));
+    rd(TFB_WS_KS(7), b1);  mm(TFB_WS_KS(6), b0, TFB_WS_KS(4));
+    rd(TFB_WS_KS(8), b0);  mm(TFB_WS_KS(7), b1, TFB_WS_KS(4));
+    rd(TFB_WS_KS(9), b1);  mm(TFB_WS_KS(8), b0, TFB_WS_KS(4));
+    rd(TFB_WS_KS(10), b0); mm(TFB_WS_KS(9), b1, TFB_WS_KS(4));
+    rd(TFB_WS_KS(11), b1); mm(TFB_WS_KS(10), b0, TFB_WS_KS(4));
+    mm(TFB_WS_KS(11), b1, TFB_WS_KS(0));
+#endif
     __builtin_amdgcn_s_setprio(0);
 #undef TFB_WS_KS
     // acc_j[4 jj + e] = D[p = 8 jj + 4 lh + e][q = 32 j + lr]
@@ -208,9 +231,10 @@ __global__ __launch_bounds__(512, 2) void gemm_ws8_kernel(Ws8Args a, Epi epi_in)
 
   // Phase ph: group 0 multiplies tile ph / 2 (ph even) or finishes it (ph odd); group 1 one phase later. Tile t + 1 is
   // requested in phase 2 t - by group 0 in front of its MFMAs, by group 1 behind its epilogue - into the stage whose tile
-  // (t - 1) group 1 stopped reading in phase 2 t - 1, and waited for at the end of phase 2 t + 1: by group 1 with nothing
-  // younger outstanding, by group 0 behind an epilogue of at least four younger stores (completion is reported in issue
-  // order).
+  // (t - 1) group 1 stopped reading in phase 2 t - 1, and waited for in phase 2 t + 1, a phase after the request: by group 1
+  // behind its MFMAs with nothing younger outstanding, by group 0 in front of its epilogue, where only the epilogue's own
+  // four operand loads (if it has any) are younger - behind the epilogue the wait would be for its stores' round trips
+  // (completion is reported in issue order, stores included).
   for (int ph = 0; ph <= 2 * T; ++ph) {
     if ((ph & 1) == grp) {
       const int t = (ph - grp) >> 1;
@@ -221,12 +245,14 @@ __global__ __launch_bounds__(512, 2) void gemm_ws8_kernel(Ws8Args a, Epi epi_in)
       }
     } else {
       const int t = (ph - 1 - grp) >> 1;  // group 0: (ph - 1) / 2; group 1: (ph - 2) / 2
+      if (grp == 0) {
+        if (kPrefetch) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
       if (ph - 1 - grp >= 0 && t < T) finish(t);
       if (grp == 1) {
         const int tn = (ph >> 1) + 1;
         if (tn < T) dma(tn);
-      } else {
-        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
       }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the staging block is complete (or read) before the roles swap
