@@ -545,6 +545,17 @@ struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*
   float hq_limit;
   long F;
   float dq = 0.f, sdp = 0.f, sh = 0.f;  // sc[SC_DQ_DH2], sc[SC_S_DP], sc[SC_S_H], read once by prepare()
+  // With a power-of-two scale (what the scale search produces) the cast of a rounded bf16 value times the scale is one
+  // instruction per pair, v_cvt_scalef32_pk_{bf8,fp8}_bf16 on the packed pair and 1 / scale: the same bytes as unpacking,
+  // multiplying and converting for every value inside the format's range (all 65536 bf16 patterns compared on the GPU
+  // for six scales); beyond the range the instruction does not saturate, so the saturation is applied to the fp32 value
+  // before its rounding, at limit / scale (a bf16 number: rounding is monotonic, so clamping before or after it is the same).
+  float inv_sdp = 0.f, lim_dp = 0.f, inv_sh = 0.f, lim_h = 0.f;
+  bool fast_dp = false, fast_h = false;
+  static __device__ __forceinline__ bool pow2(float x) {
+    const uint32_t b = __float_as_uint(x);
+    return (b & 0x807fffffu) == 0 && (b >> 23) > 16 && (b >> 23) < 238;
+  }
   __device__ __forceinline__ EpiDh for_group(int g) const {
     EpiDh e = *this;
     e.sc = sc + g * NSC;
@@ -555,28 +566,71 @@ struct EpiDh {  // dh = dy8 @ wp8: dpre = bf16((acc*dq_dh2)*r), dp8 = e5m2(dpre*
     e.dq = sc[SC_DQ_DH2];
     e.sdp = sc[SC_S_DP];
     e.sh = sc[SC_S_H];
+#ifndef TFB_DH_FASTCAST
+#define TFB_DH_FASTCAST 1
+#endif
+    if (TFB_DH_FASTCAST) {
+      e.fast_dp = pow2(e.sdp);
+      e.inv_sdp = 1.0f / e.sdp;
+      e.lim_dp = TFB_E5M2_MAX * e.inv_sdp;
+      const float lim = fminf(hq_limit, TFB_E4M3_MAX);
+      e.inv_sh = 1.0f / e.sh;
+      e.lim_h = lim * e.inv_sh;
+      e.fast_h = pow2(e.sh) && hq8 && !h && lim > 0.f && (__float_as_uint(e.lim_h) & 0xffffu) == 0;
+    }
     return e;
   }
   typedef u32x4 pre_t;  // the 8 values of r this chunk needs, requested before the k-loop
   __device__ __forceinline__ pre_t prefetch(int p, int q) const {
     return __builtin_nontemporal_load((const u32x4*)(r + (long)q * F + p));   // read once
   }
+  typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+  typedef short s2_t __attribute__((ext_vector_type(2)));
+  template <int FMT>
+  static __device__ __forceinline__ uint32_t cast4_scaled(uint32_t lo_pair, uint32_t hi_pair, float inv_scale) {
+    s2_t o = {0, 0};
+    if (FMT == TFB_FMT_E5M2) {
+      o = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(o, __builtin_bit_cast(bf2_t, lo_pair), inv_scale, false);
+      o = __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(o, __builtin_bit_cast(bf2_t, hi_pair), inv_scale, true);
+    } else {
+      o = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o, __builtin_bit_cast(bf2_t, lo_pair), inv_scale, false);
+      o = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o, __builtin_bit_cast(bf2_t, hi_pair), inv_scale, true);
+    }
+    return __builtin_bit_cast(uint32_t, o);
+  }
   __device__ __forceinline__ void operator()(int p, int q, const float (&v)[8], const pre_t& rv, int) const {
     const long off = (long)q * F + p;
     float rr[8], dp[8];
     unpack8bf(rv, rr);
     u32x4 dbits;
+    if (fast_dp) {
 #pragma unroll
-    for (int i = 0; i < 8; i += 2) {
-      dp[i] = (v[i] * dq) * rr[i];
-      dp[i + 1] = (v[i + 1] * dq) * rr[i + 1];
-      dbits[i >> 1] = round2_bf(dp[i], dp[i + 1]);           // dpre = bf16((acc dq_dh2) r)
+      for (int i = 0; i < 8; ++i) dp[i] = (v[i] * dq) * rr[i];
+      if (dpre) *(u32x4*)(dpre + off) = pack8bf(dp);                 // dpre = bf16((acc dq_dh2) r)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dp[i] = dp[i] != dp[i] ? dp[i] : fminf(fmaxf(dp[i], -lim_dp), lim_dp);
+      dbits = pack8bf(dp);
+      u32x2 o = {cast4_scaled<TFB_FMT_E5M2>(dbits[0], dbits[1], inv_sdp), cast4_scaled<TFB_FMT_E5M2>(dbits[2], dbits[3], inv_sdp)};
+      *(u32x2*)(dp8 + off) = o;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; i += 2) {
+        dp[i] = (v[i] * dq) * rr[i];
+        dp[i + 1] = (v[i + 1] * dq) * rr[i + 1];
+        dbits[i >> 1] = round2_bf(dp[i], dp[i + 1]);           // dpre = bf16((acc dq_dh2) r)
+      }
+      if (dpre) *(u32x4*)(dpre + off) = dbits;
+      u32x2 o = {cvt4_fp8<TFB_FMT_E5M2>(dp[0] * sdp, dp[1] * sdp, dp[2] * sdp, dp[3] * sdp),
+                 cvt4_fp8<TFB_FMT_E5M2>(dp[4] * sdp, dp[5] * sdp, dp[6] * sdp, dp[7] * sdp)};
+      *(u32x2*)(dp8 + off) = o;
     }
-    if (dpre) *(u32x4*)(dpre + off) = dbits;
-    u32x2 o = {cvt4_fp8<TFB_FMT_E5M2>(dp[0] * sdp, dp[1] * sdp, dp[2] * sdp, dp[3] * sdp),
-               cvt4_fp8<TFB_FMT_E5M2>(dp[4] * sdp, dp[5] * sdp, dp[6] * sdp, dp[7] * sdp)};
-    *(u32x2*)(dp8 + off) = o;
-    if (h || hq8) {
+    if (fast_h) {   // hq8 only: e4m3(min(bf16(r^2) s_h, limit)) = cast(bf16(min(r^2, limit / s_h)), 1 / s_h)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) rr[i] = fminf(rr[i] * rr[i], lim_h);
+      const u32x4 hb = pack8bf(rr);
+      u32x2 q8 = {cast4_scaled<TFB_FMT_E4M3>(hb[0], hb[1], inv_sh), cast4_scaled<TFB_FMT_E4M3>(hb[2], hb[3], inv_sh)};
+      *(u32x2*)(hq8 + off) = q8;
+    } else if (h || hq8) {
       u32x4 hbits;
 #pragma unroll
       for (int i = 0; i < 8; i += 2) {
