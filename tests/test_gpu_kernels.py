@@ -613,6 +613,28 @@ def test_mlp8_weight_stationary_kernel_equals_the_tiled_kernel(ops, dev, M, Ms, 
     assert torch.equal(dp8[:Ms], dp8s) and torch.equal(hq8[:Ms], hq8s) and torch.equal(dxq[:Ms], dxqs) and torch.equal(dxq, dx)
 
 
+@pytest.mark.parametrize("fmt", [0, 1])
+def test_fp8_projection_weight_stationary_kernel_equals_the_tiled_kernel(ops, dev, fmt):
+    """tfb_gemm_fp8 / tfb_gemm_fp8_res with a contraction of 768 bytes: a batch of a multiple of 512 tokens runs the
+    weight-stationary kernel, a shorter one the tiled kernel; the rows they share are equal bit for bit (e4m3 activations and
+    e5m2 gradients, plain store and the store with the residual add)."""
+    M, Ms, K, N = 2048, 1920, 768, 2304
+    g = _g(99 + fmt)
+    a8 = ops.quant_fp8(torch.randn(M, K, generator=g).bfloat16().to(dev), 4.0, fmt)
+    b8 = ops.quant_fp8((0.05 * torch.randn(N, K, generator=g)).bfloat16().to(dev), 64.0, 0)
+    dq = torch.tensor([1.0 / 256.0], device=dev)
+    y = ops.gemm_fp8(a8, b8, fmt, dq_a=dq, dq=0.5)
+    ys = ops.gemm_fp8(a8[:Ms].contiguous(), b8, fmt, dq_a=dq, dq=0.5)
+    assert torch.equal(y[:Ms], ys)
+    want = (a8.view(torch.float8_e5m2 if fmt else torch.float8_e4m3fn).float() @ b8.view(torch.float8_e4m3fn).float().t()) / 512.0
+    assert rel_l2(y, want) < BF16_TOL
+    if fmt == 0:
+        res = torch.randn(M, N, generator=g).bfloat16().to(dev)
+        z = ops.gemm_fp8_res(a8, b8, res, dq_a=dq, dq=0.5)
+        zs = ops.gemm_fp8_res(a8[:Ms].contiguous(), b8, res[:Ms].contiguous(), dq_a=dq, dq=0.5)
+        assert torch.equal(z[:Ms], zs) and torch.equal(z, (res.float() + y.float()).bfloat16())
+
+
 @pytest.mark.parametrize("shape", [(512, 256, 512), (16384, 768, 3072)])
 def test_mlp8_as_the_benchmark_times_it(ops, dev, shape):
     """Configuration 3 of BASELINE.json in the form bench.py times: OCP e4m3 at 448, the activation scale from the tensor's

@@ -822,6 +822,8 @@ using Cfg8g = GemmCfg<128, 128, 2, 2, 1, TFB_K_CONTIG, TFB_K_CONTIG, TFB_FMT_E4M
 // sums in the same order, the epilogue's values bit for bit), else the 128 x 128 kernel.
 template <class Cfg, class Epi>
 static int launch8(GemmOperand P, GemmOperand Q, int np, int nq, long kbytes, Epi e, hipStream_t s) {
+  // a contraction of 768 bytes (the fp8 attention projections of a 768-wide model): the weight-stationary kernel
+  if (gemm_ws8_applies(np, nq, kbytes)) return gemm_ws8_launch<Cfg::FMTP, Cfg::FMTQ>(P, Q, np, nq, kbytes, e, s);
   if (gemm_pp_applies(np, nq, kbytes)) return gemm_pp_launch<1, Cfg::FMTP, Cfg::FMTQ>(P, Q, np, nq, kbytes, e, s);
   return gemm_launch<Cfg>(P, Q, np, nq, kbytes, 1, LoadIdentity{}, LoadIdentity{}, e, s);
 }
